@@ -1,0 +1,148 @@
+"""
+ctypes binding of the C oracle in ``oracle/lstm2_oracle.c`` -- test infrastructure only.
+
+The C file restates the reference op (returnn/native_op.py:1081-1121, :1184-1285;
+returnn/native_op.cpp:1032-1067) and is the checker for the HIP path and the timed
+CPU baseline.  It is never the product: nothing under ``returnn_amd/`` imports it.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from typing import Optional, Tuple
+
+import numpy
+
+_dir = os.path.dirname(os.path.abspath(__file__))
+_so = os.path.join(_dir, "liblstm2_oracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with the Makefile next to it. Returns the path of the library."""
+    if force and os.path.exists(_so):
+        os.remove(_so)
+    subprocess.check_call(["make", "-s", "-C", _dir])
+    return _so
+
+
+def _load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_so):
+            build()
+        lib = ctypes.CDLL(_so)
+        for suffix, ptr in (("f32", ctypes.POINTER(ctypes.c_float)), ("f64", ctypes.POINTER(ctypes.c_double))):
+            fwd = getattr(lib, "lstm2_oracle_fwd_" + suffix)
+            fwd.restype = ctypes.c_int
+            fwd.argtypes = [ptr] * 5 + [ctypes.c_int32, ctypes.c_int32] + [ptr] * 5 + [
+                ctypes.c_int64,
+                ctypes.c_int32,
+                ctypes.c_int32,
+                ctypes.c_int32,
+            ]
+            last = getattr(lib, "lstm2_oracle_last_output_" + suffix)
+            last.restype = ctypes.c_int
+            last.argtypes = [ptr] * 3 + [ctypes.c_int32, ctypes.c_int32, ptr, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
+        lib.lstm2_oracle_max_threads.restype = ctypes.c_int
+        _lib = lib
+    return _lib
+
+
+def max_threads() -> int:
+    """Number of OpenMP threads the GEMM part can use on this host."""
+    return int(_load().lstm2_oracle_max_threads())
+
+
+def _prep(a, dtype, shape, name):
+    a = numpy.ascontiguousarray(a, dtype=dtype)
+    if a.shape != shape:
+        raise ValueError("oracle: %s has shape %r, expected %r" % (name, a.shape, shape))
+    return a
+
+
+def native_lstm2_fwd(
+    X, W, y0, c0, i, start: int = 0, step: int = 1, *, dtype=numpy.float32, threads: int = 1
+) -> Tuple[numpy.ndarray, numpy.ndarray, numpy.ndarray, numpy.ndarray, numpy.ndarray]:
+    """
+    Reference semantics of ``NativeLstm2`` forward (returnn/native_op.py:1184-1285).
+
+    :param X: [T,B,4n] pre-projected gate inputs, gate order cell-in, input, forget, output
+    :param W: [n,4n] recurrent weights
+    :param y0: [B,n] initial output
+    :param c0: [B,n] initial cell state
+    :param i: [T,B] 0/1 mask
+    :param start: first frame (for step<0 counted from the end)
+    :param step: +-1 direction, or a wider stride
+    :param dtype: numpy.float32 (the reference's arithmetic) or numpy.float64
+    :param threads: OpenMP threads for the recurrent GEMM; the pointwise part is always sequential
+    :return: Y [T,B,n], C [T,B,n], H [T,B,4n], d [B,n], y_last [B,n]
+      (y_last is the final carry of the last valid output, not an output of the reference op:
+      it is what the caller derives with ``_lstm_last_output``, returnn/tf/native_op.py:913-929)
+    """
+    dtype = numpy.dtype(dtype)
+    if dtype == numpy.float32:
+        suffix, ctype = "f32", ctypes.c_float
+    elif dtype == numpy.float64:
+        suffix, ctype = "f64", ctypes.c_double
+    else:
+        raise ValueError("oracle: dtype must be float32 or float64")
+    i = numpy.ascontiguousarray(i, dtype=dtype)
+    y0 = numpy.ascontiguousarray(y0, dtype=dtype)
+    if i.ndim != 2 or y0.ndim != 2:
+        raise ValueError("oracle: i must be [T,B] and y0 [B,n]")
+    T, B = i.shape
+    n = y0.shape[1]
+    X = _prep(X, dtype, (T, B, 4 * n), "X")
+    W = _prep(W, dtype, (n, 4 * n), "W")
+    y0 = _prep(y0, dtype, (B, n), "y0")
+    c0 = _prep(c0, dtype, (B, n), "c0")
+    Y = numpy.empty((T, B, n), dtype=dtype)
+    C = numpy.empty((T, B, n), dtype=dtype)
+    H = numpy.empty((T, B, 4 * n), dtype=dtype)
+    d = numpy.empty((B, n), dtype=dtype)
+    y_last = numpy.empty((B, n), dtype=dtype)
+    p = ctypes.POINTER(ctype)
+    fwd = getattr(_load(), "lstm2_oracle_fwd_" + suffix)
+    rc = fwd(
+        *(a.ctypes.data_as(p) for a in (X, W, y0, c0, i)),
+        int(start),
+        int(step),
+        *(a.ctypes.data_as(p) for a in (Y, C, H, d, y_last)),
+        T,
+        B,
+        n,
+        int(threads),
+    )
+    if rc == 2:
+        raise ValueError("oracle: need 0 <= start < T and step != 0 (start=%r, step=%r, T=%r)" % (start, step, T))
+    if rc != 0:
+        raise RuntimeError("oracle: error code %i" % rc)
+    return Y, C, H, d, y_last
+
+
+def lstm_last_output(Y, y0, i, start: int = 0, step: int = 1, *, dtype=numpy.float32) -> numpy.ndarray:
+    """
+    Caller-side final output per sequence (returnn/tf/native_op.py:913-929).
+
+    :param Y: [T,B,n] op output
+    :param y0: [B,n]
+    :param i: [T,B] mask
+    :return: [B,n]
+    """
+    dtype = numpy.dtype(dtype)
+    suffix, ctype = ("f32", ctypes.c_float) if dtype == numpy.float32 else ("f64", ctypes.c_double)
+    Y = numpy.ascontiguousarray(Y, dtype=dtype)
+    T, B, n = Y.shape
+    y0 = _prep(y0, dtype, (B, n), "y0")
+    i = _prep(i, dtype, (T, B), "i")
+    out = numpy.empty((B, n), dtype=dtype)
+    p = ctypes.POINTER(ctype)
+    rc = getattr(_load(), "lstm2_oracle_last_output_" + suffix)(
+        Y.ctypes.data_as(p), y0.ctypes.data_as(p), i.ctypes.data_as(p), int(start), int(step), out.ctypes.data_as(p), T, B, n
+    )
+    if rc != 0:
+        raise ValueError("oracle: last_output error code %i" % rc)
+    return out

@@ -1,0 +1,332 @@
+"""
+Pins the CPU oracle (oracle/lstm2_oracle.c) before anything is compared against it.
+
+Every check here uses something the oracle's code does not contain: the reference's own
+deterministic fixture and comparison rules run through an independently written textbook
+LSTM, torch's LSTM, closed forms, invariants of the op and an fp64 brute force.
+"""
+
+from __future__ import annotations
+
+import numpy
+import pytest
+from numpy.testing import assert_allclose
+
+from oracle import lstm2_oracle as oracle
+from _textbook import (
+    REFERENCE_START_STEP,
+    reference_fixture,
+    sigmoid,
+    textbook_lstm,
+    torch_lstm,
+    visited_slice,
+)
+
+
+def _project(fx):
+    """X for the op = x . W_f + b (tests/test_TFNativeOp.py:801-804)."""
+    return fx["x"] @ fx["W_f"] + fx["b"][None, None, :]
+
+
+@pytest.mark.parametrize("start,step", REFERENCE_START_STEP)
+@pytest.mark.parametrize("dtype", [numpy.float32, numpy.float64])
+def test_reference_fixture_vs_textbook(start, step, dtype):
+    """tests/test_TFNativeOp.py:902-906 (test_native_lstm2_impl), rules of :851-854, rtol 1e-6."""
+    fx = reference_fixture(dtype)
+    T = fx["x"].shape[0]
+    Y, C, H, d, y_last = oracle.native_lstm2_fwd(
+        _project(fx), fx["W_r"], fx["h_0"], fx["c_0"], fx["mask"], start, step, dtype=dtype
+    )
+    h2, c2, cT, hT = textbook_lstm(start=start, step=step, dtype=numpy.float64, **fx)
+    sl = visited_slice(T, start, step)
+    m = fx["mask"][:, :, None]
+    rtol = 1e-6
+    assert_allclose(Y[sl] * m[sl], h2[sl] * m[sl], rtol=rtol)
+    assert_allclose(C[sl] * m[sl], c2[sl] * m[sl], rtol=rtol)
+    assert_allclose(d, cT, rtol=rtol)
+    assert_allclose(y_last, hT, rtol=rtol)
+    # the caller-side formula and the kernel's carry must be the same thing
+    assert_allclose(oracle.lstm_last_output(Y, fx["h_0"], fx["mask"], start, step, dtype=dtype), y_last, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("start,step", REFERENCE_START_STEP + [(2, 3), (3, -2), (4, 1)])
+def test_start_step_slice_equivalence(start, step):
+    """tests/test_TFNativeOp.py:897-899: op(start, step) == op(0, 1) on x[start_::step], scattered back."""
+    rng = numpy.random.default_rng(3)
+    T, B, n = 7, 3, 4
+    X = rng.normal(0, 0.5, (T, B, 4 * n)).astype(numpy.float32)
+    W = rng.uniform(-0.5, 0.5, (n, 4 * n)).astype(numpy.float32)
+    y0 = rng.normal(0, 0.3, (B, n)).astype(numpy.float32)
+    c0 = rng.normal(0, 0.3, (B, n)).astype(numpy.float32)
+    i = (rng.uniform(size=(T, B)) < 0.7).astype(numpy.float32)
+    Y, C, H, d, yl = oracle.native_lstm2_fwd(X, W, y0, c0, i, start, step)
+    sl = visited_slice(T, start, step)
+    Ys, Cs, Hs, ds, yls = oracle.native_lstm2_fwd(X[sl], W, y0, c0, i[sl], 0, 1)
+    Y2 = numpy.zeros_like(Y)
+    C2 = numpy.zeros_like(C)
+    H2 = X.copy()
+    Y2[sl], C2[sl], H2[sl] = Ys, Cs, Hs
+    # bit-exact: same arithmetic on the same numbers in the same order
+    for a, b in ((Y, Y2), (C, C2), (H, H2), (d, ds), (yl, yls)):
+        assert numpy.array_equal(a, b)
+
+
+def _random_problem(rng, T, B, n, scale_w=None):
+    scale_w = scale_w if scale_w is not None else 1.0 / numpy.sqrt(n)
+    X = rng.normal(0, 0.5, (T, B, 4 * n))
+    W = rng.uniform(-scale_w, scale_w, (n, 4 * n))
+    y0 = rng.normal(0, 0.3, (B, n))
+    c0 = rng.normal(0, 0.3, (B, n))
+    return X, W, y0, c0
+
+
+def test_vs_torch_lstm_full_length():
+    rng = numpy.random.default_rng(0)
+    T, B, n = 11, 3, 5
+    X, W, y0, c0 = _random_problem(rng, T, B, n)
+    i = numpy.ones((T, B))
+    Y, C, H, d, yl = oracle.native_lstm2_fwd(X, W, y0, c0, i, dtype=numpy.float64)
+    Yt, hT, cT = torch_lstm(X, W, y0, c0)
+    assert_allclose(Y, Yt, rtol=1e-10, atol=1e-12)
+    assert_allclose(d, cT, rtol=1e-10, atol=1e-12)
+    assert_allclose(yl, hT, rtol=1e-10, atol=1e-12)
+    # float32 oracle agrees with that to float32 rounding
+    Y32, C32, H32, d32, yl32 = oracle.native_lstm2_fwd(X, W, y0, c0, i, dtype=numpy.float32)
+    assert_allclose(Y32, Yt, rtol=2e-5, atol=2e-6)
+    assert_allclose(d32, cT, rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("step", [1, -1])
+def test_vs_torch_lstm_packed_ragged(step):
+    """Ragged batch with right padding; backward direction starts at each sequence's last valid frame
+    without any reversal of X (returnn/tf/native_op.py:835, does_direction_handling)."""
+    rng = numpy.random.default_rng(1)
+    T, B, n = 9, 4, 3
+    X, W, y0, c0 = _random_problem(rng, T, B, n)
+    lens = numpy.array([9, 4, 1, 6])
+    i = (numpy.arange(T)[:, None] < lens[None, :]).astype(numpy.float64)
+    Y, C, H, d, yl = oracle.native_lstm2_fwd(X, W, y0, c0, i, 0, step, dtype=numpy.float64)
+    Yt, hT, cT = torch_lstm(X, W, y0, c0, lens=lens, reverse=(step < 0))
+    assert_allclose(Y, Yt, rtol=1e-10, atol=1e-12)  # torch pads with zeros; so does the op (Y = 0 where mask = 0)
+    assert_allclose(d, cT, rtol=1e-10, atol=1e-12)
+    assert_allclose(yl, hT, rtol=1e-10, atol=1e-12)
+
+
+def test_closed_form_single_cell():
+    """T=B=n=1 (pattern of tests/test_TFNativeOp.py:264-297): every term written out by hand."""
+    x = numpy.array([0.3, -0.2, 0.5, 0.1])
+    w = numpy.array([0.7, -0.4, 0.2, 0.9])
+    y0, c0 = 0.6, -0.8
+    g = x + y0 * w
+    c = sigmoid(g[2]) * c0 + sigmoid(g[1]) * numpy.tanh(g[0])
+    y = sigmoid(g[3]) * numpy.tanh(c)
+    Y, C, H, d, yl = oracle.native_lstm2_fwd(
+        x.reshape(1, 1, 4), w.reshape(1, 4), [[y0]], [[c0]], [[1.0]], dtype=numpy.float64
+    )
+    assert_allclose(C[0, 0, 0], c, rtol=1e-14)
+    assert_allclose(Y[0, 0, 0], y, rtol=1e-14)
+    assert_allclose(H[0, 0], [numpy.tanh(g[0]), sigmoid(g[1]), sigmoid(g[2]), sigmoid(g[3])], rtol=1e-14)
+    assert_allclose(d[0, 0], c, rtol=1e-14)
+    assert_allclose(yl[0, 0], y, rtol=1e-14)
+
+
+def test_closed_form_gate_layout():
+    """Each gate block of X drives exactly the role the layout says (cell-in, input, forget, output).
+    W = 0 and a large bias on one block at a time saturate one gate; a transposed or permuted block fails."""
+    n, B = 3, 2
+    W = numpy.zeros((n, 4 * n))
+    y0 = numpy.zeros((B, n))
+    c0 = numpy.full((B, n), 0.5)
+    i = numpy.ones((1, B))
+    big = 40.0
+
+    def run(blocks):
+        X = numpy.zeros((1, B, 4 * n))
+        for blk, v in blocks.items():
+            X[:, :, blk * n : (blk + 1) * n] = v
+        Y, C, H, d, yl = oracle.native_lstm2_fwd(X, W, y0, c0, i, dtype=numpy.float64)
+        return Y[0], C[0]
+
+    # forget gate open, input gate closed: c = c0; y = sigmoid(0) * tanh(c0)
+    Y, C = run({2: big, 1: -big})
+    assert_allclose(C, 0.5, rtol=1e-12)
+    assert_allclose(Y, 0.5 * numpy.tanh(0.5), rtol=1e-12)
+    # forget closed, input open, cell-in saturated to +1: c = 1; output gate open: y = tanh(1)
+    Y, C = run({2: -big, 1: big, 0: big, 3: big})
+    assert_allclose(C, 1.0, rtol=1e-12)
+    assert_allclose(Y, numpy.tanh(1.0), rtol=1e-12)
+    # output gate closed: y = 0 whatever c is
+    Y, C = run({3: -big})
+    assert_allclose(Y, 0.0, atol=1e-15)
+
+
+def test_closed_form_zero_input_and_weights():
+    """X = 0, W = 0: c_t = c_{t-1}/2, y_t = tanh(c_t)/2."""
+    T, B, n = 6, 2, 3
+    c0 = numpy.array([[1.0, -2.0, 0.25], [0.5, 4.0, -1.0]])
+    Y, C, H, d, yl = oracle.native_lstm2_fwd(
+        numpy.zeros((T, B, 4 * n)), numpy.zeros((n, 4 * n)), numpy.zeros((B, n)), c0, numpy.ones((T, B)), dtype=numpy.float64
+    )
+    for t in range(T):
+        assert_allclose(C[t], c0 * 0.5 ** (t + 1), rtol=1e-14)
+        assert_allclose(Y[t], 0.5 * numpy.tanh(c0 * 0.5 ** (t + 1)), rtol=1e-14)
+    assert_allclose(H[:, :, :n], 0.0, atol=0)
+    assert_allclose(H[:, :, n:], 0.5, rtol=0)
+    assert_allclose(d, C[-1], rtol=0)
+
+
+def test_closed_form_mask_zero():
+    """mask == 0 everywhere: Y = 0, C[t] = c0, d = c0, final output = y0, H = act(X + y0 . W) on every frame."""
+    rng = numpy.random.default_rng(5)
+    T, B, n = 4, 3, 2
+    X, W, y0, c0 = _random_problem(rng, T, B, n)
+    Y, C, H, d, yl = oracle.native_lstm2_fwd(X, W, y0, c0, numpy.zeros((T, B)), dtype=numpy.float64)
+    assert numpy.array_equal(Y, numpy.zeros_like(Y))
+    for t in range(T):
+        assert numpy.array_equal(C[t], c0)
+    assert numpy.array_equal(d, c0)
+    assert numpy.array_equal(yl, y0)
+    G = X + (y0 @ W)[None]
+    expect = numpy.concatenate([numpy.tanh(G[..., :n]), sigmoid(G[..., n:])], axis=-1)
+    assert_allclose(H, expect, rtol=1e-13)
+
+
+def test_zero_length():
+    """T = 0: d = c0 (returnn/native_op.py:1236-1237; tests/test_TFNativeOp.py:448-464)."""
+    B, n = 2, 3
+    c0 = numpy.arange(B * n, dtype=numpy.float32).reshape(B, n)
+    y0 = -c0
+    Y, C, H, d, yl = oracle.native_lstm2_fwd(
+        numpy.zeros((0, B, 4 * n)), numpy.zeros((n, 4 * n)), y0, c0, numpy.zeros((0, B))
+    )
+    assert Y.shape == (0, B, n) and C.shape == (0, B, n) and H.shape == (0, B, 4 * n)
+    assert numpy.array_equal(d, c0)
+    assert numpy.array_equal(yl, y0)
+
+
+def test_zeros_run():
+    """tests/test_TFNativeOp.py:368-384 (T=2, B=1, n=3, all-zero input through the cell)."""
+    T, B, n = 2, 1, 3
+    Y, C, H, d, yl = oracle.native_lstm2_fwd(
+        numpy.zeros((T, B, 4 * n)), numpy.zeros((n, 4 * n)), numpy.zeros((B, n)), numpy.zeros((B, n)), numpy.ones((T, B))
+    )
+    assert numpy.array_equal(Y, numpy.zeros((T, B, n), dtype=numpy.float32))
+    assert numpy.array_equal(d, numpy.zeros((B, n), dtype=numpy.float32))
+
+
+def test_unvisited_frames_and_masked_h():
+    """Frames the loop does not visit keep Y = C = 0 and H = X; masked visited frames still get activated H."""
+    rng = numpy.random.default_rng(7)
+    T, B, n = 6, 2, 3
+    X, W, y0, c0 = _random_problem(rng, T, B, n)
+    i = numpy.ones((T, B))
+    i[2, 1] = 0.0
+    Y, C, H, d, yl = oracle.native_lstm2_fwd(X, W, y0, c0, i, 1, 2, dtype=numpy.float64)
+    for t in (0, 2, 4):
+        assert numpy.array_equal(Y[t], numpy.zeros((B, n)))
+        assert numpy.array_equal(C[t], numpy.zeros((B, n)))
+        assert numpy.array_equal(H[t], X[t])
+    Y, C, H, d, yl = oracle.native_lstm2_fwd(X, W, y0, c0, i, 0, 1, dtype=numpy.float64)
+    assert numpy.array_equal(Y[2, 1], numpy.zeros(n))
+    assert numpy.array_equal(C[2, 1], C[1, 1])  # cell carried
+    assert numpy.all(numpy.abs(H[2, 1, :n]) < 1) and numpy.all((H[2, 1, n:] > 0) & (H[2, 1, n:] < 1))
+    assert not numpy.array_equal(H[2, 1], X[2, 1])
+    assert numpy.array_equal(d, C[T - 1])
+
+
+def test_time_reversal_symmetry():
+    """Full-length mask: op(X, step=-1) == flip_T(op(flip_T(X), step=+1))."""
+    rng = numpy.random.default_rng(9)
+    T, B, n = 8, 2, 4
+    X, W, y0, c0 = _random_problem(rng, T, B, n)
+    i = numpy.ones((T, B))
+    a = oracle.native_lstm2_fwd(X, W, y0, c0, i, 0, -1)
+    b = oracle.native_lstm2_fwd(X[::-1], W, y0, c0, i, 0, 1)
+    for k in range(3):
+        assert numpy.array_equal(a[k], b[k][::-1])
+    assert numpy.array_equal(a[3], b[3])
+    assert numpy.array_equal(a[4], b[4])
+
+
+def test_batch_row_independence():
+    """Each batch row is an independent sequence (single-vs-batched check in the manner of tests/rf_utils.py)."""
+    rng = numpy.random.default_rng(11)
+    T, B, n = 5, 4, 3
+    X, W, y0, c0 = _random_problem(rng, T, B, n)
+    lens = numpy.array([5, 2, 3, 1])
+    i = (numpy.arange(T)[:, None] < lens[None, :]).astype(numpy.float64)
+    full = oracle.native_lstm2_fwd(X, W, y0, c0, i, dtype=numpy.float64)
+    for b in range(B):
+        one = oracle.native_lstm2_fwd(X[:, b : b + 1], W, y0[b : b + 1], c0[b : b + 1], i[:, b : b + 1], dtype=numpy.float64)
+        for k in range(3):
+            assert numpy.array_equal(full[k][:, b : b + 1], one[k])
+        assert numpy.array_equal(full[3][b : b + 1], one[3])
+
+
+def test_brute_force_fp64_tiny():
+    """Scalar triple loops, no matrix products, on a tiny ragged case with a non-0/1 start and stride."""
+    rng = numpy.random.default_rng(13)
+    T, B, n = 5, 2, 2
+    X, W, y0, c0 = _random_problem(rng, T, B, n)
+    i = numpy.array([[1, 1], [1, 0], [0, 1], [1, 1], [1, 0]], dtype=numpy.float64)
+    for start, step in [(0, 1), (0, -1), (1, 2), (1, -2)]:
+        Y, C, H, d, yl = oracle.native_lstm2_fwd(X, W, y0, c0, i, start, step, dtype=numpy.float64)
+        ts = list(range(start, T, step)) if step > 0 else list(range(T - start - 1, -1, step))
+        for b in range(B):
+            y = list(y0[b])
+            c = list(c0[b])
+            for t in ts:
+                g = [X[t, b, col] + sum(y[k] * W[k, col] for k in range(n)) for col in range(4 * n)]
+                m = i[t, b]
+                y_new, c_new = [], []
+                for j in range(n):
+                    a0 = numpy.tanh(g[j])
+                    a1, a2, a3 = (sigmoid(g[q * n + j]) for q in (1, 2, 3))
+                    cj = (c[j] * a2 + a0 * a1) * m + c[j] * (1 - m)
+                    yj = numpy.tanh(cj) * a3 * m
+                    assert_allclose(H[t, b, [j, n + j, 2 * n + j, 3 * n + j]], [a0, a1, a2, a3], rtol=1e-13)
+                    assert_allclose(C[t, b, j], cj, rtol=1e-13, atol=1e-15)
+                    assert_allclose(Y[t, b, j], yj, rtol=1e-13, atol=1e-15)
+                    c_new.append(cj)
+                    y_new.append(yj + y[j] * (1 - m))
+                y, c = y_new, c_new
+            assert_allclose(d[b], c, rtol=1e-13)
+            assert_allclose(yl[b], y, rtol=1e-13)
+
+
+def test_threads_do_not_change_results():
+    rng = numpy.random.default_rng(17)
+    T, B, n = 6, 5, 96
+    X, W, y0, c0 = _random_problem(rng, T, B, n)
+    i = numpy.ones((T, B))
+    a = oracle.native_lstm2_fwd(X, W, y0, c0, i, threads=1)
+    b = oracle.native_lstm2_fwd(X, W, y0, c0, i, threads=4)
+    for u, v in zip(a, b):
+        assert numpy.array_equal(u, v)
+
+
+def test_f32_close_to_f64_cfg1():
+    """BASELINE config 1 (T=32, B=4, n=64): float32 oracle within 1e-5 relative of the float64 one."""
+    from returnn_amd import synthetic
+
+    p = synthetic.make_config("cfg1")
+    a = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, p.start, p.step, dtype=numpy.float32)
+    b = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, p.start, p.step, dtype=numpy.float64)
+    for u, v in zip(a, b):
+        assert_allclose(u, v, rtol=1e-5, atol=1e-6)
+
+
+def test_error_paths():
+    T, B, n = 3, 2, 2
+    z = lambda *s: numpy.zeros(s, dtype=numpy.float32)  # noqa: E731
+    args = (z(T, B, 4 * n), z(n, 4 * n), z(B, n), z(B, n), z(T, B))
+    with pytest.raises(ValueError):
+        oracle.native_lstm2_fwd(*args, 3, 1)  # start >= T
+    with pytest.raises(ValueError):
+        oracle.native_lstm2_fwd(*args, -1, 1)
+    with pytest.raises(ValueError):
+        oracle.native_lstm2_fwd(*args, 0, 0)  # step == 0
+    with pytest.raises(ValueError):
+        oracle.native_lstm2_fwd(z(T, B, 4 * n + 1), *args[1:])  # X last dim
+    with pytest.raises(ValueError):
+        oracle.native_lstm2_fwd(args[0], z(n, 4 * n + 4), *args[2:])
