@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""
+Benchmark of the NativeLstm2 forward hot path on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+Workload (default): BASELINE config 3, the bidirectional pair at n=1024 -- T=1000, B=32, bf16 weights and
+activations with fp32 accumulate and cell state, ragged lengths in [500,1000]; one step = two op calls on
+the same inputs (step=+1 and step=-1), issued through the C ABI with inputs, outputs and workspace already
+resident in HBM.  ``value`` = timesteps x sequences processed per second = 2*T*B*K / elapsed (padded frames
+counted, both directions).
+
+Prints ONE JSON line with the throughput, a ``roofline`` object for the dominant kernel (the persistent
+step kernel; algorithmic GEMM flops 8*T*B*n^2 per launch over the HIP-event duration of a call on the launch
+stream) and a ``cpu_baseline`` object (the CPU restatement of the reference's path -- per-step BLAS SGEMM plus
+the sequential pointwise loop -- timed on this host on a bounded sample of the same shape in fp32).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+_root = os.path.dirname(os.path.abspath(__file__))
+if _root not in sys.path:
+    sys.path.insert(0, _root)
+
+PEAK_MFMA = {"bf16": 2.5e15, "f32": 157.3e12}  # MI355X dense matrix peaks, FLOP/s
+PEAK_HBM = 8.0e12  # B/s
+
+
+def algorithmic_bytes_per_unit(n: int, dtype: str) -> int:
+    """HBM bytes per timestep x sequence: read X (4n), write H (4n), Y (n) in the activation type,
+    write C (n, fp32), read the mask (4 bytes)."""
+    e = 2 if dtype == "bf16" else 4
+    return e * 4 * n + e * 4 * n + e * n + 4 * n + 4
+
+
+def cpu_baseline(name: str, target_seconds: float = 15.0):
+    """Times the CPU restatement (test infrastructure, used here only as the reported baseline)."""
+    import numpy
+
+    from oracle import lstm2_oracle
+    from returnn_amd import synthetic
+
+    try:
+        from threadpoolctl import threadpool_info
+
+        blas_threads = max([int(i.get("num_threads", 1)) for i in threadpool_info() if i.get("user_api") == "blas"] or [1])
+    except Exception:
+        blas_threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    probe_T = 25
+    p = synthetic.make_config(name, T=probe_T)
+    lstm2_oracle.native_lstm2_fwd_blas(p.X[:2], p.W, p.y0, p.c0, p.i[:2])  # warm-up (BLAS thread pool, page-in)
+    t0 = time.perf_counter()
+    lstm2_oracle.native_lstm2_fwd_blas(p.X, p.W, p.y0, p.c0, p.i)
+    per_frame = (time.perf_counter() - t0) / probe_T
+    full_T = synthetic.make_config.__globals__["_SPECS"][name]["T"]
+    T = int(max(probe_T, min(full_T, target_seconds / max(per_frame, 1e-9))))
+    p = synthetic.make_config(name, T=T)
+    t0 = time.perf_counter()
+    lstm2_oracle.native_lstm2_fwd_blas(p.X, p.W, p.y0, p.c0, p.i)
+    dt = time.perf_counter() - t0
+    return {
+        "value": p.T * p.B / dt,
+        "unit": "timesteps*seqs/s",
+        "cores": blas_threads,
+        "kind": "port",
+        "sample": "%s shape fp32, one direction, first T=%i of %i frames (B=%i, n=%i), %.1f s; GEMM on %i BLAS threads, "
+        "pointwise loop on 1 thread as the reference's CPU path" % (name, p.T, full_T, p.B, p.n, dt, blas_threads),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg5"])
+    ap.add_argument("--mode", default="auto", choices=["auto", "persistent", "graph", "stepwise"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the recurrence is one sequential chain per batch; "
+              "see DESIGN.md for how it would shard); --gpus %i is not supported." % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from returnn_amd import build as rbuild
+    from returnn_amd import lib, synthetic
+
+    if not os.path.exists(rbuild.LIB_PATH):
+        rbuild.build_library()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    cabi = lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    p = synthetic.make_config(args.workload)
+    T, B, n = p.T, p.B, p.n
+    dtype = p.dtype
+    act = torch.bfloat16 if dtype == "bf16" else torch.float32
+    dt_code = lib.DTYPE_BF16 if dtype == "bf16" else lib.DTYPE_F32
+    mode = lib.MODES[args.mode]
+    directions = [1, -1] if args.workload == "cfg3" else [1]
+
+    X = torch.from_numpy(p.X).to(dev).to(act)
+    W = torch.from_numpy(p.W).to(dev).to(act)
+    y0 = torch.from_numpy(p.y0).to(dev).to(act)
+    c0 = torch.from_numpy(p.c0).to(dev)
+    msk = torch.from_numpy(p.i).to(dev)
+    ws_bytes = lib.workspace_bytes(T, B, n, dt_code, mode)
+    outs = []
+    for _ in directions:
+        outs.append(
+            dict(
+                Y=torch.empty((T, B, n), dtype=act, device=dev),
+                C=torch.empty((T, B, n), dtype=torch.float32, device=dev),
+                H=torch.empty((T, B, 4 * n), dtype=act, device=dev),
+                d=torch.empty((B, n), dtype=torch.float32, device=dev),
+                ws=torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=dev),
+            )
+        )
+    stream = torch.cuda.current_stream(dev)
+
+    def one_call(k):
+        o = outs[k]
+        rc = cabi.rtn_native_lstm2_fwd(
+            X.data_ptr(), W.data_ptr(), y0.data_ptr(), c0.data_ptr(), msk.data_ptr(), 0, directions[k],
+            o["Y"].data_ptr(), o["C"].data_ptr(), o["H"].data_ptr(), o["d"].data_ptr(), T, B, n, dt_code, mode,
+            o["ws"].data_ptr(), o["ws"].numel(), stream.cuda_stream,
+        )  # fmt: skip
+        lib.check(rc)
+
+    for _ in range(args.warmup):
+        for k in range(len(directions)):
+            one_call(k)
+    torch.cuda.synchronize()
+    for k in range(len(directions)):
+        lib.check(cabi.rtn_native_lstm2_fwd_status(outs[k]["ws"].data_ptr(), stream.cuda_stream))
+
+    events = []
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        for k in range(len(directions)):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            one_call(k)
+            e1.record(stream)
+            events.append((e0, e1))
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    for k in range(len(directions)):
+        lib.check(cabi.rtn_native_lstm2_fwd_status(outs[k]["ws"].data_ptr(), stream.cuda_stream))
+    assert all(bool(torch.isfinite(o["d"]).all()) for o in outs)
+
+    call_ms = sum(a.elapsed_time(b) for a, b in events) / len(events)
+    units_per_step = len(directions) * T * B
+    value = units_per_step * args.steps / elapsed
+    flops_per_launch = 8.0 * T * B * n * n
+    achieved = flops_per_launch / (call_ms * 1e-3)
+    peak = PEAK_MFMA[dtype]
+    bytes_per_launch = algorithmic_bytes_per_unit(n, dtype) * T * B
+    plan = lib.describe_plan(T, B, n, dt_code, mode)
+
+    result = {
+        "metric": "LSTM fwd timesteps*seqs/sec (T*B/s) at n=%i" % n,
+        "value": value,
+        "unit": "timesteps*seqs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": elapsed * 1e3 / args.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype,
+        "data": "synthetic",
+        "config": {
+            "workload": "%s: NativeLstm2 forward%s, T=%i B=%i n=%i %s, ragged=%s"
+            % (args.workload, " bidirectional pair (two calls: step=+1, step=-1)" if len(directions) == 2 else "", T, B, n,
+               dtype, p.lens is not None),
+            "calls_per_step": len(directions),
+            "units_per_step": units_per_step,
+            "mode": args.mode,
+            "plan": plan,
+            "sync_policy": os.environ.get("RTN_LSTM2_SYNC", "default"),
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": achieved / 1e12,
+            "peak": peak / 1e12,
+            "unit": "TFLOP/s",
+            "frac": achieved / peak,
+            "traffic": None,
+            "kernel": "k_lstm2_mfma (one launch = one op call of T*B = %i units, 8*n^2 flops each)" % (T * B),
+            "launch_ms": call_ms,
+            "hbm_algorithmic_GBps": bytes_per_launch / (call_ms * 1e-3) / 1e9,
+            "hbm_frac": bytes_per_launch / (call_ms * 1e-3) / PEAK_HBM,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.workload, args.cpu_seconds)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,123 @@
+/*
+ * C ABI of the MI355X (gfx950) NativeLstm2 forward library (librtn_native_lstm2.so).
+ *
+ * Plain pointers and sizes only; all data pointers are DEVICE pointers on the
+ * current HIP device, `hip_stream` is a hipStream_t (NULL = the default stream).
+ * Every entry point only enqueues work on that stream: no device synchronisation,
+ * no allocation of device memory (scratch comes in through `workspace`), inputs are
+ * never written, outputs are caller-allocated and fully overwritten (the callee
+ * does not rely on them being zeroed).
+ *
+ * The reference has no C ABI of its own for this operator: it generates a C++
+ * translation unit per op at run time (returnn/torch/util/native_op.py:83-376)
+ * whose body is the op's `c_fw_code` string.  Each function below names the piece
+ * of that generated code it stands in for.
+ */
+#ifndef RTN_NATIVE_LSTM2_H
+#define RTN_NATIVE_LSTM2_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes.  The reference signals these through TORCH_CHECK / assert_cmp
+ * (returnn/native_op.cpp:60-69, 660); under its -DNDEBUG build the range checks only
+ * print.  Here they are hard errors and nothing is enqueued when one is returned. */
+#define RTN_OK 0
+#define RTN_ERR_SHAPE 1       /* negative or inconsistent T / B / n */
+#define RTN_ERR_RANGE 2       /* need 0 <= start < T and step != 0 (returnn/native_op.py:1249-1252) */
+#define RTN_ERR_ARG 3         /* null pointer, misaligned pointer, unknown dtype or mode */
+#define RTN_ERR_WORKSPACE 4   /* workspace missing or smaller than rtn_native_lstm2_fwd_workspace_bytes() */
+#define RTN_ERR_HIP 5         /* a HIP runtime call failed (HANDLE_LAST_ERROR, returnn/native_op.cpp:773-780) */
+#define RTN_ERR_UNSUPPORTED 6 /* the requested mode cannot run this shape on this device */
+#define RTN_ERR_ABORTED 7     /* reported by rtn_native_lstm2_fwd_status: a bounded in-kernel wait expired */
+
+/* Element type of X, W, y0, Y and H.  The mask i, the cell states c0, C and d are
+ * always float32.  F32 is the reference's arithmetic (Ndarray_DEV_DATA casts to float*,
+ * returnn/native_op.cpp:647).  BF16 keeps float32 accumulation, gates and cell state. */
+#define RTN_DTYPE_F32 0
+#define RTN_DTYPE_BF16 1
+
+/* Execution mode.
+ * AUTO:       PERSISTENT when the shape and device allow it and the stream is not
+ *             being captured, else GRAPH.
+ * PERSISTENT: one cooperative kernel runs all time steps; the recurrent weights stay
+ *             on chip and the workgroups exchange the hidden state through the
+ *             workspace with a per-step flag barrier.
+ * GRAPH:      one kernel launch per time step; outside stream capture the launches
+ *             are replayed through a library-owned hipGraph, under capture they are
+ *             recorded into the caller's graph.
+ * STEPWISE:   like GRAPH but always plain launches (no library-owned graph). */
+#define RTN_MODE_AUTO 0
+#define RTN_MODE_PERSISTENT 1
+#define RTN_MODE_GRAPH 2
+#define RTN_MODE_STEPWISE 3
+
+/*
+ * NativeLstm2 forward.  Replaces the generated op body `c_fw_code`
+ * (returnn/native_op.py:1184-1285) together with `lstm_kernel` (:1081-1121), the
+ * per-step `affine_raw` GEMM (returnn/native_op.cpp:1032-1067), the `H := X` copy and
+ * the zero-initialisation of the outputs done by the generated wrapper
+ * (returnn/torch/util/native_op.py:170-184).
+ *
+ *   X  [T,B,4n]  pre-projected gate inputs; last axis = cell-in | input | forget | output
+ *   W  [n,4n]    recurrent weights, same gate order
+ *   y0 [B,n]     initial output          c0 [B,n] initial cell state (float32)
+ *   i  [T,B]     float32 0/1 mask (right padded batches)
+ *   start, step  host ints; step > 0 visits start, start+step, ...; step < 0 visits
+ *                T-1-start, T-1-start+step, ... (returnn/native_op.py:1253-1259)
+ *   Y  [T,B,n]   output, exactly 0 on masked frames
+ *   C  [T,B,n]   cell states (float32), carried over masked frames
+ *   H  [T,B,4n]  activated gates, also written on masked frames; frames that are
+ *                not visited keep Y = C = 0 and H = X
+ *   d  [B,n]     final cell state (float32) = C of the last visited frame; c0 if T == 0
+ *
+ * All arrays are row-major contiguous and 16-byte aligned.  Returns RTN_OK or an error
+ * code; rtn_last_error() describes the last error of the calling thread.
+ */
+int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const float* c0, const float* i,
+                         int32_t start, int32_t step, void* Y, float* C, void* H, float* d, int64_t T,
+                         int32_t B, int32_t n, int32_t dtype, int32_t mode, void* workspace,
+                         size_t workspace_bytes, void* hip_stream);
+
+/* Bytes of device scratch rtn_native_lstm2_fwd needs for this problem.  Stands in for
+ * the op's `device_malloc` of y_prev (returnn/native_op.py:1244, returnn/native_op.cpp:952-960):
+ * the caller allocates from its own caching allocator instead.  Calls that overlap in
+ * time need distinct workspaces.  Returns 0 on invalid arguments. */
+size_t rtn_native_lstm2_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode);
+
+/* Synchronous check of the last rtn_native_lstm2_fwd that used `workspace`: waits for
+ * `hip_stream`, then returns RTN_OK, RTN_ERR_ABORTED (a bounded wait inside the persistent
+ * kernel expired, outputs are invalid) or RTN_ERR_HIP.  Stands in for HANDLE_LAST_ERROR
+ * after the loop (returnn/native_op.py:1279); optional, for callers that can afford a sync. */
+int rtn_native_lstm2_fwd_status(const void* workspace, void* hip_stream);
+
+/*
+ * Final output per sequence.  Replaces the caller-side `_lstm_last_output`
+ * (returnn/tf/native_op.py:913-929): out[b] = Y[t*, b] for the last visited frame t*
+ * (in processing order) with i[t*, b] != 0, else y0[b].  Y, y0, out have element
+ * type `dtype`; needs no workspace.
+ */
+int rtn_native_lstm2_last_output(const void* Y, const void* y0, const float* i, int32_t start, int32_t step,
+                                 void* out, int64_t T, int32_t B, int32_t n, int32_t dtype, void* hip_stream);
+
+/* Text of the calling thread's last error ("" if none).  Stands in for the message of the
+ * exception TORCH_CHECK raises (returnn/native_op.cpp:660). */
+const char* rtn_last_error(void);
+
+/* The plan the library would use for this problem, as text
+ * ("mode=persistent mt=1 nt=2 groups=1 wgs=256 lds=40960 ..."); for logs and tests.
+ * Counterpart of the reference's compile log next to the .so (returnn/util/native_code_compiler.py:348-352). */
+const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode);
+
+/* ABI version of this header. */
+int rtn_native_lstm2_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* RTN_NATIVE_LSTM2_H */

@@ -53,24 +53,23 @@
  * with transpose flags false and alpha = beta = 1.  The column range is split
  * over `threads` OpenMP threads (the reference's CPU GEMM back-end is a
  * multi-threaded contraction, returnn/native_op.cpp:557-620); with threads <= 1
- * it is a plain sequential loop.  Accumulation order over k is ascending and
- * identical for every thread count, so results do not depend on `threads`. */
+ * it is a plain sequential loop.  Every C element is updated over ascending k,
+ * whatever the thread count, so results do not depend on `threads`. */
 #define DEFINE_AFFINE(NAME, REAL)                                                     \
   static void NAME(const REAL* A, int a0, int a1, const REAL* Bm, int b1, REAL* C,    \
                    int threads) {                                                     \
-    const int blk = 256;                                                              \
+    const int blk = 128;                                                              \
     const int nblk = (b1 + blk - 1) / blk;                                            \
     (void)threads;                                                                    \
     _Pragma("omp parallel for schedule(static) num_threads(threads) if (threads > 1)") \
     for (int jb = 0; jb < nblk; ++jb) {                                               \
       const int j0 = jb * blk;                                                        \
       const int j1 = (j0 + blk < b1) ? j0 + blk : b1;                                 \
-      for (int r = 0; r < a0; ++r) {                                                  \
-        REAL* c = C + (size_t)r * b1;                                                 \
-        const REAL* a = A + (size_t)r * a1;                                           \
-        for (int k = 0; k < a1; ++k) {                                                \
-          const REAL av = a[k];                                                       \
-          const REAL* w = Bm + (size_t)k * b1;                                        \
+      for (int k = 0; k < a1; ++k) {                                                  \
+        const REAL* w = Bm + (size_t)k * b1;                                          \
+        for (int r = 0; r < a0; ++r) {                                                \
+          REAL* c = C + (size_t)r * b1;                                               \
+          const REAL av = A[(size_t)r * a1 + k];                                      \
           for (int j = j0; j < j1; ++j) c[j] += av * w[j];                            \
         }                                                                             \
       }                                                                               \
@@ -191,6 +190,14 @@ DEFINE_FWD(lstm2_oracle_fwd_f64, double, affine_f64, pointwise_f64)
 
 DEFINE_LAST_OUTPUT(lstm2_oracle_last_output_f32, float)
 DEFINE_LAST_OUTPUT(lstm2_oracle_last_output_f64, double)
+
+/* One pointwise step on its own (returnn/native_op.py:1081-1121), for a driver that does the
+ * recurrent GEMM with a BLAS, as the reference's CPU path does (returnn/native_op.cpp:535-620). */
+void lstm2_oracle_pointwise_f32(int32_t n_batch, int32_t n_cells, const float* mask, float* h,
+                                const float* prev_y, const float* prev_c, float* y, float* c,
+                                float* y_prev_out) {
+  pointwise_f32(n_batch, n_cells, mask, h, prev_y, prev_c, y, c, y_prev_out);
+}
 
 int lstm2_oracle_max_threads(void) {
 #ifdef _OPENMP

@@ -47,6 +47,9 @@ def _load():
             last.restype = ctypes.c_int
             last.argtypes = [ptr] * 3 + [ctypes.c_int32, ctypes.c_int32, ptr, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
         lib.lstm2_oracle_max_threads.restype = ctypes.c_int
+        fp = ctypes.POINTER(ctypes.c_float)
+        lib.lstm2_oracle_pointwise_f32.restype = None
+        lib.lstm2_oracle_pointwise_f32.argtypes = [ctypes.c_int32, ctypes.c_int32] + [fp] * 7
         _lib = lib
     return _lib
 
@@ -146,3 +149,45 @@ def lstm_last_output(Y, y0, i, start: int = 0, step: int = 1, *, dtype=numpy.flo
     if rc != 0:
         raise ValueError("oracle: last_output error code %i" % rc)
     return out
+
+
+def native_lstm2_fwd_blas(X, W, y0, c0, i, start: int = 0, step: int = 1):
+    """
+    Same op, float32, with the structure of the reference's CPU path: per visited frame one SGEMM
+    ``H[t] += y_prev . W`` through the BLAS numpy links (multi-threaded, like the reference's GEMM back-ends,
+    returnn/native_op.cpp:535-620) followed by the sequential pointwise kernel of ``oracle/lstm2_oracle.c``.
+    This is the variant the benchmark times as the CPU baseline; it agrees with :func:`native_lstm2_fwd`
+    up to the summation order inside the BLAS.
+
+    :return: Y, C, H, d, y_last as in :func:`native_lstm2_fwd`
+    """
+    f32 = numpy.float32
+    i = numpy.ascontiguousarray(i, dtype=f32)
+    y0 = numpy.ascontiguousarray(y0, dtype=f32)
+    T, B = i.shape
+    n = y0.shape[1]
+    X = _prep(X, f32, (T, B, 4 * n), "X")
+    W = _prep(W, f32, (n, 4 * n), "W")
+    c0 = _prep(c0, f32, (B, n), "c0")
+    Y = numpy.zeros((T, B, n), dtype=f32)
+    C = numpy.zeros((T, B, n), dtype=f32)
+    d = numpy.zeros((B, n), dtype=f32)
+    if T == 0:
+        return Y, C, numpy.zeros((T, B, 4 * n), dtype=f32), c0.copy(), y0.copy()
+    if not (0 <= start < T) or step == 0:
+        raise ValueError("oracle: need 0 <= start < T and step != 0 (start=%r, step=%r, T=%r)" % (start, step, T))
+    H = X.copy()
+    y_prev = numpy.empty((B, n), dtype=f32)
+    first, end = (start, T - 1) if step > 0 else (T - start - 1, 0)
+    pointwise = _load().lstm2_oracle_pointwise_f32
+    fp = ctypes.POINTER(ctypes.c_float)
+    ptr = lambda a: a.ctypes.data_as(fp)  # noqa: E731
+    t = first
+    while (t <= end) if step > 0 else (t >= end):
+        y_in = y0 if t == first else y_prev
+        c_in = c0 if t == first else C[t - step]
+        H[t] += y_in @ W
+        pointwise(B, n, ptr(i[t]), ptr(H[t]), ptr(y_in), ptr(c_in), ptr(Y[t]), ptr(C[t]), ptr(y_prev))
+        t += step
+    d[...] = C[t - step]
+    return Y, C, H, d, y_prev

@@ -1,0 +1,485 @@
+// gfx950 (CDNA4) kernels of the NativeLstm2 forward op.
+//
+// Semantics follow the reference operator: host loop returnn/native_op.py:1184-1285,
+// pointwise step returnn/native_op.py:1081-1121, recurrent term H[t] += y_prev . W
+// (returnn/native_op.cpp:1032-1067).  The structure does not: the recurrent GEMM, the gate
+// non-linearities, the cell update and the mask are one fused step, the cell state and
+// the last valid output of every (sequence, cell) live in registers of the thread that
+// owns that pair, and in the persistent kernel the recurrent weights stay in LDS for
+// all time steps.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "lstm2_params.h"
+
+namespace rtn {
+
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4;
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+
+constexpr int kWgThreads = 256;  // 4 wavefronts of 64
+constexpr int kWaves = 4;
+constexpr int kFragBytes = 16;   // one MFMA operand fragment per lane
+constexpr int kTileBytes = 64 * kFragBytes;
+constexpr unsigned kBufFlags = 0x00020000;  // raw buffer descriptor word 3 (32-bit data format)
+constexpr int kAuxDevice = 16;  // cache policy: device scope (sc1) for raw buffer loads/stores
+
+// Per element type: how many elements fill one 16-byte fragment (KE) and how many k
+// indices one macro step of the MFMA loop consumes (KM = 4 lane groups * KE).
+template <typename AT>
+struct Elem;
+
+template <>
+struct Elem<float> {
+  static constexpr int KE = 4;
+  static constexpr int KM = 16;
+  static __device__ __forceinline__ float load(const void* p, size_t i) { return ((const float*)p)[i]; }
+  static __device__ __forceinline__ void store(void* p, size_t i, float v) { ((float*)p)[i] = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+  // D[16x16] += A[16x16] * B[16x16] as four 16x16x4 MFMAs, one per fragment element.
+  static __device__ __forceinline__ f32x4 mma(i32x4 a, i32x4 b, f32x4 c) {
+    f32x4 af = __builtin_bit_cast(f32x4, a), bf = __builtin_bit_cast(f32x4, b);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[0], bf[0], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[1], bf[1], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[2], bf[2], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[3], bf[3], c, 0, 0, 0);
+    return c;
+  }
+  static __device__ __forceinline__ void store_coherent(__amdgpu_buffer_rsrc_t rs, unsigned off, float v) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rs, off, 0, kAuxDevice);
+  }
+};
+
+template <>
+struct Elem<__bf16> {
+  static constexpr int KE = 8;
+  static constexpr int KM = 32;
+  static __device__ __forceinline__ float load(const void* p, size_t i) { return (float)((const __bf16*)p)[i]; }
+  static __device__ __forceinline__ void store(void* p, size_t i, float v) { ((__bf16*)p)[i] = (__bf16)v; }
+  static __device__ __forceinline__ float round(float v) { return (float)(__bf16)v; }
+  static __device__ __forceinline__ f32x4 mma(i32x4 a, i32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                   0, 0);
+  }
+  static __device__ __forceinline__ void store_coherent(__amdgpu_buffer_rsrc_t rs, unsigned off, float v) {
+    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, (__bf16)v), rs, off, 0, kAuxDevice);
+  }
+};
+
+// sigmoid exactly as the reference writes it (returnn/native_op.py:1102-1104)
+__device__ __forceinline__ float sigmoid_ref(float x) { return 1.f / (1.f + expf(-x)); }
+
+// Frame visited at step s.
+__device__ __forceinline__ long long frame_of(const Lstm2Params& p, int s) {
+  return (long long)p.first + (long long)s * p.step;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Small helper kernels
+// ---------------------------------------------------------------------------------------------
+
+// T == 0: d := c0 (returnn/native_op.py:1236-1237)
+__global__ void k_copy_f32(const float* __restrict__ src, float* __restrict__ dst, long long count) {
+  for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < count;
+       i += (long long)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
+// Frames the loop does not visit keep Y = C = 0 and H = X (zero-initialised outputs plus the
+// H := X copy of the reference, returnn/native_op.py:1247).  Only launched when start > 0 or |step| > 1.
+template <typename AT>
+__global__ void k_fill_unvisited(Lstm2Params p) {
+  const long long bn = (long long)p.B * p.n;
+  const long long per_frame = bn * 4;
+  const long long total = p.T * per_frame;
+  for (long long idx = blockIdx.x * (long long)blockDim.x + threadIdx.x; idx < total;
+       idx += (long long)gridDim.x * blockDim.x) {
+    const long long t = idx / per_frame;
+    const long long delta = t - p.first;
+    bool visited;
+    if (p.step > 0)
+      visited = delta >= 0 && (delta % p.step) == 0;
+    else
+      visited = delta <= 0 && ((-delta) % (-p.step)) == 0;
+    if (visited) continue;
+    ((AT*)p.H)[idx] = ((const AT*)p.X)[idx];
+    const long long rem = idx - t * per_frame;
+    if (rem < bn) {
+      Elem<AT>::store(p.Y, t * bn + rem, 0.f);
+      p.C[t * bn + rem] = 0.f;
+    }
+  }
+}
+
+// Before the MFMA kernels: clears status and flags, writes y0 into buffer 0 of every group's
+// hidden-state exchange area (in B-operand order) and packs W into A-operand order.
+//
+// Packed W: fragment (m, sm, lane) holds, for row i = lane%16 of M-tile m and lane group
+// kg = lane/16, the KE elements W[KM*sm + KE*kg + e][gate*n + 4*m + cell] with
+// cell = i/4, gate = i%4 -- i.e. the 16 rows of an M-tile are the 4 gates of 4 adjacent cells,
+// so that after the MFMA one lane holds all four gate pre-activations of one (cell, sequence).
+template <typename AT>
+__global__ void k_prepare_mfma(Lstm2Params p, int n_flags) {
+  constexpr int KE = Elem<AT>::KE;
+  constexpr int KM = Elem<AT>::KM;
+  const long long gtid = blockIdx.x * (long long)blockDim.x + threadIdx.x;
+  const long long gsz = (long long)gridDim.x * blockDim.x;
+  for (long long i = gtid; i < 64; i += gsz) p.status[i] = 0;
+  for (long long i = gtid; i < n_flags; i += gsz) p.flags[i] = 0;
+  // y0 -> hx[g][0][kb][b_local][e]
+  const long long bn = (long long)p.B * p.n;
+  const long long hx_buf = (long long)p.n * p.Bp;  // elements of one buffer
+  for (long long idx = gtid; idx < bn; idx += gsz) {
+    const int b = (int)(idx / p.n), c = (int)(idx % p.n);
+    const int g = b / p.Bg, bl = b % p.Bg;
+    const long long dst = ((long long)g * 2) * hx_buf + ((long long)(c / KE) * p.Bp + bl) * KE + (c % KE);
+    ((AT*)p.hx)[dst] = ((const AT*)p.y0)[idx];
+  }
+  // W -> Wp
+  const int S = p.n / KM;
+  const long long n_frag = (long long)(p.n / 4) * S * 64;
+  for (long long f = gtid; f < n_frag; f += gsz) {
+    const int lane = (int)(f & 63);
+    const long long ms = f >> 6;
+    const int sm = (int)(ms % S);
+    const int m = (int)(ms / S);
+    const int i = lane & 15, kg = lane >> 4;
+    const int col = (i & 3) * p.n + 4 * m + (i >> 2);
+    const int k0 = KM * sm + KE * kg;
+    AT* dst = (AT*)p.Wp + f * KE;
+#pragma unroll
+    for (int e = 0; e < KE; ++e) dst[e] = ((const AT*)p.W)[(long long)(k0 + e) * 4 * p.n + col];
+  }
+}
+
+// Clears the status word for the generic path.
+__global__ void k_clear_status(unsigned* status) {
+  if (threadIdx.x < 64) status[threadIdx.x] = 0;
+}
+
+// Caller-side final output (returnn/tf/native_op.py:913-929): one workgroup per sequence finds the
+// last visited frame (in processing order) with a non-zero mask and copies that row of Y, else y0.
+template <typename AT>
+__global__ void k_last_output(const void* Y, const void* y0, const float* mask, void* out, long long T, int B, int n,
+                              int first, int step, int nsteps) {
+  __shared__ int s_last;
+  const int b = blockIdx.x;
+  if (threadIdx.x == 0) s_last = -1;
+  __syncthreads();
+  int last = -1;
+  for (int s = threadIdx.x; s < nsteps; s += blockDim.x) {
+    const long long t = (long long)first + (long long)s * step;
+    if ((int)mask[t * B + b] != 0) last = s;
+  }
+  if (last >= 0) atomicMax(&s_last, last);
+  __syncthreads();
+  last = s_last;
+  const AT* src = (last >= 0) ? (const AT*)Y + (((long long)first + (long long)last * step) * B + b) * n
+                              : (const AT*)y0 + (long long)b * n;
+  for (int j = threadIdx.x; j < n; j += blockDim.x) ((AT*)out)[(long long)b * n + j] = src[j];
+}
+
+// ---------------------------------------------------------------------------------------------
+// Generic per-step kernel: any B and n, one thread per (sequence, cell).  Accumulates X + y.W
+// over ascending k in float32, the order of a plain sequential GEMM.
+// Step s reads the carry buffer (s & 1) (y0 at s == 0) and writes buffer ((s + 1) & 1).
+// ---------------------------------------------------------------------------------------------
+template <typename AT>
+__global__ void k_step_generic(Lstm2Params p, int s) {
+  const long long bn = (long long)p.B * p.n;
+  const long long idx = blockIdx.x * (long long)blockDim.x + threadIdx.x;
+  if (idx >= bn) return;
+  const int n = p.n;
+  const int b = (int)(idx / n), j = (int)(idx % n);
+  const long long t = frame_of(p, s);
+  const void* y_in = (s == 0) ? p.y0 : (const void*)((const AT*)p.ycarry + (size_t)(s & 1) * bn);
+  void* y_out = (void*)((AT*)p.ycarry + (size_t)((s + 1) & 1) * bn);
+  const float* c_in = (s == 0) ? p.c0 : p.C + (t - p.step) * bn;
+  const size_t xoff = ((size_t)t * p.B + b) * 4 * n + j;
+  float g0 = Elem<AT>::load(p.X, xoff);
+  float g1 = Elem<AT>::load(p.X, xoff + n);
+  float g2 = Elem<AT>::load(p.X, xoff + 2 * (size_t)n);
+  float g3 = Elem<AT>::load(p.X, xoff + 3 * (size_t)n);
+  const size_t yrow = (size_t)b * n;
+  for (int k = 0; k < n; ++k) {
+    const float yk = Elem<AT>::load(y_in, yrow + k);
+    const size_t w = (size_t)k * 4 * n + j;
+    g0 += yk * Elem<AT>::load(p.W, w);
+    g1 += yk * Elem<AT>::load(p.W, w + n);
+    g2 += yk * Elem<AT>::load(p.W, w + 2 * (size_t)n);
+    g3 += yk * Elem<AT>::load(p.W, w + 3 * (size_t)n);
+  }
+  const float m = p.mask[t * p.B + b];
+  const float a0 = tanhf(g0), a1 = sigmoid_ref(g1), a2 = sigmoid_ref(g2), a3 = sigmoid_ref(g3);
+  Elem<AT>::store(p.H, xoff, a0);
+  Elem<AT>::store(p.H, xoff + n, a1);
+  Elem<AT>::store(p.H, xoff + 2 * (size_t)n, a2);
+  Elem<AT>::store(p.H, xoff + 3 * (size_t)n, a3);
+  const float pc = c_in[idx];
+  const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
+  p.C[t * bn + idx] = c;
+  const float y = Elem<AT>::round(tanhf(c) * a3 * m);
+  Elem<AT>::store(p.Y, t * bn + idx, y);
+  Elem<AT>::store(y_out, idx, y + Elem<AT>::load(y_in, idx) * (1.f - m));
+  if (s == p.nsteps - 1) p.d[idx] = c;
+}
+
+// ---------------------------------------------------------------------------------------------
+// MFMA kernel.  Grid = groups * wgs_per_group workgroups of 256 threads.
+//
+// A group owns Bg batch rows; inside it workgroup rank r owns the MT*4 cells
+// [4*MT*r, 4*MT*(r+1)) = MT M-tiles of 16 gate columns.  Per step every workgroup computes
+// G^T[16*MT, 16*NT] = Wslice^T[16*MT, n] . h^T[n, 16*NT] with the k range dealt round-robin
+// to the 4 wavefronts (macro step sm belongs to wave sm % 4), sums the four partial tiles
+// through LDS, and the thread that owns (sequence, cell) applies gates, cell update and mask
+// and publishes its new hidden value in B-operand order for everybody's next step.
+//
+// s_begin/s_end: steps run by this launch.  With s_end - s_begin > 1 the launch must be
+// co-resident (cooperative launch): steps are separated by a flag wait, bounded by
+// timeout_ticks; an expired wait sets status[0] and every later wait returns at once,
+// so the grid always drains.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void map_block(const Lstm2Params& p, int bid, int& g, int& r) {
+  const int NG = p.groups, G = p.wgs_per_group, X = p.xcds;
+  // Consecutive workgroup ids go round-robin over the XCDs (each with its own L2).  Put a
+  // group on as few XCDs as possible and give the workgroups of one XCD adjacent cells, so that
+  // their partial cache-line reads of X and writes of Y/C/H meet in that XCD's L2.
+  if (X > 1 && NG <= X && X % NG == 0 && G % (X / NG) == 0) {
+    const int xpg = X / NG;
+    const int x = bid % X, q = bid / X;
+    g = x / xpg;
+    r = (x % xpg) * (G / xpg) + q;
+  } else if (X > 1 && NG % X == 0) {
+    g = bid % NG;
+    r = bid / NG;
+  } else {
+    g = bid / G;
+    r = bid % G;
+  }
+}
+
+__device__ __forceinline__ void wait_flags(const Lstm2Params& p, const unsigned* flags, int G, unsigned need,
+                                           int lane) {
+  unsigned long long t0 = 0;
+  unsigned spins = 0;
+  for (;;) {
+    bool ok = true;
+    for (int r = lane; r < G; r += 64)
+      ok = ok && (__hip_atomic_load(flags + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= need);
+    if (__all(ok)) break;
+    if ((spins++ & 31u) == 0) {
+      if (__hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+      const unsigned long long now = wall_clock64();
+      if (spins == 1) {
+        t0 = now;
+      } else if (now - t0 > p.timeout_ticks) {
+        __hip_atomic_store(p.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
+  if (p.sync_policy & kAcquireFence) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+}
+
+template <typename AT, int MT, int NT>
+__global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, const int s_begin, const int s_end) {
+  using E = Elem<AT>;
+  constexpr int KE = E::KE;
+  constexpr int KM = E::KM;
+  constexpr int TILES = MT * NT;
+  constexpr int EPT = (TILES + kWaves - 1) / kWaves;  // epilogue tiles per thread
+  constexpr int U = (NT >= 4) ? 4 : 8;                // macro steps whose h fragments are in flight together
+
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = p.n, S = n / KM;
+  i32x4* Wl = (i32x4*)smem;                                  // [MT][S][64] fragments
+  f32x4* red = (f32x4*)(smem + (size_t)MT * S * kTileBytes);  // [kWaves][TILES][64]
+
+  int g, r;
+  map_block(p, blockIdx.x, g, r);
+  const int b_base = g * p.Bg;
+  const int rows = min(p.Bg, p.B - b_base);
+  const bool persist = (s_end - s_begin) > 1;
+  const long long bn = (long long)p.B * n;
+  const size_t hx_buf_bytes = (size_t)n * p.Bp * sizeof(AT);
+  unsigned char* hx_g = (unsigned char*)p.hx + (size_t)g * 2 * hx_buf_bytes;
+  const unsigned* flags_g = p.flags + (size_t)g * p.wgs_per_group;
+
+  // W slice of this workgroup: global (already in fragment order) -> LDS, once per launch.
+  {
+    const i32x4* src = (const i32x4*)p.Wp + (size_t)r * MT * S * 64;
+    for (int i = tid; i < MT * S * 64; i += kWgThreads) Wl[i] = src[i];
+  }
+
+  // State of the (sequence, cell) pairs this thread owns.
+  float c_state[EPT], h_prev[EPT];
+  int e_b[EPT], e_cell[EPT];
+  bool e_valid[EPT];
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int e = wave + kWaves * j;
+    const int mt = e / NT, nt = e % NT;
+    const int bl = 16 * nt + (lane & 15);
+    e_cell[j] = 4 * (r * MT + mt) + (lane >> 4);
+    e_b[j] = bl;
+    e_valid[j] = (e < TILES) && (bl < rows);
+    c_state[j] = 0.f;
+    h_prev[j] = 0.f;
+    if (e_valid[j]) {
+      const long long bc = (long long)(b_base + bl) * n + e_cell[j];
+      if (s_begin == 0) {
+        c_state[j] = p.c0[bc];
+        h_prev[j] = E::load(p.y0, bc);
+      } else {
+        c_state[j] = p.C[(frame_of(p, s_begin) - p.step) * bn + bc];
+        const size_t ho = ((size_t)(e_cell[j] / KE) * p.Bp + bl) * KE + (e_cell[j] % KE);
+        h_prev[j] = E::load(hx_g + (size_t)(s_begin & 1) * hx_buf_bytes, ho);
+      }
+    }
+  }
+  __syncthreads();
+
+  const int kg = lane >> 4, jl = lane & 15;
+
+  for (int s = s_begin; s < s_end; ++s) {
+    const long long t = frame_of(p, s);
+
+    // Gate inputs and mask of this step: independent of the recurrence, issued before the wait.
+    float xg[EPT][4], msk[EPT];
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      msk[j] = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) xg[j][q] = 0.f;
+      if (e_valid[j]) {
+        const size_t xo = ((size_t)t * p.B + (b_base + e_b[j])) * 4 * n + e_cell[j];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) xg[j][q] = E::load(p.X, xo + (size_t)q * n);
+        msk[j] = p.mask[t * p.B + b_base + e_b[j]];
+      }
+    }
+
+    if (persist && s > s_begin) wait_flags(p, flags_g, p.wgs_per_group, (unsigned)s, lane);
+
+    // Recurrent GEMM: this wave's share of k.
+    f32x4 acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const unsigned char* hx_cur = hx_g + (size_t)(s & 1) * hx_buf_bytes;
+    __amdgpu_buffer_rsrc_t hx_rs = __builtin_amdgcn_make_buffer_rsrc((void*)hx_cur, 0, 0x7fffffff, kBufFlags);
+    const bool ld_coherent = persist && (p.sync_policy & kLoadCoherent);
+    for (int sm0 = wave; sm0 < S; sm0 += kWaves * U) {
+      i32x4 bf[U][NT];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int sm = sm0 + kWaves * u;
+        if (sm < S) {
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            const unsigned off = (unsigned)(((4 * sm + kg) * p.Bp + 16 * nt + jl) * kFragBytes);
+            if (ld_coherent)
+              bf[u][nt] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(hx_rs, off, 0, kAuxDevice));
+            else
+              bf[u][nt] = *(const i32x4*)(hx_cur + off);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int sm = sm0 + kWaves * u;
+        if (sm < S) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const i32x4 af = Wl[(mt * S + sm) * 64 + lane];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(af, bf[u][nt], acc[mt][nt]);
+          }
+        }
+      }
+    }
+
+    // Partial tiles -> LDS.
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) red[(wave * TILES + mt * NT + nt) * 64 + lane] = acc[mt][nt];
+    __syncthreads();
+
+    // Epilogue: gates, cell update, mask; publish the new hidden value first (critical path).
+    unsigned char* hx_nxt = hx_g + (size_t)((s + 1) & 1) * hx_buf_bytes;
+    __amdgpu_buffer_rsrc_t nx_rs = __builtin_amdgcn_make_buffer_rsrc((void*)hx_nxt, 0, 0x7fffffff, kBufFlags);
+    const bool st_coherent = persist && (p.sync_policy & kStoreCoherent);
+    float a_out[EPT][4], y_out[EPT];
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      const int e = wave + kWaves * j;
+      if (e < TILES) {
+        f32x4 gsum = red[(0 * TILES + e) * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) gsum += red[(w * TILES + e) * 64 + lane];
+        const float m = msk[j];
+        const float a0 = tanhf(gsum[0] + xg[j][0]);
+        const float a1 = sigmoid_ref(gsum[1] + xg[j][1]);
+        const float a2 = sigmoid_ref(gsum[2] + xg[j][2]);
+        const float a3 = sigmoid_ref(gsum[3] + xg[j][3]);
+        const float pc = c_state[j];
+        const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
+        const float y = E::round(tanhf(c) * a3 * m);
+        const float hn = E::round(y + h_prev[j] * (1.f - m));
+        c_state[j] = c;
+        h_prev[j] = hn;
+        y_out[j] = y;
+        a_out[j][0] = a0;
+        a_out[j][1] = a1;
+        a_out[j][2] = a2;
+        a_out[j][3] = a3;
+        if (e_valid[j]) {
+          const unsigned ho =
+              (unsigned)((((e_cell[j] / KE) * p.Bp + e_b[j]) * KE + (e_cell[j] % KE)) * (int)sizeof(AT));
+          if (st_coherent)
+            E::store_coherent(nx_rs, ho, hn);
+          else
+            E::store(hx_nxt, ho / sizeof(AT), hn);
+        }
+      }
+    }
+    if (persist) {
+      // Every thread's hidden-state stores have left the CU before the workgroup's flag goes up.
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();  // also frees `red` for the next step
+    if (persist && tid == 0) {
+      if (p.sync_policy & kReleaseFence) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      __hip_atomic_store(p.flags + (size_t)g * p.wgs_per_group + r, (unsigned)(s + 1), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // Outputs of the op (off the critical path).
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      if (e_valid[j]) {
+        const long long bc = (long long)(b_base + e_b[j]) * n + e_cell[j];
+        const size_t xo = ((size_t)t * p.B + (b_base + e_b[j])) * 4 * n + e_cell[j];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) E::store(p.H, xo + (size_t)q * n, a_out[j][q]);
+        p.C[t * bn + bc] = c_state[j];
+        E::store(p.Y, t * bn + bc, y_out[j]);
+      }
+    }
+  }
+
+  if (s_end == p.nsteps) {
+#pragma unroll
+    for (int j = 0; j < EPT; ++j)
+      if (e_valid[j]) p.d[(long long)(b_base + e_b[j]) * n + e_cell[j]] = c_state[j];
+  }
+}
+
+}  // namespace rtn

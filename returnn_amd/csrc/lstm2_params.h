@@ -1,0 +1,51 @@
+// Parameter block shared by the host driver and the gfx950 kernels of the NativeLstm2 forward op.
+#pragma once
+
+#include <stdint.h>
+
+namespace rtn {
+
+// How the hidden state is made visible between workgroups in the persistent kernel.
+// A valid policy has (store_coherent || release_fence) and (load_coherent || acquire_fence).
+enum SyncBits : int {
+  kStoreCoherent = 1,  // publish h with device-scope write-through stores
+  kReleaseFence = 2,   // device-scope release fence (L2 write-back) before the flag store
+  kLoadCoherent = 4,   // read h with device-scope loads that bypass non-coherent caches
+  kAcquireFence = 8,   // device-scope acquire fence (cache invalidate) after the flag wait
+};
+
+struct Lstm2Params {
+  // inputs (device)
+  const void* X;      // [T,B,4n] AT
+  const void* W;      // [n,4n] AT (row major, as given by the caller)
+  const void* y0;     // [B,n] AT
+  const float* c0;    // [B,n]
+  const float* mask;  // [T,B]
+  // outputs (device)
+  void* Y;   // [T,B,n] AT
+  float* C;  // [T,B,n]
+  void* H;   // [T,B,4n] AT
+  float* d;  // [B,n]
+  // workspace sections (device)
+  unsigned* status;  // [64]   status[0] != 0: a bounded wait expired
+  unsigned* flags;   // [groups*wgs_per_group] last published step (+1) of each workgroup
+  void* hx;          // [groups][2][n/KE][Bp][KE] AT: hidden state in MFMA B-operand order, double buffered
+  void* Wp;          // [n/4][S][64][16 bytes]: W in MFMA A-operand order
+  void* ycarry;      // [2][B][n] AT: hidden-state carry of the generic per-step kernels
+  // sizes
+  long long T;
+  int B, n;
+  int first;   // first visited frame
+  int step;    // signed stride between visited frames
+  int nsteps;  // number of visited frames
+  // decomposition of the MFMA kernels
+  int groups;         // independent batch groups
+  int wgs_per_group;  // workgroups per group (each owns MT*4 cells)
+  int Bg;             // batch rows per group
+  int Bp;             // rows of one hx buffer (= 16*NT)
+  int xcds;           // XCDs assumed for the blockIdx -> (group, rank) mapping
+  int sync_policy;    // SyncBits
+  unsigned long long timeout_ticks;  // bound of one flag wait, in 100 MHz wall-clock ticks
+};
+
+}  // namespace rtn

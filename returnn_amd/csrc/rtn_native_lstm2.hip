@@ -1,0 +1,553 @@
+// Host driver and C ABI of the gfx950 NativeLstm2 forward library.
+//
+// Validates the operator contract (returnn/native_op.py:1054-1068, 1203-1234, 1249-1252), picks a
+// decomposition, lays out the caller's workspace and enqueues the kernels of lstm2_kernels.h on the
+// caller's stream.  No device memory is allocated here and the stream is never synchronised, so a
+// call can sit inside a captured graph (per-step modes) like the reference's ops do
+// (returnn/torch/util/graph_capture.py:1-80).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <list>
+#include <mutex>
+#include <string>
+
+#include "../../include/rtn_native_lstm2.h"
+#include "lstm2_kernels.h"
+
+namespace rtn {
+namespace {
+
+thread_local std::string g_last_error;
+thread_local std::string g_plan_text;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+#define RTN_HIP(call)                                                                                  \
+  do {                                                                                                 \
+    hipError_t err_ = (call);                                                                          \
+    if (err_ != hipSuccess)                                                                            \
+      return fail(RTN_ERR_HIP, "NativeLstm2: HIP error '%s' in %s (%s:%d)", hipGetErrorString(err_), #call, \
+                  __FILE__, __LINE__);                                                                 \
+  } while (0)
+
+long env_long(const char* name, long dflt) {
+  const char* v = getenv(name);
+  if (!v || !*v) return dflt;
+  char* end = nullptr;
+  long r = strtol(v, &end, 0);
+  return (end && *end == 0) ? r : dflt;
+}
+
+struct DeviceInfo {
+  int cus = 256;
+  int xcds = 8;
+  size_t lds_per_wg = 160 * 1024;
+  bool cooperative = true;
+  bool valid = false;
+};
+
+// Properties of the current device; falls back to MI355X's published figures when no device is
+// visible (the workspace-size and plan queries must work on a build host without a GPU).
+DeviceInfo device_info() {
+  static std::mutex mu;
+  static DeviceInfo cache[64];
+  int dev = 0;
+  DeviceInfo fallback;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    (void)hipGetLastError();
+    return fallback;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (!cache[dev].valid) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+      (void)hipGetLastError();
+      return fallback;
+    }
+    DeviceInfo di;
+    di.cus = prop.multiProcessorCount;
+    di.xcds = (di.cus % 8 == 0 && di.cus >= 64) ? 8 : 1;
+    di.lds_per_wg = prop.sharedMemPerBlockOptin ? (size_t)prop.sharedMemPerBlockOptin : (size_t)prop.sharedMemPerBlock;
+    if (di.lds_per_wg < (size_t)prop.sharedMemPerBlock) di.lds_per_wg = prop.sharedMemPerBlock;
+    di.cooperative = prop.cooperativeLaunch != 0;
+    di.valid = true;
+    cache[dev] = di;
+  }
+  return cache[dev];
+}
+
+enum PlanKind { kPlanEmpty, kPlanGeneric, kPlanMfma };
+
+struct Plan {
+  PlanKind kind = kPlanGeneric;
+  int mode = RTN_MODE_STEPWISE;  // resolved: PERSISTENT, GRAPH or STEPWISE
+  int MT = 1, NT = 1;
+  int groups = 1, wgs_per_group = 1, Bg = 1, Bp = 16;
+  size_t lds_bytes = 0;
+  // workspace layout (byte offsets)
+  size_t off_status = 0, off_flags = 0, off_hx = 0, off_wp = 0, off_ycarry = 0, total = 0;
+  int n_flags = 0;
+};
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+size_t esize(int dtype) { return dtype == RTN_DTYPE_BF16 ? 2 : 4; }
+int round_nt(int nt) { return nt <= 1 ? 1 : (nt <= 2 ? 2 : 4); }
+
+size_t mfma_lds_bytes(int n, int dtype, int MT, int NT) {
+  const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
+  return (size_t)MT * (n / KM) * kTileBytes + (size_t)kWaves * MT * NT * kTileBytes;
+}
+
+// Chooses the decomposition.  `want_mode` is the caller's mode; `capturing` says the stream is
+// under capture (a cooperative launch cannot be recorded).  Returns false with a reason when
+// mode == PERSISTENT is impossible.
+bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing, Plan* out, std::string* why) {
+  Plan pl;
+  const DeviceInfo di = device_info();
+  const size_t es = esize(dtype);
+  if (T == 0 || B == 0 || n == 0) {
+    pl.kind = kPlanEmpty;
+    pl.mode = RTN_MODE_STEPWISE;
+    pl.total = 256;
+    *out = pl;
+    return true;
+  }
+  const bool mfma_shape = (n % 32) == 0;
+  const long force_generic = env_long("RTN_LSTM2_FORCE_GENERIC", 0);
+  bool persistent_ok = false;
+  if (mfma_shape && !force_generic) {
+    pl.kind = kPlanMfma;
+    // Persistent candidates: smallest MT whose grid fits the device and whose W slice fits LDS.
+    const long env_mt = env_long("RTN_LSTM2_MT", 0);
+    const long env_groups = env_long("RTN_LSTM2_GROUPS", 0);
+    if (want_mode == RTN_MODE_AUTO || want_mode == RTN_MODE_PERSISTENT) {
+      for (int MT : {1, 2, 4}) {
+        if (env_mt && MT != env_mt) continue;
+        if ((n / 4) % MT) continue;
+        const int G = n / (4 * MT);
+        if (G > di.cus) continue;
+        int max_groups = di.cus / G;
+        int groups = std::min(max_groups, (B + 15) / 16);
+        if (env_groups) groups = (int)std::min<long>(env_groups, max_groups);
+        groups = std::max(1, std::min(groups, B));
+        int Bg = (B + groups - 1) / groups;
+        groups = (B + Bg - 1) / Bg;
+        int NT = round_nt((Bg + 15) / 16);
+        if ((Bg + 15) / 16 > 4) continue;
+        const size_t lds = mfma_lds_bytes(n, dtype, MT, NT);
+        if (lds > di.lds_per_wg) continue;
+        pl.MT = MT;
+        pl.NT = NT;
+        pl.groups = groups;
+        pl.wgs_per_group = G;
+        pl.Bg = Bg;
+        pl.lds_bytes = lds;
+        persistent_ok = true;
+        break;
+      }
+      if (!persistent_ok && why) *why = "no decomposition keeps W on chip with all workgroups co-resident";
+    }
+    if (persistent_ok && capturing) {
+      persistent_ok = false;
+      if (why) *why = "the stream is being captured; a cooperative launch cannot be recorded";
+    }
+    if (persistent_ok && !di.cooperative) {
+      persistent_ok = false;
+      if (why) *why = "the device does not support cooperative launches";
+    }
+    if (!persistent_ok) {
+      // Per-step launches have no co-residency limit: 4 cells per workgroup, groups of <= 64 rows.
+      int MT = 1;
+      if (mfma_lds_bytes(n, dtype, 1, 4) > di.lds_per_wg) {
+        pl.kind = kPlanGeneric;  // a W slice of 16 columns does not fit LDS (n far beyond the target sizes)
+      } else {
+        int groups = (B + 63) / 64;
+        int Bg = (B + groups - 1) / groups;
+        groups = (B + Bg - 1) / Bg;
+        pl.MT = MT;
+        pl.NT = round_nt((Bg + 15) / 16);
+        pl.groups = groups;
+        pl.wgs_per_group = n / 4;
+        pl.Bg = Bg;
+        pl.lds_bytes = mfma_lds_bytes(n, dtype, pl.MT, pl.NT);
+      }
+    }
+  } else {
+    pl.kind = kPlanGeneric;
+    if (why) *why = mfma_shape ? "RTN_LSTM2_FORCE_GENERIC is set" : "n is not a multiple of 32";
+  }
+  if (want_mode == RTN_MODE_PERSISTENT && !persistent_ok) return false;
+  if (persistent_ok)
+    pl.mode = RTN_MODE_PERSISTENT;
+  else if (want_mode == RTN_MODE_STEPWISE || capturing)
+    pl.mode = RTN_MODE_STEPWISE;
+  else
+    pl.mode = RTN_MODE_GRAPH;
+  pl.Bp = 16 * pl.NT;
+
+  size_t off = 0;
+  pl.off_status = off;
+  off += 256;
+  pl.off_flags = off;
+  pl.n_flags = (pl.kind == kPlanMfma) ? pl.groups * pl.wgs_per_group : 0;
+  off = align_up(off + (size_t)pl.n_flags * 4, 256);
+  if (pl.kind == kPlanMfma) {
+    pl.off_hx = off;
+    off = align_up(off + (size_t)pl.groups * 2 * n * pl.Bp * es, 256);
+    pl.off_wp = off;
+    off = align_up(off + (size_t)4 * n * n * es, 256);
+  } else {
+    pl.off_ycarry = off;
+    off = align_up(off + (size_t)2 * B * n * es, 256);
+  }
+  pl.total = off;
+  *out = pl;
+  return true;
+}
+
+const char* mode_name(int mode) {
+  switch (mode) {
+    case RTN_MODE_PERSISTENT: return "persistent";
+    case RTN_MODE_GRAPH: return "graph";
+    case RTN_MODE_STEPWISE: return "stepwise";
+    default: return "auto";
+  }
+}
+
+typedef void (*MfmaKernel)(const Lstm2Params, const int, const int);
+
+template <typename AT>
+MfmaKernel mfma_kernel_for(int MT, int NT) {
+#define RTN_CASE(mt, nt) \
+  if (MT == mt && NT == nt) return &k_lstm2_mfma<AT, mt, nt>;
+  RTN_CASE(1, 1) RTN_CASE(1, 2) RTN_CASE(1, 4)
+  RTN_CASE(2, 1) RTN_CASE(2, 2) RTN_CASE(2, 4)
+  RTN_CASE(4, 1) RTN_CASE(4, 2) RTN_CASE(4, 4)
+#undef RTN_CASE
+  return nullptr;
+}
+
+MfmaKernel mfma_kernel(int dtype, int MT, int NT) {
+  return dtype == RTN_DTYPE_BF16 ? mfma_kernel_for<__bf16>(MT, NT) : mfma_kernel_for<float>(MT, NT);
+}
+
+// Kernels that use more than the default LDS limit need the limit raised once per device.
+int ensure_lds_limit(MfmaKernel k, size_t lds_bytes) {
+  static std::mutex mu;
+  static std::list<std::pair<std::pair<int, MfmaKernel>, size_t>> done;
+  int dev = 0;
+  RTN_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  for (auto& e : done)
+    if (e.first.first == dev && e.first.second == k && e.second >= lds_bytes) return RTN_OK;
+  RTN_HIP(hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  done.push_back({{dev, k}, lds_bytes});
+  return RTN_OK;
+}
+
+// Library-owned graphs of the per-step launches, keyed by everything a launch depends on.
+struct GraphKey {
+  Lstm2Params p;
+  int dtype, MT, NT, kind, dev;
+  size_t lds;
+  bool operator==(const GraphKey& o) const { return memcmp(this, &o, sizeof(GraphKey)) == 0; }
+};
+struct GraphEntry {
+  GraphKey key;
+  hipGraph_t graph;
+  hipGraphExec_t exec;
+};
+std::mutex g_graph_mu;
+std::list<GraphEntry> g_graphs;  // most recently used first
+constexpr size_t kMaxGraphs = 8;
+
+int launch_steps(const Lstm2Params& p, const Plan& pl, int dtype, hipStream_t stream) {
+  if (pl.kind == kPlanMfma) {
+    MfmaKernel k = mfma_kernel(dtype, pl.MT, pl.NT);
+    const dim3 grid(pl.groups * pl.wgs_per_group), block(kWgThreads);
+    for (int s = 0; s < p.nsteps; ++s) hipLaunchKernelGGL(k, grid, block, pl.lds_bytes, stream, p, s, s + 1);
+  } else {
+    const long long bn = (long long)p.B * p.n;
+    const dim3 grid((unsigned)((bn + 255) / 256)), block(256);
+    for (int s = 0; s < p.nsteps; ++s) {
+      if (dtype == RTN_DTYPE_BF16)
+        hipLaunchKernelGGL(k_step_generic<__bf16>, grid, block, 0, stream, p, s);
+      else
+        hipLaunchKernelGGL(k_step_generic<float>, grid, block, 0, stream, p, s);
+    }
+  }
+  RTN_HIP(hipGetLastError());
+  return RTN_OK;
+}
+
+int launch_steps_graph(const Lstm2Params& p, const Plan& pl, int dtype, hipStream_t stream) {
+  GraphKey key;
+  memset(&key, 0, sizeof(key));
+  key.p = p;
+  key.dtype = dtype;
+  key.MT = pl.MT;
+  key.NT = pl.NT;
+  key.kind = pl.kind;
+  key.lds = pl.lds_bytes;
+  RTN_HIP(hipGetDevice(&key.dev));
+  std::lock_guard<std::mutex> lock(g_graph_mu);
+  for (auto it = g_graphs.begin(); it != g_graphs.end(); ++it) {
+    if (it->key == key) {
+      g_graphs.splice(g_graphs.begin(), g_graphs, it);
+      RTN_HIP(hipGraphLaunch(g_graphs.front().exec, stream));
+      return RTN_OK;
+    }
+  }
+  // Record the launches on a private stream; nothing runs until the graph is launched.
+  hipStream_t cap = nullptr;
+  RTN_HIP(hipStreamCreateWithFlags(&cap, hipStreamNonBlocking));
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  int rc = RTN_OK;
+  hipError_t e = hipStreamBeginCapture(cap, hipStreamCaptureModeThreadLocal);
+  if (e == hipSuccess) {
+    rc = launch_steps(p, pl, dtype, cap);
+    hipError_t e2 = hipStreamEndCapture(cap, &graph);
+    if (rc == RTN_OK && e2 != hipSuccess) rc = fail(RTN_ERR_HIP, "NativeLstm2: hipStreamEndCapture: %s", hipGetErrorString(e2));
+  } else {
+    rc = fail(RTN_ERR_HIP, "NativeLstm2: hipStreamBeginCapture: %s", hipGetErrorString(e));
+  }
+  (void)hipStreamDestroy(cap);
+  if (rc != RTN_OK) {
+    if (graph) (void)hipGraphDestroy(graph);
+    return rc;
+  }
+  e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGraphDestroy(graph);
+    return fail(RTN_ERR_HIP, "NativeLstm2: hipGraphInstantiate: %s", hipGetErrorString(e));
+  }
+  g_graphs.push_front(GraphEntry{key, graph, exec});
+  while (g_graphs.size() > kMaxGraphs) {
+    (void)hipGraphExecDestroy(g_graphs.back().exec);
+    (void)hipGraphDestroy(g_graphs.back().graph);
+    g_graphs.pop_back();
+  }
+  RTN_HIP(hipGraphLaunch(exec, stream));
+  return RTN_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_dims(int64_t T, int32_t B, int32_t n, int32_t dtype) {
+  if (T < 0 || B < 0 || n < 0) return fail(RTN_ERR_SHAPE, "NativeLstm2: negative dimension (T=%lld, B=%d, n=%d)", (long long)T, B, n);
+  if (dtype != RTN_DTYPE_F32 && dtype != RTN_DTYPE_BF16) return fail(RTN_ERR_ARG, "NativeLstm2: unknown dtype %d", dtype);
+  if (T > 0x7fffffffLL) return fail(RTN_ERR_SHAPE, "NativeLstm2: T=%lld exceeds the supported 2^31-1 frames", (long long)T);
+  if ((long long)B * n > 0x7fffffffLL / 16 || (long long)n * n > 0x7fffffffLL / 16)
+    return fail(RTN_ERR_SHAPE, "NativeLstm2: B*n or n*n too large (B=%d, n=%d)", B, n);
+  return RTN_OK;
+}
+
+}  // namespace
+}  // namespace rtn
+
+using namespace rtn;
+
+extern "C" {
+
+int rtn_native_lstm2_abi_version(void) { return 1; }
+
+const char* rtn_last_error(void) { return g_last_error.c_str(); }
+
+size_t rtn_native_lstm2_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
+  if (check_dims(T, B, n, dtype) != RTN_OK) return 0;
+  if (mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return 0;
+  // The largest layout any resolution of `mode` can need: AUTO may fall back to per-step launches.
+  size_t need = 0;
+  Plan pl;
+  std::string why;
+  if (make_plan(T, B, n, dtype, mode, false, &pl, &why)) need = std::max(need, pl.total);
+  if (mode == RTN_MODE_AUTO || mode == RTN_MODE_PERSISTENT)
+    if (make_plan(T, B, n, dtype, RTN_MODE_STEPWISE, true, &pl, &why)) need = std::max(need, pl.total);
+  return need;
+}
+
+const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
+  Plan pl;
+  std::string why;
+  char buf[512];
+  if (check_dims(T, B, n, dtype) != RTN_OK) {
+    g_plan_text = "invalid: " + g_last_error;
+  } else if (!make_plan(T, B, n, dtype, mode, false, &pl, &why)) {
+    g_plan_text = "unsupported: " + why;
+  } else {
+    snprintf(buf, sizeof(buf), "mode=%s kernel=%s mt=%d nt=%d groups=%d wgs_per_group=%d wgs=%d rows_per_group=%d lds=%zu workspace=%zu",
+             mode_name(pl.mode), pl.kind == kPlanMfma ? "mfma" : (pl.kind == kPlanGeneric ? "generic" : "empty"), pl.MT,
+             pl.NT, pl.groups, pl.wgs_per_group, pl.groups * pl.wgs_per_group, pl.Bg, pl.lds_bytes, pl.total);
+    g_plan_text = buf;
+  }
+  return g_plan_text.c_str();
+}
+
+int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const float* c0, const float* i, int32_t start,
+                         int32_t step, void* Y, float* C, void* H, float* d, int64_t T, int32_t B, int32_t n,
+                         int32_t dtype, int32_t mode, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  g_last_error.clear();
+  int rc = check_dims(T, B, n, dtype);
+  if (rc != RTN_OK) return rc;
+  if (mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return fail(RTN_ERR_ARG, "NativeLstm2: unknown mode %d", mode);
+  hipStream_t stream = (hipStream_t)hip_stream;
+  const long long bn = (long long)B * n;
+
+  if (bn > 0 && (!c0 || !d)) return fail(RTN_ERR_ARG, "NativeLstm2: c0 and d must not be null");
+  if (T == 0 || bn == 0) {
+    // returnn/native_op.py:1236-1237: no frames, the final cell state is the initial one.
+    if (bn > 0) {
+      hipLaunchKernelGGL(k_copy_f32, dim3((unsigned)std::min<long long>((bn + 255) / 256, 1024)), dim3(256), 0, stream, c0, d, bn);
+      RTN_HIP(hipGetLastError());
+    }
+    return RTN_OK;
+  }
+  if (start < 0 || start >= T) return fail(RTN_ERR_RANGE, "NativeLstm2: need 0 <= start < T, got start=%d, T=%lld", start, (long long)T);
+  if (step == 0) return fail(RTN_ERR_RANGE, "NativeLstm2: step must not be 0");
+  const void* ptrs[] = {X, W, y0, c0, i, Y, C, H, d};
+  const char* names[] = {"X", "W", "y0", "c0", "i", "Y", "C", "H", "d"};
+  for (int k = 0; k < 9; ++k) {
+    if (!ptrs[k]) return fail(RTN_ERR_ARG, "NativeLstm2: %s must not be null", names[k]);
+    if (k != 4 && !aligned16(ptrs[k])) return fail(RTN_ERR_ARG, "NativeLstm2: %s must be 16-byte aligned", names[k]);
+  }
+
+  hipStreamCaptureStatus cap_status = hipStreamCaptureStatusNone;
+  if (stream) RTN_HIP(hipStreamIsCapturing(stream, &cap_status));
+  const bool capturing = cap_status != hipStreamCaptureStatusNone;
+
+  Plan pl;
+  std::string why;
+  if (!make_plan(T, B, n, dtype, mode, capturing, &pl, &why))
+    return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: persistent mode unavailable for T=%lld B=%d n=%d: %s", (long long)T, B, n, why.c_str());
+  if (!workspace || workspace_bytes < pl.total)
+    return fail(RTN_ERR_WORKSPACE, "NativeLstm2: workspace of %zu bytes needed, got %zu", pl.total, workspace ? workspace_bytes : (size_t)0);
+  if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2: workspace must be 16-byte aligned");
+
+  Lstm2Params p;
+  memset(&p, 0, sizeof(p));
+  p.X = X; p.W = W; p.y0 = y0; p.c0 = c0; p.mask = i;
+  p.Y = Y; p.C = C; p.H = H; p.d = d;
+  unsigned char* ws = (unsigned char*)workspace;
+  p.status = (unsigned*)(ws + pl.off_status);
+  p.flags = (unsigned*)(ws + pl.off_flags);
+  p.hx = ws + pl.off_hx;
+  p.Wp = ws + pl.off_wp;
+  p.ycarry = ws + pl.off_ycarry;
+  p.T = T; p.B = B; p.n = n;
+  // returnn/native_op.py:1253-1259
+  if (step > 0) {
+    p.first = start;
+    p.nsteps = (int)((T - 1 - start) / step + 1);
+  } else {
+    p.first = (int)(T - start - 1);
+    p.nsteps = (int)(p.first / (-(long long)step) + 1);
+  }
+  p.step = step;
+  p.groups = pl.groups; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
+  p.xcds = device_info().xcds;
+  p.sync_policy = (int)env_long("RTN_LSTM2_SYNC", kStoreCoherent | kLoadCoherent);
+  if (!((p.sync_policy & (kStoreCoherent | kReleaseFence)) && (p.sync_policy & (kLoadCoherent | kAcquireFence))))
+    return fail(RTN_ERR_ARG, "NativeLstm2: RTN_LSTM2_SYNC=%d is not a valid publication policy", p.sync_policy);
+  p.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);  // 2 s at 100 MHz
+
+  // Frames the loop never visits.
+  if (p.nsteps != T) {
+    const long long total = T * bn * 4;
+    const dim3 grid((unsigned)std::min<long long>((total + 255) / 256, 65535)), block(256);
+    if (dtype == RTN_DTYPE_BF16)
+      hipLaunchKernelGGL(k_fill_unvisited<__bf16>, grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL(k_fill_unvisited<float>, grid, block, 0, stream, p);
+    RTN_HIP(hipGetLastError());
+  }
+
+  if (pl.kind == kPlanMfma) {
+    MfmaKernel k = mfma_kernel(dtype, pl.MT, pl.NT);
+    if (!k) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d", pl.MT, pl.NT);
+    rc = ensure_lds_limit(k, pl.lds_bytes);
+    if (rc != RTN_OK) return rc;
+    const long long work = std::max<long long>((long long)n * n, bn);
+    const dim3 pgrid((unsigned)std::min<long long>((work + 255) / 256, 2048)), pblock(256);
+    if (dtype == RTN_DTYPE_BF16)
+      hipLaunchKernelGGL(k_prepare_mfma<__bf16>, pgrid, pblock, 0, stream, p, pl.n_flags);
+    else
+      hipLaunchKernelGGL(k_prepare_mfma<float>, pgrid, pblock, 0, stream, p, pl.n_flags);
+    RTN_HIP(hipGetLastError());
+    if (pl.mode == RTN_MODE_PERSISTENT) {
+      const int wgs = pl.groups * pl.wgs_per_group;
+      int per_cu = 0;
+      RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)k, kWgThreads, pl.lds_bytes));
+      if ((long long)per_cu * device_info().cus < wgs) {
+        if (mode == RTN_MODE_PERSISTENT)
+          return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: %d workgroups cannot be co-resident (%d per CU)", wgs, per_cu);
+        pl.mode = RTN_MODE_GRAPH;  // AUTO: fall through to the per-step path with the same layout
+      } else {
+        int s_begin = 0, s_end = p.nsteps;
+        void* args[] = {(void*)&p, (void*)&s_begin, (void*)&s_end};
+        RTN_HIP(hipLaunchCooperativeKernel((const void*)k, dim3(wgs), dim3(kWgThreads), args, (unsigned)pl.lds_bytes, stream));
+        return RTN_OK;
+      }
+    }
+  } else {
+    hipLaunchKernelGGL(k_clear_status, dim3(1), dim3(64), 0, stream, p.status);
+    RTN_HIP(hipGetLastError());
+  }
+  if (pl.mode == RTN_MODE_GRAPH && !capturing) return launch_steps_graph(p, pl, dtype, stream);
+  return launch_steps(p, pl, dtype, stream);
+}
+
+int rtn_native_lstm2_fwd_status(const void* workspace, void* hip_stream) {
+  g_last_error.clear();
+  if (!workspace) return fail(RTN_ERR_ARG, "NativeLstm2: workspace must not be null");
+  unsigned status = 0;
+  hipStream_t stream = (hipStream_t)hip_stream;
+  RTN_HIP(hipMemcpyAsync(&status, workspace, sizeof(status), hipMemcpyDeviceToHost, stream));
+  RTN_HIP(hipStreamSynchronize(stream));
+  if (status != 0) return fail(RTN_ERR_ABORTED, "NativeLstm2: a bounded wait in the persistent kernel expired; outputs are invalid");
+  return RTN_OK;
+}
+
+int rtn_native_lstm2_last_output(const void* Y, const void* y0, const float* i, int32_t start, int32_t step, void* out,
+                                 int64_t T, int32_t B, int32_t n, int32_t dtype, void* hip_stream) {
+  g_last_error.clear();
+  int rc = check_dims(T, B, n, dtype);
+  if (rc != RTN_OK) return rc;
+  if ((long long)B * n == 0) return RTN_OK;
+  if (!y0 || !out) return fail(RTN_ERR_ARG, "NativeLstm2: y0 and out must not be null");
+  int first = 0, nsteps = 0;
+  if (T > 0) {
+    if (start < 0 || start >= T) return fail(RTN_ERR_RANGE, "NativeLstm2: need 0 <= start < T, got start=%d, T=%lld", start, (long long)T);
+    if (step == 0) return fail(RTN_ERR_RANGE, "NativeLstm2: step must not be 0");
+    if (!Y || !i) return fail(RTN_ERR_ARG, "NativeLstm2: Y and i must not be null");
+    if (step > 0) {
+      first = start;
+      nsteps = (int)((T - 1 - start) / step + 1);
+    } else {
+      first = (int)(T - start - 1);
+      nsteps = (int)(first / (-(long long)step) + 1);
+    }
+  }
+  hipStream_t stream = (hipStream_t)hip_stream;
+  if (dtype == RTN_DTYPE_BF16)
+    hipLaunchKernelGGL(k_last_output<__bf16>, dim3(B), dim3(256), 0, stream, Y, y0, i, out, (long long)T, B, n, first, step, nsteps);
+  else
+    hipLaunchKernelGGL(k_last_output<float>, dim3(B), dim3(256), 0, stream, Y, y0, i, out, (long long)T, B, n, first, step, nsteps);
+  RTN_HIP(hipGetLastError());
+  return RTN_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,102 @@
+"""
+ctypes binding of ``librtn_native_lstm2.so`` (C ABI declared in ``include/rtn_native_lstm2.h``).
+
+The library is the only implementation: there is no fallback.  If it has not been built,
+:func:`load` raises and says how to build it.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from typing import Optional
+
+from . import build as _build
+
+RTN_OK = 0
+RTN_ERR_SHAPE = 1
+RTN_ERR_RANGE = 2
+RTN_ERR_ARG = 3
+RTN_ERR_WORKSPACE = 4
+RTN_ERR_HIP = 5
+RTN_ERR_UNSUPPORTED = 6
+RTN_ERR_ABORTED = 7
+
+DTYPE_F32 = 0
+DTYPE_BF16 = 1
+
+MODE_AUTO = 0
+MODE_PERSISTENT = 1
+MODE_GRAPH = 2
+MODE_STEPWISE = 3
+MODES = {"auto": MODE_AUTO, "persistent": MODE_PERSISTENT, "graph": MODE_GRAPH, "stepwise": MODE_STEPWISE}
+
+# every symbol include/rtn_native_lstm2.h declares
+SYMBOLS = (
+    "rtn_native_lstm2_fwd",
+    "rtn_native_lstm2_fwd_workspace_bytes",
+    "rtn_native_lstm2_fwd_status",
+    "rtn_native_lstm2_last_output",
+    "rtn_last_error",
+    "rtn_native_lstm2_describe_plan",
+    "rtn_native_lstm2_abi_version",
+)
+
+_lock = threading.RLock()
+_lib: Optional[ctypes.CDLL] = None
+
+
+class NativeLibraryMissing(RuntimeError):
+    """The HIP library has not been built."""
+
+
+def load() -> ctypes.CDLL:
+    """Load the built library (once per process). Never builds, never falls back."""
+    global _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = _build.LIB_PATH
+        if not os.path.exists(path):
+            raise NativeLibraryMissing(
+                "%s not found. Build it with `python -m returnn_amd.build` (needs hipcc; "
+                "cross-compiles for gfx950 without a GPU)." % path
+            )
+        lib = ctypes.CDLL(path)
+        vp, i32, i64, sz = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_size_t
+        lib.rtn_native_lstm2_fwd.restype = ctypes.c_int
+        lib.rtn_native_lstm2_fwd.argtypes = [vp, vp, vp, vp, vp, i32, i32, vp, vp, vp, vp, i64, i32, i32, i32, i32, vp, sz, vp]
+        lib.rtn_native_lstm2_fwd_workspace_bytes.restype = sz
+        lib.rtn_native_lstm2_fwd_workspace_bytes.argtypes = [i64, i32, i32, i32, i32]
+        lib.rtn_native_lstm2_fwd_status.restype = ctypes.c_int
+        lib.rtn_native_lstm2_fwd_status.argtypes = [vp, vp]
+        lib.rtn_native_lstm2_last_output.restype = ctypes.c_int
+        lib.rtn_native_lstm2_last_output.argtypes = [vp, vp, vp, i32, i32, vp, i64, i32, i32, i32, vp]
+        lib.rtn_last_error.restype = ctypes.c_char_p
+        lib.rtn_last_error.argtypes = []
+        lib.rtn_native_lstm2_describe_plan.restype = ctypes.c_char_p
+        lib.rtn_native_lstm2_describe_plan.argtypes = [i64, i32, i32, i32, i32]
+        lib.rtn_native_lstm2_abi_version.restype = ctypes.c_int
+        lib.rtn_native_lstm2_abi_version.argtypes = []
+        _lib = lib
+        return lib
+
+
+def last_error() -> str:
+    return load().rtn_last_error().decode("utf8", "replace")
+
+
+def check(rc: int) -> None:
+    """Turn a status code of the C ABI into the exception the reference's wrapper would raise
+    (TORCH_CHECK -> RuntimeError, returnn/native_op.cpp:660)."""
+    if rc != RTN_OK:
+        raise RuntimeError(last_error() or ("NativeLstm2: error code %i" % rc))
+
+
+def describe_plan(T: int, B: int, n: int, dtype: int, mode: int) -> str:
+    return load().rtn_native_lstm2_describe_plan(T, B, n, dtype, mode).decode("utf8", "replace")
+
+
+def workspace_bytes(T: int, B: int, n: int, dtype: int, mode: int) -> int:
+    return int(load().rtn_native_lstm2_fwd_workspace_bytes(T, B, n, dtype, mode))

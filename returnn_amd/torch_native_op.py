@@ -1,0 +1,231 @@
+"""
+The native op as a PyTorch operator on HIP tensors.
+
+Drop-in for the reference's ``returnn.torch.util.native_op.make_op`` (returnn/torch/util/native_op.py:450-458)
+for the op this package implements: ``make_op(NativeLstm2)`` returns ``torch.ops.NativeLstm2.NativeLstm2`` with
+the schema the reference's generator would register (:242-277)::
+
+    NativeLstm2(Tensor X, Tensor W, Tensor y0, Tensor c0, Tensor i, int start, int step)
+        -> (Tensor, Tensor, Tensor, Tensor)
+
+Where the reference generates and compiles a C++ translation unit per op, this module registers the schema
+with ``torch.library`` from Python and the device implementation calls the prebuilt gfx950 library through
+its C ABI with raw device pointers and the current stream.  PyTorch only supplies memory and streams.
+
+Argument handling follows the generated wrapper (:144-193): dtype normalisation, ndim checks,
+``.contiguous()`` for ``need_contiguous`` inputs, device guard on the first tensor, outputs allocated on
+that device.  Differences, on purpose: bfloat16 inputs stay bfloat16 (X, W, y0, Y, H in bf16; c0, C, d,
+mask in float32) instead of being up-cast; outputs are not zero-filled first because the library writes
+every element; CPU tensors are rejected (no CPU implementation is shipped).
+"""
+
+from __future__ import annotations
+
+import sys
+from threading import RLock
+from typing import Any, Dict, Optional
+
+import torch
+
+from . import lib as _lib
+from . import native_op
+from .native_op import OpDescription
+
+_DTYPE_MAP = {"float32": torch.float32, "int32": torch.int32}
+
+
+def _schema_type_str(v: Dict[str, Any]) -> str:
+    if v.get("host_memory", False):
+        assert v["ndim"] == 0
+        return {"float32": "float", "int32": "int"}[v.get("dtype", "float32")]
+    return "Tensor"
+
+
+class OpMaker:
+    """
+    Registers one op with ``torch.library`` and hands out the ``torch.ops`` callable.
+    Cached per op name under a process-wide lock, like the reference's OpMaker (:33-36, :430-447).
+    """
+
+    global_lock = RLock()
+    op_cache: Dict[str, Any] = {}  # cache_key -> op
+    lib_cache: Dict[str, Any] = {}  # cache_key -> torch.library.Library (kept alive)
+    options: Dict[str, Dict[str, Any]] = {}  # cache_key -> run-time options of the device implementation
+    log_stream = sys.stdout
+
+    def __init__(
+        self,
+        description: OpDescription,
+        *,
+        compiler_opts: Optional[Dict[str, str]] = None,
+        with_cuda: Optional[bool] = None,
+        mode: Optional[str] = None,
+    ):
+        """
+        :param description:
+        :param compiler_opts: accepted for signature compatibility; the library is prebuilt, nothing is compiled here
+        :param with_cuda: accepted for signature compatibility; the device path is always HIP
+        :param mode: "auto" (default), "persistent", "graph" or "stepwise": execution mode of the library
+        """
+        del compiler_opts, with_cuda
+        self.description = description
+        self.name = description.name
+        if mode is not None and mode not in _lib.MODES:
+            raise ValueError("mode must be one of %r" % sorted(_lib.MODES))
+        self.mode = mode
+
+    @property
+    def op_name(self) -> str:
+        return self.name
+
+    @property
+    def cache_key(self) -> str:
+        return self.name
+
+    def schema(self) -> str:
+        d = self.description
+        args = ", ".join("%s %s" % (_schema_type_str(v), v["name"]) for v in d.in_info)
+        rets = ", ".join(_schema_type_str(v) for v in d.out_info)
+        return "%s(%s) -> (%s)" % (self.op_name, args, rets)
+
+    def _impl_for(self):
+        if self.description.c_abi_fw == "rtn_native_lstm2_fwd":
+            return _native_lstm2_device_impl
+        raise NotImplementedError("no gfx950 implementation for op %r" % self.name)
+
+    def make_op(self):
+        with self.global_lock:
+            if self.mode is not None or self.cache_key not in self.options:
+                self.options.setdefault(self.cache_key, {})["mode"] = self.mode or "auto"
+            if self.cache_key in self.op_cache:
+                return self.op_cache[self.cache_key]
+            _lib.load()  # fail now, loudly, if the HIP library is not there
+            impl = self._impl_for()
+            tlib = torch.library.Library(self.op_name, "DEF")
+            tlib.define(self.schema())
+            tlib.impl(self.op_name, impl, "CUDA")  # the dispatch key PyTorch-ROCm uses for HIP tensors
+            tlib.impl(self.op_name, _cpu_not_supported(self.op_name), "CPU")
+            self._register_fake_impl()
+            op = getattr(getattr(torch.ops, self.op_name), self.op_name)
+            self.lib_cache[self.cache_key] = tlib
+            self.op_cache[self.cache_key] = op
+            return op
+
+    def _register_fake_impl(self):
+        """Shapes from ``out_info`` for fake-tensor tracing (role of :396-428 in the reference)."""
+        description = self.description
+
+        def _fake_impl(*args):
+            tensors = [a for a in args if isinstance(a, torch.Tensor)]
+            device = tensors[0].device
+            shapes = description.infer_shape(None, [tuple(a.shape) if isinstance(a, torch.Tensor) else () for a in args])
+            act = torch.bfloat16 if tensors[0].dtype == torch.bfloat16 else torch.float32
+            dtypes = {"Y": act, "H": act}
+            return tuple(
+                torch.empty(shape, dtype=dtypes.get(o["name"], torch.float32), device=device)
+                for o, shape in zip(description.out_info, shapes)
+            )
+
+        torch.library.register_fake("%s::%s" % (self.op_name, self.op_name), _fake_impl)
+
+
+def make_op(cls, **kwargs):
+    """
+    :param type[returnn_amd.native_op.NativeOpGenBase] cls: e.g. :class:`returnn_amd.native_op.NativeLstm2`
+    :param kwargs: passed to :class:`OpMaker`
+    :return: op, ``(X, W, y0, c0, i, start, step) -> (Y, C, H, d)``
+    """
+    maker = OpMaker(OpDescription.from_gen_base(cls), **kwargs)
+    return maker.make_op()
+
+
+def _cpu_not_supported(name):
+    def _impl(*args):
+        raise RuntimeError(
+            "%s: this build implements the op for HIP (MI355X) tensors only; got CPU tensors. "
+            "Move the inputs to the GPU." % name
+        )
+
+    return _impl
+
+
+def _check_ndim(t: torch.Tensor, info: Dict[str, Any]):
+    if t.dim() != info["ndim"]:
+        raise RuntimeError("%s shape ndim is not %i, got shape %s" % (info["name"], info["ndim"], tuple(t.shape)))
+
+
+def _native_lstm2_device_impl(X, W, y0, c0, i, start, step):
+    """``NativeLstm2`` on HIP tensors: normalise the arguments, allocate outputs and scratch, enqueue the library call."""
+    infos = native_op.NativeLstm2.in_info
+    for t, info in zip((X, W, y0, c0, i), infos):
+        _check_ndim(t, info)
+    device = X.device
+    for t, info in zip((W, y0, c0, i), infos[1:]):
+        if t.device != device:
+            raise RuntimeError("%s is on %s but X is on %s" % (info["name"], t.device, device))
+    bf16 = X.dtype == torch.bfloat16
+    act = torch.bfloat16 if bf16 else torch.float32
+    X, W, y0 = (t if t.dtype == act else t.to(act) for t in (X, W, y0))
+    c0, i = (t if t.dtype == torch.float32 else t.to(torch.float32) for t in (c0, i))
+    X, W, y0, c0, i = (t if t.is_contiguous() else t.contiguous() for t in (X, W, y0, c0, i))
+    T, B = i.shape
+    n = y0.shape[1]
+    # the reference's shape asserts (returnn/native_op.py:1215-1223); hard errors here
+    expect = {"X": (T, B, 4 * n), "W": (n, 4 * n), "y0": (B, n), "c0": (B, n)}
+    for name, t in (("X", X), ("W", W), ("y0", y0), ("c0", c0)):
+        if tuple(t.shape) != expect[name]:
+            raise RuntimeError(
+                "NativeLstm2: %s has shape %s, expected %s (T=%i, B=%i from i; n=%i from y0)"
+                % (name, tuple(t.shape), expect[name], T, B, n)
+            )
+    lib = _lib.load()
+    dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
+    mode = _lib.MODES[OpMaker.options.get("NativeLstm2", {}).get("mode", "auto")]
+    with torch.cuda.device(device):
+        Y = torch.empty((T, B, n), dtype=act, device=device)
+        C = torch.empty((T, B, n), dtype=torch.float32, device=device)
+        H = torch.empty((T, B, 4 * n), dtype=act, device=device)
+        d = torch.empty((B, n), dtype=torch.float32, device=device)
+        ws_bytes = int(lib.rtn_native_lstm2_fwd_workspace_bytes(T, B, n, dtype, mode))
+        ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=device)
+        stream = torch.cuda.current_stream(device).cuda_stream
+        rc = lib.rtn_native_lstm2_fwd(
+            X.data_ptr(), W.data_ptr(), y0.data_ptr(), c0.data_ptr(), i.data_ptr(), int(start), int(step),
+            Y.data_ptr(), C.data_ptr(), H.data_ptr(), d.data_ptr(), T, B, n, dtype, mode,
+            ws.data_ptr(), ws.numel(), stream,
+        )  # fmt: skip
+    _lib.check(rc)
+    # The workspace goes back to the caching allocator here; the allocator keeps it out of other
+    # streams' hands until the work queued on this stream has passed it (stream-ordered reuse).
+    return Y, C, H, d
+
+
+def lstm_last_output(Y: torch.Tensor, y0: torch.Tensor, i: torch.Tensor, start: int = 0, step: int = 1) -> torch.Tensor:
+    """
+    Final output per sequence, the caller-side ``_lstm_last_output`` of the reference
+    (returnn/tf/native_op.py:913-929), computed by the library on the device.
+
+    :param Y: [T,B,n] output of the op
+    :param y0: [B,n]
+    :param i: [T,B] mask
+    :return: [B,n]
+    """
+    if not Y.is_cuda:
+        raise RuntimeError("lstm_last_output: this build implements the op for HIP (MI355X) tensors only")
+    bf16 = Y.dtype == torch.bfloat16
+    act = torch.bfloat16 if bf16 else torch.float32
+    Y = Y.to(act).contiguous()
+    y0 = y0.to(act).contiguous()
+    i = i.to(torch.float32).contiguous()
+    T, B, n = Y.shape
+    if tuple(y0.shape) != (B, n) or tuple(i.shape) != (T, B):
+        raise RuntimeError("lstm_last_output: y0 %s / i %s do not match Y %s" % (tuple(y0.shape), tuple(i.shape), tuple(Y.shape)))
+    lib = _lib.load()
+    with torch.cuda.device(Y.device):
+        out = torch.empty((B, n), dtype=act, device=Y.device)
+        rc = lib.rtn_native_lstm2_last_output(
+            Y.data_ptr(), y0.data_ptr(), i.data_ptr(), int(start), int(step), out.data_ptr(), T, B, n,
+            _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32, torch.cuda.current_stream(Y.device).cuda_stream,
+        )  # fmt: skip
+    _lib.check(rc)
+    return out

@@ -1,0 +1,134 @@
+"""
+CPU-side checks of the C-ABI library: it loads, exports every symbol the header declares, and its
+host logic (argument validation, plan, workspace size) behaves -- no kernel is launched here.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from returnn_amd import build, lib
+
+_root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    if not os.path.exists(build.LIB_PATH):
+        build.build_library()
+    return lib.load()
+
+
+def test_header_symbols_are_exported(cabi):
+    header = open(os.path.join(_root, "include", "rtn_native_lstm2.h")).read()
+    declared = set(re.findall(r"\b(rtn_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(lib.SYMBOLS)
+    for name in declared:
+        assert getattr(cabi, name) is not None
+
+
+def test_abi_version(cabi):
+    assert cabi.rtn_native_lstm2_abi_version() == 1
+
+
+def test_error_codes_match_header():
+    header = open(os.path.join(_root, "include", "rtn_native_lstm2.h")).read()
+    for name, value in re.findall(r"#define (RTN_[A-Z0-9_]+) (\d+)", header):
+        py = {"RTN_DTYPE_F32": "DTYPE_F32", "RTN_DTYPE_BF16": "DTYPE_BF16"}.get(name, name.replace("RTN_MODE_", "MODE_"))
+        assert getattr(lib, py) == int(value), name
+
+
+def _call(cabi, T, B, n, start=0, step=1, dtype=0, mode=0, ptr=4096, ws=None, ws_bytes=0):
+    p = ctypes.c_void_p(ptr)
+    return cabi.rtn_native_lstm2_fwd(p, p, p, p, p, start, step, p, p, p, p, T, B, n, dtype, mode, ws, ws_bytes, None)
+
+
+def test_range_and_argument_errors(cabi):
+    """The reference only prints on these under NDEBUG (returnn/native_op.cpp:60-69, native_op.py:1249-1252); here they are errors."""
+    assert _call(cabi, 3, 2, 2, start=3) == lib.RTN_ERR_RANGE
+    assert "start" in lib.last_error()
+    assert _call(cabi, 3, 2, 2, start=-1) == lib.RTN_ERR_RANGE
+    assert _call(cabi, 3, 2, 2, step=0) == lib.RTN_ERR_RANGE
+    assert "step" in lib.last_error()
+    assert _call(cabi, -1, 2, 2) == lib.RTN_ERR_SHAPE
+    assert _call(cabi, 3, -2, 2) == lib.RTN_ERR_SHAPE
+    assert _call(cabi, 3, 2, 2, dtype=7) == lib.RTN_ERR_ARG
+    assert _call(cabi, 3, 2, 2, mode=9) == lib.RTN_ERR_ARG
+    assert _call(cabi, 3, 2, 2, ptr=0) == lib.RTN_ERR_ARG  # null pointers
+    assert _call(cabi, 3, 2, 2, ptr=4100) == lib.RTN_ERR_ARG  # misaligned
+    assert "aligned" in lib.last_error()
+    assert _call(cabi, 3, 2, 2) == lib.RTN_ERR_WORKSPACE  # no workspace
+    assert "workspace" in lib.last_error()
+    # persistent mode is refused, not silently replaced, for a shape the MFMA kernel cannot take
+    assert _call(cabi, 3, 2, 3, mode=lib.MODE_PERSISTENT) == lib.RTN_ERR_UNSUPPORTED
+
+
+def test_workspace_and_plan(cabi):
+    # BASELINE config 3: bf16, T=1000, B=32, n=1024: persistent, all weights on chip
+    text = lib.describe_plan(1000, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
+    assert "mode=persistent" in text and "kernel=mfma" in text
+    ws = lib.workspace_bytes(1000, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
+    assert ws >= 4 * 1024 * 1024 * 2  # at least the packed W
+    # odd n: generic per-step kernels
+    text = lib.describe_plan(3, 2, 2, lib.DTYPE_F32, lib.MODE_AUTO)
+    assert "kernel=generic" in text and "mode=graph" in text
+    assert lib.workspace_bytes(3, 2, 2, lib.DTYPE_F32, lib.MODE_AUTO) >= 2 * 2 * 2 * 4
+    assert lib.workspace_bytes(-1, 2, 2, lib.DTYPE_F32, lib.MODE_AUTO) == 0
+    # the workspace of AUTO covers its per-step fallback
+    for T, B, n, dt in [(10, 64, 512, 0), (10, 32, 1024, 1), (10, 1, 1024, 1), (10, 200, 1024, 1), (5, 7, 96, 0)]:
+        assert lib.workspace_bytes(T, B, n, dt, lib.MODE_AUTO) >= lib.workspace_bytes(T, B, n, dt, lib.MODE_STEPWISE)
+
+
+def test_op_description_contract():
+    """Names, order, ndim and host-memory flags of returnn/native_op.py:1054-1068."""
+    from returnn_amd import native_op
+
+    d = native_op.OpDescription.from_gen_base(native_op.NativeLstm2)
+    assert d.name == "NativeLstm2"
+    assert [v["name"] for v in d.in_info] == ["X", "W", "y0", "c0", "i", "start", "step"]
+    assert [v["ndim"] for v in d.in_info] == [3, 2, 2, 2, 2, 0, 0]
+    assert all(v.get("host_memory") and v["dtype"] == "int32" for v in d.in_info[5:])
+    assert [v["name"] for v in d.out_info] == ["Y", "C", "H", "d"]
+    T, B, n = 7, 3, 5
+    shapes = d.infer_shape(None, [(T, B, 4 * n), (n, 4 * n), (B, n), (B, n), (T, B), (), ()])
+    assert shapes == [(T, B, n), (T, B, n), (T, B, 4 * n), (B, n)]
+    assert len(native_op.NativeLstm2.grad_input_map(*range(15))) == 12
+
+
+def test_schema_string():
+    from returnn_amd import native_op, torch_native_op
+
+    maker = torch_native_op.OpMaker(native_op.OpDescription.from_gen_base(native_op.NativeLstm2))
+    assert maker.schema() == (
+        "NativeLstm2(Tensor X, Tensor W, Tensor y0, Tensor c0, Tensor i, int start, int step) -> (Tensor, Tensor, Tensor, Tensor)"
+    )
+
+
+def test_make_op_rejects_cpu_tensors(cabi):
+    """No CPU implementation is shipped: the op must fail loudly instead of computing somewhere else."""
+    import torch
+
+    from returnn_amd import native_op, torch_native_op
+
+    op = torch_native_op.make_op(native_op.NativeLstm2)
+    assert op is torch_native_op.make_op(native_op.NativeLstm2)  # cached per name
+    T, B, n = 3, 2, 2
+    with pytest.raises(RuntimeError, match="HIP"):
+        op(torch.zeros(T, B, 4 * n), torch.zeros(n, 4 * n), torch.zeros(B, n), torch.zeros(B, n), torch.ones(T, B), 0, 1)
+
+
+def test_fake_impl_shapes(cabi):
+    import torch
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from returnn_amd import native_op, torch_native_op
+
+    op = torch_native_op.make_op(native_op.NativeLstm2)
+    T, B, n = 5, 3, 4
+    with FakeTensorMode():
+        outs = op(torch.zeros(T, B, 4 * n), torch.zeros(n, 4 * n), torch.zeros(B, n), torch.zeros(B, n), torch.ones(T, B), 0, 1)
+    assert [tuple(o.shape) for o in outs] == [(T, B, n), (T, B, n), (T, B, 4 * n), (B, n)]

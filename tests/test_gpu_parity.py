@@ -1,0 +1,337 @@
+"""
+Parity of the HIP path (through the C ABI) with the CPU oracle on the same seeded inputs.
+
+Tolerances:
+* float32: ``rtol=1e-5`` (the bar the operator is specified to) with ``atol=2e-6`` for values near zero
+  (outputs are O(1); the reference's own check of this op uses rtol=1e-6 on a 3-frame fixture,
+  tests/test_TFNativeOp.py:902-906, here sequences are up to 500 frames long and the GEMM summation order differs).
+* bfloat16 activations/weights with float32 accumulate and cell state: ``atol=2e-2`` on Y and C against the
+  float32 oracle fed the *identical float32* inputs, as the operator is specified.
+"""
+
+from __future__ import annotations
+
+import numpy
+import pytest
+from numpy.testing import assert_allclose
+
+from oracle import lstm2_oracle as oracle
+from returnn_amd import synthetic
+from _gpu_util import announce, env, random_problem, run_op, run_raw
+from _textbook import REFERENCE_START_STEP, reference_fixture, textbook_lstm, visited_slice
+
+pytestmark = pytest.mark.gpu
+
+F32_RTOL, F32_ATOL = 1e-5, 2e-6
+BF16_ATOL = 2e-2
+SYNC_POLICIES = {"coherent": 5, "fences": 10}  # SyncBits of the persistent kernel's hidden-state exchange
+
+
+def check_f32(got, want, what=""):
+    names = ("Y", "C", "H", "d", "y_last")
+    for name, g, w in zip(names, got, want):
+        assert g.shape == w.shape, (what, name)
+        assert_allclose(g, w, rtol=F32_RTOL, atol=F32_ATOL, err_msg="%s %s" % (what, name))
+
+
+def check_bf16(got, want, what="", atol=BF16_ATOL):
+    names = ("Y", "C", "H", "d", "y_last")
+    for name, g, w in zip(names, got, want):
+        assert g.shape == w.shape, (what, name)
+        assert numpy.all(numpy.isfinite(g)), (what, name)
+        assert_allclose(g, w, rtol=0, atol=atol, err_msg="%s %s" % (what, name))
+
+
+@pytest.mark.parametrize("start,step", REFERENCE_START_STEP)
+def test_reference_fixture(start, step):
+    """tests/test_TFNativeOp.py:866-889 fixture x :824 (start, step) pairs, :851-854 comparison rules, against
+    the textbook LSTM directly (not via the oracle) and against the oracle on everything incl. H."""
+    announce("reference_fixture", start, step)
+    fx = reference_fixture(numpy.float32)
+    X = fx["x"] @ fx["W_f"] + fx["b"][None, None, :]
+    got = run_op(X, fx["W_r"], fx["h_0"], fx["c_0"], fx["mask"], start, step)
+    h2, c2, cT, hT = textbook_lstm(start=start, step=step, **fx)
+    sl = visited_slice(3, start, step)
+    m = fx["mask"][:, :, None]
+    assert_allclose(got[0][sl] * m[sl], h2[sl] * m[sl], rtol=1e-5, atol=1e-6)
+    assert_allclose(got[1][sl] * m[sl], c2[sl] * m[sl], rtol=1e-5, atol=1e-6)
+    assert_allclose(got[3], cT, rtol=1e-5, atol=1e-6)
+    assert_allclose(got[4], hT, rtol=1e-5, atol=1e-6)
+    check_f32(got, oracle.native_lstm2_fwd(X, fx["W_r"], fx["h_0"], fx["c_0"], fx["mask"], start, step), "fixture")
+
+
+@pytest.mark.parametrize("T,B,n", [(1, 1, 1), (2, 1, 3), (5, 3, 7), (9, 4, 33), (4, 70, 5), (6, 2, 130)])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_generic_shapes(T, B, n, dtype):
+    """Cell counts that are not a multiple of 32 take the generic per-step kernels."""
+    announce("generic_shapes", T, B, n, dtype)
+    for start, step in [(0, 1), (0, -1), (1, 2)]:
+        if start >= T:
+            continue
+        p = random_problem(100 + T + B + n, T, B, n)
+        want = oracle.native_lstm2_fwd(*p, start, step)
+        got = run_op(*p, start, step, dtype=dtype)
+        (check_f32 if dtype == "f32" else check_bf16)(got, want, "generic %s" % ((T, B, n, start, step),))
+
+
+MFMA_SHAPES = [(7, 1, 32), (6, 3, 64), (5, 16, 96), (5, 17, 128), (4, 33, 64), (4, 64, 160), (3, 100, 64), (12, 5, 256)]
+
+
+@pytest.mark.parametrize("T,B,n", MFMA_SHAPES)
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("mode", ["persistent", "graph", "stepwise"])
+def test_mfma_shapes(T, B, n, dtype, mode):
+    announce("mfma_shapes", T, B, n, dtype, mode)
+    for start, step in [(0, 1), (0, -1), (1, 1), (1, -1), (0, 2), (0, -2)]:
+        p = random_problem(200 + T + B + n, T, B, n)
+        want = oracle.native_lstm2_fwd(*p, start, step)
+        got = run_op(*p, start, step, dtype=dtype, mode=mode)
+        (check_f32 if dtype == "f32" else check_bf16)(got, want, "mfma %s" % ((T, B, n, start, step, mode),))
+
+
+@pytest.mark.parametrize("policy", sorted(SYNC_POLICIES))
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_persistent_sync_policies(policy, dtype):
+    """Both ways of publishing the hidden state between workgroups give the per-step kernels' result bit for bit."""
+    announce("sync_policy", policy, dtype)
+    p = random_problem(7, 40, 24, 256)
+    base = run_op(*p, 0, 1, dtype=dtype, mode="stepwise")
+    with env(RTN_LSTM2_SYNC=SYNC_POLICIES[policy]):
+        for step in (1, -1):
+            ref = run_op(*p, 0, step, dtype=dtype, mode="stepwise")
+            got = run_op(*p, 0, step, dtype=dtype, mode="persistent")
+            for a, b in zip(got, ref):
+                assert numpy.array_equal(a, b)
+    assert numpy.array_equal(base[0], run_op(*p, 0, 1, dtype=dtype, mode="stepwise")[0])  # deterministic
+
+
+@pytest.mark.parametrize("mt,groups", [(1, 1), (2, 2), (4, 4), (2, 1), (4, 8)])
+def test_decompositions(mt, groups):
+    """Cells per workgroup and batch groups are a tuning choice, never a change of results (up to summation order)."""
+    announce("decompositions", mt, groups)
+    p = random_problem(11, 30, 48, 512)
+    want = oracle.native_lstm2_fwd(*p, 0, 1)
+    with env(RTN_LSTM2_MT=mt, RTN_LSTM2_GROUPS=groups):
+        for dtype, chk in (("f32", check_f32), ("bf16", check_bf16)):
+            got = run_op(*p, 0, 1, dtype=dtype, mode="persistent")
+            chk(got, want, "decomposition mt=%i groups=%i %s" % (mt, groups, dtype))
+
+
+def test_cfg1_fp32():
+    """BASELINE config 1: T=32, B=4, n=64, fp32, full-length, 1e-5 relative."""
+    announce("cfg1")
+    p = synthetic.make_config("cfg1")
+    want = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, p.start, p.step)
+    for mode in ("persistent", "graph", "auto"):
+        got = run_op(p.X, p.W, p.y0, p.c0, p.i, p.start, p.step, mode=mode)
+        check_f32(got, want, "cfg1 " + mode)
+
+
+def test_cfg2_fp32_full():
+    """BASELINE config 2 at full size: T=500, B=64, n=512, fp32, ragged lengths in [250,500]."""
+    announce("cfg2 full")
+    p = synthetic.make_config("cfg2")
+    want = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, p.start, p.step, threads=oracle.max_threads())
+    got = run_op(p.X, p.W, p.y0, p.c0, p.i, p.start, p.step, mode="auto")
+    check_f32(got, want, "cfg2")
+    # size-independent properties at full size
+    m = p.i[:, :, None]
+    assert numpy.array_equal(got[0] * (1 - m), numpy.zeros_like(got[0]))  # Y exactly 0 on padded frames
+    for b in range(p.B):
+        L = int(p.lens[b])
+        assert numpy.array_equal(got[3][b], got[1][L - 1, b])  # d = C at the last valid frame
+        assert numpy.array_equal(got[1][-1, b], got[1][L - 1, b])  # cell carried over the padding
+        assert numpy.array_equal(got[4][b], got[0][L - 1, b])  # final output = Y at the last valid frame
+
+
+@pytest.mark.parametrize("step", [1, -1])
+def test_cfg3_bf16_reduced(step):
+    """BASELINE config 3 shape (B=32, n=1024, bf16) at T=120, both directions of the bidirectional pair:
+    2e-2 absolute on Y and C against the fp32 oracle on the identical fp32 inputs."""
+    announce("cfg3 reduced", step)
+    p = synthetic.make_config("cfg3", T=120, step=step)
+    want = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, p.start, p.step, threads=oracle.max_threads())
+    for mode in ("persistent", "graph"):
+        got = run_op(p.X, p.W, p.y0, p.c0, p.i, p.start, p.step, dtype="bf16", mode=mode)
+        check_bf16(got, want, "cfg3 T=120 step=%i %s" % (step, mode))
+    # error of the kernel alone: oracle fed the bf16-rounded X, W (quantisation of the inputs taken out)
+    want_q = oracle.native_lstm2_fwd(
+        synthetic.round_to_bf16(p.X), synthetic.round_to_bf16(p.W), p.y0, p.c0, p.i, p.start, p.step,
+        threads=oracle.max_threads(),
+    )  # fmt: skip
+    err = max(float(numpy.abs(g - w).max()) for g, w in zip(got[:2], want_q[:2]))
+    print("cfg3 T=120 step=%i: max |Y,C - oracle(bf16-rounded inputs)| = %.3e" % (step, err))
+    assert err < BF16_ATOL
+
+
+def test_cfg3_bf16_full_size():
+    """BASELINE config 3 at full size (T=1000, B=32, n=1024, bf16), forward and backward call."""
+    announce("cfg3 full")
+    p = synthetic.make_config("cfg3")
+    want = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, 0, 1, threads=oracle.max_threads())
+    got = run_op(p.X, p.W, p.y0, p.c0, p.i, 0, 1, dtype="bf16", mode="auto")
+    check_bf16(got, want, "cfg3 full fwd")
+    # the backward call of the pair: properties that need no second oracle pass
+    announce("cfg3 full backward")
+    gotb = run_op(p.X, p.W, p.y0, p.c0, p.i, 0, -1, dtype="bf16", mode="auto")
+    m = p.i[:, :, None]
+    assert numpy.all(numpy.isfinite(gotb[0])) and numpy.all(numpy.isfinite(gotb[1]))
+    assert numpy.array_equal(gotb[0] * (1 - m), numpy.zeros_like(gotb[0]))
+    for b in range(p.B):
+        L = int(p.lens[b])
+        assert numpy.array_equal(gotb[3][b], gotb[1][0, b])  # backward: last visited frame is t = 0
+        assert numpy.array_equal(gotb[1][L:, b], numpy.broadcast_to(p.c0[b], (p.T - L, p.n)))  # padding carries c0
+        assert numpy.array_equal(gotb[4][b], gotb[0][0, b])
+    # time reversal of each sequence: backward call == forward call on the sequence reversed within its length
+    Xr = p.X.copy()
+    for b in range(p.B):
+        L = int(p.lens[b])
+        Xr[:L, b] = p.X[:L, b][::-1]
+    gotr = run_op(Xr, p.W, p.y0, p.c0, p.i, 0, 1, dtype="bf16", mode="auto")
+    for b in range(p.B):
+        L = int(p.lens[b])
+        assert numpy.array_equal(gotb[0][:L, b], gotr[0][:L, b][::-1])
+        assert numpy.array_equal(gotb[1][:L, b], gotr[1][:L, b][::-1])
+
+
+def test_cfg5_bf16_single_stream():
+    """BASELINE config 5 shape (B=1, n=1024, bf16), T=600 against the oracle; full T=4000 through properties."""
+    announce("cfg5 T=600")
+    p = synthetic.make_config("cfg5", T=600)
+    want = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, 0, 1, threads=oracle.max_threads())
+    got = run_op(p.X, p.W, p.y0, p.c0, p.i, 0, 1, dtype="bf16", mode="auto")
+    check_bf16(got, want, "cfg5 T=600")
+    announce("cfg5 full")
+    pf = synthetic.make_config("cfg5")
+    a = run_op(pf.X, pf.W, pf.y0, pf.c0, pf.i, 0, 1, dtype="bf16", mode="persistent")
+    # prefix property: the first 600 frames of the long run are the short run (same seed -> same leading X? no:
+    # X is drawn per shape, so compare against a per-step run of the same inputs instead)
+    b = run_op(pf.X, pf.W, pf.y0, pf.c0, pf.i, 0, 1, dtype="bf16", mode="stepwise")
+    for u, v in zip(a, b):
+        assert numpy.array_equal(u, v)
+    assert numpy.array_equal(a[3][0], a[1][-1, 0])
+
+
+def test_zero_length_and_empty():
+    """T = 0: d = c0 (returnn/native_op.py:1236-1237, tests/test_TFNativeOp.py:448-464); B = 0 and n = 0 are no-ops."""
+    announce("zero length")
+    B, n = 3, 64
+    rng = numpy.random.default_rng(0)
+    c0 = rng.normal(size=(B, n)).astype(numpy.float32)
+    y0 = rng.normal(size=(B, n)).astype(numpy.float32)
+    for dtype in ("f32", "bf16"):
+        Y, C, H, d, yl = run_op(numpy.zeros((0, B, 4 * n)), numpy.zeros((n, 4 * n)), y0, c0, numpy.zeros((0, B)), dtype=dtype)
+        assert Y.shape == (0, B, n) and H.shape == (0, B, 4 * n)
+        assert numpy.array_equal(d, c0)
+    Y, C, H, d, yl = run_op(numpy.zeros((4, 0, 4 * n)), numpy.zeros((n, 4 * n)), numpy.zeros((0, n)), numpy.zeros((0, n)), numpy.zeros((4, 0)))
+    assert Y.shape == (4, 0, n) and d.shape == (0, n)
+
+
+def test_zeros_run():
+    """tests/test_TFNativeOp.py:368-384: T=2, B=1, n=3, all-zero input."""
+    announce("zeros run")
+    T, B, n = 2, 1, 3
+    Y, C, H, d, yl = run_op(numpy.zeros((T, B, 4 * n)), numpy.zeros((n, 4 * n)), numpy.zeros((B, n)), numpy.zeros((B, n)), numpy.ones((T, B)))
+    assert numpy.array_equal(Y, numpy.zeros((T, B, n), dtype=numpy.float32))
+    assert numpy.array_equal(d, numpy.zeros((B, n), dtype=numpy.float32))
+    assert_allclose(H[..., n:], 0.5, rtol=1e-6)
+
+
+@pytest.mark.parametrize("n", [3, 64])
+def test_outputs_fully_written_and_unvisited_frames(n):
+    """Outputs handed over as NaN come back fully defined; frames the loop skips have Y = C = 0 and H = X."""
+    announce("poisoned outputs", n)
+    T, B = 7, 5
+    p = random_problem(21, T, B, n)
+    for start, step in [(0, 1), (2, 3), (1, -2)]:
+        for dtype in ("f32", "bf16"):
+            rc, status, got = run_raw(*p, start, step, dtype=dtype)
+            assert rc == 0 and status == 0
+            for g in got:
+                assert numpy.all(numpy.isfinite(g))
+            want = oracle.native_lstm2_fwd(*p, start, step)
+            (check_f32 if dtype == "f32" else check_bf16)(got, want[:4], "poisoned %s" % ((n, start, step, dtype),))
+            sl = visited_slice(T, start, step)
+            unvisited = numpy.ones(T, dtype=bool)
+            unvisited[sl] = False
+            assert numpy.array_equal(got[0][unvisited], numpy.zeros_like(got[0][unvisited]))
+            assert numpy.array_equal(got[1][unvisited], numpy.zeros_like(got[1][unvisited]))
+            Xq = p[0] if dtype == "f32" else synthetic.round_to_bf16(p[0])
+            assert numpy.array_equal(got[2][unvisited], Xq[unvisited])
+
+
+def test_mask_zero_everywhere():
+    announce("mask zero")
+    T, B, n = 5, 4, 64
+    X, W, y0, c0, _ = random_problem(31, T, B, n)
+    Y, C, H, d, yl = run_op(X, W, y0, c0, numpy.zeros((T, B)))
+    assert numpy.array_equal(Y, numpy.zeros_like(Y))
+    for t in range(T):
+        assert numpy.array_equal(C[t], c0)
+    assert numpy.array_equal(d, c0)
+    assert numpy.array_equal(yl, y0)
+
+
+def test_batch_row_independence():
+    """Single-vs-batched: each sequence alone gives the rows it gives inside the batch (same decomposition of k,
+    so bit for bit)."""
+    announce("row independence")
+    T, B, n = 9, 6, 128
+    p = random_problem(41, T, B, n)
+    full = run_op(*p, 0, 1, mode="stepwise")
+    for b in (0, 3, 5):
+        one = run_op(p[0][:, b : b + 1], p[1], p[2][b : b + 1], p[3][b : b + 1], p[4][:, b : b + 1], 0, 1, mode="stepwise")
+        for k in range(3):
+            assert numpy.array_equal(full[k][:, b : b + 1], one[k])
+        assert numpy.array_equal(full[3][b : b + 1], one[3])
+
+
+def test_argument_handling():
+    """Error behaviour and input normalisation of the generated wrapper (returnn/torch/util/native_op.py:144-193)."""
+    import torch
+
+    from _gpu_util import get_op
+
+    announce("argument handling")
+    op = get_op()
+    T, B, n = 4, 3, 64
+    X, W, y0, c0, i = (torch.from_numpy(a).cuda() for a in random_problem(51, T, B, n))
+    with pytest.raises(RuntimeError, match="start"):
+        op(X, W, y0, c0, i, T, 1)
+    with pytest.raises(RuntimeError, match="step"):
+        op(X, W, y0, c0, i, 0, 0)
+    with pytest.raises(RuntimeError, match="ndim"):
+        op(X[0], W, y0, c0, i, 0, 1)
+    with pytest.raises(RuntimeError, match="shape"):
+        op(X[:, :, :-4], W, y0, c0, i, 0, 1)
+    with pytest.raises(RuntimeError, match="shape"):
+        op(X, W[:, :-4], y0, c0, i, 0, 1)
+    # non-contiguous and non-float32 inputs are normalised, not rejected
+    want = op(X, W, y0, c0, i, 0, 1)
+    Xnc = X.transpose(0, 1).contiguous().transpose(0, 1)
+    assert not Xnc.is_contiguous()
+    got = op(Xnc, W.double(), y0, c0.double(), i.to(torch.int32), 0, 1)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    # python ints and 0-dim tensors both work for the host scalars
+    got = op(X, W, y0, c0, i, int(torch.tensor(0)), int(torch.tensor(1)))
+    assert torch.equal(got[0], want[0])
+
+
+def test_bounded_wait_expires_cleanly():
+    """A wait bound of zero ticks forced from the host: the persistent kernel must still drain; the status call
+    then reports either success (nobody had to wait) or the abort."""
+    from returnn_amd import lib
+
+    announce("bounded wait")
+    p = random_problem(61, 50, 8, 256)
+    with env(RTN_LSTM2_TIMEOUT_TICKS=0):
+        rc, status, got = run_raw(*p, 0, 1, mode="persistent")
+    assert rc == 0
+    assert status in (lib.RTN_OK, lib.RTN_ERR_ABORTED)
+    if status == lib.RTN_OK:
+        check_f32(got, oracle.native_lstm2_fwd(*p, 0, 1)[:4], "bounded wait")
+    # and the next ordinary call is unaffected
+    rc, status, got = run_raw(*p, 0, 1, mode="persistent")
+    assert rc == 0 and status == 0
+    check_f32(got, oracle.native_lstm2_fwd(*p, 0, 1)[:4], "after bounded wait")
