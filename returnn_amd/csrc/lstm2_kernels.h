@@ -71,6 +71,29 @@ struct Elem<__bf16> {
 // sigmoid exactly as the reference writes it (returnn/native_op.py:1102-1104)
 __device__ __forceinline__ float sigmoid_ref(float x) { return 1.f / (1.f + expf(-x)); }
 
+// Gate non-linearities.  float32 runs use the accurate library functions in the reference's own
+// formulation (1e-5 relative is the bar there).  bfloat16 runs round every result to 8 bits of
+// mantissa anyway, so they use the hardware exp2 and reciprocal (about 1 ulp of float32 each):
+// sigmoid(x) = 1 / (1 + 2^(-x log2 e)), tanh(x) = 2 sigmoid(2x) - 1.
+template <typename AT>
+struct Act;
+
+template <>
+struct Act<float> {
+  static __device__ __forceinline__ float sigmoid(float x) { return sigmoid_ref(x); }
+  static __device__ __forceinline__ float tanh(float x) { return tanhf(x); }
+};
+
+template <>
+struct Act<__bf16> {
+  static __device__ __forceinline__ float sigmoid(float x) {
+    return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+  }
+  static __device__ __forceinline__ float tanh(float x) {
+    return 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-2.8853900817779268f * x)) - 1.f;
+  }
+};
+
 // Frame visited at step s.
 __device__ __forceinline__ long long frame_of(const Lstm2Params& p, int s) {
   return (long long)p.first + (long long)s * p.step;
@@ -134,8 +157,15 @@ __global__ void k_prepare_mfma(Lstm2Params p, int n_flags) {
   for (long long idx = gtid; idx < bn; idx += gsz) {
     const int b = (int)(idx / p.n), c = (int)(idx % p.n);
     const int g = b / p.Bg, bl = b % p.Bg;
-    const long long dst = ((long long)g * 2) * hx_buf + ((long long)(c / KE) * p.Bp + bl) * KE + (c % KE);
+    const long long dst = ((long long)g * p.hx_bufs) * hx_buf + ((long long)(c / KE) * p.Bp + bl) * KE + (c % KE);
     ((AT*)p.hx)[dst] = ((const AT*)p.y0)[idx];
+  }
+  if (p.hx_sentinel) {
+    // buffers 1.. of every group: all ones = "not yet written"
+    const long long words_per_buf = hx_buf * (long long)sizeof(AT) / 4;
+    const long long total = (long long)p.groups * p.hx_bufs * words_per_buf;
+    for (long long w = gtid; w < total; w += gsz)
+      if ((w / words_per_buf) % p.hx_bufs != 0) ((unsigned*)p.hx)[w] = 0xFFFFFFFFu;
   }
   // W -> Wp
   const int S = p.n / KM;
@@ -212,7 +242,7 @@ __global__ void k_step_generic(Lstm2Params p, int s) {
     g3 += yk * Elem<AT>::load(p.W, w + 3 * (size_t)n);
   }
   const float m = p.mask[t * p.B + b];
-  const float a0 = tanhf(g0), a1 = sigmoid_ref(g1), a2 = sigmoid_ref(g2), a3 = sigmoid_ref(g3);
+  const float a0 = Act<AT>::tanh(g0), a1 = Act<AT>::sigmoid(g1), a2 = Act<AT>::sigmoid(g2), a3 = Act<AT>::sigmoid(g3);
   Elem<AT>::store(p.H, xoff, a0);
   Elem<AT>::store(p.H, xoff + n, a1);
   Elem<AT>::store(p.H, xoff + 2 * (size_t)n, a2);
@@ -220,7 +250,7 @@ __global__ void k_step_generic(Lstm2Params p, int s) {
   const float pc = c_in[idx];
   const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
   p.C[t * bn + idx] = c;
-  const float y = Elem<AT>::round(tanhf(c) * a3 * m);
+  const float y = Elem<AT>::round(Act<AT>::tanh(c) * a3 * m);
   Elem<AT>::store(p.Y, t * bn + idx, y);
   Elem<AT>::store(y_out, idx, y + Elem<AT>::load(y_in, idx) * (1.f - m));
   if (s == p.nsteps - 1) p.d[idx] = c;
@@ -294,7 +324,8 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
   constexpr int U = (NT >= 4) ? 4 : 8;                // macro steps whose h fragments are in flight together
 
   extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in a scalar register
   const int n = p.n, S = n / KM;
   i32x4* Wl = (i32x4*)smem;                                  // [MT][S][64] fragments
   f32x4* red = (f32x4*)(smem + (size_t)MT * S * kTileBytes);  // [kWaves][TILES][64]
@@ -306,7 +337,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
   const bool persist = (s_end - s_begin) > 1;
   const long long bn = (long long)p.B * n;
   const size_t hx_buf_bytes = (size_t)n * p.Bp * sizeof(AT);
-  unsigned char* hx_g = (unsigned char*)p.hx + (size_t)g * 2 * hx_buf_bytes;
+  unsigned char* hx_g = (unsigned char*)p.hx + (size_t)g * p.hx_bufs * hx_buf_bytes;
   const unsigned* flags_g = p.flags + (size_t)g * p.wgs_per_group;
 
   // W slice of this workgroup: global (already in fragment order) -> LDS, once per launch.
@@ -425,13 +456,13 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
 #pragma unroll
         for (int w = 1; w < kWaves; ++w) gsum += red[(w * TILES + e) * 64 + lane];
         const float m = msk[j];
-        const float a0 = tanhf(gsum[0] + xg[j][0]);
-        const float a1 = sigmoid_ref(gsum[1] + xg[j][1]);
-        const float a2 = sigmoid_ref(gsum[2] + xg[j][2]);
-        const float a3 = sigmoid_ref(gsum[3] + xg[j][3]);
+        const float a0 = Act<AT>::tanh(gsum[0] + xg[j][0]);
+        const float a1 = Act<AT>::sigmoid(gsum[1] + xg[j][1]);
+        const float a2 = Act<AT>::sigmoid(gsum[2] + xg[j][2]);
+        const float a3 = Act<AT>::sigmoid(gsum[3] + xg[j][3]);
         const float pc = c_state[j];
         const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
-        const float y = E::round(tanhf(c) * a3 * m);
+        const float y = E::round(Act<AT>::tanh(c) * a3 * m);
         const float hn = E::round(y + h_prev[j] * (1.f - m));
         c_state[j] = c;
         h_prev[j] = hn;
@@ -480,6 +511,269 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
     for (int j = 0; j < EPT; ++j)
       if (e_valid[j]) p.d[(long long)(b_base + e_b[j]) * n + e_cell[j]] = c_state[j];
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Persistent kernel with the recurrent weights in registers and a barrier-free exchange.
+//
+// Same decomposition and the same arithmetic per output element as k_lstm2_mfma (k dealt
+// round-robin to the 4 wavefronts, partial tiles summed in wave order), but:
+//  * every wavefront keeps the A-operand fragments of its k share in VGPRs for all steps
+//    (MT * KSMAX fragments of 4 registers), so a step reads no weights from LDS or memory;
+//  * there is no flag barrier.  The hidden state travels through a ring of 4 buffers whose
+//    elements validate themselves: a buffer starts as all-ones words ("not yet written", a NaN
+//    pattern the producers never emit), every element is written exactly once per use by the
+//    workgroup that owns the cell, and a consumer simply re-reads the fragments it needs, with
+//    device-scope loads, until none of their elements is all-ones.  One store -> load hop per
+//    step instead of store, acknowledge, flag, poll, load.
+//    Step s reads buffer s%4, writes its outputs to (s+1)%4 and re-arms its own elements of
+//    (s+3)%4 = (s-1)%4, which every workgroup has finished reading (this workgroup has seen
+//    all outputs of step s-1).  The re-arm stores are acknowledged (vmcnt(0)) before this
+//    workgroup's next output stores, which precede anybody's first look at that buffer for step
+//    s+3, so a consumer can never mistake an old value for a new one.
+// Waits are bounded as in k_lstm2_mfma.
+// ---------------------------------------------------------------------------------------------
+template <typename AT>
+struct Sentinel;
+
+template <>
+struct Sentinel<float> {
+  static __device__ __forceinline__ bool complete(i32x4 v) {
+    const unsigned a = max(max((unsigned)v[0], (unsigned)v[1]), max((unsigned)v[2], (unsigned)v[3]));
+    return a != 0xFFFFFFFFu;
+  }
+  // value as stored: NaNs are canonicalised so that no payload equals the sentinel
+  static __device__ __forceinline__ unsigned bits(float v) { return (v != v) ? 0x7FC00000u : __builtin_bit_cast(unsigned, v); }
+  static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t rs, unsigned off, unsigned bits) {
+    __builtin_amdgcn_raw_buffer_store_b32(bits, rs, off, 0, kAuxDevice);
+  }
+  static constexpr unsigned kSentinel = 0xFFFFFFFFu;
+};
+
+template <>
+struct Sentinel<__bf16> {
+  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ bool complete(i32x4 v) {
+    const u16x2 a = __builtin_elementwise_max(
+        __builtin_elementwise_max(__builtin_bit_cast(u16x2, v[0]), __builtin_bit_cast(u16x2, v[1])),
+        __builtin_elementwise_max(__builtin_bit_cast(u16x2, v[2]), __builtin_bit_cast(u16x2, v[3])));
+    return a.x != 0xFFFFu && a.y != 0xFFFFu;
+  }
+  static __device__ __forceinline__ unsigned bits(float v) {
+    return (v != v) ? 0x7FC0u : (unsigned)__builtin_bit_cast(unsigned short, (__bf16)v);
+  }
+  static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t rs, unsigned off, unsigned bits) {
+    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)bits, rs, off, 0, kAuxDevice);
+  }
+  static constexpr unsigned kSentinel = 0xFFFFu;
+};
+
+constexpr int kHxRing = 4;
+
+template <typename AT, int MT, int NT, int KSMAX>
+__global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) {
+  using E = Elem<AT>;
+  using SN = Sentinel<AT>;
+  constexpr int KE = E::KE;
+  constexpr int KM = E::KM;
+  constexpr int TILES = MT * NT;
+  constexpr int EPT = (TILES + kWaves - 1) / kWaves;
+  static_assert(KSMAX * NT <= 32, "pending mask is 32 bits");
+
+  __shared__ f32x4 red[2][kWaves][TILES][64];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in a scalar register
+  const int n = p.n, S = n / KM;
+  int g, r;
+  map_block(p, blockIdx.x, g, r);
+  const int b_base = g * p.Bg;
+  const int rows = min(p.Bg, p.B - b_base);
+  const long long bn = (long long)p.B * n;
+  const size_t hx_buf_bytes = (size_t)n * p.Bp * sizeof(AT);
+  unsigned char* hx_g = (unsigned char*)p.hx + (size_t)g * kHxRing * hx_buf_bytes;
+  const int kg = lane >> 4, jl = lane & 15;
+  const int ks_count = (S > wave) ? (S - wave + kWaves - 1) / kWaves : 0;  // macro steps of this wave
+
+  // A-operand fragments of this wave's k share: registers, for the whole sequence.
+  i32x4 wreg[MT][KSMAX];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks) {
+      const int sm = wave + kWaves * ks;
+      wreg[mt][ks] = i32x4{0, 0, 0, 0};
+      if (ks < ks_count) wreg[mt][ks] = ((const i32x4*)p.Wp)[((size_t)(r * MT + mt) * S + sm) * 64 + lane];
+    }
+
+  // Fragments this lane has to fetch each step: bit ks*NT+nt.
+  unsigned pend0 = 0;
+#pragma unroll
+  for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      if (ks < ks_count && 16 * nt + jl < rows) pend0 |= 1u << (ks * NT + nt);
+
+  float c_state[EPT], h_prev[EPT];
+  int e_b[EPT], e_cell[EPT];
+  bool e_valid[EPT];
+  unsigned e_hoff[EPT];
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int e = wave + kWaves * j;
+    const int mt = e / NT, nt = e % NT;
+    const int bl = 16 * nt + (lane & 15);
+    e_cell[j] = 4 * (r * MT + mt) + (lane >> 4);
+    e_b[j] = bl;
+    e_valid[j] = (e < TILES) && (bl < rows);
+    e_hoff[j] = (unsigned)((((e_cell[j] / KE) * p.Bp + bl) * KE + (e_cell[j] % KE)) * (int)sizeof(AT));
+    c_state[j] = 0.f;
+    h_prev[j] = 0.f;
+    if (e_valid[j]) {
+      const long long bc = (long long)(b_base + bl) * n + e_cell[j];
+      c_state[j] = p.c0[bc];
+      h_prev[j] = E::load(p.y0, bc);
+    }
+  }
+
+  for (int s = 0; s < p.nsteps; ++s) {
+    const long long t = frame_of(p, s);
+
+    float xg[EPT][4], msk[EPT];
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      msk[j] = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) xg[j][q] = 0.f;
+      if (e_valid[j]) {
+        const size_t xo = ((size_t)t * p.B + (b_base + e_b[j])) * 4 * n + e_cell[j];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) xg[j][q] = E::load(p.X, xo + (size_t)q * n);
+        msk[j] = p.mask[t * p.B + b_base + e_b[j]];
+      }
+    }
+
+    // Fetch this wave's share of h_{s-1}; repeat for the fragments that are not complete yet.
+    const unsigned char* hx_cur = hx_g + (size_t)(s & (kHxRing - 1)) * hx_buf_bytes;
+    __amdgpu_buffer_rsrc_t cur_rs = __builtin_amdgcn_make_buffer_rsrc((void*)hx_cur, 0, 0x7fffffff, kBufFlags);
+    i32x4 bf[KSMAX][NT];
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) bf[ks][nt] = i32x4{0, 0, 0, 0};
+    unsigned pend = pend0;
+    unsigned long long t0 = 0;
+    unsigned spins = 0;
+    for (;;) {
+      asm volatile("" ::: "memory");  // other workgroups write this memory: load again on every trip
+#pragma unroll
+      for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          if (pend & (1u << (ks * NT + nt))) {
+            const unsigned off = (unsigned)(((4 * (wave + kWaves * ks) + kg) * p.Bp + 16 * nt + jl) * kFragBytes);
+            bf[ks][nt] =
+                __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(cur_rs, off, 0, kAuxDevice));
+          }
+#pragma unroll
+      for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          if ((pend & (1u << (ks * NT + nt))) && SN::complete(bf[ks][nt])) pend &= ~(1u << (ks * NT + nt));
+      if (!__any(pend != 0)) break;
+      if ((spins++ & 15u) == 0) {
+        if (__hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+        const unsigned long long now = wall_clock64();
+        if (spins == 1) {
+          t0 = now;
+        } else if (now - t0 > p.timeout_ticks) {
+          __hip_atomic_store(p.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+      }
+    }
+
+    f32x4 acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks)
+      if (ks < ks_count) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+      }
+
+    f32x4(*redbuf)[TILES][64] = red[s & 1];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) redbuf[wave][mt * NT + nt][lane] = acc[mt][nt];
+    __syncthreads();  // the only workgroup barrier of a step; `red` alternates between two copies
+
+    __amdgpu_buffer_rsrc_t nxt_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(hx_g + (size_t)((s + 1) & (kHxRing - 1)) * hx_buf_bytes), 0, 0x7fffffff, kBufFlags);
+    __amdgpu_buffer_rsrc_t arm_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(hx_g + (size_t)((s + 3) & (kHxRing - 1)) * hx_buf_bytes), 0, 0x7fffffff, kBufFlags);
+    float a_out[EPT][4], y_out[EPT];
+    unsigned h_bits[EPT];
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      const int e = wave + kWaves * j;
+      h_bits[j] = 0;
+      if (e < TILES) {
+        f32x4 gsum = redbuf[0][e][lane];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) gsum += redbuf[w][e][lane];
+        const float m = msk[j];
+        const float a0 = Act<AT>::tanh(gsum[0] + xg[j][0]);
+        const float a1 = Act<AT>::sigmoid(gsum[1] + xg[j][1]);
+        const float a2 = Act<AT>::sigmoid(gsum[2] + xg[j][2]);
+        const float a3 = Act<AT>::sigmoid(gsum[3] + xg[j][3]);
+        const float pc = c_state[j];
+        const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
+        const float y = E::round(Act<AT>::tanh(c) * a3 * m);
+        const float hn = E::round(y + h_prev[j] * (1.f - m));
+        c_state[j] = c;
+        h_prev[j] = hn;
+        y_out[j] = y;
+        a_out[j][0] = a0;
+        a_out[j][1] = a1;
+        a_out[j][2] = a2;
+        a_out[j][3] = a3;
+        h_bits[j] = SN::bits(hn);
+      }
+    }
+    // The re-arm stores of the previous step (and everything older) are acknowledged before the
+    // new hidden values go out.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int j = 0; j < EPT; ++j)
+      if (e_valid[j]) SN::store(nxt_rs, e_hoff[j], h_bits[j]);
+
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      if (e_valid[j]) {
+        const long long bc = (long long)(b_base + e_b[j]) * n + e_cell[j];
+        const size_t xo = ((size_t)t * p.B + (b_base + e_b[j])) * 4 * n + e_cell[j];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) E::store(p.H, xo + (size_t)q * n, a_out[j][q]);
+        p.C[t * bn + bc] = c_state[j];
+        E::store(p.Y, t * bn + bc, y_out[j]);
+      }
+    }
+    // Re-arm this thread's elements of the buffer everybody read one step ago.
+#pragma unroll
+    for (int j = 0; j < EPT; ++j)
+      if (e_valid[j]) SN::store(arm_rs, e_hoff[j], SN::kSentinel);
+  }
+
+#pragma unroll
+  for (int j = 0; j < EPT; ++j)
+    if (e_valid[j]) p.d[(long long)(b_base + e_b[j]) * n + e_cell[j]] = c_state[j];
 }
 
 }  // namespace rtn

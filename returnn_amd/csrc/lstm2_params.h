@@ -29,7 +29,7 @@ struct Lstm2Params {
   // workspace sections (device)
   unsigned* status;  // [64]   status[0] != 0: a bounded wait expired
   unsigned* flags;   // [groups*wgs_per_group] last published step (+1) of each workgroup
-  void* hx;          // [groups][2][n/KE][Bp][KE] AT: hidden state in MFMA B-operand order, double buffered
+  void* hx;          // [groups][hx_bufs][n/KE][Bp][KE] AT: hidden state in MFMA B-operand order, ring of buffers
   void* Wp;          // [n/4][S][64][16 bytes]: W in MFMA A-operand order
   void* ycarry;      // [2][B][n] AT: hidden-state carry of the generic per-step kernels
   // sizes
@@ -43,6 +43,8 @@ struct Lstm2Params {
   int wgs_per_group;  // workgroups per group (each owns MT*4 cells)
   int Bg;             // batch rows per group
   int Bp;             // rows of one hx buffer (= 16*NT)
+  int hx_bufs;        // buffers in the hx ring: 2 with the flag barrier, 4 with self-validating data
+  int hx_sentinel;    // 1: buffers 1.. start filled with the "not yet written" bit pattern (all ones)
   int xcds;           // XCDs assumed for the blockIdx -> (group, rank) mapping
   int sync_policy;    // SyncBits
   unsigned long long timeout_ticks;  // bound of one flag wait, in 100 MHz wall-clock ticks

@@ -94,6 +94,8 @@ enum PlanKind { kPlanEmpty, kPlanGeneric, kPlanMfma };
 struct Plan {
   PlanKind kind = kPlanGeneric;
   int mode = RTN_MODE_STEPWISE;  // resolved: PERSISTENT, GRAPH or STEPWISE
+  bool regw = false;             // persistent kernel with W in registers and self-validating exchange
+  int KSMAX = 0;                 // its macro steps per wavefront (template bound)
   int MT = 1, NT = 1;
   int groups = 1, wgs_per_group = 1, Bg = 1, Bp = 16;
   size_t lds_bytes = 0;
@@ -130,33 +132,55 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
   bool persistent_ok = false;
   if (mfma_shape && !force_generic) {
     pl.kind = kPlanMfma;
-    // Persistent candidates: smallest MT whose grid fits the device and whose W slice fits LDS.
+    // Persistent candidates: every (MT, groups) whose grid fits the device with W on chip.  The register
+    // kernel is preferred; among its candidates the estimated step time decides: MFMA cycles of one
+    // wavefront plus an exchange term that grows with the number of workgroups that have to hear of
+    // each other and with the rows every one of them has to fetch.
     const long env_mt = env_long("RTN_LSTM2_MT", 0);
     const long env_groups = env_long("RTN_LSTM2_GROUPS", 0);
+    const long env_kernel = env_long("RTN_LSTM2_KERNEL", 0);  // 0 auto, 1 LDS + flag barrier, 2 registers + self-validating data
+    const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
+    const int S = n / KM;
+    const int ks = (S + kWaves - 1) / kWaves;
+    const int KSMAX = ks <= 8 ? 8 : (ks <= 16 ? 16 : 0);
     if (want_mode == RTN_MODE_AUTO || want_mode == RTN_MODE_PERSISTENT) {
-      for (int MT : {1, 2, 4}) {
-        if (env_mt && MT != env_mt) continue;
-        if ((n / 4) % MT) continue;
-        const int G = n / (4 * MT);
-        if (G > di.cus) continue;
-        int max_groups = di.cus / G;
-        int groups = std::min(max_groups, (B + 15) / 16);
-        if (env_groups) groups = (int)std::min<long>(env_groups, max_groups);
-        groups = std::max(1, std::min(groups, B));
-        int Bg = (B + groups - 1) / groups;
-        groups = (B + Bg - 1) / Bg;
-        int NT = round_nt((Bg + 15) / 16);
-        if ((Bg + 15) / 16 > 4) continue;
-        const size_t lds = mfma_lds_bytes(n, dtype, MT, NT);
-        if (lds > di.lds_per_wg) continue;
-        pl.MT = MT;
-        pl.NT = NT;
-        pl.groups = groups;
-        pl.wgs_per_group = G;
-        pl.Bg = Bg;
-        pl.lds_bytes = lds;
-        persistent_ok = true;
-        break;
+      double best = 1e30;
+      for (int use_regw = 1; use_regw >= 0; --use_regw) {
+        if (use_regw && (env_kernel == 1 || KSMAX == 0)) continue;
+        if (!use_regw && (env_kernel == 2 || persistent_ok)) continue;
+        for (int MT : {1, 2, 4}) {
+          if (env_mt && MT != env_mt) continue;
+          if ((n / 4) % MT) continue;
+          const int G = n / (4 * MT);
+          if (G > di.cus) continue;
+          if (use_regw && MT * KSMAX > 32) continue;
+          const int max_groups = di.cus / G;
+          for (int groups = 1; groups <= std::min(max_groups, B); ++groups) {
+            if (env_groups && groups != std::min<long>(env_groups, std::min(max_groups, B))) continue;
+            const int Bg = (B + groups - 1) / groups;
+            if ((B + Bg - 1) / Bg != groups) continue;  // same rows per group would need fewer groups
+            if ((Bg + 15) / 16 > 4) continue;
+            const int NT = round_nt((Bg + 15) / 16);
+            if (use_regw && NT * KSMAX > 32) continue;
+            const size_t lds = use_regw ? (size_t)2 * kWaves * MT * NT * kTileBytes : mfma_lds_bytes(n, dtype, MT, NT);
+            if (lds > (use_regw ? (size_t)64 * 1024 : di.lds_per_wg)) continue;
+            const double mfma_us = (double)MT * NT * ks * (dtype == RTN_DTYPE_BF16 ? 16 : 128) / 2400.0;
+            const double exch_us = 1.0 + 0.004 * G + 0.01 * Bg;
+            const double est = mfma_us + exch_us;
+            if (est < best) {
+              best = est;
+              pl.regw = use_regw != 0;
+              pl.KSMAX = use_regw ? KSMAX : 0;
+              pl.MT = MT;
+              pl.NT = NT;
+              pl.groups = groups;
+              pl.wgs_per_group = G;
+              pl.Bg = Bg;
+              pl.lds_bytes = use_regw ? 0 : lds;
+              persistent_ok = true;
+            }
+          }
+        }
       }
       if (!persistent_ok && why) *why = "no decomposition keeps W on chip with all workgroups co-resident";
     }
@@ -171,6 +195,8 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
     if (!persistent_ok) {
       // Per-step launches have no co-residency limit: 4 cells per workgroup, groups of <= 64 rows.
       int MT = 1;
+      pl.regw = false;
+      pl.KSMAX = 0;
       if (mfma_lds_bytes(n, dtype, 1, 4) > di.lds_per_wg) {
         pl.kind = kPlanGeneric;  // a W slice of 16 columns does not fit LDS (n far beyond the target sizes)
       } else {
@@ -206,7 +232,7 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
   off = align_up(off + (size_t)pl.n_flags * 4, 256);
   if (pl.kind == kPlanMfma) {
     pl.off_hx = off;
-    off = align_up(off + (size_t)pl.groups * 2 * n * pl.Bp * es, 256);
+    off = align_up(off + (size_t)pl.groups * kHxRing * n * pl.Bp * es, 256);
     pl.off_wp = off;
     off = align_up(off + (size_t)4 * n * n * es, 256);
   } else {
@@ -242,6 +268,25 @@ MfmaKernel mfma_kernel_for(int MT, int NT) {
 
 MfmaKernel mfma_kernel(int dtype, int MT, int NT) {
   return dtype == RTN_DTYPE_BF16 ? mfma_kernel_for<__bf16>(MT, NT) : mfma_kernel_for<float>(MT, NT);
+}
+
+typedef void (*RegwKernel)(const Lstm2Params);
+
+template <typename AT>
+RegwKernel regw_kernel_for(int MT, int NT, int KSMAX) {
+#define RTN_CASE(mt, nt, ks) \
+  if (MT == mt && NT == nt && KSMAX == ks) return &k_lstm2_regw<AT, mt, nt, ks>;
+  RTN_CASE(1, 1, 8) RTN_CASE(1, 2, 8) RTN_CASE(1, 4, 8)
+  RTN_CASE(2, 1, 8) RTN_CASE(2, 2, 8) RTN_CASE(2, 4, 8)
+  RTN_CASE(4, 1, 8) RTN_CASE(4, 2, 8) RTN_CASE(4, 4, 8)
+  RTN_CASE(1, 1, 16) RTN_CASE(1, 2, 16)
+  RTN_CASE(2, 1, 16) RTN_CASE(2, 2, 16)
+#undef RTN_CASE
+  return nullptr;
+}
+
+RegwKernel regw_kernel(int dtype, int MT, int NT, int KSMAX) {
+  return dtype == RTN_DTYPE_BF16 ? regw_kernel_for<__bf16>(MT, NT, KSMAX) : regw_kernel_for<float>(MT, NT, KSMAX);
 }
 
 // Kernels that use more than the default LDS limit need the limit raised once per device.
@@ -390,7 +435,8 @@ const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int3
     g_plan_text = "unsupported: " + why;
   } else {
     snprintf(buf, sizeof(buf), "mode=%s kernel=%s mt=%d nt=%d groups=%d wgs_per_group=%d wgs=%d rows_per_group=%d lds=%zu workspace=%zu",
-             mode_name(pl.mode), pl.kind == kPlanMfma ? "mfma" : (pl.kind == kPlanGeneric ? "generic" : "empty"), pl.MT,
+             mode_name(pl.mode),
+             pl.kind == kPlanMfma ? (pl.regw ? "mfma_regw" : "mfma_lds") : (pl.kind == kPlanGeneric ? "generic" : "empty"), pl.MT,
              pl.NT, pl.groups, pl.wgs_per_group, pl.groups * pl.wgs_per_group, pl.Bg, pl.lds_bytes, pl.total);
     g_plan_text = buf;
   }
@@ -458,6 +504,8 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
   }
   p.step = step;
   p.groups = pl.groups; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
+  p.hx_bufs = kHxRing;
+  p.hx_sentinel = pl.regw ? 1 : 0;
   p.xcds = device_info().xcds;
   p.sync_policy = (int)env_long("RTN_LSTM2_SYNC", kStoreCoherent | kLoadCoherent);
   if (!((p.sync_policy & (kStoreCoherent | kReleaseFence)) && (p.sync_policy & (kLoadCoherent | kAcquireFence))))
@@ -476,10 +524,37 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
   }
 
   if (pl.kind == kPlanMfma) {
+    const void* pk = nullptr;  // the persistent kernel, if any
+    if (pl.mode == RTN_MODE_PERSISTENT) {
+      pk = pl.regw ? (const void*)regw_kernel(dtype, pl.MT, pl.NT, pl.KSMAX) : (const void*)mfma_kernel(dtype, pl.MT, pl.NT);
+      if (!pk) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d ks=%d", pl.MT, pl.NT, pl.KSMAX);
+      if (!pl.regw) {
+        rc = ensure_lds_limit((MfmaKernel)pk, pl.lds_bytes);
+        if (rc != RTN_OK) return rc;
+      }
+      // All workgroups have to be on the device together.
+      const int wgs = pl.groups * pl.wgs_per_group;
+      int per_cu = 0;
+      RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, pk, kWgThreads, pl.lds_bytes));
+      if ((long long)per_cu * device_info().cus < wgs) {
+        if (mode == RTN_MODE_PERSISTENT)
+          return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: %d workgroups cannot be co-resident (%d per CU)", wgs, per_cu);
+        // AUTO: plan again for per-step launches (same workspace, it was sized for both).
+        if (!make_plan(T, B, n, dtype, RTN_MODE_GRAPH, capturing, &pl, &why) || workspace_bytes < pl.total)
+          return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no per-step plan fits the workspace");
+        p.hx = ws + pl.off_hx;
+        p.Wp = ws + pl.off_wp;
+        p.groups = pl.groups; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
+        p.hx_sentinel = 0;
+        pk = nullptr;
+      }
+    }
     MfmaKernel k = mfma_kernel(dtype, pl.MT, pl.NT);
-    if (!k) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d", pl.MT, pl.NT);
-    rc = ensure_lds_limit(k, pl.lds_bytes);
-    if (rc != RTN_OK) return rc;
+    if (!pk) {
+      if (!k) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d", pl.MT, pl.NT);
+      rc = ensure_lds_limit(k, pl.lds_bytes);
+      if (rc != RTN_OK) return rc;
+    }
     const long long work = std::max<long long>((long long)n * n, bn);
     const dim3 pgrid((unsigned)std::min<long long>((work + 255) / 256, 2048)), pblock(256);
     if (dtype == RTN_DTYPE_BF16)
@@ -487,20 +562,14 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
     else
       hipLaunchKernelGGL(k_prepare_mfma<float>, pgrid, pblock, 0, stream, p, pl.n_flags);
     RTN_HIP(hipGetLastError());
-    if (pl.mode == RTN_MODE_PERSISTENT) {
+    if (pk) {
       const int wgs = pl.groups * pl.wgs_per_group;
-      int per_cu = 0;
-      RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)k, kWgThreads, pl.lds_bytes));
-      if ((long long)per_cu * device_info().cus < wgs) {
-        if (mode == RTN_MODE_PERSISTENT)
-          return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: %d workgroups cannot be co-resident (%d per CU)", wgs, per_cu);
-        pl.mode = RTN_MODE_GRAPH;  // AUTO: fall through to the per-step path with the same layout
-      } else {
-        int s_begin = 0, s_end = p.nsteps;
-        void* args[] = {(void*)&p, (void*)&s_begin, (void*)&s_end};
-        RTN_HIP(hipLaunchCooperativeKernel((const void*)k, dim3(wgs), dim3(kWgThreads), args, (unsigned)pl.lds_bytes, stream));
-        return RTN_OK;
-      }
+      int s_begin = 0, s_end = p.nsteps;
+      void* args_lds[] = {(void*)&p, (void*)&s_begin, (void*)&s_end};
+      void* args_regw[] = {(void*)&p};
+      RTN_HIP(hipLaunchCooperativeKernel(pk, dim3(wgs), dim3(kWgThreads), pl.regw ? args_regw : args_lds,
+                                         (unsigned)pl.lds_bytes, stream));
+      return RTN_OK;
     }
   } else {
     hipLaunchKernelGGL(k_clear_status, dim3(1), dim3(64), 0, stream, p.status);

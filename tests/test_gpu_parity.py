@@ -92,11 +92,12 @@ def test_mfma_shapes(T, B, n, dtype, mode):
 @pytest.mark.parametrize("policy", sorted(SYNC_POLICIES))
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_persistent_sync_policies(policy, dtype):
-    """Both ways of publishing the hidden state between workgroups give the per-step kernels' result bit for bit."""
+    """LDS-resident persistent kernel with its flag barrier: both ways of publishing the hidden state between
+    workgroups give the per-step kernels' result bit for bit."""
     announce("sync_policy", policy, dtype)
     p = random_problem(7, 40, 24, 256)
     base = run_op(*p, 0, 1, dtype=dtype, mode="stepwise")
-    with env(RTN_LSTM2_SYNC=SYNC_POLICIES[policy]):
+    with env(RTN_LSTM2_SYNC=SYNC_POLICIES[policy], RTN_LSTM2_KERNEL=1):
         for step in (1, -1):
             ref = run_op(*p, 0, step, dtype=dtype, mode="stepwise")
             got = run_op(*p, 0, step, dtype=dtype, mode="persistent")
@@ -106,15 +107,38 @@ def test_persistent_sync_policies(policy, dtype):
 
 
 @pytest.mark.parametrize("mt,groups", [(1, 1), (2, 2), (4, 4), (2, 1), (4, 8)])
-def test_decompositions(mt, groups):
-    """Cells per workgroup and batch groups are a tuning choice, never a change of results (up to summation order)."""
-    announce("decompositions", mt, groups)
+@pytest.mark.parametrize("kernel", [1, 2])
+def test_decompositions(mt, groups, kernel):
+    """Cells per workgroup, batch groups and the persistent kernel variant (1: W in LDS + flag barrier, 2: W in
+    registers + self-validating exchange) are tuning choices: every one of them reproduces the per-step kernels
+    bit for bit (same split of k over wavefronts, same summation order) and matches the oracle."""
+    announce("decompositions", mt, groups, kernel)
     p = random_problem(11, 30, 48, 512)
     want = oracle.native_lstm2_fwd(*p, 0, 1)
-    with env(RTN_LSTM2_MT=mt, RTN_LSTM2_GROUPS=groups):
-        for dtype, chk in (("f32", check_f32), ("bf16", check_bf16)):
+    for dtype, chk in (("f32", check_f32), ("bf16", check_bf16)):
+        ref = run_op(*p, 0, 1, dtype=dtype, mode="stepwise")
+        with env(RTN_LSTM2_MT=mt, RTN_LSTM2_GROUPS=groups, RTN_LSTM2_KERNEL=kernel):
             got = run_op(*p, 0, 1, dtype=dtype, mode="persistent")
-            chk(got, want, "decomposition mt=%i groups=%i %s" % (mt, groups, dtype))
+        chk(got, want, "decomposition mt=%i groups=%i kernel=%i %s" % (mt, groups, kernel, dtype))
+        for a, b in zip(got, ref):
+            assert numpy.array_equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_register_kernel_long_ring(dtype):
+    """The exchange ring of 4 buffers wraps many times; ragged lengths, both directions, NaN-free and equal to the
+    per-step result bit for bit.  n=1024 (bf16: 8 macro steps per wavefront; f32: 16)."""
+    announce("register kernel ring", dtype)
+    p = random_problem(71, 203, 9, 1024)
+    for step in (1, -1):
+        ref = run_op(*p, 0, step, dtype=dtype, mode="stepwise")
+        with env(RTN_LSTM2_KERNEL=2):
+            got = run_op(*p, 0, step, dtype=dtype, mode="persistent")
+        for a, b in zip(got, ref):
+            assert numpy.array_equal(a, b)
+    want = oracle.native_lstm2_fwd(*p, 0, 1, threads=oracle.max_threads())
+    got = run_op(*p, 0, 1, dtype=dtype, mode="persistent")
+    (check_f32 if dtype == "f32" else check_bf16)(got, want, "ring " + dtype)
 
 
 def test_cfg1_fp32():
@@ -325,13 +349,15 @@ def test_bounded_wait_expires_cleanly():
 
     announce("bounded wait")
     p = random_problem(61, 50, 8, 256)
-    with env(RTN_LSTM2_TIMEOUT_TICKS=0):
-        rc, status, got = run_raw(*p, 0, 1, mode="persistent")
-    assert rc == 0
-    assert status in (lib.RTN_OK, lib.RTN_ERR_ABORTED)
-    if status == lib.RTN_OK:
-        check_f32(got, oracle.native_lstm2_fwd(*p, 0, 1)[:4], "bounded wait")
-    # and the next ordinary call is unaffected
-    rc, status, got = run_raw(*p, 0, 1, mode="persistent")
-    assert rc == 0 and status == 0
-    check_f32(got, oracle.native_lstm2_fwd(*p, 0, 1)[:4], "after bounded wait")
+    for kernel in (1, 2):
+        with env(RTN_LSTM2_TIMEOUT_TICKS=0, RTN_LSTM2_KERNEL=kernel):
+            rc, status, got = run_raw(*p, 0, 1, mode="persistent")
+        assert rc == 0
+        assert status in (lib.RTN_OK, lib.RTN_ERR_ABORTED)
+        if status == lib.RTN_OK:
+            check_f32(got, oracle.native_lstm2_fwd(*p, 0, 1)[:4], "bounded wait")
+        # and the next ordinary call is unaffected
+        with env(RTN_LSTM2_KERNEL=kernel):
+            rc, status, got = run_raw(*p, 0, 1, mode="persistent")
+        assert rc == 0 and status == 0
+        check_f32(got, oracle.native_lstm2_fwd(*p, 0, 1)[:4], "after bounded wait")
