@@ -552,12 +552,14 @@ struct Sentinel<float> {
 
 template <>
 struct Sentinel<__bf16> {
-  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+  // Non-zero iff one of the two halfwords of x is 0xFFFF: the classic "has a zero lane" test on ~x
+  // (exact for the any-lane question).
+  static __device__ __forceinline__ unsigned has_ffff(unsigned x) {
+    const unsigned y = ~x;
+    return (y - 0x00010001u) & x & 0x80008000u;
+  }
   static __device__ __forceinline__ bool complete(i32x4 v) {
-    const u16x2 a = __builtin_elementwise_max(
-        __builtin_elementwise_max(__builtin_bit_cast(u16x2, v[0]), __builtin_bit_cast(u16x2, v[1])),
-        __builtin_elementwise_max(__builtin_bit_cast(u16x2, v[2]), __builtin_bit_cast(u16x2, v[3])));
-    return a.x != 0xFFFFu && a.y != 0xFFFFu;
+    return (has_ffff((unsigned)v[0]) | has_ffff((unsigned)v[1]) | has_ffff((unsigned)v[2]) | has_ffff((unsigned)v[3])) == 0;
   }
   static __device__ __forceinline__ unsigned bits(float v) {
     return (v != v) ? 0x7FC0u : (unsigned)__builtin_bit_cast(unsigned short, (__bf16)v);
