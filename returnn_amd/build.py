@@ -31,11 +31,14 @@ def hipcc_path() -> str:
 
 
 def compile_command(output: Optional[str] = None) -> List[str]:
-    """The exact hipcc line.  Packed fp32 VALU instructions are disabled on purpose."""
+    """The exact hipcc line.  Packed fp32 VALU instructions are disabled on purpose.  Floating-point
+    contraction is off so that every kernel variant and decomposition rounds the gate and cell arithmetic
+    identically (results do not depend on the execution mode) and like the CPU reference code."""
     return [
         hipcc_path(),
         "--offload-arch=%s" % OFFLOAD_ARCH,
         "-O3",
+        "-ffp-contract=off",
         "-std=c++17",
         "-fPIC",
         "-shared",

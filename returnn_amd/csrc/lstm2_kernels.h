@@ -518,21 +518,31 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
 //
 // Same decomposition and the same arithmetic per output element as k_lstm2_mfma (k dealt
 // round-robin to the 4 wavefronts, partial tiles summed in wave order), but:
-//  * every wavefront keeps the A-operand fragments of its k share in VGPRs for all steps
+//  * every wavefront keeps the A-operand fragments of its k share in registers for all steps
 //    (MT * KSMAX fragments of 4 registers), so a step reads no weights from LDS or memory;
 //  * there is no flag barrier.  The hidden state travels through a ring of 4 buffers whose
 //    elements validate themselves: a buffer starts as all-ones words ("not yet written", a NaN
 //    pattern the producers never emit), every element is written exactly once per use by the
-//    workgroup that owns the cell, and a consumer simply re-reads the fragments it needs, with
-//    device-scope loads, until none of their elements is all-ones.  One store -> load hop per
-//    step instead of store, acknowledge, flag, poll, load.
+//    workgroup that owns the cell, and a consumer simply re-reads the fragments it needs
+//    until none of their elements is all-ones.  One store -> load hop per step instead of
+//    store, acknowledge, flag, poll, load.
 //    Step s reads buffer s%4, writes its outputs to (s+1)%4 and re-arms its own elements of
 //    (s+3)%4 = (s-1)%4, which every workgroup has finished reading (this workgroup has seen
 //    all outputs of step s-1).  The re-arm stores are acknowledged (vmcnt(0)) before this
 //    workgroup's next output stores, which precede anybody's first look at that buffer for step
 //    s+3, so a consumer can never mistake an old value for a new one.
+//  * the scope of the exchange follows the placement.  An MI355X has 8 XCDs with one L2 each;
+//    workgroups on the same XCD can meet in that L2 (loads that only skip the per-CU cache),
+//    workgroups on different XCDs have to go to device scope (memory side).  At start every
+//    workgroup publishes the id of the XCD it runs on (device scope) and reads the ids of its
+//    group: if they are all equal the group exchanges through its L2, else at device scope.
+//    The decision is a function of the complete id table, so all members take the same one; no
+//    assumption about how the hardware deals workgroups to XCDs is needed for correctness
+//    (the blockIdx -> (group, rank) mapping only makes the good case likely).
 // Waits are bounded as in k_lstm2_mfma.
 // ---------------------------------------------------------------------------------------------
+constexpr int kAuxGroup = 1;  // cache policy: skip the per-CU cache, meet in this XCD's L2 (sc0)
+
 template <typename AT>
 struct Sentinel;
 
@@ -544,8 +554,9 @@ struct Sentinel<float> {
   }
   // value as stored: NaNs are canonicalised so that no payload equals the sentinel
   static __device__ __forceinline__ unsigned bits(float v) { return (v != v) ? 0x7FC00000u : __builtin_bit_cast(unsigned, v); }
+  template <int AUX>
   static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t rs, unsigned off, unsigned bits) {
-    __builtin_amdgcn_raw_buffer_store_b32(bits, rs, off, 0, kAuxDevice);
+    __builtin_amdgcn_raw_buffer_store_b32(bits, rs, off, 0, AUX);
   }
   static constexpr unsigned kSentinel = 0xFFFFFFFFu;
 };
@@ -564,13 +575,34 @@ struct Sentinel<__bf16> {
   static __device__ __forceinline__ unsigned bits(float v) {
     return (v != v) ? 0x7FC0u : (unsigned)__builtin_bit_cast(unsigned short, (__bf16)v);
   }
+  template <int AUX>
   static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t rs, unsigned off, unsigned bits) {
-    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)bits, rs, off, 0, kAuxDevice);
+    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)bits, rs, off, 0, AUX);
   }
   static constexpr unsigned kSentinel = 0xFFFFu;
 };
 
 constexpr int kHxRing = 4;
+
+template <int V>
+struct IntTag {
+  static constexpr int value = V;
+};
+
+// blockIdx -> (group, rank) for the register kernel.  With map_compact the grid is
+// xcds * ceil(groups / xcds) * wgs_per_group workgroups; under round-robin dealing of workgroup
+// ids to XCDs, XCD x then holds the whole groups x, x + xcds, ...; surplus workgroups (when
+// groups is not a multiple of xcds) get g = -1 and leave at once.
+__device__ __forceinline__ void map_block_regw(const Lstm2Params& p, int bid, int& g, int& r) {
+  if (p.map_compact) {
+    const int x = bid % p.xcds, q = bid / p.xcds;
+    g = (q / p.wgs_per_group) * p.xcds + x;
+    r = q % p.wgs_per_group;
+    if (g >= p.groups) g = -1;
+  } else {
+    map_block(p, bid, g, r);
+  }
+}
 
 template <typename AT, int MT, int NT, int KSMAX>
 __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) {
@@ -583,12 +615,15 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
   static_assert(KSMAX * NT <= 32, "pending mask is 32 bits");
 
   __shared__ f32x4 red[2][kWaves][TILES][64];
+  int* s_same_xcd = (int*)&red[0][0][0][0];  // borrowed before the first step (static LDS is capped at 64 KB)
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in a scalar register
   const int n = p.n, S = n / KM;
   int g, r;
-  map_block(p, blockIdx.x, g, r);
+  map_block_regw(p, blockIdx.x, g, r);
+  if (g < 0) return;
+  const int G = p.wgs_per_group;
   const int b_base = g * p.Bg;
   const int rows = min(p.Bg, p.B - b_base);
   const long long bn = (long long)p.B * n;
@@ -596,6 +631,44 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
   unsigned char* hx_g = (unsigned char*)p.hx + (size_t)g * kHxRing * hx_buf_bytes;
   const int kg = lane >> 4, jl = lane & 15;
   const int ks_count = (S > wave) ? (S - wave + kWaves - 1) / kWaves : 0;  // macro steps of this wave
+
+  // Where does the group run?  Publish this workgroup's XCD id (+1) and read the group's table.
+  {
+    unsigned* ids = p.flags + (size_t)g * G;
+    if (tid == 0) {
+      const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 0xFu;  // XCC_ID, bits [3:0]
+      __hip_atomic_store(ids + r, xcc + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (wave == 0) {
+      unsigned long long t0 = 0;
+      unsigned spins = 0;
+      bool same = true;
+      for (;;) {
+        bool all_there = true;
+        same = true;
+        const unsigned mine = __hip_atomic_load(ids + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int k = lane; k < G; k += 64) {
+          const unsigned v = __hip_atomic_load(ids + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          all_there = all_there && (v != 0);
+          same = same && (v == mine);
+        }
+        if (__all(all_there && mine != 0)) break;
+        if ((spins++ & 15u) == 0) {
+          if (__hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+          const unsigned long long now = wall_clock64();
+          if (spins == 1) {
+            t0 = now;
+          } else if (now - t0 > p.timeout_ticks) {
+            __hip_atomic_store(p.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+      const int same_all = __all(same) ? 1 : 0;
+      if (lane == 0) *s_same_xcd = (same_all && p.allow_l2_exchange) ? 1 : 0;
+    }
+  }
 
   // A-operand fragments of this wave's k share: registers, for the whole sequence.
   i32x4 wreg[MT][KSMAX];
@@ -637,141 +710,152 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
       h_prev[j] = E::load(p.y0, bc);
     }
   }
+  __syncthreads();
+  const bool same_xcd = *s_same_xcd != 0;
+  __syncthreads();  // everybody has read it; `red` is free for the steps
 
-  for (int s = 0; s < p.nsteps; ++s) {
-    const long long t = frame_of(p, s);
+  // All time steps, with the cache policy AUX for the hidden-state exchange.
+  auto run = [&](auto aux_tag) {
+    constexpr int AUX = decltype(aux_tag)::value;
+    for (int s = 0; s < p.nsteps; ++s) {
+      const long long t = frame_of(p, s);
 
-    float xg[EPT][4], msk[EPT];
+      // Gate inputs and mask of this step: independent of the recurrence, issued before the wait.
+      float xg[EPT][4], msk[EPT];
 #pragma unroll
-    for (int j = 0; j < EPT; ++j) {
-      msk[j] = 0.f;
+      for (int j = 0; j < EPT; ++j) {
+        msk[j] = 0.f;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) xg[j][q] = 0.f;
-      if (e_valid[j]) {
-        const size_t xo = ((size_t)t * p.B + (b_base + e_b[j])) * 4 * n + e_cell[j];
+        for (int q = 0; q < 4; ++q) xg[j][q] = 0.f;
+        if (e_valid[j]) {
+          const size_t xo = ((size_t)t * p.B + (b_base + e_b[j])) * 4 * n + e_cell[j];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) xg[j][q] = E::load(p.X, xo + (size_t)q * n);
-        msk[j] = p.mask[t * p.B + b_base + e_b[j]];
-      }
-    }
-
-    // Fetch this wave's share of h_{s-1}; repeat for the fragments that are not complete yet.
-    const unsigned char* hx_cur = hx_g + (size_t)(s & (kHxRing - 1)) * hx_buf_bytes;
-    __amdgpu_buffer_rsrc_t cur_rs = __builtin_amdgcn_make_buffer_rsrc((void*)hx_cur, 0, 0x7fffffff, kBufFlags);
-    i32x4 bf[KSMAX][NT];
-#pragma unroll
-    for (int ks = 0; ks < KSMAX; ++ks)
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) bf[ks][nt] = i32x4{0, 0, 0, 0};
-    unsigned pend = pend0;
-    unsigned long long t0 = 0;
-    unsigned spins = 0;
-    for (;;) {
-      asm volatile("" ::: "memory");  // other workgroups write this memory: load again on every trip
-#pragma unroll
-      for (int ks = 0; ks < KSMAX; ++ks)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          if (pend & (1u << (ks * NT + nt))) {
-            const unsigned off = (unsigned)(((4 * (wave + kWaves * ks) + kg) * p.Bp + 16 * nt + jl) * kFragBytes);
-            bf[ks][nt] =
-                __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(cur_rs, off, 0, kAuxDevice));
-          }
-#pragma unroll
-      for (int ks = 0; ks < KSMAX; ++ks)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          if ((pend & (1u << (ks * NT + nt))) && SN::complete(bf[ks][nt])) pend &= ~(1u << (ks * NT + nt));
-      if (!__any(pend != 0)) break;
-      if ((spins++ & 15u) == 0) {
-        if (__hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
-        const unsigned long long now = wall_clock64();
-        if (spins == 1) {
-          t0 = now;
-        } else if (now - t0 > p.timeout_ticks) {
-          __hip_atomic_store(p.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          break;
+          for (int q = 0; q < 4; ++q) xg[j][q] = E::load(p.X, xo + (size_t)q * n);
+          msk[j] = p.mask[t * p.B + b_base + e_b[j]];
         }
       }
-    }
 
-    f32x4 acc[MT][NT];
+      // Fetch this wave's share of h_{s-1}; repeat for the fragments that are not complete yet.
+      const unsigned char* hx_cur = hx_g + (size_t)(s & (kHxRing - 1)) * hx_buf_bytes;
+      __amdgpu_buffer_rsrc_t cur_rs = __builtin_amdgcn_make_buffer_rsrc((void*)hx_cur, 0, 0x7fffffff, kBufFlags);
+      i32x4 bf[KSMAX][NT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+      for (int ks = 0; ks < KSMAX; ++ks)
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int nt = 0; nt < NT; ++nt) bf[ks][nt] = i32x4{0, 0, 0, 0};
+      unsigned pend = pend0;
+      unsigned long long t0 = 0;
+      unsigned spins = 0;
+      for (;;) {
+        asm volatile("" ::: "memory");  // other workgroups write this memory: load again on every trip
 #pragma unroll
-    for (int ks = 0; ks < KSMAX; ++ks)
-      if (ks < ks_count) {
+        for (int ks = 0; ks < KSMAX; ++ks)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+          for (int nt = 0; nt < NT; ++nt)
+            if (pend & (1u << (ks * NT + nt))) {
+              const unsigned off = (unsigned)(((4 * (wave + kWaves * ks) + kg) * p.Bp + 16 * nt + jl) * kFragBytes);
+              bf[ks][nt] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(cur_rs, off, 0, AUX));
+            }
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+        for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            if ((pend & (1u << (ks * NT + nt))) && SN::complete(bf[ks][nt])) pend &= ~(1u << (ks * NT + nt));
+        if (!__any(pend != 0)) break;
+        if ((spins++ & 15u) == 0) {
+          if (__hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+          const unsigned long long now = wall_clock64();
+          if (spins == 1) {
+            t0 = now;
+          } else if (now - t0 > p.timeout_ticks) {
+            __hip_atomic_store(p.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+        }
       }
 
-    f32x4(*redbuf)[TILES][64] = red[s & 1];
+      f32x4 acc[MT][NT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+      for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) redbuf[wave][mt * NT + nt][lane] = acc[mt][nt];
-    __syncthreads();  // the only workgroup barrier of a step; `red` alternates between two copies
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KSMAX; ++ks)
+        if (ks < ks_count) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+        }
 
-    __amdgpu_buffer_rsrc_t nxt_rs = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(hx_g + (size_t)((s + 1) & (kHxRing - 1)) * hx_buf_bytes), 0, 0x7fffffff, kBufFlags);
-    __amdgpu_buffer_rsrc_t arm_rs = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(hx_g + (size_t)((s + 3) & (kHxRing - 1)) * hx_buf_bytes), 0, 0x7fffffff, kBufFlags);
-    float a_out[EPT][4], y_out[EPT];
-    unsigned h_bits[EPT];
+      f32x4(*redbuf)[TILES][64] = red[s & 1];
 #pragma unroll
-    for (int j = 0; j < EPT; ++j) {
-      const int e = wave + kWaves * j;
-      h_bits[j] = 0;
-      if (e < TILES) {
-        f32x4 gsum = redbuf[0][e][lane];
+      for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) gsum += redbuf[w][e][lane];
-        const float m = msk[j];
-        const float a0 = Act<AT>::tanh(gsum[0] + xg[j][0]);
-        const float a1 = Act<AT>::sigmoid(gsum[1] + xg[j][1]);
-        const float a2 = Act<AT>::sigmoid(gsum[2] + xg[j][2]);
-        const float a3 = Act<AT>::sigmoid(gsum[3] + xg[j][3]);
-        const float pc = c_state[j];
-        const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
-        const float y = E::round(Act<AT>::tanh(c) * a3 * m);
-        const float hn = E::round(y + h_prev[j] * (1.f - m));
-        c_state[j] = c;
-        h_prev[j] = hn;
-        y_out[j] = y;
-        a_out[j][0] = a0;
-        a_out[j][1] = a1;
-        a_out[j][2] = a2;
-        a_out[j][3] = a3;
-        h_bits[j] = SN::bits(hn);
+        for (int nt = 0; nt < NT; ++nt) redbuf[wave][mt * NT + nt][lane] = acc[mt][nt];
+      __syncthreads();  // the only workgroup barrier of a step; `red` alternates between two copies
+
+      __amdgpu_buffer_rsrc_t nxt_rs = __builtin_amdgcn_make_buffer_rsrc(
+          (void*)(hx_g + (size_t)((s + 1) & (kHxRing - 1)) * hx_buf_bytes), 0, 0x7fffffff, kBufFlags);
+      __amdgpu_buffer_rsrc_t arm_rs = __builtin_amdgcn_make_buffer_rsrc(
+          (void*)(hx_g + (size_t)((s + 3) & (kHxRing - 1)) * hx_buf_bytes), 0, 0x7fffffff, kBufFlags);
+      float a_out[EPT][4], y_out[EPT];
+      unsigned h_bits[EPT];
+#pragma unroll
+      for (int j = 0; j < EPT; ++j) {
+        const int e = wave + kWaves * j;
+        h_bits[j] = 0;
+        if (e < TILES) {
+          f32x4 gsum = redbuf[0][e][lane];
+#pragma unroll
+          for (int w = 1; w < kWaves; ++w) gsum += redbuf[w][e][lane];
+          const float m = msk[j];
+          const float a0 = Act<AT>::tanh(gsum[0] + xg[j][0]);
+          const float a1 = Act<AT>::sigmoid(gsum[1] + xg[j][1]);
+          const float a2 = Act<AT>::sigmoid(gsum[2] + xg[j][2]);
+          const float a3 = Act<AT>::sigmoid(gsum[3] + xg[j][3]);
+          const float pc = c_state[j];
+          const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
+          const float y = E::round(Act<AT>::tanh(c) * a3 * m);
+          const float hn = E::round(y + h_prev[j] * (1.f - m));
+          c_state[j] = c;
+          h_prev[j] = hn;
+          y_out[j] = y;
+          a_out[j][0] = a0;
+          a_out[j][1] = a1;
+          a_out[j][2] = a2;
+          a_out[j][3] = a3;
+          h_bits[j] = SN::bits(hn);
+        }
       }
-    }
-    // The re-arm stores of the previous step (and everything older) are acknowledged before the
-    // new hidden values go out.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      // The re-arm stores of the previous step (and everything older) are acknowledged before the
+      // new hidden values go out.
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-    for (int j = 0; j < EPT; ++j)
-      if (e_valid[j]) SN::store(nxt_rs, e_hoff[j], h_bits[j]);
+      for (int j = 0; j < EPT; ++j)
+        if (e_valid[j]) SN::template store<AUX>(nxt_rs, e_hoff[j], h_bits[j]);
 
 #pragma unroll
-    for (int j = 0; j < EPT; ++j) {
-      if (e_valid[j]) {
-        const long long bc = (long long)(b_base + e_b[j]) * n + e_cell[j];
-        const size_t xo = ((size_t)t * p.B + (b_base + e_b[j])) * 4 * n + e_cell[j];
+      for (int j = 0; j < EPT; ++j) {
+        if (e_valid[j]) {
+          const long long bc = (long long)(b_base + e_b[j]) * n + e_cell[j];
+          const size_t xo = ((size_t)t * p.B + (b_base + e_b[j])) * 4 * n + e_cell[j];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) E::store(p.H, xo + (size_t)q * n, a_out[j][q]);
-        p.C[t * bn + bc] = c_state[j];
-        E::store(p.Y, t * bn + bc, y_out[j]);
+          for (int q = 0; q < 4; ++q) E::store(p.H, xo + (size_t)q * n, a_out[j][q]);
+          p.C[t * bn + bc] = c_state[j];
+          E::store(p.Y, t * bn + bc, y_out[j]);
+        }
       }
-    }
-    // Re-arm this thread's elements of the buffer everybody read one step ago.
+      // Re-arm this thread's elements of the buffer everybody read one step ago.
 #pragma unroll
-    for (int j = 0; j < EPT; ++j)
-      if (e_valid[j]) SN::store(arm_rs, e_hoff[j], SN::kSentinel);
-  }
+      for (int j = 0; j < EPT; ++j)
+        if (e_valid[j]) SN::template store<AUX>(arm_rs, e_hoff[j], SN::kSentinel);
+    }
+  };
+  if (same_xcd)
+    run(IntTag<kAuxGroup>{});
+  else
+    run(IntTag<kAuxDevice>{});
 
 #pragma unroll
   for (int j = 0; j < EPT; ++j)

@@ -46,6 +46,8 @@ struct Lstm2Params {
   int hx_bufs;        // buffers in the hx ring: 2 with the flag barrier, 4 with self-validating data
   int hx_sentinel;    // 1: buffers 1.. start filled with the "not yet written" bit pattern (all ones)
   int xcds;           // XCDs assumed for the blockIdx -> (group, rank) mapping
+  int map_compact;    // register kernel: whole groups per XCD (see map_block_regw)
+  int allow_l2_exchange;  // register kernel: groups found on one XCD may exchange through its L2
   int sync_policy;    // SyncBits
   unsigned long long timeout_ticks;  // bound of one flag wait, in 100 MHz wall-clock ticks
 };

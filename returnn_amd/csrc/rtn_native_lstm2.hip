@@ -95,6 +95,8 @@ struct Plan {
   PlanKind kind = kPlanGeneric;
   int mode = RTN_MODE_STEPWISE;  // resolved: PERSISTENT, GRAPH or STEPWISE
   bool regw = false;             // persistent kernel with W in registers and self-validating exchange
+  bool compact = false;          // its groups are laid out one XCD each (see map_block_regw)
+  int grid = 0;                  // workgroups launched by the persistent kernel
   int KSMAX = 0;                 // its macro steps per wavefront (template bound)
   int MT = 1, NT = 1;
   int groups = 1, wgs_per_group = 1, Bg = 1, Bp = 16;
@@ -148,12 +150,13 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
       for (int use_regw = 1; use_regw >= 0; --use_regw) {
         if (use_regw && (env_kernel == 1 || KSMAX == 0)) continue;
         if (!use_regw && (env_kernel == 2 || persistent_ok)) continue;
-        for (int MT : {1, 2, 4}) {
+        for (int MT : {1, 2, 4, 8}) {
           if (env_mt && MT != env_mt) continue;
+          if (MT == 8 && !use_regw) continue;
           if ((n / 4) % MT) continue;
           const int G = n / (4 * MT);
           if (G > di.cus) continue;
-          if (use_regw && MT * KSMAX > 32) continue;
+          if (use_regw && MT * KSMAX > (KSMAX == 8 ? 64 : 32)) continue;
           const int max_groups = di.cus / G;
           for (int groups = 1; groups <= std::min(max_groups, B); ++groups) {
             if (env_groups && groups != std::min<long>(env_groups, std::min(max_groups, B))) continue;
@@ -164,12 +167,18 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
             if (use_regw && NT * KSMAX > 32) continue;
             const size_t lds = use_regw ? (size_t)2 * kWaves * MT * NT * kTileBytes : mfma_lds_bytes(n, dtype, MT, NT);
             if (lds > (use_regw ? (size_t)64 * 1024 : di.lds_per_wg)) continue;
+            // Whole groups per XCD when they fit: the exchange then stays inside one L2.
+            const int cus_per_xcd = di.cus / di.xcds;
+            const bool compact = use_regw && di.xcds > 1 && !env_long("RTN_LSTM2_NO_COMPACT", 0) &&
+                                 (long long)G * ((groups + di.xcds - 1) / di.xcds) <= cus_per_xcd;
             const double mfma_us = (double)MT * NT * ks * (dtype == RTN_DTYPE_BF16 ? 16 : 128) / 2400.0;
-            const double exch_us = 1.0 + 0.004 * G + 0.01 * Bg;
+            const double exch_us = compact ? 1.0 + 0.01 * Bg : 2.0 + 0.004 * G + 0.01 * Bg;
             const double est = mfma_us + exch_us;
             if (est < best) {
               best = est;
               pl.regw = use_regw != 0;
+              pl.compact = compact;
+              pl.grid = compact ? di.xcds * ((groups + di.xcds - 1) / di.xcds) * G : groups * G;
               pl.KSMAX = use_regw ? KSMAX : 0;
               pl.MT = MT;
               pl.NT = NT;
@@ -196,6 +205,7 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
       // Per-step launches have no co-residency limit: 4 cells per workgroup, groups of <= 64 rows.
       int MT = 1;
       pl.regw = false;
+      pl.compact = false;
       pl.KSMAX = 0;
       if (mfma_lds_bytes(n, dtype, 1, 4) > di.lds_per_wg) {
         pl.kind = kPlanGeneric;  // a W slice of 16 columns does not fit LDS (n far beyond the target sizes)
@@ -279,6 +289,7 @@ RegwKernel regw_kernel_for(int MT, int NT, int KSMAX) {
   RTN_CASE(1, 1, 8) RTN_CASE(1, 2, 8) RTN_CASE(1, 4, 8)
   RTN_CASE(2, 1, 8) RTN_CASE(2, 2, 8) RTN_CASE(2, 4, 8)
   RTN_CASE(4, 1, 8) RTN_CASE(4, 2, 8) RTN_CASE(4, 4, 8)
+  RTN_CASE(8, 1, 8)
   RTN_CASE(1, 1, 16) RTN_CASE(1, 2, 16)
   RTN_CASE(2, 1, 16) RTN_CASE(2, 2, 16)
 #undef RTN_CASE
@@ -434,10 +445,11 @@ const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int3
   } else if (!make_plan(T, B, n, dtype, mode, false, &pl, &why)) {
     g_plan_text = "unsupported: " + why;
   } else {
-    snprintf(buf, sizeof(buf), "mode=%s kernel=%s mt=%d nt=%d groups=%d wgs_per_group=%d wgs=%d rows_per_group=%d lds=%zu workspace=%zu",
+    snprintf(buf, sizeof(buf), "mode=%s kernel=%s mt=%d nt=%d groups=%d wgs_per_group=%d wgs=%d rows_per_group=%d group_per_xcd=%d lds=%zu workspace=%zu",
              mode_name(pl.mode),
              pl.kind == kPlanMfma ? (pl.regw ? "mfma_regw" : "mfma_lds") : (pl.kind == kPlanGeneric ? "generic" : "empty"), pl.MT,
-             pl.NT, pl.groups, pl.wgs_per_group, pl.groups * pl.wgs_per_group, pl.Bg, pl.lds_bytes, pl.total);
+             pl.NT, pl.groups, pl.wgs_per_group, (pl.mode == RTN_MODE_PERSISTENT && pl.regw) ? pl.grid : pl.groups * pl.wgs_per_group,
+             pl.Bg, pl.compact ? 1 : 0, pl.lds_bytes, pl.total);
     g_plan_text = buf;
   }
   return g_plan_text.c_str();
@@ -506,6 +518,8 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
   p.groups = pl.groups; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
   p.hx_bufs = kHxRing;
   p.hx_sentinel = pl.regw ? 1 : 0;
+  p.map_compact = pl.compact ? 1 : 0;
+  p.allow_l2_exchange = env_long("RTN_LSTM2_L2X", 1) ? 1 : 0;
   p.xcds = device_info().xcds;
   p.sync_policy = (int)env_long("RTN_LSTM2_SYNC", kStoreCoherent | kLoadCoherent);
   if (!((p.sync_policy & (kStoreCoherent | kReleaseFence)) && (p.sync_policy & (kLoadCoherent | kAcquireFence))))
@@ -533,7 +547,7 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
         if (rc != RTN_OK) return rc;
       }
       // All workgroups have to be on the device together.
-      const int wgs = pl.groups * pl.wgs_per_group;
+      const int wgs = pl.regw ? pl.grid : pl.groups * pl.wgs_per_group;
       int per_cu = 0;
       RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, pk, kWgThreads, pl.lds_bytes));
       if ((long long)per_cu * device_info().cus < wgs) {
@@ -546,6 +560,7 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
         p.Wp = ws + pl.off_wp;
         p.groups = pl.groups; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
         p.hx_sentinel = 0;
+        p.map_compact = 0;
         pk = nullptr;
       }
     }
@@ -563,7 +578,7 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
       hipLaunchKernelGGL(k_prepare_mfma<float>, pgrid, pblock, 0, stream, p, pl.n_flags);
     RTN_HIP(hipGetLastError());
     if (pk) {
-      const int wgs = pl.groups * pl.wgs_per_group;
+      const int wgs = pl.regw ? pl.grid : pl.groups * pl.wgs_per_group;
       int s_begin = 0, s_end = p.nsteps;
       void* args_lds[] = {(void*)&p, (void*)&s_begin, (void*)&s_end};
       void* args_regw[] = {(void*)&p};

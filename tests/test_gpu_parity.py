@@ -125,6 +125,23 @@ def test_decompositions(mt, groups, kernel):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("B,n", [(40, 512), (4, 1024), (9, 128)])
+def test_exchange_scopes(dtype, B, n):
+    """Register kernel: the hidden-state exchange through one XCD's L2 (groups placed whole on an XCD), the same
+    placement forced to device scope, and groups spread over XCDs all give the per-step result bit for bit."""
+    announce("exchange scopes", dtype, B, n)
+    p = random_problem(81, 64, B, n)
+    for step in (1, -1):
+        ref = run_op(*p, 0, step, dtype=dtype, mode="stepwise")
+        for settings in (dict(RTN_LSTM2_L2X=1), dict(RTN_LSTM2_L2X=0), dict(RTN_LSTM2_NO_COMPACT=1)):
+            with env(RTN_LSTM2_KERNEL=2, **settings):
+                rc, status, got = run_raw(*p, 0, step, dtype=dtype, mode="persistent")
+            assert rc == 0 and status == 0, settings
+            for a, b in zip(got, ref[:4]):
+                assert numpy.array_equal(a, b), settings
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_register_kernel_long_ring(dtype):
     """The exchange ring of 4 buffers wraps many times; ragged lengths, both directions, NaN-free and equal to the
     per-step result bit for bit.  n=1024 (bf16: 8 macro steps per wavefront; f32: 16)."""
