@@ -514,34 +514,40 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Persistent kernel with the recurrent weights in registers and a barrier-free exchange.
+// Persistent kernel with the recurrent weights in registers, a barrier-free exchange and a
+// decoupled input and output streams.
 //
 // Same decomposition and the same arithmetic per output element as k_lstm2_mfma (k dealt
-// round-robin to the 4 wavefronts, partial tiles summed in wave order), but:
-//  * every wavefront keeps the A-operand fragments of its k share in registers for all steps
-//    (MT * KSMAX fragments of 4 registers), so a step reads no weights from LDS or memory;
+// round-robin to 4 compute wavefronts, partial tiles summed in wave order), but:
+//  * every compute wavefront keeps the A-operand fragments of its k share in registers for all
+//    steps (MT * KSMAX fragments of 4 registers): a step reads no weights from LDS or memory;
 //  * there is no flag barrier.  The hidden state travels through a ring of 4 buffers whose
 //    elements validate themselves: a buffer starts as all-ones words ("not yet written", a NaN
 //    pattern the producers never emit), every element is written exactly once per use by the
-//    workgroup that owns the cell, and a consumer simply re-reads the fragments it needs
-//    until none of their elements is all-ones.  One store -> load hop per step instead of
-//    store, acknowledge, flag, poll, load.
+//    workgroup that owns the cell, and a consumer re-reads the fragments it needs until none
+//    of their elements is all-ones.  One store -> load hop per step instead of store,
+//    acknowledge, flag, poll, load.  The first read of step s+1 is issued right after the
+//    hidden values of step s have gone out.
 //    Step s reads buffer s%4, writes its outputs to (s+1)%4 and re-arms its own elements of
 //    (s+3)%4 = (s-1)%4, which every workgroup has finished reading (this workgroup has seen
-//    all outputs of step s-1).  The re-arm stores are acknowledged (vmcnt(0)) before this
-//    workgroup's next output stores, which precede anybody's first look at that buffer for step
-//    s+3, so a consumer can never mistake an old value for a new one.
-//  * the scope of the exchange follows the placement.  An MI355X has 8 XCDs with one L2 each;
-//    workgroups on the same XCD can meet in that L2 (loads that only skip the per-CU cache),
-//    workgroups on different XCDs have to go to device scope (memory side).  At start every
-//    workgroup publishes the id of the XCD it runs on (device scope) and reads the ids of its
-//    group: if they are all equal the group exchanges through its L2, else at device scope.
-//    The decision is a function of the complete id table, so all members take the same one; no
-//    assumption about how the hardware deals workgroups to XCDs is needed for correctness
-//    (the blockIdx -> (group, rank) mapping only makes the good case likely).
+//    all outputs of step s-1).  A wavefront's re-arm stores are acknowledged (vmcnt(0) after its
+//    next successful read) before its next hidden-value stores, which precede anybody's first
+//    look at that buffer for step s+3, so a consumer can never mistake an old value for a new one.
+//  * the op's streams are decoupled from the recurrence: X[t] and the mask are fetched two steps
+//    ahead as 16-byte chunks spread over the workgroup, parked in registers and handed over
+//    through LDS; H[t], Y[t], C[t] are staged in LDS by the threads that compute them and written
+//    out one step later, again 16 bytes per thread.  So the waits of the recurrence never contain
+//    the HBM latency of a stream, and the streams are coalesced.  One workgroup barrier per step
+//    (after the partial tiles are in LDS) orders everything.
+//  * exchange scope: the memory side of the device (sc1 loads and stores), which is valid
+//    wherever the workgroups of a group run.  Every workgroup records the XCD it runs on and
+//    the group's table is read back at start (it doubles as the check that the whole group is
+//    resident); `exchange` may select an experimental same-XCD policy when the table is uniform.
 // Waits are bounded as in k_lstm2_mfma.
 // ---------------------------------------------------------------------------------------------
-constexpr int kAuxGroup = 1;  // cache policy: skip the per-CU cache, meet in this XCD's L2 (sc0)
+constexpr int kExDevice = 0;  // device-scope loads and stores: always valid
+constexpr int kExNt = 1;      // experimental, same-XCD groups only: plain stores, non-temporal loads
+constexpr int kExNtSc0 = 2;   // experimental, same-XCD groups only: plain stores, workgroup-scope non-temporal loads
 
 template <typename AT>
 struct Sentinel;
@@ -589,6 +595,24 @@ struct IntTag {
   static constexpr int value = V;
 };
 
+// LDS layout of k_lstm2_regw (bytes), shared with the host for the launch.
+struct RegwLds {
+  unsigned red, xl, ml, hs, ys, cs, total;
+};
+__host__ __device__ constexpr RegwLds regw_lds(int es, int MT, int NT) {
+  RegwLds l{};
+  const unsigned rows = 16u * NT, cells = 4u * MT;
+  unsigned off = 0;
+  l.red = off; off += 2u * kWaves * MT * NT * kTileBytes;
+  l.xl = off; off += 2u * (rows * 4u * cells * es + 16u);  // each copy is followed by a 16-byte slot nobody reads
+  l.hs = off; off += 2u * rows * 4u * cells * es;
+  l.ys = off; off += (2u * rows * cells * es + 15u) / 16u * 16u;
+  l.cs = off; off += 2u * rows * cells * 4u;
+  l.ml = off; off += 2u * rows * 4u;
+  l.total = off;
+  return l;
+}
+
 // blockIdx -> (group, rank) for the register kernel.  With map_compact the grid is
 // xcds * ceil(groups / xcds) * wgs_per_group workgroups; under round-robin dealing of workgroup
 // ids to XCDs, XCD x then holds the whole groups x, x + xcds, ...; surplus workgroups (when
@@ -604,18 +628,85 @@ __device__ __forceinline__ void map_block_regw(const Lstm2Params& p, int bid, in
   }
 }
 
+// 16-byte (or 8-byte) chunk moves of the stream wavefront.
+template <int CH>
+struct Chunk;
+template <>
+struct Chunk<16> {
+  typedef i32x4 T;
+  static __device__ __forceinline__ T load(__amdgpu_buffer_rsrc_t rs, unsigned off) {
+    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, 0));
+  }
+  static __device__ __forceinline__ void store(T v, __amdgpu_buffer_rsrc_t rs, unsigned off) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v), rs, off, 0, 0);
+  }
+};
+template <>
+struct Chunk<8> {
+  typedef unsigned long long T;
+  static __device__ __forceinline__ T load(__amdgpu_buffer_rsrc_t rs, unsigned off) {
+    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, 0));
+  }
+  static __device__ __forceinline__ void store(T v, __amdgpu_buffer_rsrc_t rs, unsigned off) {
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(__attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned, v), rs, off, 0, 0);
+  }
+};
+
+// Running maximum over the 16-bit (bf16) or 32-bit (float) lanes of the words of a fragment: a lane
+// of the result is all-ones iff some element seen so far was the "not yet written" pattern.
+template <typename AT>
+struct LaneMax;
+template <>
+struct LaneMax<float> {
+  static __device__ __forceinline__ unsigned fold(unsigned acc, unsigned x) { return max(acc, x); }
+  static __device__ __forceinline__ bool has_sentinel(unsigned acc) { return acc == 0xFFFFFFFFu; }
+};
+template <>
+struct LaneMax<__bf16> {
+  static __device__ __forceinline__ unsigned fold(unsigned acc, unsigned x) {
+    unsigned r;
+    asm("v_pk_max_u16 %0, %1, %2" : "=v"(r) : "v"(acc), "v"(x));
+    return r;
+  }
+  static __device__ __forceinline__ bool has_sentinel(unsigned acc) {
+    return (acc & 0xFFFFu) == 0xFFFFu || (acc >> 16) == 0xFFFFu;
+  }
+};
+
+// Optional instrumentation (-DRTN_LSTM2_TRACE): wave 0 of every workgroup accumulates shader-clock
+// cycles per phase of k_lstm2_regw's step and writes the 8 totals to trace[blockIdx * 8 ..] at the end.
+#ifdef RTN_LSTM2_TRACE
+#define RTN_TRACE_DECL unsigned long long tr_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long tr_last = clock64();
+#define RTN_TRACE_MARK(k) { const unsigned long long tr_now = clock64(); tr_acc[k] += tr_now - tr_last; tr_last = tr_now; }
+#define RTN_TRACE_ADD(k, v) { tr_acc[k] += (v); }
+#define RTN_TRACE_FLUSH(p) if ((p).trace && threadIdx.x == 0) { for (int k = 0; k < 8; ++k) (p).trace[(size_t)blockIdx.x * 8 + k] = tr_acc[k]; }
+#else
+#define RTN_TRACE_DECL
+#define RTN_TRACE_MARK(k)
+#define RTN_TRACE_ADD(k, v)
+#define RTN_TRACE_FLUSH(p)
+#endif
+
+constexpr unsigned kOobOffset = 0xFFFFFF00u;  // a buffer offset beyond any frame: loads give 0, stores are dropped
+
 template <typename AT, int MT, int NT, int KSMAX>
 __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) {
   using E = Elem<AT>;
   using SN = Sentinel<AT>;
+  using LM = LaneMax<AT>;
   constexpr int KE = E::KE;
   constexpr int KM = E::KM;
+  constexpr int ES = (int)sizeof(AT);
   constexpr int TILES = MT * NT;
   constexpr int EPT = (TILES + kWaves - 1) / kWaves;
-  static_assert(KSMAX * NT <= 32, "pending mask is 32 bits");
+  constexpr int ROWS = 16 * NT;   // rows of the MFMA tiles (>= valid rows of the group)
+  constexpr int CELLS = 4 * MT;   // cells owned by this workgroup
+  constexpr RegwLds L = regw_lds(ES, MT, NT);
 
-  __shared__ f32x4 red[2][kWaves][TILES][64];
-  int* s_same_xcd = (int*)&red[0][0][0][0];  // borrowed before the first step (static LDS is capped at 64 KB)
+  extern __shared__ __align__(16) unsigned char smem[];
+  typedef f32x4 RedBuf[kWaves][TILES][64];
+  RedBuf* red = (RedBuf*)(smem + L.red);  // [2]
+  int* s_same_xcd = (int*)(smem + L.ml);  // borrowed before the first step
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in a scalar register
@@ -627,10 +718,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
   const int b_base = g * p.Bg;
   const int rows = min(p.Bg, p.B - b_base);
   const long long bn = (long long)p.B * n;
-  const size_t hx_buf_bytes = (size_t)n * p.Bp * sizeof(AT);
-  unsigned char* hx_g = (unsigned char*)p.hx + (size_t)g * kHxRing * hx_buf_bytes;
-  const int kg = lane >> 4, jl = lane & 15;
-  const int ks_count = (S > wave) ? (S - wave + kWaves - 1) / kWaves : 0;  // macro steps of this wave
+  const int nsteps = p.nsteps;
 
   // Where does the group run?  Publish this workgroup's XCD id (+1) and read the group's table.
   {
@@ -666,102 +754,182 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
         __builtin_amdgcn_s_sleep(2);
       }
       const int same_all = __all(same) ? 1 : 0;
-      if (lane == 0) *s_same_xcd = (same_all && p.allow_l2_exchange) ? 1 : 0;
-    }
-  }
-
-  // A-operand fragments of this wave's k share: registers, for the whole sequence.
-  i32x4 wreg[MT][KSMAX];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int ks = 0; ks < KSMAX; ++ks) {
-      const int sm = wave + kWaves * ks;
-      wreg[mt][ks] = i32x4{0, 0, 0, 0};
-      if (ks < ks_count) wreg[mt][ks] = ((const i32x4*)p.Wp)[((size_t)(r * MT + mt) * S + sm) * 64 + lane];
-    }
-
-  // Fragments this lane has to fetch each step: bit ks*NT+nt.
-  unsigned pend0 = 0;
-#pragma unroll
-  for (int ks = 0; ks < KSMAX; ++ks)
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-      if (ks < ks_count && 16 * nt + jl < rows) pend0 |= 1u << (ks * NT + nt);
-
-  float c_state[EPT], h_prev[EPT];
-  int e_b[EPT], e_cell[EPT];
-  bool e_valid[EPT];
-  unsigned e_hoff[EPT];
-#pragma unroll
-  for (int j = 0; j < EPT; ++j) {
-    const int e = wave + kWaves * j;
-    const int mt = e / NT, nt = e % NT;
-    const int bl = 16 * nt + (lane & 15);
-    e_cell[j] = 4 * (r * MT + mt) + (lane >> 4);
-    e_b[j] = bl;
-    e_valid[j] = (e < TILES) && (bl < rows);
-    e_hoff[j] = (unsigned)((((e_cell[j] / KE) * p.Bp + bl) * KE + (e_cell[j] % KE)) * (int)sizeof(AT));
-    c_state[j] = 0.f;
-    h_prev[j] = 0.f;
-    if (e_valid[j]) {
-      const long long bc = (long long)(b_base + bl) * n + e_cell[j];
-      c_state[j] = p.c0[bc];
-      h_prev[j] = E::load(p.y0, bc);
+      if (lane == 0) *s_same_xcd = same_all;
     }
   }
   __syncthreads();
   const bool same_xcd = *s_same_xcd != 0;
-  __syncthreads();  // everybody has read it; `red` is free for the steps
+  __syncthreads();  // everybody has read it; LDS is free for the steps
 
-  // All time steps, with the cache policy AUX for the hidden-state exchange.
-  auto run = [&](auto aux_tag) {
-    constexpr int AUX = decltype(aux_tag)::value;
-    for (int s = 0; s < p.nsteps; ++s) {
-      const long long t = frame_of(p, s);
+  // ---- the op's streams: X[t], mask[t] in; H[t], Y[t], C[t] out, as 16-byte (8-byte) chunks spread
+  // over the 256 threads.  X is fetched two steps ahead into registers and copied to LDS before the
+  // barrier of its step; the outputs are staged in LDS by the threads that compute them and written
+  // out after the barrier of the following step.  Chunks of rows the group does not have carry an
+  // out-of-range buffer offset: their loads return 0 and their stores are dropped, without a branch.
+  AT* Xl = (AT*)(smem + L.xl);
+  float* Ml = (float*)(smem + L.ml);
+  AT* Hs = (AT*)(smem + L.hs);
+  AT* Ys = (AT*)(smem + L.ys);
+  float* Cs = (float*)(smem + L.cs);
+  constexpr int SEG = CELLS * ES;               // contiguous bytes of one (row, gate) in X and H
+  constexpr int kXlCopy = ROWS * 4 * SEG + 16;  // one LDS copy of X[t] plus the spare slot
+  constexpr int CH = SEG < 16 ? 8 : 16;         // bytes moved per thread and chunk
+  constexpr int CPS = SEG / CH;                 // chunks per (row, gate)
+  constexpr int XCH = (ROWS * 4 * CPS + kWgThreads - 1) / kWgThreads;  // chunks per thread, X and H
+  constexpr int CHY = SEG < 16 ? 8 : 16;        // one row of Y is SEG bytes too
+  constexpr int YCH = (ROWS * (SEG / CHY) + kWgThreads - 1) / kWgThreads;
+  constexpr int SEGC = CELLS * 4;               // one row of C (float)
+  constexpr int CCH = (ROWS * (SEGC / 16) + kWgThreads - 1) / kWgThreads;
+  typedef Chunk<CH> XC;
+  typedef Chunk<CHY> YC;
+  typedef Chunk<16> CC;
+  const int cell0 = CELLS * r;
+  unsigned xoff[XCH], yoff[YCH], coff[CCH];  // byte offsets inside one frame (kOobOffset: nothing to move)
+  unsigned xlds[XCH], ylds[YCH], clds[CCH];  // byte offsets inside one LDS copy
+#pragma unroll
+  for (int i = 0; i < XCH; ++i) {
+    const int c = tid + kWgThreads * i;
+    const int row = c / (4 * CPS), gate = (c / CPS) % 4, part = c % CPS;
+    xoff[i] = row < rows ? (unsigned)((((b_base + row) * 4 * n) + gate * n + cell0) * ES + part * CH) : kOobOffset;
+    xlds[i] = (unsigned)(min(c, ROWS * 4 * CPS) * CH);  // threads beyond the tile write to / read from the spare slot
+  }
+#pragma unroll
+  for (int i = 0; i < YCH; ++i) {
+    const int c = tid + kWgThreads * i;
+    const int row = c / (SEG / CHY), part = c % (SEG / CHY);
+    yoff[i] = row < rows ? (unsigned)(((b_base + row) * n + cell0) * ES + part * CHY) : kOobOffset;
+    ylds[i] = (unsigned)(min(c, ROWS * (SEG / CHY) - 1) * CHY);
+  }
+#pragma unroll
+  for (int i = 0; i < CCH; ++i) {
+    const int c = tid + kWgThreads * i;
+    const int row = c / (SEGC / 16), part = c % (SEGC / 16);
+    coff[i] = row < rows ? (unsigned)(((b_base + row) * n + cell0) * 4 + part * 16) : kOobOffset;
+    clds[i] = (unsigned)(min(c, ROWS * (SEGC / 16) - 1) * 16);
+  }
+  const unsigned moff = tid < rows ? (unsigned)((b_base + tid) * 4) : kOobOffset;
+  const unsigned frame_x = (unsigned)((size_t)p.B * 4 * n * ES), frame_y = (unsigned)(bn * ES),
+                 frame_c = (unsigned)(bn * 4), frame_m = (unsigned)(p.B * 4);
+  typename XC::T xv[2][XCH];
+  float mv[2] = {0.f, 0.f};
+  auto fetch = [&](int s, auto par_tag) {  // issue the loads of X[t_s] and mask[t_s] into register set PAR
+    constexpr int PAR = decltype(par_tag)::value;
+    const long long t = frame_of(p, s);
+    __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.X + (size_t)t * frame_x, 0, frame_x, kBufFlags);
+    __amdgpu_buffer_rsrc_t mr = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.mask + (size_t)t * frame_m, 0, frame_m, kBufFlags);
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) xv[PAR][i] = XC::load(xr, xoff[i]);
+    mv[PAR] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(mr, moff, 0, 0));
+  };
+  auto put = [&](auto par_tag) {  // register set PAR -> LDS copy PAR
+    constexpr int PAR = decltype(par_tag)::value;
+    unsigned char* xl = (unsigned char*)Xl + (size_t)PAR * kXlCopy;
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) *(typename XC::T*)(xl + xlds[i]) = xv[PAR][i];
+    if (tid < ROWS) Ml[PAR * ROWS + tid] = mv[PAR];
+  };
+  auto flush = [&](int s, auto par_tag) {  // staged outputs of step s (LDS copy PAR) -> H[t], Y[t], C[t]
+    constexpr int PAR = decltype(par_tag)::value;
+    const long long t = frame_of(p, s);
+    const unsigned char* hs = smem + L.hs + (size_t)PAR * ROWS * 4 * SEG;
+    const unsigned char* ys = smem + L.ys + (size_t)PAR * ROWS * SEG;
+    const unsigned char* cs = smem + L.cs + (size_t)PAR * ROWS * SEGC;
+    __amdgpu_buffer_rsrc_t hr = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.H + (size_t)t * frame_x, 0, frame_x, kBufFlags);
+    __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.Y + (size_t)t * frame_y, 0, frame_y, kBufFlags);
+    __amdgpu_buffer_rsrc_t cr = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.C + (size_t)t * frame_c, 0, frame_c, kBufFlags);
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) XC::store(*(const typename XC::T*)(hs + xlds[i]), hr, xoff[i]);
+#pragma unroll
+    for (int i = 0; i < YCH; ++i) YC::store(*(const typename YC::T*)(ys + ylds[i]), yr, yoff[i]);
+#pragma unroll
+    for (int i = 0; i < CCH; ++i) CC::store(*(const typename CC::T*)(cs + clds[i]), cr, coff[i]);
+  };
 
-      // Gate inputs and mask of this step: independent of the recurrence, issued before the wait.
-      float xg[EPT][4], msk[EPT];
-#pragma unroll
-      for (int j = 0; j < EPT; ++j) {
-        msk[j] = 0.f;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) xg[j][q] = 0.f;
-        if (e_valid[j]) {
-          const size_t xo = ((size_t)t * p.B + (b_base + e_b[j])) * 4 * n + e_cell[j];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) xg[j][q] = E::load(p.X, xo + (size_t)q * n);
-          msk[j] = p.mask[t * p.B + b_base + e_b[j]];
-        }
-      }
+  // ---- the recurrence
+  const unsigned hx_buf_bytes = (unsigned)((size_t)n * p.Bp * sizeof(AT));
+  unsigned char* hx_g = (unsigned char*)p.hx + (size_t)g * kHxRing * hx_buf_bytes;
+  __amdgpu_buffer_rsrc_t ring_rs = __builtin_amdgcn_make_buffer_rsrc((void*)hx_g, 0, kHxRing * hx_buf_bytes, kBufFlags);
+  const int kg = lane >> 4, jl = lane & 15;
+  const int ks_count = (S > wave) ? (S - wave + kWaves - 1) / kWaves : 0;  // macro steps of this wave
 
-      // Fetch this wave's share of h_{s-1}; repeat for the fragments that are not complete yet.
-      const unsigned char* hx_cur = hx_g + (size_t)(s & (kHxRing - 1)) * hx_buf_bytes;
-      __amdgpu_buffer_rsrc_t cur_rs = __builtin_amdgcn_make_buffer_rsrc((void*)hx_cur, 0, 0x7fffffff, kBufFlags);
-      i32x4 bf[KSMAX][NT];
+  // A-operand fragments of this wave's k share: registers, for the whole sequence.  Slots past the
+  // wave's share hold zeros and are paired with any complete fragment, so the step has no branches.
+  i32x4 wreg[MT][KSMAX];
+  unsigned foff[KSMAX][NT];  // where this lane's B-operand fragments are inside a ring buffer
+#pragma unroll
+  for (int ks = 0; ks < KSMAX; ++ks) {
+    const bool mine = ks < ks_count;
+    const int sm = mine ? wave + kWaves * ks : 0;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      wreg[mt][ks] = i32x4{0, 0, 0, 0};
+      if (mine) wreg[mt][ks] = ((const i32x4*)p.Wp)[((size_t)(r * MT + mt) * S + sm) * 64 + lane];
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int row = (16 * nt + jl < rows) ? 16 * nt + jl : 0;  // rows the group does not have: read row 0
+      foff[ks][nt] = (unsigned)(((4 * sm + kg) * p.Bp + row) * kFragBytes);
+    }
+  }
+
+  // The (sequence, cell) pairs whose state this thread keeps.
+  float c_state[EPT], h_prev[EPT];
+  bool e_valid[EPT];
+  unsigned e_hoff[EPT];            // byte offset of the pair's element in an exchange buffer
+  unsigned e_row[EPT], e_cl[EPT];  // row and cell inside the workgroup's tile
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int e = min(wave + kWaves * j, TILES - 1);
+    const int mt = e / NT, nt = e % NT;
+    const int bl = 16 * nt + (lane & 15);
+    const int cell = 4 * (r * MT + mt) + (lane >> 4);
+    e_row[j] = (unsigned)bl;
+    e_cl[j] = (unsigned)(4 * mt + (lane >> 4));
+    e_valid[j] = (wave + kWaves * j < TILES) && (bl < rows);
+    e_hoff[j] = (unsigned)((((cell / KE) * p.Bp + bl) * KE + (cell % KE)) * ES);
+    c_state[j] = 0.f;
+    h_prev[j] = 0.f;
+    if (e_valid[j]) {
+      const long long bc = (long long)(b_base + bl) * n + cell;
+      c_state[j] = p.c0[bc];
+      h_prev[j] = E::load(p.y0, bc);
+    }
+  }
+
+  auto run = [&](auto ex_tag) {
+    constexpr int EX = decltype(ex_tag)::value;
+    constexpr int AUXS = (EX == kExDevice) ? kAuxDevice : 0;                        // stores
+    constexpr int AUXL = (EX == kExDevice) ? kAuxDevice : (EX == kExNt ? 2 : 3);    // loads
+    i32x4 bf[KSMAX][NT];
+    // Issue the loads of this wave's fragments of ring buffer s%4.
+    auto issue = [&](int s) {
+      const unsigned soff = (unsigned)(s & (kHxRing - 1)) * hx_buf_bytes;
+      asm volatile("" ::: "memory");  // other workgroups write this memory: really load again
 #pragma unroll
       for (int ks = 0; ks < KSMAX; ++ks)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) bf[ks][nt] = i32x4{0, 0, 0, 0};
-      unsigned pend = pend0;
+        for (int nt = 0; nt < NT; ++nt)
+          bf[ks][nt] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(ring_rs, foff[ks][nt], soff, AUXL));
+    };
+    RTN_TRACE_DECL
+    int delay = p.poll_delay;  // in units of s_sleep(1), about 64 clocks; adapts, see below
+    // One time step; PAR = s & 1 selects the register set and the LDS copies.
+    auto step = [&](int s, auto par_tag) {
+      constexpr int PAR = decltype(par_tag)::value;
+      RTN_TRACE_MARK(5)  // loop overhead between steps
+
+      // Complete this wave's share of h_{s-1}: if anything that came back is not written yet, read again.
       unsigned long long t0 = 0;
       unsigned spins = 0;
       for (;;) {
-        asm volatile("" ::: "memory");  // other workgroups write this memory: load again on every trip
+        unsigned m = 0;
 #pragma unroll
         for (int ks = 0; ks < KSMAX; ++ks)
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt)
-            if (pend & (1u << (ks * NT + nt))) {
-              const unsigned off = (unsigned)(((4 * (wave + kWaves * ks) + kg) * p.Bp + 16 * nt + jl) * kFragBytes);
-              bf[ks][nt] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(cur_rs, off, 0, AUX));
-            }
 #pragma unroll
-        for (int ks = 0; ks < KSMAX; ++ks)
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
-            if ((pend & (1u << (ks * NT + nt))) && SN::complete(bf[ks][nt])) pend &= ~(1u << (ks * NT + nt));
-        if (!__any(pend != 0)) break;
+            for (int w = 0; w < 4; ++w) m = LM::fold(m, (unsigned)bf[ks][nt][w]);
+        if (!__any(LM::has_sentinel(m))) break;
         if ((spins++ & 15u) == 0) {
           if (__hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
           const unsigned long long now = wall_clock64();
@@ -772,7 +940,22 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
             break;
           }
         }
+        issue(s);
       }
+      // Everything this wave stored before (re-arm stores included) is acknowledged, and X[t_s],
+      // fetched two steps ago, is in its registers.
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      // The first read is held back by `delay` so that it usually comes back complete: a read that
+      // comes back incomplete costs a whole extra round trip.  Lengthen the delay when that happened,
+      // shorten it slowly while it does not.
+      if (spins)
+        delay = min(delay + 2, 64);
+      else if ((s & 7) == 7 && delay > 0)
+        --delay;
+      RTN_TRACE_MARK(0)  // wait for h_{s-1}
+      RTN_TRACE_ADD(6, spins)
+      put(par_tag);
+      if (s + 2 < nsteps) fetch(s + 2, par_tag);
 
       f32x4 acc[MT][NT];
 #pragma unroll
@@ -781,85 +964,96 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
         for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < KSMAX; ++ks)
-        if (ks < ks_count) {
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
-        }
-
-      f32x4(*redbuf)[TILES][64] = red[s & 1];
+          for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+      RedBuf& redbuf = red[PAR];
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) redbuf[wave][mt * NT + nt][lane] = acc[mt][nt];
-      __syncthreads();  // the only workgroup barrier of a step; `red` alternates between two copies
+      RTN_TRACE_MARK(1)  // put + fetch + MFMA + partial tiles to LDS
+      __syncthreads();  // the one barrier of a step: partial tiles, X[t_s] and the outputs of step s-1 are in LDS
+      RTN_TRACE_MARK(2)  // barrier
 
-      __amdgpu_buffer_rsrc_t nxt_rs = __builtin_amdgcn_make_buffer_rsrc(
-          (void*)(hx_g + (size_t)((s + 1) & (kHxRing - 1)) * hx_buf_bytes), 0, 0x7fffffff, kBufFlags);
-      __amdgpu_buffer_rsrc_t arm_rs = __builtin_amdgcn_make_buffer_rsrc(
-          (void*)(hx_g + (size_t)((s + 3) & (kHxRing - 1)) * hx_buf_bytes), 0, 0x7fffffff, kBufFlags);
-      float a_out[EPT][4], y_out[EPT];
       unsigned h_bits[EPT];
 #pragma unroll
       for (int j = 0; j < EPT; ++j) {
-        const int e = wave + kWaves * j;
         h_bits[j] = 0;
-        if (e < TILES) {
+        if (TILES % kWaves == 0 || wave + kWaves * j < TILES) {  // wave-uniform
+          const int e = wave + kWaves * j;
           f32x4 gsum = redbuf[0][e][lane];
 #pragma unroll
           for (int w = 1; w < kWaves; ++w) gsum += redbuf[w][e][lane];
-          const float m = msk[j];
-          const float a0 = Act<AT>::tanh(gsum[0] + xg[j][0]);
-          const float a1 = Act<AT>::sigmoid(gsum[1] + xg[j][1]);
-          const float a2 = Act<AT>::sigmoid(gsum[2] + xg[j][2]);
-          const float a3 = Act<AT>::sigmoid(gsum[3] + xg[j][3]);
+          const unsigned xi = ((PAR * ROWS + e_row[j]) * 4) * CELLS + e_cl[j];  // in the staging copies
+          const AT* xin = (const AT*)((const unsigned char*)Xl + PAR * kXlCopy) + (e_row[j] * 4) * CELLS + e_cl[j];
+          const float m = Ml[PAR * ROWS + e_row[j]];
+          const float a0 = Act<AT>::tanh(gsum[0] + (float)xin[0]);
+          const float a1 = Act<AT>::sigmoid(gsum[1] + (float)xin[CELLS]);
+          const float a2 = Act<AT>::sigmoid(gsum[2] + (float)xin[2 * CELLS]);
+          const float a3 = Act<AT>::sigmoid(gsum[3] + (float)xin[3 * CELLS]);
           const float pc = c_state[j];
           const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
           const float y = E::round(Act<AT>::tanh(c) * a3 * m);
           const float hn = E::round(y + h_prev[j] * (1.f - m));
           c_state[j] = c;
           h_prev[j] = hn;
-          y_out[j] = y;
-          a_out[j][0] = a0;
-          a_out[j][1] = a1;
-          a_out[j][2] = a2;
-          a_out[j][3] = a3;
           h_bits[j] = SN::bits(hn);
+          // stage the op's outputs of this step
+          Hs[xi] = (AT)a0;
+          Hs[xi + CELLS] = (AT)a1;
+          Hs[xi + 2 * CELLS] = (AT)a2;
+          Hs[xi + 3 * CELLS] = (AT)a3;
+          const unsigned yi = (PAR * ROWS + e_row[j]) * CELLS + e_cl[j];
+          Ys[yi] = (AT)y;
+          Cs[yi] = c;
         }
       }
-      // The re-arm stores of the previous step (and everything older) are acknowledged before the
-      // new hidden values go out.
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      RTN_TRACE_MARK(3)  // gates, cell update, staging
+      // New hidden values out; re-arm the elements everybody read one step ago; first read of the next step.
+      // (Rows the group does not have own slots of the exchange buffers too, so no lane is switched off.)
+      {
+        const unsigned nxt = (unsigned)((s + 1) & (kHxRing - 1)) * hx_buf_bytes;
+        const unsigned arm = (unsigned)((s + 3) & (kHxRing - 1)) * hx_buf_bytes;
 #pragma unroll
-      for (int j = 0; j < EPT; ++j)
-        if (e_valid[j]) SN::template store<AUX>(nxt_rs, e_hoff[j], h_bits[j]);
-
+        for (int j = 0; j < EPT; ++j)
+          if (TILES % kWaves == 0 || wave + kWaves * j < TILES) SN::template store<AUXS>(ring_rs, e_hoff[j] + nxt, h_bits[j]);
 #pragma unroll
-      for (int j = 0; j < EPT; ++j) {
-        if (e_valid[j]) {
-          const long long bc = (long long)(b_base + e_b[j]) * n + e_cell[j];
-          const size_t xo = ((size_t)t * p.B + (b_base + e_b[j])) * 4 * n + e_cell[j];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) E::store(p.H, xo + (size_t)q * n, a_out[j][q]);
-          p.C[t * bn + bc] = c_state[j];
-          E::store(p.Y, t * bn + bc, y_out[j]);
-        }
+        for (int j = 0; j < EPT; ++j)
+          if (TILES % kWaves == 0 || wave + kWaves * j < TILES) SN::template store<AUXS>(ring_rs, e_hoff[j] + arm, SN::kSentinel);
       }
-      // Re-arm this thread's elements of the buffer everybody read one step ago.
-#pragma unroll
-      for (int j = 0; j < EPT; ++j)
-        if (e_valid[j]) SN::template store<AUX>(arm_rs, e_hoff[j], SN::kSentinel);
+      if (s + 1 < nsteps) {
+        for (int k = 0; k < delay; ++k) __builtin_amdgcn_s_sleep(1);
+        issue(s + 1);
+      }
+      if (s >= 1) flush(s - 1, IntTag<1 - PAR>{});
+      RTN_TRACE_MARK(4)  // exchange stores, first read of the next step, output stores
+    };
+    fetch(0, IntTag<0>{});
+    if (nsteps > 1) fetch(1, IntTag<1>{});
+    issue(0);
+    for (int s = 0; s < nsteps; s += 2) {
+      step(s, IntTag<0>{});
+      if (s + 1 < nsteps) step(s + 1, IntTag<1>{});
     }
+    RTN_TRACE_FLUSH(p)
   };
-  if (same_xcd)
-    run(IntTag<kAuxGroup>{});
+  if (same_xcd && p.exchange == kExNt)
+    run(IntTag<kExNt>{});
+  else if (same_xcd && p.exchange == kExNtSc0)
+    run(IntTag<kExNtSc0>{});
   else
-    run(IntTag<kAuxDevice>{});
+    run(IntTag<kExDevice>{});
+  __syncthreads();  // the last step's outputs are staged
+  if ((nsteps - 1) & 1)
+    flush(nsteps - 1, IntTag<1>{});
+  else
+    flush(nsteps - 1, IntTag<0>{});
 
 #pragma unroll
   for (int j = 0; j < EPT; ++j)
-    if (e_valid[j]) p.d[(long long)(b_base + e_b[j]) * n + e_cell[j]] = c_state[j];
+    if (e_valid[j]) p.d[(long long)(b_base + e_row[j]) * n + 4 * MT * r + e_cl[j]] = c_state[j];
 }
 
 }  // namespace rtn

@@ -102,7 +102,7 @@ struct Plan {
   int groups = 1, wgs_per_group = 1, Bg = 1, Bp = 16;
   size_t lds_bytes = 0;
   // workspace layout (byte offsets)
-  size_t off_status = 0, off_flags = 0, off_hx = 0, off_wp = 0, off_ycarry = 0, total = 0;
+  size_t off_status = 0, off_flags = 0, off_hx = 0, off_wp = 0, off_ycarry = 0, off_trace = 0, total = 0;
   int n_flags = 0;
 };
 
@@ -118,8 +118,12 @@ size_t mfma_lds_bytes(int n, int dtype, int MT, int NT) {
 // Chooses the decomposition.  `want_mode` is the caller's mode; `capturing` says the stream is
 // under capture (a cooperative launch cannot be recorded).  Returns false with a reason when
 // mode == PERSISTENT is impossible.
-bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing, Plan* out, std::string* why) {
+bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing, Plan* out, std::string* why,
+               int max_wgs_per_cu = 2) {
   Plan pl;
+  // Two workgroups per CU and whole groups per XCD only pay off with the (experimental) same-XCD exchange.
+  const bool xcd_local = env_long("RTN_LSTM2_EXCHANGE", 0) != 0;
+  max_wgs_per_cu = (int)std::max<long>(1, std::min<long>(max_wgs_per_cu, env_long("RTN_LSTM2_WGS_PER_CU", xcd_local ? 2 : 1)));
   const DeviceInfo di = device_info();
   const size_t es = esize(dtype);
   if (T == 0 || B == 0 || n == 0) {
@@ -144,7 +148,7 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
     const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
     const int S = n / KM;
     const int ks = (S + kWaves - 1) / kWaves;
-    const int KSMAX = ks <= 8 ? 8 : (ks <= 16 ? 16 : 0);
+    const int KSMAX = ks <= 2 ? 2 : (ks <= 4 ? 4 : (ks <= 8 ? 8 : (ks <= 16 ? 16 : 0)));
     if (want_mode == RTN_MODE_AUTO || want_mode == RTN_MODE_PERSISTENT) {
       double best = 1e30;
       for (int use_regw = 1; use_regw >= 0; --use_regw) {
@@ -155,25 +159,34 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
           if (MT == 8 && !use_regw) continue;
           if ((n / 4) % MT) continue;
           const int G = n / (4 * MT);
-          if (G > di.cus) continue;
-          if (use_regw && MT * KSMAX > (KSMAX == 8 ? 64 : 32)) continue;
-          const int max_groups = di.cus / G;
+          // Workgroups that can share a CU: the register kernel with few fragments per wavefront fits twice.
+          const int per_cu = (use_regw && MT * KSMAX <= 32 && KSMAX <= 8) ? max_wgs_per_cu : 1;
+          if (G > di.cus * per_cu) continue;
+          if (use_regw && (MT * KSMAX > (KSMAX == 16 ? 32 : 64) || (MT == 8 && KSMAX != 8))) continue;
+          const int max_groups = di.cus * per_cu / G;
           for (int groups = 1; groups <= std::min(max_groups, B); ++groups) {
             if (env_groups && groups != std::min<long>(env_groups, std::min(max_groups, B))) continue;
             const int Bg = (B + groups - 1) / groups;
             if ((B + Bg - 1) / Bg != groups) continue;  // same rows per group would need fewer groups
             if ((Bg + 15) / 16 > 4) continue;
             const int NT = round_nt((Bg + 15) / 16);
-            if (use_regw && NT * KSMAX > 32) continue;
-            const size_t lds = use_regw ? (size_t)2 * kWaves * MT * NT * kTileBytes : mfma_lds_bytes(n, dtype, MT, NT);
-            if (lds > (use_regw ? (size_t)64 * 1024 : di.lds_per_wg)) continue;
+            if (use_regw && (NT * KSMAX > 32 || MT * NT > 8)) continue;  // register budget of one wavefront
+            const size_t lds = use_regw ? (size_t)regw_lds((int)es, MT, NT).total : mfma_lds_bytes(n, dtype, MT, NT);
+            if (lds > di.lds_per_wg) continue;
+            int pc = per_cu;  // workgroups per CU that LDS allows as well
+            while (pc > 1 && lds * pc > di.lds_per_wg) --pc;
+            if ((long long)groups * G > (long long)di.cus * pc) continue;
             // Whole groups per XCD when they fit: the exchange then stays inside one L2.
             const int cus_per_xcd = di.cus / di.xcds;
-            const bool compact = use_regw && di.xcds > 1 && !env_long("RTN_LSTM2_NO_COMPACT", 0) &&
-                                 (long long)G * ((groups + di.xcds - 1) / di.xcds) <= cus_per_xcd;
+            const bool compact = use_regw && di.xcds > 1 && xcd_local && !env_long("RTN_LSTM2_NO_COMPACT", 0) &&
+                                 (long long)G * ((groups + di.xcds - 1) / di.xcds) <= (long long)cus_per_xcd * pc;
+            // Step time model fitted to MI355X measurements (microseconds): MFMA issue time of one
+            // wavefront, a second round of gate arithmetic when a thread owns two pairs, the number of
+            // workgroups that exchange with each other, the fragments a wavefront reads per step and
+            // the fragments it holds.
             const double mfma_us = (double)MT * NT * ks * (dtype == RTN_DTYPE_BF16 ? 16 : 128) / 2400.0;
-            const double exch_us = compact ? 1.0 + 0.01 * Bg : 2.0 + 0.004 * G + 0.01 * Bg;
-            const double est = mfma_us + exch_us;
+            const int ept = (MT * NT + kWaves - 1) / kWaves;
+            const double est = 2.0 * mfma_us + 0.4 * (ept - 1) + (compact ? 0.0 : 0.004 * G) + 0.03 * ks * NT + 0.01 * MT * ks;
             if (est < best) {
               best = est;
               pl.regw = use_regw != 0;
@@ -185,7 +198,7 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
               pl.groups = groups;
               pl.wgs_per_group = G;
               pl.Bg = Bg;
-              pl.lds_bytes = use_regw ? 0 : lds;
+              pl.lds_bytes = lds;
               persistent_ok = true;
             }
           }
@@ -249,6 +262,11 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
     pl.off_ycarry = off;
     off = align_up(off + (size_t)2 * B * n * es, 256);
   }
+  if (env_long("RTN_LSTM2_TRACE", 0)) {
+    // debugging aid (instrumented builds): 8 cycle totals per workgroup at the end of the workspace
+    pl.off_trace = off;
+    off = align_up(off + (size_t)1024 * 8 * sizeof(unsigned long long), 256);
+  }
   pl.total = off;
   *out = pl;
   return true;
@@ -286,9 +304,15 @@ template <typename AT>
 RegwKernel regw_kernel_for(int MT, int NT, int KSMAX) {
 #define RTN_CASE(mt, nt, ks) \
   if (MT == mt && NT == nt && KSMAX == ks) return &k_lstm2_regw<AT, mt, nt, ks>;
+  RTN_CASE(1, 1, 2) RTN_CASE(1, 2, 2) RTN_CASE(1, 4, 2)
+  RTN_CASE(2, 1, 2) RTN_CASE(2, 2, 2) RTN_CASE(2, 4, 2)
+  RTN_CASE(4, 1, 2) RTN_CASE(4, 2, 2)
+  RTN_CASE(1, 1, 4) RTN_CASE(1, 2, 4) RTN_CASE(1, 4, 4)
+  RTN_CASE(2, 1, 4) RTN_CASE(2, 2, 4) RTN_CASE(2, 4, 4)
+  RTN_CASE(4, 1, 4) RTN_CASE(4, 2, 4)
   RTN_CASE(1, 1, 8) RTN_CASE(1, 2, 8) RTN_CASE(1, 4, 8)
   RTN_CASE(2, 1, 8) RTN_CASE(2, 2, 8) RTN_CASE(2, 4, 8)
-  RTN_CASE(4, 1, 8) RTN_CASE(4, 2, 8) RTN_CASE(4, 4, 8)
+  RTN_CASE(4, 1, 8) RTN_CASE(4, 2, 8)
   RTN_CASE(8, 1, 8)
   RTN_CASE(1, 1, 16) RTN_CASE(1, 2, 16)
   RTN_CASE(2, 1, 16) RTN_CASE(2, 2, 16)
@@ -301,15 +325,15 @@ RegwKernel regw_kernel(int dtype, int MT, int NT, int KSMAX) {
 }
 
 // Kernels that use more than the default LDS limit need the limit raised once per device.
-int ensure_lds_limit(MfmaKernel k, size_t lds_bytes) {
+int ensure_lds_limit(const void* k, size_t lds_bytes) {
   static std::mutex mu;
-  static std::list<std::pair<std::pair<int, MfmaKernel>, size_t>> done;
+  static std::list<std::pair<std::pair<int, const void*>, size_t>> done;
   int dev = 0;
   RTN_HIP(hipGetDevice(&dev));
   std::lock_guard<std::mutex> lock(mu);
   for (auto& e : done)
     if (e.first.first == dev && e.first.second == k && e.second >= lds_bytes) return RTN_OK;
-  RTN_HIP(hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  RTN_HIP(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   done.push_back({{dev, k}, lds_bytes});
   return RTN_OK;
 }
@@ -431,8 +455,11 @@ size_t rtn_native_lstm2_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int
   Plan pl;
   std::string why;
   if (make_plan(T, B, n, dtype, mode, false, &pl, &why)) need = std::max(need, pl.total);
-  if (mode == RTN_MODE_AUTO || mode == RTN_MODE_PERSISTENT)
+  if (mode == RTN_MODE_AUTO || mode == RTN_MODE_PERSISTENT) {
+    // what the call may settle on when the device gives the kernel fewer workgroups per CU, or none at all
+    if (make_plan(T, B, n, dtype, mode, false, &pl, &why, 1)) need = std::max(need, pl.total);
     if (make_plan(T, B, n, dtype, RTN_MODE_STEPWISE, true, &pl, &why)) need = std::max(need, pl.total);
+  }
   return need;
 }
 
@@ -450,6 +477,7 @@ const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int3
              pl.kind == kPlanMfma ? (pl.regw ? "mfma_regw" : "mfma_lds") : (pl.kind == kPlanGeneric ? "generic" : "empty"), pl.MT,
              pl.NT, pl.groups, pl.wgs_per_group, (pl.mode == RTN_MODE_PERSISTENT && pl.regw) ? pl.grid : pl.groups * pl.wgs_per_group,
              pl.Bg, pl.compact ? 1 : 0, pl.lds_bytes, pl.total);
+    if (pl.off_trace) snprintf(buf + strlen(buf), sizeof(buf) - strlen(buf), " trace_offset=%zu", pl.off_trace);
     g_plan_text = buf;
   }
   return g_plan_text.c_str();
@@ -491,6 +519,26 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
   std::string why;
   if (!make_plan(T, B, n, dtype, mode, capturing, &pl, &why))
     return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: persistent mode unavailable for T=%lld B=%d n=%d: %s", (long long)T, B, n, why.c_str());
+  // A persistent plan needs all its workgroups on the device together: check against what the kernel
+  // really gets per CU, plan again for that if the plan was too optimistic, else fall back to per-step launches.
+  const void* pk = nullptr;  // the persistent kernel, if any
+  for (int attempt = 0; pl.kind == kPlanMfma && pl.mode == RTN_MODE_PERSISTENT; ++attempt) {
+    pk = pl.regw ? (const void*)regw_kernel(dtype, pl.MT, pl.NT, pl.KSMAX) : (const void*)mfma_kernel(dtype, pl.MT, pl.NT);
+    if (!pk) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d ks=%d", pl.MT, pl.NT, pl.KSMAX);
+    rc = ensure_lds_limit(pk, pl.lds_bytes);
+    if (rc != RTN_OK) return rc;
+    const int wgs = pl.regw ? pl.grid : pl.groups * pl.wgs_per_group;
+    int per_cu = 0;
+    RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, pk, kWgThreads, pl.lds_bytes));
+    if ((long long)per_cu * device_info().cus >= wgs) break;
+    pk = nullptr;
+    if (attempt == 0 && per_cu >= 1 && make_plan(T, B, n, dtype, mode, capturing, &pl, &why, per_cu)) continue;
+    if (mode == RTN_MODE_PERSISTENT)
+      return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: %d workgroups cannot be co-resident (%d per CU)", wgs, per_cu);
+    if (!make_plan(T, B, n, dtype, RTN_MODE_GRAPH, capturing, &pl, &why))
+      return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no per-step plan: %s", why.c_str());
+    break;
+  }
   if (!workspace || workspace_bytes < pl.total)
     return fail(RTN_ERR_WORKSPACE, "NativeLstm2: workspace of %zu bytes needed, got %zu", pl.total, workspace ? workspace_bytes : (size_t)0);
   if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2: workspace must be 16-byte aligned");
@@ -505,6 +553,7 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
   p.hx = ws + pl.off_hx;
   p.Wp = ws + pl.off_wp;
   p.ycarry = ws + pl.off_ycarry;
+  p.trace = pl.off_trace ? (unsigned long long*)(ws + pl.off_trace) : nullptr;
   p.T = T; p.B = B; p.n = n;
   // returnn/native_op.py:1253-1259
   if (step > 0) {
@@ -519,7 +568,11 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
   p.hx_bufs = kHxRing;
   p.hx_sentinel = pl.regw ? 1 : 0;
   p.map_compact = pl.compact ? 1 : 0;
-  p.allow_l2_exchange = env_long("RTN_LSTM2_L2X", 1) ? 1 : 0;
+  p.exchange = (int)env_long("RTN_LSTM2_EXCHANGE", 0);
+  if (p.exchange < 0 || p.exchange > 2) p.exchange = 0;
+  // Device-scope stores take about a microsecond to become visible: a first read issued at once would
+  // come back incomplete and cost a second round trip, so it is held back (tuned on MI355X).
+  p.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", p.exchange == 0 ? 20 : 8)));
   p.xcds = device_info().xcds;
   p.sync_policy = (int)env_long("RTN_LSTM2_SYNC", kStoreCoherent | kLoadCoherent);
   if (!((p.sync_policy & (kStoreCoherent | kReleaseFence)) && (p.sync_policy & (kLoadCoherent | kAcquireFence))))
@@ -538,36 +591,10 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
   }
 
   if (pl.kind == kPlanMfma) {
-    const void* pk = nullptr;  // the persistent kernel, if any
-    if (pl.mode == RTN_MODE_PERSISTENT) {
-      pk = pl.regw ? (const void*)regw_kernel(dtype, pl.MT, pl.NT, pl.KSMAX) : (const void*)mfma_kernel(dtype, pl.MT, pl.NT);
-      if (!pk) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d ks=%d", pl.MT, pl.NT, pl.KSMAX);
-      if (!pl.regw) {
-        rc = ensure_lds_limit((MfmaKernel)pk, pl.lds_bytes);
-        if (rc != RTN_OK) return rc;
-      }
-      // All workgroups have to be on the device together.
-      const int wgs = pl.regw ? pl.grid : pl.groups * pl.wgs_per_group;
-      int per_cu = 0;
-      RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, pk, kWgThreads, pl.lds_bytes));
-      if ((long long)per_cu * device_info().cus < wgs) {
-        if (mode == RTN_MODE_PERSISTENT)
-          return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: %d workgroups cannot be co-resident (%d per CU)", wgs, per_cu);
-        // AUTO: plan again for per-step launches (same workspace, it was sized for both).
-        if (!make_plan(T, B, n, dtype, RTN_MODE_GRAPH, capturing, &pl, &why) || workspace_bytes < pl.total)
-          return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no per-step plan fits the workspace");
-        p.hx = ws + pl.off_hx;
-        p.Wp = ws + pl.off_wp;
-        p.groups = pl.groups; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
-        p.hx_sentinel = 0;
-        p.map_compact = 0;
-        pk = nullptr;
-      }
-    }
     MfmaKernel k = mfma_kernel(dtype, pl.MT, pl.NT);
     if (!pk) {
       if (!k) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d", pl.MT, pl.NT);
-      rc = ensure_lds_limit(k, pl.lds_bytes);
+      rc = ensure_lds_limit((const void*)k, pl.lds_bytes);
       if (rc != RTN_OK) return rc;
     }
     const long long work = std::max<long long>((long long)n * n, bn);
@@ -582,8 +609,8 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
       int s_begin = 0, s_end = p.nsteps;
       void* args_lds[] = {(void*)&p, (void*)&s_begin, (void*)&s_end};
       void* args_regw[] = {(void*)&p};
-      RTN_HIP(hipLaunchCooperativeKernel(pk, dim3(wgs), dim3(kWgThreads), pl.regw ? args_regw : args_lds,
-                                         (unsigned)pl.lds_bytes, stream));
+      RTN_HIP(hipLaunchCooperativeKernel(pk, dim3(wgs), dim3(kWgThreads),
+                                         pl.regw ? args_regw : args_lds, (unsigned)pl.lds_bytes, stream));
       return RTN_OK;
     }
   } else {

@@ -57,7 +57,7 @@ def load() -> ctypes.CDLL:
     with _lock:
         if _lib is not None:
             return _lib
-        path = _build.LIB_PATH
+        path = os.environ.get("RTN_NATIVE_LSTM2_LIB") or _build.LIB_PATH  # override: an instrumented build
         if not os.path.exists(path):
             raise NativeLibraryMissing(
                 "%s not found. Build it with `python -m returnn_amd.build` (needs hipcc; "
