@@ -31,6 +31,13 @@ if _root not in sys.path:
 PEAK_MFMA = {"bf16": 2.5e15, "f32": 157.3e12}  # MI355X dense matrix peaks, FLOP/s
 PEAK_HBM = 8.0e12  # B/s
 
+# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by
+# what the same counter reads for a plain 1 GiB device copy); see profiles/k_lstm2_regw_cfg3_hbm_traffic.txt.
+# Keyed by (workload, plan as rtn_native_lstm2_describe_plan reports it up to the LDS size).
+MEASURED_TRAFFIC_BYTES = {
+    ("cfg3", "mode=persistent kernel=mfma_regw mt=2 nt=1 groups=2 wgs_per_group=128 wgs=256 rows_per_group=16"): 1268.4e6,
+}
+
 
 def algorithmic_bytes_per_unit(n: int, dtype: str) -> int:
     """HBM bytes per timestep x sequence: read X (4n), write H (4n), Y (n) in the activation type,
@@ -61,16 +68,19 @@ def cpu_baseline(name: str, target_seconds: float = 15.0):
     full_T = synthetic.make_config.__globals__["_SPECS"][name]["T"]
     T = int(max(probe_T, min(full_T, target_seconds / max(per_frame, 1e-9))))
     p = synthetic.make_config(name, T=T)
+    reps = int(max(1, min(50, round(target_seconds / max(per_frame * T, 1e-9)))))
     t0 = time.perf_counter()
-    lstm2_oracle.native_lstm2_fwd_blas(p.X, p.W, p.y0, p.c0, p.i)
+    for _ in range(reps):
+        lstm2_oracle.native_lstm2_fwd_blas(p.X, p.W, p.y0, p.c0, p.i)
     dt = time.perf_counter() - t0
     return {
-        "value": p.T * p.B / dt,
+        "value": reps * p.T * p.B / dt,
         "unit": "timesteps*seqs/s",
         "cores": blas_threads,
         "kind": "port",
-        "sample": "%s shape fp32, one direction, first T=%i of %i frames (B=%i, n=%i), %.1f s; GEMM on %i BLAS threads, "
-        "pointwise loop on 1 thread as the reference's CPU path" % (name, p.T, full_T, p.B, p.n, dt, blas_threads),
+        "sample": "%s shape in fp32, one direction, first T=%i of %i frames (B=%i, n=%i), %i passes, %.1f s; "
+        "per frame one SGEMM on %i BLAS threads, pointwise loop on 1 thread, as the reference's CPU path"
+        % (name, p.T, full_T, p.B, p.n, reps, dt, blas_threads),
     }
 
 
@@ -83,6 +93,9 @@ def main():
     ap.add_argument("--mode", default="auto", choices=["auto", "persistent", "graph", "stepwise"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--copy-calibration-mib", type=int, default=0,
+                    help="also run one plain device copy of this many MiB (a kernel of known traffic, to scale "
+                         "rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the recurrence is one sequential chain per batch; "
@@ -136,6 +149,13 @@ def main():
             o["ws"].data_ptr(), o["ws"].numel(), stream.cuda_stream,
         )  # fmt: skip
         lib.check(rc)
+
+    if args.copy_calibration_mib > 0:
+        src = torch.empty((args.copy_calibration_mib << 20,), dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads and writes copy_calibration_mib MiB each
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         for k in range(len(directions)):
@@ -199,8 +219,10 @@ def main():
             "peak": peak / 1e12,
             "unit": "TFLOP/s",
             "frac": achieved / peak,
-            "traffic": None,
-            "kernel": "k_lstm2_mfma (one launch = one op call of T*B = %i units, 8*n^2 flops each)" % (T * B),
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, plan.split(" group_per_xcd")[0])),
+            "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE); algorithmic: %i" % bytes_per_launch,
+            "kernel": "%s (one launch = one op call of T*B = %i units, 8*n^2 flops each)"
+            % ("k_lstm2_regw" if "mfma_regw" in plan else ("k_lstm2_mfma" if "mfma_lds" in plan else "k_step_generic"), T * B),
             "launch_ms": call_ms,
             "hbm_algorithmic_GBps": bytes_per_launch / (call_ms * 1e-3) / 1e9,
             "hbm_frac": bytes_per_launch / (call_ms * 1e-3) / PEAK_HBM,
