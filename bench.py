@@ -98,8 +98,9 @@ def main():
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on exactly one GPU (the recurrence is one sequential chain per batch; "
-              "see DESIGN.md for how it would shard); --gpus %i is not supported." % args.gpus, file=sys.stderr)
+        print("bench.py: this build runs on exactly one GPU (the recurrence is one sequential chain per batch row; "
+              "more GPUs would each take a share of the batch with no exchange); --gpus %i is not supported."
+              % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import torch
