@@ -163,7 +163,8 @@ def main():
             one_call(k)
     torch.cuda.synchronize()
     for k in range(len(directions)):
-        lib.check(cabi.rtn_native_lstm2_fwd_status(outs[k]["ws"].data_ptr(), stream.cuda_stream))
+        if os.environ.get("RTN_LSTM2_EXCHANGE") != "3":
+            lib.check(cabi.rtn_native_lstm2_fwd_status(outs[k]["ws"].data_ptr(), stream.cuda_stream))
 
     events = []
     torch.cuda.synchronize()
@@ -178,9 +179,11 @@ def main():
             events.append((e0, e1))
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    measuring_only = os.environ.get("RTN_LSTM2_EXCHANGE") == "3"  # no-exchange timing aid: results are invalid
     for k in range(len(directions)):
-        lib.check(cabi.rtn_native_lstm2_fwd_status(outs[k]["ws"].data_ptr(), stream.cuda_stream))
-    assert all(bool(torch.isfinite(o["d"]).all()) for o in outs)
+        if not measuring_only:
+            lib.check(cabi.rtn_native_lstm2_fwd_status(outs[k]["ws"].data_ptr(), stream.cuda_stream))
+    assert measuring_only or all(bool(torch.isfinite(o["d"]).all()) for o in outs)
 
     call_ms = sum(a.elapsed_time(b) for a, b in events) / len(events)
     units_per_step = len(directions) * T * B

@@ -548,6 +548,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
 constexpr int kExDevice = 0;  // device-scope loads and stores: always valid
 constexpr int kExNt = 1;      // experimental, same-XCD groups only: plain stores, non-temporal loads
 constexpr int kExNtSc0 = 2;   // experimental, same-XCD groups only: plain stores, workgroup-scope non-temporal loads
+constexpr int kExNoWait = 3;  // measurement aid: never wait for the other workgroups (results are WRONG; status is set to 2)
 
 template <typename AT>
 struct Sentinel;
@@ -898,8 +899,8 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
 
   auto run = [&](auto ex_tag) {
     constexpr int EX = decltype(ex_tag)::value;
-    constexpr int AUXS = (EX == kExDevice) ? kAuxDevice : 0;                        // stores
-    constexpr int AUXL = (EX == kExDevice) ? kAuxDevice : (EX == kExNt ? 2 : 3);    // loads
+    constexpr int AUXS = (EX == kExDevice || EX == kExNoWait) ? kAuxDevice : 0;                        // stores
+    constexpr int AUXL = (EX == kExDevice || EX == kExNoWait) ? kAuxDevice : (EX == kExNt ? 2 : 3);    // loads
     i32x4 bf[KSMAX][NT];
     // Issue the loads of this wave's fragments of ring buffer s%4.
     auto issue = [&](int s) {
@@ -929,7 +930,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
           for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int w = 0; w < 4; ++w) m = LM::fold(m, (unsigned)bf[ks][nt][w]);
-        if (!__any(LM::has_sentinel(m))) break;
+        if (EX == kExNoWait || !__any(LM::has_sentinel(m))) break;
         if ((spins++ & 15u) == 0) {
           if (__hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
           const unsigned long long now = wall_clock64();
@@ -950,7 +951,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
       // shorten it slowly while it does not.
       if (spins)
         delay = min(delay + 2, 64);
-      else if ((s & 7) == 7 && delay > 0)
+      else if ((s & 15) == 15 && delay > 0)
         --delay;
       RTN_TRACE_MARK(0)  // wait for h_{s-1}
       RTN_TRACE_ADD(6, spins)
@@ -1043,7 +1044,10 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
     run(IntTag<kExNt>{});
   else if (same_xcd && p.exchange == kExNtSc0)
     run(IntTag<kExNtSc0>{});
-  else
+  else if (p.exchange == kExNoWait) {
+    if (tid == 0) __hip_atomic_store(p.status, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    run(IntTag<kExNoWait>{});
+  } else
     run(IntTag<kExDevice>{});
   __syncthreads();  // the last step's outputs are staged
   if ((nsteps - 1) & 1)

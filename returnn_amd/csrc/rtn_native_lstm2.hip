@@ -122,7 +122,8 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
                int max_wgs_per_cu = 2) {
   Plan pl;
   // Two workgroups per CU and whole groups per XCD only pay off with the (experimental) same-XCD exchange.
-  const bool xcd_local = env_long("RTN_LSTM2_EXCHANGE", 0) != 0;
+  const long env_exchange = env_long("RTN_LSTM2_EXCHANGE", 0);
+  const bool xcd_local = env_exchange == 1 || env_exchange == 2;
   max_wgs_per_cu = (int)std::max<long>(1, std::min<long>(max_wgs_per_cu, env_long("RTN_LSTM2_WGS_PER_CU", xcd_local ? 2 : 1)));
   const DeviceInfo di = device_info();
   const size_t es = esize(dtype);
@@ -569,7 +570,7 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
   p.hx_sentinel = pl.regw ? 1 : 0;
   p.map_compact = pl.compact ? 1 : 0;
   p.exchange = (int)env_long("RTN_LSTM2_EXCHANGE", 0);
-  if (p.exchange < 0 || p.exchange > 2) p.exchange = 0;
+  if (p.exchange < 0 || p.exchange > 3) p.exchange = 0;  // 3: measurement aid, results invalid (status 2)
   // Device-scope stores take about a microsecond to become visible: a first read issued at once would
   // come back incomplete and cost a second round trip, so it is held back (tuned on MI355X).
   p.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", p.exchange == 0 ? 20 : 8)));
