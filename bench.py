@@ -84,12 +84,91 @@ def cpu_baseline(name: str, target_seconds: float = 15.0):
     }
 
 
+def bench_encoder(args, dev):
+    """
+    Config 4: forward of the 6-layer bidirectional encoder (per layer one projection GEMM and one op call per
+    direction, outputs concatenated).  One step = one forward of the stack; value counts the op-level units,
+    12 * T * B per step.  The projection GEMMs (hipBLASLt) are timed again on their own to split the step time.
+    """
+    import torch
+
+    from returnn_amd import lstm as rlstm
+    from returnn_amd import synthetic
+
+    prob = synthetic.make_encoder_config("cfg4")
+    T, B, n, L = prob.T, prob.B, prob.n, prob.num_layers
+    bf = torch.bfloat16
+    enc = rlstm.BlstmEncoder.from_params(prob.layers, device=dev, dtype=bf)
+    x = torch.from_numpy(prob.features).to(dev).to(bf)
+    lens = torch.from_numpy(prob.lens).to(dev)
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            y = enc(x, seq_lens=lens)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            y = enc(x, seq_lens=lens)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        assert bool(torch.isfinite(y.float()).all())
+        # the projections alone, same shapes and weights
+        ws = [(m._weights(bf), d_in) for m, d_in in
+              [(m, enc.in_dim if li == 0 else 2 * n) for li in range(L) for m in (enc.fwd[li], enc.bwd[li])]]
+        srcs = {d: torch.randn((T * B, d), device=dev).to(bf) for d in {enc.in_dim, 2 * n}}
+        for w, d_in in ws:
+            torch.addmm(w.bias, srcs[d_in], w.ff)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            for w, d_in in ws:
+                torch.addmm(w.bias, srcs[d_in], w.ff)
+        torch.cuda.synchronize()
+        proj = time.perf_counter() - t1
+    step_ms = elapsed * 1e3 / args.steps
+    proj_ms = proj * 1e3 / args.steps
+    rec_flops = 2 * L * 8.0 * T * B * n * n
+    proj_flops = 2 * sum(2.0 * T * B * (enc.in_dim if li == 0 else 2 * n) * 4 * n for li in range(L))
+    units = 2 * L * T * B
+    return {
+        "metric": "LSTM fwd timesteps*seqs/sec (T*B/s) at n=%i" % n,
+        "value": units * args.steps / elapsed,
+        "unit": "timesteps*seqs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": step_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "cfg4: %i-layer bidirectional LSTM encoder forward, T=%i B=%i in=%i n=%i bf16, ragged=True; "
+            "per layer and direction one projection GEMM and one NativeLstm2 call" % (L, T, B, enc.in_dim, n),
+            "calls_per_step": 2 * L,
+            "units_per_step": units,
+            "projection_ms_per_step": proj_ms,
+            "recurrent_and_glue_ms_per_step": step_ms - proj_ms,
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": (rec_flops + proj_flops) / (step_ms * 1e-3) / 1e12,
+            "peak": PEAK_MFMA["bf16"] / 1e12,
+            "unit": "TFLOP/s",
+            "frac": (rec_flops + proj_flops) / (step_ms * 1e-3) / PEAK_MFMA["bf16"],
+            "traffic": None,
+            "kernel": "whole stack: recurrent %.3g TFLOP + projections %.3g TFLOP per step over the step time"
+            % (rec_flops / 1e12, proj_flops / 1e12),
+        },
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg5"])
+    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
     ap.add_argument("--mode", default="auto", choices=["auto", "persistent", "graph", "stepwise"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
@@ -114,6 +193,10 @@ def main():
     cabi = lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.workload == "cfg4":
+        print(json.dumps(bench_encoder(args, dev)))
+        return
 
     p = synthetic.make_config(args.workload)
     T, B, n = p.T, p.B, p.n

@@ -1,0 +1,282 @@
+"""
+LSTM layer forward on top of the NativeLstm2 op: the raw-tensor side of the reference's frontend LSTM.
+
+The reference's ``rf.LSTM`` (returnn/frontend/rec.py:16-77) holds ``ff_weight [4*out,in]``,
+``rec_weight [4*out,out]`` and ``bias [4*out]`` in PyTorch's gate order (input, forget, cell-in, output) and
+hands them to the backend; ``TorchBackend.lstm`` (returnn/torch/frontend/_backend.py:2718-2850) makes the
+input time-major, packs it by the sequence lengths, calls ``torch.lstm`` and returns the padded output
+plus the state after each sequence's last frame.  The TF-layers backend shows the mapping onto the native op
+(returnn/tf/frontend_layers/_backend.py:1199-1222): gates reordered to cell-in, input, forget, output, weights
+transposed to ``[in|out, 4*out]``, the input projection computed outside the op.
+
+:func:`lstm` is that backend function on plain HIP tensors (time-major ``[T,B,in]``, lengths as a tensor
+instead of a ``Dim``): one projection GEMM (hipBLASLt through ``torch.addmm``) into the op's ``X`` layout,
+then one ``NativeLstm2`` call with the right-padded 0/1 mask; output frames beyond a sequence's length are 0
+(what ``pad_packed_sequence`` yields), the new state is ``(h, c)`` after the last valid frame.
+``direction=-1`` runs the recurrence from each sequence's last frame to its first without reversing anything
+in memory (the caller protocol of returnn/tf/layers/rec.py:1229-1270).
+
+:class:`LSTM` and :class:`LstmState` mirror the module and its state; :class:`BlstmEncoder` stacks
+bidirectional layers (forward and backward op call per layer on one shared input, outputs concatenated).
+"""
+
+from __future__ import annotations
+
+import math
+from typing import NamedTuple, Optional, Sequence, Tuple, Union
+
+import torch
+
+from . import native_op
+from .torch_native_op import lstm_last_output, make_op
+
+__all__ = ["lstm", "prepare_weights", "LstmWeights", "LSTM", "LstmState", "BlstmEncoder", "sequence_mask_time_major"]
+
+
+class LstmState(NamedTuple):
+    """``h`` and ``c``, both [B,out] (returnn/frontend/rec.py:86-93)."""
+
+    h: torch.Tensor
+    c: torch.Tensor
+
+
+class LstmWeights(NamedTuple):
+    """Weights in the op's layout: gate order cell-in, input, forget, output along the ``4*out`` axis."""
+
+    ff: torch.Tensor  # [in, 4*out]
+    rec: torch.Tensor  # [out, 4*out]
+    bias: Optional[torch.Tensor]  # [4*out] or None
+
+
+def _to_native_gate_order(w: torch.Tensor) -> torch.Tensor:
+    """[4*out, ...] in (input, forget, cell-in, output) blocks -> (cell-in, input, forget, output)."""
+    i, f, g, o = w.chunk(4, dim=0)
+    return torch.cat((g, i, f, o), dim=0)
+
+
+def prepare_weights(
+    ff_weight: torch.Tensor, rec_weight: torch.Tensor, bias: Optional[torch.Tensor], *, dtype: Optional[torch.dtype] = None
+) -> LstmWeights:
+    """
+    Frontend parameters -> op layout (returnn/tf/frontend_layers/_backend.py:1199-1222): reorder the gate blocks
+    and transpose.  Worth caching while the parameters do not change; :class:`LSTM` does.
+
+    :param ff_weight: [4*out, in]
+    :param rec_weight: [4*out, out]
+    :param bias: [4*out] or None
+    :param dtype: activation type of the run (float32 or bfloat16); default: as ``ff_weight``
+    """
+    if ff_weight.dim() != 2 or rec_weight.dim() != 2 or ff_weight.shape[0] != rec_weight.shape[0]:
+        raise ValueError("lstm: ff_weight %s / rec_weight %s" % (tuple(ff_weight.shape), tuple(rec_weight.shape)))
+    out4, out = rec_weight.shape
+    if out4 != 4 * out:
+        raise ValueError("lstm: rec_weight must be [4*out,out], got %s" % (tuple(rec_weight.shape),))
+    if bias is not None and tuple(bias.shape) != (out4,):
+        raise ValueError("lstm: bias must be [4*out], got %s" % (tuple(bias.shape),))
+    dtype = dtype or ff_weight.dtype
+    ff = _to_native_gate_order(ff_weight).t().to(dtype).contiguous()
+    rec = _to_native_gate_order(rec_weight).t().to(dtype).contiguous()
+    b = None if bias is None else _to_native_gate_order(bias).to(dtype).contiguous()
+    return LstmWeights(ff=ff, rec=rec, bias=b)
+
+
+def sequence_mask_time_major(lengths: torch.Tensor, *, maxlen: int) -> torch.Tensor:
+    """[B] lengths -> [maxlen,B] float32 0/1 mask, right padded (returnn/torch/util/array_.py:196-208)."""
+    idx = torch.arange(maxlen, dtype=lengths.dtype, device=lengths.device)
+    return (idx[:, None] < lengths[None, :]).to(torch.float32)
+
+
+def _native_lstm2():
+    return make_op(native_op.NativeLstm2)
+
+
+def lstm(
+    source: torch.Tensor,
+    *,
+    state_h: torch.Tensor,
+    state_c: torch.Tensor,
+    ff_weight: Optional[torch.Tensor] = None,
+    rec_weight: Optional[torch.Tensor] = None,
+    bias: Optional[torch.Tensor] = None,
+    weights: Optional[LstmWeights] = None,
+    seq_lens: Optional[torch.Tensor] = None,
+    direction: int = 1,
+) -> Tuple[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
+    """
+    :param source: [T,B,in] time-major, or [B,in] for a single step (``single_step_dim`` in the reference);
+        float32 or bfloat16, on the GPU
+    :param state_h: [B,out] initial output
+    :param state_c: [B,out] initial cell
+    :param ff_weight: [4*out,in], gate order input, forget, cell-in, output (PyTorch's)
+    :param rec_weight: [4*out,out]
+    :param bias: [4*out] or None
+    :param weights: already prepared weights (:func:`prepare_weights`) instead of the three above
+    :param seq_lens: [B] integer lengths (any device), None = all sequences have T frames
+    :param direction: +1, or -1 for the backward-in-time layer of a bidirectional pair
+    :return: output [T,B,out] (or [B,out]), (h [B,out], c [B,out]) after each sequence's last processed frame;
+        output and h in the type of ``source``, c in float32
+    """
+    if direction not in (1, -1):
+        raise ValueError("lstm: direction must be +1 or -1")
+    single_step = source.dim() == 2
+    if single_step:
+        source = source[None]
+    if source.dim() != 3:
+        raise ValueError("lstm: source must be [T,B,in] or [B,in], got %s" % (tuple(source.shape),))
+    if not source.is_cuda:
+        raise RuntimeError("lstm: this build implements the LSTM for HIP (MI355X) tensors only; got a CPU tensor")
+    act = torch.bfloat16 if source.dtype == torch.bfloat16 else torch.float32
+    if weights is None:
+        if ff_weight is None or rec_weight is None:
+            raise ValueError("lstm: give ff_weight and rec_weight, or weights")
+        weights = prepare_weights(ff_weight, rec_weight, bias, dtype=act)
+    T, B, in_dim = source.shape
+    n = weights.rec.shape[0]
+    if weights.ff.shape[0] != in_dim:
+        raise ValueError("lstm: source has %i features, ff_weight expects %i" % (in_dim, weights.ff.shape[0]))
+    if tuple(state_h.shape) != (B, n) or tuple(state_c.shape) != (B, n):
+        raise ValueError("lstm: state_h %s / state_c %s, expected %s" % (tuple(state_h.shape), tuple(state_c.shape), (B, n)))
+    device = source.device
+    src2 = source.to(act).reshape(T * B, in_dim)
+    ff = weights.ff.to(act)
+    if weights.bias is not None:
+        X = torch.addmm(weights.bias.to(act), src2, ff)
+    else:
+        X = torch.mm(src2, ff)
+    X = X.view(T, B, 4 * n)
+    if seq_lens is None:
+        mask = torch.ones((T, B), dtype=torch.float32, device=device)
+    else:
+        if tuple(seq_lens.shape) != (B,):
+            raise ValueError("lstm: seq_lens must be [B]=[%i], got %s" % (B, tuple(seq_lens.shape)))
+        mask = sequence_mask_time_major(seq_lens.to(device), maxlen=T)
+    Y, _C, _H, d = _native_lstm2()(X, weights.rec, state_h, state_c, mask, 0, direction)
+    h = lstm_last_output(Y, state_h, mask, 0, direction) if T > 0 else state_h.to(act)
+    if single_step:
+        Y = Y[0]
+    return Y, (h, d)
+
+
+class LSTM(torch.nn.Module):
+    """
+    The module of returnn/frontend/rec.py:16-83 with integer dims: parameters ``ff_weight [4*out,in]``,
+    ``rec_weight [4*out,out]`` (both Glorot-uniform, returnn/frontend/init.py:189-197) and ``bias [4*out]`` (zeros).
+    """
+
+    def __init__(self, in_dim: int, out_dim: int, *, with_bias: bool = True, device=None, dtype=None):
+        super().__init__()
+        self.in_dim = int(in_dim)
+        self.out_dim = int(out_dim)
+        kw = dict(device=device, dtype=dtype)
+        self.ff_weight = torch.nn.Parameter(torch.empty((4 * self.out_dim, self.in_dim), **kw))
+        self.rec_weight = torch.nn.Parameter(torch.empty((4 * self.out_dim, self.out_dim), **kw))
+        self.bias = torch.nn.Parameter(torch.zeros((4 * self.out_dim,), **kw)) if with_bias else None
+        self.reset_parameters()
+        self._prepared = None  # (key, LstmWeights)
+
+    def reset_parameters(self, generator: Optional[torch.Generator] = None):
+        with torch.no_grad():
+            for p in (self.ff_weight, self.rec_weight):
+                limit = math.sqrt(6.0 / (p.shape[0] + p.shape[1]))  # scale 1 / fan_avg, uniform: sqrt(3*scale)
+                p.uniform_(-limit, limit, generator=generator)
+            if self.bias is not None:
+                self.bias.zero_()
+
+    def _weights(self, act: torch.dtype) -> LstmWeights:
+        ps = [self.ff_weight, self.rec_weight] + ([self.bias] if self.bias is not None else [])
+        key = (act,) + tuple((p.data_ptr(), p._version, p.device) for p in ps)
+        if self._prepared is None or self._prepared[0] != key:
+            with torch.no_grad():
+                self._prepared = (key, prepare_weights(self.ff_weight, self.rec_weight, self.bias, dtype=act))
+        return self._prepared[1]
+
+    def forward(
+        self, source: torch.Tensor, *, state: LstmState, seq_lens: Optional[torch.Tensor] = None, direction: int = 1
+    ) -> Tuple[torch.Tensor, LstmState]:
+        """
+        :param source: [T,B,in], or [B,in] for a single step
+        :param state: h and c, [B,out]
+        :param seq_lens: [B] or None
+        :return: output [T,B,out] (or [B,out]), new state
+        """
+        if state.h is None or state.c is None:
+            raise ValueError("%s: state %r needs attributes ``h`` (hidden) and ``c`` (cell)." % (self, state))
+        if source.shape[-1] != self.in_dim:
+            raise ValueError("%s: input %s does not have in_dim %i" % (self, tuple(source.shape), self.in_dim))
+        act = torch.bfloat16 if source.dtype == torch.bfloat16 else torch.float32
+        out, (h, c) = lstm(
+            source, state_h=state.h, state_c=state.c, weights=self._weights(act), seq_lens=seq_lens, direction=direction
+        )
+        return out, LstmState(h=h, c=c)
+
+    def default_initial_state(self, *, batch_dims: Sequence[int], device=None) -> LstmState:
+        """zeros (returnn/frontend/rec.py:78-83); h in the parameters' type, c in float32"""
+        device = device or self.rec_weight.device
+        shape = tuple(batch_dims) + (self.out_dim,)
+        return LstmState(
+            h=torch.zeros(shape, dtype=self.rec_weight.dtype, device=device),
+            c=torch.zeros(shape, dtype=torch.float32, device=device),
+        )
+
+    def extra_repr(self) -> str:
+        return "in_dim=%i, out_dim=%i, with_bias=%s" % (self.in_dim, self.out_dim, self.bias is not None)
+
+
+class BlstmEncoder(torch.nn.Module):
+    """
+    Stack of bidirectional LSTM layers: per layer a forward-in-time and a backward-in-time :class:`LSTM` on the same
+    input, outputs concatenated to ``2*out_dim`` features, which feed the next layer.  All layers use the same
+    sequence lengths; states start at zero.
+    """
+
+    def __init__(self, in_dim: int, out_dim: int, num_layers: int, *, with_bias: bool = True, device=None, dtype=None):
+        super().__init__()
+        self.in_dim, self.out_dim, self.num_layers = int(in_dim), int(out_dim), int(num_layers)
+        self.fwd = torch.nn.ModuleList()
+        self.bwd = torch.nn.ModuleList()
+        for layer in range(self.num_layers):
+            d_in = self.in_dim if layer == 0 else 2 * self.out_dim
+            self.fwd.append(LSTM(d_in, self.out_dim, with_bias=with_bias, device=device, dtype=dtype))
+            self.bwd.append(LSTM(d_in, self.out_dim, with_bias=with_bias, device=device, dtype=dtype))
+
+    def reset_parameters(self, generator: Optional[torch.Generator] = None):
+        for m in list(self.fwd) + list(self.bwd):
+            m.reset_parameters(generator)
+
+    @classmethod
+    def from_params(cls, layers, *, device=None, dtype=None) -> "BlstmEncoder":
+        """
+        :param layers: per layer ``{"fwd": p, "bwd": p}`` with ``p = {"ff_weight" [4n,in], "rec_weight" [4n,n], "bias" [4n] or None}``
+            (arrays or tensors, frontend layout)
+        """
+        first = layers[0]["fwd"]
+        n = first["rec_weight"].shape[1]
+        with_bias = first.get("bias") is not None
+        enc = cls(first["ff_weight"].shape[1], n, len(layers), with_bias=with_bias, device=device, dtype=dtype)
+        with torch.no_grad():
+            for layer, mods in zip(layers, zip(enc.fwd, enc.bwd)):
+                for key, mod in zip(("fwd", "bwd"), mods):
+                    for name in ("ff_weight", "rec_weight") + (("bias",) if with_bias else ()):
+                        getattr(mod, name).copy_(torch.as_tensor(layer[key][name]))
+        return enc
+
+    def forward(
+        self, source: torch.Tensor, *, seq_lens: Optional[torch.Tensor] = None, collect_states: bool = False
+    ) -> Union[torch.Tensor, Tuple[torch.Tensor, list]]:
+        """
+        :param source: [T,B,in]
+        :param seq_lens: [B] or None
+        :param collect_states: also return per layer ``(LstmState fwd, LstmState bwd)``
+        :return: [T,B,2*out_dim]
+        """
+        x = source
+        B = source.shape[1]
+        states = []
+        for f, b in zip(self.fwd, self.bwd):
+            s0 = f.default_initial_state(batch_dims=(B,), device=source.device)
+            s0 = LstmState(h=s0.h.to(x.dtype), c=s0.c)
+            yf, sf = f(x, state=s0, seq_lens=seq_lens, direction=1)
+            yb, sb = b(x, state=s0, seq_lens=seq_lens, direction=-1)
+            x = torch.cat((yf, yb), dim=-1)
+            states.append((sf, sb))
+        return (x, states) if collect_states else x

@@ -106,3 +106,80 @@ def round_to_bf16(a: numpy.ndarray) -> numpy.ndarray:
     nan = numpy.isnan(a)
     out[nan] = numpy.nan
     return out
+
+
+@dataclasses.dataclass
+class EncoderProblem:
+    """A stack of bidirectional LSTM layers: features, lengths and per layer and direction the frontend parameters."""
+
+    name: str
+    features: numpy.ndarray  # [T,B,in]
+    lens: numpy.ndarray  # [B]
+    layers: list  # per layer {"fwd": params, "bwd": params}; params = {"ff_weight" [4n,in_l], "rec_weight" [4n,n], "bias" [4n]}
+    n: int
+    dtype: str
+
+    @property
+    def T(self) -> int:
+        return self.features.shape[0]
+
+    @property
+    def B(self) -> int:
+        return self.features.shape[1]
+
+    @property
+    def in_dim(self) -> int:
+        return self.features.shape[2]
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+
+def glorot_uniform(rng: numpy.random.Generator, shape) -> numpy.ndarray:
+    """Uniform in +-sqrt(6/(d0+d1)): variance scaling with scale 1, mode fan_avg (returnn/frontend/init.py:172-197, 236-238)."""
+    limit = math.sqrt(6.0 / (shape[0] + shape[1]))
+    return rng.uniform(-limit, limit, shape).astype(numpy.float32)
+
+
+def make_encoder_config(
+    name: str = "cfg4",
+    *,
+    seed: int = 0,
+    T: Optional[int] = None,
+    B: Optional[int] = None,
+    n: Optional[int] = None,
+    num_layers: Optional[int] = None,
+    in_dim: Optional[int] = None,
+    bias_std: float = 0.0,
+) -> EncoderProblem:
+    """
+    "cfg4": 6-layer bidirectional LSTM encoder, bf16: features [1000,32,80] ~ N(0,1), n=1024 per direction,
+    layer inputs 80 then 2048, weights Glorot-uniform in the frontend layout (``ff_weight [4n,in]``,
+    ``rec_weight [4n,n]``, gate order input, forget, cell-in, output), bias zero, lengths uniform in [500,1000]
+    shared by all layers.  The overrides give scaled-down variants; ``bias_std`` > 0 draws a random bias instead.
+    """
+    assert name == "cfg4"
+    T_full = 1000
+    T = T_full if T is None else int(T)
+    B = 32 if B is None else int(B)
+    n = 1024 if n is None else int(n)
+    num_layers = 6 if num_layers is None else int(num_layers)
+    in_dim = 80 if in_dim is None else int(in_dim)
+    rng = numpy.random.default_rng(seed)
+    features = rng.standard_normal((T, B, in_dim), dtype=numpy.float32)
+    lo = max(1, (500 * T) // T_full)
+    lens = rng.integers(lo, T + 1, size=(B,))
+    lens[0] = T
+    layers = []
+    for layer in range(num_layers):
+        d_in = in_dim if layer == 0 else 2 * n
+        entry = {}
+        for direction in ("fwd", "bwd"):
+            entry[direction] = {
+                "ff_weight": glorot_uniform(rng, (4 * n, d_in)),
+                "rec_weight": glorot_uniform(rng, (4 * n, n)),
+                "bias": (rng.standard_normal((4 * n,)) * bias_std).astype(numpy.float32),
+            }
+        layers.append(entry)
+    return EncoderProblem(name=name, features=features, lens=lens, layers=layers, n=n, dtype="bf16")

@@ -1,0 +1,127 @@
+"""
+CPU checks of the LSTM layer's host logic: the parameter mapping onto the op (gate reorder, transpose,
+projection outside the op, mask from lengths, direction) is pinned by running the mapped problem through the
+CPU oracle and comparing with ``torch.nn.LSTM`` on the packed batch -- the behaviour the reference's frontend
+test expects of the layer (tests/test_rf_rec.py:13-43 via the torch backend).
+"""
+
+from __future__ import annotations
+
+import math
+
+import numpy
+import pytest
+import torch
+from numpy.testing import assert_allclose
+
+from oracle import lstm2_oracle as oracle
+from returnn_amd import lstm as rlstm
+from returnn_amd import synthetic
+from _torch_ref import blstm_layer
+
+
+def _params(rng, n, d_in, bias=True):
+    return {
+        "ff_weight": synthetic.glorot_uniform(rng, (4 * n, d_in)),
+        "rec_weight": synthetic.glorot_uniform(rng, (4 * n, n)),
+        "bias": rng.standard_normal(4 * n).astype(numpy.float32) * 0.3 if bias else None,
+    }
+
+
+def _layer_via_oracle(x, lens, p, h0, c0, direction):
+    """The steps of returnn_amd.lstm.lstm with numpy and the oracle in place of the GPU."""
+    w = rlstm.prepare_weights(
+        torch.from_numpy(p["ff_weight"]), torch.from_numpy(p["rec_weight"]),
+        None if p["bias"] is None else torch.from_numpy(p["bias"]), dtype=torch.float32,
+    )  # fmt: skip
+    T, B, _ = x.shape
+    X = x.astype(numpy.float64) @ w.ff.numpy().astype(numpy.float64)
+    if w.bias is not None:
+        X = X + w.bias.numpy()[None, None, :]
+    mask = numpy.ones((T, B), numpy.float32) if lens is None else rlstm.sequence_mask_time_major(torch.as_tensor(lens), maxlen=T).numpy()
+    Y, C, H, d, y_last = oracle.native_lstm2_fwd(X, w.rec.numpy(), h0, c0, mask, 0, direction, dtype=numpy.float64)
+    return Y, y_last, d
+
+
+@pytest.mark.parametrize("ragged", [False, True])
+@pytest.mark.parametrize("bias", [False, True])
+def test_mapping_matches_torch_lstm(ragged, bias):
+    rng = numpy.random.default_rng(11)
+    T, B, d_in, n = 9, 5, 7, 13  # dims of the reference's frontend test
+    x = rng.standard_normal((T, B, d_in)).astype(numpy.float32)
+    lens = numpy.array([9, 3, 1, 7, 9]) if ragged else None
+    fwd, bwd = _params(rng, n, d_in, bias), _params(rng, n, d_in, bias)
+    h0 = rng.standard_normal((2, B, n)).astype(numpy.float32) * 0.5
+    c0 = rng.standard_normal((2, B, n)).astype(numpy.float32) * 0.5
+    out, h, c = blstm_layer(x, lens, fwd, bwd, h0, c0)
+    for k, (p, direction) in enumerate(((fwd, 1), (bwd, -1))):
+        Y, y_last, d = _layer_via_oracle(x, lens, p, h0[k], c0[k], direction)
+        assert_allclose(Y, out[:, :, k * n : (k + 1) * n], rtol=1e-9, atol=1e-12)
+        assert_allclose(y_last, h[k], rtol=1e-9, atol=1e-12)
+        assert_allclose(d, c[k], rtol=1e-9, atol=1e-12)
+
+
+def test_gate_reorder_is_a_permutation_of_blocks():
+    n = 3
+    w = torch.arange(4 * n, dtype=torch.float32)[:, None] * torch.ones(1, 2)
+    lw = rlstm.prepare_weights(w, torch.zeros(4 * n, n), torch.arange(4 * n, dtype=torch.float32))
+    # input, forget, cell-in, output -> cell-in, input, forget, output
+    expect = list(range(2 * n, 3 * n)) + list(range(0, n)) + list(range(n, 2 * n)) + list(range(3 * n, 4 * n))
+    assert lw.ff.shape == (2, 4 * n) and lw.rec.shape == (n, 4 * n)
+    assert lw.ff[0].tolist() == expect and lw.bias.tolist() == expect
+    assert lw.ff.is_contiguous() and lw.rec.is_contiguous()
+
+
+def test_sequence_mask_time_major():
+    m = rlstm.sequence_mask_time_major(torch.tensor([3, 0, 5]), maxlen=5)
+    assert m.dtype == torch.float32 and m.shape == (5, 3)
+    assert m.t().tolist() == [[1, 1, 1, 0, 0], [0, 0, 0, 0, 0], [1, 1, 1, 1, 1]]
+
+
+def test_module_parameters_and_init():
+    torch.manual_seed(0)
+    m = rlstm.LSTM(80, 64)
+    assert m.ff_weight.shape == (256, 80) and m.rec_weight.shape == (256, 64) and m.bias.shape == (256,)
+    assert float(m.bias.detach().abs().max()) == 0.0
+    for p in (m.ff_weight, m.rec_weight):
+        limit = math.sqrt(6.0 / sum(p.shape))
+        p = p.detach()
+        assert float(p.abs().max()) <= limit
+        assert float(p.abs().max()) > 0.9 * limit
+        assert abs(float(p.var()) - limit * limit / 3.0) < 0.1 * limit * limit / 3.0  # variance 1/fan_avg
+    assert rlstm.LSTM(4, 4, with_bias=False).bias is None
+    s = m.default_initial_state(batch_dims=(3,))
+    assert s.h.shape == (3, 64) and s.c.shape == (3, 64) and float(s.h.abs().sum() + s.c.abs().sum()) == 0.0
+
+
+def test_no_cpu_implementation():
+    m = rlstm.LSTM(4, 8)
+    s = m.default_initial_state(batch_dims=(2,))
+    with pytest.raises(RuntimeError, match="HIP"):
+        m(torch.zeros(3, 2, 4), state=s)
+
+
+def test_argument_errors():
+    m = rlstm.LSTM(4, 8)
+    s = m.default_initial_state(batch_dims=(2,))
+    with pytest.raises(ValueError, match="in_dim"):
+        m(torch.zeros(3, 2, 5), state=s)
+    with pytest.raises(ValueError, match="needs attributes"):
+        m(torch.zeros(3, 2, 4), state=rlstm.LstmState(h=None, c=s.c))
+    with pytest.raises(ValueError, match="rec_weight"):
+        rlstm.prepare_weights(torch.zeros(32, 4), torch.zeros(32, 9), None)
+    with pytest.raises(ValueError, match="bias"):
+        rlstm.prepare_weights(torch.zeros(32, 4), torch.zeros(32, 8), torch.zeros(31))
+
+
+def test_encoder_config_shapes():
+    p = synthetic.make_encoder_config("cfg4", T=20, B=3, n=16, num_layers=3)
+    assert p.features.shape == (20, 3, 80) and p.lens.shape == (3,) and p.lens[0] == 20
+    assert p.lens.min() >= 10 and p.lens.max() <= 20
+    assert [l["fwd"]["ff_weight"].shape for l in p.layers] == [(64, 80), (64, 32), (64, 32)]
+    assert all(l[k]["rec_weight"].shape == (64, 16) for l in p.layers for k in ("fwd", "bwd"))
+    w = p.layers[1]["bwd"]["ff_weight"]
+    assert numpy.abs(w).max() <= math.sqrt(6.0 / (64 + 32))
+    enc = rlstm.BlstmEncoder.from_params(p.layers)
+    assert enc.num_layers == 3 and enc.in_dim == 80 and enc.out_dim == 16
+    assert torch.equal(enc.bwd[2].rec_weight.detach(), torch.from_numpy(p.layers[2]["bwd"]["rec_weight"]))
