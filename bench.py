@@ -33,9 +33,9 @@ PEAK_HBM = 8.0e12  # B/s
 
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by
 # what the same counter reads for a plain 1 GiB device copy); see profiles/k_lstm2_regw_cfg3_hbm_traffic.txt.
-# Keyed by (workload, plan as rtn_native_lstm2_describe_plan reports it up to the LDS size).
+# Keyed by (workload, launches per step, plan as rtn_native_lstm2_describe_plan reports it up to the LDS size).
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg3", "mode=persistent kernel=mfma_regw mt=2 nt=1 groups=2 wgs_per_group=128 wgs=256 rows_per_group=16"): 1268.4e6,
+    ("cfg3", 2, "mode=persistent kernel=mfma_regw mt=2 nt=1 groups=2 wgs_per_group=128 wgs=256 rows_per_group=16"): 1268.4e6,
 }
 
 
@@ -170,6 +170,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
     ap.add_argument("--mode", default="auto", choices=["auto", "persistent", "graph", "stepwise"])
+    ap.add_argument("--pair", default="fused", choices=["fused", "separate"],
+                    help="cfg3: issue the two directions through the multi-call entry (one launch when the device "
+                         "holds both; default) or as two separate op calls")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -224,8 +227,33 @@ def main():
             )
         )
     stream = torch.cuda.current_stream(dev)
+    fused = len(directions) == 2 and args.pair == "fused"
+    if fused:
+        call_list = (lib.Lstm2Call * 2)()
+        for k, o in enumerate(outs):
+            call_list[k] = lib.Lstm2Call(
+                X.data_ptr(), W.data_ptr(), y0.data_ptr(), c0.data_ptr(), msk.data_ptr(), 0, directions[k],
+                o["Y"].data_ptr(), o["C"].data_ptr(), o["H"].data_ptr(), o["d"].data_ptr(),
+            )  # fmt: skip
+        ws_pair = torch.empty((max(cabi.rtn_native_lstm2_fwd_multi_workspace_bytes(2, T, B, n, dt_code, mode), 256),),
+                              dtype=torch.uint8, device=dev)
+
+    def pair_call():
+        lib.check(cabi.rtn_native_lstm2_fwd_multi(call_list, 2, T, B, n, dt_code, mode, ws_pair.data_ptr(),
+                                                  ws_pair.numel(), stream.cuda_stream))  # fmt: skip
+
+    def check_status():
+        if os.environ.get("RTN_LSTM2_EXCHANGE") == "3":  # no-exchange timing aid: results are invalid
+            return
+        if fused:
+            lib.check(cabi.rtn_native_lstm2_fwd_multi_status(ws_pair.data_ptr(), 2, T, B, n, dt_code, mode, stream.cuda_stream))
+        else:
+            for k in range(len(directions)):
+                lib.check(cabi.rtn_native_lstm2_fwd_status(outs[k]["ws"].data_ptr(), stream.cuda_stream))
 
     def one_call(k):
+        if fused:
+            return pair_call()
         o = outs[k]
         rc = cabi.rtn_native_lstm2_fwd(
             X.data_ptr(), W.data_ptr(), y0.data_ptr(), c0.data_ptr(), msk.data_ptr(), 0, directions[k],
@@ -241,19 +269,18 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    launches = 1 if fused else len(directions)  # library entries per step
     for _ in range(args.warmup):
-        for k in range(len(directions)):
+        for k in range(launches):
             one_call(k)
     torch.cuda.synchronize()
-    for k in range(len(directions)):
-        if os.environ.get("RTN_LSTM2_EXCHANGE") != "3":
-            lib.check(cabi.rtn_native_lstm2_fwd_status(outs[k]["ws"].data_ptr(), stream.cuda_stream))
+    check_status()
 
     events = []
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        for k in range(len(directions)):
+        for k in range(launches):
             e0 = torch.cuda.Event(enable_timing=True)
             e1 = torch.cuda.Event(enable_timing=True)
             e0.record(stream)
@@ -262,20 +289,19 @@ def main():
             events.append((e0, e1))
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    measuring_only = os.environ.get("RTN_LSTM2_EXCHANGE") == "3"  # no-exchange timing aid: results are invalid
-    for k in range(len(directions)):
-        if not measuring_only:
-            lib.check(cabi.rtn_native_lstm2_fwd_status(outs[k]["ws"].data_ptr(), stream.cuda_stream))
+    measuring_only = os.environ.get("RTN_LSTM2_EXCHANGE") == "3"
+    check_status()
     assert measuring_only or all(bool(torch.isfinite(o["d"]).all()) for o in outs)
 
     call_ms = sum(a.elapsed_time(b) for a, b in events) / len(events)
     units_per_step = len(directions) * T * B
     value = units_per_step * args.steps / elapsed
-    flops_per_launch = 8.0 * T * B * n * n
+    units_per_launch = units_per_step // launches
+    flops_per_launch = 8.0 * n * n * units_per_launch
     achieved = flops_per_launch / (call_ms * 1e-3)
     peak = PEAK_MFMA[dtype]
-    bytes_per_launch = algorithmic_bytes_per_unit(n, dtype) * T * B
-    plan = lib.describe_plan(T, B, n, dt_code, mode)
+    bytes_per_launch = algorithmic_bytes_per_unit(n, dtype) * units_per_launch
+    plan = lib.describe_multi_plan(2 if fused else 1, T, B, n, dt_code, mode)
 
     result = {
         "metric": "LSTM fwd timesteps*seqs/sec (T*B/s) at n=%i" % n,
@@ -292,9 +318,12 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "%s: NativeLstm2 forward%s, T=%i B=%i n=%i %s, ragged=%s"
-            % (args.workload, " bidirectional pair (two calls: step=+1, step=-1)" if len(directions) == 2 else "", T, B, n,
-               dtype, p.lens is not None),
+            % (args.workload,
+               (" bidirectional pair (two op calls, step=+1 and step=-1, %s)"
+                % ("through the multi-call entry: one launch" if fused else "two entries")) if len(directions) == 2 else "",
+               T, B, n, dtype, p.lens is not None),
             "calls_per_step": len(directions),
+            "launches_per_step": launches,
             "units_per_step": units_per_step,
             "mode": args.mode,
             "plan": plan,
@@ -306,10 +335,11 @@ def main():
             "peak": peak / 1e12,
             "unit": "TFLOP/s",
             "frac": achieved / peak,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, plan.split(" group_per_xcd")[0])),
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, launches, plan.split(" group_per_xcd")[0])),
             "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE); algorithmic: %i" % bytes_per_launch,
-            "kernel": "%s (one launch = one op call of T*B = %i units, 8*n^2 flops each)"
-            % ("k_lstm2_regw" if "mfma_regw" in plan else ("k_lstm2_mfma" if "mfma_lds" in plan else "k_step_generic"), T * B),
+            "kernel": "%s (one launch = %i op call(s) = %i units of T*B, 8*n^2 flops each)"
+            % ("k_lstm2_regw" if "mfma_regw" in plan else ("k_lstm2_mfma" if "mfma_lds" in plan else "k_step_generic"),
+               len(directions) // launches, units_per_launch),
             "launch_ms": call_ms,
             "hbm_algorithmic_GBps": bytes_per_launch / (call_ms * 1e-3) / 1e9,
             "hbm_frac": bytes_per_launch / (call_ms * 1e-3) / PEAK_HBM,

@@ -96,6 +96,43 @@ size_t rtn_native_lstm2_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int
 int rtn_native_lstm2_fwd_status(const void* workspace, void* hip_stream);
 
 /*
+ * Several independent NativeLstm2 forward calls of one shape (T, B, n, dtype) in one entry: the two
+ * directions of a bidirectional layer (one op call with step=+1 and one with step=-1 on the same
+ * frames, returnn/tf/layers/rec.py:1229-1270), or the same layer of several streams.  Each element
+ * holds the arguments of one rtn_native_lstm2_fwd call and gets exactly that call's results.  When
+ * the device can hold the persistent kernel of all of them at once, they run in ONE cooperative
+ * launch and hide each other's exchange latency; otherwise they are enqueued back to back.
+ * `workspace` holds `count` equal slices, slice k for call k;
+ * rtn_native_lstm2_fwd_multi_workspace_bytes(count, ...) gives the total (a slice can be larger than a single
+ * call's workspace, because the decomposition may differ when several problems share the device).  The calls must not alias each
+ * other's outputs.
+ */
+typedef struct rtn_lstm2_call {
+  const void* X;
+  const void* W;
+  const void* y0;
+  const float* c0;
+  const float* i;
+  int32_t start;
+  int32_t step;
+  void* Y;
+  float* C;
+  void* H;
+  float* d;
+} rtn_lstm2_call;
+
+int rtn_native_lstm2_fwd_multi(const rtn_lstm2_call* calls, int32_t count, int64_t T, int32_t B, int32_t n,
+                               int32_t dtype, int32_t mode, void* workspace, size_t workspace_bytes,
+                               void* hip_stream);
+
+size_t rtn_native_lstm2_fwd_multi_workspace_bytes(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype,
+                                                  int32_t mode);
+
+/* rtn_native_lstm2_fwd_status over all `count` slices of a multi-call workspace; first failure wins. */
+int rtn_native_lstm2_fwd_multi_status(const void* workspace, int32_t count, int64_t T, int32_t B, int32_t n,
+                                      int32_t dtype, int32_t mode, void* hip_stream);
+
+/*
  * Final output per sequence.  Replaces the caller-side `_lstm_last_output`
  * (returnn/tf/native_op.py:913-929): out[b] = Y[t*, b] for the last visited frame t*
  * (in processing order) with i[t*, b] != 0, else y0[b].  Y, y0, out have element
@@ -112,6 +149,11 @@ const char* rtn_last_error(void);
  * ("mode=persistent mt=1 nt=2 groups=1 wgs=256 lds=40960 ..."); for logs and tests.
  * Counterpart of the reference's compile log next to the .so (returnn/util/native_code_compiler.py:348-352). */
 const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode);
+
+/* The plan used when `count` problems of this shape come in through rtn_native_lstm2_fwd_multi
+ * (count = 1: same as rtn_native_lstm2_describe_plan). */
+const char* rtn_native_lstm2_describe_multi_plan(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype,
+                                                 int32_t mode);
 
 /* ABI version of this header. */
 int rtn_native_lstm2_abi_version(void);

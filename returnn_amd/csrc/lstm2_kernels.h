@@ -675,23 +675,28 @@ struct LaneMax<__bf16> {
 };
 
 // Optional instrumentation (-DRTN_LSTM2_TRACE): wave 0 of every workgroup accumulates shader-clock
-// cycles per phase of k_lstm2_regw's step and writes the 8 totals to trace[blockIdx * 8 ..] at the end.
+// cycles per phase of k_lstm2_regw's step and writes the 8 totals to trace[workgroup * 8 ..] at the end.
 #ifdef RTN_LSTM2_TRACE
 #define RTN_TRACE_DECL unsigned long long tr_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long tr_last = clock64();
 #define RTN_TRACE_MARK(k) { const unsigned long long tr_now = clock64(); tr_acc[k] += tr_now - tr_last; tr_last = tr_now; }
 #define RTN_TRACE_ADD(k, v) { tr_acc[k] += (v); }
-#define RTN_TRACE_FLUSH(p) if ((p).trace && threadIdx.x == 0) { for (int k = 0; k < 8; ++k) (p).trace[(size_t)blockIdx.x * 8 + k] = tr_acc[k]; }
+#define RTN_TRACE_FLUSH(p, bid) if ((p).trace && threadIdx.x == 0) { for (int k = 0; k < 8; ++k) (p).trace[(size_t)(bid) * 8 + k] = tr_acc[k]; }
 #else
 #define RTN_TRACE_DECL
 #define RTN_TRACE_MARK(k)
 #define RTN_TRACE_ADD(k, v)
-#define RTN_TRACE_FLUSH(p)
+#define RTN_TRACE_FLUSH(p, bid)
 #endif
 
 constexpr unsigned kOobOffset = 0xFFFFFF00u;  // a buffer offset beyond any frame: loads give 0, stores are dropped
 
 template <typename AT, int MT, int NT, int KSMAX>
-__global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) {
+__global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi multi) {
+  // Which of the launch's problems this workgroup works on (uniform over the workgroup).
+  const int which = (int)blockIdx.x / multi.wgs_each;
+  const int bid = (int)blockIdx.x - which * multi.wgs_each;
+  if (which >= multi.count || bid >= multi.grid) return;
+  const Lstm2Params p = multi.p[which];
   using E = Elem<AT>;
   using SN = Sentinel<AT>;
   using LM = LaneMax<AT>;
@@ -713,7 +718,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in a scalar register
   const int n = p.n, S = n / KM;
   int g, r;
-  map_block_regw(p, blockIdx.x, g, r);
+  map_block_regw(p, bid, g, r);
   if (g < 0) return;
   const int G = p.wgs_per_group;
   const int b_base = g * p.Bg;
@@ -1038,7 +1043,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Params p) 
       step(s, IntTag<0>{});
       if (s + 1 < nsteps) step(s + 1, IntTag<1>{});
     }
-    RTN_TRACE_FLUSH(p)
+    RTN_TRACE_FLUSH(p, bid)
   };
   if (same_xcd && p.exchange == kExNt)
     run(IntTag<kExNt>{});

@@ -55,4 +55,15 @@ struct Lstm2Params {
   unsigned long long timeout_ticks;  // bound of one flag wait, in 100 MHz wall-clock ticks
 };
 
+// Several independent problems of one shape in one launch of the persistent register kernel: workgroups
+// [k * wgs_each, k * wgs_each + grid) run problem k; the rest of each slice leaves at once.
+constexpr int kMaxMulti = 4;
+struct Lstm2Multi {
+  int count;     // problems, 1..kMaxMulti
+  int wgs_each;  // workgroup ids reserved per problem, a multiple of the XCD count (keeps the id -> XCD dealing in phase)
+  int grid;      // workgroups a problem really uses (<= wgs_each)
+  int pad_;
+  Lstm2Params p[kMaxMulti];
+};
+
 }  // namespace rtn

@@ -119,7 +119,7 @@ size_t mfma_lds_bytes(int n, int dtype, int MT, int NT) {
 // under capture (a cooperative launch cannot be recorded).  Returns false with a reason when
 // mode == PERSISTENT is impossible.
 bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing, Plan* out, std::string* why,
-               int max_wgs_per_cu = 2) {
+               int max_wgs_per_cu = 2, int count = 1) {
   Plan pl;
   // Two workgroups per CU and whole groups per XCD only pay off with the (experimental) same-XCD exchange.
   const long env_exchange = env_long("RTN_LSTM2_EXCHANGE", 0);
@@ -187,7 +187,19 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
             // the fragments it holds.
             const double mfma_us = (double)MT * NT * ks * (dtype == RTN_DTYPE_BF16 ? 16 : 128) / 2400.0;
             const int ept = (MT * NT + kWaves - 1) / kWaves;
-            const double est = 2.0 * mfma_us + 0.4 * (ept - 1) + (compact ? 0.0 : 0.004 * G) + 0.03 * ks * NT + 0.01 * MT * ks;
+            double est = 2.0 * mfma_us + 0.4 * (ept - 1) + (compact ? 0.0 : 0.004 * G) + 0.03 * ks * NT + 0.01 * MT * ks;
+            // Several problems in one launch: as long as every workgroup has a CU to itself they do not slow
+            // each other down; sharing CUs costs about a third, running in turns costs the whole time again.
+            if (count > 1) {
+              const long long each = (long long)align_up((size_t)(groups * G), (size_t)di.xcds);
+              const long long fit1 = di.cus / each, fit2 = 2 * (long long)di.cus / each;
+              if (fit1 >= count)
+                ;
+              else if (use_regw && fit2 >= count)
+                est *= 1.35;
+              else
+                est *= (double)((count + std::max<long long>(fit2, 1) - 1) / std::max<long long>(fit2, 1)) * (fit2 >= 2 ? 1.35 : 1.0);
+            }
             if (est < best) {
               best = est;
               pl.regw = use_regw != 0;
@@ -299,7 +311,7 @@ MfmaKernel mfma_kernel(int dtype, int MT, int NT) {
   return dtype == RTN_DTYPE_BF16 ? mfma_kernel_for<__bf16>(MT, NT) : mfma_kernel_for<float>(MT, NT);
 }
 
-typedef void (*RegwKernel)(const Lstm2Params);
+typedef void (*RegwKernel)(const Lstm2Multi);
 
 template <typename AT>
 RegwKernel regw_kernel_for(int MT, int NT, int KSMAX) {
@@ -437,79 +449,59 @@ int check_dims(int64_t T, int32_t B, int32_t n, int32_t dtype) {
   return RTN_OK;
 }
 
-}  // namespace
-}  // namespace rtn
 
-using namespace rtn;
-
-extern "C" {
-
-int rtn_native_lstm2_abi_version(void) { return 1; }
-
-const char* rtn_last_error(void) { return g_last_error.c_str(); }
-
-size_t rtn_native_lstm2_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
-  if (check_dims(T, B, n, dtype) != RTN_OK) return 0;
-  if (mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return 0;
-  // The largest layout any resolution of `mode` can need: AUTO may fall back to per-step launches.
+// Workspace of one problem of an entry with `count` problems: the largest layout any resolution of `mode`
+// can need (AUTO may fall back to per-step launches, and the plan depends on how many problems share a launch).
+size_t workspace_each(int count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
   size_t need = 0;
   Plan pl;
   std::string why;
-  if (make_plan(T, B, n, dtype, mode, false, &pl, &why)) need = std::max(need, pl.total);
-  if (mode == RTN_MODE_AUTO || mode == RTN_MODE_PERSISTENT) {
-    // what the call may settle on when the device gives the kernel fewer workgroups per CU, or none at all
-    if (make_plan(T, B, n, dtype, mode, false, &pl, &why, 1)) need = std::max(need, pl.total);
-    if (make_plan(T, B, n, dtype, RTN_MODE_STEPWISE, true, &pl, &why)) need = std::max(need, pl.total);
+  for (int c : {1, std::max(1, std::min(count, kMaxMulti))}) {
+    if (make_plan(T, B, n, dtype, mode, false, &pl, &why, 2, c)) need = std::max(need, pl.total);
+    if (mode == RTN_MODE_AUTO || mode == RTN_MODE_PERSISTENT) {
+      // what the call may settle on when the device gives the kernel fewer workgroups per CU, or none at all
+      if (make_plan(T, B, n, dtype, mode, false, &pl, &why, 1, c)) need = std::max(need, pl.total);
+      if (make_plan(T, B, n, dtype, RTN_MODE_STEPWISE, true, &pl, &why)) need = std::max(need, pl.total);
+    }
   }
   return need;
 }
 
-const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
-  Plan pl;
-  std::string why;
-  char buf[512];
-  if (check_dims(T, B, n, dtype) != RTN_OK) {
-    g_plan_text = "invalid: " + g_last_error;
-  } else if (!make_plan(T, B, n, dtype, mode, false, &pl, &why)) {
-    g_plan_text = "unsupported: " + why;
-  } else {
-    snprintf(buf, sizeof(buf), "mode=%s kernel=%s mt=%d nt=%d groups=%d wgs_per_group=%d wgs=%d rows_per_group=%d group_per_xcd=%d lds=%zu workspace=%zu",
-             mode_name(pl.mode),
-             pl.kind == kPlanMfma ? (pl.regw ? "mfma_regw" : "mfma_lds") : (pl.kind == kPlanGeneric ? "generic" : "empty"), pl.MT,
-             pl.NT, pl.groups, pl.wgs_per_group, (pl.mode == RTN_MODE_PERSISTENT && pl.regw) ? pl.grid : pl.groups * pl.wgs_per_group,
-             pl.Bg, pl.compact ? 1 : 0, pl.lds_bytes, pl.total);
-    if (pl.off_trace) snprintf(buf + strlen(buf), sizeof(buf) - strlen(buf), " trace_offset=%zu", pl.off_trace);
-    g_plan_text = buf;
-  }
-  return g_plan_text.c_str();
-}
-
-int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const float* c0, const float* i, int32_t start,
-                         int32_t step, void* Y, float* C, void* H, float* d, int64_t T, int32_t B, int32_t n,
-                         int32_t dtype, int32_t mode, void* workspace, size_t workspace_bytes, void* hip_stream) {
-  g_last_error.clear();
+// The calls of one entry: `count` independent problems of one shape.  Each gets the slice
+// [k * each, (k + 1) * each) of the workspace, each = workspace_each(count, ...).
+// When the persistent register kernel fits that many times on the device at once, all of them run
+// in one cooperative launch (their workgroups share the CUs and hide each other's exchange waits);
+// otherwise they are enqueued one after the other.
+int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode,
+              void* workspace, size_t workspace_bytes, void* hip_stream) {
   int rc = check_dims(T, B, n, dtype);
   if (rc != RTN_OK) return rc;
   if (mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return fail(RTN_ERR_ARG, "NativeLstm2: unknown mode %d", mode);
   hipStream_t stream = (hipStream_t)hip_stream;
   const long long bn = (long long)B * n;
 
-  if (bn > 0 && (!c0 || !d)) return fail(RTN_ERR_ARG, "NativeLstm2: c0 and d must not be null");
+  for (int k = 0; k < count; ++k)
+    if (bn > 0 && (!calls[k].c0 || !calls[k].d)) return fail(RTN_ERR_ARG, "NativeLstm2: c0 and d must not be null");
   if (T == 0 || bn == 0) {
     // returnn/native_op.py:1236-1237: no frames, the final cell state is the initial one.
-    if (bn > 0) {
-      hipLaunchKernelGGL(k_copy_f32, dim3((unsigned)std::min<long long>((bn + 255) / 256, 1024)), dim3(256), 0, stream, c0, d, bn);
+    for (int k = 0; k < count && bn > 0; ++k) {
+      hipLaunchKernelGGL(k_copy_f32, dim3((unsigned)std::min<long long>((bn + 255) / 256, 1024)), dim3(256), 0, stream,
+                         calls[k].c0, calls[k].d, bn);
       RTN_HIP(hipGetLastError());
     }
     return RTN_OK;
   }
-  if (start < 0 || start >= T) return fail(RTN_ERR_RANGE, "NativeLstm2: need 0 <= start < T, got start=%d, T=%lld", start, (long long)T);
-  if (step == 0) return fail(RTN_ERR_RANGE, "NativeLstm2: step must not be 0");
-  const void* ptrs[] = {X, W, y0, c0, i, Y, C, H, d};
-  const char* names[] = {"X", "W", "y0", "c0", "i", "Y", "C", "H", "d"};
-  for (int k = 0; k < 9; ++k) {
-    if (!ptrs[k]) return fail(RTN_ERR_ARG, "NativeLstm2: %s must not be null", names[k]);
-    if (k != 4 && !aligned16(ptrs[k])) return fail(RTN_ERR_ARG, "NativeLstm2: %s must be 16-byte aligned", names[k]);
+  for (int k = 0; k < count; ++k) {
+    const rtn_lstm2_call& c = calls[k];
+    if (c.start < 0 || c.start >= T)
+      return fail(RTN_ERR_RANGE, "NativeLstm2: need 0 <= start < T, got start=%d, T=%lld", c.start, (long long)T);
+    if (c.step == 0) return fail(RTN_ERR_RANGE, "NativeLstm2: step must not be 0");
+    const void* ptrs[] = {c.X, c.W, c.y0, c.c0, c.i, c.Y, c.C, c.H, c.d};
+    const char* names[] = {"X", "W", "y0", "c0", "i", "Y", "C", "H", "d"};
+    for (int q = 0; q < 9; ++q) {
+      if (!ptrs[q]) return fail(RTN_ERR_ARG, "NativeLstm2: %s must not be null", names[q]);
+      if (q != 4 && !aligned16(ptrs[q])) return fail(RTN_ERR_ARG, "NativeLstm2: %s must be 16-byte aligned", names[q]);
+    }
   }
 
   hipStreamCaptureStatus cap_status = hipStreamCaptureStatusNone;
@@ -518,11 +510,13 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
 
   Plan pl;
   std::string why;
-  if (!make_plan(T, B, n, dtype, mode, capturing, &pl, &why))
+  const int plan_count = env_long("RTN_LSTM2_NO_FUSE", 0) ? 1 : std::min(count, kMaxMulti);
+  if (!make_plan(T, B, n, dtype, mode, capturing, &pl, &why, 2, plan_count))
     return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: persistent mode unavailable for T=%lld B=%d n=%d: %s", (long long)T, B, n, why.c_str());
   // A persistent plan needs all its workgroups on the device together: check against what the kernel
   // really gets per CU, plan again for that if the plan was too optimistic, else fall back to per-step launches.
   const void* pk = nullptr;  // the persistent kernel, if any
+  int fused = 1;             // problems per cooperative launch
   for (int attempt = 0; pl.kind == kPlanMfma && pl.mode == RTN_MODE_PERSISTENT; ++attempt) {
     pk = pl.regw ? (const void*)regw_kernel(dtype, pl.MT, pl.NT, pl.KSMAX) : (const void*)mfma_kernel(dtype, pl.MT, pl.NT);
     if (!pk) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d ks=%d", pl.MT, pl.NT, pl.KSMAX);
@@ -531,95 +525,200 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
     const int wgs = pl.regw ? pl.grid : pl.groups * pl.wgs_per_group;
     int per_cu = 0;
     RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, pk, kWgThreads, pl.lds_bytes));
-    if ((long long)per_cu * device_info().cus >= wgs) break;
+    const long long capacity = (long long)per_cu * device_info().cus;
+    if (capacity >= wgs) {
+      if (pl.regw && count > 1 && !env_long("RTN_LSTM2_NO_FUSE", 0)) {
+        const long long each = (long long)align_up((size_t)wgs, (size_t)device_info().xcds);
+        fused = (int)std::min<long long>(std::min(count, kMaxMulti), capacity / each);
+        if (fused < 1) fused = 1;
+      }
+      break;
+    }
     pk = nullptr;
-    if (attempt == 0 && per_cu >= 1 && make_plan(T, B, n, dtype, mode, capturing, &pl, &why, per_cu)) continue;
+    if (attempt == 0 && per_cu >= 1 && make_plan(T, B, n, dtype, mode, capturing, &pl, &why, per_cu, plan_count)) continue;
     if (mode == RTN_MODE_PERSISTENT)
       return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: %d workgroups cannot be co-resident (%d per CU)", wgs, per_cu);
     if (!make_plan(T, B, n, dtype, RTN_MODE_GRAPH, capturing, &pl, &why))
       return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no per-step plan: %s", why.c_str());
     break;
   }
-  if (!workspace || workspace_bytes < pl.total)
-    return fail(RTN_ERR_WORKSPACE, "NativeLstm2: workspace of %zu bytes needed, got %zu", pl.total, workspace ? workspace_bytes : (size_t)0);
+  const size_t each_ws = count > 1 ? workspace_each(count, T, B, n, dtype, mode) : pl.total;
+  if (each_ws < pl.total) return fail(RTN_ERR_WORKSPACE, "NativeLstm2: internal: workspace slice %zu < layout %zu", each_ws, pl.total);
+  if (!workspace || workspace_bytes < each_ws * (size_t)count)
+    return fail(RTN_ERR_WORKSPACE, "NativeLstm2: workspace of %zu bytes needed, got %zu", each_ws * (size_t)count,
+                workspace ? workspace_bytes : (size_t)0);
   if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2: workspace must be 16-byte aligned");
 
-  Lstm2Params p;
-  memset(&p, 0, sizeof(p));
-  p.X = X; p.W = W; p.y0 = y0; p.c0 = c0; p.mask = i;
-  p.Y = Y; p.C = C; p.H = H; p.d = d;
-  unsigned char* ws = (unsigned char*)workspace;
-  p.status = (unsigned*)(ws + pl.off_status);
-  p.flags = (unsigned*)(ws + pl.off_flags);
-  p.hx = ws + pl.off_hx;
-  p.Wp = ws + pl.off_wp;
-  p.ycarry = ws + pl.off_ycarry;
-  p.trace = pl.off_trace ? (unsigned long long*)(ws + pl.off_trace) : nullptr;
-  p.T = T; p.B = B; p.n = n;
-  // returnn/native_op.py:1253-1259
-  if (step > 0) {
-    p.first = start;
-    p.nsteps = (int)((T - 1 - start) / step + 1);
-  } else {
-    p.first = (int)(T - start - 1);
-    p.nsteps = (int)(p.first / (-(long long)step) + 1);
-  }
-  p.step = step;
-  p.groups = pl.groups; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
-  p.hx_bufs = kHxRing;
-  p.hx_sentinel = pl.regw ? 1 : 0;
-  p.map_compact = pl.compact ? 1 : 0;
-  p.exchange = (int)env_long("RTN_LSTM2_EXCHANGE", 0);
-  if (p.exchange < 0 || p.exchange > 3) p.exchange = 0;  // 3: measurement aid, results invalid (status 2)
-  // Device-scope stores take about a microsecond to become visible: a first read issued at once would
-  // come back incomplete and cost a second round trip, so it is held back (tuned on MI355X).
-  p.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", p.exchange == 0 ? 20 : 8)));
-  p.xcds = device_info().xcds;
-  p.sync_policy = (int)env_long("RTN_LSTM2_SYNC", kStoreCoherent | kLoadCoherent);
-  if (!((p.sync_policy & (kStoreCoherent | kReleaseFence)) && (p.sync_policy & (kLoadCoherent | kAcquireFence))))
-    return fail(RTN_ERR_ARG, "NativeLstm2: RTN_LSTM2_SYNC=%d is not a valid publication policy", p.sync_policy);
-  p.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);  // 2 s at 100 MHz
-
-  // Frames the loop never visits.
-  if (p.nsteps != T) {
-    const long long total = T * bn * 4;
-    const dim3 grid((unsigned)std::min<long long>((total + 255) / 256, 65535)), block(256);
-    if (dtype == RTN_DTYPE_BF16)
-      hipLaunchKernelGGL(k_fill_unvisited<__bf16>, grid, block, 0, stream, p);
-    else
-      hipLaunchKernelGGL(k_fill_unvisited<float>, grid, block, 0, stream, p);
-    RTN_HIP(hipGetLastError());
-  }
-
-  if (pl.kind == kPlanMfma) {
-    MfmaKernel k = mfma_kernel(dtype, pl.MT, pl.NT);
-    if (!pk) {
-      if (!k) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d", pl.MT, pl.NT);
-      rc = ensure_lds_limit((const void*)k, pl.lds_bytes);
-      if (rc != RTN_OK) return rc;
+  Lstm2Multi multi;
+  memset(&multi, 0, sizeof(multi));
+  int pending = 0;  // problems prepared for the next cooperative launch
+  for (int k = 0; k < count; ++k) {
+    const rtn_lstm2_call& c = calls[k];
+    Lstm2Params p;
+    memset(&p, 0, sizeof(p));
+    p.X = c.X; p.W = c.W; p.y0 = c.y0; p.c0 = c.c0; p.mask = c.i;
+    p.Y = c.Y; p.C = c.C; p.H = c.H; p.d = c.d;
+    unsigned char* ws = (unsigned char*)workspace + (size_t)k * each_ws;
+    p.status = (unsigned*)(ws + pl.off_status);
+    p.flags = (unsigned*)(ws + pl.off_flags);
+    p.hx = ws + pl.off_hx;
+    p.Wp = ws + pl.off_wp;
+    p.ycarry = ws + pl.off_ycarry;
+    p.trace = pl.off_trace ? (unsigned long long*)(ws + pl.off_trace) : nullptr;
+    p.T = T; p.B = B; p.n = n;
+    // returnn/native_op.py:1253-1259
+    if (c.step > 0) {
+      p.first = c.start;
+      p.nsteps = (int)((T - 1 - c.start) / c.step + 1);
+    } else {
+      p.first = (int)(T - c.start - 1);
+      p.nsteps = (int)(p.first / (-(long long)c.step) + 1);
     }
-    const long long work = std::max<long long>((long long)n * n, bn);
-    const dim3 pgrid((unsigned)std::min<long long>((work + 255) / 256, 2048)), pblock(256);
-    if (dtype == RTN_DTYPE_BF16)
-      hipLaunchKernelGGL(k_prepare_mfma<__bf16>, pgrid, pblock, 0, stream, p, pl.n_flags);
-    else
-      hipLaunchKernelGGL(k_prepare_mfma<float>, pgrid, pblock, 0, stream, p, pl.n_flags);
-    RTN_HIP(hipGetLastError());
-    if (pk) {
-      const int wgs = pl.regw ? pl.grid : pl.groups * pl.wgs_per_group;
-      int s_begin = 0, s_end = p.nsteps;
-      void* args_lds[] = {(void*)&p, (void*)&s_begin, (void*)&s_end};
-      void* args_regw[] = {(void*)&p};
-      RTN_HIP(hipLaunchCooperativeKernel(pk, dim3(wgs), dim3(kWgThreads),
-                                         pl.regw ? args_regw : args_lds, (unsigned)pl.lds_bytes, stream));
-      return RTN_OK;
+    p.step = c.step;
+    p.groups = pl.groups; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
+    p.hx_bufs = kHxRing;
+    p.hx_sentinel = pl.regw ? 1 : 0;
+    p.map_compact = pl.compact ? 1 : 0;
+    p.exchange = (int)env_long("RTN_LSTM2_EXCHANGE", 0);
+    if (p.exchange < 0 || p.exchange > 3) p.exchange = 0;  // 3: measurement aid, results invalid (status 2)
+    // Device-scope stores take about a microsecond to become visible: a first read issued at once would
+    // come back incomplete and cost a second round trip, so it is held back (tuned on MI355X).
+    p.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", p.exchange == 0 ? 20 : 8)));
+    p.xcds = device_info().xcds;
+    p.sync_policy = (int)env_long("RTN_LSTM2_SYNC", kStoreCoherent | kLoadCoherent);
+    if (!((p.sync_policy & (kStoreCoherent | kReleaseFence)) && (p.sync_policy & (kLoadCoherent | kAcquireFence))))
+      return fail(RTN_ERR_ARG, "NativeLstm2: RTN_LSTM2_SYNC=%d is not a valid publication policy", p.sync_policy);
+    p.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);  // 2 s at 100 MHz
+
+    // Frames the loop never visits.
+    if (p.nsteps != T) {
+      const long long total = T * bn * 4;
+      const dim3 grid((unsigned)std::min<long long>((total + 255) / 256, 65535)), block(256);
+      if (dtype == RTN_DTYPE_BF16)
+        hipLaunchKernelGGL(k_fill_unvisited<__bf16>, grid, block, 0, stream, p);
+      else
+        hipLaunchKernelGGL(k_fill_unvisited<float>, grid, block, 0, stream, p);
+      RTN_HIP(hipGetLastError());
     }
-  } else {
-    hipLaunchKernelGGL(k_clear_status, dim3(1), dim3(64), 0, stream, p.status);
-    RTN_HIP(hipGetLastError());
+
+    if (pl.kind == kPlanMfma) {
+      MfmaKernel mk = mfma_kernel(dtype, pl.MT, pl.NT);
+      if (!pk) {
+        if (!mk) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d", pl.MT, pl.NT);
+        rc = ensure_lds_limit((const void*)mk, pl.lds_bytes);
+        if (rc != RTN_OK) return rc;
+      }
+      const long long work = std::max<long long>((long long)n * n, bn);
+      const dim3 pgrid((unsigned)std::min<long long>((work + 255) / 256, 2048)), pblock(256);
+      if (dtype == RTN_DTYPE_BF16)
+        hipLaunchKernelGGL(k_prepare_mfma<__bf16>, pgrid, pblock, 0, stream, p, pl.n_flags);
+      else
+        hipLaunchKernelGGL(k_prepare_mfma<float>, pgrid, pblock, 0, stream, p, pl.n_flags);
+      RTN_HIP(hipGetLastError());
+      if (pk && pl.regw) {
+        multi.p[pending++] = p;
+        if (pending == fused || k + 1 == count) {
+          multi.count = pending;
+          multi.grid = pl.grid;
+          multi.wgs_each = (int)align_up((size_t)pl.grid, (size_t)device_info().xcds);
+          void* args[] = {(void*)&multi};
+          const int wgs = pending == 1 ? pl.grid : multi.wgs_each * pending;
+          RTN_HIP(hipLaunchCooperativeKernel(pk, dim3(wgs), dim3(kWgThreads), args, (unsigned)pl.lds_bytes, stream));
+          pending = 0;
+        }
+        continue;
+      }
+      if (pk) {
+        int s_begin = 0, s_end = p.nsteps;
+        void* args_lds[] = {(void*)&p, (void*)&s_begin, (void*)&s_end};
+        RTN_HIP(hipLaunchCooperativeKernel(pk, dim3(pl.groups * pl.wgs_per_group), dim3(kWgThreads), args_lds,
+                                           (unsigned)pl.lds_bytes, stream));
+        continue;
+      }
+    } else {
+      hipLaunchKernelGGL(k_clear_status, dim3(1), dim3(64), 0, stream, p.status);
+      RTN_HIP(hipGetLastError());
+    }
+    rc = (pl.mode == RTN_MODE_GRAPH && !capturing) ? launch_steps_graph(p, pl, dtype, stream) : launch_steps(p, pl, dtype, stream);
+    if (rc != RTN_OK) return rc;
   }
-  if (pl.mode == RTN_MODE_GRAPH && !capturing) return launch_steps_graph(p, pl, dtype, stream);
-  return launch_steps(p, pl, dtype, stream);
+  return RTN_OK;
+}
+
+}  // namespace
+}  // namespace rtn
+
+using namespace rtn;
+
+extern "C" {
+
+int rtn_native_lstm2_abi_version(void) { return 2; }
+
+const char* rtn_last_error(void) { return g_last_error.c_str(); }
+
+size_t rtn_native_lstm2_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
+  if (check_dims(T, B, n, dtype) != RTN_OK) return 0;
+  if (mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return 0;
+  return workspace_each(1, T, B, n, dtype, mode);
+}
+
+const char* rtn_native_lstm2_describe_multi_plan(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
+  Plan pl;
+  std::string why;
+  char buf[512];
+  const int c = env_long("RTN_LSTM2_NO_FUSE", 0) ? 1 : std::max(1, std::min(count, kMaxMulti));
+  if (check_dims(T, B, n, dtype) != RTN_OK) {
+    g_plan_text = "invalid: " + g_last_error;
+  } else if (!make_plan(T, B, n, dtype, mode, false, &pl, &why, 2, c)) {
+    g_plan_text = "unsupported: " + why;
+  } else {
+    snprintf(buf, sizeof(buf), "mode=%s kernel=%s mt=%d nt=%d groups=%d wgs_per_group=%d wgs=%d rows_per_group=%d group_per_xcd=%d lds=%zu workspace=%zu",
+             mode_name(pl.mode),
+             pl.kind == kPlanMfma ? (pl.regw ? "mfma_regw" : "mfma_lds") : (pl.kind == kPlanGeneric ? "generic" : "empty"), pl.MT,
+             pl.NT, pl.groups, pl.wgs_per_group, (pl.mode == RTN_MODE_PERSISTENT && pl.regw) ? pl.grid : pl.groups * pl.wgs_per_group,
+             pl.Bg, pl.compact ? 1 : 0, pl.lds_bytes, count > 1 ? workspace_each(count, T, B, n, dtype, mode) : pl.total);
+    if (pl.off_trace) snprintf(buf + strlen(buf), sizeof(buf) - strlen(buf), " trace_offset=%zu", pl.off_trace);
+    g_plan_text = buf;
+  }
+  return g_plan_text.c_str();
+}
+
+const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
+  return rtn_native_lstm2_describe_multi_plan(1, T, B, n, dtype, mode);
+}
+
+int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const float* c0, const float* i, int32_t start,
+                         int32_t step, void* Y, float* C, void* H, float* d, int64_t T, int32_t B, int32_t n,
+                         int32_t dtype, int32_t mode, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  g_last_error.clear();
+  rtn_lstm2_call call = {X, W, y0, c0, i, start, step, Y, C, H, d};
+  return fwd_calls(&call, 1, T, B, n, dtype, mode, workspace, workspace_bytes, hip_stream);
+}
+
+int rtn_native_lstm2_fwd_multi(const rtn_lstm2_call* calls, int32_t count, int64_t T, int32_t B, int32_t n,
+                               int32_t dtype, int32_t mode, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  g_last_error.clear();
+  if (count < 0 || (count > 0 && !calls)) return fail(RTN_ERR_ARG, "NativeLstm2: bad call list (count=%d)", count);
+  if (count == 0) return RTN_OK;
+  return fwd_calls(calls, count, T, B, n, dtype, mode, workspace, workspace_bytes, hip_stream);
+}
+
+size_t rtn_native_lstm2_fwd_multi_workspace_bytes(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
+  if (count < 0 || check_dims(T, B, n, dtype) != RTN_OK) return 0;
+  if (mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return 0;
+  return (size_t)count * workspace_each(count, T, B, n, dtype, mode);
+}
+
+int rtn_native_lstm2_fwd_multi_status(const void* workspace, int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype,
+                                      int32_t mode, void* hip_stream) {
+  g_last_error.clear();
+  const size_t each = count > 1 ? workspace_each(count, T, B, n, dtype, mode) : rtn_native_lstm2_fwd_workspace_bytes(T, B, n, dtype, mode);
+  if (!workspace || each == 0 || count < 0) return fail(RTN_ERR_ARG, "NativeLstm2: bad arguments to the status query");
+  for (int k = 0; k < count; ++k) {
+    const int rc = rtn_native_lstm2_fwd_status((const unsigned char*)workspace + (size_t)k * each, hip_stream);
+    if (rc != RTN_OK) return rc;
+  }
+  return RTN_OK;
 }
 
 int rtn_native_lstm2_fwd_status(const void* workspace, void* hip_stream) {

@@ -37,11 +37,35 @@ SYMBOLS = (
     "rtn_native_lstm2_fwd",
     "rtn_native_lstm2_fwd_workspace_bytes",
     "rtn_native_lstm2_fwd_status",
+    "rtn_native_lstm2_fwd_multi",
+    "rtn_native_lstm2_fwd_multi_workspace_bytes",
+    "rtn_native_lstm2_fwd_multi_status",
     "rtn_native_lstm2_last_output",
     "rtn_last_error",
     "rtn_native_lstm2_describe_plan",
+    "rtn_native_lstm2_describe_multi_plan",
     "rtn_native_lstm2_abi_version",
 )
+
+
+
+class Lstm2Call(ctypes.Structure):
+    """``rtn_lstm2_call``: the arguments of one op call inside ``rtn_native_lstm2_fwd_multi``."""
+
+    _fields_ = [
+        ("X", ctypes.c_void_p),
+        ("W", ctypes.c_void_p),
+        ("y0", ctypes.c_void_p),
+        ("c0", ctypes.c_void_p),
+        ("i", ctypes.c_void_p),
+        ("start", ctypes.c_int32),
+        ("step", ctypes.c_int32),
+        ("Y", ctypes.c_void_p),
+        ("C", ctypes.c_void_p),
+        ("H", ctypes.c_void_p),
+        ("d", ctypes.c_void_p),
+    ]
+
 
 _lock = threading.RLock()
 _lib: Optional[ctypes.CDLL] = None
@@ -71,12 +95,20 @@ def load() -> ctypes.CDLL:
         lib.rtn_native_lstm2_fwd_workspace_bytes.argtypes = [i64, i32, i32, i32, i32]
         lib.rtn_native_lstm2_fwd_status.restype = ctypes.c_int
         lib.rtn_native_lstm2_fwd_status.argtypes = [vp, vp]
+        lib.rtn_native_lstm2_fwd_multi.restype = ctypes.c_int
+        lib.rtn_native_lstm2_fwd_multi.argtypes = [ctypes.POINTER(Lstm2Call), i32, i64, i32, i32, i32, i32, vp, sz, vp]
+        lib.rtn_native_lstm2_fwd_multi_workspace_bytes.restype = sz
+        lib.rtn_native_lstm2_fwd_multi_workspace_bytes.argtypes = [i32, i64, i32, i32, i32, i32]
+        lib.rtn_native_lstm2_fwd_multi_status.restype = ctypes.c_int
+        lib.rtn_native_lstm2_fwd_multi_status.argtypes = [vp, i32, i64, i32, i32, i32, i32, vp]
         lib.rtn_native_lstm2_last_output.restype = ctypes.c_int
         lib.rtn_native_lstm2_last_output.argtypes = [vp, vp, vp, i32, i32, vp, i64, i32, i32, i32, vp]
         lib.rtn_last_error.restype = ctypes.c_char_p
         lib.rtn_last_error.argtypes = []
         lib.rtn_native_lstm2_describe_plan.restype = ctypes.c_char_p
         lib.rtn_native_lstm2_describe_plan.argtypes = [i64, i32, i32, i32, i32]
+        lib.rtn_native_lstm2_describe_multi_plan.restype = ctypes.c_char_p
+        lib.rtn_native_lstm2_describe_multi_plan.argtypes = [i32, i64, i32, i32, i32, i32]
         lib.rtn_native_lstm2_abi_version.restype = ctypes.c_int
         lib.rtn_native_lstm2_abi_version.argtypes = []
         _lib = lib
@@ -96,6 +128,10 @@ def check(rc: int) -> None:
 
 def describe_plan(T: int, B: int, n: int, dtype: int, mode: int) -> str:
     return load().rtn_native_lstm2_describe_plan(T, B, n, dtype, mode).decode("utf8", "replace")
+
+
+def describe_multi_plan(count: int, T: int, B: int, n: int, dtype: int, mode: int) -> str:
+    return load().rtn_native_lstm2_describe_multi_plan(count, T, B, n, dtype, mode).decode("utf8", "replace")
 
 
 def workspace_bytes(T: int, B: int, n: int, dtype: int, mode: int) -> int:

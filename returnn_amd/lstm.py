@@ -17,7 +17,8 @@ then one ``NativeLstm2`` call with the right-padded 0/1 mask; output frames beyo
 in memory (the caller protocol of returnn/tf/layers/rec.py:1229-1270).
 
 :class:`LSTM` and :class:`LstmState` mirror the module and its state; :class:`BlstmEncoder` stacks
-bidirectional layers (forward and backward op call per layer on one shared input, outputs concatenated).
+bidirectional layers (:func:`blstm`: both directions of a layer go through the library's multi-call entry, which
+runs them in one launch when the device can hold both; outputs concatenated).
 """
 
 from __future__ import annotations
@@ -28,9 +29,9 @@ from typing import NamedTuple, Optional, Sequence, Tuple, Union
 import torch
 
 from . import native_op
-from .torch_native_op import lstm_last_output, make_op
+from .torch_native_op import lstm_last_output, make_op, native_lstm2_multi
 
-__all__ = ["lstm", "prepare_weights", "LstmWeights", "LSTM", "LstmState", "BlstmEncoder", "sequence_mask_time_major"]
+__all__ = ["lstm", "blstm", "prepare_weights", "LstmWeights", "LSTM", "LstmState", "BlstmEncoder", "sequence_mask_time_major"]
 
 
 class LstmState(NamedTuple):
@@ -137,13 +138,7 @@ def lstm(
     if tuple(state_h.shape) != (B, n) or tuple(state_c.shape) != (B, n):
         raise ValueError("lstm: state_h %s / state_c %s, expected %s" % (tuple(state_h.shape), tuple(state_c.shape), (B, n)))
     device = source.device
-    src2 = source.to(act).reshape(T * B, in_dim)
-    ff = weights.ff.to(act)
-    if weights.bias is not None:
-        X = torch.addmm(weights.bias.to(act), src2, ff)
-    else:
-        X = torch.mm(src2, ff)
-    X = X.view(T, B, 4 * n)
+    X = _project(source, weights, act)
     if seq_lens is None:
         mask = torch.ones((T, B), dtype=torch.float32, device=device)
     else:
@@ -155,6 +150,65 @@ def lstm(
     if single_step:
         Y = Y[0]
     return Y, (h, d)
+
+
+def _project(source: torch.Tensor, weights: LstmWeights, act: torch.dtype) -> torch.Tensor:
+    """``X = source . ff + bias`` in the op's layout [T,B,4*out]."""
+    T, B, in_dim = source.shape
+    src2 = source.to(act).reshape(T * B, in_dim)
+    ff = weights.ff.to(act)
+    X = torch.addmm(weights.bias.to(act), src2, ff) if weights.bias is not None else torch.mm(src2, ff)
+    return X.view(T, B, ff.shape[1])
+
+
+def blstm(
+    source: torch.Tensor,
+    *,
+    fwd: LstmWeights,
+    bwd: LstmWeights,
+    state_fwd: LstmState,
+    state_bwd: LstmState,
+    seq_lens: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, LstmState, LstmState]:
+    """
+    Forward-in-time and backward-in-time layer on the same input: two projections, then both recurrences through
+    the library's multi-call entry (one launch when the device holds both), outputs concatenated.  Same results
+    as two :func:`lstm` calls with ``direction=+1`` and ``-1``.
+
+    :param source: [T,B,in]
+    :return: [T,B,2*out] (forward | backward), new forward state, new backward state
+    """
+    if source.dim() != 3:
+        raise ValueError("blstm: source must be [T,B,in], got %s" % (tuple(source.shape),))
+    if not source.is_cuda:
+        raise RuntimeError("blstm: this build implements the LSTM for HIP (MI355X) tensors only; got a CPU tensor")
+    act = torch.bfloat16 if source.dtype == torch.bfloat16 else torch.float32
+    T, B, in_dim = source.shape
+    n = fwd.rec.shape[0]
+    if bwd.rec.shape[0] != n or fwd.ff.shape[0] != in_dim or bwd.ff.shape[0] != in_dim:
+        raise ValueError("blstm: weights do not match each other or the input")
+    for st in (state_fwd, state_bwd):
+        if tuple(st.h.shape) != (B, n) or tuple(st.c.shape) != (B, n):
+            raise ValueError("blstm: state %s / %s, expected %s" % (tuple(st.h.shape), tuple(st.c.shape), (B, n)))
+    if seq_lens is None:
+        mask = torch.ones((T, B), dtype=torch.float32, device=source.device)
+    else:
+        if tuple(seq_lens.shape) != (B,):
+            raise ValueError("blstm: seq_lens must be [B]=[%i], got %s" % (B, tuple(seq_lens.shape)))
+        mask = sequence_mask_time_major(seq_lens.to(source.device), maxlen=T)
+    _native_lstm2()  # registers the op and fails loudly without the library
+    (Yf, _, _, df), (Yb, _, _, db) = native_lstm2_multi(
+        [
+            (_project(source, fwd, act), fwd.rec, state_fwd.h, state_fwd.c, mask, 0, 1),
+            (_project(source, bwd, act), bwd.rec, state_bwd.h, state_bwd.c, mask, 0, -1),
+        ]
+    )
+    if T > 0:
+        hf = lstm_last_output(Yf, state_fwd.h, mask, 0, 1)
+        hb = lstm_last_output(Yb, state_bwd.h, mask, 0, -1)
+    else:
+        hf, hb = state_fwd.h.to(act), state_bwd.h.to(act)
+    return torch.cat((Yf, Yb), dim=-1), LstmState(h=hf, c=df), LstmState(h=hb, c=db)
 
 
 class LSTM(torch.nn.Module):
@@ -275,8 +329,7 @@ class BlstmEncoder(torch.nn.Module):
         for f, b in zip(self.fwd, self.bwd):
             s0 = f.default_initial_state(batch_dims=(B,), device=source.device)
             s0 = LstmState(h=s0.h.to(x.dtype), c=s0.c)
-            yf, sf = f(x, state=s0, seq_lens=seq_lens, direction=1)
-            yb, sb = b(x, state=s0, seq_lens=seq_lens, direction=-1)
-            x = torch.cat((yf, yb), dim=-1)
+            act = torch.bfloat16 if x.dtype == torch.bfloat16 else torch.float32
+            x, sf, sb = blstm(x, fwd=f._weights(act), bwd=b._weights(act), state_fwd=s0, state_bwd=s0, seq_lens=seq_lens)
             states.append((sf, sb))
         return (x, states) if collect_states else x

@@ -154,8 +154,9 @@ def _check_ndim(t: torch.Tensor, info: Dict[str, Any]):
         raise RuntimeError("%s shape ndim is not %i, got shape %s" % (info["name"], info["ndim"], tuple(t.shape)))
 
 
-def _native_lstm2_device_impl(X, W, y0, c0, i, start, step):
-    """``NativeLstm2`` on HIP tensors: normalise the arguments, allocate outputs and scratch, enqueue the library call."""
+def _normalise_lstm2_args(X, W, y0, c0, i):
+    """Argument handling of the generated wrapper (returnn/torch/util/native_op.py:144-193) plus the op's shape
+    asserts (returnn/native_op.py:1215-1223) as hard errors.  Returns the tensors to hand to the library and (T, B, n, bf16)."""
     infos = native_op.NativeLstm2.in_info
     for t, info in zip((X, W, y0, c0, i), infos):
         _check_ndim(t, info)
@@ -170,7 +171,6 @@ def _native_lstm2_device_impl(X, W, y0, c0, i, start, step):
     X, W, y0, c0, i = (t if t.is_contiguous() else t.contiguous() for t in (X, W, y0, c0, i))
     T, B = i.shape
     n = y0.shape[1]
-    # the reference's shape asserts (returnn/native_op.py:1215-1223); hard errors here
     expect = {"X": (T, B, 4 * n), "W": (n, 4 * n), "y0": (B, n), "c0": (B, n)}
     for name, t in (("X", X), ("W", W), ("y0", y0), ("c0", c0)):
         if tuple(t.shape) != expect[name]:
@@ -178,14 +178,27 @@ def _native_lstm2_device_impl(X, W, y0, c0, i, start, step):
                 "NativeLstm2: %s has shape %s, expected %s (T=%i, B=%i from i; n=%i from y0)"
                 % (name, tuple(t.shape), expect[name], T, B, n)
             )
+    return (X, W, y0, c0, i), (T, B, n, bf16)
+
+
+def _alloc_lstm2_outputs(T, B, n, bf16, device):
+    act = torch.bfloat16 if bf16 else torch.float32
+    Y = torch.empty((T, B, n), dtype=act, device=device)
+    C = torch.empty((T, B, n), dtype=torch.float32, device=device)
+    H = torch.empty((T, B, 4 * n), dtype=act, device=device)
+    d = torch.empty((B, n), dtype=torch.float32, device=device)
+    return Y, C, H, d
+
+
+def _native_lstm2_device_impl(X, W, y0, c0, i, start, step):
+    """``NativeLstm2`` on HIP tensors: normalise the arguments, allocate outputs and scratch, enqueue the library call."""
+    (X, W, y0, c0, i), (T, B, n, bf16) = _normalise_lstm2_args(X, W, y0, c0, i)
+    device = X.device
     lib = _lib.load()
     dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
     mode = _lib.MODES[OpMaker.options.get("NativeLstm2", {}).get("mode", "auto")]
     with torch.cuda.device(device):
-        Y = torch.empty((T, B, n), dtype=act, device=device)
-        C = torch.empty((T, B, n), dtype=torch.float32, device=device)
-        H = torch.empty((T, B, 4 * n), dtype=act, device=device)
-        d = torch.empty((B, n), dtype=torch.float32, device=device)
+        Y, C, H, d = _alloc_lstm2_outputs(T, B, n, bf16, device)
         ws_bytes = int(lib.rtn_native_lstm2_fwd_workspace_bytes(T, B, n, dtype, mode))
         ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=device)
         stream = torch.cuda.current_stream(device).cuda_stream
@@ -198,6 +211,53 @@ def _native_lstm2_device_impl(X, W, y0, c0, i, start, step):
     # The workspace goes back to the caching allocator here; the allocator keeps it out of other
     # streams' hands until the work queued on this stream has passed it (stream-ordered reuse).
     return Y, C, H, d
+
+
+def native_lstm2_multi(calls, *, mode: Optional[str] = None):
+    """
+    Several independent ``NativeLstm2`` calls of one shape through one entry of the library, e.g. the forward and
+    the backward direction of a bidirectional layer.  Same results as calling the op once per element; when the
+    device can hold them together they run in a single launch and overlap.
+
+    :param calls: sequence of ``(X, W, y0, c0, i, start, step)``, all with the same T, B, n and element type
+    :param mode: as for :class:`OpMaker`; default: the mode the op was made with
+    :return: list of ``(Y, C, H, d)``
+    """
+    calls = list(calls)
+    if not calls:
+        return []
+    lib = _lib.load()
+    norm = [_normalise_lstm2_args(*c[:5]) for c in calls]
+    shape = norm[0][1]
+    device = norm[0][0][0].device
+    for tensors, sh in norm:
+        if sh != shape:
+            raise RuntimeError("native_lstm2_multi: all calls need the same T, B, n and element type; got %r and %r" % (shape, sh))
+        if tensors[0].device != device:
+            raise RuntimeError("native_lstm2_multi: all calls must be on one device")
+    if not norm[0][0][0].is_cuda:
+        raise RuntimeError("NativeLstm2: this build implements the op for HIP (MI355X) tensors only; got CPU tensors.")
+    T, B, n, bf16 = shape
+    dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
+    mode_code = _lib.MODES[mode or OpMaker.options.get("NativeLstm2", {}).get("mode", "auto")]
+    count = len(calls)
+    arr = (_lib.Lstm2Call * count)()
+    outs = []
+    with torch.cuda.device(device):
+        for k, ((X, W, y0, c0, i), c) in enumerate(zip((t for t, _ in norm), calls)):
+            Y, C, H, d = _alloc_lstm2_outputs(T, B, n, bf16, device)
+            outs.append((Y, C, H, d))
+            arr[k] = _lib.Lstm2Call(
+                X.data_ptr(), W.data_ptr(), y0.data_ptr(), c0.data_ptr(), i.data_ptr(), int(c[5]), int(c[6]),
+                Y.data_ptr(), C.data_ptr(), H.data_ptr(), d.data_ptr(),
+            )  # fmt: skip
+        ws_bytes = int(lib.rtn_native_lstm2_fwd_multi_workspace_bytes(count, T, B, n, dtype, mode_code))
+        ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=device)
+        stream = torch.cuda.current_stream(device).cuda_stream
+        rc = lib.rtn_native_lstm2_fwd_multi(arr, count, T, B, n, dtype, mode_code, ws.data_ptr(), ws.numel(), stream)
+    _lib.check(rc)
+    del norm  # the normalised inputs stay alive until here; the stream-ordered allocator covers the rest
+    return outs
 
 
 def lstm_last_output(Y: torch.Tensor, y0: torch.Tensor, i: torch.Tensor, start: int = 0, step: int = 1) -> torch.Tensor:
