@@ -922,7 +922,6 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     // One time step; PAR = s & 1 selects the register set and the LDS copies.
     auto step = [&](int s, auto par_tag) {
       constexpr int PAR = decltype(par_tag)::value;
-      RTN_TRACE_MARK(5)  // loop overhead between steps
 
       // Complete this wave's share of h_{s-1}: if anything that came back is not written yet, read again.
       unsigned long long t0 = 0;
@@ -948,9 +947,13 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
         }
         issue(s);
       }
+      RTN_TRACE_MARK(0)  // wait for h_{s-1}
       // Everything this wave stored before (re-arm stores included) is acknowledged, and X[t_s],
       // fetched two steps ago, is in its registers.
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      // (The builtin rather than inline assembly: the compiler's own wait-count bookkeeping sees it and does
+      // not make the MFMAs below wait for the loads of X[t_{s+2}] that are issued after this point.)
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      asm volatile("" ::: "memory");
       // The first read is held back by `delay` so that it usually comes back complete: a read that
       // comes back incomplete costs a whole extra round trip.  Lengthen the delay when that happened,
       // shorten it slowly while it does not.
@@ -958,10 +961,9 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
         delay = min(delay + 2, 64);
       else if ((s & 15) == 15 && delay > 0)
         --delay;
-      RTN_TRACE_MARK(0)  // wait for h_{s-1}
+      RTN_TRACE_MARK(7)  // outstanding stores acknowledged
       RTN_TRACE_ADD(6, spins)
       put(par_tag);
-      if (s + 2 < nsteps) fetch(s + 2, par_tag);
 
       f32x4 acc[MT][NT];
 #pragma unroll
@@ -979,11 +981,16 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) redbuf[wave][mt * NT + nt][lane] = acc[mt][nt];
-      RTN_TRACE_MARK(1)  // put + fetch + MFMA + partial tiles to LDS
+      // X[t_{s+2}] from memory: issued here, after the MFMAs, so that nothing on the way to the barrier waits for it.
+      if (s + 2 < nsteps) fetch(s + 2, par_tag);
+      RTN_TRACE_MARK(1)  // put + MFMA + partial tiles to LDS + fetch
       __syncthreads();  // the one barrier of a step: partial tiles, X[t_s] and the outputs of step s-1 are in LDS
       RTN_TRACE_MARK(2)  // barrier
 
+      // Gates and cell update first, then straight away the new hidden values (the step's critical path);
+      // staging of the op's outputs comes after those stores are on their way.
       unsigned h_bits[EPT];
+      float g_act[EPT][4], y_out[EPT];
 #pragma unroll
       for (int j = 0; j < EPT; ++j) {
         h_bits[j] = 0;
@@ -992,7 +999,6 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
           f32x4 gsum = redbuf[0][e][lane];
 #pragma unroll
           for (int w = 1; w < kWaves; ++w) gsum += redbuf[w][e][lane];
-          const unsigned xi = ((PAR * ROWS + e_row[j]) * 4) * CELLS + e_cl[j];  // in the staging copies
           const AT* xin = (const AT*)((const unsigned char*)Xl + PAR * kXlCopy) + (e_row[j] * 4) * CELLS + e_cl[j];
           const float m = Ml[PAR * ROWS + e_row[j]];
           const float a0 = Act<AT>::tanh(gsum[0] + (float)xin[0]);
@@ -1006,18 +1012,11 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
           c_state[j] = c;
           h_prev[j] = hn;
           h_bits[j] = SN::bits(hn);
-          // stage the op's outputs of this step
-          Hs[xi] = (AT)a0;
-          Hs[xi + CELLS] = (AT)a1;
-          Hs[xi + 2 * CELLS] = (AT)a2;
-          Hs[xi + 3 * CELLS] = (AT)a3;
-          const unsigned yi = (PAR * ROWS + e_row[j]) * CELLS + e_cl[j];
-          Ys[yi] = (AT)y;
-          Cs[yi] = c;
+          g_act[j][0] = a0; g_act[j][1] = a1; g_act[j][2] = a2; g_act[j][3] = a3;
+          y_out[j] = y;
         }
       }
-      RTN_TRACE_MARK(3)  // gates, cell update, staging
-      // New hidden values out; re-arm the elements everybody read one step ago; first read of the next step.
+      // New hidden values out; re-arm the elements everybody read one step ago.
       // (Rows the group does not have own slots of the exchange buffers too, so no lane is switched off.)
       {
         const unsigned nxt = (unsigned)((s + 1) & (kHxRing - 1)) * hx_buf_bytes;
@@ -1029,12 +1028,29 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
         for (int j = 0; j < EPT; ++j)
           if (TILES % kWaves == 0 || wave + kWaves * j < TILES) SN::template store<AUXS>(ring_rs, e_hoff[j] + arm, SN::kSentinel);
       }
+      RTN_TRACE_MARK(3)  // gates, cell update, exchange stores
+      // stage the op's outputs of this step
+#pragma unroll
+      for (int j = 0; j < EPT; ++j) {
+        if (TILES % kWaves == 0 || wave + kWaves * j < TILES) {
+          const unsigned xi = ((PAR * ROWS + e_row[j]) * 4) * CELLS + e_cl[j];  // in the staging copies
+          Hs[xi] = (AT)g_act[j][0];
+          Hs[xi + CELLS] = (AT)g_act[j][1];
+          Hs[xi + 2 * CELLS] = (AT)g_act[j][2];
+          Hs[xi + 3 * CELLS] = (AT)g_act[j][3];
+          const unsigned yi = (PAR * ROWS + e_row[j]) * CELLS + e_cl[j];
+          Ys[yi] = (AT)y_out[j];
+          Cs[yi] = c_state[j];
+        }
+      }
+      // First read of the next step.
       if (s + 1 < nsteps) {
         for (int k = 0; k < delay; ++k) __builtin_amdgcn_s_sleep(1);
         issue(s + 1);
       }
+      RTN_TRACE_MARK(4)  // staging, delay, first read of the next step
       if (s >= 1) flush(s - 1, IntTag<1 - PAR>{});
-      RTN_TRACE_MARK(4)  // exchange stores, first read of the next step, output stores
+      RTN_TRACE_MARK(5)  // output stores
     };
     fetch(0, IntTag<0>{});
     if (nsteps > 1) fetch(1, IntTag<1>{});
@@ -1043,6 +1059,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       step(s, IntTag<0>{});
       if (s + 1 < nsteps) step(s + 1, IntTag<1>{});
     }
+    RTN_TRACE_ADD(6, (unsigned long long)delay << 40)
     RTN_TRACE_FLUSH(p, bid)
   };
   if (same_xcd && p.exchange == kExNt)
