@@ -533,9 +533,10 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
 //    all outputs of step s-1).  A wavefront's re-arm stores are acknowledged (vmcnt(0) after its
 //    next successful read) before its next hidden-value stores, which precede anybody's first
 //    look at that buffer for step s+3, so a consumer can never mistake an old value for a new one.
-//  * the op's streams are decoupled from the recurrence: X[t] and the mask are fetched two steps
-//    ahead as 16-byte chunks spread over the workgroup, parked in registers and handed over
-//    through LDS; H[t], Y[t], C[t] are staged in LDS by the threads that compute them and written
+//  * the op's streams are decoupled from the recurrence: X[t] and the mask are fetched four steps
+//    ahead as 16-byte chunks spread over the workgroup, parked in registers, handed over through
+//    LDS two steps before their own and read into the registers of the thread that needs them one
+//    step before -- all of it while the workgroup waits for the exchange anyway; H[t], Y[t], C[t] are staged in LDS by the threads that compute them and written
 //    out one step later, again 16 bytes per thread.  So the waits of the recurrence never contain
 //    the HBM latency of a stream, and the streams are coalesced.  One workgroup barrier per step
 //    (after the partial tiles are in LDS) orders everything.
@@ -768,8 +769,8 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   __syncthreads();  // everybody has read it; LDS is free for the steps
 
   // ---- the op's streams: X[t], mask[t] in; H[t], Y[t], C[t] out, as 16-byte (8-byte) chunks spread
-  // over the 256 threads.  X is fetched two steps ahead into registers and copied to LDS before the
-  // barrier of its step; the outputs are staged in LDS by the threads that compute them and written
+  // over the 256 threads.  X is fetched four steps ahead into registers and copied to LDS two steps
+  // before its own (a barrier lies between that copy and its readers); the outputs are staged in LDS by the threads that compute them and written
   // out after the barrier of the following step.  Chunks of rows the group does not have carry an
   // out-of-range buffer offset: their loads return 0 and their stores are dropped, without a branch.
   AT* Xl = (AT*)(smem + L.xl);
@@ -917,6 +918,18 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
         for (int nt = 0; nt < NT; ++nt)
           bf[ks][nt] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(ring_rs, foff[ks][nt], soff, AUXL));
     };
+    // This thread's gate inputs and mask of the step to come, read from the LDS copy PAR.
+    float x_in[EPT][4], m_in[EPT];
+    auto load_gate_inputs = [&](auto par_tag) {
+      constexpr int PAR = decltype(par_tag)::value;
+#pragma unroll
+      for (int j = 0; j < EPT; ++j) {
+        const AT* xin = (const AT*)((const unsigned char*)Xl + PAR * kXlCopy) + (e_row[j] * 4) * CELLS + e_cl[j];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) x_in[j][q] = (float)xin[q * CELLS];
+        m_in[j] = Ml[PAR * ROWS + e_row[j]];
+      }
+    };
     RTN_TRACE_DECL
     int delay = p.poll_delay;  // in units of s_sleep(1), about 64 clocks; adapts, see below
     // One time step; PAR = s & 1 selects the register set and the LDS copies.
@@ -948,10 +961,9 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
         issue(s);
       }
       RTN_TRACE_MARK(0)  // wait for h_{s-1}
-      // Everything this wave stored before (re-arm stores included) is acknowledged, and X[t_s],
+      // Everything this wave stored before (re-arm stores included) is acknowledged, and X[t_{s+2}],
       // fetched two steps ago, is in its registers.
-      // (The builtin rather than inline assembly: the compiler's own wait-count bookkeeping sees it and does
-      // not make the MFMAs below wait for the loads of X[t_{s+2}] that are issued after this point.)
+      // (The builtin rather than inline assembly, so that the compiler's own wait-count bookkeeping sees it.)
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
       asm volatile("" ::: "memory");
       // The first read is held back by `delay` so that it usually comes back complete: a read that
@@ -963,7 +975,6 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
         --delay;
       RTN_TRACE_MARK(7)  // outstanding stores acknowledged
       RTN_TRACE_ADD(6, spins)
-      put(par_tag);
 
       f32x4 acc[MT][NT];
 #pragma unroll
@@ -981,10 +992,8 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) redbuf[wave][mt * NT + nt][lane] = acc[mt][nt];
-      // X[t_{s+2}] from memory: issued here, after the MFMAs, so that nothing on the way to the barrier waits for it.
-      if (s + 2 < nsteps) fetch(s + 2, par_tag);
-      RTN_TRACE_MARK(1)  // put + MFMA + partial tiles to LDS + fetch
-      __syncthreads();  // the one barrier of a step: partial tiles, X[t_s] and the outputs of step s-1 are in LDS
+      RTN_TRACE_MARK(1)  // MFMA, partial tiles to LDS
+      __syncthreads();  // the one barrier of a step: partial tiles, X[t_{s+1}] and the outputs of step s-1 are in LDS
       RTN_TRACE_MARK(2)  // barrier
 
       // Gates and cell update first, then straight away the new hidden values (the step's critical path);
@@ -999,12 +1008,11 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
           f32x4 gsum = redbuf[0][e][lane];
 #pragma unroll
           for (int w = 1; w < kWaves; ++w) gsum += redbuf[w][e][lane];
-          const AT* xin = (const AT*)((const unsigned char*)Xl + PAR * kXlCopy) + (e_row[j] * 4) * CELLS + e_cl[j];
-          const float m = Ml[PAR * ROWS + e_row[j]];
-          const float a0 = Act<AT>::tanh(gsum[0] + (float)xin[0]);
-          const float a1 = Act<AT>::sigmoid(gsum[1] + (float)xin[CELLS]);
-          const float a2 = Act<AT>::sigmoid(gsum[2] + (float)xin[2 * CELLS]);
-          const float a3 = Act<AT>::sigmoid(gsum[3] + (float)xin[3 * CELLS]);
+          const float m = m_in[j];
+          const float a0 = Act<AT>::tanh(gsum[0] + x_in[j][0]);
+          const float a1 = Act<AT>::sigmoid(gsum[1] + x_in[j][1]);
+          const float a2 = Act<AT>::sigmoid(gsum[2] + x_in[j][2]);
+          const float a3 = Act<AT>::sigmoid(gsum[3] + x_in[j][3]);
           const float pc = c_state[j];
           const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
           const float y = E::round(Act<AT>::tanh(c) * a3 * m);
@@ -1043,17 +1051,29 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
           Cs[yi] = c_state[j];
         }
       }
-      // First read of the next step.
+      // While the new hidden values travel: X[t_{s+2}] from registers to LDS, X[t_{s+4}] from memory into the
+      // registers that have just become free; after the delay the first read of the next step; and behind that
+      // read, in its shadow, this thread's gate inputs of the next step from LDS to registers (X[t_{s+1}] got
+      // there one step ago) and the outputs of the previous step from LDS to memory.
+      if (s + 2 < nsteps) put(par_tag);
+      if (s + 4 < nsteps) fetch(s + 4, par_tag);
       if (s + 1 < nsteps) {
         for (int k = 0; k < delay; ++k) __builtin_amdgcn_s_sleep(1);
         issue(s + 1);
       }
-      RTN_TRACE_MARK(4)  // staging, delay, first read of the next step
+      RTN_TRACE_MARK(4)  // staging, put, fetch, delay, first read of the next step
+      if (s + 1 < nsteps) load_gate_inputs(IntTag<1 - PAR>{});
       if (s >= 1) flush(s - 1, IntTag<1 - PAR>{});
-      RTN_TRACE_MARK(5)  // output stores
+      RTN_TRACE_MARK(5)  // gate inputs, output stores
     };
     fetch(0, IntTag<0>{});
     if (nsteps > 1) fetch(1, IntTag<1>{});
+    put(IntTag<0>{});
+    if (nsteps > 1) put(IntTag<1>{});
+    __syncthreads();
+    load_gate_inputs(IntTag<0>{});
+    if (nsteps > 2) fetch(2, IntTag<0>{});
+    if (nsteps > 3) fetch(3, IntTag<1>{});
     issue(0);
     for (int s = 0; s < nsteps; s += 2) {
       step(s, IntTag<0>{});
