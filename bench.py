@@ -46,6 +46,27 @@ def algorithmic_bytes_per_unit(n: int, dtype: str) -> int:
     return e * 4 * n + e * 4 * n + e * n + 4 * n + 4
 
 
+def achievable_fields(probe_us, rows, n, dtype, T, call_ms):
+    """
+    The dependency-bound ceiling of the recurrent GEMM: the T steps are sequential, and a step cannot be shorter than
+    one hand-over of the hidden state between the CUs that hold W (``probe_us``: measured with the library's latency
+    probe -- device-scope store, visible on every CU, device-scope load, at a tiny volume) plus the time the whole
+    chip's matrix cores need for the step's GEMM at their peak (``8 n^2`` flops for each of the ``rows`` sequences of
+    a launch).  ``achievable`` is the GEMM rate at that ceiling, ``frac_of_achievable`` = ceiling time / measured time.
+    """
+    if probe_us is None:
+        return {}
+    step_flops = 8.0 * n * n * rows
+    mfma_us = step_flops / PEAK_MFMA[dtype] * 1e6
+    ceiling_ms = (probe_us + mfma_us) * T * 1e-3
+    return {
+        "handover_latency_us": probe_us,
+        "mfma_peak_us_per_step": mfma_us,
+        "achievable": step_flops * T / (ceiling_ms * 1e-3) / 1e12,
+        "frac_of_achievable": ceiling_ms / call_ms,
+    }
+
+
 def cpu_baseline(name: str, target_seconds: float = 15.0):
     """Times the CPU restatement (test infrastructure, used here only as the reported baseline)."""
     import numpy
@@ -294,6 +315,26 @@ def main():
     assert measuring_only or all(bool(torch.isfinite(o["d"]).all()) for o in outs)
 
     call_ms = sum(a.elapsed_time(b) for a, b in events) / len(events)
+
+    # The latency of one hand-over of values between CUs (device-scope store -> load), measured live with the library's
+    # probe: a lower bound of a time step of any kernel that keeps W spread over CUs.
+    probe_us = None
+    probe_rounds = 4000
+    probe_ws = torch.empty((32768,), dtype=torch.uint8, device=dev)
+    pe = []
+    for _ in range(1 + 3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        rc = cabi.rtn_handover_latency_probe(probe_ws.data_ptr(), probe_ws.numel(), probe_rounds, stream.cuda_stream)
+        e1.record(stream)
+        if rc != lib.RTN_OK:
+            pe = []
+            break
+        pe.append((e0, e1))
+    torch.cuda.synchronize()
+    if pe and cabi.rtn_native_lstm2_fwd_status(probe_ws.data_ptr(), stream.cuda_stream) == lib.RTN_OK:
+        probe_us = min(a.elapsed_time(b) for a, b in pe[1:]) * 1e3 / probe_rounds
+
     units_per_step = len(directions) * T * B
     value = units_per_step * args.steps / elapsed
     units_per_launch = units_per_step // launches
@@ -341,6 +382,7 @@ def main():
             % ("k_lstm2_regw" if "mfma_regw" in plan else ("k_lstm2_mfma" if "mfma_lds" in plan else "k_step_generic"),
                len(directions) // launches, units_per_launch),
             "launch_ms": call_ms,
+            **achievable_fields(probe_us, units_per_launch // T, n, dtype, T, call_ms),
             "hbm_algorithmic_GBps": bytes_per_launch / (call_ms * 1e-3) / 1e9,
             "hbm_frac": bytes_per_launch / (call_ms * 1e-3) / PEAK_HBM,
         },

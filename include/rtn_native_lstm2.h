@@ -133,6 +133,17 @@ int rtn_native_lstm2_fwd_multi_status(const void* workspace, int32_t count, int6
                                       int32_t dtype, int32_t mode, void* hip_stream);
 
 /*
+ * Measurement aid, not part of the operator: the latency of handing a value from every workgroup to every other
+ * one the way the persistent kernel hands over the hidden state (device-scope store, device-scope load until the
+ * value has arrived, one workgroup barrier), with 16 workgroups on 16 CUs, 256 bytes each and nothing else going on.
+ * Enqueues `rounds` such hand-overs; the caller times the call (events on `hip_stream`) and divides by `rounds`.
+ * That time is a lower bound of one time step of any kernel that keeps W spread over several CUs.  `workspace`:
+ * at least 16 640 bytes; rtn_native_lstm2_fwd_status(workspace, stream) afterwards tells whether a wait expired.
+ * No counterpart in the reference.
+ */
+int rtn_handover_latency_probe(void* workspace, size_t workspace_bytes, int32_t rounds, void* hip_stream);
+
+/*
  * Final output per sequence.  Replaces the caller-side `_lstm_last_output`
  * (returnn/tf/native_op.py:913-929): out[b] = Y[t*, b] for the last visited frame t*
  * (in processing order) with i[t*, b] != 0, else y0[b].  Y, y0, out have element

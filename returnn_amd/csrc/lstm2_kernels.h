@@ -185,6 +185,12 @@ __global__ void k_prepare_mfma(Lstm2Params p, int n_flags) {
 }
 
 // Clears the status word for the generic path.
+__global__ void k_fill_u32(unsigned* dst, unsigned value, long long count) {
+  for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < count;
+       i += (long long)gridDim.x * blockDim.x)
+    dst[i] = value;
+}
+
 __global__ void k_clear_status(unsigned* status) {
   if (threadIdx.x < 64) status[threadIdx.x] = 0;
 }
@@ -541,14 +547,10 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
 //    the HBM latency of a stream, and the streams are coalesced.  One workgroup barrier per step
 //    (after the partial tiles are in LDS) orders everything.
 //  * exchange scope: the memory side of the device (sc1 loads and stores), which is valid
-//    wherever the workgroups of a group run.  Every workgroup records the XCD it runs on and
-//    the group's table is read back at start (it doubles as the check that the whole group is
-//    resident); `exchange` may select an experimental same-XCD policy when the table is uniform.
+//    wherever the workgroups of a group run.
 // Waits are bounded as in k_lstm2_mfma.
 // ---------------------------------------------------------------------------------------------
 constexpr int kExDevice = 0;  // device-scope loads and stores: always valid
-constexpr int kExNt = 1;      // experimental, same-XCD groups only: plain stores, non-temporal loads
-constexpr int kExNtSc0 = 2;   // experimental, same-XCD groups only: plain stores, workgroup-scope non-temporal loads
 constexpr int kExNoWait = 3;  // measurement aid: never wait for the other workgroups (results are WRONG; status is set to 2)
 
 template <typename AT>
@@ -613,21 +615,6 @@ __host__ __device__ constexpr RegwLds regw_lds(int es, int MT, int NT) {
   l.ml = off; off += 2u * rows * 4u;
   l.total = off;
   return l;
-}
-
-// blockIdx -> (group, rank) for the register kernel.  With map_compact the grid is
-// xcds * ceil(groups / xcds) * wgs_per_group workgroups; under round-robin dealing of workgroup
-// ids to XCDs, XCD x then holds the whole groups x, x + xcds, ...; surplus workgroups (when
-// groups is not a multiple of xcds) get g = -1 and leave at once.
-__device__ __forceinline__ void map_block_regw(const Lstm2Params& p, int bid, int& g, int& r) {
-  if (p.map_compact) {
-    const int x = bid % p.xcds, q = bid / p.xcds;
-    g = (q / p.wgs_per_group) * p.xcds + x;
-    r = q % p.wgs_per_group;
-    if (g >= p.groups) g = -1;
-  } else {
-    map_block(p, bid, g, r);
-  }
 }
 
 // 16-byte (or 8-byte) chunk moves of the stream wavefront.
@@ -713,60 +700,17 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   extern __shared__ __align__(16) unsigned char smem[];
   typedef f32x4 RedBuf[kWaves][TILES][64];
   RedBuf* red = (RedBuf*)(smem + L.red);  // [2]
-  int* s_same_xcd = (int*)(smem + L.ml);  // borrowed before the first step
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in a scalar register
   const int n = p.n, S = n / KM;
   int g, r;
-  map_block_regw(p, bid, g, r);
-  if (g < 0) return;
+  map_block(p, bid, g, r);
   const int G = p.wgs_per_group;
   const int b_base = g * p.Bg;
   const int rows = min(p.Bg, p.B - b_base);
   const long long bn = (long long)p.B * n;
   const int nsteps = p.nsteps;
-
-  // Where does the group run?  Publish this workgroup's XCD id (+1) and read the group's table.
-  {
-    unsigned* ids = p.flags + (size_t)g * G;
-    if (tid == 0) {
-      const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 0xFu;  // XCC_ID, bits [3:0]
-      __hip_atomic_store(ids + r, xcc + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    if (wave == 0) {
-      unsigned long long t0 = 0;
-      unsigned spins = 0;
-      bool same = true;
-      for (;;) {
-        bool all_there = true;
-        same = true;
-        const unsigned mine = __hip_atomic_load(ids + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        for (int k = lane; k < G; k += 64) {
-          const unsigned v = __hip_atomic_load(ids + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          all_there = all_there && (v != 0);
-          same = same && (v == mine);
-        }
-        if (__all(all_there && mine != 0)) break;
-        if ((spins++ & 15u) == 0) {
-          if (__hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
-          const unsigned long long now = wall_clock64();
-          if (spins == 1) {
-            t0 = now;
-          } else if (now - t0 > p.timeout_ticks) {
-            __hip_atomic_store(p.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            break;
-          }
-        }
-        __builtin_amdgcn_s_sleep(2);
-      }
-      const int same_all = __all(same) ? 1 : 0;
-      if (lane == 0) *s_same_xcd = same_all;
-    }
-  }
-  __syncthreads();
-  const bool same_xcd = *s_same_xcd != 0;
-  __syncthreads();  // everybody has read it; LDS is free for the steps
 
   // ---- the op's streams: X[t], mask[t] in; H[t], Y[t], C[t] out, as 16-byte (8-byte) chunks spread
   // over the 256 threads.  X is fetched four steps ahead into registers and copied to LDS two steps
@@ -905,8 +849,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
 
   auto run = [&](auto ex_tag) {
     constexpr int EX = decltype(ex_tag)::value;
-    constexpr int AUXS = (EX == kExDevice || EX == kExNoWait) ? kAuxDevice : 0;                        // stores
-    constexpr int AUXL = (EX == kExDevice || EX == kExNoWait) ? kAuxDevice : (EX == kExNt ? 2 : 3);    // loads
+    constexpr int AUXS = kAuxDevice, AUXL = kAuxDevice;  // exchange stores and loads: device scope
     i32x4 bf[KSMAX][NT];
     // Issue the loads of this wave's fragments of ring buffer s%4.
     auto issue = [&](int s) {
@@ -976,6 +919,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       RTN_TRACE_MARK(7)  // outstanding stores acknowledged
       RTN_TRACE_ADD(6, spins)
 
+      RedBuf& redbuf = red[PAR];
       f32x4 acc[MT][NT];
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
@@ -987,7 +931,6 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
-      RedBuf& redbuf = red[PAR];
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -1082,15 +1025,12 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     RTN_TRACE_ADD(6, (unsigned long long)delay << 40)
     RTN_TRACE_FLUSH(p, bid)
   };
-  if (same_xcd && p.exchange == kExNt)
-    run(IntTag<kExNt>{});
-  else if (same_xcd && p.exchange == kExNtSc0)
-    run(IntTag<kExNtSc0>{});
-  else if (p.exchange == kExNoWait) {
+  if (p.exchange == kExNoWait) {
     if (tid == 0) __hip_atomic_store(p.status, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     run(IntTag<kExNoWait>{});
-  } else
+  } else {
     run(IntTag<kExDevice>{});
+  }
   __syncthreads();  // the last step's outputs are staged
   if ((nsteps - 1) & 1)
     flush(nsteps - 1, IntTag<1>{});
@@ -1100,6 +1040,47 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
 #pragma unroll
   for (int j = 0; j < EPT; ++j)
     if (e_valid[j]) p.d[(long long)(b_base + e_row[j]) * n + 4 * MT * r + e_cl[j]] = c_state[j];
+}
+
+
+// Measurement aid: the latency of handing a value from every workgroup to every other one, the way the persistent
+// kernel hands over the hidden state (device-scope store, device-scope load until the value is there), with nothing
+// else going on: G workgroups on G CUs; per round each stores its 256-byte block of ring buffer round%4 (value =
+// round number) and reads all G blocks, 16 lanes per block, until every word carries the round number; one
+// workgroup barrier per round.  A value from an earlier use of the buffer differs from the round number, so a
+// stale read can only cost a retry.  G <= 16.  status[0] is set to 1 if a wait runs into `timeout_ticks`.
+__global__ __launch_bounds__(kWgThreads) void k_handover_latency(unsigned* ring, unsigned* status, int G, int rounds,
+                                                                 unsigned long long timeout_ticks) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = blockIdx.x;
+  const unsigned buf_bytes = (unsigned)G * 256u;
+  __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)ring, 0, 4 * buf_bytes, kBufFlags);
+  const int blk = wave * 4 + (lane >> 4);  // the block this lane reads a 16-byte piece of
+  const unsigned roff = blk < G ? (unsigned)blk * 256u + (unsigned)(lane & 15) * 16u : kOobOffset;
+  for (int s = 1; s <= rounds; ++s) {
+    const unsigned base = (unsigned)(s & 3) * buf_bytes;
+    const unsigned v = (unsigned)s;
+    if (tid < 64) __builtin_amdgcn_raw_buffer_store_b32(v, rs, base + (unsigned)r * 256u + (unsigned)tid * 4u, 0, kAuxDevice);
+    unsigned long long t0 = 0;
+    unsigned spins = 0;
+    for (;;) {
+      asm volatile("" ::: "memory");
+      const i32x4 x = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, roff, base, kAuxDevice));
+      const bool ok = blk >= G || ((unsigned)x[0] == v && (unsigned)x[1] == v && (unsigned)x[2] == v && (unsigned)x[3] == v);
+      if (__all(ok)) break;
+      if ((spins++ & 15u) == 0) {
+        if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+        const unsigned long long now = wall_clock64();
+        if (spins == 1) {
+          t0 = now;
+        } else if (now - t0 > timeout_ticks) {
+          __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+      }
+    }
+    __syncthreads();
+  }
 }
 
 }  // namespace rtn

@@ -46,8 +46,7 @@ struct Lstm2Params {
   int hx_bufs;        // buffers in the hx ring: 2 with the flag barrier, 4 with self-validating data
   int hx_sentinel;    // 1: buffers 1.. start filled with the "not yet written" bit pattern (all ones)
   int xcds;           // XCDs assumed for the blockIdx -> (group, rank) mapping
-  int map_compact;    // register kernel: whole groups per XCD (see map_block_regw)
-  int exchange;       // register kernel: exchange policy for groups found on one XCD (0: device scope, always valid)
+  int exchange;       // register kernel: 0 = normal operation; 3, 4 = measurement aids (see kExNoWait, kExProbe)
   int poll_delay;     // register kernel: s_sleep(1) repeats between the hidden-value stores and the first read of the next step
   unsigned long long* trace;  // optional [workgroups][8] cycle totals per phase (instrumented builds only)
   int zero;           // always 0; an operand the compiler cannot fold (idempotent atomics used as L2 reads)

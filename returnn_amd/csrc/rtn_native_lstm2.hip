@@ -95,7 +95,6 @@ struct Plan {
   PlanKind kind = kPlanGeneric;
   int mode = RTN_MODE_STEPWISE;  // resolved: PERSISTENT, GRAPH or STEPWISE
   bool regw = false;             // persistent kernel with W in registers and self-validating exchange
-  bool compact = false;          // its groups are laid out one XCD each (see map_block_regw)
   int grid = 0;                  // workgroups launched by the persistent kernel
   int KSMAX = 0;                 // its macro steps per wavefront (template bound)
   int MT = 1, NT = 1;
@@ -121,10 +120,8 @@ size_t mfma_lds_bytes(int n, int dtype, int MT, int NT) {
 bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing, Plan* out, std::string* why,
                int max_wgs_per_cu = 2, int count = 1) {
   Plan pl;
-  // Two workgroups per CU and whole groups per XCD only pay off with the (experimental) same-XCD exchange.
-  const long env_exchange = env_long("RTN_LSTM2_EXCHANGE", 0);
-  const bool xcd_local = env_exchange == 1 || env_exchange == 2;
-  max_wgs_per_cu = (int)std::max<long>(1, std::min<long>(max_wgs_per_cu, env_long("RTN_LSTM2_WGS_PER_CU", xcd_local ? 2 : 1)));
+  // One problem on its own is planned with a CU per workgroup (sharing CUs did not pay off in measurements).
+  max_wgs_per_cu = (int)std::max<long>(1, std::min<long>(max_wgs_per_cu, env_long("RTN_LSTM2_WGS_PER_CU", 1)));
   const DeviceInfo di = device_info();
   const size_t es = esize(dtype);
   if (T == 0 || B == 0 || n == 0) {
@@ -177,17 +174,13 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
             int pc = per_cu;  // workgroups per CU that LDS allows as well
             while (pc > 1 && lds * pc > di.lds_per_wg) --pc;
             if ((long long)groups * G > (long long)di.cus * pc) continue;
-            // Whole groups per XCD when they fit: the exchange then stays inside one L2.
-            const int cus_per_xcd = di.cus / di.xcds;
-            const bool compact = use_regw && di.xcds > 1 && xcd_local && !env_long("RTN_LSTM2_NO_COMPACT", 0) &&
-                                 (long long)G * ((groups + di.xcds - 1) / di.xcds) <= (long long)cus_per_xcd * pc;
             // Step time model fitted to MI355X measurements (microseconds): MFMA issue time of one
             // wavefront, a second round of gate arithmetic when a thread owns two pairs, the number of
             // workgroups that exchange with each other, the fragments a wavefront reads per step and
             // the fragments it holds.
             const double mfma_us = (double)MT * NT * ks * (dtype == RTN_DTYPE_BF16 ? 16 : 128) / 2400.0;
             const int ept = (MT * NT + kWaves - 1) / kWaves;
-            double est = 2.0 * mfma_us + 0.4 * (ept - 1) + (compact ? 0.0 : 0.004 * G) + 0.03 * ks * NT + 0.01 * MT * ks;
+            double est = 2.0 * mfma_us + 0.4 * (ept - 1) + 0.004 * G + 0.03 * ks * NT + 0.01 * MT * ks;
             // Several problems in one launch: as long as every workgroup has a CU to itself they do not slow
             // each other down; sharing CUs costs about a third, running in turns costs the whole time again.
             if (count > 1) {
@@ -203,8 +196,7 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
             if (est < best) {
               best = est;
               pl.regw = use_regw != 0;
-              pl.compact = compact;
-              pl.grid = compact ? di.xcds * ((groups + di.xcds - 1) / di.xcds) * G : groups * G;
+              pl.grid = groups * G;
               pl.KSMAX = use_regw ? KSMAX : 0;
               pl.MT = MT;
               pl.NT = NT;
@@ -231,7 +223,6 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
       // Per-step launches have no co-residency limit: 4 cells per workgroup, groups of <= 64 rows.
       int MT = 1;
       pl.regw = false;
-      pl.compact = false;
       pl.KSMAX = 0;
       if (mfma_lds_bytes(n, dtype, 1, 4) > di.lds_per_wg) {
         pl.kind = kPlanGeneric;  // a W slice of 16 columns does not fit LDS (n far beyond the target sizes)
@@ -578,12 +569,11 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     p.groups = pl.groups; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
     p.hx_bufs = kHxRing;
     p.hx_sentinel = pl.regw ? 1 : 0;
-    p.map_compact = pl.compact ? 1 : 0;
     p.exchange = (int)env_long("RTN_LSTM2_EXCHANGE", 0);
-    if (p.exchange < 0 || p.exchange > 3) p.exchange = 0;  // 3: measurement aid, results invalid (status 2)
+    if (p.exchange != kExNoWait) p.exchange = kExDevice;  // no-wait: a timing aid, results invalid (status 2)
     // Device-scope stores take about a microsecond to become visible: a first read issued at once would
     // come back incomplete and cost a second round trip, so it is held back (tuned on MI355X).
-    p.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", p.exchange == 0 ? 20 : 8)));
+    p.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", 20)));
     p.xcds = device_info().xcds;
     p.sync_policy = (int)env_long("RTN_LSTM2_SYNC", kStoreCoherent | kLoadCoherent);
     if (!((p.sync_policy & (kStoreCoherent | kReleaseFence)) && (p.sync_policy & (kLoadCoherent | kAcquireFence))))
@@ -672,11 +662,11 @@ const char* rtn_native_lstm2_describe_multi_plan(int32_t count, int64_t T, int32
   } else if (!make_plan(T, B, n, dtype, mode, false, &pl, &why, 2, c)) {
     g_plan_text = "unsupported: " + why;
   } else {
-    snprintf(buf, sizeof(buf), "mode=%s kernel=%s mt=%d nt=%d groups=%d wgs_per_group=%d wgs=%d rows_per_group=%d group_per_xcd=%d lds=%zu workspace=%zu",
+    snprintf(buf, sizeof(buf), "mode=%s kernel=%s mt=%d nt=%d groups=%d wgs_per_group=%d wgs=%d rows_per_group=%d lds=%zu workspace=%zu",
              mode_name(pl.mode),
              pl.kind == kPlanMfma ? (pl.regw ? "mfma_regw" : "mfma_lds") : (pl.kind == kPlanGeneric ? "generic" : "empty"), pl.MT,
              pl.NT, pl.groups, pl.wgs_per_group, (pl.mode == RTN_MODE_PERSISTENT && pl.regw) ? pl.grid : pl.groups * pl.wgs_per_group,
-             pl.Bg, pl.compact ? 1 : 0, pl.lds_bytes, count > 1 ? workspace_each(count, T, B, n, dtype, mode) : pl.total);
+             pl.Bg, pl.lds_bytes, count > 1 ? workspace_each(count, T, B, n, dtype, mode) : pl.total);
     if (pl.off_trace) snprintf(buf + strlen(buf), sizeof(buf) - strlen(buf), " trace_offset=%zu", pl.off_trace);
     g_plan_text = buf;
   }
@@ -701,6 +691,27 @@ int rtn_native_lstm2_fwd_multi(const rtn_lstm2_call* calls, int32_t count, int64
   if (count < 0 || (count > 0 && !calls)) return fail(RTN_ERR_ARG, "NativeLstm2: bad call list (count=%d)", count);
   if (count == 0) return RTN_OK;
   return fwd_calls(calls, count, T, B, n, dtype, mode, workspace, workspace_bytes, hip_stream);
+}
+
+int rtn_handover_latency_probe(void* workspace, size_t workspace_bytes, int32_t rounds, void* hip_stream) {
+  g_last_error.clear();
+  constexpr int G = 16;
+  const size_t need = 256 + (size_t)4 * G * 256;
+  if (!workspace || workspace_bytes < need) return fail(RTN_ERR_WORKSPACE, "handover probe: workspace of %zu bytes needed", need);
+  if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "handover probe: workspace must be 16-byte aligned");
+  if (rounds < 1 || rounds > (1 << 24)) return fail(RTN_ERR_ARG, "handover probe: rounds must be in [1, 2^24]");
+  if (!device_info().cooperative || device_info().cus < G) return fail(RTN_ERR_UNSUPPORTED, "handover probe: needs cooperative launch and %d CUs", G);
+  hipStream_t stream = (hipStream_t)hip_stream;
+  unsigned* status = (unsigned*)workspace;
+  unsigned* ring = (unsigned*)((unsigned char*)workspace + 256);
+  const long long words = (long long)(need / 4);
+  hipLaunchKernelGGL(k_fill_u32, dim3(8), dim3(256), 0, stream, (unsigned*)workspace, 0u, words);
+  RTN_HIP(hipGetLastError());
+  int g = G, rnd = rounds;
+  unsigned long long ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);
+  void* args[] = {(void*)&ring, (void*)&status, (void*)&g, (void*)&rnd, (void*)&ticks};
+  RTN_HIP(hipLaunchCooperativeKernel((const void*)k_handover_latency, dim3(G), dim3(kWgThreads), args, 0, stream));
+  return RTN_OK;
 }
 
 size_t rtn_native_lstm2_fwd_multi_workspace_bytes(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
@@ -728,6 +739,8 @@ int rtn_native_lstm2_fwd_status(const void* workspace, void* hip_stream) {
   hipStream_t stream = (hipStream_t)hip_stream;
   RTN_HIP(hipMemcpyAsync(&status, workspace, sizeof(status), hipMemcpyDeviceToHost, stream));
   RTN_HIP(hipStreamSynchronize(stream));
+  if (status == 2)
+    return fail(RTN_ERR_ABORTED, "NativeLstm2: the last run on this workspace was a measurement aid (exchange probe or no-wait timing); it computes no outputs");
   if (status != 0) return fail(RTN_ERR_ABORTED, "NativeLstm2: a bounded wait in the persistent kernel expired; outputs are invalid");
   return RTN_OK;
 }

@@ -40,6 +40,7 @@ SYMBOLS = (
     "rtn_native_lstm2_fwd_multi",
     "rtn_native_lstm2_fwd_multi_workspace_bytes",
     "rtn_native_lstm2_fwd_multi_status",
+    "rtn_handover_latency_probe",
     "rtn_native_lstm2_last_output",
     "rtn_last_error",
     "rtn_native_lstm2_describe_plan",
@@ -101,6 +102,8 @@ def load() -> ctypes.CDLL:
         lib.rtn_native_lstm2_fwd_multi_workspace_bytes.argtypes = [i32, i64, i32, i32, i32, i32]
         lib.rtn_native_lstm2_fwd_multi_status.restype = ctypes.c_int
         lib.rtn_native_lstm2_fwd_multi_status.argtypes = [vp, i32, i64, i32, i32, i32, i32, vp]
+        lib.rtn_handover_latency_probe.restype = ctypes.c_int
+        lib.rtn_handover_latency_probe.argtypes = [vp, sz, i32, vp]
         lib.rtn_native_lstm2_last_output.restype = ctypes.c_int
         lib.rtn_native_lstm2_last_output.argtypes = [vp, vp, vp, i32, i32, vp, i64, i32, i32, i32, vp]
         lib.rtn_last_error.restype = ctypes.c_char_p

@@ -16,8 +16,10 @@ import pytest
 from numpy.testing import assert_allclose
 
 from oracle import lstm2_oracle as oracle
-from returnn_amd import synthetic
-from _gpu_util import announce, env, random_problem, run_op, run_raw
+import torch
+
+from returnn_amd import lib, synthetic
+from _gpu_util import announce, env, get_op, random_problem, run_op, run_raw, to_dev
 from _textbook import REFERENCE_START_STEP, reference_fixture, textbook_lstm, visited_slice
 
 pytestmark = pytest.mark.gpu
@@ -124,21 +126,30 @@ def test_decompositions(mt, groups, kernel):
             assert numpy.array_equal(a, b)
 
 
-@pytest.mark.parametrize("dtype", ["f32", "bf16"])
-@pytest.mark.parametrize("B,n", [(40, 512), (4, 1024), (9, 128)])
-def test_exchange_scopes(dtype, B, n):
-    """Register kernel: the hidden-state exchange through one XCD's L2 (groups placed whole on an XCD), the same
-    placement forced to device scope, and groups spread over XCDs all give the per-step result bit for bit."""
-    announce("exchange scopes", dtype, B, n)
-    p = random_problem(81, 64, B, n)
-    for step in (1, -1):
-        ref = run_op(*p, 0, step, dtype=dtype, mode="stepwise")
-        for settings in (dict(RTN_LSTM2_L2X=1), dict(RTN_LSTM2_L2X=0), dict(RTN_LSTM2_NO_COMPACT=1)):
-            with env(RTN_LSTM2_KERNEL=2, **settings):
-                rc, status, got = run_raw(*p, 0, step, dtype=dtype, mode="persistent")
-            assert rc == 0 and status == 0, settings
-            for a, b in zip(got, ref[:4]):
-                assert numpy.array_equal(a, b), settings
+def test_handover_latency_probe():
+    """The latency probe (a measurement aid of the library) runs to completion within its bounded waits, refuses bad
+    arguments, and the op is still right afterwards."""
+    announce("handover latency probe")
+    get_op()
+    cabi = lib.load()
+    ws = torch.empty((32768,), dtype=torch.uint8, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    lib.check(cabi.rtn_handover_latency_probe(ws.data_ptr(), ws.numel(), 500, stream))
+    e1.record()
+    lib.check(cabi.rtn_native_lstm2_fwd_status(ws.data_ptr(), stream))
+    us = e0.elapsed_time(e1) * 1e3 / 500
+    print("hand-over latency %.3f us" % us)
+    assert 0.05 < us < 50.0
+    assert cabi.rtn_handover_latency_probe(ws.data_ptr(), 100, 500, stream) == lib.RTN_ERR_WORKSPACE
+    assert cabi.rtn_handover_latency_probe(ws.data_ptr(), ws.numel(), 0, stream) == lib.RTN_ERR_ARG
+    X, W, y0, c0, i = random_problem(5, 20, 20, 256)
+    ref = run_op(X, W, y0, c0, i, 0, 1, dtype="bf16", mode="stepwise")
+    rc, status, got = run_raw(X, W, y0, c0, i, 0, 1, dtype="bf16", mode="persistent")
+    assert rc == 0 and status == 0
+    for a, b in zip(got, ref[:4]):
+        assert numpy.array_equal(a, b)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
