@@ -46,6 +46,9 @@ def _load():
             last = getattr(lib, "lstm2_oracle_last_output_" + suffix)
             last.restype = ctypes.c_int
             last.argtypes = [ptr] * 3 + [ctypes.c_int32, ctypes.c_int32, ptr, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
+            bwd = getattr(lib, "lstm2_oracle_bwd_" + suffix)
+            bwd.restype = ctypes.c_int
+            bwd.argtypes = [ptr] * 5 + [ctypes.c_int32, ctypes.c_int32] + [ptr] * 9 + [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
         lib.lstm2_oracle_max_threads.restype = ctypes.c_int
         fp = ctypes.POINTER(ctypes.c_float)
         lib.lstm2_oracle_pointwise_f32.restype = None
@@ -191,3 +194,50 @@ def native_lstm2_fwd_blas(X, W, y0, c0, i, start: int = 0, step: int = 1):
         t += step
     d[...] = C[t - step]
     return Y, C, H, d, y_prev
+
+
+def native_lstm2_bwd(X, W, y0, c0, i, start, step, Y, C, H, DY, Dd, *, dtype=numpy.float32):
+    """
+    Reference semantics of the ``NativeLstm2`` gradient op (returnn/native_op.py:1288-1464, inputs as
+    ``grad_input_map`` :1071-1077 arranges them).
+
+    :param X, W, y0, c0, i, start, step: the forward op's inputs
+    :param Y, C, H: the forward op's outputs (H = activated gates)
+    :param DY: [T,B,n] error signal on Y
+    :param Dd: [B,n] error signal on the final cell state
+    :return: DX [T,B,4n], DW [n,4n], Dy0 [B,n], Dc0 [B,n]
+    """
+    dtype = numpy.dtype(dtype)
+    if dtype == numpy.float32:
+        suffix, ctype = "f32", ctypes.c_float
+    elif dtype == numpy.float64:
+        suffix, ctype = "f64", ctypes.c_double
+    else:
+        raise ValueError("oracle: dtype must be float32 or float64")
+    i = numpy.ascontiguousarray(i, dtype=dtype)
+    y0 = numpy.ascontiguousarray(y0, dtype=dtype)
+    T, B = i.shape
+    n = y0.shape[1]
+    X = _prep(X, dtype, (T, B, 4 * n), "X")
+    W = _prep(W, dtype, (n, 4 * n), "W")
+    c0 = _prep(c0, dtype, (B, n), "c0")
+    Y = _prep(Y, dtype, (T, B, n), "Y")
+    C = _prep(C, dtype, (T, B, n), "C")
+    H = _prep(H, dtype, (T, B, 4 * n), "H")
+    DY = _prep(DY, dtype, (T, B, n), "DY")
+    Dd = _prep(Dd, dtype, (B, n), "Dd")
+    DX = numpy.zeros((T, B, 4 * n), dtype=dtype)
+    DW = numpy.empty((n, 4 * n), dtype=dtype)
+    Dy0 = numpy.empty((B, n), dtype=dtype)
+    Dc0 = numpy.empty((B, n), dtype=dtype)
+    p = ctypes.POINTER(ctype)
+    bwd = getattr(_load(), "lstm2_oracle_bwd_" + suffix)
+    rc = bwd(
+        *(a.ctypes.data_as(p) for a in (X, W, y0, c0, i)), int(start), int(step),
+        *(a.ctypes.data_as(p) for a in (Y, C, H, DY, Dd, DX, DW, Dy0, Dc0)), T, B, n,
+    )  # fmt: skip
+    if rc == 2:
+        raise ValueError("oracle: need 0 <= start < T and step != 0 (start=%r, step=%r, T=%r)" % (start, step, T))
+    if rc != 0:
+        raise RuntimeError("oracle: error code %i" % rc)
+    return DX, DW, Dy0, Dc0
