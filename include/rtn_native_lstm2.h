@@ -144,6 +144,31 @@ int rtn_native_lstm2_fwd_multi_status(const void* workspace, int32_t count, int6
 int rtn_handover_latency_probe(void* workspace, size_t workspace_bytes, int32_t rounds, void* hip_stream);
 
 /*
+ * NativeLstm2 gradient.  Replaces the generated body `c_bw_code` (returnn/native_op.py:1288-1464) with
+ * `lstm_bwd_kernel` (:1123-1180) and its `affine_raw` GEMMs; the arguments are the ones `grad_input_map`
+ * (:1071-1077) hands to the gradient op, minus X, which the computation never reads.
+ *
+ *   W y0 c0 i start step   the forward call's inputs
+ *   Y C H                  the forward call's outputs (H = activated gates)
+ *   DY [T,B,n]             error signal on Y (values on masked frames are ignored)
+ *   Dd [B,n]               error signal on the final cell state d (float32)
+ *   DX  [T,B,4n]           out: gradient of X (0 on masked and on unvisited frames)
+ *   DW  [n,4n]             out: gradient of W, always float32
+ *   Dy0 [B,n]              out: gradient of y0        Dc0 [B,n]  out: gradient of c0 (float32)
+ *
+ * Element type `dtype` for W y0 Y H DY DX Dy0; c0 C i Dd Dc0 DW are float32.  This first implementation runs one
+ * pointwise launch and one MFMA launch (Dy0 += DX[t] W^T) per visited frame and leaves the large weight-gradient
+ * GEMM (Y^T DX over all frames) to rocBLAS, which may allocate its own device workspace on first use; it cannot be
+ * recorded into a graph.  `workspace`: rtn_native_lstm2_bwd_workspace_bytes().
+ */
+int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const float* i, int32_t start, int32_t step,
+                         const void* Y, const float* C, const void* H, const void* DY, const float* Dd, void* DX,
+                         float* DW, void* Dy0, float* Dc0, int64_t T, int32_t B, int32_t n, int32_t dtype,
+                         void* workspace, size_t workspace_bytes, void* hip_stream);
+
+size_t rtn_native_lstm2_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype);
+
+/*
  * Final output per sequence.  Replaces the caller-side `_lstm_last_output`
  * (returnn/tf/native_op.py:913-929): out[b] = Y[t*, b] for the last visited frame t*
  * (in processing order) with i[t*, b] != 0, else y0[b].  Y, y0, out have element

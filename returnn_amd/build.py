@@ -19,8 +19,9 @@ CSRC_DIR = os.path.join(_dir, "csrc")
 LIB_NAME = "librtn_native_lstm2.so"
 LIB_PATH = os.path.join(CSRC_DIR, LIB_NAME)
 SOURCES = ["rtn_native_lstm2.hip"]
-HEADERS = ["lstm2_kernels.h", "lstm2_params.h", os.path.join("..", "..", "include", "rtn_native_lstm2.h")]
+HEADERS = ["lstm2_kernels.h", "lstm2_bwd_kernels.h", "lstm2_params.h", os.path.join("..", "..", "include", "rtn_native_lstm2.h")]
 OFFLOAD_ARCH = "gfx950"
+ROCM_LIB_DIR = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib")  # rocBLAS (weight-gradient GEMM of the backward op)
 
 
 def hipcc_path() -> str:
@@ -50,7 +51,7 @@ def compile_command(output: Optional[str] = None) -> List[str]:
         "-Wno-unused-command-line-argument",
         "-o",
         output or LIB_PATH,
-    ] + [os.path.join(CSRC_DIR, s) for s in SOURCES]
+    ] + [os.path.join(CSRC_DIR, s) for s in SOURCES] + ["-L%s" % ROCM_LIB_DIR, "-lrocblas", "-Wl,-rpath,%s" % ROCM_LIB_DIR]
 
 
 def needs_build() -> bool:

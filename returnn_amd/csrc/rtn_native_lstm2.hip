@@ -16,7 +16,10 @@
 #include <mutex>
 #include <string>
 
+#include <rocblas/rocblas.h>
+
 #include "../../include/rtn_native_lstm2.h"
+#include "lstm2_bwd_kernels.h"
 #include "lstm2_kernels.h"
 
 namespace rtn {
@@ -635,6 +638,53 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
   return RTN_OK;
 }
 
+
+// One rocBLAS handle per device, created on first use and kept for the life of the process.
+int blas_handle(rocblas_handle* out) {
+  static std::mutex mu;
+  static rocblas_handle handles[64] = {nullptr};
+  int dev = 0;
+  RTN_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) return fail(RTN_ERR_HIP, "NativeLstm2: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!handles[dev]) {
+    if (rocblas_create_handle(&handles[dev]) != rocblas_status_success) {
+      handles[dev] = nullptr;
+      return fail(RTN_ERR_HIP, "NativeLstm2: rocblas_create_handle failed");
+    }
+  }
+  *out = handles[dev];
+  return RTN_OK;
+}
+
+// DW[n,4n] (row major, float32) += A[rows,n]^T * Bm[rows,4n] with A, Bm of element type `dtype`, row major.
+int dw_accumulate(rocblas_handle h, const void* A, const void* Bm, float* DW, long long rows, int n, int dtype) {
+  if (rows <= 0) return RTN_OK;
+  const float alpha = 1.f, beta = 1.f;
+  const rocblas_datatype in = dtype == RTN_DTYPE_BF16 ? rocblas_datatype_bf16_r : rocblas_datatype_f32_r;
+  // Row-major DW[n,4n] is column-major [4n,n]: DW^T = Bm^T * A, with row-major Bm[rows,4n] = column-major [4n,rows]
+  // (no transpose) and row-major A[rows,n] = column-major [n,rows] (transpose).
+  const rocblas_status st = rocblas_gemm_ex(h, rocblas_operation_none, rocblas_operation_transpose, 4 * n, n, (rocblas_int)rows,
+                                            &alpha, Bm, in, 4 * n, A, in, n, &beta, DW, rocblas_datatype_f32_r, 4 * n, DW,
+                                            rocblas_datatype_f32_r, 4 * n, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+  if (st != rocblas_status_success) return fail(RTN_ERR_HIP, "NativeLstm2: rocblas_gemm_ex failed with status %d", (int)st);
+  return RTN_OK;
+}
+
+struct BwdLayout {
+  size_t off_dyw = 0, off_dx0 = 0, total = 0;
+};
+BwdLayout bwd_layout(int B, int n, int dtype) {
+  BwdLayout l;
+  size_t off = 256;  // status block, as in the forward workspace
+  l.off_dyw = off;
+  off = align_up(off + (size_t)B * n * 4, 256);
+  l.off_dx0 = off;
+  off = align_up(off + (size_t)B * 4 * n * esize(dtype), 256);
+  l.total = off;
+  return l;
+}
+
 }  // namespace
 }  // namespace rtn
 
@@ -729,6 +779,136 @@ int rtn_native_lstm2_fwd_multi_status(const void* workspace, int32_t count, int6
     const int rc = rtn_native_lstm2_fwd_status((const unsigned char*)workspace + (size_t)k * each, hip_stream);
     if (rc != RTN_OK) return rc;
   }
+  return RTN_OK;
+}
+
+size_t rtn_native_lstm2_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype) {
+  if (check_dims(T, B, n, dtype) != RTN_OK) return 0;
+  return bwd_layout(B, n, dtype).total;
+}
+
+int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const float* i, int32_t start, int32_t step,
+                         const void* Y, const float* C, const void* H, const void* DY, const float* Dd, void* DX, float* DW,
+                         void* Dy0, float* Dc0, int64_t T, int32_t B, int32_t n, int32_t dtype, void* workspace,
+                         size_t workspace_bytes, void* hip_stream) {
+  g_last_error.clear();
+  int rc = check_dims(T, B, n, dtype);
+  if (rc != RTN_OK) return rc;
+  hipStream_t stream = (hipStream_t)hip_stream;
+  const long long bn = (long long)B * n;
+  const long long nn4 = (long long)n * n * 4;
+  hipStreamCaptureStatus cap_status = hipStreamCaptureStatusNone;
+  if (stream) RTN_HIP(hipStreamIsCapturing(stream, &cap_status));
+  if (cap_status != hipStreamCaptureStatusNone)
+    return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2 backward: cannot be recorded into a graph (it calls rocBLAS)");
+  if (nn4 > 0 && !DW) return fail(RTN_ERR_ARG, "NativeLstm2 backward: DW must not be null");
+  if (bn > 0 && (!Dd || !Dy0 || !Dc0)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: Dd, Dy0 and Dc0 must not be null");
+  const dim3 fill_grid(256), fill_block(256);
+  // returnn/native_op.py:1365-1370: DW := 0, Dy0 := 0, Dc0 := Dd
+  if (nn4 > 0) {
+    hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)DW, 0u, nn4);
+    RTN_HIP(hipGetLastError());
+  }
+  if (bn > 0) {
+    hipLaunchKernelGGL(k_copy_f32, fill_grid, fill_block, 0, stream, Dd, Dc0, bn);
+    RTN_HIP(hipGetLastError());
+  }
+  if (T == 0 || bn == 0) {
+    if (bn > 0) {
+      RTN_HIP(hipMemsetAsync(Dy0, 0, (size_t)bn * esize(dtype), stream));
+    }
+    return RTN_OK;
+  }
+  if (start < 0 || start >= T) return fail(RTN_ERR_RANGE, "NativeLstm2 backward: need 0 <= start < T, got start=%d, T=%lld", start, (long long)T);
+  if (step == 0) return fail(RTN_ERR_RANGE, "NativeLstm2 backward: step must not be 0");
+  const void* ptrs[] = {W, y0, c0, i, Y, C, H, DY, Dd, DX, DW, Dy0, Dc0};
+  const char* names[] = {"W", "y0", "c0", "i", "Y", "C", "H", "DY", "Dd", "DX", "DW", "Dy0", "Dc0"};
+  for (int q = 0; q < 13; ++q) {
+    if (!ptrs[q]) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must not be null", names[q]);
+    if (q != 3 && !aligned16(ptrs[q])) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must be 16-byte aligned", names[q]);
+  }
+  const BwdLayout lay = bwd_layout(B, n, dtype);
+  if (!workspace || workspace_bytes < lay.total)
+    return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: workspace of %zu bytes needed, got %zu", lay.total, workspace ? workspace_bytes : (size_t)0);
+  if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: workspace must be 16-byte aligned");
+  rocblas_handle blas = nullptr;
+  rc = blas_handle(&blas);
+  if (rc != RTN_OK) return rc;
+  if (rocblas_set_stream(blas, stream) != rocblas_status_success) return fail(RTN_ERR_HIP, "NativeLstm2 backward: rocblas_set_stream failed");
+
+  Lstm2BwdParams p;
+  memset(&p, 0, sizeof(p));
+  p.W = W; p.c0 = c0; p.mask = i; p.C = C; p.H = H; p.DY = DY;
+  p.DX = DX; p.Dc0 = Dc0;
+  unsigned char* ws = (unsigned char*)workspace;
+  p.dyw = (float*)(ws + lay.off_dyw);
+  p.dx0 = ws + lay.off_dx0;
+  p.T = T; p.B = B; p.n = n;
+  const size_t es = esize(dtype);
+  hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)ws, 0u, (long long)(lay.total / 4));
+  RTN_HIP(hipGetLastError());
+
+  // returnn/native_op.py:1383-1407: which frames are visited, and in which order
+  const long long abs_step = step > 0 ? step : -(long long)step;
+  const long long num_steps = (T - start + abs_step - 1) / abs_step;
+  const long long first = step > 0 ? start : T - start - 1;
+  const long long end = first + (num_steps - 1) * step;  // inclusive
+  if (num_steps != T) {
+    // frames the loop does not visit keep DX = 0 (:1385-1388)
+    const long long words = (long long)((size_t)T * bn * 4 * es / 4);
+    hipLaunchKernelGGL(k_fill_u32, dim3(1024), fill_block, 0, stream, (unsigned*)DX, 0u, words);
+    RTN_HIP(hipGetLastError());
+  }
+  const bool mfma = (n % 16) == 0 && !env_long("RTN_LSTM2_FORCE_GENERIC", 0);
+  const int NT = B > 16 ? 2 : 1;
+  const dim3 pw_grid((unsigned)((bn + 255) / 256)), pw_block(256);
+  const dim3 mm_grid((unsigned)((n / 16) * ((B + 16 * NT - 1) / (16 * NT)))), mm_block(kWgThreads);
+  for (long long t = end; step > 0 ? t >= first : t <= first; t -= step) {
+    const bool right = step > 0 ? (t - step >= first) : (t - step <= first);
+    const long long prev_t = right ? t - step : -1;
+    if (dtype == RTN_DTYPE_BF16) {
+      hipLaunchKernelGGL(k_bwd_pointwise<__bf16>, pw_grid, pw_block, 0, stream, p, t, prev_t);
+      if (!mfma)
+        hipLaunchKernelGGL(k_bwd_gemm_dy_generic<__bf16>, pw_grid, pw_block, 0, stream, p, t);
+      else if (NT == 2)
+        hipLaunchKernelGGL((k_bwd_gemm_dy<__bf16, 2>), mm_grid, mm_block, 0, stream, p, t);
+      else
+        hipLaunchKernelGGL((k_bwd_gemm_dy<__bf16, 1>), mm_grid, mm_block, 0, stream, p, t);
+    } else {
+      hipLaunchKernelGGL(k_bwd_pointwise<float>, pw_grid, pw_block, 0, stream, p, t, prev_t);
+      if (!mfma)
+        hipLaunchKernelGGL(k_bwd_gemm_dy_generic<float>, pw_grid, pw_block, 0, stream, p, t);
+      else if (NT == 2)
+        hipLaunchKernelGGL((k_bwd_gemm_dy<float, 2>), mm_grid, mm_block, 0, stream, p, t);
+      else
+        hipLaunchKernelGGL((k_bwd_gemm_dy<float, 1>), mm_grid, mm_block, 0, stream, p, t);
+    }
+  }
+  RTN_HIP(hipGetLastError());
+
+  // DW = sum over consecutive visited frames Y[t - step]^T * DX[t]  (:1433-1452), then += y0^T * dx0 (:1456-1460)
+  const unsigned char* Yb = (const unsigned char*)Y;
+  const unsigned char* DXb = (const unsigned char*)DX;
+  if (num_steps > 1) {
+    if (abs_step == 1) {
+      const long long lo = std::min(first, end);
+      rc = dw_accumulate(blas, Yb + (size_t)(lo + std::max(0, -step)) * bn * es, DXb + (size_t)(lo + std::max(0, step)) * bn * 4 * es,
+                         DW, (num_steps - 1) * B, n, dtype);
+      if (rc != RTN_OK) return rc;
+    } else {
+      for (long long t = end - step; step > 0 ? t >= first : t <= first; t -= step) {
+        rc = dw_accumulate(blas, Yb + (size_t)t * bn * es, DXb + (size_t)(t + step) * bn * 4 * es, DW, B, n, dtype);
+        if (rc != RTN_OK) return rc;
+      }
+    }
+  }
+  rc = dw_accumulate(blas, y0, p.dx0, DW, B, n, dtype);
+  if (rc != RTN_OK) return rc;
+  if (dtype == RTN_DTYPE_BF16)
+    hipLaunchKernelGGL(k_convert_from_f32<__bf16>, fill_grid, fill_block, 0, stream, p.dyw, Dy0, bn);
+  else
+    hipLaunchKernelGGL(k_convert_from_f32<float>, fill_grid, fill_block, 0, stream, p.dyw, Dy0, bn);
+  RTN_HIP(hipGetLastError());
   return RTN_OK;
 }
 

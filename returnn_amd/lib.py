@@ -41,6 +41,8 @@ SYMBOLS = (
     "rtn_native_lstm2_fwd_multi_workspace_bytes",
     "rtn_native_lstm2_fwd_multi_status",
     "rtn_handover_latency_probe",
+    "rtn_native_lstm2_bwd",
+    "rtn_native_lstm2_bwd_workspace_bytes",
     "rtn_native_lstm2_last_output",
     "rtn_last_error",
     "rtn_native_lstm2_describe_plan",
@@ -102,6 +104,10 @@ def load() -> ctypes.CDLL:
         lib.rtn_native_lstm2_fwd_multi_workspace_bytes.argtypes = [i32, i64, i32, i32, i32, i32]
         lib.rtn_native_lstm2_fwd_multi_status.restype = ctypes.c_int
         lib.rtn_native_lstm2_fwd_multi_status.argtypes = [vp, i32, i64, i32, i32, i32, i32, vp]
+        lib.rtn_native_lstm2_bwd.restype = ctypes.c_int
+        lib.rtn_native_lstm2_bwd.argtypes = [vp, vp, vp, vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, vp, sz, vp]
+        lib.rtn_native_lstm2_bwd_workspace_bytes.restype = sz
+        lib.rtn_native_lstm2_bwd_workspace_bytes.argtypes = [i64, i32, i32, i32]
         lib.rtn_handover_latency_probe.restype = ctypes.c_int
         lib.rtn_handover_latency_probe.argtypes = [vp, sz, i32, vp]
         lib.rtn_native_lstm2_last_output.restype = ctypes.c_int

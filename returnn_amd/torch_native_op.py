@@ -260,6 +260,76 @@ def native_lstm2_multi(calls, *, mode: Optional[str] = None):
     return outs
 
 
+def native_lstm2_grad(W, y0, c0, i, start, step, Y, C, H, DY, Dd):
+    """
+    The gradient op of ``NativeLstm2`` on HIP tensors (returnn/native_op.py:1288-1464; arguments as
+    ``grad_input_map`` :1071-1077 without X, which the computation does not read).
+
+    :return: DX [T,B,4n] and Dy0 [B,n] in the element type of Y; DW [n,4n] and Dc0 [B,n] in float32
+    """
+    if not Y.is_cuda:
+        raise RuntimeError("NativeLstm2 gradient: this build implements the op for HIP (MI355X) tensors only; got CPU tensors.")
+    bf16 = Y.dtype == torch.bfloat16
+    act = torch.bfloat16 if bf16 else torch.float32
+    device = Y.device
+    W, y0, Y, H, DY = (t.to(act).contiguous() for t in (W, y0, Y, H, DY))
+    c0, i, C, Dd = (t.to(torch.float32).contiguous() for t in (c0, i, C, Dd))
+    T, B = i.shape
+    n = y0.shape[1]
+    expect = {"W": (n, 4 * n), "y0": (B, n), "c0": (B, n), "Y": (T, B, n), "C": (T, B, n), "H": (T, B, 4 * n),
+              "DY": (T, B, n), "Dd": (B, n)}  # fmt: skip
+    for name, t in (("W", W), ("y0", y0), ("c0", c0), ("Y", Y), ("C", C), ("H", H), ("DY", DY), ("Dd", Dd)):
+        if tuple(t.shape) != expect[name]:
+            raise RuntimeError("NativeLstm2 gradient: %s has shape %s, expected %s" % (name, tuple(t.shape), expect[name]))
+        if t.device != device:
+            raise RuntimeError("NativeLstm2 gradient: %s is on %s but Y is on %s" % (name, t.device, device))
+    lib = _lib.load()
+    dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
+    with torch.cuda.device(device):
+        DX = torch.empty((T, B, 4 * n), dtype=act, device=device)
+        DW = torch.empty((n, 4 * n), dtype=torch.float32, device=device)
+        Dy0 = torch.empty((B, n), dtype=act, device=device)
+        Dc0 = torch.empty((B, n), dtype=torch.float32, device=device)
+        ws_bytes = int(lib.rtn_native_lstm2_bwd_workspace_bytes(T, B, n, dtype))
+        ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=device)
+        rc = lib.rtn_native_lstm2_bwd(
+            W.data_ptr(), y0.data_ptr(), c0.data_ptr(), i.data_ptr(), int(start), int(step), Y.data_ptr(), C.data_ptr(),
+            H.data_ptr(), DY.data_ptr(), Dd.data_ptr(), DX.data_ptr(), DW.data_ptr(), Dy0.data_ptr(), Dc0.data_ptr(),
+            T, B, n, dtype, ws.data_ptr(), ws.numel(), torch.cuda.current_stream(device).cuda_stream,
+        )  # fmt: skip
+    _lib.check(rc)
+    return DX, DW, Dy0, Dc0
+
+
+class NativeLstm2Function(torch.autograd.Function):
+    """
+    ``NativeLstm2`` with its gradient, for training through autograd: ``Y, C, H, d = NativeLstm2Function.apply(X, W,
+    y0, c0, i, start, step)``.  Gradients flow from Y and d to X, W, y0 and c0; C and H are marked non-differentiable
+    (the reference's gradient op ignores error signals on them too, returnn/native_op.py:1071-1077); the mask gets none.
+    """
+
+    @staticmethod
+    def forward(ctx, X, W, y0, c0, i, start, step):
+        op = make_op(native_op.NativeLstm2)
+        Y, C, H, d = op(X, W, y0, c0, i, int(start), int(step))
+        ctx.save_for_backward(W, y0, c0, i, Y, C, H)
+        ctx.start, ctx.step = int(start), int(step)
+        ctx.in_dtypes = (X.dtype, W.dtype, y0.dtype, c0.dtype)
+        ctx.mark_non_differentiable(C, H)
+        return Y, C, H, d
+
+    @staticmethod
+    def backward(ctx, DY, _DC, _DH, Dd):
+        W, y0, c0, i, Y, C, H = ctx.saved_tensors
+        if DY is None:
+            DY = torch.zeros_like(Y)
+        if Dd is None:
+            Dd = torch.zeros_like(c0, dtype=torch.float32)
+        DX, DW, Dy0, Dc0 = native_lstm2_grad(W, y0, c0, i, ctx.start, ctx.step, Y, C, H, DY, Dd)
+        dX, dW, dy0, dc0 = (g.to(t) for g, t in zip((DX, DW, Dy0, Dc0), ctx.in_dtypes))
+        return dX, dW, dy0, dc0, None, None, None
+
+
 def lstm_last_output(Y: torch.Tensor, y0: torch.Tensor, i: torch.Tensor, start: int = 0, step: int = 1) -> torch.Tensor:
     """
     Final output per sequence, the caller-side ``_lstm_last_output`` of the reference

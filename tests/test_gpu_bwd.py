@@ -1,0 +1,128 @@
+"""
+GPU parity of the NativeLstm2 gradient op (C ABI ``rtn_native_lstm2_bwd``) against the CPU oracle of the reference's
+gradient code, on the forward results of the HIP path itself.
+
+Tolerances.  The north star fixes tolerances for the forward outputs only; gradients are sums over up to T*B terms
+whose summation order differs between MFMA tiles and a sequential loop, so they are judged relative to the largest
+magnitude of each array: float32 within 2e-5 of it (the float32 oracle itself is that far from the float64 oracle),
+bfloat16 (bf16 activations, gates and DX; float32 accumulation) within 2e-2 of it.
+"""
+
+from __future__ import annotations
+
+import numpy
+import pytest
+import torch
+
+from oracle import lstm2_oracle as oracle
+from returnn_amd import lib, synthetic, torch_native_op
+from _gpu_util import announce, get_op, random_problem, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _rel_to_max(got, want):
+    scale = max(float(numpy.abs(want).max()), 1e-30)
+    return float(numpy.abs(got - want).max()) / scale
+
+
+def _run(T, B, n, dtype, start, step, seed=0, scale_x=0.5):
+    X, W, y0, c0, i = random_problem(seed, T, B, n, scale_x=scale_x)
+    rng = numpy.random.default_rng(seed + 1000)
+    DY = rng.normal(0, 1.0, (T, B, n)).astype(numpy.float32)
+    Dd = rng.normal(0, 1.0, (B, n)).astype(numpy.float32)
+    op = get_op()
+    torch_native_op.OpMaker.options["NativeLstm2"]["mode"] = "auto"
+    Xd, Wd, y0d, DYd = (to_dev(a, dtype) for a in (X, W, y0, DY))
+    c0d, id_, Ddd = (to_dev(a, "f32") for a in (c0, i, Dd))
+    Y, C, H, d = op(Xd, Wd, y0d, c0d, id_, start, step)
+    got = torch_native_op.native_lstm2_grad(Wd, y0d, c0d, id_, start, step, Y, C, H, DYd, Ddd)
+    torch.cuda.synchronize()
+    got = [g.float().cpu().numpy() for g in got]
+    # the checker gets what the GPU's gradient op got: the GPU's own forward results and the same (rounded) inputs
+    f = lambda t: t.float().cpu().numpy().astype(numpy.float64)  # noqa: E731
+    want = oracle.native_lstm2_bwd(f(Xd), f(Wd), f(y0d), c0, i, start, step, f(Y), f(C), f(H), f(DYd), Dd, dtype=numpy.float64)
+    return got, want, (X, W, y0, c0, i, DY, Dd)
+
+
+@pytest.mark.parametrize("start,step", [(0, 1), (0, -1), (1, 2), (2, -3)])
+@pytest.mark.parametrize("T,B,n", [(7, 3, 16), (12, 20, 64), (9, 40, 128), (6, 5, 20), (5, 2, 3)])
+def test_bwd_f32(T, B, n, start, step):
+    announce("bwd f32", T, B, n, start, step)
+    got, want, _ = _run(T, B, n, "f32", start, step, seed=T + n)
+    for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), got, want):
+        assert a.shape == b.shape
+        assert _rel_to_max(a, b) <= 2e-5, (name, _rel_to_max(a, b))
+
+
+@pytest.mark.parametrize("step", [1, -1])
+@pytest.mark.parametrize("T,B,n", [(10, 16, 64), (16, 32, 256), (6, 5, 24)])
+def test_bwd_bf16(T, B, n, step):
+    announce("bwd bf16", T, B, n, step)
+    got, want, _ = _run(T, B, n, "bf16", 0, step, seed=T + n)
+    for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), got, want):
+        assert _rel_to_max(a, b) <= 2e-2, (name, _rel_to_max(a, b))
+
+
+def test_bwd_cfg2_reduced_f32():
+    announce("bwd cfg2 reduced")
+    p = synthetic.make_config("cfg2", T=60)
+    rng = numpy.random.default_rng(2)
+    DY = rng.normal(0, 1.0, (p.T, p.B, p.n)).astype(numpy.float32)
+    Dd = rng.normal(0, 1.0, (p.B, p.n)).astype(numpy.float32)
+    op = get_op()
+    args = [to_dev(a, "f32") for a in (p.X, p.W, p.y0, p.c0, p.i)]
+    Y, C, H, d = op(*args, 0, 1)
+    got = torch_native_op.native_lstm2_grad(args[1], args[2], args[3], args[4], 0, 1, Y, C, H, to_dev(DY, "f32"), to_dev(Dd, "f32"))
+    f = lambda t: t.float().cpu().numpy()  # noqa: E731
+    want = oracle.native_lstm2_bwd(p.X, p.W, p.y0, p.c0, p.i, 0, 1, f(Y), f(C), f(H), DY, Dd, dtype=numpy.float64)
+    for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), got, want):
+        assert _rel_to_max(f(a), b) <= 2e-5, (name, _rel_to_max(f(a), b))
+
+
+def test_bwd_autograd_function_matches_torch_lstm():
+    """End to end through autograd: loss on Y and d, gradients equal those of torch.nn.LSTM on the CPU (float64)."""
+    announce("bwd autograd")
+    from test_oracle_bwd import torch_lstm_grads
+
+    get_op()
+    T, B, n = 9, 6, 32
+    rng = numpy.random.default_rng(4)
+    X = rng.normal(0, 0.7, (T, B, 4 * n)).astype(numpy.float32)
+    W = (rng.normal(0, 1.0, (n, 4 * n)) / numpy.sqrt(n)).astype(numpy.float32)
+    y0 = rng.normal(0, 0.4, (B, n)).astype(numpy.float32)
+    c0 = rng.normal(0, 0.4, (B, n)).astype(numpy.float32)
+    lens = numpy.array([9, 4, 1, 7, 9, 2])
+    mask = (numpy.arange(T)[:, None] < lens[None, :]).astype(numpy.float32)
+    GY = rng.normal(0, 1.0, (T, B, n)).astype(numpy.float32)
+    Gd = rng.normal(0, 1.0, (B, n)).astype(numpy.float32)
+    for reverse in (False, True):
+        want = torch_lstm_grads(*(a.astype(numpy.float64) for a in (X, W, y0, c0)), lens, reverse, GY.astype(numpy.float64), Gd.astype(numpy.float64))
+        leaves = [to_dev(a, "f32").requires_grad_(True) for a in (X, W, y0, c0)]
+        Y, C, H, d = torch_native_op.NativeLstm2Function.apply(*leaves, to_dev(mask, "f32"), 0, -1 if reverse else 1)
+        assert not C.requires_grad and not H.requires_grad
+        loss = (Y * to_dev(GY, "f32")).sum() + (d * to_dev(Gd, "f32")).sum()
+        loss.backward()
+        for name, leaf, b in zip(("X", "W", "y0", "c0"), leaves, want):
+            assert _rel_to_max(leaf.grad.cpu().numpy().astype(numpy.float64), b) <= 2e-5, (name, reverse)
+
+
+def test_bwd_edge_cases_and_errors():
+    announce("bwd edge cases")
+    get_op()
+    cabi = lib.load()
+    B, n = 3, 16
+    z = lambda *s: torch.zeros(s, device="cuda:0")  # noqa: E731
+    Dd = torch.ones((B, n), device="cuda:0")
+    DX, DW, Dy0, Dc0 = torch_native_op.native_lstm2_grad(z(n, 4 * n), z(B, n), z(B, n), z(0, B), 0, 1, z(0, B, n), z(0, B, n),
+                                                         z(0, B, 4 * n), z(0, B, n), Dd)  # fmt: skip
+    assert DX.shape == (0, B, 4 * n) and float(DW.abs().max()) == 0 and float(Dy0.abs().max()) == 0 and bool((Dc0 == 1).all())
+    with pytest.raises(RuntimeError, match="start"):
+        torch_native_op.native_lstm2_grad(z(n, 4 * n), z(B, n), z(B, n), z(4, B), 9, 1, z(4, B, n), z(4, B, n), z(4, B, 4 * n), z(4, B, n), Dd)
+    with pytest.raises(RuntimeError, match="shape"):
+        torch_native_op.native_lstm2_grad(z(n, 4 * n), z(B, n), z(B, n), z(4, B), 0, 1, z(4, B, n), z(4, B, n), z(4, B, n), z(4, B, n), Dd)
+    with pytest.raises(RuntimeError, match="HIP"):
+        torch_native_op.native_lstm2_grad(*(t.cpu() for t in (z(n, 4 * n), z(B, n), z(B, n), z(4, B))), 0, 1,
+                                          *(t.cpu() for t in (z(4, B, n), z(4, B, n), z(4, B, 4 * n), z(4, B, n), Dd)))  # fmt: skip
+    assert cabi.rtn_native_lstm2_bwd_workspace_bytes(10, B, n, 0) > 0
+    assert cabi.rtn_native_lstm2_bwd_workspace_bytes(-1, B, n, 0) == 0
