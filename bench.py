@@ -185,6 +185,134 @@ def bench_encoder(args, dev):
     }
 
 
+def cpu_baseline_gradient(name: str, target_seconds: float = 15.0):
+    """Times the CPU restatement of the gradient op in its BLAS-structured form on a bounded sample."""
+    import numpy
+
+    from oracle import lstm2_oracle
+    from returnn_amd import synthetic
+
+    try:
+        from threadpoolctl import threadpool_info
+
+        blas_threads = max([int(i.get("num_threads", 1)) for i in threadpool_info() if i.get("user_api") == "blas"] or [1])
+    except Exception:
+        blas_threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    full_T = synthetic.make_config.__globals__["_SPECS"][name]["T"]
+    T = min(full_T, 25)
+    rng = numpy.random.default_rng(1)
+    for attempt in range(2):
+        p = synthetic.make_config(name, T=T)
+        Y, C, H, d, _ = lstm2_oracle.native_lstm2_fwd_blas(p.X, p.W, p.y0, p.c0, p.i)
+        DY = rng.standard_normal(Y.shape, dtype=numpy.float32)
+        Dd = rng.standard_normal(d.shape, dtype=numpy.float32)
+        lstm2_oracle.native_lstm2_bwd_blas(p.W, p.y0, p.c0, p.i, 0, 1, Y, C, H, DY, Dd)  # warm-up (BLAS thread pool, page-in)
+        t0 = time.perf_counter()
+        lstm2_oracle.native_lstm2_bwd_blas(p.W, p.y0, p.c0, p.i, 0, 1, Y, C, H, DY, Dd)
+        dt = time.perf_counter() - t0
+        if attempt == 0:
+            T2 = int(max(T, min(full_T, target_seconds / max(dt / T, 1e-9))))
+            if T2 == T:
+                break
+            T = T2
+    return {
+        "value": p.T * p.B / dt,
+        "unit": "timesteps*seqs/s",
+        "cores": blas_threads,
+        "kind": "port",
+        "sample": "gradient op, %s shape in fp32, one direction, first T=%i of %i frames (B=%i, n=%i), 1 pass, %.1f s; per frame the "
+        "sequential pointwise loop on 1 thread and one SGEMM on %i BLAS threads, one large SGEMM for the weight gradient, "
+        "as the reference's CPU path" % (name, p.T, full_T, p.B, p.n, dt, blas_threads),
+    }
+
+
+def bench_gradient(args, dev, cabi):
+    """
+    The gradient op (``rtn_native_lstm2_bwd``) of one direction of the workload, on the results of a forward run, all
+    resident in HBM.  One step = one gradient call; value = T*B*K / elapsed.  Algorithmic work per timestep x sequence:
+    8 n^2 flops for the recurrent GEMM (Dy0 += DX[t] W^T) plus 8 n^2 for the weight gradient (Y^T DX).
+    """
+    import torch
+
+    from returnn_amd import lib, native_op, synthetic, torch_native_op
+
+    p = synthetic.make_config(args.workload)
+    T, B, n = p.T, p.B, p.n
+    dtype = p.dtype
+    act = torch.bfloat16 if dtype == "bf16" else torch.float32
+    dt_code = lib.DTYPE_BF16 if dtype == "bf16" else lib.DTYPE_F32
+    op = torch_native_op.make_op(native_op.NativeLstm2)
+    X = torch.from_numpy(p.X).to(dev).to(act)
+    W = torch.from_numpy(p.W).to(dev).to(act)
+    y0 = torch.from_numpy(p.y0).to(dev).to(act)
+    c0 = torch.from_numpy(p.c0).to(dev)
+    msk = torch.from_numpy(p.i).to(dev)
+    Y, C, H, d = op(X, W, y0, c0, msk, 0, 1)
+    del X
+    gen = torch.Generator(device=dev).manual_seed(0)
+    DY = torch.randn(Y.shape, device=dev, generator=gen).to(act)
+    Dd = torch.randn(d.shape, device=dev, generator=gen)
+    DX = torch.empty((T, B, 4 * n), dtype=act, device=dev)
+    DW = torch.empty((n, 4 * n), dtype=torch.float32, device=dev)
+    Dy0 = torch.empty((B, n), dtype=act, device=dev)
+    Dc0 = torch.empty((B, n), dtype=torch.float32, device=dev)
+    ws = torch.empty((max(cabi.rtn_native_lstm2_bwd_workspace_bytes(T, B, n, dt_code), 256),), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev)
+
+    def call():
+        lib.check(cabi.rtn_native_lstm2_bwd(
+            W.data_ptr(), y0.data_ptr(), c0.data_ptr(), msk.data_ptr(), 0, 1, Y.data_ptr(), C.data_ptr(), H.data_ptr(),
+            DY.data_ptr(), Dd.data_ptr(), DX.data_ptr(), DW.data_ptr(), Dy0.data_ptr(), Dc0.data_ptr(), T, B, n, dt_code,
+            ws.data_ptr(), ws.numel(), stream.cuda_stream))  # fmt: skip
+
+    for _ in range(args.warmup):
+        call()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        call()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    assert bool(torch.isfinite(DW).all()) and bool(torch.isfinite(Dc0).all())
+    call_ms = elapsed * 1e3 / args.steps
+    flops = 16.0 * n * n * T * B
+    peak = PEAK_MFMA[dtype]
+    result = {
+        "metric": "LSTM gradient op timesteps*seqs/sec (T*B/s) at n=%i" % n,
+        "value": T * B * args.steps / elapsed,
+        "unit": "timesteps*seqs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": call_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype,
+        "data": "synthetic",
+        "config": {
+            "workload": "%s: NativeLstm2 gradient op, one direction, T=%i B=%i n=%i %s, ragged=%s"
+            % (args.workload, T, B, n, dtype, p.lens is not None),
+            "calls_per_step": 1,
+            "units_per_step": T * B,
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": flops / (call_ms * 1e-3) / 1e12,
+            "peak": peak / 1e12,
+            "unit": "TFLOP/s",
+            "frac": flops / (call_ms * 1e-3) / peak,
+            "traffic": None,
+            "kernel": "whole gradient call: per frame k_bwd_pointwise + k_bwd_gemm_dy (8*n^2 flops per unit), then the "
+            "weight-gradient GEMM in rocBLAS (8*n^2 flops per unit)",
+            "launch_ms": call_ms,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline_gradient(args.workload, args.cpu_seconds)
+    return result
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -195,6 +323,9 @@ def main():
     ap.add_argument("--pair", default="fused", choices=["fused", "separate"],
                     help="cfg3: issue the two directions through the multi-call entry (one launch when the device "
                          "holds both; default) or as two separate op calls")
+    ap.add_argument("--op", default="fwd", choices=["fwd", "bwd"],
+                    help="fwd: the forward op (default, the headline metric); bwd: the gradient op of one direction of "
+                         "the workload (cfg1/cfg2/cfg3/cfg5)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -221,6 +352,9 @@ def main():
 
     if args.workload == "cfg4":
         print(json.dumps(bench_encoder(args, dev)))
+        return
+    if args.op == "bwd":
+        print(json.dumps(bench_gradient(args, dev, cabi)))
         return
 
     p = synthetic.make_config(args.workload)

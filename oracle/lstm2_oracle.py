@@ -53,6 +53,8 @@ def _load():
         fp = ctypes.POINTER(ctypes.c_float)
         lib.lstm2_oracle_pointwise_f32.restype = None
         lib.lstm2_oracle_pointwise_f32.argtypes = [ctypes.c_int32, ctypes.c_int32] + [fp] * 7
+        lib.lstm2_oracle_bwd_pointwise_f32.restype = None
+        lib.lstm2_oracle_bwd_pointwise_f32.argtypes = [ctypes.c_int32, ctypes.c_int32] + [fp] * 8
         _lib = lib
     return _lib
 
@@ -240,4 +242,57 @@ def native_lstm2_bwd(X, W, y0, c0, i, start, step, Y, C, H, DY, Dd, *, dtype=num
         raise ValueError("oracle: need 0 <= start < T and step != 0 (start=%r, step=%r, T=%r)" % (start, step, T))
     if rc != 0:
         raise RuntimeError("oracle: error code %i" % rc)
+    return DX, DW, Dy0, Dc0
+
+
+def native_lstm2_bwd_blas(W, y0, c0, i, start, step, Y, C, H, DY, Dd):
+    """
+    The gradient op in float32 with the structure of the reference's CPU path: per visited frame the sequential
+    pointwise kernel, then ``Dy0 += DX[t] . W^T`` through the BLAS numpy links; afterwards the weight gradient as one
+    large GEMM (``|step| == 1``) or one per frame, and ``y0^T . dx0`` (returnn/native_op.py:1365-1462).  This is the
+    variant the benchmark times as the CPU baseline of the gradient op; it agrees with :func:`native_lstm2_bwd` up to
+    the summation order inside the BLAS.
+    """
+    f32 = numpy.float32
+    i = numpy.ascontiguousarray(i, dtype=f32)
+    y0 = numpy.ascontiguousarray(y0, dtype=f32)
+    T, B = i.shape
+    n = y0.shape[1]
+    W = _prep(W, f32, (n, 4 * n), "W")
+    c0 = _prep(c0, f32, (B, n), "c0")
+    Y = _prep(Y, f32, (T, B, n), "Y")
+    C = _prep(C, f32, (T, B, n), "C")
+    H = _prep(H, f32, (T, B, 4 * n), "H")
+    DY = _prep(DY, f32, (T, B, n), "DY")
+    DX = numpy.zeros((T, B, 4 * n), dtype=f32)
+    DW = numpy.zeros((n, 4 * n), dtype=f32)
+    Dy0 = numpy.zeros((B, n), dtype=f32)
+    Dc0 = _prep(Dd, f32, (B, n), "Dd").copy()
+    if T == 0:
+        return DX, DW, Dy0, Dc0
+    if not (0 <= start < T) or step == 0:
+        raise ValueError("oracle: need 0 <= start < T and step != 0 (start=%r, step=%r, T=%r)" % (start, step, T))
+    dx0 = numpy.zeros((B, 4 * n), dtype=f32)
+    abs_step = abs(step)
+    num_steps = (T - start + abs_step - 1) // abs_step
+    first = start if step > 0 else T - start - 1
+    end = first + (num_steps - 1) * step
+    pointwise = _load().lstm2_oracle_bwd_pointwise_f32
+    fp = ctypes.POINTER(ctypes.c_float)
+    ptr = lambda a: a.ctypes.data_as(fp)  # noqa: E731
+    WT = numpy.ascontiguousarray(W.T)
+    for t in range(end, first - step, -step):
+        prev_c = C[t - step] if t != first else c0
+        pointwise(B, n, ptr(i[t]), ptr(H[t]), ptr(prev_c), ptr(DY[t]), ptr(Dy0), ptr(Dc0), ptr(DX[t]), ptr(dx0))
+        Dy0 += DX[t] @ WT
+    if num_steps > 1:
+        if abs_step == 1:
+            lo = min(first, end)
+            ys = Y[lo + max(0, -step) : lo + max(0, -step) + num_steps - 1].reshape(-1, n)
+            dxs = DX[lo + max(0, step) : lo + max(0, step) + num_steps - 1].reshape(-1, 4 * n)
+            DW += ys.T @ dxs
+        else:
+            for t in range(end - step, first - step, -step):
+                DW += Y[t].T @ DX[t + step]
+    DW += y0.T @ dx0
     return DX, DW, Dy0, Dc0

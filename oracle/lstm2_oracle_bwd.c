@@ -26,7 +26,41 @@
 #define LSTM2_ERR_RANGE 2
 #define LSTM2_ERR_ALLOC 3
 
-#define DEFINE_BWD(NAME, REAL, TANHF)                                                                              \
+/* lstm_bwd_kernel (returnn/native_op.py:1123-1180) for one frame, executed sequentially like the reference's CPU
+ * emulation of a kernel launch (returnn/native_op.cpp:782-858). */
+#define DEFINE_BWD_POINTWISE(NAME, REAL, TANHF)                                                                    \
+  static void NAME(int32_t B, int32_t n, const REAL* m, const REAL* h, const REAL* prev_c, const REAL* d_y,        \
+                   REAL* d_h, REAL* d_c, REAL* d_x, REAL* dx0) {                                                   \
+    const int64_t bn = (int64_t)B * n, n4 = (int64_t)n * 4;                                                        \
+    for (int64_t idx = 0; idx < bn; ++idx) {                                                                       \
+      const int64_t b = idx / n, cell = idx % n;                                                                   \
+      const int64_t io = b * n4 + cell;                                                                            \
+      const REAL mask_b = m[b];                                                                                    \
+      const REAL d_y_b = (d_y[idx] + d_h[idx]) * mask_b;                                                           \
+      const REAL d_c_b = d_c[idx] * mask_b;                                                                        \
+      const REAL prev_c_b = prev_c[idx];                                                                           \
+      const REAL cellIn = h[io], inpGate = h[io + n], fgtGate = h[io + 2 * n], outGate = h[io + 3 * n];            \
+      const REAL c_b = prev_c_b * fgtGate + cellIn * inpGate;                                                      \
+      const REAL gc = TANHF(c_b);                                                                                  \
+      const REAL d_outGate_in = ((REAL)1 - outGate) * outGate * gc * d_y_b;                                        \
+      const REAL d_c2 = d_c_b + outGate * d_y_b * ((REAL)1 - gc * gc);                                             \
+      const REAL d_cellIn_in = ((REAL)1 - cellIn * cellIn) * inpGate * d_c2;                                       \
+      const REAL d_inpGate_in = ((REAL)1 - inpGate) * inpGate * cellIn * d_c2;                                     \
+      const REAL d_fgtGate_in = ((REAL)1 - fgtGate) * fgtGate * prev_c_b * d_c2;                                   \
+      d_c[idx] = fgtGate * d_c2 + d_c[idx] * ((REAL)1 - mask_b);                                                   \
+      d_x[io] = d_cellIn_in;                                                                                       \
+      d_x[io + n] = d_inpGate_in;                                                                                  \
+      d_x[io + 2 * n] = d_fgtGate_in;                                                                              \
+      d_x[io + 3 * n] = d_outGate_in;                                                                              \
+      for (int g = 0; g < 4; ++g) dx0[io + g * n] = d_x[io + g * n] + dx0[io + g * n] * ((REAL)1 - mask_b);        \
+      d_h[idx] *= ((REAL)1 - mask_b);                                                                              \
+    }                                                                                                              \
+  }
+
+DEFINE_BWD_POINTWISE(bwd_pointwise_f32, float, tanhf)
+DEFINE_BWD_POINTWISE(bwd_pointwise_f64, double, tanh)
+
+#define DEFINE_BWD(NAME, REAL, POINTWISE)                                                                            \
   int NAME(const REAL* X, const REAL* W, const REAL* y0, const REAL* c0, const REAL* mask, int32_t start,          \
            int32_t step, const REAL* Y, const REAL* C, const REAL* H, const REAL* DY, const REAL* Dd, REAL* DX,    \
            REAL* DW, REAL* Dy0, REAL* Dc0, int64_t T, int32_t B, int32_t n) {                                      \
@@ -52,29 +86,7 @@
       const REAL* d_y = DY + t * bn;                                                                               \
       REAL* d_x = DX + t * bn4;                                                                                    \
       const REAL* m = mask + t * B;                                                                                \
-      for (int64_t idx = 0; idx < bn; ++idx) {                                                                     \
-        const int64_t b = idx / n, cell = idx % n;                                                                 \
-        const int64_t io = b * n4 + cell;                                                                          \
-        const REAL mask_b = m[b];                                                                                  \
-        const REAL d_y_b = (d_y[idx] + Dy0[idx]) * mask_b;                                                         \
-        const REAL d_c_b = Dc0[idx] * mask_b;                                                                      \
-        const REAL prev_c_b = prev_c[idx];                                                                         \
-        const REAL cellIn = h[io], inpGate = h[io + n], fgtGate = h[io + 2 * n], outGate = h[io + 3 * n];          \
-        const REAL c_b = prev_c_b * fgtGate + cellIn * inpGate;                                                    \
-        const REAL gc = TANHF(c_b);                                                                                \
-        const REAL d_outGate_in = ((REAL)1 - outGate) * outGate * gc * d_y_b;                                      \
-        const REAL d_c2 = d_c_b + outGate * d_y_b * ((REAL)1 - gc * gc);                                           \
-        const REAL d_cellIn_in = ((REAL)1 - cellIn * cellIn) * inpGate * d_c2;                                     \
-        const REAL d_inpGate_in = ((REAL)1 - inpGate) * inpGate * cellIn * d_c2;                                   \
-        const REAL d_fgtGate_in = ((REAL)1 - fgtGate) * fgtGate * prev_c_b * d_c2;                                 \
-        Dc0[idx] = fgtGate * d_c2 + Dc0[idx] * ((REAL)1 - mask_b);                                                 \
-        d_x[io] = d_cellIn_in;                                                                                     \
-        d_x[io + n] = d_inpGate_in;                                                                                \
-        d_x[io + 2 * n] = d_fgtGate_in;                                                                            \
-        d_x[io + 3 * n] = d_outGate_in;                                                                            \
-        for (int g = 0; g < 4; ++g) dx0[io + g * n] = d_x[io + g * n] + dx0[io + g * n] * ((REAL)1 - mask_b);      \
-        Dy0[idx] *= ((REAL)1 - mask_b);                                                                            \
-      }                                                                                                            \
+      POINTWISE(B, n, m, h, prev_c, d_y, Dy0, Dc0, d_x, dx0);                                                      \
       /* Dy0 += DX[t] * W^T */                                                                                     \
       for (int64_t b = 0; b < B; ++b)                                                                              \
         for (int64_t k = 0; k < n; ++k) {                                                                          \
@@ -109,5 +121,11 @@
     return LSTM2_OK;                                                                                               \
   }
 
-DEFINE_BWD(lstm2_oracle_bwd_f32, float, tanhf)
-DEFINE_BWD(lstm2_oracle_bwd_f64, double, tanh)
+DEFINE_BWD(lstm2_oracle_bwd_f32, float, bwd_pointwise_f32)
+DEFINE_BWD(lstm2_oracle_bwd_f64, double, bwd_pointwise_f64)
+
+/* The pointwise kernel alone (for the BLAS-based variant the benchmark times as CPU baseline). */
+void lstm2_oracle_bwd_pointwise_f32(int32_t B, int32_t n, const float* m, const float* h, const float* prev_c,
+                                    const float* d_y, float* d_h, float* d_c, float* d_x, float* dx0) {
+  bwd_pointwise_f32(B, n, m, h, prev_c, d_y, d_h, d_c, d_x, dx0);
+}

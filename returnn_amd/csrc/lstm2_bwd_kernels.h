@@ -1,5 +1,5 @@
-// gfx950 kernels of the NativeLstm2 gradient op: one pointwise launch and one recurrent-GEMM launch per visited
-// frame, in reverse processing order (returnn/native_op.py:1288-1464, lstm_bwd_kernel :1123-1180).
+// gfx950 kernels of the NativeLstm2 gradient op: one launch per visited frame, in reverse processing order
+// (returnn/native_op.py:1288-1464, lstm_bwd_kernel :1123-1180).
 #pragma once
 
 #include "lstm2_kernels.h"
@@ -61,50 +61,105 @@ __global__ void k_bwd_pointwise(Lstm2BwdParams p, long long t, long long prev_t)
   p.dyw[idx] = dyw * (1.f - m);
 }
 
-// dyw[b,k] += sum_j DX[t][b,j] * W[k,j]  (j over the 4n gate columns) on MFMA.  Both operands are contiguous along j
-// in memory, which is exactly an MFMA fragment (16 bytes per lane): A = 16 rows of W, B = 16 rows of DX[t].
-// One workgroup per 16 values of k and 16*NT batch rows; j dealt round-robin to the 4 wavefronts, partial tiles
-// summed through LDS in wave order.  Needs n % 16 == 0.
+// One launch per visited frame on MFMA shapes (n % 16 == 0): the recurrent GEMM of the frame processed before
+// (t_gemm >= 0: dyw[b,k] += sum_j DX[t_gemm][b,j] * W[k,j], j over the 4n gate columns) followed, for the same (b, k)
+// pairs, by the pointwise part of frame t (t >= 0; prev_t < 0: the frame before is the initial state).  The last
+// launch of a call has t < 0: only the GEMM.
+// Both GEMM operands are contiguous along j in memory, which is exactly an MFMA fragment (16 bytes per lane): A = 16
+// rows of W, B = 16 rows of DX[t_gemm].  One workgroup per 16 values of k and 16*NT batch rows; j dealt round-robin
+// to the 4 wavefronts, partial tiles summed through LDS in wave order.  Every (b, k) pair belongs to exactly one
+// workgroup; dyw, Dc0 and dx0 of the pair live in memory between launches.
 template <typename AT, int NT>
-__global__ __launch_bounds__(kWgThreads) void k_bwd_gemm_dy(Lstm2BwdParams p, long long t) {
+__global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long long t_gemm, long long t, long long prev_t) {
   using E = Elem<AT>;
   constexpr int KE = E::KE, KM = E::KM;
   __shared__ f32x4 red[kWaves][NT][64];
+  __shared__ float tile[NT][16][17];  // [nt][b][k] sums of the GEMM, padded against bank conflicts
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = p.n, n4 = 4 * n;
   const int ktiles = n / 16;
   const int k0 = ((int)blockIdx.x % ktiles) * 16;
   const int b0 = ((int)blockIdx.x / ktiles) * 16 * NT;
-  const int S = n4 / KM;
-  const AT* Wr = (const AT*)p.W + (size_t)(k0 + (lane & 15)) * n4 + KE * (lane >> 4);
-  const AT* Dx = (const AT*)p.DX + (size_t)t * p.B * n4 + KE * (lane >> 4);
-  int brow[NT];
+  if (t_gemm >= 0) {
+    const int S = n4 / KM;
+    const AT* Wr = (const AT*)p.W + (size_t)(k0 + (lane & 15)) * n4 + KE * (lane >> 4);
+    const AT* Dx = (const AT*)p.DX + (size_t)t_gemm * p.B * n4 + KE * (lane >> 4);
+    int brow[NT];
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) brow[nt] = min(b0 + 16 * nt + (lane & 15), p.B - 1);  // rows past B: any row, dropped below
-  f32x4 acc[NT];
+    for (int nt = 0; nt < NT; ++nt) brow[nt] = min(b0 + 16 * nt + (lane & 15), p.B - 1);  // rows past B: any row, dropped below
+    f32x4 acc[NT];
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int s = wave; s < S; s += kWaves) {
-    const i32x4 a = *(const i32x4*)(Wr + (size_t)KM * s);
+    for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // U macro steps at a time: all their loads are issued before the first MFMA, so the memory latency is paid once
+    // per chunk and not once per macro step.
+    constexpr int U = 8;
+    for (int s0 = wave; s0 < S; s0 += kWaves * U) {
+      i32x4 a[U], bfrag[U][NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const i32x4 bfrag = *(const i32x4*)(Dx + (size_t)brow[nt] * n4 + (size_t)KM * s);
-      acc[nt] = E::mma(a, bfrag, acc[nt]);
+      for (int u = 0; u < U; ++u) {
+        const int s = min(s0 + kWaves * u, S - 1);  // past the end: a valid address, the product is dropped
+        a[u] = *(const i32x4*)(Wr + (size_t)KM * s);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) bfrag[u][nt] = *(const i32x4*)(Dx + (size_t)brow[nt] * n4 + (size_t)KM * s);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (s0 + kWaves * u < S) {
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) acc[nt] = E::mma(a[u], bfrag[u][nt], acc[nt]);
+        }
+      }
     }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) red[wave][nt][lane] = acc[nt];
+    __syncthreads();
+    for (int nt = wave; nt < NT; nt += kWaves) {
+      f32x4 sum = red[0][nt][lane];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) sum += red[w][nt][lane];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) tile[nt][lane & 15][4 * (lane >> 4) + r] = sum[r];
+    }
+    __syncthreads();
   }
+  // the (b, k) pairs of the tile, one or NT per thread
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) red[wave][nt][lane] = acc[nt];
-  __syncthreads();
-  for (int nt = wave; nt < NT; nt += kWaves) {
-    f32x4 sum = red[0][nt][lane];
+  for (int nt = 0; nt < NT; ++nt) {
+    const int bl = tid >> 4, kl = tid & 15;
+    const int b = b0 + 16 * nt + bl, k = k0 + kl;
+    if (b >= p.B) continue;
+    const long long idx = (long long)b * n + k;
+    float dyw = p.dyw[idx];
+    if (t_gemm >= 0) dyw += tile[nt][bl][kl];
+    if (t >= 0) {
+      const long long bn = (long long)p.B * n;
+      const long long io = (long long)b * n4 + k;
+      const long long fo = t * bn * 4 + io;
+      const float m = p.mask[t * p.B + b];
+      const float d_y_b = (E::load(p.DY, t * bn + idx) + dyw) * m;
+      const float dc = p.Dc0[idx];
+      const float d_c_b = dc * m;
+      const float prev_c = prev_t >= 0 ? p.C[prev_t * bn + idx] : p.c0[idx];
+      const float cellIn = E::load(p.H, fo), inpGate = E::load(p.H, fo + n), fgtGate = E::load(p.H, fo + 2 * n),
+                  outGate = E::load(p.H, fo + 3 * n);
+      const float c_b = prev_c * fgtGate + cellIn * inpGate;
+      const float gc = Act<AT>::tanh(c_b);
+      const float d_out = (1.f - outGate) * outGate * gc * d_y_b;
+      const float d_c2 = d_c_b + outGate * d_y_b * (1.f - gc * gc);
+      const float d_cin = (1.f - cellIn * cellIn) * inpGate * d_c2;
+      const float d_inp = (1.f - inpGate) * inpGate * cellIn * d_c2;
+      const float d_fgt = (1.f - fgtGate) * fgtGate * prev_c * d_c2;
+      p.Dc0[idx] = fgtGate * d_c2 + dc * (1.f - m);
+      const float dx[4] = {E::round(d_cin), E::round(d_inp), E::round(d_fgt), E::round(d_out)};
 #pragma unroll
-    for (int w = 1; w < kWaves; ++w) sum += red[w][nt][lane];
-    const int b = b0 + 16 * nt + (lane & 15);
-    if (b < p.B) {
-      float* out = p.dyw + (size_t)b * n + k0 + 4 * (lane >> 4);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) out[r] += sum[r];
+      for (int g = 0; g < 4; ++g) {
+        E::store(p.DX, fo + g * n, dx[g]);
+        const float old = E::load(p.dx0, io + g * n);
+        E::store(p.dx0, io + g * n, dx[g] + old * (1.f - m));
+      }
+      dyw *= (1.f - m);
     }
+    p.dyw[idx] = dyw;
   }
 }
 
@@ -128,6 +183,192 @@ template <typename AT>
 __global__ void k_convert_from_f32(const float* src, void* dst, long long count) {
   for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < count; i += (long long)gridDim.x * blockDim.x)
     Elem<AT>::store(dst, i, src[i]);
+}
+
+
+// ---------------------------------------------------------------------------------------------------------------
+// Persistent gradient kernel: all frames in one cooperative launch, W on chip for the whole call.
+//
+//  * decomposition: `groups` batch groups of up to 16 rows; inside a group, workgroup r owns 16 values of k: the
+//    rows k of W (A operand of  d_h[b,k] = sum_j DX[b,j] W[k,j],  16 x 4n values, in registers for the whole call:
+//    wavefront w holds the macro steps [w*KSB, (w+1)*KSB) of j) and, in the pointwise part, the cells k of its rows.
+//  * exchange: DX itself.  The host fills DX with all-ones words (a NaN pattern no result can have: NaNs are
+//    canonicalised) before the launch; the workgroup that owns (b, k) writes the four gate derivatives of a frame
+//    once, with device-scope stores; every workgroup of the group reads the frame's rows as MFMA B fragments (DX is
+//    contiguous along j: a fragment is 16 bytes of a row) with device-scope loads and reads again until no element
+//    is all-ones.  A frame's memory is written once and never reused, so there is nothing to re-arm.
+//  * per frame: wait for DX of the frame processed before, MFMA, sum of the 4 partial tiles through LDS, the
+//    pointwise part of this frame (inputs H, DY, C, mask fetched one frame ahead), DX out, first read of the
+//    next wait after an adaptive delay.  The cell error, the output error carried on and dx0 stay in registers.
+//  * all waits are bounded as in the forward kernel (status[0] = 1, everybody leaves).
+struct Lstm2BwdPersistent {
+  Lstm2BwdParams p;
+  const float* Dd;    // [B,n]
+  void* Dy0;          // [B,n] AT, out
+  unsigned* status;   // [0] != 0: a bounded wait expired
+  long long t_end;    // first frame processed (the last one the forward pass visited)
+  int step;           // the forward pass's signed stride; frames are processed t_end, t_end - step, ...
+  int nframes;        // number of visited frames
+  int groups, Bg;     // batch groups and rows per group (<= 16)
+  int poll_delay;
+  unsigned long long timeout_ticks;
+};
+
+template <typename AT, int KSB>
+__global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdPersistent q) {
+  using E = Elem<AT>;
+  using SN = Sentinel<AT>;
+  using LM = LaneMax<AT>;
+  constexpr int KE = E::KE, KM = E::KM, ES = (int)sizeof(AT);
+  const Lstm2BwdParams& p = q.p;
+  __shared__ f32x4 red[kWaves][64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = p.n, n4 = 4 * n;
+  const int ktiles = n / 16;
+  const int g = (int)blockIdx.x / ktiles, k0 = ((int)blockIdx.x % ktiles) * 16;
+  const int b_base = g * q.Bg;
+  const int rows = min(q.Bg, p.B - b_base);
+  const long long bn = (long long)p.B * n;
+  const unsigned frame_bytes = (unsigned)((size_t)p.B * n4 * ES);
+
+  // A fragments: this wavefront's macro steps of the 16 rows of W.
+  i32x4 wreg[KSB];
+  unsigned foff[KSB];  // byte offset of this lane's B fragments inside a frame of DX
+  {
+    const AT* Wr = (const AT*)p.W + (size_t)(k0 + (lane & 15)) * n4 + KE * (lane >> 4);
+    const int row = b_base + (((lane & 15) < rows) ? (lane & 15) : 0);  // rows the group does not have: read row 0
+#pragma unroll
+    for (int ks = 0; ks < KSB; ++ks) {
+      const int s = wave * KSB + ks;
+      wreg[ks] = *(const i32x4*)(Wr + (size_t)KM * s);
+      foff[ks] = (unsigned)(((size_t)row * n4 + (size_t)KM * s + KE * (lane >> 4)) * ES);
+    }
+  }
+
+  // The (row, k) pair of this thread.
+  const int bl = tid >> 4, kl = tid & 15;
+  const bool valid = bl < rows;
+  const int b = b_base + (valid ? bl : 0), k = k0 + kl;
+  const long long idx = (long long)b * n + k;
+  const long long io = (long long)b * n4 + k;
+  float dyw = 0.f, dc = valid ? q.Dd[idx] : 0.f;
+  float dx0[4] = {0.f, 0.f, 0.f, 0.f};
+  // where the pair's element of the summed tile is: tile element D[kl][bl] sits in lane (kl/4)*16 + bl, component kl%4
+  const int red_lane = (kl >> 2) * 16 + bl, red_comp = kl & 3;
+
+  // inputs of a frame, fetched one frame ahead
+  float in_gate[4], in_dy, in_pc, in_m;
+  auto fetch = [&](long long t, long long prev_t) {
+    const long long fo = t * bn * 4 + io;
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) in_gate[gq] = E::load(p.H, fo + (long long)gq * n);
+    in_dy = E::load(p.DY, t * bn + idx);
+    in_pc = prev_t >= 0 ? p.C[prev_t * bn + idx] : p.c0[idx];
+    in_m = p.mask[t * p.B + b];
+  };
+  auto frame = [&](int f) { return q.t_end - (long long)f * q.step; };
+
+  i32x4 bf[KSB];
+  auto issue = [&](long long t) {
+    __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
+    asm volatile("" ::: "memory");  // other workgroups write this memory: really load again
+#pragma unroll
+    for (int ks = 0; ks < KSB; ++ks) bf[ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, foff[ks], 0, kAuxDevice));
+  };
+  int delay = q.poll_delay;
+  bool aborted = false;
+  // d_h of the pair from DX of frame t (whose first read has been issued): wait, MFMA, sum over the wavefronts.
+  auto gemm = [&](long long t) -> float {
+    unsigned long long t0 = 0;
+    unsigned spins = 0;
+    for (;;) {
+      unsigned m = 0;
+#pragma unroll
+      for (int ks = 0; ks < KSB; ++ks)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) m = LM::fold(m, (unsigned)bf[ks][w]);
+      if (!__any(LM::has_sentinel(m))) break;
+      if ((spins++ & 15u) == 0) {
+        if (__hip_atomic_load(q.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { aborted = true; break; }
+        const unsigned long long now = wall_clock64();
+        if (spins == 1) {
+          t0 = now;
+        } else if (now - t0 > q.timeout_ticks) {
+          __hip_atomic_store(q.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          aborted = true;
+          break;
+        }
+      }
+      issue(t);
+    }
+    if (spins)
+      delay = min(delay + 2, 64);
+    else if (delay > 0)
+      delay -= ((t & 15) == 15) ? 1 : 0;
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KSB; ++ks) acc = E::mma(wreg[ks], bf[ks], acc);
+    red[wave][lane] = acc;
+    __syncthreads();
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) sum += ((const float*)&red[w][red_lane])[red_comp];
+    __syncthreads();  // red is free for the next frame
+    return sum;
+  };
+
+  const int F = q.nframes;
+  fetch(frame(0), F > 1 ? frame(1) : -1);
+  for (int f = 0; f < F; ++f) {
+    const long long t = frame(f);
+    if (f > 0) dyw += gemm(frame(f - 1));
+    // pointwise part of frame t (returnn/native_op.py:1123-1180)
+    const float m = in_m;
+    const float d_y_b = (in_dy + dyw) * m;
+    const float d_c_b = dc * m;
+    const float cellIn = in_gate[0], inpGate = in_gate[1], fgtGate = in_gate[2], outGate = in_gate[3];
+    const float c_b = in_pc * fgtGate + cellIn * inpGate;
+    const float gc = Act<AT>::tanh(c_b);
+    const float d_out = (1.f - outGate) * outGate * gc * d_y_b;
+    const float d_c2 = d_c_b + outGate * d_y_b * (1.f - gc * gc);
+    const float dx[4] = {E::round((1.f - cellIn * cellIn) * inpGate * d_c2), E::round((1.f - inpGate) * inpGate * cellIn * d_c2),
+                         E::round((1.f - fgtGate) * fgtGate * in_pc * d_c2), E::round(d_out)};
+    dc = fgtGate * d_c2 + dc * (1.f - m);
+    if (valid) {
+      __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) SN::template store<kAuxDevice>(rs, (unsigned)((io + (long long)gq * n) * ES), SN::bits(dx[gq]));
+    }
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) dx0[gq] = dx[gq] + dx0[gq] * (1.f - m);
+    dyw *= (1.f - m);
+    // while the derivatives travel: the inputs of the next frame, then the first read of this frame's DX
+    if (f + 1 < F) fetch(frame(f + 1), f + 2 < F ? frame(f + 2) : -1);
+    if (!aborted)
+      for (int d = 0; d < delay; ++d) __builtin_amdgcn_s_sleep(1);
+    issue(t);
+  }
+  dyw += gemm(frame(F - 1));
+  if (valid) {
+    E::store(q.Dy0, idx, dyw);
+    p.Dc0[idx] = dc;
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) E::store(p.dx0, io + (long long)gq * n, dx0[gq]);
+  }
+}
+
+// Frames the forward pass did not visit: DX = 0 (they still hold the all-ones fill of the persistent kernel).
+template <typename AT>
+__global__ void k_bwd_zero_unvisited(void* DX, long long T, long long frame_words, long long first, long long step, long long nframes) {
+  const long long lo = step > 0 ? first : first + (nframes - 1) * step;
+  const long long astep = step > 0 ? step : -step;
+  unsigned* w = (unsigned*)DX;
+  for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < T * frame_words; i += (long long)gridDim.x * blockDim.x) {
+    const long long t = i / frame_words;
+    const bool visited = t >= lo && t <= lo + (nframes - 1) * astep && ((t - lo) % astep) == 0;
+    if (!visited) w[i] = 0u;
+  }
 }
 
 }  // namespace rtn

@@ -345,15 +345,9 @@ int ensure_lds_limit(const void* k, size_t lds_bytes) {
   return RTN_OK;
 }
 
-// Library-owned graphs of the per-step launches, keyed by everything a launch depends on.
-struct GraphKey {
-  Lstm2Params p;
-  int dtype, MT, NT, kind, dev;
-  size_t lds;
-  bool operator==(const GraphKey& o) const { return memcmp(this, &o, sizeof(GraphKey)) == 0; }
-};
+// Library-owned graphs of per-step launch sequences, keyed by everything the launches depend on (a byte string).
 struct GraphEntry {
-  GraphKey key;
+  std::string key;
   hipGraph_t graph;
   hipGraphExec_t exec;
 };
@@ -361,35 +355,9 @@ std::mutex g_graph_mu;
 std::list<GraphEntry> g_graphs;  // most recently used first
 constexpr size_t kMaxGraphs = 8;
 
-int launch_steps(const Lstm2Params& p, const Plan& pl, int dtype, hipStream_t stream) {
-  if (pl.kind == kPlanMfma) {
-    MfmaKernel k = mfma_kernel(dtype, pl.MT, pl.NT);
-    const dim3 grid(pl.groups * pl.wgs_per_group), block(kWgThreads);
-    for (int s = 0; s < p.nsteps; ++s) hipLaunchKernelGGL(k, grid, block, pl.lds_bytes, stream, p, s, s + 1);
-  } else {
-    const long long bn = (long long)p.B * p.n;
-    const dim3 grid((unsigned)((bn + 255) / 256)), block(256);
-    for (int s = 0; s < p.nsteps; ++s) {
-      if (dtype == RTN_DTYPE_BF16)
-        hipLaunchKernelGGL(k_step_generic<__bf16>, grid, block, 0, stream, p, s);
-      else
-        hipLaunchKernelGGL(k_step_generic<float>, grid, block, 0, stream, p, s);
-    }
-  }
-  RTN_HIP(hipGetLastError());
-  return RTN_OK;
-}
-
-int launch_steps_graph(const Lstm2Params& p, const Plan& pl, int dtype, hipStream_t stream) {
-  GraphKey key;
-  memset(&key, 0, sizeof(key));
-  key.p = p;
-  key.dtype = dtype;
-  key.MT = pl.MT;
-  key.NT = pl.NT;
-  key.kind = pl.kind;
-  key.lds = pl.lds_bytes;
-  RTN_HIP(hipGetDevice(&key.dev));
+// Launches the graph recorded for `key`; records it first (on a private stream, by calling `record`) if there is none.
+template <typename Record>
+int replay_graph(const std::string& key, hipStream_t stream, Record record) {
   std::lock_guard<std::mutex> lock(g_graph_mu);
   for (auto it = g_graphs.begin(); it != g_graphs.end(); ++it) {
     if (it->key == key) {
@@ -406,7 +374,7 @@ int launch_steps_graph(const Lstm2Params& p, const Plan& pl, int dtype, hipStrea
   int rc = RTN_OK;
   hipError_t e = hipStreamBeginCapture(cap, hipStreamCaptureModeThreadLocal);
   if (e == hipSuccess) {
-    rc = launch_steps(p, pl, dtype, cap);
+    rc = record(cap);
     hipError_t e2 = hipStreamEndCapture(cap, &graph);
     if (rc == RTN_OK && e2 != hipSuccess) rc = fail(RTN_ERR_HIP, "NativeLstm2: hipStreamEndCapture: %s", hipGetErrorString(e2));
   } else {
@@ -430,6 +398,40 @@ int launch_steps_graph(const Lstm2Params& p, const Plan& pl, int dtype, hipStrea
   }
   RTN_HIP(hipGraphLaunch(exec, stream));
   return RTN_OK;
+}
+
+template <typename T>
+void key_append(std::string* key, const T& v) {
+  key->append(reinterpret_cast<const char*>(&v), sizeof(T));
+}
+
+int launch_steps(const Lstm2Params& p, const Plan& pl, int dtype, hipStream_t stream) {
+  if (pl.kind == kPlanMfma) {
+    MfmaKernel k = mfma_kernel(dtype, pl.MT, pl.NT);
+    const dim3 grid(pl.groups * pl.wgs_per_group), block(kWgThreads);
+    for (int s = 0; s < p.nsteps; ++s) hipLaunchKernelGGL(k, grid, block, pl.lds_bytes, stream, p, s, s + 1);
+  } else {
+    const long long bn = (long long)p.B * p.n;
+    const dim3 grid((unsigned)((bn + 255) / 256)), block(256);
+    for (int s = 0; s < p.nsteps; ++s) {
+      if (dtype == RTN_DTYPE_BF16)
+        hipLaunchKernelGGL(k_step_generic<__bf16>, grid, block, 0, stream, p, s);
+      else
+        hipLaunchKernelGGL(k_step_generic<float>, grid, block, 0, stream, p, s);
+    }
+  }
+  RTN_HIP(hipGetLastError());
+  return RTN_OK;
+}
+
+int launch_steps_graph(const Lstm2Params& p, const Plan& pl, int dtype, hipStream_t stream) {
+  std::string key("fwd");
+  int dev = 0;
+  RTN_HIP(hipGetDevice(&dev));
+  key.append(reinterpret_cast<const char*>(&p), sizeof(p));  // the caller zeroed p before filling it in: padding compares equal
+  key_append(&key, dtype); key_append(&key, pl.MT); key_append(&key, pl.NT); key_append(&key, (int)pl.kind);
+  key_append(&key, pl.lds_bytes); key_append(&key, dev);
+  return replay_graph(key, stream, [&](hipStream_t cap) { return launch_steps(p, pl, dtype, cap); });
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -638,6 +640,20 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
   return RTN_OK;
 }
 
+
+typedef void (*BwdRegwKernel)(const Lstm2BwdPersistent);
+
+template <typename AT>
+BwdRegwKernel bwd_regw_kernel_for(int KSB) {
+  switch (KSB) {
+    case 2: return &k_lstm2_bwd_regw<AT, 2>;
+    case 4: return &k_lstm2_bwd_regw<AT, 4>;
+    case 8: return &k_lstm2_bwd_regw<AT, 8>;
+    case 16: return &k_lstm2_bwd_regw<AT, 16>;
+    case 32: return &k_lstm2_bwd_regw<AT, 32>;
+    default: return nullptr;
+  }
+}
 
 // One rocBLAS handle per device, created on first use and kept for the life of the process.
 int blas_handle(rocblas_handle* out) {
@@ -860,31 +876,111 @@ int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const f
     RTN_HIP(hipGetLastError());
   }
   const bool mfma = (n % 16) == 0 && !env_long("RTN_LSTM2_FORCE_GENERIC", 0);
-  const int NT = B > 16 ? 2 : 1;
-  const dim3 pw_grid((unsigned)((bn + 255) / 256)), pw_block(256);
-  const dim3 mm_grid((unsigned)((n / 16) * ((B + 16 * NT - 1) / (16 * NT)))), mm_block(kWgThreads);
-  for (long long t = end; step > 0 ? t >= first : t <= first; t -= step) {
-    const bool right = step > 0 ? (t - step >= first) : (t - step <= first);
-    const long long prev_t = right ? t - step : -1;
-    if (dtype == RTN_DTYPE_BF16) {
-      hipLaunchKernelGGL(k_bwd_pointwise<__bf16>, pw_grid, pw_block, 0, stream, p, t, prev_t);
-      if (!mfma)
-        hipLaunchKernelGGL(k_bwd_gemm_dy_generic<__bf16>, pw_grid, pw_block, 0, stream, p, t);
-      else if (NT == 2)
-        hipLaunchKernelGGL((k_bwd_gemm_dy<__bf16, 2>), mm_grid, mm_block, 0, stream, p, t);
+  // Persistent kernel: W in registers for the whole call, if a wavefront's share of the 16 x 4n slice fits
+  // (2..32 fragments) and all workgroups can be on the device together.
+  const void* pk = nullptr;
+  int KSB = 0;
+  const int bgroups = (B + 15) / 16;
+  {
+    const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
+    const int S = 4 * n / KM;
+    const bool shape_ok = mfma && (4 * n) % KM == 0 && S % kWaves == 0;
+    KSB = shape_ok ? S / kWaves : 0;
+    const long bwd_kernel = env_long("RTN_LSTM2_BWD_KERNEL", 0);  // 0 auto, 1 per-frame launches, 2 persistent
+    if (shape_ok && bwd_kernel != 1 && device_info().cooperative) {
+      BwdRegwKernel k = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(KSB) : bwd_regw_kernel_for<float>(KSB);
+      if (k) {
+        int per_cu = 0;
+        RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)k, kWgThreads, 0));
+        if ((long long)per_cu * device_info().cus >= (long long)bgroups * (n / 16)) pk = (const void*)k;
+      }
+    }
+    if (bwd_kernel == 2 && !pk)
+      return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2 backward: the persistent kernel cannot run T=%lld B=%d n=%d", (long long)T, B, n);
+  }
+  if (pk) {
+    // DX doubles as the exchange medium: armed with all-ones words, every visited frame is written by the kernel.
+    const long long words = (long long)((size_t)T * bn * 4 * es / 4);
+    hipLaunchKernelGGL(k_fill_u32, dim3(2048), fill_block, 0, stream, (unsigned*)DX, 0xFFFFFFFFu, words);
+    RTN_HIP(hipGetLastError());
+    Lstm2BwdPersistent q;
+    memset(&q, 0, sizeof(q));
+    q.p = p;
+    q.Dd = Dd;
+    q.Dy0 = Dy0;
+    q.status = (unsigned*)ws;
+    q.t_end = end;
+    q.step = step;
+    q.nframes = (int)num_steps;
+    q.groups = bgroups;
+    q.Bg = (B + bgroups - 1) / bgroups;
+    q.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", 20)));
+    q.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);
+    void* args[] = {(void*)&q};
+    RTN_HIP(hipLaunchCooperativeKernel(pk, dim3((unsigned)(bgroups * (n / 16))), dim3(kWgThreads), args, 0, stream));
+    if (num_steps != T) {
+      const long long frame_words = (long long)((size_t)bn * 4 * es / 4);
+      if (dtype == RTN_DTYPE_BF16)
+        hipLaunchKernelGGL(k_bwd_zero_unvisited<__bf16>, dim3(1024), fill_block, 0, stream, DX, (long long)T, frame_words, first, (long long)step, num_steps);
       else
-        hipLaunchKernelGGL((k_bwd_gemm_dy<__bf16, 1>), mm_grid, mm_block, 0, stream, p, t);
-    } else {
-      hipLaunchKernelGGL(k_bwd_pointwise<float>, pw_grid, pw_block, 0, stream, p, t, prev_t);
-      if (!mfma)
-        hipLaunchKernelGGL(k_bwd_gemm_dy_generic<float>, pw_grid, pw_block, 0, stream, p, t);
-      else if (NT == 2)
-        hipLaunchKernelGGL((k_bwd_gemm_dy<float, 2>), mm_grid, mm_block, 0, stream, p, t);
-      else
-        hipLaunchKernelGGL((k_bwd_gemm_dy<float, 1>), mm_grid, mm_block, 0, stream, p, t);
+        hipLaunchKernelGGL(k_bwd_zero_unvisited<float>, dim3(1024), fill_block, 0, stream, DX, (long long)T, frame_words, first, (long long)step, num_steps);
+      RTN_HIP(hipGetLastError());
     }
   }
-  RTN_HIP(hipGetLastError());
+  const int NT = B > 32 ? 2 : 1;  // up to 32 rows: more, smaller workgroups
+  // The launches of all frames, in reverse processing order.  MFMA shapes: one fused launch per frame (the GEMM of
+  // the frame processed before, then this frame's pointwise part) and a last GEMM-only launch; other shapes: a
+  // pointwise and a generic GEMM launch per frame.
+  auto record = [&](hipStream_t st) -> int {
+    const dim3 pw_grid((unsigned)((bn + 255) / 256)), pw_block(256);
+    const dim3 mm_grid((unsigned)((n / 16) * ((B + 16 * NT - 1) / (16 * NT)))), mm_block(kWgThreads);
+    long long t_done = -1;  // frame whose DX still has to go through the GEMM
+    for (long long t = end;; t -= step) {
+      const bool more = step > 0 ? t >= first : t <= first;
+      const bool right = more && (step > 0 ? (t - step >= first) : (t - step <= first));
+      const long long prev_t = right ? t - step : -1;
+      const long long tt = more ? t : -1;
+      if (mfma) {
+        if (dtype == RTN_DTYPE_BF16) {
+          if (NT == 2)
+            hipLaunchKernelGGL((k_bwd_step<__bf16, 2>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
+          else
+            hipLaunchKernelGGL((k_bwd_step<__bf16, 1>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
+        } else {
+          if (NT == 2)
+            hipLaunchKernelGGL((k_bwd_step<float, 2>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
+          else
+            hipLaunchKernelGGL((k_bwd_step<float, 1>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
+        }
+      } else if (more) {
+        if (dtype == RTN_DTYPE_BF16) {
+          hipLaunchKernelGGL(k_bwd_pointwise<__bf16>, pw_grid, pw_block, 0, st, p, t, prev_t);
+          hipLaunchKernelGGL(k_bwd_gemm_dy_generic<__bf16>, pw_grid, pw_block, 0, st, p, t);
+        } else {
+          hipLaunchKernelGGL(k_bwd_pointwise<float>, pw_grid, pw_block, 0, st, p, t, prev_t);
+          hipLaunchKernelGGL(k_bwd_gemm_dy_generic<float>, pw_grid, pw_block, 0, st, p, t);
+        }
+      }
+      if (!more) break;
+      t_done = t;
+    }
+    RTN_HIP(hipGetLastError());
+    return RTN_OK;
+  };
+  if (pk) {
+    rc = RTN_OK;
+  } else if (env_long("RTN_LSTM2_BWD_NO_GRAPH", 0)) {
+    rc = record(stream);
+  } else {
+    std::string key("bwd");
+    int dev = 0;
+    RTN_HIP(hipGetDevice(&dev));
+    key.append(reinterpret_cast<const char*>(&p), sizeof(p));  // p was zeroed before it was filled in
+    key_append(&key, dtype); key_append(&key, (int)start); key_append(&key, (int)step); key_append(&key, dev);
+    key_append(&key, (int)mfma);
+    rc = replay_graph(key, stream, record);
+  }
+  if (rc != RTN_OK) return rc;
 
   // DW = sum over consecutive visited frames Y[t - step]^T * DX[t]  (:1433-1452), then += y0^T * dx0 (:1456-1460)
   const unsigned char* Yb = (const unsigned char*)Y;
@@ -904,11 +1000,13 @@ int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const f
   }
   rc = dw_accumulate(blas, y0, p.dx0, DW, B, n, dtype);
   if (rc != RTN_OK) return rc;
-  if (dtype == RTN_DTYPE_BF16)
-    hipLaunchKernelGGL(k_convert_from_f32<__bf16>, fill_grid, fill_block, 0, stream, p.dyw, Dy0, bn);
-  else
-    hipLaunchKernelGGL(k_convert_from_f32<float>, fill_grid, fill_block, 0, stream, p.dyw, Dy0, bn);
-  RTN_HIP(hipGetLastError());
+  if (!pk) {
+    if (dtype == RTN_DTYPE_BF16)
+      hipLaunchKernelGGL(k_convert_from_f32<__bf16>, fill_grid, fill_block, 0, stream, p.dyw, Dy0, bn);
+    else
+      hipLaunchKernelGGL(k_convert_from_f32<float>, fill_grid, fill_block, 0, stream, p.dyw, Dy0, bn);
+    RTN_HIP(hipGetLastError());
+  }
   return RTN_OK;
 }
 

@@ -149,3 +149,14 @@ def test_bwd_zero_length_and_float32():
         assert_allclose(a, b, rtol=2e-4, atol=2e-5)
     with pytest.raises(ValueError):
         _oracle_grads(X, W, y0, c0, mask, 8, 1, GY, Gd)
+
+
+@pytest.mark.parametrize("start,step", [(0, 1), (0, -1), (1, 2), (2, -3)])
+def test_bwd_blas_variant_equals_the_restatement(start, step):
+    """The BLAS-structured variant that the benchmark times computes the same thing."""
+    X, W, y0, c0, mask, lens, GY, Gd = _problem(17, 10, 5, 12)
+    Y, C, H, d, _ = oracle.native_lstm2_fwd(X, W, y0, c0, mask, start, step, dtype=numpy.float32)
+    want = oracle.native_lstm2_bwd(X, W, y0, c0, mask, start, step, Y, C, H, GY, Gd, dtype=numpy.float32)
+    got = oracle.native_lstm2_bwd_blas(W, y0, c0, mask, start, step, Y, C, H, GY, Gd)
+    for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), got, want):
+        assert_allclose(a, b, rtol=1e-4, atol=1e-5, err_msg=name)
