@@ -306,9 +306,16 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdPer
       delay = min(delay + 2, 64);
     else if (delay > 0)
       delay -= ((t & 15) == 15) ? 1 : 0;
-    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    // independent partial sums keep the MFMA pipeline full (one chain would wait for every result)
+    constexpr int NACC = KSB >= 4 ? 4 : KSB;
+    f32x4 part[NACC];
 #pragma unroll
-    for (int ks = 0; ks < KSB; ++ks) acc = E::mma(wreg[ks], bf[ks], acc);
+    for (int a = 0; a < NACC; ++a) part[a] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KSB; ++ks) part[ks % NACC] = E::mma(wreg[ks], bf[ks], part[ks % NACC]);
+    f32x4 acc = part[0];
+#pragma unroll
+    for (int a = 1; a < NACC; ++a) acc += part[a];
     red[wave][lane] = acc;
     __syncthreads();
     float sum = 0.f;
