@@ -189,9 +189,11 @@ __global__ void k_convert_from_f32(const float* src, void* dst, long long count)
 // ---------------------------------------------------------------------------------------------------------------
 // Persistent gradient kernel: all frames in one cooperative launch, W on chip for the whole call.
 //
-//  * decomposition: `groups` batch groups of up to 16 rows; inside a group, workgroup r owns 16 values of k: the
-//    rows k of W (A operand of  d_h[b,k] = sum_j DX[b,j] W[k,j],  16 x 4n values, in registers for the whole call:
+//  * decomposition: `groups` batch groups of up to 16 rows; inside a group, workgroup r owns 16*MT values of k: the
+//    rows k of W (A operand of  d_h[b,k] = sum_j DX[b,j] W[k,j],  16*MT x 4n values, in registers for the whole call:
 //    wavefront w holds the macro steps [w*KSB, (w+1)*KSB) of j) and, in the pointwise part, the cells k of its rows.
+//    What a workgroup has to read per frame (rows x 4n values) is what its step time grows with -- a CU gets
+//    device-scope loads at only about 36 GB/s -- so the groups are made small (8 rows) when the device has the CUs.
 //  * exchange: DX itself.  The host fills DX with all-ones words (a NaN pattern no result can have: NaNs are
 //    canonicalised) before the launch; the workgroup that owns (b, k) writes the four gate derivatives of a frame
 //    once, with device-scope stores; every workgroup of the group reads the frame's rows as MFMA B fragments (DX is
@@ -214,57 +216,66 @@ struct Lstm2BwdPersistent {
   unsigned long long timeout_ticks;
 };
 
-template <typename AT, int KSB>
+template <typename AT, int KSB, int MT>
 __global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdPersistent q) {
   using E = Elem<AT>;
   using SN = Sentinel<AT>;
   using LM = LaneMax<AT>;
   constexpr int KE = E::KE, KM = E::KM, ES = (int)sizeof(AT);
   const Lstm2BwdParams& p = q.p;
-  __shared__ f32x4 red[kWaves][64];
+  __shared__ f32x4 red[kWaves][MT][64];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = p.n, n4 = 4 * n;
-  const int ktiles = n / 16;
-  const int g = (int)blockIdx.x / ktiles, k0 = ((int)blockIdx.x % ktiles) * 16;
+  const int kblocks = n / (16 * MT);  // workgroups per group; each owns MT tiles of 16 values of k
+  const int g = (int)blockIdx.x / kblocks, k0 = ((int)blockIdx.x % kblocks) * 16 * MT;
   const int b_base = g * q.Bg;
   const int rows = min(q.Bg, p.B - b_base);
   const long long bn = (long long)p.B * n;
   const unsigned frame_bytes = (unsigned)((size_t)p.B * n4 * ES);
 
-  // A fragments: this wavefront's macro steps of the 16 rows of W.
-  i32x4 wreg[KSB];
-  unsigned foff[KSB];  // byte offset of this lane's B fragments inside a frame of DX
-  {
-    const AT* Wr = (const AT*)p.W + (size_t)(k0 + (lane & 15)) * n4 + KE * (lane >> 4);
-    const int row = b_base + (((lane & 15) < rows) ? (lane & 15) : 0);  // rows the group does not have: read row 0
+  // A fragments: this wavefront's macro steps [wave*KSB, (wave+1)*KSB) of the 16*MT rows of W.
+  i32x4 wreg[MT][KSB];
 #pragma unroll
-    for (int ks = 0; ks < KSB; ++ks) {
-      const int s = wave * KSB + ks;
-      wreg[ks] = *(const i32x4*)(Wr + (size_t)KM * s);
-      foff[ks] = (unsigned)(((size_t)row * n4 + (size_t)KM * s + KE * (lane >> 4)) * ES);
-    }
+  for (int mt = 0; mt < MT; ++mt) {
+    const AT* Wr = (const AT*)p.W + (size_t)(k0 + 16 * mt + (lane & 15)) * n4 + (size_t)KM * KSB * wave + KE * (lane >> 4);
+#pragma unroll
+    for (int ks = 0; ks < KSB; ++ks) wreg[mt][ks] = *(const i32x4*)(Wr + (size_t)KM * ks);
   }
+  // byte offset of this lane's first B fragment inside a frame of DX; the others follow at KM*ES bytes each
+  const unsigned foff0 = (unsigned)(((size_t)(b_base + (((lane & 15) < rows) ? (lane & 15) : 0)) * n4  // rows the group lacks: row 0
+                                     + (size_t)KM * KSB * wave + KE * (lane >> 4)) * ES);
 
-  // The (row, k) pair of this thread.
+  // The (row, k) pairs of this thread, one per tile.
   const int bl = tid >> 4, kl = tid & 15;
   const bool valid = bl < rows;
-  const int b = b_base + (valid ? bl : 0), k = k0 + kl;
-  const long long idx = (long long)b * n + k;
-  const long long io = (long long)b * n4 + k;
-  float dyw = 0.f, dc = valid ? q.Dd[idx] : 0.f;
-  float dx0[4] = {0.f, 0.f, 0.f, 0.f};
-  // where the pair's element of the summed tile is: tile element D[kl][bl] sits in lane (kl/4)*16 + bl, component kl%4
+  const int b = b_base + (valid ? bl : 0);
+  long long idx[MT], io[MT];
+  float dyw[MT], dc[MT], dx0[MT][4];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int k = k0 + 16 * mt + kl;
+    idx[mt] = (long long)b * n + k;
+    io[mt] = (long long)b * n4 + k;
+    dyw[mt] = 0.f;
+    dc[mt] = valid ? q.Dd[idx[mt]] : 0.f;
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) dx0[mt][gq] = 0.f;
+  }
+  // where a pair's element of the summed tile is: tile element D[kl][bl] sits in lane (kl/4)*16 + bl, component kl%4
   const int red_lane = (kl >> 2) * 16 + bl, red_comp = kl & 3;
 
   // inputs of a frame, fetched one frame ahead
-  float in_gate[4], in_dy, in_pc, in_m;
+  float in_gate[MT][4], in_dy[MT], in_pc[MT], in_m;
   auto fetch = [&](long long t, long long prev_t) {
-    const long long fo = t * bn * 4 + io;
 #pragma unroll
-    for (int gq = 0; gq < 4; ++gq) in_gate[gq] = E::load(p.H, fo + (long long)gq * n);
-    in_dy = E::load(p.DY, t * bn + idx);
-    in_pc = prev_t >= 0 ? p.C[prev_t * bn + idx] : p.c0[idx];
+    for (int mt = 0; mt < MT; ++mt) {
+      const long long fo = t * bn * 4 + io[mt];
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) in_gate[mt][gq] = E::load(p.H, fo + (long long)gq * n);
+      in_dy[mt] = E::load(p.DY, t * bn + idx[mt]);
+      in_pc[mt] = prev_t >= 0 ? p.C[prev_t * bn + idx[mt]] : p.c0[idx[mt]];
+    }
     in_m = p.mask[t * p.B + b];
   };
   auto frame = [&](int f) { return q.t_end - (long long)f * q.step; };
@@ -274,12 +285,14 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdPer
     __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
     asm volatile("" ::: "memory");  // other workgroups write this memory: really load again
 #pragma unroll
-    for (int ks = 0; ks < KSB; ++ks) bf[ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, foff[ks], 0, kAuxDevice));
+    for (int ks = 0; ks < KSB; ++ks)
+      bf[ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, foff0 + (unsigned)(ks * KM * ES), 0, kAuxDevice));
   };
   int delay = q.poll_delay;
   bool aborted = false;
-  // d_h of the pair from DX of frame t (whose first read has been issued): wait, MFMA, sum over the wavefronts.
-  auto gemm = [&](long long t) -> float {
+  // d_h of the thread's pairs from DX of frame t (whose first read has been issued): wait, MFMA, sum over the
+  // wavefronts; added to dyw.
+  auto gemm = [&](long long t) {
     unsigned long long t0 = 0;
     unsigned spins = 0;
     for (;;) {
@@ -307,61 +320,77 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdPer
     else if (delay > 0)
       delay -= ((t & 15) == 15) ? 1 : 0;
     // independent partial sums keep the MFMA pipeline full (one chain would wait for every result)
-    constexpr int NACC = KSB >= 4 ? 4 : KSB;
-    f32x4 part[NACC];
+    constexpr int NACC = (MT >= 4 || KSB < 2) ? 1 : (MT == 2 || KSB < 4 ? 2 : 4);
+    f32x4 part[MT][NACC];
 #pragma unroll
-    for (int a = 0; a < NACC; ++a) part[a] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int ks = 0; ks < KSB; ++ks) part[ks % NACC] = E::mma(wreg[ks], bf[ks], part[ks % NACC]);
-    f32x4 acc = part[0];
+      for (int a = 0; a < NACC; ++a) part[mt][a] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int a = 1; a < NACC; ++a) acc += part[a];
-    red[wave][lane] = acc;
+    for (int ks = 0; ks < KSB; ++ks)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) part[mt][ks % NACC] = E::mma(wreg[mt][ks], bf[ks], part[mt][ks % NACC]);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      f32x4 acc = part[mt][0];
+#pragma unroll
+      for (int a = 1; a < NACC; ++a) acc += part[mt][a];
+      red[wave][mt][lane] = acc;
+    }
     __syncthreads();
-    float sum = 0.f;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) sum += ((const float*)&red[w][red_lane])[red_comp];
+    for (int mt = 0; mt < MT; ++mt) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) sum += ((const float*)&red[w][mt][red_lane])[red_comp];
+      dyw[mt] += sum;
+    }
     __syncthreads();  // red is free for the next frame
-    return sum;
   };
 
   const int F = q.nframes;
   fetch(frame(0), F > 1 ? frame(1) : -1);
   for (int f = 0; f < F; ++f) {
     const long long t = frame(f);
-    if (f > 0) dyw += gemm(frame(f - 1));
+    if (f > 0) gemm(frame(f - 1));
     // pointwise part of frame t (returnn/native_op.py:1123-1180)
     const float m = in_m;
-    const float d_y_b = (in_dy + dyw) * m;
-    const float d_c_b = dc * m;
-    const float cellIn = in_gate[0], inpGate = in_gate[1], fgtGate = in_gate[2], outGate = in_gate[3];
-    const float c_b = in_pc * fgtGate + cellIn * inpGate;
-    const float gc = Act<AT>::tanh(c_b);
-    const float d_out = (1.f - outGate) * outGate * gc * d_y_b;
-    const float d_c2 = d_c_b + outGate * d_y_b * (1.f - gc * gc);
-    const float dx[4] = {E::round((1.f - cellIn * cellIn) * inpGate * d_c2), E::round((1.f - inpGate) * inpGate * cellIn * d_c2),
-                         E::round((1.f - fgtGate) * fgtGate * in_pc * d_c2), E::round(d_out)};
-    dc = fgtGate * d_c2 + dc * (1.f - m);
-    if (valid) {
-      __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
+    __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
 #pragma unroll
-      for (int gq = 0; gq < 4; ++gq) SN::template store<kAuxDevice>(rs, (unsigned)((io + (long long)gq * n) * ES), SN::bits(dx[gq]));
+    for (int mt = 0; mt < MT; ++mt) {
+      const float d_y_b = (in_dy[mt] + dyw[mt]) * m;
+      const float d_c_b = dc[mt] * m;
+      const float cellIn = in_gate[mt][0], inpGate = in_gate[mt][1], fgtGate = in_gate[mt][2], outGate = in_gate[mt][3];
+      const float c_b = in_pc[mt] * fgtGate + cellIn * inpGate;
+      const float gc = Act<AT>::tanh(c_b);
+      const float d_out = (1.f - outGate) * outGate * gc * d_y_b;
+      const float d_c2 = d_c_b + outGate * d_y_b * (1.f - gc * gc);
+      const float dx[4] = {E::round((1.f - cellIn * cellIn) * inpGate * d_c2), E::round((1.f - inpGate) * inpGate * cellIn * d_c2),
+                           E::round((1.f - fgtGate) * fgtGate * in_pc[mt] * d_c2), E::round(d_out)};
+      dc[mt] = fgtGate * d_c2 + dc[mt] * (1.f - m);
+      if (valid) {
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) SN::template store<kAuxDevice>(rs, (unsigned)((io[mt] + (long long)gq * n) * ES), SN::bits(dx[gq]));
+      }
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) dx0[mt][gq] = dx[gq] + dx0[mt][gq] * (1.f - m);
+      dyw[mt] *= (1.f - m);
     }
-#pragma unroll
-    for (int gq = 0; gq < 4; ++gq) dx0[gq] = dx[gq] + dx0[gq] * (1.f - m);
-    dyw *= (1.f - m);
     // while the derivatives travel: the inputs of the next frame, then the first read of this frame's DX
     if (f + 1 < F) fetch(frame(f + 1), f + 2 < F ? frame(f + 2) : -1);
     if (!aborted)
       for (int d = 0; d < delay; ++d) __builtin_amdgcn_s_sleep(1);
     issue(t);
   }
-  dyw += gemm(frame(F - 1));
+  gemm(frame(F - 1));
   if (valid) {
-    E::store(q.Dy0, idx, dyw);
-    p.Dc0[idx] = dc;
 #pragma unroll
-    for (int gq = 0; gq < 4; ++gq) E::store(p.dx0, io + (long long)gq * n, dx0[gq]);
+    for (int mt = 0; mt < MT; ++mt) {
+      E::store(q.Dy0, idx[mt], dyw[mt]);
+      p.Dc0[idx[mt]] = dc[mt];
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) E::store(p.dx0, io[mt] + (long long)gq * n, dx0[mt][gq]);
+    }
   }
 }
 

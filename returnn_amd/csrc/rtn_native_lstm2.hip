@@ -644,15 +644,14 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
 typedef void (*BwdRegwKernel)(const Lstm2BwdPersistent);
 
 template <typename AT>
-BwdRegwKernel bwd_regw_kernel_for(int KSB) {
-  switch (KSB) {
-    case 2: return &k_lstm2_bwd_regw<AT, 2>;
-    case 4: return &k_lstm2_bwd_regw<AT, 4>;
-    case 8: return &k_lstm2_bwd_regw<AT, 8>;
-    case 16: return &k_lstm2_bwd_regw<AT, 16>;
-    case 32: return &k_lstm2_bwd_regw<AT, 32>;
-    default: return nullptr;
-  }
+BwdRegwKernel bwd_regw_kernel_for(int KSB, int MT) {
+#define RTN_CASE(ks, mt) \
+  if (KSB == ks && MT == mt) return &k_lstm2_bwd_regw<AT, ks, mt>;
+  RTN_CASE(2, 1) RTN_CASE(4, 1) RTN_CASE(8, 1) RTN_CASE(16, 1) RTN_CASE(32, 1)
+  RTN_CASE(2, 2) RTN_CASE(4, 2) RTN_CASE(8, 2) RTN_CASE(16, 2) RTN_CASE(32, 2)
+  RTN_CASE(2, 4) RTN_CASE(4, 4) RTN_CASE(8, 4) RTN_CASE(16, 4)
+#undef RTN_CASE
+  return nullptr;
 }
 
 // One rocBLAS handle per device, created on first use and kept for the life of the process.
@@ -879,8 +878,13 @@ int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const f
   // Persistent kernel: W in registers for the whole call, if a wavefront's share of the 16 x 4n slice fits
   // (2..32 fragments) and all workgroups can be on the device together.
   const void* pk = nullptr;
-  int KSB = 0;
-  const int bgroups = (B + 15) / 16;
+  int KSB = 0, bwd_mt = 1;
+  // Rows per batch group: 8 when the device has a CU for every workgroup then (a workgroup's step time grows with
+  // the rows x 4n values of DX it has to read per frame), else 16.
+  int rows_per_group = (int)env_long("RTN_LSTM2_BWD_ROWS", 0);
+  if (rows_per_group < 1 || rows_per_group > 16)
+    rows_per_group = ((long long)((B + 7) / 8) * (n / 16) <= device_info().cus) ? 8 : 16;
+  const int bgroups = (B + rows_per_group - 1) / rows_per_group;
   {
     const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
     const int S = 4 * n / KM;
@@ -888,11 +892,20 @@ int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const f
     KSB = shape_ok ? S / kWaves : 0;
     const long bwd_kernel = env_long("RTN_LSTM2_BWD_KERNEL", 0);  // 0 auto, 1 per-frame launches, 2 persistent
     if (shape_ok && bwd_kernel != 1 && device_info().cooperative) {
-      BwdRegwKernel k = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(KSB) : bwd_regw_kernel_for<float>(KSB);
-      if (k) {
+      // k tiles per workgroup: one, unless more are needed for the workgroups to fit on the device together.
+      const long env_mt = env_long("RTN_LSTM2_BWD_MT", 0);
+      for (int mt : {1, 2, 4}) {
+        if (env_mt && mt != env_mt) continue;
+        if (mt * KSB > 64 || (n / 16) % mt) continue;
+        BwdRegwKernel k = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(KSB, mt) : bwd_regw_kernel_for<float>(KSB, mt);
+        if (!k) continue;
         int per_cu = 0;
         RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)k, kWgThreads, 0));
-        if ((long long)per_cu * device_info().cus >= (long long)bgroups * (n / 16)) pk = (const void*)k;
+        if ((long long)per_cu * device_info().cus >= (long long)bgroups * (n / (16 * mt))) {
+          pk = (const void*)k;
+          bwd_mt = mt;
+          break;
+        }
       }
     }
     if (bwd_kernel == 2 && !pk)
@@ -917,7 +930,7 @@ int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const f
     q.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", 20)));
     q.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);
     void* args[] = {(void*)&q};
-    RTN_HIP(hipLaunchCooperativeKernel(pk, dim3((unsigned)(bgroups * (n / 16))), dim3(kWgThreads), args, 0, stream));
+    RTN_HIP(hipLaunchCooperativeKernel(pk, dim3((unsigned)(bgroups * (n / (16 * bwd_mt)))), dim3(kWgThreads), args, 0, stream));
     if (num_steps != T) {
       const long long frame_words = (long long)((size_t)bn * 4 * es / 4);
       if (dtype == RTN_DTYPE_BF16)
