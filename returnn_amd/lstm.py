@@ -16,6 +16,9 @@ then one ``NativeLstm2`` call with the right-padded 0/1 mask; output frames beyo
 ``direction=-1`` runs the recurrence from each sequence's last frame to its first without reversing anything
 in memory (the caller protocol of returnn/tf/layers/rec.py:1229-1270).
 
+With gradients enabled and an input that requires them, the same functions go through
+``NativeLstm2Function`` (the op with its gradient op) and torch's autograd, so the layer trains like ``rf.LSTM``.
+
 :class:`LSTM` and :class:`LstmState` mirror the module and its state; :class:`BlstmEncoder` stacks
 bidirectional layers (:func:`blstm`: both directions of a layer go through the library's multi-call entry, which
 runs them in one launch when the device can hold both; outputs concatenated).
@@ -29,7 +32,7 @@ from typing import NamedTuple, Optional, Sequence, Tuple, Union
 import torch
 
 from . import native_op
-from .torch_native_op import lstm_last_output, make_op, native_lstm2_multi
+from .torch_native_op import NativeLstm2Function, lstm_last_output, make_op, native_lstm2_multi
 
 __all__ = ["lstm", "blstm", "prepare_weights", "LstmWeights", "LSTM", "LstmState", "BlstmEncoder", "sequence_mask_time_major"]
 
@@ -145,11 +148,38 @@ def lstm(
         if tuple(seq_lens.shape) != (B,):
             raise ValueError("lstm: seq_lens must be [B]=[%i], got %s" % (B, tuple(seq_lens.shape)))
         mask = sequence_mask_time_major(seq_lens.to(device), maxlen=T)
-    Y, _C, _H, d = _native_lstm2()(X, weights.rec, state_h, state_c, mask, 0, direction)
-    h = lstm_last_output(Y, state_h, mask, 0, direction) if T > 0 else state_h.to(act)
+    if _wants_grad(X, weights.rec, state_h, state_c):
+        _native_lstm2()
+        Y, _C, _H, d = NativeLstm2Function.apply(X, weights.rec, state_h, state_c, mask, 0, direction)
+        h = _last_output_autograd(Y, state_h, seq_lens, direction)
+    else:
+        Y, _C, _H, d = _native_lstm2()(X, weights.rec, state_h, state_c, mask, 0, direction)
+        h = lstm_last_output(Y, state_h, mask, 0, direction) if T > 0 else state_h.to(act)
     if single_step:
         Y = Y[0]
     return Y, (h, d)
+
+
+def _wants_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+def _last_output_autograd(Y: torch.Tensor, y0: torch.Tensor, seq_lens: Optional[torch.Tensor], direction: int) -> torch.Tensor:
+    """
+    The final output per sequence with torch indexing, so that gradients flow (the library routine behind
+    :func:`lstm_last_output` has no gradient).  Valid for the right-padded masks this module builds from lengths: the
+    last processed valid frame is ``len-1`` going forward and frame 0 going backward; empty sequences keep ``y0``.
+    """
+    T, B, n = Y.shape
+    if T == 0:
+        return y0.to(Y.dtype)
+    lens = torch.full((B,), T, dtype=torch.int64, device=Y.device) if seq_lens is None else seq_lens.to(Y.device).to(torch.int64).clamp(max=T)
+    if direction > 0:
+        idx = (lens - 1).clamp(min=0)
+        last = Y[idx, torch.arange(B, device=Y.device)]
+    else:
+        last = Y[0]
+    return torch.where((lens > 0)[:, None], last, y0.to(Y.dtype))
 
 
 def _project(source: torch.Tensor, weights: LstmWeights, act: torch.dtype) -> torch.Tensor:
@@ -197,11 +227,16 @@ def blstm(
             raise ValueError("blstm: seq_lens must be [B]=[%i], got %s" % (B, tuple(seq_lens.shape)))
         mask = sequence_mask_time_major(seq_lens.to(source.device), maxlen=T)
     _native_lstm2()  # registers the op and fails loudly without the library
+    Xf, Xb = _project(source, fwd, act), _project(source, bwd, act)
+    if _wants_grad(Xf, Xb, fwd.rec, bwd.rec, state_fwd.h, state_fwd.c, state_bwd.h, state_bwd.c):
+        # training: one differentiable op call per direction (the gradient op runs per direction anyway)
+        Yf, _, _, df = NativeLstm2Function.apply(Xf, fwd.rec, state_fwd.h, state_fwd.c, mask, 0, 1)
+        Yb, _, _, db = NativeLstm2Function.apply(Xb, bwd.rec, state_bwd.h, state_bwd.c, mask, 0, -1)
+        hf = _last_output_autograd(Yf, state_fwd.h, seq_lens, 1)
+        hb = _last_output_autograd(Yb, state_bwd.h, seq_lens, -1)
+        return torch.cat((Yf, Yb), dim=-1), LstmState(h=hf, c=df), LstmState(h=hb, c=db)
     (Yf, _, _, df), (Yb, _, _, db) = native_lstm2_multi(
-        [
-            (_project(source, fwd, act), fwd.rec, state_fwd.h, state_fwd.c, mask, 0, 1),
-            (_project(source, bwd, act), bwd.rec, state_bwd.h, state_bwd.c, mask, 0, -1),
-        ]
+        [(Xf, fwd.rec, state_fwd.h, state_fwd.c, mask, 0, 1), (Xb, bwd.rec, state_bwd.h, state_bwd.c, mask, 0, -1)]
     )
     if T > 0:
         hf = lstm_last_output(Yf, state_fwd.h, mask, 0, 1)
@@ -238,6 +273,8 @@ class LSTM(torch.nn.Module):
 
     def _weights(self, act: torch.dtype) -> LstmWeights:
         ps = [self.ff_weight, self.rec_weight] + ([self.bias] if self.bias is not None else [])
+        if _wants_grad(*ps):
+            return prepare_weights(self.ff_weight, self.rec_weight, self.bias, dtype=act)  # differentiable, not cached
         key = (act,) + tuple((p.data_ptr(), p._version, p.device) for p in ps)
         if self._prepared is None or self._prepared[0] != key:
             with torch.no_grad():

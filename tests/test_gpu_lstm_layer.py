@@ -208,3 +208,90 @@ def test_blstm_encoder_cfg4_reduced_bf16():
     assert torch.equal(full, x)
     assert worst_layer <= BF16_ATOL
     assert worst_chain <= 5e-2
+
+
+def test_blstm_layer_gradients_vs_torch():
+    """Training through the layer: gradients of all parameters, the input and the initial states equal those of a
+    bidirectional torch.nn.LSTM on the CPU in float64 (loss on the outputs and on both final states)."""
+    announce("blstm layer gradients")
+    get_op()
+    rng = numpy.random.default_rng(21)
+    T, B, d_in, n = 11, 6, 10, 32
+    x = rng.standard_normal((T, B, d_in)).astype(numpy.float32)
+    lens = numpy.array([11, 3, 7, 1, 11, 5])
+    fwd, bwd = _params(rng, n, d_in), _params(rng, n, d_in)
+    h0 = (rng.standard_normal((2, B, n)) * 0.5).astype(numpy.float32)
+    c0 = (rng.standard_normal((2, B, n)) * 0.5).astype(numpy.float32)
+    G = rng.standard_normal((T, B, 2 * n)).astype(numpy.float32)
+    Gh = rng.standard_normal((2, B, n)).astype(numpy.float32)
+    Gc = rng.standard_normal((2, B, n)).astype(numpy.float32)
+
+    # reference: torch.nn.LSTM, float64, CPU
+    dt = torch.float64
+    m = torch.nn.LSTM(d_in, n, bidirectional=True).to(dt)
+    with torch.no_grad():
+        for sfx, p in (("", fwd), ("_reverse", bwd)):
+            getattr(m, "weight_ih_l0" + sfx).copy_(torch.as_tensor(p["ff_weight"], dtype=dt))
+            getattr(m, "weight_hh_l0" + sfx).copy_(torch.as_tensor(p["rec_weight"], dtype=dt))
+            getattr(m, "bias_ih_l0" + sfx).copy_(torch.as_tensor(p["bias"], dtype=dt) * 0.5)
+            getattr(m, "bias_hh_l0" + sfx).copy_(torch.as_tensor(p["bias"], dtype=dt) * 0.5)
+    xr = torch.tensor(x, dtype=dt, requires_grad=True)
+    h0r = torch.tensor(h0, dtype=dt, requires_grad=True)
+    c0r = torch.tensor(c0, dtype=dt, requires_grad=True)
+    packed = torch.nn.utils.rnn.pack_padded_sequence(xr, torch.as_tensor(lens), enforce_sorted=False)
+    out, (hT, cT) = m(packed, (h0r, c0r))
+    out, _ = torch.nn.utils.rnn.pad_packed_sequence(out, total_length=T)
+    ((out * torch.tensor(G, dtype=dt)).sum() + (hT * torch.tensor(Gh, dtype=dt)).sum() + (cT * torch.tensor(Gc, dtype=dt)).sum()).backward()
+
+    # this package, float32, GPU
+    mods = []
+    for p in (fwd, bwd):
+        mod = rlstm.LSTM(d_in, n, device=DEV)
+        with torch.no_grad():
+            for k in ("ff_weight", "rec_weight", "bias"):
+                getattr(mod, k).copy_(_dev(p[k]))
+        mods.append(mod)
+    xg = _dev(x).requires_grad_(True)
+    h0g = _dev(h0).requires_grad_(True)
+    c0g = _dev(c0).requires_grad_(True)
+    y, sf, sb = rlstm.blstm(xg, fwd=mods[0]._weights(torch.float32), bwd=mods[1]._weights(torch.float32),
+                            state_fwd=rlstm.LstmState(h0g[0], c0g[0]), state_bwd=rlstm.LstmState(h0g[1], c0g[1]),
+                            seq_lens=torch.from_numpy(lens))  # fmt: skip
+    loss = (y * _dev(G)).sum() + (sf.h * _dev(Gh[0])).sum() + (sb.h * _dev(Gh[1])).sum() + (sf.c * _dev(Gc[0])).sum() + (sb.c * _dev(Gc[1])).sum()
+    loss.backward()
+    assert_allclose(_np(y), out.detach().numpy(), rtol=F32_RTOL, atol=F32_ATOL)
+
+    def close(got, want, what):
+        want = want.detach().numpy() if isinstance(want, torch.Tensor) else want
+        scale = max(float(numpy.abs(want).max()), 1e-30)
+        assert float(numpy.abs(_np(got) - want).max()) / scale <= 3e-5, what
+
+    close(xg.grad, xr.grad, "x")
+    close(h0g.grad, h0r.grad, "h0")
+    close(c0g.grad, c0r.grad, "c0")
+    for mod, sfx in zip(mods, ("", "_reverse")):
+        close(mod.ff_weight.grad, getattr(m, "weight_ih_l0" + sfx).grad, "ff_weight" + sfx)
+        close(mod.rec_weight.grad, getattr(m, "weight_hh_l0" + sfx).grad, "rec_weight" + sfx)
+        close(mod.bias.grad, getattr(m, "bias_ih_l0" + sfx).grad, "bias" + sfx)  # either half of torch's bias sees the gradient of the sum
+
+
+def test_lstm_module_trains_one_step():
+    """The module under an optimizer: one SGD step lowers a simple loss (forward and gradient op end to end, bf16)."""
+    announce("lstm module trains")
+    get_op()
+    torch.manual_seed(0)
+    mod = rlstm.LSTM(16, 32, device=DEV, dtype=torch.bfloat16)
+    x = torch.randn(20, 8, 16, device=DEV).bfloat16()
+    target = torch.randn(20, 8, 32, device=DEV) * 0.1
+    lens = torch.tensor([20, 20, 15, 9, 20, 3, 12, 20])
+    s0 = mod.default_initial_state(batch_dims=(8,))
+    opt = torch.optim.SGD(mod.parameters(), lr=0.5)
+    losses = []
+    for _ in range(3):
+        opt.zero_grad()
+        y, _ = mod(x, state=s0, seq_lens=lens)
+        loss = ((y.float() - target) ** 2).mean()
+        loss.backward()
+        opt.step()
+        losses.append(float(loss.detach()))
+    assert all(numpy.isfinite(losses)) and losses[-1] < losses[0], losses
