@@ -156,11 +156,14 @@ int rtn_handover_latency_probe(void* workspace, size_t workspace_bytes, int32_t 
  *   DW  [n,4n]             out: gradient of W, always float32
  *   Dy0 [B,n]              out: gradient of y0        Dc0 [B,n]  out: gradient of c0 (float32)
  *
- * Element type `dtype` for W y0 Y H DY DX Dy0; c0 C i Dd Dc0 DW are float32.  This implementation runs one
- * launch per visited frame (the MFMA GEMM Dy0 += DX[t'] W^T of the frame processed before, fused with the frame's
- * pointwise part), replayed through a library-owned hipGraph, and leaves the large weight-gradient GEMM (Y^T DX over
- * all frames) to rocBLAS, which may allocate its own device workspace on first use; the call cannot be recorded
- * into a caller's graph.  `workspace`: rtn_native_lstm2_bwd_workspace_bytes().
+ * Element type `dtype` for W y0 Y H DY DX Dy0; c0 C i Dd Dc0 DW are float32.  Where the shape allows (n a multiple of
+ * 16, a wavefront's share of 16 rows of W fits its registers, all workgroups fit on the device) ONE persistent
+ * cooperative kernel runs all frames: W stays in registers, DX doubles as the self-validating exchange medium between
+ * workgroups.  Otherwise one launch per visited frame (the MFMA GEMM Dy0 += DX[t'] W^T of the frame processed before,
+ * fused with the frame's pointwise part), replayed through a library-owned hipGraph.  The large weight-gradient GEMM
+ * (Y^T DX over all frames) is left to rocBLAS, which may allocate its own device workspace on first use; the call
+ * cannot be recorded into a caller's graph.  `workspace`: rtn_native_lstm2_bwd_workspace_bytes();
+ * rtn_native_lstm2_fwd_status(workspace, stream) reports an expired bounded wait of the persistent kernel.
  */
 int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const float* i, int32_t start, int32_t step,
                          const void* Y, const float* C, const void* H, const void* DY, const float* Dd, void* DX,
