@@ -707,7 +707,7 @@ using namespace rtn;
 
 extern "C" {
 
-int rtn_native_lstm2_abi_version(void) { return 2; }
+int rtn_native_lstm2_abi_version(void) { return 3; }
 
 const char* rtn_last_error(void) { return g_last_error.c_str(); }
 
