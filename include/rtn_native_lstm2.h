@@ -174,6 +174,37 @@ int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const f
 size_t rtn_native_lstm2_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype);
 
 /*
+ * Sibling ops of NativeLstm2 on the same kernels (returnn/native_op.py:333-574 and :577-1026), forward pass.  In both,
+ * the recurrent input of a frame is the OUTPUT of the frame before -- 0 where that frame was masked -- instead of the
+ * last valid output carried over masked frames as in NativeLstm2.
+ *
+ * LstmGenericBase (c_fw_code :486-523, lstm_kernel :381-429; `NativeLstmCell` of the TF back-end):
+ *   Z [T,B,4n] gate inputs, V_h [n,4n], c [B,n] initial cell (float32), i [T,B]  ->  Y [T,B,n], H [T,B,4n] whose first
+ *   block holds the CELL STATE and the other three the activated input, forget and output gates, d [B,n] final cell.
+ *   No initial output (zero), always all frames in forward order, T > 0.  The reference works in place on Z; here H is
+ *   a separate array that must not overlap Z.
+ *
+ * LstmLowMem (c_fw_code :771-836, lstm_kernel :624-655):
+ *   X [T,B,n_in] raw input, W [n_in+n,4n] stacked input and recurrent weights, b [4n], y0, c0 [B,n], i, start, step
+ *   ->  Y, C [T,B,n], d [B,n].  start/step as for NativeLstm2 with one difference kept from the reference (:827-833): with
+ *   a negative step the loop runs from frame T-start-1 down to frame `start`, not down to frame 0.  Where that visits no
+ *   frame (2*start > T-1) the reference returns an unwritten d; here the call is refused with RTN_ERR_RANGE.  Frames the
+ *   loop does not visit are zero in Y and C (unwritten in the reference).  The input projection X.W[:n_in] + b is one rocBLAS GEMM over all frames into the
+ *   workspace (so the call cannot be recorded into a graph and, unlike the reference, needs T*B*8n elements of scratch:
+ *   the low memory footprint of the reference's variant is not reproduced, only its results).
+ */
+int rtn_lstm_generic_base_fwd(const void* Z, const void* V_h, const float* c, const float* i, void* Y, void* H, float* d,
+                              int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode, void* workspace,
+                              size_t workspace_bytes, void* hip_stream);
+size_t rtn_lstm_generic_base_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode);
+
+int rtn_lstm_low_mem_fwd(const void* X, const void* W, const void* b, const void* y0, const float* c0, const float* i,
+                         int32_t start, int32_t step, void* Y, float* C, float* d, int64_t T, int32_t B, int32_t n_in,
+                         int32_t n, int32_t dtype, int32_t mode, void* workspace, size_t workspace_bytes,
+                         void* hip_stream);
+size_t rtn_lstm_low_mem_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n_in, int32_t n, int32_t dtype, int32_t mode);
+
+/*
  * Final output per sequence.  Replaces the caller-side `_lstm_last_output`
  * (returnn/tf/native_op.py:913-929): out[b] = Y[t*, b] for the last visited frame t*
  * (in processing order) with i[t*, b] != 0, else y0[b].  Y, y0, out have element

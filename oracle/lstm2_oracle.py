@@ -49,6 +49,12 @@ def _load():
             bwd = getattr(lib, "lstm2_oracle_bwd_" + suffix)
             bwd.restype = ctypes.c_int
             bwd.argtypes = [ptr] * 5 + [ctypes.c_int32, ctypes.c_int32] + [ptr] * 9 + [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
+            gb = getattr(lib, "lstm_generic_base_oracle_fwd_" + suffix)
+            gb.restype = ctypes.c_int
+            gb.argtypes = [ptr] * 7 + [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
+            lm = getattr(lib, "lstm_low_mem_oracle_fwd_" + suffix)
+            lm.restype = ctypes.c_int
+            lm.argtypes = [ptr] * 6 + [ctypes.c_int32, ctypes.c_int32] + [ptr] * 3 + [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
         lib.lstm2_oracle_max_threads.restype = ctypes.c_int
         fp = ctypes.POINTER(ctypes.c_float)
         lib.lstm2_oracle_pointwise_f32.restype = None
@@ -296,3 +302,75 @@ def native_lstm2_bwd_blas(W, y0, c0, i, start, step, Y, C, H, DY, Dd):
                 DW += Y[t].T @ DX[t + step]
     DW += y0.T @ dx0
     return DX, DW, Dy0, Dc0
+
+
+def _suffix(dtype):
+    dtype = numpy.dtype(dtype)
+    if dtype == numpy.float32:
+        return dtype, "f32", ctypes.c_float
+    if dtype == numpy.float64:
+        return dtype, "f64", ctypes.c_double
+    raise ValueError("oracle: dtype must be float32 or float64")
+
+
+def lstm_generic_base_fwd(Z, V_h, c, i, *, dtype=numpy.float32):
+    """
+    Reference semantics of ``LstmGenericBase`` forward (returnn/native_op.py:381-429, :486-523).
+
+    :param Z: [T,B,4n] gate inputs (cell-in, input, forget, output)
+    :param V_h: [n,4n]
+    :param c: [B,n] initial cell state
+    :param i: [T,B] 0/1 mask
+    :return: Y [T,B,n], H [T,B,4n] (cell state, then the activated input, forget, output gates), d [B,n]
+    """
+    dtype, suffix, ctype = _suffix(dtype)
+    i = numpy.ascontiguousarray(i, dtype=dtype)
+    c = numpy.ascontiguousarray(c, dtype=dtype)
+    T, B = i.shape
+    n = c.shape[1]
+    Z = _prep(Z, dtype, (T, B, 4 * n), "Z")
+    V_h = _prep(V_h, dtype, (n, 4 * n), "V_h")
+    Y = numpy.zeros((T, B, n), dtype=dtype)
+    H = numpy.zeros((T, B, 4 * n), dtype=dtype)
+    d = numpy.zeros((B, n), dtype=dtype)
+    p = ctypes.POINTER(ctype)
+    rc = getattr(_load(), "lstm_generic_base_oracle_fwd_" + suffix)(*(a.ctypes.data_as(p) for a in (Z, V_h, c, i, Y, H, d)), T, B, n)
+    if rc != 0:
+        raise ValueError("oracle: LstmGenericBase needs T > 0")
+    return Y, H, d
+
+
+def lstm_low_mem_fwd(X, W, b, y0, c0, i, start: int = 0, step: int = 1, *, dtype=numpy.float32):
+    """
+    Reference semantics of ``LstmLowMem`` forward (returnn/native_op.py:624-655, :771-836).
+
+    :param X: [T,B,n_in]
+    :param W: [n_in+n,4n] input weights stacked on recurrent weights
+    :param b: [4n]
+    :return: Y [T,B,n], C [T,B,n], d [B,n]
+    """
+    dtype, suffix, ctype = _suffix(dtype)
+    i = numpy.ascontiguousarray(i, dtype=dtype)
+    y0 = numpy.ascontiguousarray(y0, dtype=dtype)
+    T, B = i.shape
+    n = y0.shape[1]
+    X = numpy.ascontiguousarray(X, dtype=dtype)
+    n_in = X.shape[2]
+    X = _prep(X, dtype, (T, B, n_in), "X")
+    W = _prep(W, dtype, (n_in + n, 4 * n), "W")
+    b = _prep(b, dtype, (4 * n,), "b")
+    c0 = _prep(c0, dtype, (B, n), "c0")
+    Y = numpy.zeros((T, B, n), dtype=dtype)
+    C = numpy.zeros((T, B, n), dtype=dtype)
+    d = numpy.zeros((B, n), dtype=dtype)
+    p = ctypes.POINTER(ctype)
+    rc = getattr(_load(), "lstm_low_mem_oracle_fwd_" + suffix)(
+        *(a.ctypes.data_as(p) for a in (X, W, b, y0, c0, i)), int(start), int(step), *(a.ctypes.data_as(p) for a in (Y, C, d)), T, B, n_in, n
+    )
+    if rc == 2:
+        raise ValueError("oracle: need 0 <= start < T and step != 0 (start=%r, step=%r, T=%r)" % (start, step, T))
+    if rc == 4:
+        raise ValueError("oracle: LstmLowMem with step < 0 runs from frame T-start-1 down to frame start; start=%r visits nothing" % start)
+    if rc != 0:
+        raise RuntimeError("oracle: error code %i" % rc)
+    return Y, C, d

@@ -123,9 +123,9 @@ __global__ void k_fill_unvisited(Lstm2Params p) {
     const long long delta = t - p.first;
     bool visited;
     if (p.step > 0)
-      visited = delta >= 0 && (delta % p.step) == 0;
+      visited = delta >= 0 && (delta % p.step) == 0 && delta / p.step < p.nsteps;
     else
-      visited = delta <= 0 && ((-delta) % (-p.step)) == 0;
+      visited = delta <= 0 && ((-delta) % (-p.step)) == 0 && delta / p.step < p.nsteps;
     if (visited) continue;
     ((AT*)p.H)[idx] = ((const AT*)p.X)[idx];
     const long long rem = idx - t * per_frame;
@@ -191,6 +191,13 @@ __global__ void k_fill_u32(unsigned* dst, unsigned value, long long count) {
     dst[i] = value;
 }
 
+// data[i] += bias[i % width]  (rows of `width` elements)
+template <typename AT>
+__global__ void k_add_bias(void* data, const void* bias, long long count, int width) {
+  for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < count; i += (long long)gridDim.x * blockDim.x)
+    Elem<AT>::store(data, i, Elem<AT>::load(data, i) + Elem<AT>::load(bias, i % width));
+}
+
 __global__ void k_clear_status(unsigned* status) {
   if (threadIdx.x < 64) status[threadIdx.x] = 0;
 }
@@ -249,16 +256,16 @@ __global__ void k_step_generic(Lstm2Params p, int s) {
   }
   const float m = p.mask[t * p.B + b];
   const float a0 = Act<AT>::tanh(g0), a1 = Act<AT>::sigmoid(g1), a2 = Act<AT>::sigmoid(g2), a3 = Act<AT>::sigmoid(g3);
-  Elem<AT>::store(p.H, xoff, a0);
+  const float pc = c_in[idx];
+  const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
+  Elem<AT>::store(p.H, xoff, (p.op_flags & kOpH0IsCell) ? c : a0);
   Elem<AT>::store(p.H, xoff + n, a1);
   Elem<AT>::store(p.H, xoff + 2 * (size_t)n, a2);
   Elem<AT>::store(p.H, xoff + 3 * (size_t)n, a3);
-  const float pc = c_in[idx];
-  const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
   p.C[t * bn + idx] = c;
   const float y = Elem<AT>::round(Act<AT>::tanh(c) * a3 * m);
   Elem<AT>::store(p.Y, t * bn + idx, y);
-  Elem<AT>::store(y_out, idx, y + Elem<AT>::load(y_in, idx) * (1.f - m));
+  Elem<AT>::store(y_out, idx, (p.op_flags & kOpNoCarry) ? y : y + Elem<AT>::load(y_in, idx) * (1.f - m));
   if (s == p.nsteps - 1) p.d[idx] = c;
 }
 
@@ -469,11 +476,11 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
         const float pc = c_state[j];
         const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
         const float y = E::round(Act<AT>::tanh(c) * a3 * m);
-        const float hn = E::round(y + h_prev[j] * (1.f - m));
+        const float hn = (p.op_flags & kOpNoCarry) ? y : E::round(y + h_prev[j] * (1.f - m));
         c_state[j] = c;
         h_prev[j] = hn;
         y_out[j] = y;
-        a_out[j][0] = a0;
+        a_out[j][0] = (p.op_flags & kOpH0IsCell) ? c : a0;
         a_out[j][1] = a1;
         a_out[j][2] = a2;
         a_out[j][3] = a3;
@@ -706,7 +713,6 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   const int n = p.n, S = n / KM;
   int g, r;
   map_block(p, bid, g, r);
-  const int G = p.wgs_per_group;
   const int b_base = g * p.Bg;
   const int rows = min(p.Bg, p.B - b_base);
   const long long bn = (long long)p.B * n;
@@ -959,11 +965,12 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
           const float pc = c_state[j];
           const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
           const float y = E::round(Act<AT>::tanh(c) * a3 * m);
-          const float hn = E::round(y + h_prev[j] * (1.f - m));
+          const float hn = (p.op_flags & kOpNoCarry) ? y : E::round(y + h_prev[j] * (1.f - m));
           c_state[j] = c;
           h_prev[j] = hn;
           h_bits[j] = SN::bits(hn);
-          g_act[j][0] = a0; g_act[j][1] = a1; g_act[j][2] = a2; g_act[j][3] = a3;
+          g_act[j][0] = (p.op_flags & kOpH0IsCell) ? c : a0;
+          g_act[j][1] = a1; g_act[j][2] = a2; g_act[j][3] = a3;
           y_out[j] = y;
         }
       }

@@ -14,6 +14,15 @@ enum SyncBits : int {
   kAcquireFence = 8,   // device-scope acquire fence (cache invalidate) after the flag wait
 };
 
+// Variations of the recurrence shared with NativeLstm2's sibling ops.
+enum OpFlags : int {
+  kOpNoCarry = 1,    // the recurrent input of a frame is the OUTPUT of the frame before (0 where that frame was masked),
+                     // not the last valid output carried over masked frames (LstmGenericBase, LstmLowMem)
+  kOpH0IsCell = 2,   // the first block of H holds the cell state instead of tanh(cell-in) (LstmGenericBase)
+  kOpEndAtStart = 4, // host side only: with a negative step the loop runs from frame T-start-1 down to frame `start`,
+                     // not down to frame 0 (LstmLowMem's loop bounds, returnn/native_op.py:827-833)
+};
+
 struct Lstm2Params {
   // inputs (device)
   const void* X;      // [T,B,4n] AT
@@ -49,6 +58,7 @@ struct Lstm2Params {
   int exchange;       // register kernel: 0 = normal operation; 3, 4 = measurement aids (see kExNoWait, kExProbe)
   int poll_delay;     // register kernel: s_sleep(1) repeats between the hidden-value stores and the first read of the next step
   unsigned long long* trace;  // optional [workgroups][8] cycle totals per phase (instrumented builds only)
+  int op_flags;       // OpFlags: variations of the recurrence for the sibling ops (0 = NativeLstm2)
   int zero;           // always 0; an operand the compiler cannot fold (idempotent atomics used as L2 reads)
   int sync_policy;    // SyncBits
   unsigned long long timeout_ticks;  // bound of one flag wait, in 100 MHz wall-clock ticks

@@ -469,7 +469,7 @@ size_t workspace_each(int count, int64_t T, int32_t B, int32_t n, int32_t dtype,
 // in one cooperative launch (their workgroups share the CUs and hide each other's exchange waits);
 // otherwise they are enqueued one after the other.
 int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode,
-              void* workspace, size_t workspace_bytes, void* hip_stream) {
+              void* workspace, size_t workspace_bytes, void* hip_stream, int op_flags = 0) {
   int rc = check_dims(T, B, n, dtype);
   if (rc != RTN_OK) return rc;
   if (mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return fail(RTN_ERR_ARG, "NativeLstm2: unknown mode %d", mode);
@@ -496,7 +496,10 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     const char* names[] = {"X", "W", "y0", "c0", "i", "Y", "C", "H", "d"};
     for (int q = 0; q < 9; ++q) {
       if (!ptrs[q]) return fail(RTN_ERR_ARG, "NativeLstm2: %s must not be null", names[q]);
-      if (q != 4 && !aligned16(ptrs[q])) return fail(RTN_ERR_ARG, "NativeLstm2: %s must be 16-byte aligned", names[q]);
+      // W is read in 16-byte fragments by the MFMA kernels only (n a multiple of 32); the generic kernels read single
+      // elements, which lets LstmLowMem pass the recurrent rows of its stacked matrix at any element offset
+      if (q != 4 && !(q == 1 && n % 32 != 0) && !aligned16(ptrs[q]))
+        return fail(RTN_ERR_ARG, "NativeLstm2: %s must be 16-byte aligned", names[q]);
     }
   }
 
@@ -568,10 +571,13 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
       p.nsteps = (int)((T - 1 - c.start) / c.step + 1);
     } else {
       p.first = (int)(T - c.start - 1);
-      p.nsteps = (int)(p.first / (-(long long)c.step) + 1);
+      const long long last = (op_flags & kOpEndAtStart) ? c.start : 0;
+      if (p.first < last) return fail(RTN_ERR_RANGE, "LstmLowMem: start=%d with a negative step visits no frame of T=%lld", c.start, (long long)T);
+      p.nsteps = (int)((p.first - last) / (-(long long)c.step) + 1);
     }
     p.step = c.step;
     p.groups = pl.groups; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
+    p.op_flags = op_flags;
     p.hx_bufs = kHxRing;
     p.hx_sentinel = pl.regw ? 1 : 0;
     p.exchange = (int)env_long("RTN_LSTM2_EXCHANGE", 0);
@@ -795,6 +801,104 @@ int rtn_native_lstm2_fwd_multi_status(const void* workspace, int32_t count, int6
     if (rc != RTN_OK) return rc;
   }
   return RTN_OK;
+}
+
+size_t rtn_lstm_generic_base_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
+  const size_t fwd = rtn_native_lstm2_fwd_workspace_bytes(T, B, n, dtype, mode);
+  if (fwd == 0) return 0;
+  // forward workspace | zero initial output [B,n] | cell states [T,B,n] float32 (the op has no C output)
+  return fwd + align_up((size_t)B * n * esize(dtype), 256) + align_up((size_t)T * B * n * 4, 256);
+}
+
+int rtn_lstm_generic_base_fwd(const void* Z, const void* V_h, const float* c, const float* i, void* Y, void* H, float* d,
+                              int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode, void* workspace,
+                              size_t workspace_bytes, void* hip_stream) {
+  g_last_error.clear();
+  int rc = check_dims(T, B, n, dtype);
+  if (rc != RTN_OK) return rc;
+  if (T == 0) return fail(RTN_ERR_SHAPE, "LstmGenericBase: needs T > 0");  // returnn/native_op.py:504
+  const size_t need = rtn_lstm_generic_base_fwd_workspace_bytes(T, B, n, dtype, mode);
+  if (!workspace || workspace_bytes < need)
+    return fail(RTN_ERR_WORKSPACE, "LstmGenericBase: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
+  if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "LstmGenericBase: workspace must be 16-byte aligned");
+  const size_t fwd = rtn_native_lstm2_fwd_workspace_bytes(T, B, n, dtype, mode);
+  unsigned char* ws = (unsigned char*)workspace;
+  void* y0 = ws + fwd;
+  const size_t y0_bytes = align_up((size_t)B * n * esize(dtype), 256);
+  float* C = (float*)(ws + fwd + y0_bytes);
+  if ((long long)B * n > 0) {
+    hipLaunchKernelGGL(k_fill_u32, dim3(64), dim3(256), 0, (hipStream_t)hip_stream, (unsigned*)y0, 0u, (long long)(y0_bytes / 4));
+    RTN_HIP(hipGetLastError());
+  }
+  rtn_lstm2_call call = {Z, V_h, y0, c, i, 0, 1, Y, C, H, d};
+  return fwd_calls(&call, 1, T, B, n, dtype, mode, workspace, fwd, hip_stream, kOpNoCarry | kOpH0IsCell);
+}
+
+size_t rtn_lstm_low_mem_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n_in, int32_t n, int32_t dtype, int32_t mode) {
+  (void)n_in;
+  const size_t fwd = rtn_native_lstm2_fwd_workspace_bytes(T, B, n, dtype, mode);
+  if (fwd == 0) return 0;
+  // forward workspace | projected input [T,B,4n] | activated gates [T,B,4n] (the op has no H output)
+  return fwd + 2 * align_up((size_t)T * B * 4 * n * esize(dtype), 256);
+}
+
+int rtn_lstm_low_mem_fwd(const void* X, const void* W, const void* b, const void* y0, const float* c0, const float* i,
+                         int32_t start, int32_t step, void* Y, float* C, float* d, int64_t T, int32_t B, int32_t n_in,
+                         int32_t n, int32_t dtype, int32_t mode, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  g_last_error.clear();
+  int rc = check_dims(T, B, n, dtype);
+  if (rc != RTN_OK) return rc;
+  if (n_in < 0) return fail(RTN_ERR_SHAPE, "LstmLowMem: negative input dimension %d", n_in);
+  if (T > 0 && (long long)B * n > 0 && step < 0 && start >= 0 && start < T && T - start - 1 < start)
+    return fail(RTN_ERR_RANGE, "LstmLowMem: start=%d with a negative step visits no frame of T=%lld", start, (long long)T);
+  hipStream_t stream = (hipStream_t)hip_stream;
+  hipStreamCaptureStatus cap_status = hipStreamCaptureStatusNone;
+  if (stream) RTN_HIP(hipStreamIsCapturing(stream, &cap_status));
+  if (cap_status != hipStreamCaptureStatusNone)
+    return fail(RTN_ERR_UNSUPPORTED, "LstmLowMem: cannot be recorded into a graph (the input projection calls rocBLAS)");
+  const size_t need = rtn_lstm_low_mem_fwd_workspace_bytes(T, B, n_in, n, dtype, mode);
+  if (!workspace || workspace_bytes < need)
+    return fail(RTN_ERR_WORKSPACE, "LstmLowMem: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
+  if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "LstmLowMem: workspace must be 16-byte aligned");
+  const size_t es = esize(dtype);
+  const size_t fwd = rtn_native_lstm2_fwd_workspace_bytes(T, B, n, dtype, mode);
+  const size_t frame_bytes = align_up((size_t)T * B * 4 * n * es, 256);
+  unsigned char* ws = (unsigned char*)workspace;
+  void* Xp = ws + fwd;
+  void* Hs = ws + fwd + frame_bytes;
+  const long long rows = (long long)T * B;
+  const unsigned char* W_rec = (const unsigned char*)W + (size_t)n_in * 4 * n * es;  // rows n_in.. of W: the recurrent part
+  if (rows > 0 && n > 0) {
+    if (!X || !W || !b) return fail(RTN_ERR_ARG, "LstmLowMem: X, W and b must not be null");
+    if (!aligned16(W)) return fail(RTN_ERR_ARG, "LstmLowMem: W must be 16-byte aligned");
+    // Xp = X . W[:n_in] + b   (returnn/native_op.py:815-826, the part of `intern` that does not depend on the recurrence)
+    rocblas_handle blas = nullptr;
+    rc = blas_handle(&blas);
+    if (rc != RTN_OK) return rc;
+    if (rocblas_set_stream(blas, stream) != rocblas_status_success) return fail(RTN_ERR_HIP, "LstmLowMem: rocblas_set_stream failed");
+    const rocblas_datatype ty = dtype == RTN_DTYPE_BF16 ? rocblas_datatype_bf16_r : rocblas_datatype_f32_r;
+    if (n_in > 0) {
+      const float alpha = 1.f, beta = 0.f;
+      // row-major Xp[rows,4n] = column-major [4n,rows] = W_ff (column-major [4n,n_in]) * X (column-major [n_in,rows])
+      const rocblas_status st = rocblas_gemm_ex(blas, rocblas_operation_none, rocblas_operation_none, 4 * n, (rocblas_int)rows, n_in, &alpha, W, ty,
+                                                4 * n, X, ty, n_in, &beta, Xp, ty, 4 * n, Xp, ty, 4 * n, rocblas_datatype_f32_r,
+                                                rocblas_gemm_algo_standard, 0, 0);
+      if (st != rocblas_status_success) return fail(RTN_ERR_HIP, "LstmLowMem: rocblas_gemm_ex failed with status %d", (int)st);
+    } else {
+      hipLaunchKernelGGL(k_fill_u32, dim3(1024), dim3(256), 0, stream, (unsigned*)Xp, 0u, (long long)(frame_bytes / 4));
+    }
+    const long long total = rows * 4 * n;
+    const dim3 grid((unsigned)std::min<long long>((total + 255) / 256, 65535)), block(256);
+    if (dtype == RTN_DTYPE_BF16)
+      hipLaunchKernelGGL(k_add_bias<__bf16>, grid, block, 0, stream, Xp, b, total, 4 * n);
+    else
+      hipLaunchKernelGGL(k_add_bias<float>, grid, block, 0, stream, Xp, b, total, 4 * n);
+    RTN_HIP(hipGetLastError());
+  }
+  rtn_lstm2_call call = {Xp, W_rec, y0, c0, i, start, step, Y, C, Hs, d};
+  // With a negative step the reference's loop ends at frame `start`, and for 2*start > T-1 it visits no frame and
+  // returns an uninitialised d (returnn/native_op.py:827-833, :834); that case is refused with RTN_ERR_RANGE.
+  return fwd_calls(&call, 1, T, B, n, dtype, mode, workspace, fwd, hip_stream, kOpNoCarry | kOpEndAtStart);
 }
 
 size_t rtn_native_lstm2_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype) {

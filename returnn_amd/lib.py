@@ -43,6 +43,10 @@ SYMBOLS = (
     "rtn_handover_latency_probe",
     "rtn_native_lstm2_bwd",
     "rtn_native_lstm2_bwd_workspace_bytes",
+    "rtn_lstm_generic_base_fwd",
+    "rtn_lstm_generic_base_fwd_workspace_bytes",
+    "rtn_lstm_low_mem_fwd",
+    "rtn_lstm_low_mem_fwd_workspace_bytes",
     "rtn_native_lstm2_last_output",
     "rtn_last_error",
     "rtn_native_lstm2_describe_plan",
@@ -108,6 +112,14 @@ def load() -> ctypes.CDLL:
         lib.rtn_native_lstm2_bwd.argtypes = [vp, vp, vp, vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, vp, sz, vp]
         lib.rtn_native_lstm2_bwd_workspace_bytes.restype = sz
         lib.rtn_native_lstm2_bwd_workspace_bytes.argtypes = [i64, i32, i32, i32]
+        lib.rtn_lstm_generic_base_fwd.restype = ctypes.c_int
+        lib.rtn_lstm_generic_base_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, vp, sz, vp]
+        lib.rtn_lstm_generic_base_fwd_workspace_bytes.restype = sz
+        lib.rtn_lstm_generic_base_fwd_workspace_bytes.argtypes = [i64, i32, i32, i32, i32]
+        lib.rtn_lstm_low_mem_fwd.restype = ctypes.c_int
+        lib.rtn_lstm_low_mem_fwd.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, vp]
+        lib.rtn_lstm_low_mem_fwd_workspace_bytes.restype = sz
+        lib.rtn_lstm_low_mem_fwd_workspace_bytes.argtypes = [i64, i32, i32, i32, i32, i32]
         lib.rtn_handover_latency_probe.restype = ctypes.c_int
         lib.rtn_handover_latency_probe.argtypes = [vp, sz, i32, vp]
         lib.rtn_native_lstm2_last_output.restype = ctypes.c_int

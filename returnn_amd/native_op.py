@@ -2,8 +2,8 @@
 Operator descriptions: the backend-neutral contract of a native op.
 
 Mirrors the role of ``returnn.native_op`` (``NativeOpGenBase`` returnn/native_op.py:300-330,
-``OpDescription`` :254-297, shape inference :138-163) for the one operator this package
-implements.  The reference's description classes carry C code strings that a generator compiles at
+``OpDescription`` :254-297, shape inference :138-163) for the operators this package
+implements (``NativeLstm2`` and, forward only, its siblings ``LstmGenericBase`` and ``LstmLowMem``).  The reference's description classes carry C code strings that a generator compiles at
 run time; here a description names the entry point of the prebuilt gfx950 library instead.
 """
 
@@ -18,7 +18,7 @@ class NativeOpGenBase:
     in_info: Optional[Tuple[Dict[str, Any], ...]] = None
     out_info: Optional[Tuple[Dict[str, Any], ...]] = None
     c_abi_fw: Optional[str] = None  # forward entry point in librtn_native_lstm2.so
-    c_abi_bw: Optional[str] = None  # backward entry point (none yet)
+    c_abi_bw: Optional[str] = None  # gradient entry point, if any
     grad_input_map = None
     cpu_support = False  # HIP only: no CPU implementation is shipped
 
@@ -130,10 +130,79 @@ class NativeLstm2(NativeOpGenBase):
         {"name": "d", "ndim": 2, "shape": ((0, 1), (1, 0)), "need_contiguous": True},
     )
     c_abi_fw = "rtn_native_lstm2_fwd"
+    c_abi_bw = "rtn_native_lstm2_bwd"
 
     # noinspection PyPep8Naming
     @classmethod
     def grad_input_map(cls, X, W, y0, c0, i, start, step, Y, C, H, d, DY, DC, DH, Dd):
-        """What a backward op would consume (returnn/native_op.py:1071-1077)."""
+        """What the gradient op consumes (returnn/native_op.py:1071-1077)."""
         del d, DC, DH
         return X, W, y0, c0, i, start, step, Y, C, H, DY, Dd
+
+
+class LstmGenericBase(NativeOpGenBase):
+    """
+    Contract of ``returnn.native_op.LstmGenericBase`` (returnn/native_op.py:333-378), forward pass:
+
+    inputs:
+      :param Z: (time,batch,dim*4) gate inputs; last axis = cell-in, input, forget, output
+      :param V_h: recurrent matrix (dim,dim*4)
+      :param c: initial cell state (batch,dim)
+      :param i: (time,batch) 0/1 mask
+    outputs:
+      :param Y: (time,batch,dim)
+      :param H: (time,batch,dim*4) cell state, then the activated input, forget and output gates
+      :param d: (batch,dim) final cell state
+
+    The reference computes H in place of Z; here H is a new array.  The recurrent input of a frame is the output of
+    the frame before (zero where that was masked), there is no initial output.
+    """
+
+    in_info = (
+        {"name": "Z", "ndim": 3, "shape": (None, None, None), "need_contiguous": True},
+        {"name": "V_h", "ndim": 2, "shape": (None, None), "need_contiguous": True},
+        {"name": "c", "ndim": 2, "shape": (None, None), "need_contiguous": True},
+        {"name": "i", "ndim": 2, "shape": (None, None), "need_contiguous": True, "gradient": "disconnected"},
+    )
+    out_info = (
+        {"name": "Y", "ndim": 3, "shape": ((0, 0), (0, 1), (1, 0)), "need_contiguous": True},
+        {"name": "H", "ndim": 3, "shape": ((0, 0), (0, 1), (0, 2)), "need_contiguous": True},
+        {"name": "d", "ndim": 2, "shape": ((2, 0), (2, 1)), "need_contiguous": True},
+    )
+    c_abi_fw = "rtn_lstm_generic_base_fwd"
+
+
+class LstmLowMem(NativeOpGenBase):
+    """
+    Contract of ``returnn.native_op.LstmLowMem`` (returnn/native_op.py:577-615), forward pass:
+
+    inputs:
+      :param X: (time,batch,in_dim) raw input
+      :param W: input weights stacked on recurrent weights (in_dim+dim,dim*4)
+      :param b: bias (dim*4,)
+      :param y0: initial output (batch,dim)
+      :param c0: initial cell state (batch,dim)
+      :param i: (time,batch) 0/1 mask
+      :param start, step: host ints as for :class:`NativeLstm2`
+    outputs:
+      :param Y: (time,batch,dim)
+      :param C: (time,batch,dim) cell states
+      :param d: (batch,dim) final cell state
+    """
+
+    in_info = (
+        {"name": "X", "ndim": 3, "shape": (None, None, None), "need_contiguous": True},
+        {"name": "W", "ndim": 2, "shape": (None, None), "need_contiguous": True},
+        {"name": "b", "ndim": 1, "shape": (None,), "need_contiguous": True},
+        {"name": "y0", "ndim": 2, "shape": (None, None), "need_contiguous": True},
+        {"name": "c0", "ndim": 2, "shape": (None, None), "need_contiguous": True},
+        {"name": "i", "ndim": 2, "shape": (None, None), "need_contiguous": True, "gradient": "disconnected"},
+        {"name": "start", "ndim": 0, "shape": (), "gradient": "disconnected", "dtype": "int32", "host_memory": True},
+        {"name": "step", "ndim": 0, "shape": (), "gradient": "disconnected", "dtype": "int32", "host_memory": True},
+    )
+    out_info = (
+        {"name": "Y", "ndim": 3, "shape": ((0, 0), (0, 1), (4, 1)), "need_contiguous": True},
+        {"name": "C", "ndim": 3, "shape": ((0, 0), (0, 1), (4, 1)), "need_contiguous": True},
+        {"name": "d", "ndim": 2, "shape": ((0, 1), (4, 1)), "need_contiguous": True},
+    )
+    c_abi_fw = "rtn_lstm_low_mem_fwd"

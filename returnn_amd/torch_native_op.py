@@ -89,9 +89,14 @@ class OpMaker:
         return "%s(%s) -> (%s)" % (self.op_name, args, rets)
 
     def _impl_for(self):
-        if self.description.c_abi_fw == "rtn_native_lstm2_fwd":
-            return _native_lstm2_device_impl
-        raise NotImplementedError("no gfx950 implementation for op %r" % self.name)
+        impl = {
+            "rtn_native_lstm2_fwd": _native_lstm2_device_impl,
+            "rtn_lstm_generic_base_fwd": _lstm_generic_base_device_impl,
+            "rtn_lstm_low_mem_fwd": _lstm_low_mem_device_impl,
+        }.get(self.description.c_abi_fw)
+        if impl is None:
+            raise NotImplementedError("no gfx950 implementation for op %r" % self.name)
+        return impl
 
     def make_op(self):
         with self.global_lock:
@@ -120,7 +125,7 @@ class OpMaker:
             device = tensors[0].device
             shapes = description.infer_shape(None, [tuple(a.shape) if isinstance(a, torch.Tensor) else () for a in args])
             act = torch.bfloat16 if tensors[0].dtype == torch.bfloat16 else torch.float32
-            dtypes = {"Y": act, "H": act}
+            dtypes = {"Y": act, "H": act}  # cell states (C, d) are always float32
             return tuple(
                 torch.empty(shape, dtype=dtypes.get(o["name"], torch.float32), device=device)
                 for o, shape in zip(description.out_info, shapes)
@@ -211,6 +216,74 @@ def _native_lstm2_device_impl(X, W, y0, c0, i, start, step):
     # The workspace goes back to the caching allocator here; the allocator keeps it out of other
     # streams' hands until the work queued on this stream has passed it (stream-ordered reuse).
     return Y, C, H, d
+
+
+def _act_and_mode(first: torch.Tensor, op_name: str):
+    bf16 = first.dtype == torch.bfloat16
+    act = torch.bfloat16 if bf16 else torch.float32
+    dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
+    mode = _lib.MODES[OpMaker.options.get(op_name, {}).get("mode", "auto")]
+    return act, dtype, mode
+
+
+def _lstm_generic_base_device_impl(Z, V_h, c, i):
+    """``LstmGenericBase`` forward on HIP tensors (returnn/native_op.py:333-523)."""
+    for t, info in zip((Z, V_h, c, i), native_op.LstmGenericBase.in_info):
+        _check_ndim(t, info)
+    device = Z.device
+    act, dtype, mode = _act_and_mode(Z, "LstmGenericBase")
+    Z, V_h = (t.to(act).contiguous() for t in (Z, V_h))
+    c, i = (t.to(torch.float32).contiguous() for t in (c, i))
+    T, B = i.shape
+    n = c.shape[1]
+    for name, t, shape in (("Z", Z, (T, B, 4 * n)), ("V_h", V_h, (n, 4 * n)), ("c", c, (B, n))):
+        if tuple(t.shape) != shape:
+            raise RuntimeError("LstmGenericBase: %s has shape %s, expected %s" % (name, tuple(t.shape), shape))
+        if t.device != device:
+            raise RuntimeError("LstmGenericBase: %s is on %s but Z is on %s" % (name, t.device, device))
+    lib = _lib.load()
+    with torch.cuda.device(device):
+        Y = torch.empty((T, B, n), dtype=act, device=device)
+        H = torch.empty((T, B, 4 * n), dtype=act, device=device)
+        d = torch.empty((B, n), dtype=torch.float32, device=device)
+        ws = torch.empty((max(int(lib.rtn_lstm_generic_base_fwd_workspace_bytes(T, B, n, dtype, mode)), 256),), dtype=torch.uint8, device=device)
+        rc = lib.rtn_lstm_generic_base_fwd(
+            Z.data_ptr(), V_h.data_ptr(), c.data_ptr(), i.data_ptr(), Y.data_ptr(), H.data_ptr(), d.data_ptr(), T, B, n, dtype, mode,
+            ws.data_ptr(), ws.numel(), torch.cuda.current_stream(device).cuda_stream,
+        )  # fmt: skip
+    _lib.check(rc)
+    return Y, H, d
+
+
+def _lstm_low_mem_device_impl(X, W, b, y0, c0, i, start, step):
+    """``LstmLowMem`` forward on HIP tensors (returnn/native_op.py:577-836)."""
+    for t, info in zip((X, W, b, y0, c0, i), native_op.LstmLowMem.in_info):
+        _check_ndim(t, info)
+    device = X.device
+    act, dtype, mode = _act_and_mode(X, "LstmLowMem")
+    X, W, b, y0 = (t.to(act).contiguous() for t in (X, W, b, y0))
+    c0, i = (t.to(torch.float32).contiguous() for t in (c0, i))
+    T, B = i.shape
+    n = y0.shape[1]
+    n_in = X.shape[2]
+    for name, t, shape in (("X", X, (T, B, n_in)), ("W", W, (n_in + n, 4 * n)), ("b", b, (4 * n,)), ("y0", y0, (B, n)), ("c0", c0, (B, n))):
+        if tuple(t.shape) != shape:
+            raise RuntimeError("LstmLowMem: %s has shape %s, expected %s" % (name, tuple(t.shape), shape))
+        if t.device != device:
+            raise RuntimeError("LstmLowMem: %s is on %s but X is on %s" % (name, t.device, device))
+    lib = _lib.load()
+    with torch.cuda.device(device):
+        Y = torch.empty((T, B, n), dtype=act, device=device)
+        C = torch.empty((T, B, n), dtype=torch.float32, device=device)
+        d = torch.empty((B, n), dtype=torch.float32, device=device)
+        ws = torch.empty((max(int(lib.rtn_lstm_low_mem_fwd_workspace_bytes(T, B, n_in, n, dtype, mode)), 256),), dtype=torch.uint8, device=device)
+        rc = lib.rtn_lstm_low_mem_fwd(
+            X.data_ptr(), W.data_ptr(), b.data_ptr(), y0.data_ptr(), c0.data_ptr(), i.data_ptr(), int(start), int(step),
+            Y.data_ptr(), C.data_ptr(), d.data_ptr(), T, B, n_in, n, dtype, mode, ws.data_ptr(), ws.numel(),
+            torch.cuda.current_stream(device).cuda_stream,
+        )  # fmt: skip
+    _lib.check(rc)
+    return Y, C, d
 
 
 def native_lstm2_multi(calls, *, mode: Optional[str] = None):

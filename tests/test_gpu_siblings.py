@@ -1,0 +1,230 @@
+"""
+Parity of the sibling ops' forward pass on the GPU (LstmGenericBase, LstmLowMem; returnn/native_op.py:333-523, :577-836)
+with their CPU oracle, through the C ABI.
+
+Both run on the NativeLstm2 kernels with two switches: the recurrent input of a frame is the masked output of the frame
+before (no carry over masked frames), and LstmGenericBase keeps the cell state where NativeLstm2 keeps the activated
+cell input.  The masks here have holes in the middle of sequences, the only place where the switches show.
+
+Tolerances as for NativeLstm2: float32 ``rtol=1e-5, atol=2e-6``; bfloat16 ``atol=2e-2`` against the float32 oracle on the
+same float32 inputs (LstmLowMem's input projection adds two roundings to bfloat16, which is why its inputs are kept
+small enough for that bound to hold).
+"""
+
+from __future__ import annotations
+
+import numpy
+import pytest
+import torch
+from numpy.testing import assert_allclose
+
+from oracle import lstm2_oracle as oracle
+from returnn_amd import lib, native_op, torch_native_op
+from _gpu_util import announce, get_op, to_dev
+from _textbook import visited_slice
+
+pytestmark = pytest.mark.gpu
+
+F32_RTOL, F32_ATOL = 1e-5, 2e-6
+BF16_ATOL = 2e-2
+
+
+def _check(got, want, dtype, what):
+    for name, g, w in zip(what[1], got, want):
+        assert g.shape == w.shape, (what, name)
+        assert numpy.all(numpy.isfinite(g)), (what, name)
+        if dtype == "f32":
+            assert_allclose(g, w, rtol=F32_RTOL, atol=F32_ATOL, err_msg="%s %s" % (what[0], name))
+        else:
+            assert_allclose(g, w, rtol=0, atol=BF16_ATOL, err_msg="%s %s" % (what[0], name))
+
+
+def _holes(rng, T, B, p_keep=0.7):
+    return (rng.random((T, B)) < p_keep).astype(numpy.float32)
+
+
+def run_generic_base(Z, V_h, c, i, *, dtype="f32", mode="auto"):
+    get_op()  # builds the library if needed
+    op = torch_native_op.make_op(native_op.LstmGenericBase)
+    torch_native_op.OpMaker.options.setdefault("LstmGenericBase", {})["mode"] = mode
+    Y, H, d = op(to_dev(Z, dtype), to_dev(V_h, dtype), to_dev(c, "f32"), to_dev(i, "f32"))
+    torch.cuda.synchronize()
+    return tuple(t.float().cpu().numpy() for t in (Y, H, d))
+
+
+def run_low_mem(X, W, b, y0, c0, i, start=0, step=1, *, dtype="f32", mode="auto"):
+    get_op()
+    op = torch_native_op.make_op(native_op.LstmLowMem)
+    torch_native_op.OpMaker.options.setdefault("LstmLowMem", {})["mode"] = mode
+    Y, C, d = op(to_dev(X, dtype), to_dev(W, dtype), to_dev(b, dtype), to_dev(y0, dtype), to_dev(c0, "f32"), to_dev(i, "f32"), start, step)
+    torch.cuda.synchronize()
+    return tuple(t.float().cpu().numpy() for t in (Y, C, d))
+
+
+def generic_base_problem(seed, T, B, n):
+    rng = numpy.random.default_rng(seed)
+    Z = rng.normal(0, 0.5, (T, B, 4 * n)).astype(numpy.float32)
+    V = (rng.uniform(-1, 1, (n, 4 * n)) / numpy.sqrt(max(n, 1))).astype(numpy.float32)
+    c = rng.normal(0, 0.3, (B, n)).astype(numpy.float32)
+    return Z, V, c, _holes(rng, T, B)
+
+
+def low_mem_problem(seed, T, B, n_in, n):
+    rng = numpy.random.default_rng(seed)
+    X = rng.normal(0, 0.5, (T, B, n_in)).astype(numpy.float32)
+    W = (rng.uniform(-1, 1, (n_in + n, 4 * n)) / numpy.sqrt(max(n_in + n, 1))).astype(numpy.float32)
+    b = rng.normal(0, 0.2, (4 * n,)).astype(numpy.float32)
+    y0 = rng.normal(0, 0.3, (B, n)).astype(numpy.float32)
+    c0 = rng.normal(0, 0.3, (B, n)).astype(numpy.float32)
+    return X, W, b, y0, c0, _holes(rng, T, B)
+
+
+def test_low_mem_reference_closed_form():
+    """tests/test_TFNativeOp.py:264-297: one frame, one sequence, one cell, all weights 1."""
+    announce("low_mem_closed_form")
+    vX, vb, vy0, vc0 = 0.2, 0.3, 0.1, 0.1
+    ones = numpy.ones
+    Y, C, d = run_low_mem(ones((1, 1, 1)) * vX, ones((2, 4)), ones((4,)) * vb, ones((1, 1)) * vy0, ones((1, 1)) * vc0, ones((1, 1)))
+    vintern = vX + vy0 + vb
+    vgates = 1.0 / (1.0 + numpy.exp(-vintern))
+    vc = vgates * vc0 + vgates * numpy.tanh(vintern)
+    vh = vgates * numpy.tanh(vc)
+    assert Y.shape == (1, 1, 1) and C.shape == (1, 1, 1) and d.shape == (1, 1)
+    assert_allclose(Y[0, 0, 0], vh, rtol=1e-6)
+    assert_allclose(C[0, 0, 0], vc, rtol=1e-6)
+    assert_allclose(d[0, 0], vc, rtol=1e-6)
+
+
+def test_generic_base_reference_zero_run():
+    """tests/test_TFNativeOp.py:234-250: zero inputs and zero state give zero output."""
+    announce("generic_base_zero_run")
+    T, B, n = 2, 1, 3
+    z = numpy.zeros
+    Y, H, d = run_generic_base(z((T, B, 4 * n)), z((n, 4 * n)), z((B, n)), numpy.ones((T, B)))
+    assert Y.shape == (T, B, n) and numpy.abs(Y).max() == 0 and numpy.abs(d).max() == 0
+    assert_allclose(H[:, :, n:], 0.5)
+    assert numpy.abs(H[:, :, :n]).max() == 0
+
+
+SHAPES = [(1, 1, 1), (5, 3, 7), (9, 4, 33), (7, 1, 32), (6, 3, 64), (5, 17, 128), (4, 33, 64), (12, 5, 256), (40, 6, 96)]
+
+
+@pytest.mark.parametrize("T,B,n", SHAPES)
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_generic_base_shapes(T, B, n, dtype):
+    announce("generic_base_shapes", T, B, n, dtype)
+    p = generic_base_problem(300 + T + B + n, T, B, n)
+    want = oracle.lstm_generic_base_fwd(*p)
+    _check(run_generic_base(*p, dtype=dtype), want, dtype, ("LstmGenericBase %s" % ((T, B, n),), "YHd"))
+
+
+@pytest.mark.parametrize("mode", ["persistent", "graph", "stepwise"])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_generic_base_modes(mode, dtype):
+    T, B, n = 25, 9, 128
+    announce("generic_base_modes", mode, dtype)
+    p = generic_base_problem(17, T, B, n)
+    want = oracle.lstm_generic_base_fwd(*p)
+    _check(run_generic_base(*p, dtype=dtype, mode=mode), want, dtype, ("LstmGenericBase " + mode, "YHd"))
+
+
+def test_generic_base_differs_from_native_lstm2_only_on_holes():
+    """Without masked frames inside sequences and with y0 = 0 the op is NativeLstm2 (its H's first block aside)."""
+    announce("generic_base_vs_native_lstm2")
+    T, B, n = 11, 5, 64
+    Z, V, c, _ = generic_base_problem(5, T, B, n)
+    lens = numpy.array([11, 3, 7, 1, 9])
+    i = (numpy.arange(T)[:, None] < lens[None, :]).astype(numpy.float32)
+    Y, H, d = run_generic_base(Z, V, c, i)
+    Y2, C2, H2, d2 = oracle.native_lstm2_fwd(Z, V, numpy.zeros((B, n), numpy.float32), c, i, 0, 1)[:4]
+    assert_allclose(Y, Y2, rtol=F32_RTOL, atol=F32_ATOL)
+    assert_allclose(d, d2, rtol=F32_RTOL, atol=F32_ATOL)
+    assert_allclose(H[:, :, :n], C2, rtol=F32_RTOL, atol=F32_ATOL)
+    m = i[:, :, None]  # past a sequence's end the gates see different recurrent input (zero here, the carried output there)
+    assert_allclose(H[:, :, n:] * m, H2[:, :, n:] * m, rtol=F32_RTOL, atol=F32_ATOL)
+
+
+LOW_MEM_SHAPES = [(1, 1, 1, 1), (5, 3, 4, 7), (6, 2, 3, 33), (7, 1, 16, 32), (6, 3, 40, 64), (5, 17, 24, 128), (12, 5, 8, 256), (30, 6, 50, 96)]
+
+
+@pytest.mark.parametrize("T,B,n_in,n", LOW_MEM_SHAPES)
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_low_mem_shapes(T, B, n_in, n, dtype):
+    announce("low_mem_shapes", T, B, n_in, n, dtype)
+    p = low_mem_problem(400 + T + B + n + n_in, T, B, n_in, n)
+    for start, step in [(0, 1), (0, -1), (1, 2), (1, -1), (2, -2)]:
+        if start >= T or (step < 0 and T - start - 1 < start):
+            continue
+        want = oracle.lstm_low_mem_fwd(*p, start, step)
+        got = run_low_mem(*p, start, step, dtype=dtype)
+        # frames the op does not visit are unspecified in the reference (its outputs are uninitialised there)
+        sl = visited_slice(T, start, step) if step > 0 else slice(T - start - 1, start - 1 if start > 0 else None, step)
+        got = (got[0][sl], got[1][sl], got[2])
+        want = (want[0][sl], want[1][sl], want[2])
+        _check(got, want, dtype, ("LstmLowMem %s" % ((T, B, n_in, n, start, step),), "YCd"))
+
+
+@pytest.mark.parametrize("mode", ["persistent", "graph", "stepwise"])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_low_mem_modes(mode, dtype):
+    T, B, n_in, n = 25, 9, 48, 128
+    announce("low_mem_modes", mode, dtype)
+    p = low_mem_problem(23, T, B, n_in, n)
+    for start, step in [(0, 1), (0, -1)]:
+        want = oracle.lstm_low_mem_fwd(*p, start, step)
+        _check(run_low_mem(*p, start, step, dtype=dtype, mode=mode), want, dtype, ("LstmLowMem " + mode, "YCd"))
+
+
+def test_low_mem_equals_native_lstm2_on_projected_input():
+    """With no holes in the mask the op is NativeLstm2 on X.W_in + b with the recurrent rows of W."""
+    announce("low_mem_vs_native_lstm2")
+    T, B, n_in, n = 9, 4, 12, 64
+    X, W, b, y0, c0, _ = low_mem_problem(31, T, B, n_in, n)
+    lens = numpy.array([9, 2, 5, 9])
+    i = (numpy.arange(T)[:, None] < lens[None, :]).astype(numpy.float32)
+    Y, C, d = run_low_mem(X, W, b, y0, c0, i)
+    Xp = (X.astype(numpy.float64) @ W[:n_in].astype(numpy.float64) + b).astype(numpy.float32)
+    Y2, C2, _, d2 = oracle.native_lstm2_fwd(Xp, W[n_in:], y0, c0, i, 0, 1)[:4]
+    # the first frame after a sequence's end still differs (y carried there vs. zero) but is masked: Y = 0, C kept
+    assert_allclose(Y, Y2, rtol=F32_RTOL, atol=F32_ATOL)
+    assert_allclose(C, C2, rtol=F32_RTOL, atol=F32_ATOL)
+    assert_allclose(d, d2, rtol=F32_RTOL, atol=F32_ATOL)
+
+
+def test_c_abi_errors():
+    """Too small a workspace and a bad start are refused with the library's error codes; empty problems are fine."""
+    announce("siblings_c_abi_errors")
+    get_op()
+    cabi = lib.load()
+    T, B, n_in, n = 4, 2, 3, 32
+    X, W, b, y0, c0, i = (to_dev(a, "f32") for a in low_mem_problem(1, T, B, n_in, n))
+    Y = torch.empty((T, B, n), device="cuda:0")
+    C = torch.empty((T, B, n), device="cuda:0")
+    d = torch.empty((B, n), device="cuda:0")
+    need = cabi.rtn_lstm_low_mem_fwd_workspace_bytes(T, B, n_in, n, lib.DTYPE_F32, 0)
+    assert need > 0
+    ws = torch.empty((need,), dtype=torch.uint8, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    args = (X.data_ptr(), W.data_ptr(), b.data_ptr(), y0.data_ptr(), c0.data_ptr(), i.data_ptr())
+    outs = (Y.data_ptr(), C.data_ptr(), d.data_ptr())
+    rc = cabi.rtn_lstm_low_mem_fwd(*args, 0, 1, *outs, T, B, n_in, n, lib.DTYPE_F32, 0, ws.data_ptr(), need - 1, stream)
+    assert rc == lib.RTN_ERR_WORKSPACE and b"workspace" in cabi.rtn_last_error()
+    rc = cabi.rtn_lstm_low_mem_fwd(*args, T, 1, *outs, T, B, n_in, n, lib.DTYPE_F32, 0, ws.data_ptr(), need, stream)
+    assert rc == lib.RTN_ERR_RANGE
+    rc = cabi.rtn_lstm_low_mem_fwd(*args, 0, 0, *outs, T, B, n_in, n, lib.DTYPE_F32, 0, ws.data_ptr(), need, stream)
+    assert rc == lib.RTN_ERR_RANGE
+    rc = cabi.rtn_lstm_low_mem_fwd(*args, 2, -1, *outs, T, B, n_in, n, lib.DTYPE_F32, 0, ws.data_ptr(), need, stream)
+    assert rc == lib.RTN_ERR_RANGE and b"visits no frame" in cabi.rtn_last_error()  # would run from frame 1 down to frame 2
+    rc = cabi.rtn_lstm_low_mem_fwd(*args, 0, 1, *outs, T, B, n_in, n, lib.DTYPE_F32, 0, ws.data_ptr(), need, stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    Z, V, c, i2 = (to_dev(a, "f32") for a in generic_base_problem(2, T, B, n))
+    H = torch.empty((T, B, 4 * n), device="cuda:0")
+    need = cabi.rtn_lstm_generic_base_fwd_workspace_bytes(T, B, n, lib.DTYPE_F32, 0)
+    ws = torch.empty((need,), dtype=torch.uint8, device="cuda:0")
+    gargs = (Z.data_ptr(), V.data_ptr(), c.data_ptr(), i2.data_ptr(), Y.data_ptr(), H.data_ptr(), d.data_ptr())
+    rc = cabi.rtn_lstm_generic_base_fwd(*gargs, T, B, n, lib.DTYPE_F32, 0, ws.data_ptr(), need - 1, stream)
+    assert rc == lib.RTN_ERR_WORKSPACE
+    rc = cabi.rtn_lstm_generic_base_fwd(*gargs, T, B, n, lib.DTYPE_F32, 0, ws.data_ptr(), need, stream)
+    assert rc == 0
+    torch.cuda.synchronize()
