@@ -314,6 +314,140 @@ def bench_gradient(args, dev, cabi):
     return result
 
 
+def cpu_baseline_sibling(name: str, op: str, n_in: int, target_seconds: float = 15.0):
+    """Times the CPU restatement of a sibling op (plain loops, one thread) on the first frames of the workload."""
+    import numpy
+
+    from oracle import lstm2_oracle
+    from returnn_amd import synthetic
+
+    full_T = synthetic.make_config.__globals__["_SPECS"][name]["T"]
+    T = 2
+    rng = numpy.random.default_rng(2)
+    for attempt in range(2):
+        p = synthetic.make_config(name, T=T)
+        if op == "generic_base":
+            run = lambda: lstm2_oracle.lstm_generic_base_fwd(p.X, p.W, p.c0, p.i)  # noqa: E731
+        else:
+            Xr = rng.standard_normal((p.T, p.B, n_in), dtype=numpy.float32)
+            Ws = numpy.concatenate([rng.standard_normal((n_in, 4 * p.n), dtype=numpy.float32) * 0.02, p.W], axis=0)
+            b = numpy.zeros((4 * p.n,), numpy.float32)
+            run = lambda: lstm2_oracle.lstm_low_mem_fwd(Xr, Ws, b, p.y0, p.c0, p.i, 0, 1)  # noqa: E731
+        t0 = time.perf_counter()
+        run()
+        dt = time.perf_counter() - t0
+        if attempt == 0:
+            T = int(max(T, min(full_T, target_seconds / max(dt / T, 1e-9))))
+    return {
+        "value": p.T * p.B / dt,
+        "unit": "timesteps*seqs/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": "%s forward, %s shape in fp32, first T=%i of %i frames (B=%i, n=%i%s), one pass, %.1f s, plain C loops on one thread"
+        % (op, name, p.T, full_T, p.B, p.n, ", n_in=%i" % n_in if op == "low_mem" else "", dt),
+    }
+
+
+def bench_sibling(args, dev, cabi):
+    """
+    Forward pass of a sibling op on the workload's shape, inputs resident in HBM.  ``generic_base``: LstmGenericBase on the
+    workload's gate inputs (8 n^2 flops per timestep x sequence).  ``low_mem``: LstmLowMem on raw input of width n_in = n
+    with the stacked weight matrix (8 n^2 recurrent + 8 n_in n projection flops per unit).
+    """
+    import torch
+
+    from returnn_amd import lib, synthetic
+
+    p = synthetic.make_config(args.workload)
+    T, B, n = p.T, p.B, p.n
+    n_in = n
+    dtype = p.dtype
+    act = torch.bfloat16 if dtype == "bf16" else torch.float32
+    dt_code = lib.DTYPE_BF16 if dtype == "bf16" else lib.DTYPE_F32
+    mode = lib.MODES[args.mode]
+    W = torch.from_numpy(p.W).to(dev).to(act)
+    y0 = torch.from_numpy(p.y0).to(dev).to(act)
+    c0 = torch.from_numpy(p.c0).to(dev)
+    msk = torch.from_numpy(p.i).to(dev)
+    Y = torch.empty((T, B, n), dtype=act, device=dev)
+    d = torch.empty((B, n), dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    if args.op == "generic_base":
+        Z = torch.from_numpy(p.X).to(dev).to(act)
+        H = torch.empty((T, B, 4 * n), dtype=act, device=dev)
+        ws = torch.empty((max(cabi.rtn_lstm_generic_base_fwd_workspace_bytes(T, B, n, dt_code, mode), 256),), dtype=torch.uint8, device=dev)
+        flops = 8.0 * n * n * T * B
+
+        def call():
+            lib.check(cabi.rtn_lstm_generic_base_fwd(
+                Z.data_ptr(), W.data_ptr(), c0.data_ptr(), msk.data_ptr(), Y.data_ptr(), H.data_ptr(), d.data_ptr(), T, B, n, dt_code, mode,
+                ws.data_ptr(), ws.numel(), stream.cuda_stream))  # fmt: skip
+
+        what = "LstmGenericBase forward"
+    else:
+        gen = torch.Generator(device=dev).manual_seed(0)
+        Xr = torch.randn((T, B, n_in), device=dev, generator=gen).to(act)
+        Wff = (torch.randn((n_in, 4 * n), device=dev, generator=gen) * 0.02).to(act)
+        Ws = torch.cat([Wff, W], dim=0).contiguous()
+        b = torch.zeros((4 * n,), dtype=act, device=dev)
+        C = torch.empty((T, B, n), dtype=torch.float32, device=dev)
+        ws = torch.empty((max(cabi.rtn_lstm_low_mem_fwd_workspace_bytes(T, B, n_in, n, dt_code, mode), 256),), dtype=torch.uint8, device=dev)
+        flops = (8.0 * n * n + 8.0 * n_in * n) * T * B
+
+        def call():
+            lib.check(cabi.rtn_lstm_low_mem_fwd(
+                Xr.data_ptr(), Ws.data_ptr(), b.data_ptr(), y0.data_ptr(), c0.data_ptr(), msk.data_ptr(), 0, 1, Y.data_ptr(), C.data_ptr(),
+                d.data_ptr(), T, B, n_in, n, dt_code, mode, ws.data_ptr(), ws.numel(), stream.cuda_stream))  # fmt: skip
+
+        what = "LstmLowMem forward, n_in=%i" % n_in
+    for _ in range(args.warmup):
+        call()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        call()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    lib.check(cabi.rtn_native_lstm2_fwd_status(ws.data_ptr(), stream.cuda_stream))
+    assert bool(torch.isfinite(Y.float()).all()) and bool(torch.isfinite(d).all())
+    call_ms = elapsed * 1e3 / args.steps
+    peak = PEAK_MFMA[dtype]
+    result = {
+        "metric": "%s timesteps*seqs/sec (T*B/s) at n=%i" % (what.split(",")[0], n),
+        "value": T * B * args.steps / elapsed,
+        "unit": "timesteps*seqs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": call_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype,
+        "data": "synthetic",
+        "config": {
+            "workload": "%s: %s, T=%i B=%i n=%i %s, ragged=%s" % (args.workload, what, T, B, n, dtype, p.lens is not None),
+            "calls_per_step": 1,
+            "units_per_step": T * B,
+            "mode": args.mode,
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": flops / (call_ms * 1e-3) / 1e12,
+            "peak": peak / 1e12,
+            "unit": "TFLOP/s",
+            "frac": flops / (call_ms * 1e-3) / peak,
+            "traffic": None,
+            "kernel": "whole call: the NativeLstm2 forward kernel with the sibling op's switches"
+            + ("" if args.op == "generic_base" else ", after the rocBLAS projection GEMM and the bias kernel"),
+            "launch_ms": call_ms,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline_sibling(args.workload, args.op, n_in, args.cpu_seconds)
+    return result
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -324,9 +458,9 @@ def main():
     ap.add_argument("--pair", default="fused", choices=["fused", "separate"],
                     help="cfg3: issue the two directions through the multi-call entry (one launch when the device "
                          "holds both; default) or as two separate op calls")
-    ap.add_argument("--op", default="fwd", choices=["fwd", "bwd"],
+    ap.add_argument("--op", default="fwd", choices=["fwd", "bwd", "generic_base", "low_mem"],
                     help="fwd: the forward op (default, the headline metric); bwd: the gradient op of one direction of "
-                         "the workload (cfg1/cfg2/cfg3/cfg5)")
+                         "the workload (cfg1/cfg2/cfg3/cfg5); generic_base, low_mem: forward of the sibling ops on the workload's shape")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -356,6 +490,9 @@ def main():
         return
     if args.op == "bwd":
         print(json.dumps(bench_gradient(args, dev, cabi)))
+        return
+    if args.op in ("generic_base", "low_mem"):
+        print(json.dumps(bench_sibling(args, dev, cabi)))
         return
 
     p = synthetic.make_config(args.workload)
