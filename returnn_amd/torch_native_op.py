@@ -89,6 +89,7 @@ class OpMaker:
         return "%s(%s) -> (%s)" % (self.op_name, args, rets)
 
     def _impl_for(self):
+        _lib.load()  # fail now, loudly, if the HIP library is not there
         impl = {
             "rtn_native_lstm2_fwd": _native_lstm2_device_impl,
             "rtn_lstm_generic_base_fwd": _lstm_generic_base_device_impl,
@@ -104,7 +105,6 @@ class OpMaker:
                 self.options.setdefault(self.cache_key, {})["mode"] = self.mode or "auto"
             if self.cache_key in self.op_cache:
                 return self.op_cache[self.cache_key]
-            _lib.load()  # fail now, loudly, if the HIP library is not there
             impl = self._impl_for()
             tlib = torch.library.Library(self.op_name, "DEF")
             tlib.define(self.schema())
@@ -134,12 +134,60 @@ class OpMaker:
         torch.library.register_fake("%s::%s" % (self.op_name, self.op_name), _fake_impl)
 
 
+class CompiledOpMaker(OpMaker):
+    """
+    An op given as source in the native-op dialect (``c_fw_code`` ...): compiled with hipcc by
+    :mod:`returnn_amd.op_loader` and registered like the prebuilt ones.  Stands in for the reference's code-generating
+    OpMaker (returnn/torch/util/native_op.py:27-447) on ROCm.
+    """
+
+    def __init__(self, cls, *, compiler_opts: Optional[Dict[str, Any]] = None, with_cuda: Optional[bool] = None):
+        """
+        :param cls: description class or object with in_info, out_info, c_fw_code, c_extra_support_code, code_version
+        :param compiler_opts: passed to :class:`returnn_amd.op_loader.HipOpCodeCompiler` (``cache_dir``, ``extra_flags``, ...)
+        :param with_cuda: accepted for signature compatibility; the device path is always HIP
+        """
+        from . import op_loader
+
+        del with_cuda
+        self.compiled = op_loader.CompiledOp(*op_loader.description_fields(cls), compiler_opts=compiler_opts)
+        description = OpDescription(
+            in_info=self.compiled.in_info, out_info=self.compiled.out_info, c_abi_fw=self.compiled.name + "_fw", name=self.compiled.name
+        )
+        super().__init__(description)
+
+    def _impl_for(self):
+        compiled = self.compiled
+        compiled.lib()  # compile (if needed) and load now; a compiler error surfaces here
+
+        def _compiled_op_impl(*args):
+            return compiled(*args)
+
+        return _compiled_op_impl
+
+    def _register_fake_impl(self):
+        description = self.description
+        dtype_map = {"float32": torch.float32, "int32": torch.int32}
+
+        def _fake_impl(*args):
+            device = next(a.device for a in args if isinstance(a, torch.Tensor))
+            shapes = description.infer_shape(None, [tuple(a.shape) if isinstance(a, torch.Tensor) else () for a in args])
+            return tuple(
+                torch.empty(shape, dtype=dtype_map[o.get("dtype", "float32")], device=device) for o, shape in zip(description.out_info, shapes)
+            )
+
+        torch.library.register_fake("%s::%s" % (self.op_name, self.op_name), _fake_impl)
+
+
 def make_op(cls, **kwargs):
     """
-    :param type[returnn_amd.native_op.NativeOpGenBase] cls: e.g. :class:`returnn_amd.native_op.NativeLstm2`
-    :param kwargs: passed to :class:`OpMaker`
-    :return: op, ``(X, W, y0, c0, i, start, step) -> (Y, C, H, d)``
+    :param type[returnn_amd.native_op.NativeOpGenBase] cls: e.g. :class:`returnn_amd.native_op.NativeLstm2`, or a
+        description that carries source in the native-op dialect (``c_fw_code``) instead of naming a prebuilt entry point
+    :param kwargs: passed to :class:`OpMaker` / :class:`CompiledOpMaker`
+    :return: op, e.g. ``(X, W, y0, c0, i, start, step) -> (Y, C, H, d)``
     """
+    if not getattr(cls, "c_abi_fw", None) and getattr(cls, "c_fw_code", None):
+        return CompiledOpMaker(cls, **kwargs).make_op()
     maker = OpMaker(OpDescription.from_gen_base(cls), **kwargs)
     return maker.make_op()
 
