@@ -106,6 +106,49 @@ def cpu_baseline(name: str, target_seconds: float = 15.0):
     }
 
 
+def torch_stack_baseline(prob, dev, steps, warmup):
+    """
+    The same encoder forward through PyTorch's own LSTM (MIOpen on ROCm) on the same GPU: the route the reference's
+    torch backend takes for an LSTM layer (pack_padded_sequence -> torch.lstm -> pad_packed_sequence,
+    returnn/torch/frontend/_backend.py:2795-2822), here in its most favourable form, one bidirectional multi-layer call.
+    Random weights of the same shapes (timing only).  ``packed``: the lengths are honoured, as the reference needs them;
+    ``padded``: lengths ignored (not the same function, but the fastest the library can go on this shape).
+    """
+    import torch
+
+    T, B, n, L, d_in = prob.T, prob.B, prob.n, prob.num_layers, prob.in_dim
+    lens_cpu = torch.from_numpy(prob.lens).to(torch.int64)
+    out = {"what": "torch.nn.LSTM(num_layers=%i, bidirectional=True), same shapes, same GPU; ms per forward" % L}
+    for dtype in (torch.bfloat16, torch.float16):
+        name = str(dtype).replace("torch.", "")
+        try:
+            net = torch.nn.LSTM(d_in, n, num_layers=L, bidirectional=True).to(dev).to(dtype).eval()
+            x = torch.from_numpy(prob.features).to(dev).to(dtype)
+
+            def run_packed():
+                packed = torch.nn.utils.rnn.pack_padded_sequence(x, lens_cpu, enforce_sorted=False)
+                return torch.nn.utils.rnn.pad_packed_sequence(net(packed)[0], total_length=T)[0]
+
+            def run_padded():
+                return net(x)[0]
+
+            for kind, run in (("packed", run_packed), ("padded", run_padded)):
+                with torch.no_grad():
+                    for _ in range(max(warmup, 1)):
+                        y = run()
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    for _ in range(steps):
+                        y = run()
+                    torch.cuda.synchronize()
+                    out["%s_%s_ms" % (kind, name)] = (time.perf_counter() - t0) * 1e3 / steps
+                assert tuple(y.shape) == (T, B, 2 * n)
+            del net, x, y
+        except Exception as exc:  # a dtype the library does not take
+            out["error_%s" % name] = "%s: %s" % (type(exc).__name__, str(exc)[:200])
+    return out
+
+
 def bench_encoder(args, dev):
     """
     Config 4: forward of the 6-layer bidirectional encoder (per layer one projection GEMM and one op call per
@@ -148,8 +191,10 @@ def bench_encoder(args, dev):
         proj = time.perf_counter() - t1
     step_ms = elapsed * 1e3 / args.steps
     proj_ms = proj * 1e3 / args.steps
+    del enc, y, srcs, ws
+    torch_stack = None if args.no_torch_baseline else torch_stack_baseline(prob, dev, max(2, args.steps // 4), 1)
     rec_flops = 2 * L * 8.0 * T * B * n * n
-    proj_flops = 2 * sum(2.0 * T * B * (enc.in_dim if li == 0 else 2 * n) * 4 * n for li in range(L))
+    proj_flops = 2 * sum(2.0 * T * B * (prob.in_dim if li == 0 else 2 * n) * 4 * n for li in range(L))
     units = 2 * L * T * B
     return {
         "metric": "LSTM fwd timesteps*seqs/sec (T*B/s) at n=%i" % n,
@@ -166,11 +211,12 @@ def bench_encoder(args, dev):
         "data": "synthetic",
         "config": {
             "workload": "cfg4: %i-layer bidirectional LSTM encoder forward, T=%i B=%i in=%i n=%i bf16, ragged=True; "
-            "per layer and direction one projection GEMM and one NativeLstm2 call" % (L, T, B, enc.in_dim, n),
+            "per layer and direction one projection GEMM and one NativeLstm2 call" % (L, T, B, prob.in_dim, n),
             "calls_per_step": 2 * L,
             "units_per_step": units,
             "projection_ms_per_step": proj_ms,
             "recurrent_and_glue_ms_per_step": step_ms - proj_ms,
+            "torch_lstm_same_gpu": torch_stack,
         },
         "roofline": {
             "bound": "mfma",
@@ -462,6 +508,7 @@ def main():
                     help="fwd: the forward op (default, the headline metric); bwd: the gradient op of one direction of "
                          "the workload (cfg1/cfg2/cfg3/cfg5); generic_base, low_mem: forward of the sibling ops on the workload's shape")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-torch-baseline", action="store_true", help="cfg4: skip timing the same stack through torch.nn.LSTM")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a kernel of known traffic, to scale "
