@@ -192,6 +192,59 @@ def make_op(cls, **kwargs):
     return maker.make_op()
 
 
+def make_op_with_grad(cls, **kwargs):
+    """
+    A differentiable callable for a description in the native-op dialect that carries ``c_bw_code``: forward = the
+    compiled op, backward = its compiled gradient op ``GradOf<name>``, wired through ``torch.autograd.Function``.
+    The reference's torch OpMaker stops short of this (returnn/torch/util/native_op.py:444-445); the rule that derives
+    the gradient op and maps its results back onto the inputs is the backend-neutral one of returnn/native_op.py:
+    189-252.
+
+    :param cls: description with in_info, out_info, c_fw_code, c_bw_code (and grad_input_map, c_extra_support_code)
+    :param kwargs: passed to :class:`CompiledOpMaker` for both ops
+    :return: function ``(*inputs) -> tuple of outputs`` (dummy outputs of ``want_inplace="dummy_out"`` included)
+    """
+    from . import op_loader
+
+    grad_cls = op_loader.grad_description(cls)
+    if grad_cls is None:
+        raise ValueError("%s has no c_bw_code" % getattr(cls, "__name__", cls))
+    fw_op = make_op(cls, **kwargs)
+    bw_op = make_op(grad_cls, **kwargs)
+    in_info = tuple(cls.in_info)
+    n_in = len(in_info)
+    n_out_declared = len(cls.out_info)
+    gi_map = grad_cls.grad_input_map_resolved
+    connected = [v.get("gradient", "") != "disconnected" for v in in_info]
+
+    class _Function(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, *inputs):
+            outs = fw_op(*inputs)
+            ctx.inputs = inputs
+            ctx.outs = outs[:n_out_declared]
+            for v, o in zip(cls.out_info, outs):
+                if v.get("gradient", "") == "disconnected":
+                    ctx.mark_non_differentiable(o)
+            return tuple(outs)
+
+        @staticmethod
+        def backward(ctx, *grad_outs):
+            grads = [g if g is not None else torch.zeros_like(o) for g, o in zip(grad_outs[:n_out_declared], ctx.outs)]
+            pool = list(ctx.inputs) + list(ctx.outs) + grads
+            results = list(bw_op(*[pool[k] for k in gi_map]))
+            per_input = []
+            for k in range(n_in):  # returnn/native_op.py:228-252
+                per_input.append(results.pop(0) if connected[k] else None)
+            return tuple(g if (g is None or isinstance(ctx.inputs[k], torch.Tensor)) else None for k, g in enumerate(per_input))
+
+    def op(*inputs):
+        return _Function.apply(*inputs)
+
+    op.forward_op, op.gradient_op = fw_op, bw_op
+    return op
+
+
 def _cpu_not_supported(name):
     def _impl(*args):
         raise RuntimeError(

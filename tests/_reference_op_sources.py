@@ -1,8 +1,9 @@
 """
 Reads the op descriptions of the reference's returnn/native_op.py as TEXT: the file is parsed with :mod:`ast` and the
-class attributes ``in_info``, ``out_info``, ``c_fw_code``, ``c_extra_support_code``, ``code_version`` are evaluated by a
-tiny evaluator that knows literals, names of module-level literals, ``copy.copy(x)``, ``Class.attr``, subscripts and
-``x.update({...})``.  Nothing of the reference is imported or executed, and nothing is written into this repository: the
+class attributes ``in_info``, ``out_info``, ``c_fw_code``, ``c_bw_code``, ``c_extra_support_code``, ``code_version`` are
+evaluated by a tiny evaluator that knows literals, names of module-level literals, ``copy.copy(x)``, ``Class.attr``,
+subscripts and ``x.update({...})``; a ``grad_input_map`` method that returns some of its arguments is read as the tuple
+of their positions.  Nothing of the reference is imported or executed, and nothing is written into this repository: the
 descriptions are handed to the HIP op loader with a temporary cache directory, to check that the reference's op sources
 compile against this package's dialect header.
 """
@@ -15,7 +16,7 @@ import os
 from typing import Any, Dict
 
 REFERENCE_NATIVE_OP = "/root/reference/returnn/native_op.py"
-FIELDS = ("in_info", "out_info", "c_fw_code", "c_extra_support_code", "code_version")
+FIELDS = ("in_info", "out_info", "c_fw_code", "c_bw_code", "c_extra_support_code", "code_version", "grad_input_map")
 
 
 class NotStatic(Exception):
@@ -79,6 +80,12 @@ def read_descriptions(path: str = REFERENCE_NATIVE_OP):
                 if isinstance(st, ast.Assign) and len(st.targets) == 1 and isinstance(st.targets[0], ast.Name):
                     if st.targets[0].id in FIELDS:
                         local[st.targets[0].id] = _eval(st.value, module_env, classes, local)
+                elif isinstance(st, ast.FunctionDef) and st.name == "grad_input_map":
+                    names = [a.arg for a in st.args.args][1:]  # without cls
+                    returns = [b for b in st.body if isinstance(b, ast.Return)]
+                    if len(returns) != 1 or not isinstance(returns[0].value, ast.Tuple):
+                        raise NotStatic("grad_input_map body")
+                    local["grad_input_map"] = tuple(names.index(e.id) for e in returns[0].value.elts)
                 elif (
                     isinstance(st, ast.Expr)
                     and isinstance(st.value, ast.Call)

@@ -11,16 +11,19 @@ class ElmanScan:
     """
     h_t = tanh(x_t + h_{t-1} W) where the mask is 1, h_{t-1} where it is 0; frames start, start+step, ... as NativeLstm2
     counts them.  Exercises: host int32 scalars, device_malloc/free, Ndarray_memcpy, data_ptr, affine_raw (rocBLAS),
-    start_dev_kernel with the default launch shape, assert_cmp, HANDLE_LAST_ERROR.
+    start_dev_kernel with the default launch shape, assert_cmp, HANDLE_LAST_ERROR; with its gradient code: the derivation
+    of the gradient op (grad_input_map as a callable that drops X and hT, bw_out_var giving DX its shape from Y,
+    disconnected inputs) and affine_raw with transposed operands.
     """
 
     in_info = (
-        {"name": "X", "ndim": 3, "shape": (None, None, None), "need_contiguous": True},
+        # the gradient op does not take X (see grad_input_map): DX gets its shape from Y, input 5 of the gradient op
+        {"name": "X", "ndim": 3, "shape": (None, None, None), "need_contiguous": True, "bw_out_var": {"shape": ((5, 0), (5, 1), (5, 2))}},
         {"name": "W", "ndim": 2, "shape": (None, None), "need_contiguous": True},
         {"name": "h0", "ndim": 2, "shape": (None, None), "need_contiguous": True},
-        {"name": "i", "ndim": 2, "shape": (None, None), "need_contiguous": True},
-        {"name": "start", "ndim": 0, "shape": (), "dtype": "int32", "host_memory": True},
-        {"name": "step", "ndim": 0, "shape": (), "dtype": "int32", "host_memory": True},
+        {"name": "i", "ndim": 2, "shape": (None, None), "need_contiguous": True, "gradient": "disconnected"},
+        {"name": "start", "ndim": 0, "shape": (), "dtype": "int32", "host_memory": True, "gradient": "disconnected"},
+        {"name": "step", "ndim": 0, "shape": (), "dtype": "int32", "host_memory": True, "gradient": "disconnected"},
     )
     out_info = (
         {"name": "Y", "ndim": 3, "shape": ((0, 0), (0, 1), (0, 2))},
@@ -32,6 +35,17 @@ class ElmanScan:
           for (long k = threadIdx.x + (long)blockDim.x * blockIdx.x; k < rows * width; k += (long)gridDim.x * blockDim.x) {
             const float keep = mask_row[k / width];
             out[k] = keep * tanhf(pre[k]) + (1.f - keep) * carry[k];
+          }
+        }
+        """,
+        "20_cell_grad": """
+        DEF_KERNEL void elman_cell_grad(long rows, long width, const float* y, const float* dy, const float* carry, const float* mask_row,
+                                        float* g, float* passed) {
+          for (long k = threadIdx.x + (long)blockDim.x * blockIdx.x; k < rows * width; k += (long)gridDim.x * blockDim.x) {
+            const float keep = mask_row[k / width];
+            const float total = dy[k] + carry[k];
+            g[k] = keep * (1.f - y[k] * y[k]) * total;
+            passed[k] = (1.f - keep) * total;
           }
         }
         """,
@@ -73,7 +87,56 @@ class ElmanScan:
         device_free(carry);
         device_free(pre);
     """
-    code_version = (1,)
+
+    # noinspection PyPep8Naming
+    @staticmethod
+    def grad_input_map(X, W, h0, i, start, step, Y, hT, DY, DhT):
+        del X, hT
+        return W, h0, i, start, step, Y, DY, DhT
+
+    c_bw_code = """
+        Ndarray* W = inputs[0];
+        Ndarray* h0 = inputs[1];
+        Ndarray* mask = inputs[2];
+        int first = Ndarray_DEV_DATA_int32_scalar(inputs[3]);
+        const int stride = Ndarray_DEV_DATA_int32_scalar(inputs[4]);
+        Ndarray* Y = inputs[5];
+        Ndarray* DY = inputs[6];
+        Ndarray* DhT = inputs[7];
+        Ndarray* DX = *outputs[0];
+        Ndarray* DW = *outputs[1];
+        Ndarray* Dh0 = *outputs[2];
+        const long frames = Ndarray_DIMS(Y)[0];
+        const int rows = (int) Ndarray_DIMS(Y)[1], width = (int) Ndarray_DIMS(Y)[2];
+        assert_cmp(Ndarray_DIMS(DX)[0], ==, frames);
+        assert_cmp(Ndarray_DIMS(DW)[0], ==, width);
+        assert_cmp(Ndarray_DIMS(Dh0)[1], ==, width);
+        assert_cmp(stride, !=, 0);
+        assert_cmp(first, >=, 0);
+        assert_cmp(first, <, frames);
+        long visited;
+        if (stride > 0) visited = (frames - 1 - first) / stride + 1;
+        else { first = (int) frames - 1 - first; visited = first / (-stride) + 1; }
+        const size_t state_bytes = sizeof(float) * rows * width;
+        float* carry = (float*) device_malloc(state_bytes);   // error arriving from the frames after this one
+        float* passed = (float*) device_malloc(state_bytes);  // the part that skips a masked frame
+        Ndarray_memcpy(carry, Ndarray_DEV_DATA(DhT), state_bytes);
+        for (long k = visited - 1; k >= 0; --k) {
+          const long t = first + k * stride;
+          float* g = data_ptr(DX, (int) t);
+          start_dev_kernel(elman_cell_grad, (rows, width, data_ptr(Y, (int) t), data_ptr(DY, (int) t), carry,
+                                             Ndarray_DEV_DATA(mask) + t * rows, g, passed));
+          HANDLE_LAST_ERROR();
+          float* before = (k == 0) ? Ndarray_DEV_DATA(h0) : data_ptr(Y, (int) (t - stride));
+          affine_raw(before, rows, width, g, rows, width, Ndarray_DEV_DATA(DW), width, width, true, false);  // DW += before^T . g
+          Ndarray_memcpy(carry, passed, state_bytes);
+          affine_raw(g, rows, width, Ndarray_DEV_DATA(W), width, width, carry, rows, width, false, true);    // carry += g . W^T
+        }
+        Ndarray_memcpy(Ndarray_DEV_DATA(Dh0), carry, state_bytes);
+        device_free(passed);
+        device_free(carry);
+    """
+    code_version = (2,)
 
 
 class RowLogSumExp:

@@ -190,3 +190,51 @@ def test_c_abi_with_the_library_allocator():
     Y2, h2 = elman_numpy(X, W, h0, mask, 0, 1)
     assert_allclose(Yh, Y2, rtol=1e-4, atol=1e-5)
     assert_allclose(hTh, h2, rtol=1e-4, atol=1e-5)
+
+
+def elman_torch(X, W, h0, mask, start, step):
+    """The scan in differentiable torch float64 (CPU): autograd through it is the independent check of c_bw_code."""
+    T = X.shape[0]
+    ys = [torch.zeros_like(X[0]) for _ in range(T)]
+    h = h0
+    t = start if step > 0 else T - 1 - start
+    while 0 <= t < T:
+        m = mask[t][:, None]
+        h = m * torch.tanh(X[t] + h @ W) + (1 - m) * h
+        ys[t] = h
+        t += step
+    return torch.stack(ys), h
+
+
+@pytest.mark.parametrize("start,step", [(0, 1), (0, -1), (1, 2)])
+def test_gradient_op_through_autograd(start, step):
+    """make_op_with_grad: forward op + derived gradient op under torch.autograd, against autograd through plain torch."""
+    announce("op_loader gradient", start, step)
+    rng = numpy.random.default_rng(21)
+    T, B, n = 9, 4, 24
+    X = rng.normal(0, 0.5, (T, B, n))
+    W = rng.uniform(-1, 1, (n, n)) / numpy.sqrt(n)
+    h0 = rng.normal(0, 0.3, (B, n))
+    mask = (rng.random((T, B)) < 0.7).astype(numpy.float64)
+    R1, R2 = rng.normal(0, 1, (T, B, n)), rng.normal(0, 1, (B, n))
+    ref = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (X, W, h0)]
+    Yr, hr = elman_torch(ref[0], ref[1], ref[2], torch.tensor(mask), start, step)
+    ((Yr * torch.tensor(R1)).sum() + (hr * torch.tensor(R2)).sum()).backward()
+
+    op = torch_native_op.make_op_with_grad(dialect_ops.ElmanScan)
+    got = [dev(a).requires_grad_(True) for a in (X, W, h0)]
+    Y, hT = op(got[0], got[1], got[2], dev(mask), start, step)
+    ((Y * dev(R1)).sum() + (hT * dev(R2)).sum()).backward()
+    torch.cuda.synchronize()
+    assert_allclose(Y.detach().cpu().numpy(), Yr.detach().numpy(), rtol=1e-4, atol=1e-5)
+    for name, g, r in zip(("DX", "DW", "Dh0"), got, ref):
+        scale = float(r.grad.abs().max())
+        assert_allclose(g.grad.cpu().numpy(), r.grad.numpy(), rtol=0, atol=2e-5 * max(scale, 1.0), err_msg=name)
+    # an output nobody differentiates gets a zero gradient: only hT contributes
+    got2 = [dev(a).requires_grad_(True) for a in (X, W, h0)]
+    _, hT2 = op(got2[0], got2[1], got2[2], dev(mask), start, step)
+    (hT2 * dev(R2)).sum().backward()
+    ref2 = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (X, W, h0)]
+    (elman_torch(ref2[0], ref2[1], ref2[2], torch.tensor(mask), start, step)[1] * torch.tensor(R2)).sum().backward()
+    torch.cuda.synchronize()
+    assert_allclose(got2[1].grad.cpu().numpy(), ref2[1].grad.numpy(), rtol=0, atol=2e-5 * max(float(ref2[1].grad.abs().max()), 1.0))

@@ -58,6 +58,24 @@ def test_want_inplace_dummy_out():
     assert dialect_ops.BucketSum.in_info[1]["want_inplace"] == "dummy_out"  # the description itself is untouched
 
 
+def test_grad_description():
+    """Derivation of the gradient op from a description with c_bw_code (rules of returnn/native_op.py:112-127, 165-226)."""
+    g = op_loader.grad_description(dialect_ops.ElmanScan)
+    assert g.__name__ == "GradOfElmanScan"
+    assert [v["name"] for v in g.in_info] == ["W", "h0", "i", "start", "step", "Y", "D_Y", "D_hT"]  # X and hT dropped by the map
+    assert g.grad_input_map_resolved == (1, 2, 3, 4, 5, 6, 8, 9)
+    assert [v["name"] for v in g.out_info] == ["X", "W", "h0"]  # mask, start and step are disconnected
+    assert g.out_info[0]["shape"] == ((5, 0), (5, 1), (5, 2))  # bw_out_var: from Y, input 5 of the gradient op
+    assert g.out_info[1]["shape"] == ((0, 0), (0, 1)) and g.out_info[2]["shape"] == ((1, 0), (1, 1))
+    assert g.c_fw_code is dialect_ops.ElmanScan.c_bw_code
+    assert op_loader.grad_description(dialect_ops.RowLogSumExp) is None
+    # default map: everything; an input whose gradient needs its shape must then be there
+    assert op_loader.convert_grad_input_map(None, 4) == (0, 1, 2, 3)
+    no_x = type("NoX", (), dict(vars(dialect_ops.ElmanScan), in_info=tuple({k: v for k, v in d.items() if k != "bw_out_var"} for d in dialect_ops.ElmanScan.in_info)))
+    with pytest.raises(ValueError, match="grad_input_map drops that input"):
+        op_loader.grad_description(no_x)
+
+
 def test_compile_cache(tmp_path):
     opts = {"cache_dir": str(tmp_path)}
     op = op_loader.compile_op(Tiny, compiler_opts=opts)
@@ -85,7 +103,9 @@ def test_compile_error_is_reported(tmp_path):
 @pytest.fixture(scope="module")
 def built_ops():
     """The test ops in the in-tree cache: what the GPU tests load.  Compiled here if this tree has not built them yet."""
-    return {cls.__name__: op_loader.compile_op(cls) for cls in dialect_ops.ALL_OPS}
+    ops = {cls.__name__: op_loader.compile_op(cls) for cls in dialect_ops.ALL_OPS}
+    ops["GradOfElmanScan"] = op_loader.compile_op(op_loader.grad_description(dialect_ops.ElmanScan))
+    return ops
 
 
 def test_compiled_ops_export_the_c_abi(built_ops):
@@ -153,6 +173,7 @@ def test_reference_op_sources_compile_for_gfx950(tmp_path):
     classes, skipped = ref_sources.read_descriptions()
     assert not skipped, skipped
     assert len(classes) >= 20
+    n_forward = len(classes)
     expected_failures = {"TwoDLSTM", "MultiEndFastBaumWelchOp", "SegmentFastBaumWelchOp"}
     # SegmentFastBaumWelchOp completes its code in its constructor (returnn/native_op.py:4914-4946); these are the lines a
     # default-constructed instance gets
@@ -162,6 +183,16 @@ def test_reference_op_sources_compile_for_gfx950(tmp_path):
         "const bool segmentwise_normalization = false;\nconst bool dump_targets = false;\nconst unsigned dump_targets_interval = 0;\n"
         + segment["c_fw_code"]
     )
+
+    # the gradient ops: derived from c_bw_code and grad_input_map by the loader's own rule
+    grads = {}
+    for name, fields in classes.items():
+        if fields.get("c_bw_code"):
+            g = op_loader.grad_description(ref_sources.as_description(name, fields))
+            grads[g.__name__] = {k: getattr(g, k) for k in ("in_info", "out_info", "c_fw_code", "c_extra_support_code", "code_version")}
+    assert {"GradOfNativeLstm2", "GradOfLstmGenericBase", "GradOfLstmLowMem"} <= set(grads)
+    classes.update(grads)
+    expected_failures |= {"GradOfTwoDLSTM"} & set(grads)
 
     def build(item):
         name, fields = item
