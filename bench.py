@@ -149,6 +149,108 @@ def torch_stack_baseline(prob, dev, steps, warmup):
     return out
 
 
+def bench_encoder_training(args, dev):
+    """
+    Config 4 with gradients: forward of the encoder, a weighted-sum loss, backward to the input and to all parameters
+    (per layer and direction the gradient op, the projection's two GEMMs).  One step = forward + backward; value counts
+    the op-level units of the forward pass, 12 * T * B per step.  The same step through torch.nn.LSTM beside it.
+    """
+    import torch
+
+    from returnn_amd import lstm as rlstm
+    from returnn_amd import synthetic
+
+    prob = synthetic.make_encoder_config("cfg4")
+    T, B, n, L = prob.T, prob.B, prob.n, prob.num_layers
+    bf = torch.bfloat16
+    x = torch.from_numpy(prob.features).to(dev).to(bf)
+    lens = torch.from_numpy(prob.lens).to(dev)
+    weight = torch.randn((T, B, 2 * n), device=dev, generator=torch.Generator(device=dev).manual_seed(0)).to(bf)
+
+    def timed(step_fn, steps, warmup):
+        for _ in range(warmup):
+            step_fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step_fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    enc = rlstm.BlstmEncoder.from_params(prob.layers, device=dev, dtype=bf).train()
+    params = [p for p in enc.parameters()]
+    xg = x.clone().requires_grad_(True)
+
+    def step_ours():
+        for p in params:
+            p.grad = None
+        xg.grad = None
+        y = enc(xg, seq_lens=lens)
+        (y * weight).sum().backward()
+
+    step_ms = timed(step_ours, args.steps, args.warmup)
+    assert all(p.grad is not None and bool(torch.isfinite(p.grad.float()).all()) for p in params) and xg.grad is not None
+    del enc, params
+
+    torch_stack = None
+    if not args.no_torch_baseline:
+        lens_cpu = torch.from_numpy(prob.lens).to(torch.int64)
+        torch_stack = {"what": "torch.nn.LSTM(num_layers=%i, bidirectional=True) on the packed batch, forward + backward, same GPU; ms per step" % L}
+        for dtype in (torch.bfloat16, torch.float16):
+            name = str(dtype).replace("torch.", "")
+            try:
+                net = torch.nn.LSTM(prob.in_dim, n, num_layers=L, bidirectional=True).to(dev).to(dtype).train()
+                xt = x.to(dtype).clone().requires_grad_(True)
+                wt = weight.to(dtype)
+
+                def step_torch():
+                    net.zero_grad(set_to_none=True)
+                    xt.grad = None
+                    packed = torch.nn.utils.rnn.pack_padded_sequence(xt, lens_cpu, enforce_sorted=False)
+                    y = torch.nn.utils.rnn.pad_packed_sequence(net(packed)[0], total_length=T)[0]
+                    (y * wt).sum().backward()
+
+                torch_stack["packed_%s_ms" % name] = timed(step_torch, max(2, args.steps // 4), 1)
+                del net, xt, wt
+            except Exception as exc:
+                torch_stack["error_%s" % name] = "%s: %s" % (type(exc).__name__, str(exc)[:200])
+
+    units = 2 * L * T * B
+    rec_flops = 3 * 2 * L * 8.0 * T * B * n * n  # forward GEMM, backward GEMM, weight gradient
+    proj_flops = 3 * 2 * sum(2.0 * T * B * (prob.in_dim if li == 0 else 2 * n) * 4 * n for li in range(L))
+    return {
+        "metric": "LSTM fwd+bwd timesteps*seqs/sec (T*B/s) at n=%i" % n,
+        "value": units * 1e3 / step_ms,
+        "unit": "timesteps*seqs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": step_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "cfg4 training step: %i-layer bidirectional LSTM encoder forward + backward (input and all parameters), "
+            "T=%i B=%i in=%i n=%i bf16, ragged=True" % (L, T, B, prob.in_dim, n),
+            "calls_per_step": 4 * L,
+            "units_per_step": units,
+            "torch_lstm_same_gpu": torch_stack,
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": (rec_flops + proj_flops) / (step_ms * 1e-3) / 1e12,
+            "peak": PEAK_MFMA["bf16"] / 1e12,
+            "unit": "TFLOP/s",
+            "frac": (rec_flops + proj_flops) / (step_ms * 1e-3) / PEAK_MFMA["bf16"],
+            "traffic": None,
+            "kernel": "whole step: recurrent %.3g TFLOP + projections %.3g TFLOP (forward, backward, weight gradients)"
+            % (rec_flops / 1e12, proj_flops / 1e12),
+        },
+    }
+
+
 def bench_encoder(args, dev):
     """
     Config 4: forward of the 6-layer bidirectional encoder (per layer one projection GEMM and one op call per
@@ -275,8 +377,10 @@ def cpu_baseline_gradient(name: str, target_seconds: float = 15.0):
 
 def bench_gradient(args, dev, cabi):
     """
-    The gradient op (``rtn_native_lstm2_bwd``) of one direction of the workload, on the results of a forward run, all
-    resident in HBM.  One step = one gradient call; value = T*B*K / elapsed.  Algorithmic work per timestep x sequence:
+    The gradient op of the workload on the results of a forward run, all resident in HBM: one direction
+    (``rtn_native_lstm2_bwd``), for cfg3 both directions of the layer (``rtn_native_lstm2_bwd_multi``, or two single
+    calls with ``--pair separate``).  One step = the gradient of the whole workload; value = units * K / elapsed.
+    Algorithmic work per timestep x sequence:
     8 n^2 flops for the recurrent GEMM (Dy0 += DX[t] W^T) plus 8 n^2 for the weight gradient (Y^T DX).
     """
     import torch
@@ -294,23 +398,37 @@ def bench_gradient(args, dev, cabi):
     y0 = torch.from_numpy(p.y0).to(dev).to(act)
     c0 = torch.from_numpy(p.c0).to(dev)
     msk = torch.from_numpy(p.i).to(dev)
-    Y, C, H, d = op(X, W, y0, c0, msk, 0, 1)
+    # cfg3 is a bidirectional layer: both directions' gradient calls in one entry unless --pair separate
+    steps_of = [1, -1] if args.workload == "cfg3" else [1]
+    fused = len(steps_of) > 1 and args.pair == "fused"
+    fw = [op(X, W, y0, c0, msk, 0, st) for st in steps_of]
     del X
     gen = torch.Generator(device=dev).manual_seed(0)
-    DY = torch.randn(Y.shape, device=dev, generator=gen).to(act)
-    Dd = torch.randn(d.shape, device=dev, generator=gen)
-    DX = torch.empty((T, B, 4 * n), dtype=act, device=dev)
-    DW = torch.empty((n, 4 * n), dtype=torch.float32, device=dev)
-    Dy0 = torch.empty((B, n), dtype=act, device=dev)
-    Dc0 = torch.empty((B, n), dtype=torch.float32, device=dev)
-    ws = torch.empty((max(cabi.rtn_native_lstm2_bwd_workspace_bytes(T, B, n, dt_code), 256),), dtype=torch.uint8, device=dev)
+    DY = [torch.randn(fw[0][0].shape, device=dev, generator=gen).to(act) for _ in steps_of]
+    Dd = [torch.randn(fw[0][3].shape, device=dev, generator=gen) for _ in steps_of]
+    DX = [torch.empty((T, B, 4 * n), dtype=act, device=dev) for _ in steps_of]
+    DW = [torch.empty((n, 4 * n), dtype=torch.float32, device=dev) for _ in steps_of]
+    Dy0 = [torch.empty((B, n), dtype=act, device=dev) for _ in steps_of]
+    Dc0 = [torch.empty((B, n), dtype=torch.float32, device=dev) for _ in steps_of]
+    each = max(cabi.rtn_native_lstm2_bwd_workspace_bytes(T, B, n, dt_code), 256)
+    ws = torch.empty((each * len(steps_of),), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev)
+    arr = (lib.Lstm2BwdCall * len(steps_of))()
+    for k, st in enumerate(steps_of):
+        Y, C, H, _ = fw[k]
+        arr[k] = lib.Lstm2BwdCall(
+            W.data_ptr(), y0.data_ptr(), c0.data_ptr(), msk.data_ptr(), 0, st, Y.data_ptr(), C.data_ptr(), H.data_ptr(),
+            DY[k].data_ptr(), Dd[k].data_ptr(), DX[k].data_ptr(), DW[k].data_ptr(), Dy0[k].data_ptr(), Dc0[k].data_ptr())  # fmt: skip
 
     def call():
-        lib.check(cabi.rtn_native_lstm2_bwd(
-            W.data_ptr(), y0.data_ptr(), c0.data_ptr(), msk.data_ptr(), 0, 1, Y.data_ptr(), C.data_ptr(), H.data_ptr(),
-            DY.data_ptr(), Dd.data_ptr(), DX.data_ptr(), DW.data_ptr(), Dy0.data_ptr(), Dc0.data_ptr(), T, B, n, dt_code,
-            ws.data_ptr(), ws.numel(), stream.cuda_stream))  # fmt: skip
+        if fused:
+            lib.check(cabi.rtn_native_lstm2_bwd_multi(arr, len(steps_of), T, B, n, dt_code, ws.data_ptr(), ws.numel(), stream.cuda_stream))
+        else:
+            for k in range(len(steps_of)):
+                a = arr[k]
+                lib.check(cabi.rtn_native_lstm2_bwd(
+                    a.W, a.y0, a.c0, a.i, a.start, a.step, a.Y, a.C, a.H, a.DY, a.Dd, a.DX, a.DW, a.Dy0, a.Dc0, T, B, n, dt_code,
+                    ws.data_ptr() + k * each, each, stream.cuda_stream))  # fmt: skip
 
     for _ in range(args.warmup):
         call()
@@ -320,13 +438,16 @@ def bench_gradient(args, dev, cabi):
         call()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    assert bool(torch.isfinite(DW).all()) and bool(torch.isfinite(Dc0).all())
+    for k in range(len(steps_of)):
+        lib.check(cabi.rtn_native_lstm2_fwd_status(ws.data_ptr() + k * each, stream.cuda_stream))
+        assert bool(torch.isfinite(DW[k]).all()) and bool(torch.isfinite(Dc0[k]).all())
     call_ms = elapsed * 1e3 / args.steps
-    flops = 16.0 * n * n * T * B
+    units = T * B * len(steps_of)
+    flops = 16.0 * n * n * units
     peak = PEAK_MFMA[dtype]
     result = {
         "metric": "LSTM gradient op timesteps*seqs/sec (T*B/s) at n=%i" % n,
-        "value": T * B * args.steps / elapsed,
+        "value": units * args.steps / elapsed,
         "unit": "timesteps*seqs/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -338,10 +459,11 @@ def bench_gradient(args, dev, cabi):
         "dtype": dtype,
         "data": "synthetic",
         "config": {
-            "workload": "%s: NativeLstm2 gradient op, one direction, T=%i B=%i n=%i %s, ragged=%s"
-            % (args.workload, T, B, n, dtype, p.lens is not None),
-            "calls_per_step": 1,
-            "units_per_step": T * B,
+            "workload": "%s: NativeLstm2 gradient op, %s, T=%i B=%i n=%i %s, ragged=%s"
+            % (args.workload, ("both directions, " + ("one entry" if fused else "two entries")) if len(steps_of) > 1 else "one direction",
+               T, B, n, dtype, p.lens is not None),
+            "calls_per_step": len(steps_of),
+            "units_per_step": units,
         },
         "roofline": {
             "bound": "mfma",
@@ -506,7 +628,7 @@ def main():
                          "holds both; default) or as two separate op calls")
     ap.add_argument("--op", default="fwd", choices=["fwd", "bwd", "generic_base", "low_mem"],
                     help="fwd: the forward op (default, the headline metric); bwd: the gradient op of one direction of "
-                         "the workload (cfg1/cfg2/cfg3/cfg5); generic_base, low_mem: forward of the sibling ops on the workload's shape")
+                         "the workload (cfg1/cfg2/cfg3/cfg5; with cfg4: the encoder's training step, forward + backward); generic_base, low_mem: forward of the sibling ops on the workload's shape")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-torch-baseline", action="store_true", help="cfg4: skip timing the same stack through torch.nn.LSTM")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
@@ -533,7 +655,7 @@ def main():
     torch.cuda.set_device(dev)
 
     if args.workload == "cfg4":
-        print(json.dumps(bench_encoder(args, dev)))
+        print(json.dumps(bench_encoder_training(args, dev) if args.op == "bwd" else bench_encoder(args, dev)))
         return
     if args.op == "bwd":
         print(json.dumps(bench_gradient(args, dev, cabi)))

@@ -174,6 +174,38 @@ int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const f
 size_t rtn_native_lstm2_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype);
 
 /*
+ * Several gradient calls of one shape (T, B, n, dtype) in one entry: the gradient ops of the two directions of a
+ * bidirectional layer, which the reference runs as two op calls (the gradient of tf/layers/rec.py:1229-1270).  Element k
+ * gives exactly what rtn_native_lstm2_bwd gives for the same arguments.  When the persistent kernel can hold all
+ * `count` problems on the device at once (count <= 2) they share one cooperative launch, with 16-row batch groups where
+ * 8-row groups would not leave every workgroup a CU; otherwise the calls are enqueued one after the other.
+ * `workspace`: rtn_native_lstm2_bwd_multi_workspace_bytes(); call k uses the k-th equal slice of it, and
+ * rtn_native_lstm2_fwd_status(slice k, stream) reports an expired bounded wait of that problem.
+ */
+typedef struct rtn_lstm2_bwd_call {
+  const void* W;
+  const void* y0;
+  const float* c0;
+  const float* i;
+  int32_t start;
+  int32_t step;
+  const void* Y;
+  const float* C;
+  const void* H;
+  const void* DY;
+  const float* Dd;
+  void* DX;
+  float* DW;
+  void* Dy0;
+  float* Dc0;
+} rtn_lstm2_bwd_call;
+
+int rtn_native_lstm2_bwd_multi(const rtn_lstm2_bwd_call* calls, int32_t count, int64_t T, int32_t B, int32_t n,
+                               int32_t dtype, void* workspace, size_t workspace_bytes, void* hip_stream);
+
+size_t rtn_native_lstm2_bwd_multi_workspace_bytes(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype);
+
+/*
  * Sibling ops of NativeLstm2 on the same kernels (returnn/native_op.py:333-574 and :577-1026), forward pass.  In both,
  * the recurrent input of a frame is the OUTPUT of the frame before -- 0 where that frame was masked -- instead of the
  * last valid output carried over masked frames as in NativeLstm2.

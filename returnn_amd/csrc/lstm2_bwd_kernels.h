@@ -216,8 +216,22 @@ struct Lstm2BwdPersistent {
   unsigned long long timeout_ticks;
 };
 
+// Several gradient problems of one shape in one launch (the two directions of a bidirectional layer):
+// workgroup id / wgs_each picks the problem, the remainder is the workgroup's id inside it.
+constexpr int kMaxBwdMulti = 2;
+struct Lstm2BwdMulti {
+  int count;     // problems, 1..kMaxBwdMulti
+  int wgs_each;  // workgroups per problem = groups * n / (16 * MT)
+  int pad_[2];
+  Lstm2BwdPersistent q[kMaxBwdMulti];
+};
+
 template <typename AT, int KSB, int MT>
-__global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdPersistent q) {
+__global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdMulti multi) {
+  const int which = (int)blockIdx.x / multi.wgs_each;
+  const int bid = (int)blockIdx.x - which * multi.wgs_each;
+  if (which >= multi.count) return;
+  const Lstm2BwdPersistent q = multi.q[which];
   using E = Elem<AT>;
   using SN = Sentinel<AT>;
   using LM = LaneMax<AT>;
@@ -228,7 +242,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdPer
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = p.n, n4 = 4 * n;
   const int kblocks = n / (16 * MT);  // workgroups per group; each owns MT tiles of 16 values of k
-  const int g = (int)blockIdx.x / kblocks, k0 = ((int)blockIdx.x % kblocks) * 16 * MT;
+  const int g = bid / kblocks, k0 = (bid % kblocks) * 16 * MT;
   const int b_base = g * q.Bg;
   const int rows = min(q.Bg, p.B - b_base);
   const long long bn = (long long)p.B * n;

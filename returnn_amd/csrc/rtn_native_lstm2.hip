@@ -647,7 +647,7 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
 }
 
 
-typedef void (*BwdRegwKernel)(const Lstm2BwdPersistent);
+typedef void (*BwdRegwKernel)(const Lstm2BwdMulti);
 
 template <typename AT>
 BwdRegwKernel bwd_regw_kernel_for(int KSB, int MT) {
@@ -713,7 +713,7 @@ using namespace rtn;
 
 extern "C" {
 
-int rtn_native_lstm2_abi_version(void) { return 3; }
+int rtn_native_lstm2_abi_version(void) { return 4; }
 
 const char* rtn_last_error(void) { return g_last_error.c_str(); }
 
@@ -906,13 +906,23 @@ size_t rtn_native_lstm2_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int
   return bwd_layout(B, n, dtype).total;
 }
 
-int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const float* i, int32_t start, int32_t step,
-                         const void* Y, const float* C, const void* H, const void* DY, const float* Dd, void* DX, float* DW,
-                         void* Dy0, float* Dc0, int64_t T, int32_t B, int32_t n, int32_t dtype, void* workspace,
-                         size_t workspace_bytes, void* hip_stream) {
-  g_last_error.clear();
+namespace {
+
+// Per-call state of the gradient entry between its three phases (prepare, recurrence, weight gradient).
+struct BwdJob {
+  Lstm2BwdParams p;
+  unsigned char* ws;
+  long long abs_step, num_steps, first, end;
+};
+
+// `count` gradient calls of one shape.  With the persistent kernel and count <= kMaxBwdMulti all of them share one
+// cooperative launch (16-row batch groups when 8-row groups of all problems would not find a CU each); otherwise they
+// are enqueued one after the other.
+int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, int32_t n, int32_t dtype, void* workspace,
+              size_t workspace_bytes, void* hip_stream) {
   int rc = check_dims(T, B, n, dtype);
   if (rc != RTN_OK) return rc;
+  if (count < 0 || (count > 0 && !calls)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: bad call list");
   hipStream_t stream = (hipStream_t)hip_stream;
   const long long bn = (long long)B * n;
   const long long nn4 = (long long)n * n * 4;
@@ -920,74 +930,62 @@ int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const f
   if (stream) RTN_HIP(hipStreamIsCapturing(stream, &cap_status));
   if (cap_status != hipStreamCaptureStatusNone)
     return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2 backward: cannot be recorded into a graph (it calls rocBLAS)");
-  if (nn4 > 0 && !DW) return fail(RTN_ERR_ARG, "NativeLstm2 backward: DW must not be null");
-  if (bn > 0 && (!Dd || !Dy0 || !Dc0)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: Dd, Dy0 and Dc0 must not be null");
   const dim3 fill_grid(256), fill_block(256);
-  // returnn/native_op.py:1365-1370: DW := 0, Dy0 := 0, Dc0 := Dd
-  if (nn4 > 0) {
-    hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)DW, 0u, nn4);
-    RTN_HIP(hipGetLastError());
+  for (int k = 0; k < count; ++k) {
+    const rtn_lstm2_bwd_call& c = calls[k];
+    if (nn4 > 0 && !c.DW) return fail(RTN_ERR_ARG, "NativeLstm2 backward: DW must not be null");
+    if (bn > 0 && (!c.Dd || !c.Dy0 || !c.Dc0)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: Dd, Dy0 and Dc0 must not be null");
   }
-  if (bn > 0) {
-    hipLaunchKernelGGL(k_copy_f32, fill_grid, fill_block, 0, stream, Dd, Dc0, bn);
-    RTN_HIP(hipGetLastError());
-  }
-  if (T == 0 || bn == 0) {
-    if (bn > 0) {
-      RTN_HIP(hipMemsetAsync(Dy0, 0, (size_t)bn * esize(dtype), stream));
+  for (int k = 0; k < count; ++k) {
+    const rtn_lstm2_bwd_call& c = calls[k];
+    // returnn/native_op.py:1365-1370: DW := 0, Dy0 := 0, Dc0 := Dd
+    if (nn4 > 0) {
+      hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)c.DW, 0u, nn4);
+      RTN_HIP(hipGetLastError());
     }
-    return RTN_OK;
+    if (bn > 0) {
+      hipLaunchKernelGGL(k_copy_f32, fill_grid, fill_block, 0, stream, c.Dd, c.Dc0, bn);
+      RTN_HIP(hipGetLastError());
+    }
+    if ((T == 0 || bn == 0) && bn > 0) {
+      hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)c.Dy0, 0u, (long long)(((size_t)bn * esize(dtype) + 3) / 4));
+      RTN_HIP(hipGetLastError());
+    }
   }
-  if (start < 0 || start >= T) return fail(RTN_ERR_RANGE, "NativeLstm2 backward: need 0 <= start < T, got start=%d, T=%lld", start, (long long)T);
-  if (step == 0) return fail(RTN_ERR_RANGE, "NativeLstm2 backward: step must not be 0");
-  const void* ptrs[] = {W, y0, c0, i, Y, C, H, DY, Dd, DX, DW, Dy0, Dc0};
-  const char* names[] = {"W", "y0", "c0", "i", "Y", "C", "H", "DY", "Dd", "DX", "DW", "Dy0", "Dc0"};
-  for (int q = 0; q < 13; ++q) {
-    if (!ptrs[q]) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must not be null", names[q]);
-    if (q != 3 && !aligned16(ptrs[q])) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must be 16-byte aligned", names[q]);
+  if (T == 0 || bn == 0 || count == 0) return RTN_OK;
+  for (int k = 0; k < count; ++k) {
+    const rtn_lstm2_bwd_call& c = calls[k];
+    if (c.start < 0 || c.start >= T)
+      return fail(RTN_ERR_RANGE, "NativeLstm2 backward: need 0 <= start < T, got start=%d, T=%lld", c.start, (long long)T);
+    if (c.step == 0) return fail(RTN_ERR_RANGE, "NativeLstm2 backward: step must not be 0");
+    const void* ptrs[] = {c.W, c.y0, c.c0, c.i, c.Y, c.C, c.H, c.DY, c.Dd, c.DX, c.DW, c.Dy0, c.Dc0};
+    const char* names[] = {"W", "y0", "c0", "i", "Y", "C", "H", "DY", "Dd", "DX", "DW", "Dy0", "Dc0"};
+    for (int q = 0; q < 13; ++q) {
+      if (!ptrs[q]) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must not be null", names[q]);
+      if (q != 3 && !aligned16(ptrs[q])) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must be 16-byte aligned", names[q]);
+    }
   }
   const BwdLayout lay = bwd_layout(B, n, dtype);
-  if (!workspace || workspace_bytes < lay.total)
-    return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: workspace of %zu bytes needed, got %zu", lay.total, workspace ? workspace_bytes : (size_t)0);
+  if (!workspace || workspace_bytes < lay.total * (size_t)count)
+    return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: workspace of %zu bytes needed, got %zu", lay.total * (size_t)count,
+                workspace ? workspace_bytes : (size_t)0);
   if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: workspace must be 16-byte aligned");
   rocblas_handle blas = nullptr;
   rc = blas_handle(&blas);
   if (rc != RTN_OK) return rc;
   if (rocblas_set_stream(blas, stream) != rocblas_status_success) return fail(RTN_ERR_HIP, "NativeLstm2 backward: rocblas_set_stream failed");
-
-  Lstm2BwdParams p;
-  memset(&p, 0, sizeof(p));
-  p.W = W; p.c0 = c0; p.mask = i; p.C = C; p.H = H; p.DY = DY;
-  p.DX = DX; p.Dc0 = Dc0;
-  unsigned char* ws = (unsigned char*)workspace;
-  p.dyw = (float*)(ws + lay.off_dyw);
-  p.dx0 = ws + lay.off_dx0;
-  p.T = T; p.B = B; p.n = n;
   const size_t es = esize(dtype);
-  hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)ws, 0u, (long long)(lay.total / 4));
-  RTN_HIP(hipGetLastError());
-
-  // returnn/native_op.py:1383-1407: which frames are visited, and in which order
-  const long long abs_step = step > 0 ? step : -(long long)step;
-  const long long num_steps = (T - start + abs_step - 1) / abs_step;
-  const long long first = step > 0 ? start : T - start - 1;
-  const long long end = first + (num_steps - 1) * step;  // inclusive
-  if (num_steps != T) {
-    // frames the loop does not visit keep DX = 0 (:1385-1388)
-    const long long words = (long long)((size_t)T * bn * 4 * es / 4);
-    hipLaunchKernelGGL(k_fill_u32, dim3(1024), fill_block, 0, stream, (unsigned*)DX, 0u, words);
-    RTN_HIP(hipGetLastError());
-  }
   const bool mfma = (n % 16) == 0 && !env_long("RTN_LSTM2_FORCE_GENERIC", 0);
+
   // Persistent kernel: W in registers for the whole call, if a wavefront's share of the 16 x 4n slice fits
-  // (2..32 fragments) and all workgroups can be on the device together.
+  // (2..32 fragments) and all workgroups of all problems can be on the device together.
   const void* pk = nullptr;
   int KSB = 0, bwd_mt = 1;
   // Rows per batch group: 8 when the device has a CU for every workgroup then (a workgroup's step time grows with
   // the rows x 4n values of DX it has to read per frame), else 16.
   int rows_per_group = (int)env_long("RTN_LSTM2_BWD_ROWS", 0);
   if (rows_per_group < 1 || rows_per_group > 16)
-    rows_per_group = ((long long)((B + 7) / 8) * (n / 16) <= device_info().cus) ? 8 : 16;
+    rows_per_group = ((long long)count * ((B + 7) / 8) * (n / 16) <= device_info().cus) ? 8 : 16;
   const int bgroups = (B + rows_per_group - 1) / rows_per_group;
   {
     const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
@@ -995,136 +993,211 @@ int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const f
     const bool shape_ok = mfma && (4 * n) % KM == 0 && S % kWaves == 0;
     KSB = shape_ok ? S / kWaves : 0;
     const long bwd_kernel = env_long("RTN_LSTM2_BWD_KERNEL", 0);  // 0 auto, 1 per-frame launches, 2 persistent
-    if (shape_ok && bwd_kernel != 1 && device_info().cooperative) {
+    if (shape_ok && bwd_kernel != 1 && device_info().cooperative && count <= kMaxBwdMulti) {
       // k tiles per workgroup: one, unless more are needed for the workgroups to fit on the device together.
       const long env_mt = env_long("RTN_LSTM2_BWD_MT", 0);
       for (int mt : {1, 2, 4}) {
         if (env_mt && mt != env_mt) continue;
         if (mt * KSB > 64 || (n / 16) % mt) continue;
-        BwdRegwKernel k = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(KSB, mt) : bwd_regw_kernel_for<float>(KSB, mt);
-        if (!k) continue;
+        BwdRegwKernel kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(KSB, mt) : bwd_regw_kernel_for<float>(KSB, mt);
+        if (!kfn) continue;
         int per_cu = 0;
-        RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)k, kWgThreads, 0));
-        if ((long long)per_cu * device_info().cus >= (long long)bgroups * (n / (16 * mt))) {
-          pk = (const void*)k;
+        RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kfn, kWgThreads, 0));
+        if ((long long)per_cu * device_info().cus >= (long long)count * bgroups * (n / (16 * mt))) {
+          pk = (const void*)kfn;
           bwd_mt = mt;
           break;
         }
       }
     }
+    if (!pk && count > 1) {
+      // no joint launch: one call after the other, each with its own slice of the workspace
+      for (int k = 0; k < count; ++k) {
+        rc = bwd_calls(calls + k, 1, T, B, n, dtype, (unsigned char*)workspace + (size_t)k * lay.total, lay.total, hip_stream);
+        if (rc != RTN_OK) return rc;
+      }
+      return RTN_OK;
+    }
     if (bwd_kernel == 2 && !pk)
       return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2 backward: the persistent kernel cannot run T=%lld B=%d n=%d", (long long)T, B, n);
   }
-  if (pk) {
-    // DX doubles as the exchange medium: armed with all-ones words, every visited frame is written by the kernel.
-    const long long words = (long long)((size_t)T * bn * 4 * es / 4);
-    hipLaunchKernelGGL(k_fill_u32, dim3(2048), fill_block, 0, stream, (unsigned*)DX, 0xFFFFFFFFu, words);
+
+  std::vector<BwdJob> jobs((size_t)count);
+  for (int k = 0; k < count; ++k) {
+    const rtn_lstm2_bwd_call& c = calls[k];
+    BwdJob& j = jobs[(size_t)k];
+    Lstm2BwdParams& p = j.p;
+    memset(&p, 0, sizeof(p));
+    p.W = c.W; p.c0 = c.c0; p.mask = c.i; p.C = c.C; p.H = c.H; p.DY = c.DY;
+    p.DX = c.DX; p.Dc0 = c.Dc0;
+    j.ws = (unsigned char*)workspace + (size_t)k * lay.total;
+    p.dyw = (float*)(j.ws + lay.off_dyw);
+    p.dx0 = j.ws + lay.off_dx0;
+    p.T = T; p.B = B; p.n = n;
+    hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)j.ws, 0u, (long long)(lay.total / 4));
     RTN_HIP(hipGetLastError());
-    Lstm2BwdPersistent q;
-    memset(&q, 0, sizeof(q));
-    q.p = p;
-    q.Dd = Dd;
-    q.Dy0 = Dy0;
-    q.status = (unsigned*)ws;
-    q.t_end = end;
-    q.step = step;
-    q.nframes = (int)num_steps;
-    q.groups = bgroups;
-    q.Bg = (B + bgroups - 1) / bgroups;
-    q.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", 20)));
-    q.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);
-    void* args[] = {(void*)&q};
-    RTN_HIP(hipLaunchCooperativeKernel(pk, dim3((unsigned)(bgroups * (n / (16 * bwd_mt)))), dim3(kWgThreads), args, 0, stream));
-    if (num_steps != T) {
-      const long long frame_words = (long long)((size_t)bn * 4 * es / 4);
-      if (dtype == RTN_DTYPE_BF16)
-        hipLaunchKernelGGL(k_bwd_zero_unvisited<__bf16>, dim3(1024), fill_block, 0, stream, DX, (long long)T, frame_words, first, (long long)step, num_steps);
-      else
-        hipLaunchKernelGGL(k_bwd_zero_unvisited<float>, dim3(1024), fill_block, 0, stream, DX, (long long)T, frame_words, first, (long long)step, num_steps);
+    // returnn/native_op.py:1383-1407: which frames are visited, and in which order
+    j.abs_step = c.step > 0 ? c.step : -(long long)c.step;
+    j.num_steps = (T - c.start + j.abs_step - 1) / j.abs_step;
+    j.first = c.step > 0 ? c.start : T - c.start - 1;
+    j.end = j.first + (j.num_steps - 1) * c.step;  // inclusive
+    const long long words = (long long)((size_t)T * bn * 4 * es / 4);
+    if (pk) {
+      // DX doubles as the exchange medium: armed with all-ones words, every visited frame is written by the kernel.
+      hipLaunchKernelGGL(k_fill_u32, dim3(2048), fill_block, 0, stream, (unsigned*)c.DX, 0xFFFFFFFFu, words);
+      RTN_HIP(hipGetLastError());
+    } else if (j.num_steps != T) {
+      // frames the loop does not visit keep DX = 0 (:1385-1388)
+      hipLaunchKernelGGL(k_fill_u32, dim3(1024), fill_block, 0, stream, (unsigned*)c.DX, 0u, words);
       RTN_HIP(hipGetLastError());
     }
   }
-  const int NT = B > 32 ? 2 : 1;  // up to 32 rows: more, smaller workgroups
-  // The launches of all frames, in reverse processing order.  MFMA shapes: one fused launch per frame (the GEMM of
-  // the frame processed before, then this frame's pointwise part) and a last GEMM-only launch; other shapes: a
-  // pointwise and a generic GEMM launch per frame.
-  auto record = [&](hipStream_t st) -> int {
-    const dim3 pw_grid((unsigned)((bn + 255) / 256)), pw_block(256);
-    const dim3 mm_grid((unsigned)((n / 16) * ((B + 16 * NT - 1) / (16 * NT)))), mm_block(kWgThreads);
-    long long t_done = -1;  // frame whose DX still has to go through the GEMM
-    for (long long t = end;; t -= step) {
-      const bool more = step > 0 ? t >= first : t <= first;
-      const bool right = more && (step > 0 ? (t - step >= first) : (t - step <= first));
-      const long long prev_t = right ? t - step : -1;
-      const long long tt = more ? t : -1;
-      if (mfma) {
-        if (dtype == RTN_DTYPE_BF16) {
-          if (NT == 2)
-            hipLaunchKernelGGL((k_bwd_step<__bf16, 2>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
-          else
-            hipLaunchKernelGGL((k_bwd_step<__bf16, 1>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
-        } else {
-          if (NT == 2)
-            hipLaunchKernelGGL((k_bwd_step<float, 2>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
-          else
-            hipLaunchKernelGGL((k_bwd_step<float, 1>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
-        }
-      } else if (more) {
-        if (dtype == RTN_DTYPE_BF16) {
-          hipLaunchKernelGGL(k_bwd_pointwise<__bf16>, pw_grid, pw_block, 0, st, p, t, prev_t);
-          hipLaunchKernelGGL(k_bwd_gemm_dy_generic<__bf16>, pw_grid, pw_block, 0, st, p, t);
-        } else {
-          hipLaunchKernelGGL(k_bwd_pointwise<float>, pw_grid, pw_block, 0, st, p, t, prev_t);
-          hipLaunchKernelGGL(k_bwd_gemm_dy_generic<float>, pw_grid, pw_block, 0, st, p, t);
-        }
-      }
-      if (!more) break;
-      t_done = t;
-    }
-    RTN_HIP(hipGetLastError());
-    return RTN_OK;
-  };
-  if (pk) {
-    rc = RTN_OK;
-  } else if (env_long("RTN_LSTM2_BWD_NO_GRAPH", 0)) {
-    rc = record(stream);
-  } else {
-    std::string key("bwd");
-    int dev = 0;
-    RTN_HIP(hipGetDevice(&dev));
-    key.append(reinterpret_cast<const char*>(&p), sizeof(p));  // p was zeroed before it was filled in
-    key_append(&key, dtype); key_append(&key, (int)start); key_append(&key, (int)step); key_append(&key, dev);
-    key_append(&key, (int)mfma);
-    rc = replay_graph(key, stream, record);
-  }
-  if (rc != RTN_OK) return rc;
 
-  // DW = sum over consecutive visited frames Y[t - step]^T * DX[t]  (:1433-1452), then += y0^T * dx0 (:1456-1460)
-  const unsigned char* Yb = (const unsigned char*)Y;
-  const unsigned char* DXb = (const unsigned char*)DX;
-  if (num_steps > 1) {
-    if (abs_step == 1) {
-      const long long lo = std::min(first, end);
-      rc = dw_accumulate(blas, Yb + (size_t)(lo + std::max(0, -step)) * bn * es, DXb + (size_t)(lo + std::max(0, step)) * bn * 4 * es,
-                         DW, (num_steps - 1) * B, n, dtype);
-      if (rc != RTN_OK) return rc;
+  if (pk) {
+    Lstm2BwdMulti multi;
+    memset(&multi, 0, sizeof(multi));
+    multi.count = count;
+    multi.wgs_each = bgroups * (n / (16 * bwd_mt));
+    for (int k = 0; k < count; ++k) {
+      Lstm2BwdPersistent& q = multi.q[k];
+      q.p = jobs[(size_t)k].p;
+      q.Dd = calls[k].Dd;
+      q.Dy0 = calls[k].Dy0;
+      q.status = (unsigned*)jobs[(size_t)k].ws;
+      q.t_end = jobs[(size_t)k].end;
+      q.step = calls[k].step;
+      q.nframes = (int)jobs[(size_t)k].num_steps;
+      q.groups = bgroups;
+      q.Bg = (B + bgroups - 1) / bgroups;
+      q.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", 20)));
+      q.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);
+    }
+    void* args[] = {(void*)&multi};
+    RTN_HIP(hipLaunchCooperativeKernel(pk, dim3((unsigned)(count * multi.wgs_each)), dim3(kWgThreads), args, 0, stream));
+    for (int k = 0; k < count; ++k) {
+      const BwdJob& j = jobs[(size_t)k];
+      if (j.num_steps == T) continue;
+      const long long frame_words = (long long)((size_t)bn * 4 * es / 4);
+      if (dtype == RTN_DTYPE_BF16)
+        hipLaunchKernelGGL(k_bwd_zero_unvisited<__bf16>, dim3(1024), fill_block, 0, stream, calls[k].DX, (long long)T, frame_words, j.first,
+                           (long long)calls[k].step, j.num_steps);
+      else
+        hipLaunchKernelGGL(k_bwd_zero_unvisited<float>, dim3(1024), fill_block, 0, stream, calls[k].DX, (long long)T, frame_words, j.first,
+                           (long long)calls[k].step, j.num_steps);
+      RTN_HIP(hipGetLastError());
+    }
+  } else {
+    // count == 1 here.  The launches of all frames, in reverse processing order.  MFMA shapes: one fused launch per
+    // frame (the GEMM of the frame processed before, then this frame's pointwise part) and a last GEMM-only launch;
+    // other shapes: a pointwise and a generic GEMM launch per frame.
+    const BwdJob& j = jobs[0];
+    const Lstm2BwdParams& p = j.p;
+    const int step = calls[0].step;
+    const long long first = j.first, end = j.end;
+    const int NT = B > 32 ? 2 : 1;  // up to 32 rows: more, smaller workgroups
+    auto record = [&](hipStream_t st) -> int {
+      const dim3 pw_grid((unsigned)((bn + 255) / 256)), pw_block(256);
+      const dim3 mm_grid((unsigned)((n / 16) * ((B + 16 * NT - 1) / (16 * NT)))), mm_block(kWgThreads);
+      long long t_done = -1;  // frame whose DX still has to go through the GEMM
+      for (long long t = end;; t -= step) {
+        const bool more = step > 0 ? t >= first : t <= first;
+        const bool right = more && (step > 0 ? (t - step >= first) : (t - step <= first));
+        const long long prev_t = right ? t - step : -1;
+        const long long tt = more ? t : -1;
+        if (mfma) {
+          if (dtype == RTN_DTYPE_BF16) {
+            if (NT == 2)
+              hipLaunchKernelGGL((k_bwd_step<__bf16, 2>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
+            else
+              hipLaunchKernelGGL((k_bwd_step<__bf16, 1>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
+          } else {
+            if (NT == 2)
+              hipLaunchKernelGGL((k_bwd_step<float, 2>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
+            else
+              hipLaunchKernelGGL((k_bwd_step<float, 1>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
+          }
+        } else if (more) {
+          if (dtype == RTN_DTYPE_BF16) {
+            hipLaunchKernelGGL(k_bwd_pointwise<__bf16>, pw_grid, pw_block, 0, st, p, t, prev_t);
+            hipLaunchKernelGGL(k_bwd_gemm_dy_generic<__bf16>, pw_grid, pw_block, 0, st, p, t);
+          } else {
+            hipLaunchKernelGGL(k_bwd_pointwise<float>, pw_grid, pw_block, 0, st, p, t, prev_t);
+            hipLaunchKernelGGL(k_bwd_gemm_dy_generic<float>, pw_grid, pw_block, 0, st, p, t);
+          }
+        }
+        if (!more) break;
+        t_done = t;
+      }
+      RTN_HIP(hipGetLastError());
+      return RTN_OK;
+    };
+    if (env_long("RTN_LSTM2_BWD_NO_GRAPH", 0)) {
+      rc = record(stream);
     } else {
-      for (long long t = end - step; step > 0 ? t >= first : t <= first; t -= step) {
-        rc = dw_accumulate(blas, Yb + (size_t)t * bn * es, DXb + (size_t)(t + step) * bn * 4 * es, DW, B, n, dtype);
+      std::string key("bwd");
+      int dev = 0;
+      RTN_HIP(hipGetDevice(&dev));
+      key.append(reinterpret_cast<const char*>(&p), sizeof(p));  // p was zeroed before it was filled in
+      key_append(&key, dtype); key_append(&key, (int)calls[0].start); key_append(&key, step); key_append(&key, dev);
+      key_append(&key, (int)mfma);
+      rc = replay_graph(key, stream, record);
+    }
+    if (rc != RTN_OK) return rc;
+  }
+
+  for (int k = 0; k < count; ++k) {
+    const rtn_lstm2_bwd_call& c = calls[k];
+    const BwdJob& j = jobs[(size_t)k];
+    const int step = c.step;
+    // DW = sum over consecutive visited frames Y[t - step]^T * DX[t]  (:1433-1452), then += y0^T * dx0 (:1456-1460)
+    const unsigned char* Yb = (const unsigned char*)c.Y;
+    const unsigned char* DXb = (const unsigned char*)c.DX;
+    if (j.num_steps > 1) {
+      if (j.abs_step == 1) {
+        const long long lo = std::min(j.first, j.end);
+        rc = dw_accumulate(blas, Yb + (size_t)(lo + std::max(0, -step)) * bn * es, DXb + (size_t)(lo + std::max(0, step)) * bn * 4 * es,
+                           c.DW, (j.num_steps - 1) * B, n, dtype);
         if (rc != RTN_OK) return rc;
+      } else {
+        for (long long t = j.end - step; step > 0 ? t >= j.first : t <= j.first; t -= step) {
+          rc = dw_accumulate(blas, Yb + (size_t)t * bn * es, DXb + (size_t)(t + step) * bn * 4 * es, c.DW, B, n, dtype);
+          if (rc != RTN_OK) return rc;
+        }
       }
     }
-  }
-  rc = dw_accumulate(blas, y0, p.dx0, DW, B, n, dtype);
-  if (rc != RTN_OK) return rc;
-  if (!pk) {
-    if (dtype == RTN_DTYPE_BF16)
-      hipLaunchKernelGGL(k_convert_from_f32<__bf16>, fill_grid, fill_block, 0, stream, p.dyw, Dy0, bn);
-    else
-      hipLaunchKernelGGL(k_convert_from_f32<float>, fill_grid, fill_block, 0, stream, p.dyw, Dy0, bn);
-    RTN_HIP(hipGetLastError());
+    rc = dw_accumulate(blas, c.y0, j.p.dx0, c.DW, B, n, dtype);
+    if (rc != RTN_OK) return rc;
+    if (!pk) {
+      if (dtype == RTN_DTYPE_BF16)
+        hipLaunchKernelGGL(k_convert_from_f32<__bf16>, fill_grid, fill_block, 0, stream, j.p.dyw, c.Dy0, bn);
+      else
+        hipLaunchKernelGGL(k_convert_from_f32<float>, fill_grid, fill_block, 0, stream, j.p.dyw, c.Dy0, bn);
+      RTN_HIP(hipGetLastError());
+    }
   }
   return RTN_OK;
+}
+
+}  // namespace
+
+int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const float* i, int32_t start, int32_t step,
+                         const void* Y, const float* C, const void* H, const void* DY, const float* Dd, void* DX, float* DW,
+                         void* Dy0, float* Dc0, int64_t T, int32_t B, int32_t n, int32_t dtype, void* workspace,
+                         size_t workspace_bytes, void* hip_stream) {
+  g_last_error.clear();
+  const rtn_lstm2_bwd_call call = {W, y0, c0, i, start, step, Y, C, H, DY, Dd, DX, DW, Dy0, Dc0};
+  return bwd_calls(&call, 1, T, B, n, dtype, workspace, workspace_bytes, hip_stream);
+}
+
+size_t rtn_native_lstm2_bwd_multi_workspace_bytes(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype) {
+  if (count < 0) return 0;
+  return (size_t)count * rtn_native_lstm2_bwd_workspace_bytes(T, B, n, dtype);
+}
+
+int rtn_native_lstm2_bwd_multi(const rtn_lstm2_bwd_call* calls, int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype,
+                               void* workspace, size_t workspace_bytes, void* hip_stream) {
+  g_last_error.clear();
+  return bwd_calls(calls, count, T, B, n, dtype, workspace, workspace_bytes, hip_stream);
 }
 
 int rtn_native_lstm2_fwd_status(const void* workspace, void* hip_stream) {

@@ -43,6 +43,8 @@ SYMBOLS = (
     "rtn_handover_latency_probe",
     "rtn_native_lstm2_bwd",
     "rtn_native_lstm2_bwd_workspace_bytes",
+    "rtn_native_lstm2_bwd_multi",
+    "rtn_native_lstm2_bwd_multi_workspace_bytes",
     "rtn_lstm_generic_base_fwd",
     "rtn_lstm_generic_base_fwd_workspace_bytes",
     "rtn_lstm_low_mem_fwd",
@@ -71,6 +73,28 @@ class Lstm2Call(ctypes.Structure):
         ("C", ctypes.c_void_p),
         ("H", ctypes.c_void_p),
         ("d", ctypes.c_void_p),
+    ]
+
+
+class Lstm2BwdCall(ctypes.Structure):
+    """``rtn_lstm2_bwd_call``: the arguments of one gradient call inside ``rtn_native_lstm2_bwd_multi``."""
+
+    _fields_ = [
+        ("W", ctypes.c_void_p),
+        ("y0", ctypes.c_void_p),
+        ("c0", ctypes.c_void_p),
+        ("i", ctypes.c_void_p),
+        ("start", ctypes.c_int32),
+        ("step", ctypes.c_int32),
+        ("Y", ctypes.c_void_p),
+        ("C", ctypes.c_void_p),
+        ("H", ctypes.c_void_p),
+        ("DY", ctypes.c_void_p),
+        ("Dd", ctypes.c_void_p),
+        ("DX", ctypes.c_void_p),
+        ("DW", ctypes.c_void_p),
+        ("Dy0", ctypes.c_void_p),
+        ("Dc0", ctypes.c_void_p),
     ]
 
 
@@ -112,6 +136,10 @@ def load() -> ctypes.CDLL:
         lib.rtn_native_lstm2_bwd.argtypes = [vp, vp, vp, vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, vp, sz, vp]
         lib.rtn_native_lstm2_bwd_workspace_bytes.restype = sz
         lib.rtn_native_lstm2_bwd_workspace_bytes.argtypes = [i64, i32, i32, i32]
+        lib.rtn_native_lstm2_bwd_multi.restype = ctypes.c_int
+        lib.rtn_native_lstm2_bwd_multi.argtypes = [ctypes.POINTER(Lstm2BwdCall), i32, i64, i32, i32, i32, vp, sz, vp]
+        lib.rtn_native_lstm2_bwd_multi_workspace_bytes.restype = sz
+        lib.rtn_native_lstm2_bwd_multi_workspace_bytes.argtypes = [i32, i64, i32, i32, i32]
         lib.rtn_lstm_generic_base_fwd.restype = ctypes.c_int
         lib.rtn_lstm_generic_base_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, vp, sz, vp]
         lib.rtn_lstm_generic_base_fwd_workspace_bytes.restype = sz

@@ -32,7 +32,7 @@ from typing import NamedTuple, Optional, Sequence, Tuple, Union
 import torch
 
 from . import native_op
-from .torch_native_op import NativeLstm2Function, lstm_last_output, make_op, native_lstm2_multi
+from .torch_native_op import NativeLstm2Function, NativeLstm2PairFunction, lstm_last_output, make_op, native_lstm2_multi
 
 __all__ = ["lstm", "blstm", "prepare_weights", "LstmWeights", "LSTM", "LstmState", "BlstmEncoder", "sequence_mask_time_major"]
 
@@ -229,9 +229,10 @@ def blstm(
     _native_lstm2()  # registers the op and fails loudly without the library
     Xf, Xb = _project(source, fwd, act), _project(source, bwd, act)
     if _wants_grad(Xf, Xb, fwd.rec, bwd.rec, state_fwd.h, state_fwd.c, state_bwd.h, state_bwd.c):
-        # training: one differentiable op call per direction (the gradient op runs per direction anyway)
-        Yf, _, _, df = NativeLstm2Function.apply(Xf, fwd.rec, state_fwd.h, state_fwd.c, mask, 0, 1)
-        Yb, _, _, db = NativeLstm2Function.apply(Xb, bwd.rec, state_bwd.h, state_bwd.c, mask, 0, -1)
+        # training: both directions in one differentiable call (forward and gradient each one library entry)
+        Yf, _, _, df, Yb, _, _, db = NativeLstm2PairFunction.apply(
+            Xf, fwd.rec, state_fwd.h, state_fwd.c, Xb, bwd.rec, state_bwd.h, state_bwd.c, mask
+        )
         hf = _last_output_autograd(Yf, state_fwd.h, seq_lens, 1)
         hb = _last_output_autograd(Yb, state_bwd.h, seq_lens, -1)
         return torch.cat((Yf, Yb), dim=-1), LstmState(h=hf, c=df), LstmState(h=hb, c=db)

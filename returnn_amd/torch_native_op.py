@@ -434,13 +434,7 @@ def native_lstm2_multi(calls, *, mode: Optional[str] = None):
     return outs
 
 
-def native_lstm2_grad(W, y0, c0, i, start, step, Y, C, H, DY, Dd):
-    """
-    The gradient op of ``NativeLstm2`` on HIP tensors (returnn/native_op.py:1288-1464; arguments as
-    ``grad_input_map`` :1071-1077 without X, which the computation does not read).
-
-    :return: DX [T,B,4n] and Dy0 [B,n] in the element type of Y; DW [n,4n] and Dc0 [B,n] in float32
-    """
+def _normalise_grad_args(W, y0, c0, i, Y, C, H, DY, Dd):
     if not Y.is_cuda:
         raise RuntimeError("NativeLstm2 gradient: this build implements the op for HIP (MI355X) tensors only; got CPU tensors.")
     bf16 = Y.dtype == torch.bfloat16
@@ -457,22 +451,66 @@ def native_lstm2_grad(W, y0, c0, i, start, step, Y, C, H, DY, Dd):
             raise RuntimeError("NativeLstm2 gradient: %s has shape %s, expected %s" % (name, tuple(t.shape), expect[name]))
         if t.device != device:
             raise RuntimeError("NativeLstm2 gradient: %s is on %s but Y is on %s" % (name, t.device, device))
+    return (W, y0, c0, i, Y, C, H, DY, Dd), (T, B, n, bf16)
+
+
+def _alloc_grad_outputs(T, B, n, bf16, device):
+    act = torch.bfloat16 if bf16 else torch.float32
+    DX = torch.empty((T, B, 4 * n), dtype=act, device=device)
+    DW = torch.empty((n, 4 * n), dtype=torch.float32, device=device)
+    Dy0 = torch.empty((B, n), dtype=act, device=device)
+    Dc0 = torch.empty((B, n), dtype=torch.float32, device=device)
+    return DX, DW, Dy0, Dc0
+
+
+def native_lstm2_grad(W, y0, c0, i, start, step, Y, C, H, DY, Dd):
+    """
+    The gradient op of ``NativeLstm2`` on HIP tensors (returnn/native_op.py:1288-1464; arguments as
+    ``grad_input_map`` :1071-1077 without X, which the computation does not read).
+
+    :return: DX [T,B,4n] and Dy0 [B,n] in the element type of Y; DW [n,4n] and Dc0 [B,n] in float32
+    """
+    return native_lstm2_grad_multi([(W, y0, c0, i, start, step, Y, C, H, DY, Dd)])[0]
+
+
+def native_lstm2_grad_multi(calls):
+    """
+    Several gradient calls of one shape in one library entry (``rtn_native_lstm2_bwd_multi``): the two directions of
+    a bidirectional layer share one kernel launch when the device can hold both.
+
+    :param calls: list of ``(W, y0, c0, i, start, step, Y, C, H, DY, Dd)``
+    :return: list of ``(DX, DW, Dy0, Dc0)``, element k as :func:`native_lstm2_grad` gives for ``calls[k]``
+    """
+    calls = list(calls)
+    if not calls:
+        return []
+    norm = []
+    shape = None
+    for W, y0, c0, i, start, step, Y, C, H, DY, Dd in calls:
+        tensors, this = _normalise_grad_args(W, y0, c0, i, Y, C, H, DY, Dd)
+        if shape is None:
+            shape, device = this, tensors[4].device
+        elif this != shape or tensors[4].device != device:
+            raise RuntimeError("native_lstm2_grad_multi: all calls must have one shape, dtype and device; got %r and %r" % (shape, this))
+        norm.append((tensors, int(start), int(step)))
+    T, B, n, bf16 = shape
     lib = _lib.load()
     dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
+    count = len(norm)
     with torch.cuda.device(device):
-        DX = torch.empty((T, B, 4 * n), dtype=act, device=device)
-        DW = torch.empty((n, 4 * n), dtype=torch.float32, device=device)
-        Dy0 = torch.empty((B, n), dtype=act, device=device)
-        Dc0 = torch.empty((B, n), dtype=torch.float32, device=device)
-        ws_bytes = int(lib.rtn_native_lstm2_bwd_workspace_bytes(T, B, n, dtype))
+        outs = [_alloc_grad_outputs(T, B, n, bf16, device) for _ in range(count)]
+        ws_bytes = int(lib.rtn_native_lstm2_bwd_multi_workspace_bytes(count, T, B, n, dtype))
         ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=device)
-        rc = lib.rtn_native_lstm2_bwd(
-            W.data_ptr(), y0.data_ptr(), c0.data_ptr(), i.data_ptr(), int(start), int(step), Y.data_ptr(), C.data_ptr(),
-            H.data_ptr(), DY.data_ptr(), Dd.data_ptr(), DX.data_ptr(), DW.data_ptr(), Dy0.data_ptr(), Dc0.data_ptr(),
-            T, B, n, dtype, ws.data_ptr(), ws.numel(), torch.cuda.current_stream(device).cuda_stream,
-        )  # fmt: skip
+        arr = (_lib.Lstm2BwdCall * count)()
+        for k, ((W, y0, c0, i, Y, C, H, DY, Dd), start, step) in enumerate(norm):
+            DX, DW, Dy0, Dc0 = outs[k]
+            arr[k] = _lib.Lstm2BwdCall(
+                W.data_ptr(), y0.data_ptr(), c0.data_ptr(), i.data_ptr(), start, step, Y.data_ptr(), C.data_ptr(), H.data_ptr(),
+                DY.data_ptr(), Dd.data_ptr(), DX.data_ptr(), DW.data_ptr(), Dy0.data_ptr(), Dc0.data_ptr(),
+            )  # fmt: skip
+        rc = lib.rtn_native_lstm2_bwd_multi(arr, count, T, B, n, dtype, ws.data_ptr(), ws.numel(), torch.cuda.current_stream(device).cuda_stream)
     _lib.check(rc)
-    return DX, DW, Dy0, Dc0
+    return outs
 
 
 class NativeLstm2Function(torch.autograd.Function):
@@ -502,6 +540,37 @@ class NativeLstm2Function(torch.autograd.Function):
         DX, DW, Dy0, Dc0 = native_lstm2_grad(W, y0, c0, i, ctx.start, ctx.step, Y, C, H, DY, Dd)
         dX, dW, dy0, dc0 = (g.to(t) for g, t in zip((DX, DW, Dy0, Dc0), ctx.in_dtypes))
         return dX, dW, dy0, dc0, None, None, None
+
+
+class NativeLstm2PairFunction(torch.autograd.Function):
+    """
+    The two directions of a bidirectional layer as one differentiable call:
+    ``Yf, Cf, Hf, df, Yb, Cb, Hb, db = NativeLstm2PairFunction.apply(Xf, Wf, y0f, c0f, Xb, Wb, y0b, c0b, i)``, the forward
+    direction with (start, step) = (0, 1), the backward direction with (0, -1).  Forward and gradient each go through
+    the library's multi-call entry (one kernel launch for both directions where the device can hold them); results are
+    those of two :class:`NativeLstm2Function` calls.
+    """
+
+    @staticmethod
+    def forward(ctx, Xf, Wf, y0f, c0f, Xb, Wb, y0b, c0b, i):
+        (Yf, Cf, Hf, df), (Yb, Cb, Hb, db) = native_lstm2_multi([(Xf, Wf, y0f, c0f, i, 0, 1), (Xb, Wb, y0b, c0b, i, 0, -1)])
+        ctx.save_for_backward(Wf, y0f, c0f, Wb, y0b, c0b, i, Yf, Cf, Hf, Yb, Cb, Hb)
+        ctx.in_dtypes = (Xf.dtype, Wf.dtype, y0f.dtype, c0f.dtype, Xb.dtype, Wb.dtype, y0b.dtype, c0b.dtype)
+        ctx.mark_non_differentiable(Cf, Hf, Cb, Hb)
+        return Yf, Cf, Hf, df, Yb, Cb, Hb, db
+
+    @staticmethod
+    def backward(ctx, DYf, _DCf, _DHf, Ddf, DYb, _DCb, _DHb, Ddb):
+        Wf, y0f, c0f, Wb, y0b, c0b, i, Yf, Cf, Hf, Yb, Cb, Hb = ctx.saved_tensors
+        DYf = torch.zeros_like(Yf) if DYf is None else DYf
+        DYb = torch.zeros_like(Yb) if DYb is None else DYb
+        Ddf = torch.zeros_like(c0f, dtype=torch.float32) if Ddf is None else Ddf
+        Ddb = torch.zeros_like(c0b, dtype=torch.float32) if Ddb is None else Ddb
+        gf, gb = native_lstm2_grad_multi(
+            [(Wf, y0f, c0f, i, 0, 1, Yf, Cf, Hf, DYf, Ddf), (Wb, y0b, c0b, i, 0, -1, Yb, Cb, Hb, DYb, Ddb)]
+        )
+        grads = [g.to(t) for g, t in zip(tuple(gf) + tuple(gb), ctx.in_dtypes)]
+        return (*grads, None)
 
 
 def lstm_last_output(Y: torch.Tensor, y0: torch.Tensor, i: torch.Tensor, start: int = 0, step: int = 1) -> torch.Tensor:

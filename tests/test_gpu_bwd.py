@@ -126,3 +126,57 @@ def test_bwd_edge_cases_and_errors():
                                           *(t.cpu() for t in (z(4, B, n), z(4, B, n), z(4, B, 4 * n), z(4, B, n), Dd)))  # fmt: skip
     assert cabi.rtn_native_lstm2_bwd_workspace_bytes(10, B, n, 0) > 0
     assert cabi.rtn_native_lstm2_bwd_workspace_bytes(-1, B, n, 0) == 0
+
+
+@pytest.mark.parametrize("T,B,n,dtype", [(14, 32, 256, "bf16"), (9, 20, 64, "f32"), (20, 32, 1024, "bf16"), (6, 5, 20, "f32"), (7, 70, 128, "bf16")])
+def test_bwd_multi_equals_single_calls(T, B, n, dtype):
+    """
+    The two directions of a layer through ``rtn_native_lstm2_bwd_multi``: against the oracle to the same bar as a single
+    call, and against two single calls (the decomposition into batch groups may differ, the sums per output value do not
+    depend on it: equal to the last bit for the recurrent part; the weight gradient goes through the same rocBLAS call).
+    """
+    announce("bwd multi", T, B, n, dtype)
+    X, W, y0, c0, i = random_problem(50 + T + n, T, B, n)
+    Wb = numpy.ascontiguousarray(W[::-1])  # another matrix for the other direction
+    rng = numpy.random.default_rng(77)
+    DY = [rng.normal(0, 1.0, (T, B, n)).astype(numpy.float32) for _ in range(2)]
+    Dd = [rng.normal(0, 1.0, (B, n)).astype(numpy.float32) for _ in range(2)]
+    op = get_op()
+    torch_native_op.OpMaker.options["NativeLstm2"]["mode"] = "auto"
+    Xd, y0d = to_dev(X, dtype), to_dev(y0, dtype)
+    Wd = [to_dev(W, dtype), to_dev(Wb, dtype)]
+    DYd = [to_dev(a, dtype) for a in DY]
+    c0d, id_ = to_dev(c0, "f32"), to_dev(i, "f32")
+    Ddd = [to_dev(a, "f32") for a in Dd]
+    steps = (1, -1)
+    fw = [op(Xd, Wd[k], y0d, c0d, id_, 0, steps[k]) for k in range(2)]
+    calls = [(Wd[k], y0d, c0d, id_, 0, steps[k], fw[k][0], fw[k][1], fw[k][2], DYd[k], Ddd[k]) for k in range(2)]
+    multi = torch_native_op.native_lstm2_grad_multi(calls)
+    single = [torch_native_op.native_lstm2_grad(*c) for c in calls]
+    torch.cuda.synchronize()
+    f = lambda t: t.float().cpu().numpy().astype(numpy.float64)  # noqa: E731
+    tol = 2e-5 if dtype == "f32" else 2e-2
+    for k in range(2):
+        Y, C, H, _ = fw[k]
+        want = oracle.native_lstm2_bwd(f(Xd), f(Wd[k]), f(y0d), c0, i, 0, steps[k], f(Y), f(C), f(H), f(DYd[k]), Dd[k], dtype=numpy.float64)
+        for name, a, s, b in zip(("DX", "DW", "Dy0", "Dc0"), multi[k], single[k], want):
+            assert _rel_to_max(f(a), b) <= tol, (k, name, _rel_to_max(f(a), b))
+            if name != "DW":
+                assert torch.equal(a, s), (k, name)
+            else:
+                assert _rel_to_max(f(a), f(s)) <= 1e-6, (k, name)
+
+
+def test_bwd_multi_errors_and_empty():
+    announce("bwd multi errors")
+    get_op()
+    cabi = lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    assert cabi.rtn_native_lstm2_bwd_multi(None, 0, 4, 2, 32, lib.DTYPE_F32, None, 0, stream) == 0  # nothing to do
+    assert cabi.rtn_native_lstm2_bwd_multi(None, 2, 4, 2, 32, lib.DTYPE_F32, None, 0, stream) == lib.RTN_ERR_ARG
+    assert cabi.rtn_native_lstm2_bwd_multi_workspace_bytes(2, 4, 2, 32, lib.DTYPE_F32) == 2 * cabi.rtn_native_lstm2_bwd_workspace_bytes(4, 2, 32, lib.DTYPE_F32)
+    with pytest.raises(RuntimeError, match="one shape"):
+        z = lambda *s: torch.zeros(*s, device="cuda:0")  # noqa: E731
+        a = (z(8, 32), z(2, 8), z(2, 8), z(3, 2), 0, 1, z(3, 2, 8), z(3, 2, 8), z(3, 2, 32), z(3, 2, 8), z(2, 8))
+        b = (z(8, 32), z(2, 8), z(2, 8), z(4, 2), 0, 1, z(4, 2, 8), z(4, 2, 8), z(4, 2, 32), z(4, 2, 8), z(2, 8))
+        torch_native_op.native_lstm2_grad_multi([a, b])
