@@ -176,9 +176,10 @@ size_t rtn_native_lstm2_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int
 /*
  * Several gradient calls of one shape (T, B, n, dtype) in one entry: the gradient ops of the two directions of a
  * bidirectional layer, which the reference runs as two op calls (the gradient of tf/layers/rec.py:1229-1270).  Element k
- * gives exactly what rtn_native_lstm2_bwd gives for the same arguments.  When the persistent kernel can hold all
- * `count` problems on the device at once (count <= 2) they share one cooperative launch, with 16-row batch groups where
- * 8-row groups would not leave every workgroup a CU; otherwise the calls are enqueued one after the other.
+ * gives what rtn_native_lstm2_bwd gives for the same arguments, up to float32 rounding (the joint launch may split the
+ * work differently, which changes the order of the partial sums).  When the persistent kernel can hold all `count`
+ * problems on the device at once (count <= 2) they share one cooperative launch, each workgroup taking more values of k
+ * so that every workgroup still has a CU; otherwise the calls are enqueued one after the other.
  * `workspace`: rtn_native_lstm2_bwd_multi_workspace_bytes(); call k uses the k-th equal slice of it, and
  * rtn_native_lstm2_fwd_status(slice k, stream) reports an expired bounded wait of that problem.
  */

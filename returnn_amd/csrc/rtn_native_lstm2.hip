@@ -981,12 +981,12 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
   // (2..32 fragments) and all workgroups of all problems can be on the device together.
   const void* pk = nullptr;
   int KSB = 0, bwd_mt = 1;
-  // Rows per batch group: 8 when the device has a CU for every workgroup then (a workgroup's step time grows with
-  // the rows x 4n values of DX it has to read per frame), else 16.
-  int rows_per_group = (int)env_long("RTN_LSTM2_BWD_ROWS", 0);
-  if (rows_per_group < 1 || rows_per_group > 16)
-    rows_per_group = ((long long)count * ((B + 7) / 8) * (n / 16) <= device_info().cus) ? 8 : 16;
-  const int bgroups = (B + rows_per_group - 1) / rows_per_group;
+  // Decomposition: batch groups of 8 or 16 rows (a workgroup's frame time grows with the rows x 4n values of DX it
+  // reads per frame at device scope) times MT tiles of 16 values of k per workgroup (more tiles: fewer workgroups, more
+  // MFMA time each).  Candidates in the order measured on MI355X (cfg3: one problem 8 x 1: 4.4 ms; two problems in one
+  // launch 8 x 2: 5.5 ms, 16 x 1: 6.5 ms, 16 x 2: 7.1 ms); the first whose workgroups are all on the device together.
+  const long env_rows = env_long("RTN_LSTM2_BWD_ROWS", 0);
+  int rows_per_group = 16;
   {
     const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
     const int S = 4 * n / KM;
@@ -994,18 +994,24 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     KSB = shape_ok ? S / kWaves : 0;
     const long bwd_kernel = env_long("RTN_LSTM2_BWD_KERNEL", 0);  // 0 auto, 1 per-frame launches, 2 persistent
     if (shape_ok && bwd_kernel != 1 && device_info().cooperative && count <= kMaxBwdMulti) {
-      // k tiles per workgroup: one, unless more are needed for the workgroups to fit on the device together.
       const long env_mt = env_long("RTN_LSTM2_BWD_MT", 0);
-      for (int mt : {1, 2, 4}) {
+      const int candidates[][2] = {{8, 1}, {8, 2}, {16, 1}, {16, 2}, {8, 4}, {16, 4}};
+      for (const auto& cand : candidates) {
+        const int rows = cand[0], mt = cand[1];
         if (env_mt && mt != env_mt) continue;
+        const bool rows_forced = env_rows >= 1 && env_rows <= 16;  // an explicit row count replaces the candidates' own
+        if (rows_forced && rows != 8) continue;                    // (one pass per MT is enough then)
+        const int use_rows = rows_forced ? (int)env_rows : rows;
         if (mt * KSB > 64 || (n / 16) % mt) continue;
         BwdRegwKernel kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(KSB, mt) : bwd_regw_kernel_for<float>(KSB, mt);
         if (!kfn) continue;
         int per_cu = 0;
         RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kfn, kWgThreads, 0));
-        if ((long long)per_cu * device_info().cus >= (long long)count * bgroups * (n / (16 * mt))) {
+        const long long groups_needed = (B + use_rows - 1) / use_rows;
+        if ((long long)per_cu * device_info().cus >= (long long)count * groups_needed * (n / (16 * mt))) {
           pk = (const void*)kfn;
           bwd_mt = mt;
+          rows_per_group = use_rows;
           break;
         }
       }
@@ -1021,6 +1027,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     if (bwd_kernel == 2 && !pk)
       return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2 backward: the persistent kernel cannot run T=%lld B=%d n=%d", (long long)T, B, n);
   }
+  const int bgroups = (B + rows_per_group - 1) / rows_per_group;
 
   std::vector<BwdJob> jobs((size_t)count);
   for (int k = 0; k < count; ++k) {

@@ -132,8 +132,9 @@ def test_bwd_edge_cases_and_errors():
 def test_bwd_multi_equals_single_calls(T, B, n, dtype):
     """
     The two directions of a layer through ``rtn_native_lstm2_bwd_multi``: against the oracle to the same bar as a single
-    call, and against two single calls (the decomposition into batch groups may differ, the sums per output value do not
-    depend on it: equal to the last bit for the recurrent part; the weight gradient goes through the same rocBLAS call).
+    call, and against two single calls.  The joint launch may use another decomposition (k tiles per workgroup), which
+    changes the order in which the MFMA partial sums are added: equal to float32 rounding, i.e. within 1e-5 of the
+    largest magnitude in float32 and within one bfloat16 step (2^-7) of it in bfloat16.
     """
     announce("bwd multi", T, B, n, dtype)
     X, W, y0, c0, i = random_problem(50 + T + n, T, B, n)
@@ -161,10 +162,7 @@ def test_bwd_multi_equals_single_calls(T, B, n, dtype):
         want = oracle.native_lstm2_bwd(f(Xd), f(Wd[k]), f(y0d), c0, i, 0, steps[k], f(Y), f(C), f(H), f(DYd[k]), Dd[k], dtype=numpy.float64)
         for name, a, s, b in zip(("DX", "DW", "Dy0", "Dc0"), multi[k], single[k], want):
             assert _rel_to_max(f(a), b) <= tol, (k, name, _rel_to_max(f(a), b))
-            if name != "DW":
-                assert torch.equal(a, s), (k, name)
-            else:
-                assert _rel_to_max(f(a), f(s)) <= 1e-6, (k, name)
+            assert _rel_to_max(f(a), f(s)) <= (1e-5 if dtype == "f32" else 2.0**-7), (k, name, _rel_to_max(f(a), f(s)))
 
 
 def test_bwd_multi_errors_and_empty():
