@@ -11,7 +11,7 @@ from __future__ import annotations
 import ctypes
 import os
 import subprocess
-from typing import Optional, Tuple
+from typing import Tuple
 
 import numpy
 

@@ -5,7 +5,6 @@ from __future__ import annotations
 import contextlib
 import os
 import sys
-from typing import Optional
 
 import numpy
 import torch

@@ -19,7 +19,7 @@ from oracle import lstm2_oracle as oracle
 import torch
 
 from returnn_amd import lib, synthetic
-from _gpu_util import announce, env, get_op, random_problem, run_op, run_raw, to_dev
+from _gpu_util import announce, env, get_op, random_problem, run_op, run_raw
 from _textbook import REFERENCE_START_STEP, reference_fixture, textbook_lstm, visited_slice
 
 pytestmark = pytest.mark.gpu
