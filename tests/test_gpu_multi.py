@@ -6,7 +6,6 @@ what the parity tests pin against the oracle.
 
 from __future__ import annotations
 
-import numpy
 import pytest
 import torch
 
