@@ -5,9 +5,10 @@
  * current HIP device, `hip_stream` is a hipStream_t (NULL = the default stream).
  * Every entry point only enqueues work on that stream: no device synchronisation
  * (the two *_status queries excepted), no allocation of device memory (scratch comes
- * in through `workspace`; the one exception is the rocBLAS call inside
- * rtn_native_lstm2_bwd), inputs are never written, outputs are caller-allocated and
- * fully overwritten (the callee does not rely on them being zeroed).
+ * in through `workspace`; the exception is rocBLAS, which the gradient entries and
+ * rtn_lstm_low_mem_fwd call and which may allocate on first use), inputs are never
+ * written, outputs are caller-allocated and fully overwritten (the callee does not
+ * rely on them being zeroed).
  *
  * The reference has no C ABI of its own for this operator: it generates a C++
  * translation unit per op at run time (returnn/torch/util/native_op.py:83-376)
