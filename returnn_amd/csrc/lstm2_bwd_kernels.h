@@ -216,6 +216,21 @@ struct Lstm2BwdPersistent {
   unsigned long long timeout_ticks;
 };
 
+// Optional instrumentation (-DRTN_LSTM2_TRACE): thread 0 of every workgroup accumulates shader-clock ticks per phase
+// of the persistent gradient kernel into a device array that rtn_debug_bwd_trace() copies out.
+#ifdef RTN_LSTM2_TRACE
+__device__ unsigned long long g_bwd_trace[1024 * 8];
+#define RTN_BTRACE_DECL unsigned long long bt_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long bt_last = clock64();
+#define RTN_BTRACE_MARK(k) { const unsigned long long bt_now = clock64(); bt_acc[k] += bt_now - bt_last; bt_last = bt_now; }
+#define RTN_BTRACE_ADD(k, v) { bt_acc[k] += (v); }
+#define RTN_BTRACE_FLUSH() if (threadIdx.x == 0 && blockIdx.x < 1024) { for (int k = 0; k < 8; ++k) g_bwd_trace[(size_t)blockIdx.x * 8 + k] = bt_acc[k]; }
+#else
+#define RTN_BTRACE_DECL
+#define RTN_BTRACE_MARK(k)
+#define RTN_BTRACE_ADD(k, v)
+#define RTN_BTRACE_FLUSH()
+#endif
+
 // Several gradient problems of one shape in one launch (the two directions of a bidirectional layer):
 // workgroup id / wgs_each picks the problem, the remainder is the workgroup's id inside it.
 constexpr int kMaxBwdMulti = 2;
@@ -226,8 +241,14 @@ struct Lstm2BwdMulti {
   Lstm2BwdPersistent q[kMaxBwdMulti];
 };
 
-template <typename AT, int KSB, int MT>
-__global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdMulti multi) {
+// WV wavefronts per workgroup (4, 8 or 16) share the contraction range: a CU moves more bytes per microsecond at device
+// scope the more wavefronts have loads in flight, and with 8 or more each wavefront's share of W and of the frame's DX
+// fits the ordinary registers.  The 256 (row, k) pairs of a tile belong to the threads with the same tid % 256; thread
+// set tid / 256 takes the tiles set, set + WV/4, ...
+template <typename AT, int KSB, int MT, int WV>
+__global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti multi) {
+  constexpr int TS = WV / 4;               // thread sets of 256
+  constexpr int PT = (MT + TS - 1) / TS;   // tiles whose pairs a thread keeps
   const int which = (int)blockIdx.x / multi.wgs_each;
   const int bid = (int)blockIdx.x - which * multi.wgs_each;
   if (which >= multi.count) return;
@@ -237,9 +258,9 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdMul
   using LM = LaneMax<AT>;
   constexpr int KE = E::KE, KM = E::KM, ES = (int)sizeof(AT);
   const Lstm2BwdParams& p = q.p;
-  __shared__ f32x4 red[kWaves][MT][64];
+  __shared__ f32x4 red[WV][MT][64];
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // 0..WV-1
   const int n = p.n, n4 = 4 * n;
   const int kblocks = n / (16 * MT);  // workgroups per group; each owns MT tiles of 16 values of k
   const int g = bid / kblocks, k0 = (bid % kblocks) * 16 * MT;
@@ -260,35 +281,38 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdMul
   const unsigned foff0 = (unsigned)(((size_t)(b_base + (((lane & 15) < rows) ? (lane & 15) : 0)) * n4  // rows the group lacks: row 0
                                      + (size_t)KM * KSB * wave + KE * (lane >> 4)) * ES);
 
-  // The (row, k) pairs of this thread, one per tile.
-  const int bl = tid >> 4, kl = tid & 15;
-  const bool valid = bl < rows;
-  const int b = b_base + (valid ? bl : 0);
-  long long idx[MT], io[MT];
-  float dyw[MT], dc[MT], dx0[MT][4];
+  // The (row, k) pairs of this thread: one in each of its tiles.
+  const int set = (TS == 1) ? 0 : __builtin_amdgcn_readfirstlane(tid >> 8);  // uniform over a wavefront
+  const int bl = (tid & 255) >> 4, kl = tid & 15;
+  const int b = b_base + ((bl < rows) ? bl : 0);
+  bool act[PT];  // the pair exists: the tile does, and the group has the row
+  long long idx[PT], io[PT];
+  float dyw[PT], dc[PT], dx0[PT][4];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int k = k0 + 16 * mt + kl;
-    idx[mt] = (long long)b * n + k;
-    io[mt] = (long long)b * n4 + k;
-    dyw[mt] = 0.f;
-    dc[mt] = valid ? q.Dd[idx[mt]] : 0.f;
+  for (int j = 0; j < PT; ++j) {
+    const int mt = set + TS * j;
+    act[j] = (mt < MT) && (bl < rows);
+    const int k = k0 + 16 * ((mt < MT) ? mt : 0) + kl;
+    idx[j] = (long long)b * n + k;
+    io[j] = (long long)b * n4 + k;
+    dyw[j] = 0.f;
+    dc[j] = act[j] ? q.Dd[idx[j]] : 0.f;
 #pragma unroll
-    for (int gq = 0; gq < 4; ++gq) dx0[mt][gq] = 0.f;
+    for (int gq = 0; gq < 4; ++gq) dx0[j][gq] = 0.f;
   }
   // where a pair's element of the summed tile is: tile element D[kl][bl] sits in lane (kl/4)*16 + bl, component kl%4
   const int red_lane = (kl >> 2) * 16 + bl, red_comp = kl & 3;
 
   // inputs of a frame, fetched one frame ahead
-  float in_gate[MT][4], in_dy[MT], in_pc[MT], in_m;
+  float in_gate[PT][4], in_dy[PT], in_pc[PT], in_m;
   auto fetch = [&](long long t, long long prev_t) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const long long fo = t * bn * 4 + io[mt];
+    for (int j = 0; j < PT; ++j) {
+      const long long fo = t * bn * 4 + io[j];
 #pragma unroll
-      for (int gq = 0; gq < 4; ++gq) in_gate[mt][gq] = E::load(p.H, fo + (long long)gq * n);
-      in_dy[mt] = E::load(p.DY, t * bn + idx[mt]);
-      in_pc[mt] = prev_t >= 0 ? p.C[prev_t * bn + idx[mt]] : p.c0[idx[mt]];
+      for (int gq = 0; gq < 4; ++gq) in_gate[j][gq] = E::load(p.H, fo + (long long)gq * n);
+      in_dy[j] = E::load(p.DY, t * bn + idx[j]);
+      in_pc[j] = prev_t >= 0 ? p.C[prev_t * bn + idx[j]] : p.c0[idx[j]];
     }
     in_m = p.mask[t * p.B + b];
   };
@@ -306,9 +330,11 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdMul
   bool aborted = false;
   // d_h of the thread's pairs from DX of frame t (whose first read has been issued): wait, MFMA, sum over the
   // wavefronts; added to dyw.
+  RTN_BTRACE_DECL
   auto gemm = [&](long long t) {
     unsigned long long t0 = 0;
     unsigned spins = 0;
+    RTN_BTRACE_MARK(4)  // pointwise tail, fetch, delay, first read
     for (;;) {
       unsigned m = 0;
 #pragma unroll
@@ -329,10 +355,21 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdMul
       }
       issue(t);
     }
+    RTN_BTRACE_MARK(0)  // wait for the frame's DX
+    RTN_BTRACE_ADD(6, spins)
     if (spins)
       delay = min(delay + 2, 64);
     else if (delay > 0)
       delay -= ((t & 15) == 15) ? 1 : 0;
+    // W lives in accumulation registers where it is at most half of that file: the B fragments of a frame fill half of
+    // the ordinary registers, and a matrix instruction reads an A operand from either file (without this the compiler
+    // parks part of W there anyway and copies four registers back in front of every MFMA, which halves the MFMA rate).
+    if constexpr (MT * KSB <= 32) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int ks = 0; ks < KSB; ++ks) asm volatile("" : "+a"(wreg[mt][ks]));
+    }
     // independent partial sums keep the MFMA pipeline full (one chain would wait for every result)
     constexpr int NACC = (MT >= 4 || KSB < 2) ? 1 : (MT == 2 || KSB < 4 ? 2 : 4);
     f32x4 part[MT][NACC];
@@ -351,15 +388,19 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdMul
       for (int a = 1; a < NACC; ++a) acc += part[mt][a];
       red[wave][mt][lane] = acc;
     }
+    RTN_BTRACE_MARK(1)  // MFMA, partial tiles to LDS
     __syncthreads();
+    RTN_BTRACE_MARK(2)  // barrier
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
+    for (int j = 0; j < PT; ++j) {
+      const int mt = (set + TS * j < MT) ? set + TS * j : 0;
       float sum = 0.f;
 #pragma unroll
-      for (int w = 0; w < kWaves; ++w) sum += ((const float*)&red[w][mt][red_lane])[red_comp];
-      dyw[mt] += sum;
+      for (int w = 0; w < WV; ++w) sum += ((const float*)&red[w][mt][red_lane])[red_comp];
+      dyw[j] += sum;
     }
     __syncthreads();  // red is free for the next frame
+    RTN_BTRACE_MARK(3)  // sum over the wavefronts, barrier
   };
 
   const int F = q.nframes;
@@ -371,25 +412,26 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdMul
     const float m = in_m;
     __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const float d_y_b = (in_dy[mt] + dyw[mt]) * m;
-      const float d_c_b = dc[mt] * m;
-      const float cellIn = in_gate[mt][0], inpGate = in_gate[mt][1], fgtGate = in_gate[mt][2], outGate = in_gate[mt][3];
-      const float c_b = in_pc[mt] * fgtGate + cellIn * inpGate;
+    for (int j = 0; j < PT; ++j) {
+      const float d_y_b = (in_dy[j] + dyw[j]) * m;
+      const float d_c_b = dc[j] * m;
+      const float cellIn = in_gate[j][0], inpGate = in_gate[j][1], fgtGate = in_gate[j][2], outGate = in_gate[j][3];
+      const float c_b = in_pc[j] * fgtGate + cellIn * inpGate;
       const float gc = Act<AT>::tanh(c_b);
       const float d_out = (1.f - outGate) * outGate * gc * d_y_b;
       const float d_c2 = d_c_b + outGate * d_y_b * (1.f - gc * gc);
       const float dx[4] = {E::round((1.f - cellIn * cellIn) * inpGate * d_c2), E::round((1.f - inpGate) * inpGate * cellIn * d_c2),
-                           E::round((1.f - fgtGate) * fgtGate * in_pc[mt] * d_c2), E::round(d_out)};
-      dc[mt] = fgtGate * d_c2 + dc[mt] * (1.f - m);
-      if (valid) {
+                           E::round((1.f - fgtGate) * fgtGate * in_pc[j] * d_c2), E::round(d_out)};
+      dc[j] = fgtGate * d_c2 + dc[j] * (1.f - m);
+      if (act[j]) {
 #pragma unroll
-        for (int gq = 0; gq < 4; ++gq) SN::template store<kAuxDevice>(rs, (unsigned)((io[mt] + (long long)gq * n) * ES), SN::bits(dx[gq]));
+        for (int gq = 0; gq < 4; ++gq) SN::template store<kAuxDevice>(rs, (unsigned)((io[j] + (long long)gq * n) * ES), SN::bits(dx[gq]));
       }
 #pragma unroll
-      for (int gq = 0; gq < 4; ++gq) dx0[mt][gq] = dx[gq] + dx0[mt][gq] * (1.f - m);
-      dyw[mt] *= (1.f - m);
+      for (int gq = 0; gq < 4; ++gq) dx0[j][gq] = dx[gq] + dx0[j][gq] * (1.f - m);
+      dyw[j] *= (1.f - m);
     }
+    RTN_BTRACE_MARK(5)  // pointwise part, stores of DX
     // while the derivatives travel: the inputs of the next frame, then the first read of this frame's DX
     if (f + 1 < F) fetch(frame(f + 1), f + 2 < F ? frame(f + 2) : -1);
     if (!aborted)
@@ -397,13 +439,15 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_bwd_regw(const Lstm2BwdMul
     issue(t);
   }
   gemm(frame(F - 1));
-  if (valid) {
+  RTN_BTRACE_ADD(7, (unsigned long long)delay)
+  RTN_BTRACE_FLUSH()
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      E::store(q.Dy0, idx[mt], dyw[mt]);
-      p.Dc0[idx[mt]] = dc[mt];
+  for (int j = 0; j < PT; ++j) {
+    if (act[j]) {
+      E::store(q.Dy0, idx[j], dyw[j]);
+      p.Dc0[idx[j]] = dc[j];
 #pragma unroll
-      for (int gq = 0; gq < 4; ++gq) E::store(p.dx0, io[mt] + (long long)gq * n, dx0[mt][gq]);
+      for (int gq = 0; gq < 4; ++gq) E::store(p.dx0, io[j] + (long long)gq * n, dx0[j][gq]);
     }
   }
 }

@@ -649,13 +649,20 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
 
 typedef void (*BwdRegwKernel)(const Lstm2BwdMulti);
 
+// KSB: fragments of W per tile and wavefront; MT: tiles of 16 values of k per workgroup; WV: wavefronts per workgroup.
 template <typename AT>
-BwdRegwKernel bwd_regw_kernel_for(int KSB, int MT) {
-#define RTN_CASE(ks, mt) \
-  if (KSB == ks && MT == mt) return &k_lstm2_bwd_regw<AT, ks, mt>;
-  RTN_CASE(2, 1) RTN_CASE(4, 1) RTN_CASE(8, 1) RTN_CASE(16, 1) RTN_CASE(32, 1)
-  RTN_CASE(2, 2) RTN_CASE(4, 2) RTN_CASE(8, 2) RTN_CASE(16, 2) RTN_CASE(32, 2)
-  RTN_CASE(2, 4) RTN_CASE(4, 4) RTN_CASE(8, 4) RTN_CASE(16, 4)
+BwdRegwKernel bwd_regw_kernel_for(int KSB, int MT, int WV) {
+#define RTN_CASE(ks, mt, wv) \
+  if (KSB == ks && MT == mt && WV == wv) return &k_lstm2_bwd_regw<AT, ks, mt, wv>;
+  RTN_CASE(2, 1, 4) RTN_CASE(4, 1, 4) RTN_CASE(8, 1, 4) RTN_CASE(16, 1, 4) RTN_CASE(32, 1, 4)
+  RTN_CASE(2, 2, 4) RTN_CASE(4, 2, 4) RTN_CASE(8, 2, 4) RTN_CASE(16, 2, 4) RTN_CASE(32, 2, 4)
+  RTN_CASE(2, 4, 4) RTN_CASE(4, 4, 4) RTN_CASE(8, 4, 4) RTN_CASE(16, 4, 4)
+  RTN_CASE(2, 1, 8) RTN_CASE(4, 1, 8) RTN_CASE(8, 1, 8) RTN_CASE(16, 1, 8)
+  RTN_CASE(2, 2, 8) RTN_CASE(4, 2, 8) RTN_CASE(8, 2, 8) RTN_CASE(16, 2, 8)
+  RTN_CASE(2, 4, 8) RTN_CASE(4, 4, 8) RTN_CASE(8, 4, 8) RTN_CASE(16, 4, 8)
+  RTN_CASE(2, 1, 16) RTN_CASE(4, 1, 16) RTN_CASE(8, 1, 16)
+  RTN_CASE(2, 2, 16) RTN_CASE(4, 2, 16) RTN_CASE(8, 2, 16)
+  RTN_CASE(2, 4, 16) RTN_CASE(4, 4, 16) RTN_CASE(8, 4, 16)
 #undef RTN_CASE
   return nullptr;
 }
@@ -981,36 +988,45 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
   // (2..32 fragments) and all workgroups of all problems can be on the device together.
   const void* pk = nullptr;
   int KSB = 0, bwd_mt = 1;
+  (void)KSB;
   // Decomposition: batch groups of 8 or 16 rows (a workgroup's frame time grows with the rows x 4n values of DX it
-  // reads per frame at device scope) times MT tiles of 16 values of k per workgroup (more tiles: fewer workgroups, more
-  // MFMA time each).  Candidates in the order measured on MI355X (cfg3: one problem 8 x 1: 4.4 ms; two problems in one
-  // launch 8 x 2: 5.5 ms, 16 x 1: 6.5 ms, 16 x 2: 7.1 ms); the first whose workgroups are all on the device together.
+  // reads per frame at device scope), MT tiles of 16 values of k per workgroup (more tiles: fewer workgroups, more
+  // MFMA time each) and 4 or 8 wavefronts per workgroup (8: more loads in flight per CU and no register spills, but
+  // only with one tile).  Candidates in the order measured on MI355X (cfg3, ms per gradient call: one problem
+  // 8 x 1 x 8: 4.22, 8 x 1 x 4: 4.37; two problems in one launch 8 x 2 x 4: 5.5, 16 x 1 x 8: 6.1, 16 x 1 x 4: 6.5,
+  // 8 x 2 x 8: 6.6, 16 x 2 x 4: 7.1); the first whose workgroups are all on the device together.
   const long env_rows = env_long("RTN_LSTM2_BWD_ROWS", 0);
-  int rows_per_group = 16;
+  int rows_per_group = 16, bwd_waves = kWaves;
   {
     const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
     const int S = 4 * n / KM;
-    const bool shape_ok = mfma && (4 * n) % KM == 0 && S % kWaves == 0;
-    KSB = shape_ok ? S / kWaves : 0;
     const long bwd_kernel = env_long("RTN_LSTM2_BWD_KERNEL", 0);  // 0 auto, 1 per-frame launches, 2 persistent
-    if (shape_ok && bwd_kernel != 1 && device_info().cooperative && count <= kMaxBwdMulti) {
+    if (mfma && (4 * n) % KM == 0 && bwd_kernel != 1 && device_info().cooperative && count <= kMaxBwdMulti) {
       const long env_mt = env_long("RTN_LSTM2_BWD_MT", 0);
-      const int candidates[][2] = {{8, 1}, {8, 2}, {16, 1}, {16, 2}, {8, 4}, {16, 4}};
+      const long env_waves = env_long("RTN_LSTM2_BWD_WAVES", 0);
+      // (rows per group, tiles per workgroup, wavefronts per workgroup)
+      const int candidates[][3] = {{8, 1, 8}, {8, 1, 4}, {8, 2, 4}, {16, 1, 8}, {16, 1, 4}, {16, 2, 4}, {8, 4, 4}, {16, 4, 4}};
       for (const auto& cand : candidates) {
         const int rows = cand[0], mt = cand[1];
+        const int wv = env_waves ? (int)env_waves : cand[2];
         if (env_mt && mt != env_mt) continue;
         const bool rows_forced = env_rows >= 1 && env_rows <= 16;  // an explicit row count replaces the candidates' own
         if (rows_forced && rows != 8) continue;                    // (one pass per MT is enough then)
         const int use_rows = rows_forced ? (int)env_rows : rows;
-        if (mt * KSB > 64 || (n / 16) % mt) continue;
-        BwdRegwKernel kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(KSB, mt) : bwd_regw_kernel_for<float>(KSB, mt);
+        if (wv != 4 && wv != 8 && wv != 16) continue;
+        if (S % wv) continue;
+        const int ksb = S / wv;
+        if (mt * ksb > 64 || (n / 16) % mt) continue;
+        BwdRegwKernel kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(ksb, mt, wv) : bwd_regw_kernel_for<float>(ksb, mt, wv);
         if (!kfn) continue;
         int per_cu = 0;
-        RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kfn, kWgThreads, 0));
+        RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kfn, 64 * wv, 0));
         const long long groups_needed = (B + use_rows - 1) / use_rows;
         if ((long long)per_cu * device_info().cus >= (long long)count * groups_needed * (n / (16 * mt))) {
           pk = (const void*)kfn;
           bwd_mt = mt;
+          bwd_waves = wv;
+          KSB = ksb;
           rows_per_group = use_rows;
           break;
         }
@@ -1080,7 +1096,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       q.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);
     }
     void* args[] = {(void*)&multi};
-    RTN_HIP(hipLaunchCooperativeKernel(pk, dim3((unsigned)(count * multi.wgs_each)), dim3(kWgThreads), args, 0, stream));
+    RTN_HIP(hipLaunchCooperativeKernel(pk, dim3((unsigned)(count * multi.wgs_each)), dim3((unsigned)(64 * bwd_waves)), args, 0, stream));
     for (int k = 0; k < count; ++k) {
       const BwdJob& j = jobs[(size_t)k];
       if (j.num_steps == T) continue;
@@ -1206,6 +1222,16 @@ int rtn_native_lstm2_bwd_multi(const rtn_lstm2_bwd_call* calls, int32_t count, i
   g_last_error.clear();
   return bwd_calls(calls, count, T, B, n, dtype, workspace, workspace_bytes, hip_stream);
 }
+
+#ifdef RTN_LSTM2_TRACE
+// Instrumented builds only: the per-workgroup phase times of the last persistent gradient launch.
+__attribute__((visibility("default"))) int rtn_debug_bwd_trace(unsigned long long* out, int workgroups) {
+  if (workgroups > 1024) workgroups = 1024;
+  RTN_HIP(hipDeviceSynchronize());
+  RTN_HIP(hipMemcpyFromSymbol(out, HIP_SYMBOL(rtn::g_bwd_trace), (size_t)workgroups * 8 * sizeof(unsigned long long)));
+  return RTN_OK;
+}
+#endif
 
 int rtn_native_lstm2_fwd_status(const void* workspace, void* hip_stream) {
   g_last_error.clear();
