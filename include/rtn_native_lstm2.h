@@ -232,6 +232,18 @@ int rtn_lstm_generic_base_fwd(const void* Z, const void* V_h, const float* c, co
                               size_t workspace_bytes, void* hip_stream);
 size_t rtn_lstm_generic_base_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode);
 
+/*
+ * Gradient op of LstmGenericBase (c_bw_code returnn/native_op.py:525-574, lstm_bwd_kernel :430-485; inputs as its
+ * grad_input_map :374-378): V_h, c, i, the forward results Y and H, DY [T,B,n], Dd [B,n] (float32)  ->  DZ [T,B,4n],
+ * DV_h [n,4n] (float32), Dc [B,n] (float32).  Runs on the NativeLstm2 gradient kernels; the reference overwrites H
+ * with DZ and DY with a working array, here both inputs are left alone.  LstmLowMem has no gradient entry point: its
+ * reference gradient (:838-1026) is marked unfinished where masks are concerned (:965).
+ */
+int rtn_lstm_generic_base_bwd(const void* V_h, const float* c, const float* i, const void* Y, const void* H, const void* DY,
+                              const float* Dd, void* DZ, float* DV_h, float* Dc, int64_t T, int32_t B, int32_t n,
+                              int32_t dtype, void* workspace, size_t workspace_bytes, void* hip_stream);
+size_t rtn_lstm_generic_base_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype);
+
 int rtn_lstm_low_mem_fwd(const void* X, const void* W, const void* b, const void* y0, const float* c0, const float* i,
                          int32_t start, int32_t step, void* Y, float* C, float* d, int64_t T, int32_t B, int32_t n_in,
                          int32_t n, int32_t dtype, int32_t mode, void* workspace, size_t workspace_bytes,
@@ -261,7 +273,7 @@ const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int3
 const char* rtn_native_lstm2_describe_multi_plan(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype,
                                                  int32_t mode);
 
-/* ABI version of this header. */
+/* ABI version of this header: 5. */
 int rtn_native_lstm2_abi_version(void);
 
 #ifdef __cplusplus

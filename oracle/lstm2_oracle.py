@@ -52,6 +52,9 @@ def _load():
             gb = getattr(lib, "lstm_generic_base_oracle_fwd_" + suffix)
             gb.restype = ctypes.c_int
             gb.argtypes = [ptr] * 7 + [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
+            gbb = getattr(lib, "lstm_generic_base_oracle_bwd_" + suffix)
+            gbb.restype = ctypes.c_int
+            gbb.argtypes = [ptr] * 10 + [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
             lm = getattr(lib, "lstm_low_mem_oracle_fwd_" + suffix)
             lm.restype = ctypes.c_int
             lm.argtypes = [ptr] * 6 + [ctypes.c_int32, ctypes.c_int32] + [ptr] * 3 + [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
@@ -338,6 +341,37 @@ def lstm_generic_base_fwd(Z, V_h, c, i, *, dtype=numpy.float32):
     if rc != 0:
         raise ValueError("oracle: LstmGenericBase needs T > 0")
     return Y, H, d
+
+
+def lstm_generic_base_bwd(V_h, c, i, Y, H, DY, Dd, *, dtype=numpy.float32):
+    """
+    Reference semantics of the ``LstmGenericBase`` gradient op (returnn/native_op.py:430-485, :525-574; inputs as its
+    ``grad_input_map`` :374-378).
+
+    :param Y, H: results of the forward pass
+    :param DY: [T,B,n] error signal on Y; Dd: [B,n] error signal on the final cell state
+    :return: DZ [T,B,4n], DV_h [n,4n], Dc [B,n]
+    """
+    dtype, suffix, ctype = _suffix(dtype)
+    i = numpy.ascontiguousarray(i, dtype=dtype)
+    c = numpy.ascontiguousarray(c, dtype=dtype)
+    T, B = i.shape
+    n = c.shape[1]
+    V_h = _prep(V_h, dtype, (n, 4 * n), "V_h")
+    Y = _prep(Y, dtype, (T, B, n), "Y")
+    H = _prep(H, dtype, (T, B, 4 * n), "H")
+    DY = _prep(DY, dtype, (T, B, n), "DY")
+    Dd = _prep(Dd, dtype, (B, n), "Dd")
+    DZ = numpy.zeros((T, B, 4 * n), dtype=dtype)
+    DV_h = numpy.zeros((n, 4 * n), dtype=dtype)
+    Dc = numpy.zeros((B, n), dtype=dtype)
+    p = ctypes.POINTER(ctype)
+    rc = getattr(_load(), "lstm_generic_base_oracle_bwd_" + suffix)(
+        *(a.ctypes.data_as(p) for a in (V_h, c, i, Y, H, DY, Dd, DZ, DV_h, Dc)), T, B, n
+    )
+    if rc != 0:
+        raise ValueError("oracle: LstmGenericBase gradient needs T > 0")
+    return DZ, DV_h, Dc
 
 
 def lstm_low_mem_fwd(X, W, b, y0, c0, i, start: int = 0, step: int = 1, *, dtype=numpy.float32):

@@ -8,10 +8,17 @@
  * LstmLowMem: returnn/native_op.py:771-836 (c_fw_code: per visited frame intern = [X[t], Y[t-step] or y0] * W + b,
  *   then the kernel; d = C of the last visited frame) and :624-655 (lstm_kernel).
  *
+ * LstmGenericBase gradient: returnn/native_op.py:525-574 (c_bw_code: frames in descending order; the error of the
+ *   output is DY[x] plus DZ[x+1] * V_h^T; the kernel; then DV_h = sum_x Y[x]^T DZ[x+1] and Dc = the error that reaches
+ *   the initial cell state) and :430-485 (lstm_bwd_kernel: works on the stored cell state and gates, recovers
+ *   tanh(cell-in) as (state - forget * old_state) / max(input, 1e-16), all gate errors multiplied by the mask).
+ *
  * Parity status: PINNED by tests/test_oracle_siblings.py -- the reference's own closed-form vector for LstmLowMem
  * (tests/test_TFNativeOp.py:264-297), its all-zero run of the LstmGenericBase cell (:234-250: zero input, zero state
  * => zero output), an independently written float64 loop with masks in the middle of sequences, torch.nn.LSTM on
- * full-length batches, and agreement with the (pinned) NativeLstm2 oracle where the semantics coincide.
+ * full-length batches, and agreement with the (pinned) NativeLstm2 oracle where the semantics coincide; the gradient
+ * by central finite differences of the pinned forward oracle (all three inputs, masks with holes) and by autograd
+ * through an independent torch restatement of the forward pass.
  */
 #include <math.h>
 #include <stdint.h>
@@ -120,3 +127,66 @@ DEFINE_GENERIC_BASE(lstm_generic_base_oracle_fwd_f64, double, exp, tanh)
 
 DEFINE_LOW_MEM(lstm_low_mem_oracle_fwd_f32, float, expf, tanhf)
 DEFINE_LOW_MEM(lstm_low_mem_oracle_fwd_f64, double, exp, tanh)
+
+/* DZ [T,B,4n], DV_h [n,4n], Dc [B,n] from V_h, c, mask, Y, H (the forward pass's results), DY, Dd. */
+#define DEFINE_GENERIC_BASE_BWD(NAME, REAL, TANHF)                                                                 \
+  int NAME(const REAL* V_h, const REAL* c, const REAL* mask, const REAL* Y, const REAL* H, const REAL* DY,          \
+           const REAL* Dd, REAL* DZ, REAL* DV_h, REAL* Dc, int64_t T, int32_t B, int32_t n) {                       \
+    if (T <= 0) return 1;                                                                                          \
+    const int64_t bn = (int64_t)B * n, n4 = (int64_t)n * 4, bn4 = bn * 4;                                          \
+    REAL* eps = (REAL*)malloc(sizeof(REAL) * (size_t)T * (size_t)bn); /* the reference works in place on DY */      \
+    if (!eps) return 3;                                                                                            \
+    memcpy(eps, DY, sizeof(REAL) * (size_t)T * (size_t)bn);                                                        \
+    memcpy(DZ, H, sizeof(REAL) * (size_t)T * (size_t)bn4); /* ... and in place on H */                              \
+    for (int64_t x = T - 1; x >= 0; --x) {                                                                         \
+      REAL* delta = DZ + x * bn4;                                                                                  \
+      REAL* epsilon = eps + x * bn;                                                                                \
+      if (x < T - 1) { /* epsilon += DZ[x+1] * V_h^T */                                                             \
+        const REAL* dn = DZ + (x + 1) * bn4;                                                                       \
+        for (int64_t b = 0; b < B; ++b)                                                                            \
+          for (int64_t k = 0; k < n; ++k) {                                                                        \
+            REAL acc = 0;                                                                                          \
+            const REAL* vr = V_h + k * n4;                                                                         \
+            const REAL* dr = dn + b * n4;                                                                          \
+            for (int64_t j = 0; j < n4; ++j) acc += dr[j] * vr[j];                                                 \
+            epsilon[b * n + k] += acc;                                                                             \
+          }                                                                                                        \
+      }                                                                                                            \
+      const REAL* next_epsilon = (x == T - 1) ? Dd : eps + (x + 1) * bn;                                           \
+      for (int64_t idx = 0; idx < bn; ++idx) {                                                                     \
+        const int64_t b = idx / n;                                                                                 \
+        const int64_t start = b * n4 + idx % n;                                                                    \
+        const REAL i_batch = mask[x * B + b];                                                                      \
+        const REAL inpGate = delta[start + n], fgtGate = delta[start + 2 * n], outGate = delta[start + 3 * n];     \
+        const REAL oldState = x > 0 ? (DZ + (x - 1) * bn4)[start] : c[idx]; /* H[x-1] is still untouched */         \
+        const REAL state = delta[start];                                                                           \
+        const REAL e = epsilon[idx];                                                                               \
+        const REAL gc = TANHF(state);                                                                              \
+        const REAL floor_ = (REAL)1e-16;                                                                           \
+        const REAL gzc = (state - fgtGate * oldState) / (inpGate > floor_ ? inpGate : floor_);                     \
+        delta[start + 3 * n] = outGate * ((REAL)1 - outGate) * gc * e * i_batch;                                   \
+        REAL epsilon_c = ((REAL)1 - gc * gc) * outGate * e;                                                        \
+        epsilon_c += next_epsilon[idx];                                                                            \
+        epsilon[idx] = epsilon_c * fgtGate * i_batch + next_epsilon[idx] * ((REAL)1 - i_batch);                    \
+        delta[start] = inpGate * ((REAL)1 - gzc * gzc) * epsilon_c * i_batch;                                      \
+        delta[start + 2 * n] = fgtGate * ((REAL)1 - fgtGate) * oldState * epsilon_c * i_batch;                     \
+        delta[start + n] = inpGate * ((REAL)1 - inpGate) * gzc * epsilon_c * i_batch;                              \
+      }                                                                                                            \
+    }                                                                                                              \
+    /* DV_h = Y[0..T-2]^T * DZ[1..T-1] */                                                                          \
+    memset(DV_h, 0, sizeof(REAL) * (size_t)n * (size_t)n4);                                                        \
+    for (int64_t x = 0; x + 1 < T; ++x)                                                                            \
+      for (int64_t b = 0; b < B; ++b)                                                                              \
+        for (int64_t k = 0; k < n; ++k) {                                                                          \
+          const REAL yv = Y[(x * B + b) * n + k];                                                                  \
+          const REAL* dr = DZ + (x + 1) * bn4 + b * n4;                                                            \
+          REAL* out = DV_h + k * n4;                                                                               \
+          for (int64_t j = 0; j < n4; ++j) out[j] += yv * dr[j];                                                   \
+        }                                                                                                          \
+    memcpy(Dc, eps, sizeof(REAL) * (size_t)bn);                                                                    \
+    free(eps);                                                                                                     \
+    return 0;                                                                                                      \
+  }
+
+DEFINE_GENERIC_BASE_BWD(lstm_generic_base_oracle_bwd_f32, float, tanhf)
+DEFINE_GENERIC_BASE_BWD(lstm_generic_base_oracle_bwd_f64, double, tanh)

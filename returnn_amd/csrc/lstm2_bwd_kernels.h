@@ -21,7 +21,41 @@ struct Lstm2BwdParams {
   void* dx0;   // [B,4n] AT: DX of each sequence's first processed valid frame
   long long T;
   int B, n;
+  int op_flags;  // OpFlags: kOpNoCarry, kOpH0IsCell select the gradient of LstmGenericBase (returnn/native_op.py:430-485)
+  int pad_;
 };
+
+// Gate derivatives of one (sequence, cell) pair in one frame (returnn/native_op.py:1148-1172).
+//   h0: first block of H -- tanh(cell-in), or with kOpH0IsCell the cell state, from which tanh(cell-in) is recovered as
+//   the reference's gradient kernel does: (state - forget * old_state) / max(input, 1e-16)  (:462-463)
+//   d_y_b, d_c_b: error of the output and of the cell state, already multiplied by the mask
+template <typename AT>
+__device__ __forceinline__ float bwd_cell(int op_flags, float h0, float inpGate, float fgtGate, float outGate, float prev_c, float d_y_b,
+                                          float d_c_b, float (&dx)[4]) {
+  using E = Elem<AT>;
+  float cellIn, gc;
+  if (op_flags & kOpH0IsCell) {
+    gc = Act<AT>::tanh(h0);
+    cellIn = (h0 - fgtGate * prev_c) / fmaxf(inpGate, 1e-16f);
+  } else {
+    cellIn = h0;
+    gc = Act<AT>::tanh(prev_c * fgtGate + cellIn * inpGate);
+  }
+  const float d_c2 = d_c_b + outGate * d_y_b * (1.f - gc * gc);
+  dx[0] = E::round((1.f - cellIn * cellIn) * inpGate * d_c2);
+  dx[1] = E::round((1.f - inpGate) * inpGate * cellIn * d_c2);
+  dx[2] = E::round((1.f - fgtGate) * fgtGate * prev_c * d_c2);
+  dx[3] = E::round((1.f - outGate) * outGate * gc * d_y_b);
+  return d_c2;
+}
+
+// Cell state of the frame before: the forward pass's C, or with kOpH0IsCell the first block of H of that frame.
+template <typename AT>
+__device__ __forceinline__ float bwd_prev_cell(const Lstm2BwdParams& p, long long prev_t, long long idx, long long io) {
+  if (prev_t < 0) return p.c0[idx];
+  if (p.op_flags & kOpH0IsCell) return Elem<AT>::load(p.H, prev_t * (long long)p.B * p.n * 4 + io);
+  return p.C[prev_t * (long long)p.B * p.n + idx];
+}
 
 // Pointwise part of one frame t: gate derivatives from the stored activations, cell error carried on.
 // prev_t < 0: the frame before is the initial state (prev_c = c0).
@@ -40,25 +74,18 @@ __global__ void k_bwd_pointwise(Lstm2BwdParams p, long long t, long long prev_t)
   const float d_y_b = (E::load(p.DY, t * bn + idx) + dyw) * m;
   const float dc = p.Dc0[idx];
   const float d_c_b = dc * m;
-  const float prev_c = prev_t >= 0 ? p.C[prev_t * bn + idx] : p.c0[idx];
-  const float cellIn = E::load(p.H, fo), inpGate = E::load(p.H, fo + n), fgtGate = E::load(p.H, fo + 2 * n),
-              outGate = E::load(p.H, fo + 3 * n);
-  const float c_b = prev_c * fgtGate + cellIn * inpGate;
-  const float gc = Act<AT>::tanh(c_b);
-  const float d_out = (1.f - outGate) * outGate * gc * d_y_b;
-  const float d_c2 = d_c_b + outGate * d_y_b * (1.f - gc * gc);
-  const float d_cin = (1.f - cellIn * cellIn) * inpGate * d_c2;
-  const float d_inp = (1.f - inpGate) * inpGate * cellIn * d_c2;
-  const float d_fgt = (1.f - fgtGate) * fgtGate * prev_c * d_c2;
+  const float prev_c = bwd_prev_cell<AT>(p, prev_t, idx, io);
+  const float fgtGate = E::load(p.H, fo + 2 * n);
+  float dx[4];
+  const float d_c2 = bwd_cell<AT>(p.op_flags, E::load(p.H, fo), E::load(p.H, fo + n), fgtGate, E::load(p.H, fo + 3 * n), prev_c, d_y_b, d_c_b, dx);
   p.Dc0[idx] = fgtGate * d_c2 + dc * (1.f - m);
-  const float dx[4] = {E::round(d_cin), E::round(d_inp), E::round(d_fgt), E::round(d_out)};
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
     E::store(p.DX, fo + g * n, dx[g]);
     const float old = E::load(p.dx0, io + g * n);
     E::store(p.dx0, io + g * n, dx[g] + old * (1.f - m));
   }
-  p.dyw[idx] = dyw * (1.f - m);
+  p.dyw[idx] = (p.op_flags & kOpNoCarry) ? 0.f : dyw * (1.f - m);
 }
 
 // One launch per visited frame on MFMA shapes (n % 16 == 0): the recurrent GEMM of the frame processed before
@@ -139,25 +166,18 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
       const float d_y_b = (E::load(p.DY, t * bn + idx) + dyw) * m;
       const float dc = p.Dc0[idx];
       const float d_c_b = dc * m;
-      const float prev_c = prev_t >= 0 ? p.C[prev_t * bn + idx] : p.c0[idx];
-      const float cellIn = E::load(p.H, fo), inpGate = E::load(p.H, fo + n), fgtGate = E::load(p.H, fo + 2 * n),
-                  outGate = E::load(p.H, fo + 3 * n);
-      const float c_b = prev_c * fgtGate + cellIn * inpGate;
-      const float gc = Act<AT>::tanh(c_b);
-      const float d_out = (1.f - outGate) * outGate * gc * d_y_b;
-      const float d_c2 = d_c_b + outGate * d_y_b * (1.f - gc * gc);
-      const float d_cin = (1.f - cellIn * cellIn) * inpGate * d_c2;
-      const float d_inp = (1.f - inpGate) * inpGate * cellIn * d_c2;
-      const float d_fgt = (1.f - fgtGate) * fgtGate * prev_c * d_c2;
+      const float prev_c = bwd_prev_cell<AT>(p, prev_t, idx, io);
+      const float fgtGate = E::load(p.H, fo + 2 * n);
+      float dx[4];
+      const float d_c2 = bwd_cell<AT>(p.op_flags, E::load(p.H, fo), E::load(p.H, fo + n), fgtGate, E::load(p.H, fo + 3 * n), prev_c, d_y_b, d_c_b, dx);
       p.Dc0[idx] = fgtGate * d_c2 + dc * (1.f - m);
-      const float dx[4] = {E::round(d_cin), E::round(d_inp), E::round(d_fgt), E::round(d_out)};
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         E::store(p.DX, fo + g * n, dx[g]);
         const float old = E::load(p.dx0, io + g * n);
         E::store(p.dx0, io + g * n, dx[g] + old * (1.f - m));
       }
-      dyw *= (1.f - m);
+      dyw = (p.op_flags & kOpNoCarry) ? 0.f : dyw * (1.f - m);
     }
     p.dyw[idx] = dyw;
   }
@@ -312,7 +332,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) in_gate[j][gq] = E::load(p.H, fo + (long long)gq * n);
       in_dy[j] = E::load(p.DY, t * bn + idx[j]);
-      in_pc[j] = prev_t >= 0 ? p.C[prev_t * bn + idx[j]] : p.c0[idx[j]];
+      in_pc[j] = bwd_prev_cell<AT>(p, prev_t, idx[j], io[j]);
     }
     in_m = p.mask[t * p.B + b];
   };
@@ -415,13 +435,9 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     for (int j = 0; j < PT; ++j) {
       const float d_y_b = (in_dy[j] + dyw[j]) * m;
       const float d_c_b = dc[j] * m;
-      const float cellIn = in_gate[j][0], inpGate = in_gate[j][1], fgtGate = in_gate[j][2], outGate = in_gate[j][3];
-      const float c_b = in_pc[j] * fgtGate + cellIn * inpGate;
-      const float gc = Act<AT>::tanh(c_b);
-      const float d_out = (1.f - outGate) * outGate * gc * d_y_b;
-      const float d_c2 = d_c_b + outGate * d_y_b * (1.f - gc * gc);
-      const float dx[4] = {E::round((1.f - cellIn * cellIn) * inpGate * d_c2), E::round((1.f - inpGate) * inpGate * cellIn * d_c2),
-                           E::round((1.f - fgtGate) * fgtGate * in_pc[j] * d_c2), E::round(d_out)};
+      const float fgtGate = in_gate[j][2];
+      float dx[4];
+      const float d_c2 = bwd_cell<AT>(p.op_flags, in_gate[j][0], in_gate[j][1], fgtGate, in_gate[j][3], in_pc[j], d_y_b, d_c_b, dx);
       dc[j] = fgtGate * d_c2 + dc[j] * (1.f - m);
       if (act[j]) {
 #pragma unroll
@@ -429,7 +445,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       }
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) dx0[j][gq] = dx[gq] + dx0[j][gq] * (1.f - m);
-      dyw[j] *= (1.f - m);
+      dyw[j] = (p.op_flags & kOpNoCarry) ? 0.f : dyw[j] * (1.f - m);
     }
     RTN_BTRACE_MARK(5)  // pointwise part, stores of DX
     // while the derivatives travel: the inputs of the next frame, then the first read of this frame's DX

@@ -720,7 +720,7 @@ using namespace rtn;
 
 extern "C" {
 
-int rtn_native_lstm2_abi_version(void) { return 4; }
+int rtn_native_lstm2_abi_version(void) { return 5; }
 
 const char* rtn_last_error(void) { return g_last_error.c_str(); }
 
@@ -926,7 +926,7 @@ struct BwdJob {
 // cooperative launch (16-row batch groups when 8-row groups of all problems would not find a CU each); otherwise they
 // are enqueued one after the other.
 int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, int32_t n, int32_t dtype, void* workspace,
-              size_t workspace_bytes, void* hip_stream) {
+              size_t workspace_bytes, void* hip_stream, int op_flags = 0) {
   int rc = check_dims(T, B, n, dtype);
   if (rc != RTN_OK) return rc;
   if (count < 0 || (count > 0 && !calls)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: bad call list");
@@ -1035,7 +1035,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     if (!pk && count > 1) {
       // no joint launch: one call after the other, each with its own slice of the workspace
       for (int k = 0; k < count; ++k) {
-        rc = bwd_calls(calls + k, 1, T, B, n, dtype, (unsigned char*)workspace + (size_t)k * lay.total, lay.total, hip_stream);
+        rc = bwd_calls(calls + k, 1, T, B, n, dtype, (unsigned char*)workspace + (size_t)k * lay.total, lay.total, hip_stream, op_flags);
         if (rc != RTN_OK) return rc;
       }
       return RTN_OK;
@@ -1057,6 +1057,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     p.dyw = (float*)(j.ws + lay.off_dyw);
     p.dx0 = j.ws + lay.off_dx0;
     p.T = T; p.B = B; p.n = n;
+    p.op_flags = op_flags;
     hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)j.ws, 0u, (long long)(lay.total / 4));
     RTN_HIP(hipGetLastError());
     // returnn/native_op.py:1383-1407: which frames are visited, and in which order
@@ -1210,6 +1211,38 @@ int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const f
   g_last_error.clear();
   const rtn_lstm2_bwd_call call = {W, y0, c0, i, start, step, Y, C, H, DY, Dd, DX, DW, Dy0, Dc0};
   return bwd_calls(&call, 1, T, B, n, dtype, workspace, workspace_bytes, hip_stream);
+}
+
+size_t rtn_lstm_generic_base_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype) {
+  const size_t bwd = rtn_native_lstm2_bwd_workspace_bytes(T, B, n, dtype);
+  if (bwd == 0) return 0;
+  // gradient workspace | zero initial output [B,n] | error of the initial output [B,n] (the op has neither)
+  return align_up(bwd, 256) + 2 * align_up((size_t)B * n * esize(dtype), 256);
+}
+
+int rtn_lstm_generic_base_bwd(const void* V_h, const float* c, const float* i, const void* Y, const void* H, const void* DY,
+                              const float* Dd, void* DZ, float* DV_h, float* Dc, int64_t T, int32_t B, int32_t n, int32_t dtype,
+                              void* workspace, size_t workspace_bytes, void* hip_stream) {
+  g_last_error.clear();
+  int rc = check_dims(T, B, n, dtype);
+  if (rc != RTN_OK) return rc;
+  if (T == 0) return fail(RTN_ERR_SHAPE, "LstmGenericBase gradient: needs T > 0");  // returnn/native_op.py:547
+  const size_t need = rtn_lstm_generic_base_bwd_workspace_bytes(T, B, n, dtype);
+  if (!workspace || workspace_bytes < need)
+    return fail(RTN_ERR_WORKSPACE, "LstmGenericBase gradient: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
+  if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "LstmGenericBase gradient: workspace must be 16-byte aligned");
+  const size_t bwd = align_up(rtn_native_lstm2_bwd_workspace_bytes(T, B, n, dtype), 256);
+  const size_t state_bytes = align_up((size_t)B * n * esize(dtype), 256);
+  unsigned char* ws = (unsigned char*)workspace;
+  void* y0 = ws + bwd;
+  void* Dy0 = ws + bwd + state_bytes;
+  if ((long long)B * n > 0) {
+    hipLaunchKernelGGL(k_fill_u32, dim3(64), dim3(256), 0, (hipStream_t)hip_stream, (unsigned*)y0, 0u, (long long)(state_bytes / 4));
+    RTN_HIP(hipGetLastError());
+  }
+  // the cell states are the first block of H (kOpH0IsCell); the C argument is not read then
+  const rtn_lstm2_bwd_call call = {V_h, y0, c, i, 0, 1, Y, (const float*)H, H, DY, Dd, DZ, DV_h, Dy0, Dc};
+  return bwd_calls(&call, 1, T, B, n, dtype, workspace, bwd, hip_stream, kOpNoCarry | kOpH0IsCell);
 }
 
 size_t rtn_native_lstm2_bwd_multi_workspace_bytes(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype) {

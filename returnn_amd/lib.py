@@ -47,6 +47,8 @@ SYMBOLS = (
     "rtn_native_lstm2_bwd_multi_workspace_bytes",
     "rtn_lstm_generic_base_fwd",
     "rtn_lstm_generic_base_fwd_workspace_bytes",
+    "rtn_lstm_generic_base_bwd",
+    "rtn_lstm_generic_base_bwd_workspace_bytes",
     "rtn_lstm_low_mem_fwd",
     "rtn_lstm_low_mem_fwd_workspace_bytes",
     "rtn_native_lstm2_last_output",
@@ -144,6 +146,10 @@ def load() -> ctypes.CDLL:
         lib.rtn_lstm_generic_base_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, vp, sz, vp]
         lib.rtn_lstm_generic_base_fwd_workspace_bytes.restype = sz
         lib.rtn_lstm_generic_base_fwd_workspace_bytes.argtypes = [i64, i32, i32, i32, i32]
+        lib.rtn_lstm_generic_base_bwd.restype = ctypes.c_int
+        lib.rtn_lstm_generic_base_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, vp, sz, vp]
+        lib.rtn_lstm_generic_base_bwd_workspace_bytes.restype = sz
+        lib.rtn_lstm_generic_base_bwd_workspace_bytes.argtypes = [i64, i32, i32, i32]
         lib.rtn_lstm_low_mem_fwd.restype = ctypes.c_int
         lib.rtn_lstm_low_mem_fwd.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, vp]
         lib.rtn_lstm_low_mem_fwd_workspace_bytes.restype = sz

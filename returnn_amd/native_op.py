@@ -170,6 +170,14 @@ class LstmGenericBase(NativeOpGenBase):
         {"name": "d", "ndim": 2, "shape": ((2, 0), (2, 1)), "need_contiguous": True},
     )
     c_abi_fw = "rtn_lstm_generic_base_fwd"
+    c_abi_bw = "rtn_lstm_generic_base_bwd"
+
+    # noinspection PyPep8Naming
+    @classmethod
+    def grad_input_map(cls, Z, V_h, c, i, Y, H, d, DY, DH, Dd):
+        """What the gradient op consumes (returnn/native_op.py:374-378)."""
+        del Z, d, DH
+        return V_h, c, i, Y, H, DY, Dd
 
 
 class LstmLowMem(NativeOpGenBase):

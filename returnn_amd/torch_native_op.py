@@ -542,6 +542,64 @@ class NativeLstm2Function(torch.autograd.Function):
         return dX, dW, dy0, dc0, None, None, None
 
 
+def lstm_generic_base_grad(V_h, c, i, Y, H, DY, Dd):
+    """
+    The gradient op of ``LstmGenericBase`` on HIP tensors (returnn/native_op.py:430-485, :525-574; arguments as its
+    ``grad_input_map`` :374-378).
+
+    :return: DZ [T,B,4n] in the element type of Y; DV_h [n,4n] and Dc [B,n] in float32
+    """
+    if not Y.is_cuda:
+        raise RuntimeError("LstmGenericBase gradient: this build implements the op for HIP (MI355X) tensors only; got CPU tensors.")
+    bf16 = Y.dtype == torch.bfloat16
+    act = torch.bfloat16 if bf16 else torch.float32
+    device = Y.device
+    V_h, Y, H, DY = (t.to(act).contiguous() for t in (V_h, Y, H, DY))
+    c, i, Dd = (t.to(torch.float32).contiguous() for t in (c, i, Dd))
+    T, B = i.shape
+    n = c.shape[1]
+    expect = {"V_h": (n, 4 * n), "c": (B, n), "Y": (T, B, n), "H": (T, B, 4 * n), "DY": (T, B, n), "Dd": (B, n)}
+    for name, t in (("V_h", V_h), ("c", c), ("Y", Y), ("H", H), ("DY", DY), ("Dd", Dd)):
+        if tuple(t.shape) != expect[name]:
+            raise RuntimeError("LstmGenericBase gradient: %s has shape %s, expected %s" % (name, tuple(t.shape), expect[name]))
+        if t.device != device:
+            raise RuntimeError("LstmGenericBase gradient: %s is on %s but Y is on %s" % (name, t.device, device))
+    lib = _lib.load()
+    dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
+    with torch.cuda.device(device):
+        DZ = torch.empty((T, B, 4 * n), dtype=act, device=device)
+        DV_h = torch.empty((n, 4 * n), dtype=torch.float32, device=device)
+        Dc = torch.empty((B, n), dtype=torch.float32, device=device)
+        ws = torch.empty((max(int(lib.rtn_lstm_generic_base_bwd_workspace_bytes(T, B, n, dtype)), 256),), dtype=torch.uint8, device=device)
+        rc = lib.rtn_lstm_generic_base_bwd(
+            V_h.data_ptr(), c.data_ptr(), i.data_ptr(), Y.data_ptr(), H.data_ptr(), DY.data_ptr(), Dd.data_ptr(), DZ.data_ptr(),
+            DV_h.data_ptr(), Dc.data_ptr(), T, B, n, dtype, ws.data_ptr(), ws.numel(), torch.cuda.current_stream(device).cuda_stream,
+        )  # fmt: skip
+    _lib.check(rc)
+    return DZ, DV_h, Dc
+
+
+class LstmGenericBaseFunction(torch.autograd.Function):
+    """``LstmGenericBase`` with its gradient: ``Y, H, d = LstmGenericBaseFunction.apply(Z, V_h, c, i)``; gradients flow from
+    Y and d to Z, V_h and c (H is a non-differentiable output, the mask gets none)."""
+
+    @staticmethod
+    def forward(ctx, Z, V_h, c, i):
+        Y, H, d = make_op(native_op.LstmGenericBase)(Z, V_h, c, i)
+        ctx.save_for_backward(V_h, c, i, Y, H)
+        ctx.in_dtypes = (Z.dtype, V_h.dtype, c.dtype)
+        ctx.mark_non_differentiable(H)
+        return Y, H, d
+
+    @staticmethod
+    def backward(ctx, DY, _DH, Dd):
+        V_h, c, i, Y, H = ctx.saved_tensors
+        DY = torch.zeros_like(Y) if DY is None else DY
+        Dd = torch.zeros_like(c, dtype=torch.float32) if Dd is None else Dd
+        grads = lstm_generic_base_grad(V_h, c, i, Y, H, DY, Dd)
+        return (*(g.to(t) for g, t in zip(grads, ctx.in_dtypes)), None)
+
+
 class NativeLstm2PairFunction(torch.autograd.Function):
     """
     The two directions of a bidirectional layer as one differentiable call:

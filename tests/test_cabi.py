@@ -32,7 +32,7 @@ def test_header_symbols_are_exported(cabi):
 
 
 def test_abi_version(cabi):
-    assert cabi.rtn_native_lstm2_abi_version() == 4
+    assert cabi.rtn_native_lstm2_abi_version() == 5
 
 
 def test_error_codes_match_header():

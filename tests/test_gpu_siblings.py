@@ -228,3 +228,66 @@ def test_c_abi_errors():
     rc = cabi.rtn_lstm_generic_base_fwd(*gargs, T, B, n, lib.DTYPE_F32, 0, ws.data_ptr(), need, stream)
     assert rc == 0
     torch.cuda.synchronize()
+
+
+def _rel_to_max(got, want):
+    return float(numpy.abs(got - want).max()) / max(float(numpy.abs(want).max()), 1e-30)
+
+
+GRAD_SHAPES = [(7, 3, 16), (9, 20, 64), (6, 5, 20), (5, 2, 3), (12, 40, 128), (16, 32, 256)]
+
+
+@pytest.mark.parametrize("T,B,n", GRAD_SHAPES)
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_generic_base_gradient(T, B, n, dtype):
+    """
+    ``rtn_lstm_generic_base_bwd`` against the float64 oracle of the reference's gradient code, fed the GPU's own forward
+    results.  Judged like the NativeLstm2 gradient: float32 within 2e-5, bfloat16 within 2e-2 of each array's largest
+    magnitude.
+    """
+    announce("generic_base_gradient", T, B, n, dtype)
+    Z, V, c, mask = generic_base_problem(500 + T + B + n, T, B, n)
+    rng = numpy.random.default_rng(600 + T + n)
+    DY = rng.normal(0, 1, (T, B, n)).astype(numpy.float32)
+    Dd = rng.normal(0, 1, (B, n)).astype(numpy.float32)
+    get_op()
+    op = torch_native_op.make_op(native_op.LstmGenericBase)
+    Vd, DYd = to_dev(V, dtype), to_dev(DY, dtype)
+    cd, md, Ddd = to_dev(c, "f32"), to_dev(mask, "f32"), to_dev(Dd, "f32")
+    Y, H, d = op(to_dev(Z, dtype), Vd, cd, md)
+    got = torch_native_op.lstm_generic_base_grad(Vd, cd, md, Y, H, DYd, Ddd)
+    torch.cuda.synchronize()
+    f = lambda t: t.float().cpu().numpy().astype(numpy.float64)  # noqa: E731
+    want = oracle.lstm_generic_base_bwd(f(Vd), c, mask, f(Y), f(H), f(DYd), Dd, dtype=numpy.float64)
+    tol = 2e-5 if dtype == "f32" else 2e-2
+    for name, a, b in zip(("DZ", "DV_h", "Dc"), got, want):
+        assert a.shape == b.shape and numpy.all(numpy.isfinite(f(a))), name
+        assert _rel_to_max(f(a), b) <= tol, (name, _rel_to_max(f(a), b))
+
+
+def test_generic_base_gradient_through_autograd():
+    """LstmGenericBaseFunction under torch.autograd against autograd through a plain torch restatement (float64, CPU)."""
+    announce("generic_base_autograd")
+    T, B, n = 8, 5, 32
+    Z, V, c, mask = generic_base_problem(77, T, B, n)
+    rng = numpy.random.default_rng(78)
+    GY, Gd = rng.normal(0, 1, (T, B, n)), rng.normal(0, 1, (B, n))
+    ref = [torch.tensor(a.astype(numpy.float64), requires_grad=True) for a in (Z, V, c)]
+    y_prev, c_prev, ys = torch.zeros((B, n), dtype=torch.float64), ref[2], []
+    mt = torch.tensor(mask.astype(numpy.float64))
+    for t in range(T):
+        z = ref[0][t] + y_prev @ ref[1]
+        g, i, fg, o = torch.tanh(z[:, :n]), torch.sigmoid(z[:, n : 2 * n]), torch.sigmoid(z[:, 2 * n : 3 * n]), torch.sigmoid(z[:, 3 * n :])
+        m = mt[t][:, None]
+        c_new = (c_prev * fg + g * i) * m + c_prev * (1 - m)
+        y_prev, c_prev = torch.tanh(c_new) * o * m, c_new
+        ys.append(y_prev)
+    ((torch.stack(ys) * torch.tensor(GY)).sum() + (c_prev * torch.tensor(Gd)).sum()).backward()
+    get_op()
+    leaves = [to_dev(a, "f32").requires_grad_(True) for a in (Z, V, c)]
+    Y, H, d = torch_native_op.LstmGenericBaseFunction.apply(*leaves, to_dev(mask, "f32"))
+    assert not H.requires_grad
+    ((Y * to_dev(GY, "f32")).sum() + (d * to_dev(Gd, "f32")).sum()).backward()
+    torch.cuda.synchronize()
+    for name, leaf, r in zip(("Z", "V_h", "c"), leaves, ref):
+        assert _rel_to_max(leaf.grad.cpu().numpy().astype(numpy.float64), r.grad.numpy()) <= 2e-5, name

@@ -163,3 +163,74 @@ def test_siblings_float32_and_errors():
         oracle.lstm_generic_base_fwd(numpy.zeros((0, 3, 16)), r["V"], r["c0"], numpy.zeros((0, 3)))
     Y, C, d = oracle.lstm_low_mem_fwd(numpy.zeros((0, 3, 2)), r["W"], r["b"], r["y0"], r["c0"], numpy.zeros((0, 3)), 0, 1)
     assert_allclose(d, r["c0"], rtol=1e-6)
+
+
+def _generic_base_loss(Z, V, c0, mask, GY, Gd):
+    Y, H, d = oracle.lstm_generic_base_fwd(Z, V, c0, mask, dtype=numpy.float64)
+    return float((Y * GY).sum() + (d * Gd).sum())
+
+
+def test_generic_base_gradient_vs_finite_differences():
+    """Central differences of the (pinned) forward oracle, all three inputs, holes in the mask."""
+    T, B, n = 6, 3, 4
+    r = _random(41, T, B, n)
+    rng = numpy.random.default_rng(42)
+    GY, Gd = rng.normal(0, 1, (T, B, n)), rng.normal(0, 1, (B, n))
+    Y, H, d = oracle.lstm_generic_base_fwd(r["Z"], r["V"], r["c0"], r["mask"], dtype=numpy.float64)
+    GY_dirty = GY + 2.0 * (1.0 - r["mask"])[:, :, None]  # error signals on masked frames must not matter
+    DZ, DV, Dc = oracle.lstm_generic_base_bwd(r["V"], r["c0"], r["mask"], Y, H, GY_dirty, Gd, dtype=numpy.float64)
+    got = {"Z": DZ, "V": DV, "c0": Dc}
+    eps = 1e-6
+    for name in ("Z", "V", "c0"):
+        flat = r[name].reshape(-1)
+        for idx in rng.choice(flat.size, size=min(flat.size, 70), replace=False):
+            old = flat[idx]
+            flat[idx] = old + eps
+            lp = _generic_base_loss(r["Z"], r["V"], r["c0"], r["mask"], GY, Gd)
+            flat[idx] = old - eps
+            lm = _generic_base_loss(r["Z"], r["V"], r["c0"], r["mask"], GY, Gd)
+            flat[idx] = old
+            num = (lp - lm) / (2 * eps)
+            assert abs(num - got[name].reshape(-1)[idx]) <= 2e-6 * max(1.0, abs(num)), (name, idx, num, got[name].reshape(-1)[idx])
+    assert numpy.abs(DZ * (1.0 - r["mask"])[:, :, None]).max() == 0.0  # masked frames get no gradient
+
+
+def test_generic_base_gradient_vs_torch_autograd():
+    """Autograd through a plain torch restatement of the forward pass (output of the frame before as recurrent input)."""
+    import torch
+
+    T, B, n = 7, 4, 5
+    r = _random(43, T, B, n)
+    rng = numpy.random.default_rng(44)
+    GY, Gd = rng.normal(0, 1, (T, B, n)), rng.normal(0, 1, (B, n))
+    Z = torch.tensor(r["Z"], requires_grad=True)
+    V = torch.tensor(r["V"], requires_grad=True)
+    c = torch.tensor(r["c0"], requires_grad=True)
+    mask = torch.tensor(r["mask"])
+    y_prev, c_prev, ys = torch.zeros((B, n), dtype=torch.float64), c, []
+    for t in range(T):
+        z = Z[t] + y_prev @ V
+        g, i, f, o = torch.tanh(z[:, :n]), torch.sigmoid(z[:, n : 2 * n]), torch.sigmoid(z[:, 2 * n : 3 * n]), torch.sigmoid(z[:, 3 * n :])
+        m = mask[t][:, None]
+        c_new = (c_prev * f + g * i) * m + c_prev * (1 - m)
+        y_prev, c_prev = torch.tanh(c_new) * o * m, c_new
+        ys.append(y_prev)
+    ((torch.stack(ys) * torch.tensor(GY)).sum() + (c_prev * torch.tensor(Gd)).sum()).backward()
+    Y, H, d = oracle.lstm_generic_base_fwd(r["Z"], r["V"], r["c0"], r["mask"], dtype=numpy.float64)
+    DZ, DV, Dc = oracle.lstm_generic_base_bwd(r["V"], r["c0"], r["mask"], Y, H, GY, Gd, dtype=numpy.float64)
+    assert_allclose(DZ, Z.grad.numpy(), rtol=1e-8, atol=1e-10)
+    assert_allclose(DV, V.grad.numpy(), rtol=1e-8, atol=1e-10)
+    assert_allclose(Dc, c.grad.numpy(), rtol=1e-8, atol=1e-10)
+
+
+def test_generic_base_gradient_float32_close_to_float64():
+    T, B, n = 12, 3, 6
+    r = _random(45, T, B, n)
+    rng = numpy.random.default_rng(46)
+    GY, Gd = rng.normal(0, 1, (T, B, n)), rng.normal(0, 1, (B, n))
+    out = {}
+    for dt in (numpy.float32, numpy.float64):
+        Y, H, d = oracle.lstm_generic_base_fwd(r["Z"], r["V"], r["c0"], r["mask"], dtype=dt)
+        out[dt] = oracle.lstm_generic_base_bwd(r["V"], r["c0"], r["mask"], Y, H, GY, Gd, dtype=dt)
+    for a, b in zip(out[numpy.float32], out[numpy.float64]):
+        assert numpy.abs(a - b).max() <= 2e-5 * max(1.0, numpy.abs(b).max())
