@@ -126,3 +126,33 @@ def torch_lstm(X, W, y0, c0, lens=None, reverse=False):
     if reverse:
         return out[:, :, n:].numpy(), hT[1].numpy(), cT[1].numpy()
     return out.numpy(), hT[0].numpy(), cT[0].numpy()
+
+
+def torch_lstm_grads(X, W, y0, c0, lens, reverse, GY, Gd):
+    """Gradients of sum(Y*GY) + sum(c_final*Gd) through torch.nn.LSTM, mapped back to the op's layout."""
+    import torch
+
+    T, B, n4 = X.shape
+    n = n4 // 4
+    # op order: g(cell-in), i, f, o  ->  torch order: i, f, g, o
+    perm = numpy.concatenate([numpy.arange(n, 2 * n), numpy.arange(2 * n, 3 * n), numpy.arange(0, n), numpy.arange(3 * n, 4 * n)])
+    inv = numpy.argsort(perm)
+    Xt = torch.tensor(X[:, :, perm], dtype=torch.float64, requires_grad=True)
+    lstm = torch.nn.LSTM(input_size=4 * n, hidden_size=n, bias=False, bidirectional=reverse).double()
+    sfx = "_reverse" if reverse else ""
+    with torch.no_grad():
+        for s in ("", "_reverse") if reverse else ("",):
+            getattr(lstm, "weight_ih_l0" + s).copy_(torch.eye(4 * n, dtype=torch.float64))
+            getattr(lstm, "weight_hh_l0" + s).copy_(torch.tensor(W[:, perm].T.copy()))
+    k = 2 if reverse else 1
+    h0 = torch.tensor(numpy.stack([y0] * k), requires_grad=True)
+    c0_ = torch.tensor(numpy.stack([c0] * k), requires_grad=True)
+    packed = torch.nn.utils.rnn.pack_padded_sequence(Xt, torch.as_tensor(lens, dtype=torch.int64), enforce_sorted=False)
+    out, (hT, cT) = lstm(packed, (h0, c0_))
+    out, _ = torch.nn.utils.rnn.pad_packed_sequence(out, total_length=T)
+    sel = slice(n, 2 * n) if reverse else slice(0, n)
+    loss = (out[:, :, sel] * torch.tensor(GY)).sum() + (cT[k - 1] * torch.tensor(Gd)).sum()
+    loss.backward()
+    DX = Xt.grad.numpy()[:, :, inv]
+    DW = getattr(lstm, "weight_hh_l0" + sfx).grad.numpy().T[:, inv]
+    return DX, DW, h0.grad.numpy()[k - 1], c0_.grad.numpy()[k - 1]
