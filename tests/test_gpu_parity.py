@@ -389,3 +389,36 @@ def test_bounded_wait_expires_cleanly():
             rc, status, got = run_raw(*p, 0, 1, mode="persistent")
         assert rc == 0 and status == 0
         check_f32(got, oracle.native_lstm2_fwd(*p, 0, 1)[:4], "after bounded wait")
+
+
+@pytest.mark.parametrize(
+    "T,B,n,dtype",
+    [(12, 8, 2048, "bf16"), (8, 300, 256, "bf16"), (8, 513, 128, "f32"), (6, 130, 1024, "bf16"), (5, 4, 3072, "bf16"), (7, 9, 736, "f32"), (9, 1, 4096, "bf16")],
+)
+def test_wide_and_large_shapes(T, B, n, dtype):
+    """Shapes beyond the BASELINE configurations: very wide layers (W no longer fits the registers of the device: the plan
+    falls back to the LDS kernel per step), many sequences (several batch groups, partly filled last group), a width that
+    is a multiple of 32 but not of 64.  Forward against the oracle, then the gradient op on the GPU's own results."""
+    announce("wide_and_large", T, B, n, dtype)
+    p = random_problem(900 + T + B + n, T, B, n)
+    want = oracle.native_lstm2_fwd(*p, 0, 1, threads=oracle.max_threads())
+    got = run_op(*p, 0, 1, dtype=dtype)
+    (check_f32 if dtype == "f32" else check_bf16)(got, want, "wide %s" % ((T, B, n),))
+    from returnn_amd import native_op, torch_native_op
+
+    X, W, y0, c0, i = p
+    rng = numpy.random.default_rng(901)
+    DY = rng.normal(0, 1, (T, B, n)).astype(numpy.float32)
+    Dd = rng.normal(0, 1, (B, n)).astype(numpy.float32)
+    from _gpu_util import to_dev
+
+    Xd, Wd, y0d, DYd = (to_dev(a, dtype) for a in (X, W, y0, DY))
+    c0d, id_, Ddd = (to_dev(a, "f32") for a in (c0, i, Dd))
+    Y, C, H, d = torch_native_op.make_op(native_op.NativeLstm2)(Xd, Wd, y0d, c0d, id_, 0, 1)
+    grads = torch_native_op.native_lstm2_grad(Wd, y0d, c0d, id_, 0, 1, Y, C, H, DYd, Ddd)
+    torch.cuda.synchronize()
+    f = lambda t: t.float().cpu().numpy().astype(numpy.float64)  # noqa: E731
+    wantg = oracle.native_lstm2_bwd(f(Xd), f(Wd), f(y0d), c0, i, 0, 1, f(Y), f(C), f(H), f(DYd), Dd, dtype=numpy.float64)
+    for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), grads, wantg):
+        rel = float(numpy.abs(f(a) - b).max() / max(numpy.abs(b).max(), 1e-30))
+        assert rel <= (2e-5 if dtype == "f32" else 2e-2), (name, rel)
