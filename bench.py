@@ -4,7 +4,7 @@ Benchmark of the NativeLstm2 forward hot path on one MI355X.
 
     python bench.py --gpus 1 --steps K --warmup W
 
-Workload (default): BASELINE config 3, the bidirectional pair at n=1024 -- T=1000, B=32, bf16 weights and
+Workload (default): benchmark configuration cfg3 (returnn_amd/synthetic.py), the bidirectional pair at n=1024 -- T=1000, B=32, bf16 weights and
 activations with fp32 accumulate and cell state, ragged lengths in [500,1000]; one step = two op calls on
 the same inputs (step=+1 and step=-1), issued through the C ABI with inputs, outputs and workspace already
 resident in HBM.  ``value`` = timesteps x sequences processed per second = 2*T*B*K / elapsed (padded frames

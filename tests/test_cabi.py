@@ -68,7 +68,7 @@ def test_range_and_argument_errors(cabi):
 
 
 def test_workspace_and_plan(cabi):
-    # BASELINE config 3: bf16, T=1000, B=32, n=1024: persistent, all weights on chip
+    # benchmark configuration cfg3 (returnn_amd/synthetic.py): bf16, T=1000, B=32, n=1024: persistent, all weights on chip
     text = lib.describe_plan(1000, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
     assert "mode=persistent" in text and "kernel=mfma" in text
     ws = lib.workspace_bytes(1000, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)

@@ -170,7 +170,7 @@ def test_register_kernel_long_ring(dtype):
 
 
 def test_cfg1_fp32():
-    """BASELINE config 1: T=32, B=4, n=64, fp32, full-length, 1e-5 relative."""
+    """benchmark configuration cfg1 (returnn_amd/synthetic.py): T=32, B=4, n=64, fp32, full-length, 1e-5 relative."""
     announce("cfg1")
     p = synthetic.make_config("cfg1")
     want = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, p.start, p.step)
@@ -180,7 +180,7 @@ def test_cfg1_fp32():
 
 
 def test_cfg2_fp32_full():
-    """BASELINE config 2 at full size: T=500, B=64, n=512, fp32, ragged lengths in [250,500]."""
+    """benchmark configuration cfg2 (returnn_amd/synthetic.py) at full size: T=500, B=64, n=512, fp32, ragged lengths in [250,500]."""
     announce("cfg2 full")
     p = synthetic.make_config("cfg2")
     want = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, p.start, p.step, threads=oracle.max_threads())
@@ -198,7 +198,7 @@ def test_cfg2_fp32_full():
 
 @pytest.mark.parametrize("step", [1, -1])
 def test_cfg3_bf16_reduced(step):
-    """BASELINE config 3 shape (B=32, n=1024, bf16) at T=120, both directions of the bidirectional pair:
+    """benchmark configuration cfg3 (returnn_amd/synthetic.py) shape (B=32, n=1024, bf16) at T=120, both directions of the bidirectional pair:
     2e-2 absolute on Y and C against the fp32 oracle on the identical fp32 inputs."""
     announce("cfg3 reduced", step)
     p = synthetic.make_config("cfg3", T=120, step=step)
@@ -217,7 +217,7 @@ def test_cfg3_bf16_reduced(step):
 
 
 def test_cfg3_bf16_full_size():
-    """BASELINE config 3 at full size (T=1000, B=32, n=1024, bf16), forward and backward call."""
+    """benchmark configuration cfg3 (returnn_amd/synthetic.py) at full size (T=1000, B=32, n=1024, bf16), forward and backward call."""
     announce("cfg3 full")
     p = synthetic.make_config("cfg3")
     want = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, 0, 1, threads=oracle.max_threads())
@@ -247,7 +247,7 @@ def test_cfg3_bf16_full_size():
 
 
 def test_cfg5_bf16_single_stream():
-    """BASELINE config 5 shape (B=1, n=1024, bf16), T=600 against the oracle; full T=4000 through properties."""
+    """benchmark configuration cfg5 (returnn_amd/synthetic.py) shape (B=1, n=1024, bf16), T=600 against the oracle; full T=4000 through properties."""
     announce("cfg5 T=600")
     p = synthetic.make_config("cfg5", T=600)
     want = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, 0, 1, threads=oracle.max_threads())
@@ -396,7 +396,7 @@ def test_bounded_wait_expires_cleanly():
     [(12, 8, 2048, "bf16"), (8, 300, 256, "bf16"), (8, 513, 128, "f32"), (6, 130, 1024, "bf16"), (5, 4, 3072, "bf16"), (7, 9, 736, "f32"), (9, 1, 4096, "bf16")],
 )
 def test_wide_and_large_shapes(T, B, n, dtype):
-    """Shapes beyond the BASELINE configurations: very wide layers (W no longer fits the registers of the device: the plan
+    """Shapes beyond the benchmark configurations cfg1-cfg5: very wide layers (W no longer fits the registers of the device: the plan
     falls back to the LDS kernel per step), many sequences (several batch groups, partly filled last group), a width that
     is a multiple of 32 but not of 64.  Forward against the oracle, then the gradient op on the GPU's own results."""
     announce("wide_and_large", T, B, n, dtype)

@@ -306,7 +306,7 @@ def test_threads_do_not_change_results():
 
 
 def test_f32_close_to_f64_cfg1():
-    """BASELINE config 1 (T=32, B=4, n=64): float32 oracle within 1e-5 relative of the float64 one."""
+    """benchmark configuration cfg1 (returnn_amd/synthetic.py) (T=32, B=4, n=64): float32 oracle within 1e-5 relative of the float64 one."""
     from returnn_amd import synthetic
 
     p = synthetic.make_config("cfg1")
