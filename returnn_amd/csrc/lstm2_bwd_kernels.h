@@ -211,7 +211,7 @@ __global__ void k_convert_from_f32(const float* src, void* dst, long long count)
 //
 //  * decomposition: `groups` batch groups of up to 16 rows; inside a group, workgroup r owns 16*MT values of k: the
 //    rows k of W (A operand of  d_h[b,k] = sum_j DX[b,j] W[k,j],  16*MT x 4n values, in registers for the whole call:
-//    wavefront w holds the macro steps [w*KSB, (w+1)*KSB) of j) and, in the pointwise part, the cells k of its rows.
+//    wavefront w holds the macro steps [w*ksb, (w+1)*ksb) of j, ksb <= KSB) and, in the pointwise part, the cells k of its rows.
 //    What a workgroup has to read per frame (rows x 4n values) is what its step time grows with -- a CU gets
 //    device-scope loads at only about 36 GB/s -- so the groups are made small (8 rows) when the device has the CUs.
 //  * exchange: DX itself.  The host fills DX with all-ones words (a NaN pattern no result can have: NaNs are
@@ -231,7 +231,9 @@ struct Lstm2BwdPersistent {
   long long t_end;    // first frame processed (the last one the forward pass visited)
   int step;           // the forward pass's signed stride; frames are processed t_end, t_end - step, ...
   int nframes;        // number of visited frames
-  int groups, Bg;     // batch groups and rows per group (<= 16)
+  int groups, Bg;     // batch groups of this launch and rows per group (<= 16)
+  int group_offset;   // index of the launch's first group (a large batch runs as several launches in turn)
+  int ksb;            // macro steps of the contraction per wavefront (<= the kernel's KSB; the rest of its slots stay empty)
   int poll_delay;
   unsigned long long timeout_ticks;
 };
@@ -283,23 +285,27 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // 0..WV-1
   const int n = p.n, n4 = 4 * n;
   const int kblocks = n / (16 * MT);  // workgroups per group; each owns MT tiles of 16 values of k
-  const int g = bid / kblocks, k0 = (bid % kblocks) * 16 * MT;
+  const int g = q.group_offset + bid / kblocks, k0 = (bid % kblocks) * 16 * MT;
   const int b_base = g * q.Bg;
   const int rows = min(q.Bg, p.B - b_base);
   const long long bn = (long long)p.B * n;
   const unsigned frame_bytes = (unsigned)((size_t)p.B * n4 * ES);
 
-  // A fragments: this wavefront's macro steps [wave*KSB, (wave+1)*KSB) of the 16*MT rows of W.
+  // A fragments: this wavefront's macro steps [wave*ksb, (wave+1)*ksb) of the 16*MT rows of W, as far as the 4n/KM macro
+  // steps reach.  Slots beyond them hold zeros, and their loads of DX carry an out-of-range buffer offset (they return 0
+  // without touching memory), so that any width whose share per wavefront is at most KSB runs on this kernel.
+  const int ksb = q.ksb;
+  const int ks_here = max(0, min(ksb, n4 / KM - ksb * wave));  // uniform over the wavefront
   i32x4 wreg[MT][KSB];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const AT* Wr = (const AT*)p.W + (size_t)(k0 + 16 * mt + (lane & 15)) * n4 + (size_t)KM * KSB * wave + KE * (lane >> 4);
+    const AT* Wr = (const AT*)p.W + (size_t)(k0 + 16 * mt + (lane & 15)) * n4 + (size_t)KM * ksb * wave + KE * (lane >> 4);
 #pragma unroll
-    for (int ks = 0; ks < KSB; ++ks) wreg[mt][ks] = *(const i32x4*)(Wr + (size_t)KM * ks);
+    for (int ks = 0; ks < KSB; ++ks) wreg[mt][ks] = (ks < ks_here) ? *(const i32x4*)(Wr + (size_t)KM * ks) : i32x4{0, 0, 0, 0};
   }
   // byte offset of this lane's first B fragment inside a frame of DX; the others follow at KM*ES bytes each
   const unsigned foff0 = (unsigned)(((size_t)(b_base + (((lane & 15) < rows) ? (lane & 15) : 0)) * n4  // rows the group lacks: row 0
-                                     + (size_t)KM * KSB * wave + KE * (lane >> 4)) * ES);
+                                     + (size_t)KM * ksb * wave + KE * (lane >> 4)) * ES);
 
   // The (row, k) pairs of this thread: one in each of its tiles.
   const int set = (TS == 1) ? 0 : __builtin_amdgcn_readfirstlane(tid >> 8);  // uniform over a wavefront
@@ -344,7 +350,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     asm volatile("" ::: "memory");  // other workgroups write this memory: really load again
 #pragma unroll
     for (int ks = 0; ks < KSB; ++ks)
-      bf[ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, foff0 + (unsigned)(ks * KM * ES), 0, kAuxDevice));
+      bf[ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (ks < ks_here) ? foff0 + (unsigned)(ks * KM * ES) : 0x80000000u, 0, kAuxDevice));
   };
   int delay = q.poll_delay;
   bool aborted = false;

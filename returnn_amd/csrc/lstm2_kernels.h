@@ -163,7 +163,7 @@ __global__ void k_prepare_mfma(Lstm2Params p, int n_flags) {
   if (p.hx_sentinel) {
     // buffers 1.. of every group: all ones = "not yet written"
     const long long words_per_buf = hx_buf * (long long)sizeof(AT) / 4;
-    const long long total = (long long)p.groups * p.hx_bufs * words_per_buf;
+    const long long total = (long long)p.groups_total * p.hx_bufs * words_per_buf;
     for (long long w = gtid; w < total; w += gsz)
       if ((w / words_per_buf) % p.hx_bufs != 0) ((unsigned*)p.hx)[w] = 0xFFFFFFFFu;
   }
@@ -345,6 +345,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
 
   int g, r;
   map_block(p, blockIdx.x, g, r);
+  g += p.group_offset;
   const int b_base = g * p.Bg;
   const int rows = min(p.Bg, p.B - b_base);
   const bool persist = (s_end - s_begin) > 1;
@@ -713,6 +714,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   const int n = p.n, S = n / KM;
   int g, r;
   map_block(p, bid, g, r);
+  g += p.group_offset;
   const int b_base = g * p.Bg;
   const int rows = min(p.Bg, p.B - b_base);
   const long long bn = (long long)p.B * n;

@@ -37,8 +37,8 @@ struct Lstm2Params {
   float* d;  // [B,n]
   // workspace sections (device)
   unsigned* status;  // [64]   status[0] != 0: a bounded wait expired
-  unsigned* flags;   // [groups*wgs_per_group] last published step (+1) of each workgroup
-  void* hx;          // [groups][hx_bufs][n/KE][Bp][KE] AT: hidden state in MFMA B-operand order, ring of buffers
+  unsigned* flags;   // [groups_total*wgs_per_group] last published step (+1) of each workgroup
+  void* hx;          // [groups_total][hx_bufs][n/KE][Bp][KE] AT: hidden state in MFMA B-operand order, ring of buffers
   void* Wp;          // [n/4][S][64][16 bytes]: W in MFMA A-operand order
   void* ycarry;      // [2][B][n] AT: hidden-state carry of the generic per-step kernels
   // sizes
@@ -48,7 +48,9 @@ struct Lstm2Params {
   int step;    // signed stride between visited frames
   int nsteps;  // number of visited frames
   // decomposition of the MFMA kernels
-  int groups;         // independent batch groups
+  int groups;         // independent batch groups worked on by this launch
+  int group_offset;   // index of the launch's first group (a large batch runs as several persistent launches in turn)
+  int groups_total;   // groups of the whole problem: the workspace sections are laid out for all of them
   int wgs_per_group;  // workgroups per group (each owns MT*4 cells)
   int Bg;             // batch rows per group
   int Bp;             // rows of one hx buffer (= 16*NT)

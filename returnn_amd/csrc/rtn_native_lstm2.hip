@@ -101,12 +101,19 @@ struct Plan {
   int grid = 0;                  // workgroups launched by the persistent kernel
   int KSMAX = 0;                 // its macro steps per wavefront (template bound)
   int MT = 1, NT = 1;
-  int groups = 1, wgs_per_group = 1, Bg = 1, Bp = 16;
+  int groups = 1, wgs_per_group = 1, Bg = 1, Bp = 16;  // groups: per persistent launch
+  int groups_total = 1;          // groups of the whole batch
+  int passes = 1;                // persistent launches in turn, each on `groups` of the groups (the last on the rest)
   size_t lds_bytes = 0;
   // workspace layout (byte offsets)
   size_t off_status = 0, off_flags = 0, off_hx = 0, off_wp = 0, off_ycarry = 0, off_trace = 0, total = 0;
   int n_flags = 0;
 };
+
+// Most persistent launches in turn that a plan may use instead of the LDS-resident persistent kernel, and instead
+// of per-step launches (from step times measured on MI355X).
+constexpr int kMaxPassesOverLds = 3;
+constexpr int kMaxPassesOverSteps = 32;
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 size_t esize(int dtype) { return dtype == RTN_DTYPE_BF16 ? 2 : 4; }
@@ -151,66 +158,104 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
     const int ks = (S + kWaves - 1) / kWaves;
     const int KSMAX = ks <= 2 ? 2 : (ks <= 4 ? 4 : (ks <= 8 ? 8 : (ks <= 16 ? 16 : 0)));
     if (want_mode == RTN_MODE_AUTO || want_mode == RTN_MODE_PERSISTENT) {
-      double best = 1e30;
-      for (int use_regw = 1; use_regw >= 0; --use_regw) {
-        if (use_regw && (env_kernel == 1 || KSMAX == 0)) continue;
-        if (!use_regw && (env_kernel == 2 || persistent_ok)) continue;
-        for (int MT : {1, 2, 4, 8}) {
-          if (env_mt && MT != env_mt) continue;
-          if (MT == 8 && !use_regw) continue;
-          if ((n / 4) % MT) continue;
-          const int G = n / (4 * MT);
-          // Workgroups that can share a CU: the register kernel with few fragments per wavefront fits twice.
-          const int per_cu = (use_regw && MT * KSMAX <= 32 && KSMAX <= 8) ? max_wgs_per_cu : 1;
-          if (G > di.cus * per_cu) continue;
-          if (use_regw && (MT * KSMAX > (KSMAX == 16 ? 32 : 64) || (MT == 8 && KSMAX != 8))) continue;
-          const int max_groups = di.cus * per_cu / G;
-          for (int groups = 1; groups <= std::min(max_groups, B); ++groups) {
-            if (env_groups && groups != std::min<long>(env_groups, std::min(max_groups, B))) continue;
-            const int Bg = (B + groups - 1) / groups;
-            if ((B + Bg - 1) / Bg != groups) continue;  // same rows per group would need fewer groups
-            if ((Bg + 15) / 16 > 4) continue;
-            const int NT = round_nt((Bg + 15) / 16);
-            if (use_regw && (NT * KSMAX > 32 || MT * NT > 8)) continue;  // register budget of one wavefront
-            const size_t lds = use_regw ? (size_t)regw_lds((int)es, MT, NT).total : mfma_lds_bytes(n, dtype, MT, NT);
-            if (lds > di.lds_per_wg) continue;
-            int pc = per_cu;  // workgroups per CU that LDS allows as well
-            while (pc > 1 && lds * pc > di.lds_per_wg) --pc;
-            if ((long long)groups * G > (long long)di.cus * pc) continue;
-            // Step time model fitted to MI355X measurements (microseconds): MFMA issue time of one
-            // wavefront, a second round of gate arithmetic when a thread owns two pairs, the number of
-            // workgroups that exchange with each other, the fragments a wavefront reads per step and
-            // the fragments it holds.
-            const double mfma_us = (double)MT * NT * ks * (dtype == RTN_DTYPE_BF16 ? 16 : 128) / 2400.0;
-            const int ept = (MT * NT + kWaves - 1) / kWaves;
-            double est = 2.0 * mfma_us + 0.4 * (ept - 1) + 0.004 * G + 0.03 * ks * NT + 0.01 * MT * ks;
-            // Several problems in one launch: as long as every workgroup has a CU to itself they do not slow
-            // each other down; sharing CUs costs about a third, running in turns costs the whole time again.
-            if (count > 1) {
-              const long long each = (long long)align_up((size_t)(groups * G), (size_t)di.xcds);
-              const long long fit1 = di.cus / each, fit2 = 2 * (long long)di.cus / each;
-              if (fit1 >= count)
-                ;
-              else if (use_regw && fit2 >= count)
-                est *= 1.35;
-              else
-                est *= (double)((count + std::max<long long>(fit2, 1) - 1) / std::max<long long>(fit2, 1)) * (fit2 >= 2 ? 1.35 : 1.0);
-            }
-            if (est < best) {
-              best = est;
-              pl.regw = use_regw != 0;
-              pl.grid = groups * G;
-              pl.KSMAX = use_regw ? KSMAX : 0;
-              pl.MT = MT;
-              pl.NT = NT;
-              pl.groups = groups;
-              pl.wgs_per_group = G;
-              pl.Bg = Bg;
-              pl.lds_bytes = lds;
-              persistent_ok = true;
+      struct Cand {
+        bool ok = false, regw = false;
+        int KSMAX = 0, MT = 1, NT = 1, groups = 1, G = 1, Bg = 1;
+        size_t lds = 0;
+        double est = 1e30;
+      };
+      // The best persistent decomposition for Bq batch rows in one launch.
+      auto search = [&](int Bq, bool regw_only) {
+        Cand best;
+        for (int use_regw = 1; use_regw >= (regw_only ? 1 : 0); --use_regw) {
+          if (use_regw && (env_kernel == 1 || KSMAX == 0)) continue;
+          if (!use_regw && (env_kernel == 2 || best.ok)) continue;
+          for (int MT : {1, 2, 4, 8}) {
+            if (env_mt && MT != env_mt) continue;
+            if (MT == 8 && !use_regw) continue;
+            if ((n / 4) % MT) continue;
+            const int G = n / (4 * MT);
+            // Workgroups that can share a CU: the register kernel with few fragments per wavefront fits twice.
+            const int per_cu = (use_regw && MT * KSMAX <= 32 && KSMAX <= 8) ? max_wgs_per_cu : 1;
+            if (G > di.cus * per_cu) continue;
+            if (use_regw && (MT * KSMAX > (KSMAX == 16 ? 32 : 64) || (MT == 8 && KSMAX != 8))) continue;
+            const int max_groups = di.cus * per_cu / G;
+            for (int groups = 1; groups <= std::min(max_groups, Bq); ++groups) {
+              if (env_groups && groups != std::min<long>(env_groups, std::min(max_groups, Bq))) continue;
+              const int Bg = (Bq + groups - 1) / groups;
+              if ((Bq + Bg - 1) / Bg != groups) continue;  // same rows per group would need fewer groups
+              if ((Bg + 15) / 16 > 4) continue;
+              const int NT = round_nt((Bg + 15) / 16);
+              if (use_regw && (NT * KSMAX > 32 || MT * NT > 8)) continue;  // register budget of one wavefront
+              const size_t lds = use_regw ? (size_t)regw_lds((int)es, MT, NT).total : mfma_lds_bytes(n, dtype, MT, NT);
+              if (lds > di.lds_per_wg) continue;
+              int pc = per_cu;  // workgroups per CU that LDS allows as well
+              while (pc > 1 && lds * pc > di.lds_per_wg) --pc;
+              if ((long long)groups * G > (long long)di.cus * pc) continue;
+              // Step time model fitted to MI355X measurements (microseconds): MFMA issue time of one
+              // wavefront, a second round of gate arithmetic when a thread owns two pairs, the number of
+              // workgroups that exchange with each other, the fragments a wavefront reads per step and
+              // the fragments it holds.
+              const double mfma_us = (double)MT * NT * ks * (dtype == RTN_DTYPE_BF16 ? 16 : 128) / 2400.0;
+              const int ept = (MT * NT + kWaves - 1) / kWaves;
+              double est = 2.0 * mfma_us + 0.4 * (ept - 1) + 0.004 * G + 0.03 * ks * NT + 0.01 * MT * ks;
+              // Several problems in one launch: as long as every workgroup has a CU to itself they do not slow
+              // each other down; sharing CUs costs about a third, running in turns costs the whole time again.
+              if (count > 1) {
+                const long long each = (long long)align_up((size_t)(groups * G), (size_t)di.xcds);
+                const long long fit1 = di.cus / each, fit2 = 2 * (long long)di.cus / each;
+                if (fit1 >= count)
+                  ;
+                else if (use_regw && fit2 >= count)
+                  est *= 1.35;
+                else
+                  est *= (double)((count + std::max<long long>(fit2, 1) - 1) / std::max<long long>(fit2, 1)) * (fit2 >= 2 ? 1.35 : 1.0);
+              }
+              if (est < best.est) {
+                best.ok = true;
+                best.est = est;
+                best.regw = use_regw != 0;
+                best.KSMAX = use_regw ? KSMAX : 0;
+                best.MT = MT;
+                best.NT = NT;
+                best.groups = groups;
+                best.G = G;
+                best.Bg = Bg;
+                best.lds = lds;
+              }
             }
           }
         }
+        return best;
+      };
+      Cand chosen = search(B, false);
+      // A batch too large for one launch of the register kernel runs as several launches in turn, each on a
+      // share of the batch groups (the rows of a batch are independent).  That beats the LDS-resident kernel
+      // for a few turns and per-step launches (which read W from HBM every step) for some more.
+      if (!(chosen.ok && chosen.regw)) {
+        const long env_passes = env_long("RTN_LSTM2_MAX_PASSES", -1);
+        const int limit = (int)(env_passes >= 0 ? env_passes : (chosen.ok ? kMaxPassesOverLds : kMaxPassesOverSteps));
+        for (int passes = 2; passes <= std::min(limit, B); ++passes) {
+          const Cand c = search((B + passes - 1) / passes, true);
+          if (!c.ok) continue;
+          if ((((B + c.Bg - 1) / c.Bg) + c.groups - 1) / c.groups > limit) continue;
+          chosen = c;
+          break;
+        }
+      }
+      if (chosen.ok) {
+        pl.regw = chosen.regw;
+        pl.KSMAX = chosen.KSMAX;
+        pl.MT = chosen.MT;
+        pl.NT = chosen.NT;
+        pl.Bg = chosen.Bg;
+        pl.wgs_per_group = chosen.G;
+        pl.groups_total = (B + chosen.Bg - 1) / chosen.Bg;
+        pl.groups = std::min(chosen.groups, pl.groups_total);
+        pl.passes = (pl.groups_total + pl.groups - 1) / pl.groups;
+        pl.grid = pl.groups * chosen.G;
+        pl.lds_bytes = chosen.lds;
+        persistent_ok = true;
       }
       if (!persistent_ok && why) *why = "no decomposition keeps W on chip with all workgroups co-resident";
     }
@@ -235,7 +280,8 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
         groups = (B + Bg - 1) / Bg;
         pl.MT = MT;
         pl.NT = round_nt((Bg + 15) / 16);
-        pl.groups = groups;
+        pl.groups = pl.groups_total = groups;
+        pl.passes = 1;
         pl.wgs_per_group = n / 4;
         pl.Bg = Bg;
         pl.lds_bytes = mfma_lds_bytes(n, dtype, pl.MT, pl.NT);
@@ -258,11 +304,11 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
   pl.off_status = off;
   off += 256;
   pl.off_flags = off;
-  pl.n_flags = (pl.kind == kPlanMfma) ? pl.groups * pl.wgs_per_group : 0;
+  pl.n_flags = (pl.kind == kPlanMfma) ? pl.groups_total * pl.wgs_per_group : 0;
   off = align_up(off + (size_t)pl.n_flags * 4, 256);
   if (pl.kind == kPlanMfma) {
     pl.off_hx = off;
-    off = align_up(off + (size_t)pl.groups * kHxRing * n * pl.Bp * es, 256);
+    off = align_up(off + (size_t)pl.groups_total * kHxRing * n * pl.Bp * es, 256);
     pl.off_wp = off;
     off = align_up(off + (size_t)4 * n * n * es, 256);
   } else {
@@ -526,7 +572,7 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, pk, kWgThreads, pl.lds_bytes));
     const long long capacity = (long long)per_cu * device_info().cus;
     if (capacity >= wgs) {
-      if (pl.regw && count > 1 && !env_long("RTN_LSTM2_NO_FUSE", 0)) {
+      if (pl.regw && count > 1 && pl.passes == 1 && !env_long("RTN_LSTM2_NO_FUSE", 0)) {
         const long long each = (long long)align_up((size_t)wgs, (size_t)device_info().xcds);
         fused = (int)std::min<long long>(std::min(count, kMaxMulti), capacity / each);
         if (fused < 1) fused = 1;
@@ -576,7 +622,8 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
       p.nsteps = (int)((p.first - last) / (-(long long)c.step) + 1);
     }
     p.step = c.step;
-    p.groups = pl.groups; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
+    p.groups = p.groups_total = pl.groups_total; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
+    p.group_offset = 0;
     p.op_flags = op_flags;
     p.hx_bufs = kHxRing;
     p.hx_sentinel = pl.regw ? 1 : 0;
@@ -616,7 +663,24 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
       else
         hipLaunchKernelGGL(k_prepare_mfma<float>, pgrid, pblock, 0, stream, p, pl.n_flags);
       RTN_HIP(hipGetLastError());
+      if (pk && pl.regw && pl.passes > 1) {
+        // the batch groups in turns: one cooperative launch per share of them
+        for (int g0 = 0; g0 < pl.groups_total; g0 += pl.groups) {
+          Lstm2Multi one;
+          memset(&one, 0, sizeof(one));
+          one.p[0] = p;
+          one.p[0].group_offset = g0;
+          one.p[0].groups = std::min(pl.groups, pl.groups_total - g0);
+          one.count = 1;
+          one.grid = one.p[0].groups * pl.wgs_per_group;
+          one.wgs_each = (int)align_up((size_t)one.grid, (size_t)device_info().xcds);
+          void* args[] = {(void*)&one};
+          RTN_HIP(hipLaunchCooperativeKernel(pk, dim3(one.grid), dim3(kWgThreads), args, (unsigned)pl.lds_bytes, stream));
+        }
+        continue;
+      }
       if (pk && pl.regw) {
+        p.groups = pl.groups;
         multi.p[pending++] = p;
         if (pending == fused || k + 1 == count) {
           multi.count = pending;
@@ -630,6 +694,7 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
         continue;
       }
       if (pk) {
+        p.groups = pl.groups;
         int s_begin = 0, s_end = p.nsteps;
         void* args_lds[] = {(void*)&p, (void*)&s_begin, (void*)&s_end};
         RTN_HIP(hipLaunchCooperativeKernel(pk, dim3(pl.groups * pl.wgs_per_group), dim3(kWgThreads), args_lds,
@@ -740,11 +805,11 @@ const char* rtn_native_lstm2_describe_multi_plan(int32_t count, int64_t T, int32
   } else if (!make_plan(T, B, n, dtype, mode, false, &pl, &why, 2, c)) {
     g_plan_text = "unsupported: " + why;
   } else {
-    snprintf(buf, sizeof(buf), "mode=%s kernel=%s mt=%d nt=%d groups=%d wgs_per_group=%d wgs=%d rows_per_group=%d lds=%zu workspace=%zu",
+    snprintf(buf, sizeof(buf), "mode=%s kernel=%s mt=%d nt=%d groups=%d wgs_per_group=%d wgs=%d rows_per_group=%d launches=%d lds=%zu workspace=%zu",
              mode_name(pl.mode),
              pl.kind == kPlanMfma ? (pl.regw ? "mfma_regw" : "mfma_lds") : (pl.kind == kPlanGeneric ? "generic" : "empty"), pl.MT,
              pl.NT, pl.groups, pl.wgs_per_group, (pl.mode == RTN_MODE_PERSISTENT && pl.regw) ? pl.grid : pl.groups * pl.wgs_per_group,
-             pl.Bg, pl.lds_bytes, count > 1 ? workspace_each(count, T, B, n, dtype, mode) : pl.total);
+             pl.Bg, pl.passes, pl.lds_bytes, count > 1 ? workspace_each(count, T, B, n, dtype, mode) : pl.total);
     if (pl.off_trace) snprintf(buf + strlen(buf), sizeof(buf) - strlen(buf), " trace_offset=%zu", pl.off_trace);
     g_plan_text = buf;
   }
@@ -987,8 +1052,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
   // Persistent kernel: W in registers for the whole call, if a wavefront's share of the 16 x 4n slice fits
   // (2..32 fragments) and all workgroups of all problems can be on the device together.
   const void* pk = nullptr;
-  int KSB = 0, bwd_mt = 1;
-  (void)KSB;
+  int KSB = 0, bwd_mt = 1;  // KSB: macro steps of the contraction per wavefront
   // Decomposition: batch groups of 8 or 16 rows (a workgroup's frame time grows with the rows x 4n values of DX it
   // reads per frame at device scope), MT tiles of 16 values of k per workgroup (more tiles: fewer workgroups, more
   // MFMA time each) and 4 or 8 wavefronts per workgroup (8: more loads in flight per CU and no register spills, but
@@ -996,7 +1060,10 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
   // 8 x 1 x 8: 4.22, 8 x 1 x 4: 4.37; two problems in one launch 8 x 2 x 4: 5.5, 16 x 1 x 8: 6.1, 16 x 1 x 4: 6.5,
   // 8 x 2 x 8: 6.6, 16 x 2 x 4: 7.1); the first whose workgroups are all on the device together.
   const long env_rows = env_long("RTN_LSTM2_BWD_ROWS", 0);
-  int rows_per_group = 16, bwd_waves = kWaves;
+  int rows_per_group = 16, bwd_waves = kWaves, groups_per_launch = 0;
+  long long turn_rows = 0;
+  const void* turn_pk = nullptr;
+  int turn_cfg[5] = {0, 0, 0, 0, 0};
   {
     const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
     const int S = 4 * n / KM;
@@ -1014,22 +1081,41 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
         if (rows_forced && rows != 8) continue;                    // (one pass per MT is enough then)
         const int use_rows = rows_forced ? (int)env_rows : rows;
         if (wv != 4 && wv != 8 && wv != 16) continue;
-        if (S % wv) continue;
-        const int ksb = S / wv;
-        if (mt * ksb > 64 || (n / 16) % mt) continue;
-        BwdRegwKernel kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(ksb, mt, wv) : bwd_regw_kernel_for<float>(ksb, mt, wv);
+        const int ksb = (S + wv - 1) / wv;  // macro steps per wavefront; the kernel has room for the next power of two
+        int ksb_room = 2;
+        while (ksb_room < ksb) ksb_room *= 2;
+        if (mt * ksb_room > 64 || (n / 16) % mt) continue;
+        BwdRegwKernel kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(ksb_room, mt, wv) : bwd_regw_kernel_for<float>(ksb_room, mt, wv);
         if (!kfn) continue;
         int per_cu = 0;
         RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kfn, 64 * wv, 0));
         const long long groups_needed = (B + use_rows - 1) / use_rows;
-        if ((long long)per_cu * device_info().cus >= (long long)count * groups_needed * (n / (16 * mt))) {
+        // batch groups of every problem that one launch can hold
+        const long long fit = (long long)per_cu * device_info().cus / ((long long)count * (n / (16 * mt)));
+        if (fit >= groups_needed) {
           pk = (const void*)kfn;
           bwd_mt = mt;
           bwd_waves = wv;
           KSB = ksb;
           rows_per_group = use_rows;
+          groups_per_launch = (int)groups_needed;
           break;
         }
+        // Too many rows for one launch: remember the candidate that takes most rows per launch; the batch groups
+        // then run in turns (the rows of a batch are independent of each other).
+        if (fit >= 1 && fit * use_rows > turn_rows && (groups_needed + fit - 1) / fit <= env_long("RTN_LSTM2_MAX_PASSES", kMaxPassesOverSteps)) {
+          turn_rows = fit * use_rows;
+          turn_pk = (const void*)kfn;
+          turn_cfg[0] = use_rows; turn_cfg[1] = mt; turn_cfg[2] = wv; turn_cfg[3] = ksb; turn_cfg[4] = (int)fit;
+        }
+      }
+      if (!pk && turn_pk) {
+        pk = turn_pk;
+        rows_per_group = turn_cfg[0];
+        bwd_mt = turn_cfg[1];
+        bwd_waves = turn_cfg[2];
+        KSB = turn_cfg[3];
+        groups_per_launch = turn_cfg[4];
       }
     }
     if (!pk && count > 1) {
@@ -1081,7 +1167,6 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     Lstm2BwdMulti multi;
     memset(&multi, 0, sizeof(multi));
     multi.count = count;
-    multi.wgs_each = bgroups * (n / (16 * bwd_mt));
     for (int k = 0; k < count; ++k) {
       Lstm2BwdPersistent& q = multi.q[k];
       q.p = jobs[(size_t)k].p;
@@ -1091,13 +1176,22 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       q.t_end = jobs[(size_t)k].end;
       q.step = calls[k].step;
       q.nframes = (int)jobs[(size_t)k].num_steps;
-      q.groups = bgroups;
       q.Bg = (B + bgroups - 1) / bgroups;
+      q.ksb = KSB;
       q.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", 20)));
       q.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);
     }
-    void* args[] = {(void*)&multi};
-    RTN_HIP(hipLaunchCooperativeKernel(pk, dim3((unsigned)(count * multi.wgs_each)), dim3((unsigned)(64 * bwd_waves)), args, 0, stream));
+    // one cooperative launch per share of the batch groups (a single one unless the batch is too large for the device)
+    for (int g0 = 0; g0 < bgroups; g0 += groups_per_launch) {
+      const int groups_now = std::min(groups_per_launch, bgroups - g0);
+      multi.wgs_each = groups_now * (n / (16 * bwd_mt));
+      for (int k = 0; k < count; ++k) {
+        multi.q[k].groups = groups_now;
+        multi.q[k].group_offset = g0;
+      }
+      void* args[] = {(void*)&multi};
+      RTN_HIP(hipLaunchCooperativeKernel(pk, dim3((unsigned)(count * multi.wgs_each)), dim3((unsigned)(64 * bwd_waves)), args, 0, stream));
+    }
     for (int k = 0; k < count; ++k) {
       const BwdJob& j = jobs[(size_t)k];
       if (j.num_steps == T) continue;

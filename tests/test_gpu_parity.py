@@ -393,7 +393,7 @@ def test_bounded_wait_expires_cleanly():
 
 @pytest.mark.parametrize(
     "T,B,n,dtype",
-    [(12, 8, 2048, "bf16"), (8, 300, 256, "bf16"), (8, 513, 128, "f32"), (6, 130, 1024, "bf16"), (5, 4, 3072, "bf16"), (7, 9, 736, "f32"), (9, 1, 4096, "bf16")],
+    [(12, 8, 2048, "bf16"), (8, 300, 256, "bf16"), (6, 256, 1024, "bf16"), (5, 300, 512, "f32"), (4, 70, 1536, "bf16"), (8, 513, 128, "f32"), (6, 130, 1024, "bf16"), (5, 4, 3072, "bf16"), (7, 9, 736, "f32"), (9, 1, 4096, "bf16")],
 )
 def test_wide_and_large_shapes(T, B, n, dtype):
     """Shapes beyond the benchmark configurations cfg1-cfg5: very wide layers (W no longer fits the registers of the device: the plan
@@ -422,3 +422,19 @@ def test_wide_and_large_shapes(T, B, n, dtype):
     for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), grads, wantg):
         rel = float(numpy.abs(f(a) - b).max() / max(numpy.abs(b).max(), 1e-30))
         assert rel <= (2e-5 if dtype == "f32" else 2e-2), (name, rel)
+
+
+@pytest.mark.parametrize("T,B,n,dtype,start,step", [(6, 256, 1024, "bf16", 0, 1), (5, 70, 1536, "bf16", 1, -1), (5, 300, 512, "f32", 0, 2), (4, 97, 2048, "bf16", 0, -1)])
+def test_batch_in_several_persistent_launches(T, B, n, dtype, start, step):
+    """A batch too large for one launch of the register kernel runs as several persistent launches in turn, each on a
+    share of the batch groups, the last one on fewer groups (and a partly filled group)."""
+    from returnn_amd import lib
+
+    announce("several_launches", T, B, n, dtype, start, step)
+    plan = lib.load().rtn_native_lstm2_describe_plan(T, B, n, lib.DTYPE_BF16 if dtype == "bf16" else lib.DTYPE_F32, lib.MODES["auto"]).decode()
+    assert "kernel=mfma_regw" in plan and "launches=1 " not in plan, plan
+    p = random_problem(950 + B + n, T, B, n)
+    want = oracle.native_lstm2_fwd(*p, start, step, threads=oracle.max_threads())
+    rc, status, got = run_raw(*p, start, step, dtype=dtype)
+    assert rc == 0 and status == 0
+    (check_f32 if dtype == "f32" else check_bf16)(got, want[:4], "several launches %s" % ((T, B, n),))
