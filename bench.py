@@ -33,7 +33,7 @@ PEAK_HBM = 8.0e12  # B/s
 
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by
 # what the same counter reads for a plain 1 GiB device copy); see profiles/k_lstm2_regw_cfg3_*_hbm_traffic.txt.
-# Keyed by (workload, launches per step, plan as rtn_native_lstm2_describe_plan reports it up to the LDS size).
+# Keyed by (workload, launches per step, plan as rtn_native_lstm2_describe_plan reports it up to the number of launches).
 MEASURED_TRAFFIC_BYTES = {
     ("cfg3", 1, "mode=persistent kernel=mfma_regw mt=4 nt=1 groups=2 wgs_per_group=64 wgs=128 rows_per_group=16"): 2524.5e6,
     ("cfg3", 2, "mode=persistent kernel=mfma_regw mt=2 nt=1 groups=2 wgs_per_group=128 wgs=256 rows_per_group=16"): 1265.2e6,
@@ -818,7 +818,7 @@ def main():
             "peak": peak / 1e12,
             "unit": "TFLOP/s",
             "frac": achieved / peak,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, launches, plan.split(" lds=")[0])),
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, launches, plan.split(" launches=")[0])),
             "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE); algorithmic: %i" % bytes_per_launch,
             "kernel": "%s (one launch = %i op call(s) = %i units of T*B, 8*n^2 flops each)"
             % ("k_lstm2_regw" if "mfma_regw" in plan else ("k_lstm2_mfma" if "mfma_lds" in plan else "k_step_generic"),

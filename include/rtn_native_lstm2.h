@@ -264,7 +264,9 @@ int rtn_native_lstm2_last_output(const void* Y, const void* y0, const float* i, 
 const char* rtn_last_error(void);
 
 /* The plan the library would use for this problem, as text
- * ("mode=persistent mt=1 nt=2 groups=1 wgs=256 lds=40960 ..."); for logs and tests.
+ * ("mode=persistent kernel=mfma_regw mt=2 nt=1 groups=2 wgs_per_group=128 wgs=256 rows_per_group=16
+ * launches=1 lds=22176 workspace=...": groups, workgroups and rows per group of one persistent launch, and how many
+ * launches in turn take the whole batch); for logs and tests.
  * Counterpart of the reference's compile log next to the .so (returnn/util/native_code_compiler.py:348-352). */
 const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode);
 

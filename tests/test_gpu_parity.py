@@ -438,3 +438,39 @@ def test_batch_in_several_persistent_launches(T, B, n, dtype, start, step):
     rc, status, got = run_raw(*p, start, step, dtype=dtype)
     assert rc == 0 and status == 0
     (check_f32 if dtype == "f32" else check_bf16)(got, want[:4], "several launches %s" % ((T, B, n),))
+
+
+@pytest.mark.parametrize("T,B,n,dtype,start,step", [(9, 5, 100, "f32", 0, 1), (6, 33, 1000, "bf16", 0, -1), (5, 3, 50, "bf16", 1, 2), (7, 4, 40, "f32", 1, -2)])
+def test_widths_that_run_zero_padded(T, B, n, dtype, start, step):
+    """Widths that are not a multiple of 32: the torch-level op pads the cells with zeros to the next multiple of 32 and
+    runs the matrix-core kernels; forward and gradient against the oracle, and the forward against the library's own
+    element-wise kernels at the original width (the C ABI called directly)."""
+    from _gpu_util import to_dev
+    from returnn_amd import native_op, torch_native_op
+
+    announce("zero_padded", T, B, n, dtype, start, step)
+    assert torch_native_op._padded_width(n) != n
+    p = random_problem(970 + n, T, B, n)
+    X, W, y0, c0, i = p
+    want = oracle.native_lstm2_fwd(*p, start, step, threads=oracle.max_threads())
+    got = run_op(*p, start, step, dtype=dtype)
+    check = check_f32 if dtype == "f32" else check_bf16
+    check(got, want, "padded %s" % ((T, B, n),))
+    rc, status, raw = run_raw(*p, start, step, dtype=dtype)
+    assert rc == 0 and status == 0
+    check(got[:4], raw, "padded against element-wise kernels")
+    rng = numpy.random.default_rng(971)
+    DY = rng.normal(0, 1, (T, B, n)).astype(numpy.float32)
+    Dd = rng.normal(0, 1, (B, n)).astype(numpy.float32)
+    Xd, Wd, y0d, DYd = (to_dev(a, dtype) for a in (X, W, y0, DY))
+    c0d, id_, Ddd = (to_dev(a, "f32") for a in (c0, i, Dd))
+    Y, C, H, d = torch_native_op.make_op(native_op.NativeLstm2)(Xd, Wd, y0d, c0d, id_, start, step)
+    assert Y.shape == (T, B, n) and H.shape == (T, B, 4 * n) and Y.is_contiguous() and H.is_contiguous()
+    grads = torch_native_op.native_lstm2_grad(Wd, y0d, c0d, id_, start, step, Y, C, H, DYd, Ddd)
+    torch.cuda.synchronize()
+    f = lambda t: t.float().cpu().numpy().astype(numpy.float64)  # noqa: E731
+    wantg = oracle.native_lstm2_bwd(f(Xd), f(Wd), f(y0d), c0, i, start, step, f(Y), f(C), f(H), f(DYd), Dd, dtype=numpy.float64)
+    for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), grads, wantg):
+        assert tuple(a.shape) == b.shape, name
+        rel = float(numpy.abs(f(a) - b).max() / max(numpy.abs(b).max(), 1e-30))
+        assert rel <= (2e-5 if dtype == "f32" else 2e-2), (name, rel)
