@@ -292,10 +292,12 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   const unsigned frame_bytes = (unsigned)((size_t)p.B * n4 * ES);
 
   // A fragments: this wavefront's macro steps [wave*ksb, (wave+1)*ksb) of the 16*MT rows of W, as far as the 4n/KM macro
-  // steps reach.  Slots beyond them hold zeros, and their loads of DX carry an out-of-range buffer offset (they return 0
-  // without touching memory), so that any width whose share per wavefront is at most KSB runs on this kernel.
+  // steps reach.  Slots beyond them hold zeros in W and read nothing (or, in the 64-slot variant, a fragment that is
+  // multiplied by that zero), so that any width whose share per wavefront is at most KSB runs on this kernel.
   const int ksb = q.ksb;
   const int ks_here = max(0, min(ksb, n4 / KM - ksb * wave));  // uniform over the wavefront
+  const int ks_last = max(ks_here, 1) - 1;
+  const int wave_at = (KSB > 32 && ks_here == 0) ? 0 : wave;  // 64-slot variant: a wavefront without a share reads the first one's
   i32x4 wreg[MT][KSB];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -305,7 +307,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   }
   // byte offset of this lane's first B fragment inside a frame of DX; the others follow at KM*ES bytes each
   const unsigned foff0 = (unsigned)(((size_t)(b_base + (((lane & 15) < rows) ? (lane & 15) : 0)) * n4  // rows the group lacks: row 0
-                                     + (size_t)KM * ksb * wave + KE * (lane >> 4)) * ES);
+                                     + (size_t)KM * ksb * wave_at + KE * (lane >> 4)) * ES);
 
   // The (row, k) pairs of this thread: one in each of its tiles.
   const int set = (TS == 1) ? 0 : __builtin_amdgcn_readfirstlane(tid >> 8);  // uniform over a wavefront
@@ -344,58 +346,39 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   };
   auto frame = [&](int f) { return q.t_end - (long long)f * q.step; };
 
-  i32x4 bf[KSB];
-  auto issue = [&](long long t) {
+  // The B fragments of a frame (the group's rows of DX, this wavefront's share of the contraction range) are taken in
+  // chunks of CH: up to 32 fragments in one go; a wider share in chunks of 16 through two sets of registers (the next
+  // chunk is in flight while the matrix cores work on this one), because W already fills half of the register file.
+  constexpr int CH = KSB > 32 ? 16 : KSB;
+  constexpr int NCH = KSB / CH;
+  i32x4 bf[NCH > 1 ? 2 : 1][CH];
+  auto issue_chunk = [&](long long t, int c, int slot) {
     __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
     asm volatile("" ::: "memory");  // other workgroups write this memory: really load again
+    if constexpr (NCH == 1) {
+      // an unused slot carries an out-of-range offset: 0 comes back and no memory is touched (the offsets stay in
+      // registers over the frames, which measured faster than instruction immediates)
 #pragma unroll
-    for (int ks = 0; ks < KSB; ++ks)
-      bf[ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (ks < ks_here) ? foff0 + (unsigned)(ks * KM * ES) : 0x80000000u, 0, kAuxDevice));
+      for (int ks = 0; ks < CH; ++ks)
+        bf[slot][ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (ks < ks_here) ? foff0 + (unsigned)(ks * KM * ES) : 0x80000000u, 0, kAuxDevice));
+    } else {
+      // 64 offsets would not fit the registers: an unused slot reads the wavefront's last used fragment again (complete
+      // when the used ones are, and multiplied by zero); worked out again for every chunk
+      int last = ks_last;
+      asm volatile("" : "+s"(last));
+#pragma unroll
+      for (int ks = 0; ks < CH; ++ks)
+        bf[slot][ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, foff0, min(c * CH + ks, last) * (KM * ES), kAuxDevice));
+    }
   };
+  auto issue = [&](long long t) { issue_chunk(t, 0, 0); };
   int delay = q.poll_delay;
   bool aborted = false;
   // d_h of the thread's pairs from DX of frame t (whose first read has been issued): wait, MFMA, sum over the
   // wavefronts; added to dyw.
   RTN_BTRACE_DECL
   auto gemm = [&](long long t) {
-    unsigned long long t0 = 0;
-    unsigned spins = 0;
     RTN_BTRACE_MARK(4)  // pointwise tail, fetch, delay, first read
-    for (;;) {
-      unsigned m = 0;
-#pragma unroll
-      for (int ks = 0; ks < KSB; ++ks)
-#pragma unroll
-        for (int w = 0; w < 4; ++w) m = LM::fold(m, (unsigned)bf[ks][w]);
-      if (!__any(LM::has_sentinel(m))) break;
-      if ((spins++ & 15u) == 0) {
-        if (__hip_atomic_load(q.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { aborted = true; break; }
-        const unsigned long long now = wall_clock64();
-        if (spins == 1) {
-          t0 = now;
-        } else if (now - t0 > q.timeout_ticks) {
-          __hip_atomic_store(q.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          aborted = true;
-          break;
-        }
-      }
-      issue(t);
-    }
-    RTN_BTRACE_MARK(0)  // wait for the frame's DX
-    RTN_BTRACE_ADD(6, spins)
-    if (spins)
-      delay = min(delay + 2, 64);
-    else if (delay > 0)
-      delay -= ((t & 15) == 15) ? 1 : 0;
-    // W lives in accumulation registers where it is at most half of that file: the B fragments of a frame fill half of
-    // the ordinary registers, and a matrix instruction reads an A operand from either file (without this the compiler
-    // parks part of W there anyway and copies four registers back in front of every MFMA, which halves the MFMA rate).
-    if constexpr (MT * KSB <= 32) {
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int ks = 0; ks < KSB; ++ks) asm volatile("" : "+a"(wreg[mt][ks]));
-    }
     // independent partial sums keep the MFMA pipeline full (one chain would wait for every result)
     constexpr int NACC = (MT >= 4 || KSB < 2) ? 1 : (MT == 2 || KSB < 4 ? 2 : 4);
     f32x4 part[MT][NACC];
@@ -404,9 +387,63 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
 #pragma unroll
       for (int a = 0; a < NACC; ++a) part[mt][a] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ks = 0; ks < KSB; ++ks)
+    for (int c = 0; c < NCH; ++c) {
+      const int slot = c & 1;
+      unsigned long long t0 = 0;
+      unsigned spins = 0;
+      for (;;) {
+        unsigned m = 0;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) part[mt][ks % NACC] = E::mma(wreg[mt][ks], bf[ks], part[mt][ks % NACC]);
+        for (int ks = 0; ks < CH; ++ks)
+#pragma unroll
+          for (int w = 0; w < 4; ++w) m = LM::fold(m, (unsigned)bf[slot][ks][w]);
+        if (!__any(LM::has_sentinel(m))) break;
+        if ((spins++ & 15u) == 0) {
+          if (__hip_atomic_load(q.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { aborted = true; break; }
+          const unsigned long long now = wall_clock64();
+          if (spins == 1) {
+            t0 = now;
+          } else if (now - t0 > q.timeout_ticks) {
+            __hip_atomic_store(q.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            aborted = true;
+            break;
+          }
+        }
+        issue_chunk(t, c, slot);
+      }
+      if (c == 0) {
+        RTN_BTRACE_MARK(0)  // wait for the frame's DX
+        RTN_BTRACE_ADD(6, spins)
+        if (spins)
+          delay = min(delay + 2, 64);
+        else if (delay > 0)
+          delay -= ((t & 15) == 15) ? 1 : 0;
+        // W lives in accumulation registers where it is at most half of that file, or all of it when the wavefront's share
+        // is taken in chunks: the B fragments fill up to half of the ordinary registers, and a matrix instruction reads an A
+        // operand from either file (without this the compiler parks part of W there anyway and copies four registers back
+        // in front of every MFMA, which halves the MFMA rate).
+        if constexpr (MT * KSB <= 32) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int ks = 0; ks < KSB; ++ks) asm volatile("" : "+a"(wreg[mt][ks]));
+        } else if constexpr (NCH > 1) {
+          // a share of 64 fragments: 56 of them there (the accumulators need room in that file as well), 8 in ordinary registers
+#pragma unroll
+          for (int ks = 0; ks < KSB; ++ks) {
+            if (ks < KSB - 8)
+              asm volatile("" : "+a"(wreg[0][ks]));
+            else
+              asm volatile("" : "+v"(wreg[0][ks]));
+          }
+        }
+      }
+      if (c + 1 < NCH) issue_chunk(t, c + 1, slot ^ 1);
+#pragma unroll
+      for (int ks = 0; ks < CH; ++ks)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) part[mt][ks % NACC] = E::mma(wreg[mt][c * CH + ks], bf[slot][ks], part[mt][ks % NACC]);
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       f32x4 acc = part[mt][0];
