@@ -16,7 +16,8 @@ Argument handling follows the generated wrapper (:144-193): dtype normalisation,
 ``.contiguous()`` for ``need_contiguous`` inputs, device guard on the first tensor, outputs allocated on
 that device.  Differences, on purpose: bfloat16 inputs stay bfloat16 (X, W, y0, Y, H in bf16; c0, C, d,
 mask in float32) instead of being up-cast; outputs are not zero-filled first because the library writes
-every element; CPU tensors are rejected (no CPU implementation is shipped).
+every element; CPU tensors are rejected (no CPU implementation is shipped); widths that are not a multiple of 32
+run zero-padded to the next multiple (see ``_padded_width``), with the results of the unpadded problem.
 """
 
 from __future__ import annotations
