@@ -383,10 +383,6 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     constexpr int NACC = (MT >= 4 || KSB < 2) ? 1 : (MT == 2 || KSB < 4 ? 2 : 4);
     f32x4 part[MT][NACC];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int a = 0; a < NACC; ++a) part[mt][a] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
     for (int c = 0; c < NCH; ++c) {
       const int slot = c & 1;
       unsigned long long t0 = 0;
@@ -439,6 +435,12 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
         }
       }
       if (c + 1 < NCH) issue_chunk(t, c + 1, slot ^ 1);
+      if (c == 0) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int a = 0; a < NACC; ++a) part[mt][a] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
 #pragma unroll
       for (int ks = 0; ks < CH; ++ks)
 #pragma unroll
