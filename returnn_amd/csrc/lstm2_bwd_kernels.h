@@ -267,8 +267,12 @@ struct Lstm2BwdMulti {
 // scope the more wavefronts have loads in flight, and with 8 or more each wavefront's share of W and of the frame's DX
 // fits the ordinary registers.  The 256 (row, k) pairs of a tile belong to the threads with the same tid % 256; thread
 // set tid / 256 takes the tiles set, set + WV/4, ...
-template <typename AT, int KSB, int MT, int WV>
+//
+// KSL > 0: a wavefront's share of W is KSB fragments in registers plus KSL fragments in LDS (dynamic shared memory,
+// WV * KSL * 1024 bytes), for layers whose slice of W does not fit the registers next to a frame's DX.
+template <typename AT, int KSB, int MT, int WV, int KSL = 0>
 __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti multi) {
+  constexpr int KST = KSB + KSL;           // fragment slots of a wavefront
   constexpr int TS = WV / 4;               // thread sets of 256
   constexpr int PT = (MT + TS - 1) / TS;   // tiles whose pairs a thread keeps
   const int which = (int)blockIdx.x / multi.wgs_each;
@@ -297,13 +301,20 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   const int ksb = q.ksb;
   const int ks_here = max(0, min(ksb, n4 / KM - ksb * wave));  // uniform over the wavefront
   const int ks_last = max(ks_here, 1) - 1;
-  const int wave_at = (KSB > 32 && ks_here == 0) ? 0 : wave;  // 64-slot variant: a wavefront without a share reads the first one's
+  const int wave_at = (KST > 32 && ks_here == 0) ? 0 : wave;  // 64-slot variant: a wavefront without a share reads the first one's
   i32x4 wreg[MT][KSB];
+  extern __shared__ __align__(16) unsigned char bwd_smem[];
+  i32x4* wl = (i32x4*)bwd_smem + (size_t)wave * (KSL > 0 ? KSL : 1) * 64 + lane;  // [WV][KSL][64]: slot s of this lane at wl[s * 64]
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const AT* Wr = (const AT*)p.W + (size_t)(k0 + 16 * mt + (lane & 15)) * n4 + (size_t)KM * ksb * wave + KE * (lane >> 4);
 #pragma unroll
     for (int ks = 0; ks < KSB; ++ks) wreg[mt][ks] = (ks < ks_here) ? *(const i32x4*)(Wr + (size_t)KM * ks) : i32x4{0, 0, 0, 0};
+    if constexpr (KSL > 0) {
+      static_assert(KSL == 0 || MT == 1, "the LDS part of W is laid out for one tile per workgroup");
+#pragma unroll
+      for (int ks = KSB; ks < KST; ++ks) wl[(ks - KSB) * 64] = (ks < ks_here) ? *(const i32x4*)(Wr + (size_t)KM * ks) : i32x4{0, 0, 0, 0};
+    }
   }
   // byte offset of this lane's first B fragment inside a frame of DX; the others follow at KM*ES bytes each
   const unsigned foff0 = (unsigned)(((size_t)(b_base + (((lane & 15) < rows) ? (lane & 15) : 0)) * n4  // rows the group lacks: row 0
@@ -347,10 +358,10 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   auto frame = [&](int f) { return q.t_end - (long long)f * q.step; };
 
   // The B fragments of a frame (the group's rows of DX, this wavefront's share of the contraction range) are taken in
-  // chunks of CH: up to 32 fragments in one go; a wider share in chunks of 16 through two sets of registers (the next
-  // chunk is in flight while the matrix cores work on this one), because W already fills half of the register file.
-  constexpr int CH = KSB > 32 ? 16 : KSB;
-  constexpr int NCH = KSB / CH;
+  // chunks of CH: up to 32 fragments in one go; a wider share (KSL > 0) in chunks of 16 through two sets of registers
+  // (the next chunk is in flight while the matrix cores work on this one).
+  constexpr int CH = KST > 32 ? 16 : KST;
+  constexpr int NCH = KST / CH;
   i32x4 bf[NCH > 1 ? 2 : 1][CH];
   auto issue_chunk = [&](long long t, int c, int slot) {
     __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
@@ -414,24 +425,14 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
           delay = min(delay + 2, 64);
         else if (delay > 0)
           delay -= ((t & 15) == 15) ? 1 : 0;
-        // W lives in accumulation registers where it is at most half of that file, or all of it when the wavefront's share
-        // is taken in chunks: the B fragments fill up to half of the ordinary registers, and a matrix instruction reads an A
-        // operand from either file (without this the compiler parks part of W there anyway and copies four registers back
-        // in front of every MFMA, which halves the MFMA rate).
+        // W lives in accumulation registers where it is at most half of that file: the B fragments fill up to half of
+        // the ordinary registers, and a matrix instruction reads an A operand from either file (without this the compiler
+        // parks part of W there anyway and copies four registers back in front of every MFMA, which halves the MFMA rate).
         if constexpr (MT * KSB <= 32) {
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int ks = 0; ks < KSB; ++ks) asm volatile("" : "+a"(wreg[mt][ks]));
-        } else if constexpr (NCH > 1) {
-          // a share of 64 fragments: 56 of them there (the accumulators need room in that file as well), 8 in ordinary registers
-#pragma unroll
-          for (int ks = 0; ks < KSB; ++ks) {
-            if (ks < KSB - 8)
-              asm volatile("" : "+a"(wreg[0][ks]));
-            else
-              asm volatile("" : "+v"(wreg[0][ks]));
-          }
         }
       }
       if (c + 1 < NCH) issue_chunk(t, c + 1, slot ^ 1);
@@ -444,7 +445,11 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
 #pragma unroll
       for (int ks = 0; ks < CH; ++ks)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) part[mt][ks % NACC] = E::mma(wreg[mt][c * CH + ks], bf[slot][ks], part[mt][ks % NACC]);
+        for (int mt = 0; mt < MT; ++mt) {
+          const int s_ = c * CH + ks;
+          const i32x4 a = (s_ < KSB) ? wreg[mt][s_ < KSB ? s_ : 0] : wl[(s_ - KSB) * 64];
+          part[mt][ks % NACC] = E::mma(a, bf[slot][ks], part[mt][ks % NACC]);
+        }
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {

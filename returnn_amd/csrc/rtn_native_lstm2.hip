@@ -714,6 +714,15 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
 
 typedef void (*BwdRegwKernel)(const Lstm2BwdMulti);
 
+// Bytes of dynamic shared memory of the variant that keeps half of a 64-fragment share of W in LDS.
+constexpr size_t kBwdLdsShareBytes = (size_t)kWaves * 32 * 64 * 16;
+
+// The variant with 32 fragments of W per wavefront in registers and 32 in LDS (one tile, 4 wavefronts).
+template <typename AT>
+BwdRegwKernel bwd_regw_lds_kernel_for() {
+  return &k_lstm2_bwd_regw<AT, 32, 1, 4, 32>;
+}
+
 // KSB: fragments of W per tile and wavefront; MT: tiles of 16 values of k per workgroup; WV: wavefronts per workgroup.
 template <typename AT>
 BwdRegwKernel bwd_regw_kernel_for(int KSB, int MT, int WV) {
@@ -1065,6 +1074,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
   long long turn_rows = 0;
   const void* turn_pk = nullptr;
   int turn_cfg[5] = {0, 0, 0, 0, 0};
+  size_t bwd_lds = 0, turn_lds = 0;  // dynamic shared memory of the chosen kernel
   {
     const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
     const int S = 4 * n / KM;
@@ -1086,11 +1096,23 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
         int ksb_room = 2;
         while (ksb_room < ksb) ksb_room *= 2;
         if (mt * ksb_room > 64 || (n / 16) % mt) continue;
-        if (ksb_room == 64 && dtype != RTN_DTYPE_BF16) continue;  // the float32 variant spills most of W: slower than per-frame launches
-        BwdRegwKernel kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(ksb_room, mt, wv) : bwd_regw_kernel_for<float>(ksb_room, mt, wv);
+        // A share of 64 fragments does not fit the registers next to a frame's DX (with all of it in registers the compiler
+        // spills part of W, in float32 most of it): half of it lives in LDS.
+        const bool lds_share = ksb_room == 64;
+        if (lds_share && (mt != 1 || wv != kWaves)) continue;
+        BwdRegwKernel kfn;
+        if (lds_share)
+          kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_lds_kernel_for<__bf16>() : bwd_regw_lds_kernel_for<float>();
+        else
+          kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(ksb_room, mt, wv) : bwd_regw_kernel_for<float>(ksb_room, mt, wv);
         if (!kfn) continue;
+        const size_t cand_lds = lds_share ? kBwdLdsShareBytes : 0;
+        if (cand_lds) {
+          rc = ensure_lds_limit((const void*)kfn, cand_lds);
+          if (rc != RTN_OK) return rc;
+        }
         int per_cu = 0;
-        RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kfn, 64 * wv, 0));
+        RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kfn, 64 * wv, cand_lds));
         const long long groups_needed = (B + use_rows - 1) / use_rows;
         // batch groups of every problem that one launch can hold
         const long long fit = (long long)per_cu * device_info().cus / ((long long)count * (n / (16 * mt)));
@@ -1101,6 +1123,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
           KSB = ksb;
           rows_per_group = use_rows;
           groups_per_launch = (int)groups_needed;
+          bwd_lds = cand_lds;
           break;
         }
         // Too many rows for one launch: remember the candidate that takes most rows per launch; the batch groups
@@ -1109,6 +1132,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
           turn_rows = fit * use_rows;
           turn_pk = (const void*)kfn;
           turn_cfg[0] = use_rows; turn_cfg[1] = mt; turn_cfg[2] = wv; turn_cfg[3] = ksb; turn_cfg[4] = (int)fit;
+          turn_lds = cand_lds;
         }
       }
       if (!pk && turn_pk) {
@@ -1118,6 +1142,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
         bwd_waves = turn_cfg[2];
         KSB = turn_cfg[3];
         groups_per_launch = turn_cfg[4];
+        bwd_lds = turn_lds;
       }
     }
     if (!pk && count > 1) {
@@ -1192,7 +1217,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
         multi.q[k].group_offset = g0;
       }
       void* args[] = {(void*)&multi};
-      RTN_HIP(hipLaunchCooperativeKernel(pk, dim3((unsigned)(count * multi.wgs_each)), dim3((unsigned)(64 * bwd_waves)), args, 0, stream));
+      RTN_HIP(hipLaunchCooperativeKernel(pk, dim3((unsigned)(count * multi.wgs_each)), dim3((unsigned)(64 * bwd_waves)), args, (unsigned)bwd_lds, stream));
     }
     for (int k = 0; k < count; ++k) {
       const BwdJob& j = jobs[(size_t)k];

@@ -46,7 +46,7 @@ def _run(T, B, n, dtype, start, step, seed=0, scale_x=0.5):
 
 
 @pytest.mark.parametrize("start,step", [(0, 1), (0, -1), (1, 2), (2, -3)])
-@pytest.mark.parametrize("T,B,n", [(7, 3, 16), (12, 20, 64), (9, 40, 128), (6, 5, 20), (5, 2, 3), (5, 9, 48), (4, 12, 400)])
+@pytest.mark.parametrize("T,B,n", [(7, 3, 16), (12, 20, 64), (9, 40, 128), (6, 5, 20), (5, 2, 3), (5, 9, 48), (4, 12, 400), (3, 9, 1024), (4, 20, 720)])
 def test_bwd_f32(T, B, n, start, step):
     announce("bwd f32", T, B, n, start, step)
     got, want, _ = _run(T, B, n, "f32", start, step, seed=T + n)
