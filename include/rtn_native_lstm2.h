@@ -43,6 +43,10 @@ extern "C" {
 #define RTN_DTYPE_F32 0
 #define RTN_DTYPE_BF16 1
 
+/* Widths: the matrix-core kernels take n that is a multiple of 32.  Any other n above 32 runs zero-padded to the next
+ * multiple of 32 on copies inside the workspace (the size queries include them); the results are those of the
+ * unpadded problem, since a padded cell has zero inputs, weights and state.  n up to 32 runs on element-wise kernels. */
+
 /* Execution mode.
  * AUTO:       PERSISTENT when the shape and device allow it and the stream is not
  *             being captured, else GRAPH.
@@ -104,10 +108,9 @@ int rtn_native_lstm2_fwd_status(const void* workspace, void* hip_stream);
  * holds the arguments of one rtn_native_lstm2_fwd call and gets exactly that call's results.  When
  * the device can hold the persistent kernel of all of them at once, they run in ONE cooperative
  * launch and hide each other's exchange latency; otherwise they are enqueued back to back.
- * `workspace` holds `count` equal slices, slice k for call k;
- * rtn_native_lstm2_fwd_multi_workspace_bytes(count, ...) gives the total (a slice can be larger than a single
- * call's workspace, because the decomposition may differ when several problems share the device).  The calls must not alias each
- * other's outputs.
+ * `workspace` is shared by the `count` calls; rtn_native_lstm2_fwd_multi_workspace_bytes(count, ...) gives the
+ * total (more than `count` single-call workspaces can be needed, because the decomposition may differ when several
+ * problems share the device).  The calls must not alias each other's outputs.
  */
 typedef struct rtn_lstm2_call {
   const void* X;

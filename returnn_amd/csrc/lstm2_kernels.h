@@ -184,6 +184,30 @@ __global__ void k_prepare_mfma(Lstm2Params p, int n_flags) {
   }
 }
 
+// Widths the matrix-core kernels do not take run zero-padded: dst[rows_dst][blocks][n_pad] takes src[rows_src][blocks][n]
+// (rows_src <= rows_dst) and zeros elsewhere; ET is an unsigned integer of the element's size (bits are copied).
+template <typename ET>
+__global__ void k_pad_cells(const ET* __restrict__ src, ET* __restrict__ dst, long long rows_src, long long rows_dst, int blocks,
+                            int n, int n_pad) {
+  const long long total = rows_dst * blocks * n_pad;
+  for (long long idx = blockIdx.x * (long long)blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
+    const int j = (int)(idx % n_pad);
+    const long long rb = idx / n_pad;  // row * blocks + block
+    dst[idx] = (j < n && rb / blocks < rows_src) ? src[rb * n + j] : (ET)0;
+  }
+}
+
+// The inverse: dst[rows][blocks][n] from src[rows][blocks][n_pad].
+template <typename ET>
+__global__ void k_unpad_cells(const ET* __restrict__ src, ET* __restrict__ dst, long long rows, int blocks, int n, int n_pad) {
+  const long long total = rows * blocks * n;
+  for (long long idx = blockIdx.x * (long long)blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
+    const int j = (int)(idx % n);
+    const long long rb = idx / n;
+    dst[idx] = src[rb * n_pad + j];
+  }
+}
+
 // Clears the status word for the generic path.
 __global__ void k_fill_u32(unsigned* dst, unsigned value, long long count) {
   for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < count;

@@ -15,6 +15,7 @@
 #include <list>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include <rocblas/rocblas.h>
 
@@ -494,7 +495,91 @@ int check_dims(int64_t T, int32_t B, int32_t n, int32_t dtype) {
 
 // Workspace of one problem of an entry with `count` problems: the largest layout any resolution of `mode`
 // can need (AUTO may fall back to per-step launches, and the plan depends on how many problems share a launch).
-size_t workspace_each(int count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
+// ---- widths the matrix-core kernels do not take ------------------------------------------------------------------
+// n that is not a multiple of 32 runs zero-padded to the next multiple: a padded cell has zero inputs, zero weights (rows
+// and columns) and a zero initial state, so its cell state and output are exactly 0 in every frame, it adds nothing to
+// the other cells' sums and all its gradients are 0 -- the results are those of the unpadded problem.  The copies cost
+// about the op's own memory traffic again, far less than the element-wise kernels that such widths would otherwise
+// run on (n=1000: 120 times slower).  Widths up to 32 stay on those kernels; RTN_LSTM2_NO_PAD=1 switches the padding off.
+int padded_width(int n) {
+  if (n % 32 == 0 || n <= 32 || env_long("RTN_LSTM2_NO_PAD", 0)) return n;
+  return (n + 31) / 32 * 32;
+}
+
+// Padded copies of one forward call's tensors (byte offsets into its share of the workspace).
+struct FwdPadLayout {
+  size_t X = 0, W = 0, y0 = 0, c0 = 0, Y = 0, C = 0, H = 0, d = 0, total = 0;
+};
+FwdPadLayout fwd_pad_layout(int64_t T, int B, int np, int dtype) {
+  const size_t es = esize(dtype), tb = (size_t)T * B, bn = (size_t)B * np;
+  FwdPadLayout l;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { const size_t at = off; off = align_up(off + bytes, 256); return at; };
+  l.X = take(tb * 4 * np * es);
+  l.W = take((size_t)np * 4 * np * es);
+  l.y0 = take(bn * es);
+  l.c0 = take(bn * 4);
+  l.Y = take(tb * np * es);
+  l.C = take(tb * np * 4);
+  l.H = take(tb * 4 * np * es);
+  l.d = take(bn * 4);
+  l.total = off;
+  return l;
+}
+
+// Padded copies of one gradient call's tensors.
+struct BwdPadLayout {
+  size_t W = 0, y0 = 0, c0 = 0, Y = 0, C = 0, H = 0, DY = 0, Dd = 0, DX = 0, DW = 0, Dy0 = 0, Dc0 = 0, total = 0;
+};
+BwdPadLayout bwd_pad_layout(int64_t T, int B, int np, int dtype) {
+  const size_t es = esize(dtype), tb = (size_t)T * B, bn = (size_t)B * np;
+  BwdPadLayout l;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { const size_t at = off; off = align_up(off + bytes, 256); return at; };
+  l.W = take((size_t)np * 4 * np * es);
+  l.y0 = take(bn * es);
+  l.c0 = take(bn * 4);
+  l.Y = take(tb * np * es);
+  l.C = take(tb * np * 4);
+  l.H = take(tb * 4 * np * es);
+  l.DY = take(tb * np * es);
+  l.Dd = take(bn * 4);
+  l.DX = take(tb * 4 * np * es);
+  l.DW = take((size_t)np * 4 * np * 4);
+  l.Dy0 = take(bn * es);
+  l.Dc0 = take(bn * 4);
+  l.total = off;
+  return l;
+}
+
+// dst[rows_dst][blocks][np] := src[rows_src][blocks][n], zeros elsewhere; elements of `es` bytes.
+int launch_pad(const void* src, void* dst, long long rows_src, long long rows_dst, int blocks, int n, int np, size_t es, hipStream_t stream) {
+  const long long total = rows_dst * blocks * np;
+  if (total <= 0) return RTN_OK;
+  const dim3 grid((unsigned)std::min<long long>((total + 255) / 256, 8192)), block(256);
+  if (es == 2)
+    hipLaunchKernelGGL(k_pad_cells<unsigned short>, grid, block, 0, stream, (const unsigned short*)src, (unsigned short*)dst, rows_src, rows_dst, blocks, n, np);
+  else
+    hipLaunchKernelGGL(k_pad_cells<unsigned>, grid, block, 0, stream, (const unsigned*)src, (unsigned*)dst, rows_src, rows_dst, blocks, n, np);
+  RTN_HIP(hipGetLastError());
+  return RTN_OK;
+}
+
+// dst[rows][blocks][n] := src[rows][blocks][np].
+int launch_unpad(const void* src, void* dst, long long rows, int blocks, int n, int np, size_t es, hipStream_t stream) {
+  const long long total = rows * blocks * n;
+  if (total <= 0) return RTN_OK;
+  const dim3 grid((unsigned)std::min<long long>((total + 255) / 256, 8192)), block(256);
+  if (es == 2)
+    hipLaunchKernelGGL(k_unpad_cells<unsigned short>, grid, block, 0, stream, (const unsigned short*)src, (unsigned short*)dst, rows, blocks, n, np);
+  else
+    hipLaunchKernelGGL(k_unpad_cells<unsigned>, grid, block, 0, stream, (const unsigned*)src, (unsigned*)dst, rows, blocks, n, np);
+  RTN_HIP(hipGetLastError());
+  return RTN_OK;
+}
+
+// Workspace of one of `count` forward calls at a width the kernels take as it is.
+size_t workspace_each_exact(int count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
   size_t need = 0;
   Plan pl;
   std::string why;
@@ -507,6 +592,15 @@ size_t workspace_each(int count, int64_t T, int32_t B, int32_t n, int32_t dtype,
     }
   }
   return need;
+}
+
+// Workspace of one of `count` forward calls: for a padded width, that of the padded problem plus the padded copies.
+// The calls' own workspaces come first (call k at k * workspace_each_exact(count, ..., padded width, ...): the status
+// queries look there), the padded copies of all calls after them.
+size_t workspace_each(int count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
+  const int np = padded_width(n);
+  if (np == n || T == 0 || B == 0) return workspace_each_exact(count, T, B, n, dtype, mode);
+  return workspace_each_exact(count, T, B, np, dtype, mode) + fwd_pad_layout(T, B, np, dtype).total;
 }
 
 // The calls of one entry: `count` independent problems of one shape.  Each gets the slice
@@ -530,6 +624,47 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
       hipLaunchKernelGGL(k_copy_f32, dim3((unsigned)std::min<long long>((bn + 255) / 256, 1024)), dim3(256), 0, stream,
                          calls[k].c0, calls[k].d, bn);
       RTN_HIP(hipGetLastError());
+    }
+    return RTN_OK;
+  }
+  const int np = padded_width(n);
+  if (np != n) {
+    // Run the problem zero-padded to a width the matrix-core kernels take (see padded_width), on copies in the workspace.
+    for (int k = 0; k < count; ++k) {
+      const rtn_lstm2_call& c = calls[k];
+      const void* ptrs[] = {c.X, c.W, c.y0, c.c0, c.i, c.Y, c.C, c.H, c.d};
+      const char* names[] = {"X", "W", "y0", "c0", "i", "Y", "C", "H", "d"};
+      for (int q = 0; q < 9; ++q)
+        if (!ptrs[q]) return fail(RTN_ERR_ARG, "NativeLstm2: %s must not be null", names[q]);
+    }
+    const size_t inner_each = workspace_each_exact(count, T, B, np, dtype, mode);
+    const FwdPadLayout L = fwd_pad_layout(T, B, np, dtype);
+    const size_t need = (size_t)count * (inner_each + L.total);
+    if (!workspace || workspace_bytes < need)
+      return fail(RTN_ERR_WORKSPACE, "NativeLstm2: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
+    if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2: workspace must be 16-byte aligned");
+    const size_t es = esize(dtype);
+    const long long tb = (long long)T * B;
+    std::vector<rtn_lstm2_call> padded((size_t)count);
+    for (int k = 0; k < count; ++k) {
+      const rtn_lstm2_call& c = calls[k];
+      unsigned char* base = (unsigned char*)workspace + (size_t)count * inner_each + (size_t)k * L.total;
+      if ((rc = launch_pad(c.X, base + L.X, tb, tb, 4, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_pad(c.W, base + L.W, n, np, 4, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_pad(c.y0, base + L.y0, B, B, 1, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_pad(c.c0, base + L.c0, B, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
+      padded[(size_t)k] = {base + L.X, base + L.W, base + L.y0, (const float*)(base + L.c0), c.i, c.start, c.step,
+                           base + L.Y, (float*)(base + L.C), base + L.H, (float*)(base + L.d)};
+    }
+    rc = fwd_calls(padded.data(), count, T, B, np, dtype, mode, workspace, (size_t)count * inner_each, hip_stream, op_flags);
+    if (rc != RTN_OK) return rc;
+    for (int k = 0; k < count; ++k) {
+      const rtn_lstm2_call& c = calls[k];
+      const rtn_lstm2_call& q = padded[(size_t)k];
+      if ((rc = launch_unpad(q.Y, c.Y, tb, 1, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_unpad(q.C, c.C, tb, 1, n, np, 4, stream)) != RTN_OK) return rc;
+      if ((rc = launch_unpad(q.H, c.H, tb, 4, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_unpad(q.d, c.d, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
     }
     return RTN_OK;
   }
@@ -810,6 +945,8 @@ const char* rtn_native_lstm2_describe_multi_plan(int32_t count, int64_t T, int32
   std::string why;
   char buf[512];
   const int c = env_long("RTN_LSTM2_NO_FUSE", 0) ? 1 : std::max(1, std::min(count, kMaxMulti));
+  const int n_asked = n;
+  if (check_dims(T, B, n, dtype) == RTN_OK && T > 0 && B > 0) n = padded_width(n);  // the plan is that of the padded problem
   if (check_dims(T, B, n, dtype) != RTN_OK) {
     g_plan_text = "invalid: " + g_last_error;
   } else if (!make_plan(T, B, n, dtype, mode, false, &pl, &why, 2, c)) {
@@ -819,7 +956,9 @@ const char* rtn_native_lstm2_describe_multi_plan(int32_t count, int64_t T, int32
              mode_name(pl.mode),
              pl.kind == kPlanMfma ? (pl.regw ? "mfma_regw" : "mfma_lds") : (pl.kind == kPlanGeneric ? "generic" : "empty"), pl.MT,
              pl.NT, pl.groups, pl.wgs_per_group, (pl.mode == RTN_MODE_PERSISTENT && pl.regw) ? pl.grid : pl.groups * pl.wgs_per_group,
-             pl.Bg, pl.passes, pl.lds_bytes, count > 1 ? workspace_each(count, T, B, n, dtype, mode) : pl.total);
+             pl.Bg, pl.passes, pl.lds_bytes,
+             (count > 1 || n != n_asked) ? workspace_each(count, T, B, n_asked, dtype, mode) : pl.total);
+    if (n != n_asked) snprintf(buf + strlen(buf), sizeof(buf) - strlen(buf), " padded_width=%d", n);
     if (pl.off_trace) snprintf(buf + strlen(buf), sizeof(buf) - strlen(buf), " trace_offset=%zu", pl.off_trace);
     g_plan_text = buf;
   }
@@ -876,7 +1015,9 @@ size_t rtn_native_lstm2_fwd_multi_workspace_bytes(int32_t count, int64_t T, int3
 int rtn_native_lstm2_fwd_multi_status(const void* workspace, int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype,
                                       int32_t mode, void* hip_stream) {
   g_last_error.clear();
-  const size_t each = count > 1 ? workspace_each(count, T, B, n, dtype, mode) : rtn_native_lstm2_fwd_workspace_bytes(T, B, n, dtype, mode);
+  if (check_dims(T, B, n, dtype) != RTN_OK || mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return RTN_ERR_ARG;
+  // call k's own workspace (for a padded width: that of the padded problem) starts at k * each
+  const size_t each = workspace_each_exact(std::max(count, 1), T, B, (T > 0 && B > 0) ? padded_width(n) : n, dtype, mode);
   if (!workspace || each == 0 || count < 0) return fail(RTN_ERR_ARG, "NativeLstm2: bad arguments to the status query");
   for (int k = 0; k < count; ++k) {
     const int rc = rtn_native_lstm2_fwd_status((const unsigned char*)workspace + (size_t)k * each, hip_stream);
@@ -985,7 +1126,10 @@ int rtn_lstm_low_mem_fwd(const void* X, const void* W, const void* b, const void
 
 size_t rtn_native_lstm2_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype) {
   if (check_dims(T, B, n, dtype) != RTN_OK) return 0;
-  return bwd_layout(B, n, dtype).total;
+  const int np = padded_width(n);
+  if (np == n || T == 0 || B == 0) return bwd_layout(B, n, dtype).total;
+  // a padded width: the workspace of the padded problem, then the padded copies
+  return bwd_layout(B, np, dtype).total + bwd_pad_layout(T, B, np, dtype).total;
 }
 
 namespace {
@@ -1046,6 +1190,47 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       if (!ptrs[q]) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must not be null", names[q]);
       if (q != 3 && !aligned16(ptrs[q])) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must be 16-byte aligned", names[q]);
     }
+  }
+  const int np = padded_width(n);
+  if (np != n) {
+    // Run the problem zero-padded to a width the matrix-core kernels take (see padded_width), on copies in the
+    // workspace: first the workspaces of the padded calls, then the copies of each call.
+    const BwdLayout lay_p = bwd_layout(B, np, dtype);
+    const BwdPadLayout L = bwd_pad_layout(T, B, np, dtype);
+    const size_t need = (size_t)count * (lay_p.total + L.total);
+    if (!workspace || workspace_bytes < need)
+      return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
+    if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: workspace must be 16-byte aligned");
+    const size_t es = esize(dtype);
+    const long long tb = (long long)T * B;
+    std::vector<rtn_lstm2_bwd_call> padded((size_t)count);
+    for (int k = 0; k < count; ++k) {
+      const rtn_lstm2_bwd_call& c = calls[k];
+      unsigned char* base = (unsigned char*)workspace + (size_t)count * lay_p.total + (size_t)k * L.total;
+      if ((rc = launch_pad(c.W, base + L.W, n, np, 4, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_pad(c.y0, base + L.y0, B, B, 1, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_pad(c.c0, base + L.c0, B, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
+      if ((rc = launch_pad(c.Y, base + L.Y, tb, tb, 1, n, np, es, stream)) != RTN_OK) return rc;
+      // the sibling op that keeps its cell states in H hands H in for C as well; it is not read then
+      if (!(op_flags & kOpH0IsCell) && (rc = launch_pad(c.C, base + L.C, tb, tb, 1, n, np, 4, stream)) != RTN_OK) return rc;
+      if ((rc = launch_pad(c.H, base + L.H, tb, tb, 4, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_pad(c.DY, base + L.DY, tb, tb, 1, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_pad(c.Dd, base + L.Dd, B, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
+      padded[(size_t)k] = {base + L.W, base + L.y0, (const float*)(base + L.c0), c.i, c.start, c.step, base + L.Y,
+                           (const float*)(base + ((op_flags & kOpH0IsCell) ? L.H : L.C)), base + L.H, base + L.DY,
+                           (const float*)(base + L.Dd), base + L.DX, (float*)(base + L.DW), base + L.Dy0, (float*)(base + L.Dc0)};
+    }
+    rc = bwd_calls(padded.data(), count, T, B, np, dtype, workspace, (size_t)count * lay_p.total, hip_stream, op_flags);
+    if (rc != RTN_OK) return rc;
+    for (int k = 0; k < count; ++k) {
+      const rtn_lstm2_bwd_call& c = calls[k];
+      const rtn_lstm2_bwd_call& q = padded[(size_t)k];
+      if ((rc = launch_unpad(q.DX, c.DX, tb, 4, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_unpad(q.DW, c.DW, n, 4, n, np, 4, stream)) != RTN_OK) return rc;
+      if ((rc = launch_unpad(q.Dy0, c.Dy0, B, 1, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_unpad(q.Dc0, c.Dc0, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
+    }
+    return RTN_OK;
   }
   const BwdLayout lay = bwd_layout(B, n, dtype);
   if (!workspace || workspace_bytes < lay.total * (size_t)count)

@@ -16,8 +16,7 @@ Argument handling follows the generated wrapper (:144-193): dtype normalisation,
 ``.contiguous()`` for ``need_contiguous`` inputs, device guard on the first tensor, outputs allocated on
 that device.  Differences, on purpose: bfloat16 inputs stay bfloat16 (X, W, y0, Y, H in bf16; c0, C, d,
 mask in float32) instead of being up-cast; outputs are not zero-filled first because the library writes
-every element; CPU tensors are rejected (no CPU implementation is shipped); widths that are not a multiple of 32
-run zero-padded to the next multiple (see ``_padded_width``), with the results of the unpadded problem.
+every element; CPU tensors are rejected (no CPU implementation is shipped).
 """
 
 from __future__ import annotations
@@ -289,40 +288,6 @@ def _normalise_lstm2_args(X, W, y0, c0, i):
 
 
 
-# Widths the matrix-core kernels do not take (n not a multiple of 32) run zero-padded to the next multiple of 32: a
-# padded cell has zero inputs, zero weights (rows and columns) and a zero initial state, so its cell state and output
-# stay exactly 0 in every frame, it adds nothing to the other cells' sums, and all its gradients are 0.  The copies cost
-# about as much memory traffic again as the op itself, which is far less than the element-wise kernels the library
-# falls back to at such widths.  Widths up to 32 stay on those kernels (cheap there); RTN_LSTM2_NO_PAD=1 switches the padding off.
-def _padded_width(n: int) -> int:
-    import os
-
-    if n % 32 == 0 or n <= 32 or os.environ.get("RTN_LSTM2_NO_PAD", "") not in ("", "0"):
-        return n
-    return (n + 31) // 32 * 32
-
-
-def _pad_cells(t: torch.Tensor, n: int, n_pad: int, blocks: int = 1) -> torch.Tensor:
-    """[..., blocks*n] -> [..., blocks*n_pad], every block of n cells followed by zeros."""
-    lead = tuple(t.shape[:-1])
-    out = t.new_zeros(lead + (blocks, n_pad))
-    out[..., :n] = t.reshape(lead + (blocks, n))
-    return out.reshape(lead + (blocks * n_pad,))
-
-
-def _unpad_cells(t: torch.Tensor, n: int, n_pad: int, blocks: int = 1) -> torch.Tensor:
-    """Inverse of :func:`_pad_cells`."""
-    lead = tuple(t.shape[:-1])
-    return t.reshape(lead + (blocks, n_pad))[..., :n].reshape(lead + (blocks * n,)).contiguous()
-
-
-def _pad_weights(W: torch.Tensor, n: int, n_pad: int) -> torch.Tensor:
-    """W [n,4n] -> [n_pad,4n_pad] with zero rows and columns for the padded cells."""
-    out = W.new_zeros((n_pad, 4, n_pad))
-    out[:n, :, :n] = W.reshape(n, 4, n)
-    return out.reshape(n_pad, 4 * n_pad)
-
-
 def _alloc_lstm2_outputs(T, B, n, bf16, device):
     act = torch.bfloat16 if bf16 else torch.float32
     Y = torch.empty((T, B, n), dtype=act, device=device)
@@ -335,12 +300,6 @@ def _alloc_lstm2_outputs(T, B, n, bf16, device):
 def _native_lstm2_device_impl(X, W, y0, c0, i, start, step):
     """``NativeLstm2`` on HIP tensors: normalise the arguments, allocate outputs and scratch, enqueue the library call."""
     (X, W, y0, c0, i), (T, B, n, bf16) = _normalise_lstm2_args(X, W, y0, c0, i)
-    n_pad = _padded_width(n)
-    if n_pad != n and T > 0 and B > 0:
-        Y, C, H, d = _native_lstm2_device_impl(
-            _pad_cells(X, n, n_pad, 4), _pad_weights(W, n, n_pad), _pad_cells(y0, n, n_pad), _pad_cells(c0, n, n_pad), i, start, step
-        )
-        return _unpad_cells(Y, n, n_pad), _unpad_cells(C, n, n_pad), _unpad_cells(H, n, n_pad, 4), _unpad_cells(d, n, n_pad)
     device = X.device
     lib = _lib.load()
     dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
@@ -384,10 +343,6 @@ def _lstm_generic_base_device_impl(Z, V_h, c, i):
             raise RuntimeError("LstmGenericBase: %s has shape %s, expected %s" % (name, tuple(t.shape), shape))
         if t.device != device:
             raise RuntimeError("LstmGenericBase: %s is on %s but Z is on %s" % (name, t.device, device))
-    n_pad = _padded_width(n)
-    if n_pad != n and T > 0 and B > 0:
-        Y, H, d = _lstm_generic_base_device_impl(_pad_cells(Z, n, n_pad, 4), _pad_weights(V_h, n, n_pad), _pad_cells(c, n, n_pad), i)
-        return _unpad_cells(Y, n, n_pad), _unpad_cells(H, n, n_pad, 4), _unpad_cells(d, n, n_pad)
     lib = _lib.load()
     with torch.cuda.device(device):
         Y = torch.empty((T, B, n), dtype=act, device=device)
@@ -418,14 +373,6 @@ def _lstm_low_mem_device_impl(X, W, b, y0, c0, i, start, step):
             raise RuntimeError("LstmLowMem: %s has shape %s, expected %s" % (name, tuple(t.shape), shape))
         if t.device != device:
             raise RuntimeError("LstmLowMem: %s is on %s but X is on %s" % (name, t.device, device))
-    n_pad = _padded_width(n)
-    if n_pad != n and T > 0 and B > 0:
-        W_pad = W.new_zeros((n_in + n_pad, 4, n_pad))  # the rows of the input part, then those of the (padded) recurrent part
-        W_pad[: n_in + n, :, :n] = W.reshape(n_in + n, 4, n)
-        Y, C, d = _lstm_low_mem_device_impl(
-            X, W_pad.reshape(n_in + n_pad, 4 * n_pad), _pad_cells(b, n, n_pad, 4), _pad_cells(y0, n, n_pad), _pad_cells(c0, n, n_pad), i, start, step
-        )
-        return _unpad_cells(Y, n, n_pad), _unpad_cells(C, n, n_pad), _unpad_cells(d, n, n_pad)
     lib = _lib.load()
     with torch.cuda.device(device):
         Y = torch.empty((T, B, n), dtype=act, device=device)
@@ -466,16 +413,6 @@ def native_lstm2_multi(calls, *, mode: Optional[str] = None):
     if not norm[0][0][0].is_cuda:
         raise RuntimeError("NativeLstm2: this build implements the op for HIP (MI355X) tensors only; got CPU tensors.")
     T, B, n, bf16 = shape
-    n_pad = _padded_width(n)
-    if n_pad != n and T > 0 and B > 0:
-        padded = [
-            (_pad_cells(X, n, n_pad, 4), _pad_weights(W, n, n_pad), _pad_cells(y0, n, n_pad), _pad_cells(c0, n, n_pad), i, c[5], c[6])
-            for (X, W, y0, c0, i), c in zip((t for t, _ in norm), calls)
-        ]
-        return [
-            (_unpad_cells(Y, n, n_pad), _unpad_cells(C, n, n_pad), _unpad_cells(H, n, n_pad, 4), _unpad_cells(d, n, n_pad))
-            for Y, C, H, d in native_lstm2_multi(padded, mode=mode)
-        ]
     dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
     mode_code = _lib.MODES[mode or OpMaker.options.get("NativeLstm2", {}).get("mode", "auto")]
     count = len(calls)
@@ -558,17 +495,6 @@ def native_lstm2_grad_multi(calls):
             raise RuntimeError("native_lstm2_grad_multi: all calls must have one shape, dtype and device; got %r and %r" % (shape, this))
         norm.append((tensors, int(start), int(step)))
     T, B, n, bf16 = shape
-    n_pad = _padded_width(n)
-    if n_pad != n and T > 0 and B > 0:
-        padded = [
-            (_pad_weights(W, n, n_pad), _pad_cells(y0, n, n_pad), _pad_cells(c0, n, n_pad), i, start, step, _pad_cells(Y, n, n_pad),
-             _pad_cells(C, n, n_pad), _pad_cells(H, n, n_pad, 4), _pad_cells(DY, n, n_pad), _pad_cells(Dd, n, n_pad))
-            for (W, y0, c0, i, Y, C, H, DY, Dd), start, step in norm
-        ]  # fmt: skip
-        return [
-            (_unpad_cells(DX, n, n_pad, 4), DW.reshape(n_pad, 4, n_pad)[:n, :, :n].reshape(n, 4 * n).contiguous(), _unpad_cells(Dy0, n, n_pad), _unpad_cells(Dc0, n, n_pad))
-            for DX, DW, Dy0, Dc0 in native_lstm2_grad_multi(padded)
-        ]
     lib = _lib.load()
     dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
     count = len(norm)
@@ -639,13 +565,6 @@ def lstm_generic_base_grad(V_h, c, i, Y, H, DY, Dd):
             raise RuntimeError("LstmGenericBase gradient: %s has shape %s, expected %s" % (name, tuple(t.shape), expect[name]))
         if t.device != device:
             raise RuntimeError("LstmGenericBase gradient: %s is on %s but Y is on %s" % (name, t.device, device))
-    n_pad = _padded_width(n)
-    if n_pad != n and T > 0 and B > 0:
-        DZ, DV_h, Dc = lstm_generic_base_grad(
-            _pad_weights(V_h, n, n_pad), _pad_cells(c, n, n_pad), i, _pad_cells(Y, n, n_pad), _pad_cells(H, n, n_pad, 4),
-            _pad_cells(DY, n, n_pad), _pad_cells(Dd, n, n_pad),
-        )  # fmt: skip
-        return _unpad_cells(DZ, n, n_pad, 4), DV_h.reshape(n_pad, 4, n_pad)[:n, :, :n].reshape(n, 4 * n).contiguous(), _unpad_cells(Dc, n, n_pad)
     lib = _lib.load()
     dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
     with torch.cuda.device(device):

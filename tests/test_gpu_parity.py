@@ -442,21 +442,26 @@ def test_batch_in_several_persistent_launches(T, B, n, dtype, start, step):
 
 @pytest.mark.parametrize("T,B,n,dtype,start,step", [(9, 5, 100, "f32", 0, 1), (6, 33, 1000, "bf16", 0, -1), (5, 3, 50, "bf16", 1, 2), (7, 4, 40, "f32", 1, -2)])
 def test_widths_that_run_zero_padded(T, B, n, dtype, start, step):
-    """Widths that are not a multiple of 32: the torch-level op pads the cells with zeros to the next multiple of 32 and
-    runs the matrix-core kernels; forward and gradient against the oracle, and the forward against the library's own
-    element-wise kernels at the original width (the C ABI called directly)."""
+    """Widths that are not a multiple of 32: the library pads the cells with zeros to the next multiple of 32 (on copies
+    in the workspace) and runs the matrix-core kernels; forward and gradient against the oracle, and the forward against
+    the library's own element-wise kernels at the original width (padding switched off)."""
     from _gpu_util import to_dev
-    from returnn_amd import native_op, torch_native_op
+    from returnn_amd import lib, native_op, torch_native_op
 
     announce("zero_padded", T, B, n, dtype, start, step)
-    assert torch_native_op._padded_width(n) != n
+    plan = lib.load().rtn_native_lstm2_describe_plan(T, B, n, lib.DTYPE_BF16 if dtype == "bf16" else lib.DTYPE_F32, lib.MODES["auto"]).decode()
+    assert "kernel=mfma_regw" in plan and "padded_width=%i" % ((n + 31) // 32 * 32) in plan, plan
     p = random_problem(970 + n, T, B, n)
     X, W, y0, c0, i = p
     want = oracle.native_lstm2_fwd(*p, start, step, threads=oracle.max_threads())
     got = run_op(*p, start, step, dtype=dtype)
     check = check_f32 if dtype == "f32" else check_bf16
     check(got, want, "padded %s" % ((T, B, n),))
-    rc, status, raw = run_raw(*p, start, step, dtype=dtype)
+    rc, status, raw = run_raw(*p, start, step, dtype=dtype)  # poisoned outputs: every element must be written
+    assert rc == 0 and status == 0
+    check(raw, want[:4], "padded, direct call")
+    with env(RTN_LSTM2_NO_PAD=1):
+        rc, status, raw = run_raw(*p, start, step, dtype=dtype)
     assert rc == 0 and status == 0
     check(got[:4], raw, "padded against element-wise kernels")
     rng = numpy.random.default_rng(971)
