@@ -296,12 +296,12 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   const unsigned frame_bytes = (unsigned)((size_t)p.B * n4 * ES);
 
   // A fragments: this wavefront's macro steps [wave*ksb, (wave+1)*ksb) of the 16*MT rows of W, as far as the 4n/KM macro
-  // steps reach.  Slots beyond them hold zeros in W and read nothing (or, in the 64-slot variant, a fragment that is
-  // multiplied by that zero), so that any width whose share per wavefront is at most KSB runs on this kernel.
+  // steps reach.  Slots beyond them hold zeros in W and read nothing (or, in the chunked variants, a fragment that is
+  // multiplied by that zero), so that any width whose share per wavefront is at most KSB + KSL runs on this kernel.
   const int ksb = q.ksb;
   const int ks_here = max(0, min(ksb, n4 / KM - ksb * wave));  // uniform over the wavefront
   const int ks_last = max(ks_here, 1) - 1;
-  const int wave_at = (KST > 32 && ks_here == 0) ? 0 : wave;  // 64-slot variant: a wavefront without a share reads the first one's
+  const int wave_at = (KSL > 0 && ks_here == 0) ? 0 : wave;  // chunked variants: a wavefront without a share reads the first one's
   i32x4 wreg[MT][KSB];
   extern __shared__ __align__(16) unsigned char bwd_smem[];
   i32x4* wl = (i32x4*)bwd_smem + (size_t)wave * (KSL > 0 ? KSL : 1) * 64 + lane;  // [WV][KSL][64]: slot s of this lane at wl[s * 64]
@@ -358,9 +358,10 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   auto frame = [&](int f) { return q.t_end - (long long)f * q.step; };
 
   // The B fragments of a frame (the group's rows of DX, this wavefront's share of the contraction range) are taken in
-  // chunks of CH: up to 32 fragments in one go; a wider share (KSL > 0) in chunks of 16 through two sets of registers
-  // (the next chunk is in flight while the matrix cores work on this one).
-  constexpr int CH = KST > 32 ? 16 : KST;
+  // chunks of CH: up to 32 fragments in one go; a wider share (KSL > 0) in chunks of 16 (8 with 8 wavefronts, which have
+  // half the registers each) through two sets of registers: the next chunk is in flight while the matrix cores work on
+  // this one.
+  constexpr int CH = KSL == 0 ? KST : (WV >= 8 ? 8 : 16);
   constexpr int NCH = KST / CH;
   i32x4 bf[NCH > 1 ? 2 : 1][CH];
   auto issue_chunk = [&](long long t, int c, int slot) {

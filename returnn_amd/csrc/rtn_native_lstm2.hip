@@ -849,12 +849,14 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
 
 typedef void (*BwdRegwKernel)(const Lstm2BwdMulti);
 
-// Bytes of dynamic shared memory of the variant that keeps half of a 64-fragment share of W in LDS.
+// Bytes of dynamic shared memory of the variants that keep half of a wavefront's share of W in LDS (4 wavefronts with
+// 32 + 32 fragments, or 8 wavefronts with 16 + 16).
 constexpr size_t kBwdLdsShareBytes = (size_t)kWaves * 32 * 64 * 16;
 
-// The variant with 32 fragments of W per wavefront in registers and 32 in LDS (one tile, 4 wavefronts).
+// The variants with half of W in registers and half in LDS (one tile per workgroup).
 template <typename AT>
-BwdRegwKernel bwd_regw_lds_kernel_for() {
+BwdRegwKernel bwd_regw_lds_kernel_for(int WV) {
+  if (WV == 8) return &k_lstm2_bwd_regw<AT, 16, 1, 8, 16>;
   return &k_lstm2_bwd_regw<AT, 32, 1, 4, 32>;
 }
 
@@ -1283,11 +1285,11 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
         if (mt * ksb_room > 64 || (n / 16) % mt) continue;
         // A share of 64 fragments does not fit the registers next to a frame's DX (with all of it in registers the compiler
         // spills part of W, in float32 most of it): half of it lives in LDS.
-        const bool lds_share = ksb_room == 64;
-        if (lds_share && (mt != 1 || wv != kWaves)) continue;
+        const bool lds_share = ksb_room * wv == 256;
+        if (lds_share && (mt != 1 || (wv != 4 && wv != 8))) continue;
         BwdRegwKernel kfn;
         if (lds_share)
-          kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_lds_kernel_for<__bf16>() : bwd_regw_lds_kernel_for<float>();
+          kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_lds_kernel_for<__bf16>(wv) : bwd_regw_lds_kernel_for<float>(wv);
         else
           kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(ksb_room, mt, wv) : bwd_regw_kernel_for<float>(ksb_room, mt, wv);
         if (!kfn) continue;
