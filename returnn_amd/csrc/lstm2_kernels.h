@@ -364,8 +364,11 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in a scalar register
   const int n = p.n, S = n / KM;
-  i32x4* Wl = (i32x4*)smem;                                  // [MT][S][64] fragments
-  f32x4* red = (f32x4*)(smem + (size_t)MT * S * kTileBytes);  // [kWaves][TILES][64]
+  // A launch of one step uses every fragment of W once: it can take them from memory directly, with many small
+  // workgroups per CU hiding the latency, instead of copying its slice to LDS first (p.w_direct).
+  const bool direct = p.w_direct != 0;
+  i32x4* Wl = (i32x4*)smem;                                                       // [MT][S][64] fragments (unless direct)
+  f32x4* red = (f32x4*)(smem + (direct ? (size_t)0 : (size_t)MT * S * kTileBytes));  // [kWaves][TILES][64]
 
   int g, r;
   map_block(p, blockIdx.x, g, r);
@@ -379,10 +382,9 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
   const unsigned* flags_g = p.flags + (size_t)g * p.wgs_per_group;
 
   // W slice of this workgroup: global (already in fragment order) -> LDS, once per launch.
-  {
-    const i32x4* src = (const i32x4*)p.Wp + (size_t)r * MT * S * 64;
-    for (int i = tid; i < MT * S * 64; i += kWgThreads) Wl[i] = src[i];
-  }
+  const i32x4* Wsrc = (const i32x4*)p.Wp + (size_t)r * MT * S * 64;
+  if (!direct)
+    for (int i = tid; i < MT * S * 64; i += kWgThreads) Wl[i] = Wsrc[i];
 
   // State of the (sequence, cell) pairs this thread owns.
   float c_state[EPT], h_prev[EPT];
@@ -445,11 +447,15 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
     __amdgpu_buffer_rsrc_t hx_rs = __builtin_amdgcn_make_buffer_rsrc((void*)hx_cur, 0, 0x7fffffff, kBufFlags);
     const bool ld_coherent = persist && (p.sync_policy & kLoadCoherent);
     for (int sm0 = wave; sm0 < S; sm0 += kWaves * U) {
-      i32x4 bf[U][NT];
+      i32x4 bf[U][NT], afd[U][MT];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int sm = sm0 + kWaves * u;
         if (sm < S) {
+          if (direct) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) afd[u][mt] = Wsrc[(mt * S + sm) * 64 + lane];
+          }
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) {
             const unsigned off = (unsigned)(((4 * sm + kg) * p.Bp + 16 * nt + jl) * kFragBytes);
@@ -466,7 +472,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
         if (sm < S) {
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
-            const i32x4 af = Wl[(mt * S + sm) * 64 + lane];
+            const i32x4 af = direct ? afd[u][mt] : Wl[(mt * S + sm) * 64 + lane];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(af, bf[u][nt], acc[mt][nt]);
           }

@@ -61,6 +61,7 @@ struct Lstm2Params {
   int poll_delay;     // register kernel: s_sleep(1) repeats between the hidden-value stores and the first read of the next step
   unsigned long long* trace;  // optional [workgroups][8] cycle totals per phase (instrumented builds only)
   int op_flags;       // OpFlags: variations of the recurrence for the sibling ops (0 = NativeLstm2)
+  int w_direct;       // per-step launches of the LDS kernel: 1 = W fragments go from memory straight to the matrix cores (no LDS copy)
   int zero;           // always 0; an operand the compiler cannot fold (idempotent atomics used as L2 reads)
   int sync_policy;    // SyncBits
   unsigned long long timeout_ticks;  // bound of one flag wait, in 100 MHz wall-clock ticks

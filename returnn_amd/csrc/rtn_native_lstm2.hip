@@ -106,6 +106,7 @@ struct Plan {
   int groups_total = 1;          // groups of the whole batch
   int passes = 1;                // persistent launches in turn, each on `groups` of the groups (the last on the rest)
   size_t lds_bytes = 0;
+  bool w_direct = false;         // per-step launches read W from memory without an LDS copy
   // workspace layout (byte offsets)
   size_t off_status = 0, off_flags = 0, off_hx = 0, off_wp = 0, off_ycarry = 0, off_trace = 0, total = 0;
   int n_flags = 0;
@@ -273,8 +274,10 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
       int MT = 1;
       pl.regw = false;
       pl.KSMAX = 0;
-      if (mfma_lds_bytes(n, dtype, 1, 4) > di.lds_per_wg) {
-        pl.kind = kPlanGeneric;  // a W slice of 16 columns does not fit LDS (n far beyond the target sizes)
+      // A step's launch takes W from memory straight into the matrix cores (every fragment is used once per launch).
+      pl.w_direct = env_long("RTN_LSTM2_W_DIRECT", 1) != 0;
+      if (!pl.w_direct && mfma_lds_bytes(n, dtype, 1, 4) > di.lds_per_wg) {
+        pl.kind = kPlanGeneric;  // copied to LDS first, a W slice of 16 columns does not fit (n far beyond the target sizes)
       } else {
         int groups = (B + 63) / 64;
         int Bg = (B + groups - 1) / groups;
@@ -285,7 +288,7 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
         pl.passes = 1;
         pl.wgs_per_group = n / 4;
         pl.Bg = Bg;
-        pl.lds_bytes = mfma_lds_bytes(n, dtype, pl.MT, pl.NT);
+        pl.lds_bytes = pl.w_direct ? (size_t)kWaves * pl.MT * pl.NT * kTileBytes : mfma_lds_bytes(n, dtype, pl.MT, pl.NT);
       }
     }
   } else {
@@ -760,6 +763,7 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     p.groups = p.groups_total = pl.groups_total; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
     p.group_offset = 0;
     p.op_flags = op_flags;
+    p.w_direct = (!pk && pl.kind == kPlanMfma && pl.w_direct) ? 1 : 0;
     p.hx_bufs = kHxRing;
     p.hx_sentinel = pl.regw ? 1 : 0;
     p.exchange = (int)env_long("RTN_LSTM2_EXCHANGE", 0);
