@@ -115,7 +115,7 @@ struct Plan {
 // Most persistent launches in turn that a plan may use instead of the LDS-resident persistent kernel, and instead
 // of per-step launches (from step times measured on MI355X).
 constexpr int kMaxPassesOverLds = 3;
-constexpr int kMaxPassesOverSteps = 32;
+constexpr int kMaxPassesOverSteps = 12;
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 size_t esize(int dtype) { return dtype == RTN_DTYPE_BF16 ? 2 : 4; }
