@@ -108,9 +108,10 @@ int rtn_native_lstm2_fwd_status(const void* workspace, void* hip_stream);
  * holds the arguments of one rtn_native_lstm2_fwd call and gets exactly that call's results.  When
  * the device can hold the persistent kernel of all of them at once, they run in ONE cooperative
  * launch and hide each other's exchange latency; otherwise they are enqueued back to back.
- * `workspace` is shared by the `count` calls; rtn_native_lstm2_fwd_multi_workspace_bytes(count, ...) gives the
- * total (more than `count` single-call workspaces can be needed, because the decomposition may differ when several
- * problems share the device).  The calls must not alias each other's outputs.
+ * `workspace` holds `count` equal slices, slice k for call k;
+ * rtn_native_lstm2_fwd_multi_workspace_bytes(count, ...) gives the total (a slice can be larger than a single
+ * call's workspace, because the decomposition may differ when several problems share the device).  The calls must
+ * not alias each other's outputs.
  */
 typedef struct rtn_lstm2_call {
   const void* X;

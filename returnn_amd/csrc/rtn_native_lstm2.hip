@@ -597,9 +597,8 @@ size_t workspace_each_exact(int count, int64_t T, int32_t B, int32_t n, int32_t 
   return need;
 }
 
-// Workspace of one of `count` forward calls: for a padded width, that of the padded problem plus the padded copies.
-// The calls' own workspaces come first (call k at k * workspace_each_exact(count, ..., padded width, ...): the status
-// queries look there), the padded copies of all calls after them.
+// Workspace of one of `count` forward calls (call k's slice starts at k times this, with its status block first): for a
+// padded width, that of the padded problem followed by the padded copies.
 size_t workspace_each(int count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {
   const int np = padded_width(n);
   if (np == n || T == 0 || B == 0) return workspace_each_exact(count, T, B, n, dtype, mode);
@@ -612,7 +611,7 @@ size_t workspace_each(int count, int64_t T, int32_t B, int32_t n, int32_t dtype,
 // in one cooperative launch (their workgroups share the CUs and hide each other's exchange waits);
 // otherwise they are enqueued one after the other.
 int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode,
-              void* workspace, size_t workspace_bytes, void* hip_stream, int op_flags = 0) {
+              void* workspace, size_t workspace_bytes, void* hip_stream, int op_flags = 0, size_t ws_stride = 0) {
   int rc = check_dims(T, B, n, dtype);
   if (rc != RTN_OK) return rc;
   if (mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return fail(RTN_ERR_ARG, "NativeLstm2: unknown mode %d", mode);
@@ -640,9 +639,11 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
       for (int q = 0; q < 9; ++q)
         if (!ptrs[q]) return fail(RTN_ERR_ARG, "NativeLstm2: %s must not be null", names[q]);
     }
+    // slice k of the workspace: the workspace of the padded call k, then its padded copies
     const size_t inner_each = workspace_each_exact(count, T, B, np, dtype, mode);
     const FwdPadLayout L = fwd_pad_layout(T, B, np, dtype);
-    const size_t need = (size_t)count * (inner_each + L.total);
+    const size_t each = inner_each + L.total;
+    const size_t need = (size_t)count * each;
     if (!workspace || workspace_bytes < need)
       return fail(RTN_ERR_WORKSPACE, "NativeLstm2: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
     if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2: workspace must be 16-byte aligned");
@@ -651,7 +652,7 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     std::vector<rtn_lstm2_call> padded((size_t)count);
     for (int k = 0; k < count; ++k) {
       const rtn_lstm2_call& c = calls[k];
-      unsigned char* base = (unsigned char*)workspace + (size_t)count * inner_each + (size_t)k * L.total;
+      unsigned char* base = (unsigned char*)workspace + (size_t)k * each + inner_each;
       if ((rc = launch_pad(c.X, base + L.X, tb, tb, 4, n, np, es, stream)) != RTN_OK) return rc;
       if ((rc = launch_pad(c.W, base + L.W, n, np, 4, n, np, es, stream)) != RTN_OK) return rc;
       if ((rc = launch_pad(c.y0, base + L.y0, B, B, 1, n, np, es, stream)) != RTN_OK) return rc;
@@ -659,7 +660,7 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
       padded[(size_t)k] = {base + L.X, base + L.W, base + L.y0, (const float*)(base + L.c0), c.i, c.start, c.step,
                            base + L.Y, (float*)(base + L.C), base + L.H, (float*)(base + L.d)};
     }
-    rc = fwd_calls(padded.data(), count, T, B, np, dtype, mode, workspace, (size_t)count * inner_each, hip_stream, op_flags);
+    rc = fwd_calls(padded.data(), count, T, B, np, dtype, mode, workspace, need, hip_stream, op_flags, each);
     if (rc != RTN_OK) return rc;
     for (int k = 0; k < count; ++k) {
       const rtn_lstm2_call& c = calls[k];
@@ -725,7 +726,8 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
       return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no per-step plan: %s", why.c_str());
     break;
   }
-  const size_t each_ws = count > 1 ? workspace_each(count, T, B, n, dtype, mode) : pl.total;
+  // distance between the calls' workspaces: given by a caller that keeps more than the workspace in a call's slice
+  const size_t each_ws = ws_stride ? ws_stride : (count > 1 ? workspace_each(count, T, B, n, dtype, mode) : pl.total);
   if (each_ws < pl.total) return fail(RTN_ERR_WORKSPACE, "NativeLstm2: internal: workspace slice %zu < layout %zu", each_ws, pl.total);
   if (!workspace || workspace_bytes < each_ws * (size_t)count)
     return fail(RTN_ERR_WORKSPACE, "NativeLstm2: workspace of %zu bytes needed, got %zu", each_ws * (size_t)count,
@@ -1022,8 +1024,7 @@ int rtn_native_lstm2_fwd_multi_status(const void* workspace, int32_t count, int6
                                       int32_t mode, void* hip_stream) {
   g_last_error.clear();
   if (check_dims(T, B, n, dtype) != RTN_OK || mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return RTN_ERR_ARG;
-  // call k's own workspace (for a padded width: that of the padded problem) starts at k * each
-  const size_t each = workspace_each_exact(std::max(count, 1), T, B, (T > 0 && B > 0) ? padded_width(n) : n, dtype, mode);
+  const size_t each = workspace_each(std::max(count, 1), T, B, n, dtype, mode);  // call k's slice starts at k * each
   if (!workspace || each == 0 || count < 0) return fail(RTN_ERR_ARG, "NativeLstm2: bad arguments to the status query");
   for (int k = 0; k < count; ++k) {
     const int rc = rtn_native_lstm2_fwd_status((const unsigned char*)workspace + (size_t)k * each, hip_stream);
@@ -1151,7 +1152,7 @@ struct BwdJob {
 // cooperative launch (16-row batch groups when 8-row groups of all problems would not find a CU each); otherwise they
 // are enqueued one after the other.
 int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, int32_t n, int32_t dtype, void* workspace,
-              size_t workspace_bytes, void* hip_stream, int op_flags = 0) {
+              size_t workspace_bytes, void* hip_stream, int op_flags = 0, size_t ws_stride = 0) {
   int rc = check_dims(T, B, n, dtype);
   if (rc != RTN_OK) return rc;
   if (count < 0 || (count > 0 && !calls)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: bad call list");
@@ -1200,10 +1201,11 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
   const int np = padded_width(n);
   if (np != n) {
     // Run the problem zero-padded to a width the matrix-core kernels take (see padded_width), on copies in the
-    // workspace: first the workspaces of the padded calls, then the copies of each call.
+    // workspace: slice k = the workspace of the padded call k, then its copies.
     const BwdLayout lay_p = bwd_layout(B, np, dtype);
     const BwdPadLayout L = bwd_pad_layout(T, B, np, dtype);
-    const size_t need = (size_t)count * (lay_p.total + L.total);
+    const size_t each = lay_p.total + L.total;
+    const size_t need = (size_t)count * each;
     if (!workspace || workspace_bytes < need)
       return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
     if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: workspace must be 16-byte aligned");
@@ -1212,7 +1214,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     std::vector<rtn_lstm2_bwd_call> padded((size_t)count);
     for (int k = 0; k < count; ++k) {
       const rtn_lstm2_bwd_call& c = calls[k];
-      unsigned char* base = (unsigned char*)workspace + (size_t)count * lay_p.total + (size_t)k * L.total;
+      unsigned char* base = (unsigned char*)workspace + (size_t)k * each + lay_p.total;
       if ((rc = launch_pad(c.W, base + L.W, n, np, 4, n, np, es, stream)) != RTN_OK) return rc;
       if ((rc = launch_pad(c.y0, base + L.y0, B, B, 1, n, np, es, stream)) != RTN_OK) return rc;
       if ((rc = launch_pad(c.c0, base + L.c0, B, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
@@ -1226,7 +1228,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
                            (const float*)(base + ((op_flags & kOpH0IsCell) ? L.H : L.C)), base + L.H, base + L.DY,
                            (const float*)(base + L.Dd), base + L.DX, (float*)(base + L.DW), base + L.Dy0, (float*)(base + L.Dc0)};
     }
-    rc = bwd_calls(padded.data(), count, T, B, np, dtype, workspace, (size_t)count * lay_p.total, hip_stream, op_flags);
+    rc = bwd_calls(padded.data(), count, T, B, np, dtype, workspace, need, hip_stream, op_flags, each);
     if (rc != RTN_OK) return rc;
     for (int k = 0; k < count; ++k) {
       const rtn_lstm2_bwd_call& c = calls[k];
@@ -1239,8 +1241,10 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     return RTN_OK;
   }
   const BwdLayout lay = bwd_layout(B, n, dtype);
-  if (!workspace || workspace_bytes < lay.total * (size_t)count)
-    return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: workspace of %zu bytes needed, got %zu", lay.total * (size_t)count,
+  const size_t stride = ws_stride ? ws_stride : lay.total;  // distance between the calls' workspaces
+  if (stride < lay.total) return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: internal: workspace slice %zu < layout %zu", stride, lay.total);
+  if (!workspace || workspace_bytes < stride * (size_t)(count - 1) + lay.total)
+    return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: workspace of %zu bytes needed, got %zu", stride * (size_t)(count - 1) + lay.total,
                 workspace ? workspace_bytes : (size_t)0);
   if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: workspace must be 16-byte aligned");
   rocblas_handle blas = nullptr;
@@ -1339,7 +1343,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     if (!pk && count > 1) {
       // no joint launch: one call after the other, each with its own slice of the workspace
       for (int k = 0; k < count; ++k) {
-        rc = bwd_calls(calls + k, 1, T, B, n, dtype, (unsigned char*)workspace + (size_t)k * lay.total, lay.total, hip_stream, op_flags);
+        rc = bwd_calls(calls + k, 1, T, B, n, dtype, (unsigned char*)workspace + (size_t)k * stride, lay.total, hip_stream, op_flags);
         if (rc != RTN_OK) return rc;
       }
       return RTN_OK;
@@ -1357,7 +1361,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     memset(&p, 0, sizeof(p));
     p.W = c.W; p.c0 = c.c0; p.mask = c.i; p.C = c.C; p.H = c.H; p.DY = c.DY;
     p.DX = c.DX; p.Dc0 = c.Dc0;
-    j.ws = (unsigned char*)workspace + (size_t)k * lay.total;
+    j.ws = (unsigned char*)workspace + (size_t)k * stride;
     p.dyw = (float*)(j.ws + lay.off_dyw);
     p.dx0 = j.ws + lay.off_dx0;
     p.T = T; p.B = B; p.n = n;

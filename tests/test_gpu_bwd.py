@@ -128,7 +128,7 @@ def test_bwd_edge_cases_and_errors():
     assert cabi.rtn_native_lstm2_bwd_workspace_bytes(-1, B, n, 0) == 0
 
 
-@pytest.mark.parametrize("T,B,n,dtype", [(14, 32, 256, "bf16"), (9, 20, 64, "f32"), (20, 32, 1024, "bf16"), (6, 5, 20, "f32"), (7, 70, 128, "bf16")])
+@pytest.mark.parametrize("T,B,n,dtype", [(14, 32, 256, "bf16"), (9, 20, 64, "f32"), (20, 32, 1024, "bf16"), (6, 5, 20, "f32"), (7, 70, 128, "bf16"), (6, 9, 100, "f32"), (5, 12, 200, "bf16")])
 def test_bwd_multi_equals_single_calls(T, B, n, dtype):
     """
     The two directions of a layer through ``rtn_native_lstm2_bwd_multi``: against the oracle to the same bar as a single
