@@ -1434,7 +1434,10 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     const Lstm2BwdParams& p = j.p;
     const int step = calls[0].step;
     const long long first = j.first, end = j.end;
-    const int NT = B > 32 ? 2 : 1;  // up to 32 rows: more, smaller workgroups
+    // Batch rows per workgroup (16 * NT): 32 if that still leaves every CU a workgroup (each batch tile reads W again),
+    // else 16 (measured: float32 n=1024 B=64 29 us per frame with 16 rows, 35 with 32; 64 rows were never faster).
+    int NT = B > 16 ? 2 : 1;
+    if (NT > 1 && (long long)(n / 16) * ((B + 16 * NT - 1) / (16 * NT)) < device_info().cus) NT = 1;
     auto record = [&](hipStream_t st) -> int {
       const dim3 pw_grid((unsigned)((bn + 255) / 256)), pw_block(256);
       const dim3 mm_grid((unsigned)((n / 16) * ((B + 16 * NT - 1) / (16 * NT)))), mm_block(kWgThreads);
@@ -1479,7 +1482,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       RTN_HIP(hipGetDevice(&dev));
       key.append(reinterpret_cast<const char*>(&p), sizeof(p));  // p was zeroed before it was filled in
       key_append(&key, dtype); key_append(&key, (int)calls[0].start); key_append(&key, step); key_append(&key, dev);
-      key_append(&key, (int)mfma);
+      key_append(&key, (int)mfma); key_append(&key, NT);
       rc = replay_graph(key, stream, record);
     }
     if (rc != RTN_OK) return rc;
