@@ -621,7 +621,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "wide"])
     ap.add_argument("--mode", default="auto", choices=["auto", "persistent", "graph", "stepwise"])
     ap.add_argument("--pair", default="fused", choices=["fused", "separate"],
                     help="cfg3: issue the two directions through the multi-call entry (one launch when the device "
@@ -829,6 +829,23 @@ def main():
             "hbm_frac": bytes_per_launch / (call_ms * 1e-3) / PEAK_HBM,
         },
     }
+    if "mode=persistent" not in plan and "kernel=mfma_lds" in plan:
+        # Per-step launches: W is read from memory once per step and used once, so memory bandwidth bounds the call.
+        e = 2 if dtype == "bf16" else 4
+        steps_bytes = T * (4 * n * n * e) + bytes_per_launch  # W every step + the op's own streams
+        result["roofline"].update({
+            "bound": "hbm",
+            "achieved": steps_bytes / (call_ms * 1e-3) / 1e9,
+            "peak": PEAK_HBM / 1e9,
+            "unit": "GB/s",
+            "frac": steps_bytes / (call_ms * 1e-3) / PEAK_HBM,
+            "traffic": None,
+            "traffic_unit": "bytes per op call; algorithmic: %i (W once per step + X, H, Y, C, mask)" % steps_bytes,
+            "kernel": "k_lstm2_mfma, one launch per step replayed through a graph (one op call = %i launches)" % T,
+            "mfma_TFLOPs": achieved / 1e12,
+        })
+        for key in ("achievable", "achievable_unit", "frac_of_achievable", "mfma_peak_us_per_step"):
+            result["roofline"].pop(key, None)  # they describe the exchange-bound persistent kernel
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, args.cpu_seconds)
     print(json.dumps(result))

@@ -53,6 +53,8 @@ _SPECS = {
     "cfg2": dict(T=500, B=64, n=512, dtype="f32", lens=(250, 500), w_lim=1.0 / math.sqrt(512.0), state_std=0.01),
     "cfg3": dict(T=1000, B=32, n=1024, dtype="bf16", lens=(500, 1000), w_lim=1.0 / 32.0, state_std=0.0),
     "cfg5": dict(T=4000, B=1, n=1024, dtype="bf16", lens=None, w_lim=1.0 / 32.0, state_std=0.0),
+    # not one of the benchmark configurations: a layer whose W (134 MB) cannot stay on chip, read from memory every step
+    "wide": dict(T=200, B=16, n=4096, dtype="bf16", lens=None, w_lim=1.0 / 64.0, state_std=0.0),
 }
 
 
@@ -64,7 +66,7 @@ def make_config(name: str, *, seed: int = 0, T: Optional[int] = None, B: Optiona
     """
     :param name: "cfg1" (T=32,B=4,n=64 fp32), "cfg2" (T=500,B=64,n=512 fp32 ragged),
         "cfg3" (T=1000,B=32,n=1024 bf16 ragged; the bidirectional pair is this with step=+1 and step=-1),
-        "cfg5" (T=4000,B=1,n=1024 bf16)
+        "cfg5" (T=4000,B=1,n=1024 bf16), "wide" (T=200,B=16,n=4096 bf16: W does not fit on chip)
     :param T: override the number of frames (scaled-down variants for quick checks; lengths scale with it)
     :param B: override the batch size
     :param step: +1 or -1
