@@ -23,7 +23,26 @@ struct Lstm2BwdParams {
   int B, n;
   int op_flags;  // OpFlags: kOpNoCarry, kOpH0IsCell select the gradient of LstmGenericBase (returnn/native_op.py:430-485)
   int pad_;
+  const void* Wpk;  // per-frame launches: W in MFMA A-operand order, [n/16][4n/KM][64] fragments of 16 bytes (else null)
 };
+
+// W[n,4n] -> fragments in the order the per-frame kernel reads them: tile kt (16 rows of W), macro step s (KM columns),
+// lane l holds row 16*kt + l%16, columns KM*s + KE*(l/16) .. +KE.  A wavefront's load of one fragment set is then 1 KB of
+// consecutive memory instead of sixteen 64-byte pieces of sixteen rows, which is what lets a launch that uses W once
+// read it at memory speed.
+template <typename AT>
+__global__ void k_bwd_pack_w(const void* __restrict__ W, void* __restrict__ Wpk, int n) {
+  constexpr int KE = Elem<AT>::KE, KM = Elem<AT>::KM;
+  const int n4 = 4 * n, S = n4 / KM;
+  const long long total = (long long)(n / 16) * S * 64;
+  for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
+    const int l = (int)(i & 63);
+    const long long ts = i >> 6;
+    const int s = (int)(ts % S);
+    const long long kt = ts / S;
+    ((i32x4*)Wpk)[i] = *(const i32x4*)((const AT*)W + (size_t)(16 * kt + (l & 15)) * n4 + (size_t)KM * s + KE * (l >> 4));
+  }
+}
 
 // Gate derivatives of one (sequence, cell) pair in one frame (returnn/native_op.py:1148-1172).
 //   h0: first block of H -- tanh(cell-in), or with kOpH0IsCell the cell state, from which tanh(cell-in) is recovered as
@@ -110,6 +129,7 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
   if (t_gemm >= 0) {
     const int S = n4 / KM;
     const AT* Wr = (const AT*)p.W + (size_t)(k0 + (lane & 15)) * n4 + KE * (lane >> 4);
+    const i32x4* Wk = p.Wpk ? (const i32x4*)p.Wpk + (size_t)(k0 / 16) * S * 64 + lane : nullptr;  // packed: fragment s at Wk[64 * s]
     const AT* Dx = (const AT*)p.DX + (size_t)t_gemm * p.B * n4 + KE * (lane >> 4);
     int brow[NT];
 #pragma unroll
@@ -125,7 +145,7 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int s = min(s0 + kWaves * u, S - 1);  // past the end: a valid address, the product is dropped
-        a[u] = *(const i32x4*)(Wr + (size_t)KM * s);
+        a[u] = Wk ? Wk[(size_t)64 * s] : *(const i32x4*)(Wr + (size_t)KM * s);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) bfrag[u][nt] = *(const i32x4*)(Dx + (size_t)brow[nt] * n4 + (size_t)KM * s);
       }

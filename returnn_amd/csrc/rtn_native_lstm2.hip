@@ -918,7 +918,7 @@ int dw_accumulate(rocblas_handle h, const void* A, const void* Bm, float* DW, lo
 }
 
 struct BwdLayout {
-  size_t off_dyw = 0, off_dx0 = 0, total = 0;
+  size_t off_dyw = 0, off_dx0 = 0, off_wpk = 0, total = 0;  // [0, off_wpk) is cleared at the start of a call
 };
 BwdLayout bwd_layout(int B, int n, int dtype) {
   BwdLayout l;
@@ -927,6 +927,8 @@ BwdLayout bwd_layout(int B, int n, int dtype) {
   off = align_up(off + (size_t)B * n * 4, 256);
   l.off_dx0 = off;
   off = align_up(off + (size_t)B * 4 * n * esize(dtype), 256);
+  l.off_wpk = off;  // W in fragment order, for per-frame launches
+  if (n % 16 == 0) off = align_up(off + (size_t)4 * n * n * esize(dtype), 256);
   l.total = off;
   return l;
 }
@@ -1366,7 +1368,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     p.dx0 = j.ws + lay.off_dx0;
     p.T = T; p.B = B; p.n = n;
     p.op_flags = op_flags;
-    hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)j.ws, 0u, (long long)(lay.total / 4));
+    hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)j.ws, 0u, (long long)(lay.off_wpk / 4));
     RTN_HIP(hipGetLastError());
     // returnn/native_op.py:1383-1407: which frames are visited, and in which order
     j.abs_step = c.step > 0 ? c.step : -(long long)c.step;
@@ -1430,7 +1432,18 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     // count == 1 here.  The launches of all frames, in reverse processing order.  MFMA shapes: one fused launch per
     // frame (the GEMM of the frame processed before, then this frame's pointwise part) and a last GEMM-only launch;
     // other shapes: a pointwise and a generic GEMM launch per frame.
-    const BwdJob& j = jobs[0];
+    BwdJob& j = jobs[0];
+    if (mfma && env_long("RTN_LSTM2_BWD_PACK_W", 1)) {
+      // every launch uses each fragment of W once: read them from a copy in fragment order (see k_bwd_pack_w)
+      j.p.Wpk = j.ws + lay.off_wpk;
+      const long long frags = (long long)(n / 16) * (4 * n / (dtype == RTN_DTYPE_BF16 ? 32 : 16)) * 64;
+      const dim3 pgrid((unsigned)std::min<long long>((frags + 255) / 256, 4096)), pblock(256);
+      if (dtype == RTN_DTYPE_BF16)
+        hipLaunchKernelGGL(k_bwd_pack_w<__bf16>, pgrid, pblock, 0, stream, calls[0].W, (void*)j.p.Wpk, n);
+      else
+        hipLaunchKernelGGL(k_bwd_pack_w<float>, pgrid, pblock, 0, stream, calls[0].W, (void*)j.p.Wpk, n);
+      RTN_HIP(hipGetLastError());
+    }
     const Lstm2BwdParams& p = j.p;
     const int step = calls[0].step;
     const long long first = j.first, end = j.end;
