@@ -178,3 +178,49 @@ def test_bwd_multi_errors_and_empty():
         a = (z(8, 32), z(2, 8), z(2, 8), z(3, 2), 0, 1, z(3, 2, 8), z(3, 2, 8), z(3, 2, 32), z(3, 2, 8), z(2, 8))
         b = (z(8, 32), z(2, 8), z(2, 8), z(4, 2), 0, 1, z(4, 2, 8), z(4, 2, 8), z(4, 2, 32), z(4, 2, 8), z(2, 8))
         torch_native_op.native_lstm2_grad_multi([a, b])
+
+
+@pytest.mark.parametrize("T,B,n,dtype", [(40, 16, 256, "bf16"), (12, 9, 1024, "f32"), (10, 40, 128, "f32")])
+def test_bwd_bounded_wait_expires_cleanly(T, B, n, dtype):
+    """A wait bound of zero ticks forced from the host: the persistent gradient kernel (the ordinary variant, the one
+    with half of W in LDS, and a batch in several groups) must still drain; the status call then reports success
+    (nobody had to wait) or the abort, and the next ordinary call on the same workspace is unaffected."""
+    from _gpu_util import env
+
+    announce("bwd bounded wait", T, B, n, dtype)
+    X, W, y0, c0, i = random_problem(77 + n, T, B, n)
+    rng = numpy.random.default_rng(78)
+    DY = rng.normal(0, 1.0, (T, B, n)).astype(numpy.float32)
+    Dd = rng.normal(0, 1.0, (B, n)).astype(numpy.float32)
+    op = get_op()
+    Xd, Wd, y0d, DYd = (to_dev(a, dtype) for a in (X, W, y0, DY))
+    c0d, id_, Ddd = (to_dev(a, "f32") for a in (c0, i, Dd))
+    Y, C, H, d = op(Xd, Wd, y0d, c0d, id_, 0, 1)
+    cabi = lib.load()
+    dt = lib.DTYPE_BF16 if dtype == "bf16" else lib.DTYPE_F32
+    act = torch.bfloat16 if dtype == "bf16" else torch.float32
+    DX = torch.empty((T, B, 4 * n), dtype=act, device="cuda:0")
+    DW = torch.empty((n, 4 * n), dtype=torch.float32, device="cuda:0")
+    Dy0 = torch.empty((B, n), dtype=act, device="cuda:0")
+    Dc0 = torch.empty((B, n), dtype=torch.float32, device="cuda:0")
+    ws = torch.empty((max(int(cabi.rtn_native_lstm2_bwd_workspace_bytes(T, B, n, dt)), 256),), dtype=torch.uint8, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def call():
+        return cabi.rtn_native_lstm2_bwd(
+            Wd.data_ptr(), y0d.data_ptr(), c0d.data_ptr(), id_.data_ptr(), 0, 1, Y.data_ptr(), C.data_ptr(), H.data_ptr(),
+            DYd.data_ptr(), Ddd.data_ptr(), DX.data_ptr(), DW.data_ptr(), Dy0.data_ptr(), Dc0.data_ptr(), T, B, n, dt,
+            ws.data_ptr(), ws.numel(), stream,
+        )  # fmt: skip
+
+    with env(RTN_LSTM2_TIMEOUT_TICKS=0, RTN_LSTM2_BWD_KERNEL=2):
+        assert call() == 0
+    status = cabi.rtn_native_lstm2_fwd_status(ws.data_ptr(), stream)
+    assert status in (lib.RTN_OK, lib.RTN_ERR_ABORTED)
+    assert call() == 0
+    assert cabi.rtn_native_lstm2_fwd_status(ws.data_ptr(), stream) == lib.RTN_OK
+    torch.cuda.synchronize()
+    f = lambda t: t.float().cpu().numpy().astype(numpy.float64)  # noqa: E731
+    want = oracle.native_lstm2_bwd(f(Xd), f(Wd), f(y0d), c0, i, 0, 1, f(Y), f(C), f(H), f(DYd), Dd, dtype=numpy.float64)
+    for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), (DX, DW, Dy0, Dc0), want):
+        assert _rel_to_max(f(a), b) <= (2e-5 if dtype == "f32" else 2e-2), name
