@@ -479,3 +479,43 @@ def test_widths_that_run_zero_padded(T, B, n, dtype, start, step):
         assert tuple(a.shape) == b.shape, name
         rel = float(numpy.abs(f(a) - b).max() / max(numpy.abs(b).max(), 1e-30))
         assert rel <= (2e-5 if dtype == "f32" else 2e-2), (name, rel)
+
+
+@pytest.mark.parametrize("T,B,n,dtype", [(12, 8, 128, "bf16"), (9, 5, 100, "f32"), (7, 3, 20, "f32")])
+def test_forward_recorded_into_a_callers_graph(T, B, n, dtype):
+    """Under stream capture the op records one launch per step into the caller's graph (a cooperative launch cannot be
+    recorded).  The graph is replayed three times, with new inputs and the program's own eager work in between; every
+    replay must equal the eager result bit for bit."""
+    from _gpu_util import to_dev
+
+    announce("captured", T, B, n, dtype)
+    from returnn_amd import torch_native_op
+
+    op = get_op()
+    torch_native_op.OpMaker.options["NativeLstm2"]["mode"] = "auto"
+    problems = [random_problem(990 + k, T, B, n) for k in range(3)]
+    X, W, y0, c0, i = problems[0]
+    Xd, Wd, y0d = (to_dev(a, dtype) for a in (X, W, y0))
+    c0d, id_ = (to_dev(a, "f32") for a in (c0, i))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        op(Xd, Wd, y0d, c0d, id_, 0, 1)  # warm-up outside the capture (module load, attribute calls)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        outs = op(Xd, Wd, y0d, c0d, id_, 0, 1)
+    for k in range(3):
+        Xk, Wk, y0k, c0k, ik = problems[k]
+        Xd.copy_(to_dev(Xk, dtype)); Wd.copy_(to_dev(Wk, dtype)); y0d.copy_(to_dev(y0k, dtype))  # noqa: E702
+        c0d.copy_(to_dev(c0k, "f32")); id_.copy_(to_dev(ik, "f32"))  # noqa: E702
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs]
+        eager = op(Xd, Wd, y0d, c0d, id_, 0, 1)  # eager work between the replays (the persistent kernel)
+        torch.cuda.synchronize()
+        for name, a, b in zip("YCHd", got, eager):
+            assert torch.equal(a, b), (k, name)
+        want = oracle.native_lstm2_fwd(*problems[k], 0, 1)
+        (check_f32 if dtype == "f32" else check_bf16)([t.float().cpu().numpy() for t in got], want[:4], "captured replay %i" % k)
