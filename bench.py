@@ -471,7 +471,11 @@ def bench_gradient(args, dev, cabi):
             "peak": peak / 1e12,
             "unit": "TFLOP/s",
             "frac": flops / (call_ms * 1e-3) / peak,
-            "traffic": None,
+            # k_lstm2_bwd_regw of the cfg3 pair in one entry, rocprofv3 FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
+            # (profiles/k_lstm2_bwd_regw_cfg3_pair_hbm_traffic.txt); algorithmic: 22 532 B per unit
+            "traffic": 6326.2e6 if (args.workload == "cfg3" and fused and len(steps_of) == 2) else None,
+            "traffic_unit": "bytes per launch of the persistent kernel; algorithmic (read H, DY, C, mask; write DX): %i"
+            % (((9 * (2 if dtype == "bf16" else 4) + 4) * n + 4) * units),
             "kernel": "whole gradient call: the persistent k_lstm2_bwd_regw (or one k_bwd_step launch per frame) with the "
             "recurrent GEMM, 8*n^2 flops per unit, then the weight-gradient GEMM in rocBLAS, 8*n^2 flops per unit",
             "launch_ms": call_ms,
