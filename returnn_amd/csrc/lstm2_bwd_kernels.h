@@ -336,9 +336,12 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       for (int ks = KSB; ks < KST; ++ks) wl[(ks - KSB) * 64] = (ks < ks_here) ? *(const i32x4*)(Wr + (size_t)KM * ks) : i32x4{0, 0, 0, 0};
     }
   }
-  // byte offset of this lane's first B fragment inside a frame of DX; the others follow at KM*ES bytes each
-  const unsigned foff0 = (unsigned)(((size_t)(b_base + (((lane & 15) < rows) ? (lane & 15) : 0)) * n4  // rows the group lacks: row 0
-                                     + (size_t)KM * ksb * wave_at + KE * (lane >> 4)) * ES);
+  // byte offset of this lane's first B fragment inside a frame of DX; the others follow at KM*ES bytes each.  The lanes
+  // of rows the group lacks (half of them with 8-row groups) carry an out-of-range offset: their loads return 0 and
+  // take nothing through the CU's memory pipeline, which moves only 64 bytes per clock.
+  const unsigned foff0 = ((lane & 15) < rows)
+                             ? (unsigned)(((size_t)(b_base + (lane & 15)) * n4 + (size_t)KM * ksb * wave_at + KE * (lane >> 4)) * ES)
+                             : 0x80000000u;
 
   // The (row, k) pairs of this thread: one in each of its tiles.
   const int set = (TS == 1) ? 0 : __builtin_amdgcn_readfirstlane(tid >> 8);  // uniform over a wavefront
