@@ -83,6 +83,25 @@ def test_workspace_and_plan(cabi):
         assert lib.workspace_bytes(T, B, n, dt, lib.MODE_AUTO) >= lib.workspace_bytes(T, B, n, dt, lib.MODE_STEPWISE)
 
 
+def test_plan_of_large_batches_padded_widths_and_wide_layers(cabi):
+    # a batch too large for one persistent launch: several in turn, each on a share of the batch groups
+    text = lib.describe_plan(100, 256, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
+    assert "mode=persistent" in text and "kernel=mfma_regw" in text and "launches=2 " in text, text
+    assert "launches=1 " in lib.describe_plan(100, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
+    # a width that is not a multiple of 32 runs zero-padded; the workspace holds the padded copies
+    text = lib.describe_plan(100, 32, 1000, lib.DTYPE_BF16, lib.MODE_AUTO)
+    assert "kernel=mfma_regw" in text and "padded_width=1024" in text, text
+    exact = lib.workspace_bytes(100, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
+    padded = lib.workspace_bytes(100, 32, 1000, lib.DTYPE_BF16, lib.MODE_AUTO)
+    copies = 100 * 32 * 1024 * (4 * 2 + 4 * 2 + 2 + 4)  # X, H, Y, C at the padded width
+    assert padded >= exact + copies
+    assert cabi.rtn_native_lstm2_bwd_workspace_bytes(100, 32, 1000, lib.DTYPE_BF16) > cabi.rtn_native_lstm2_bwd_workspace_bytes(100, 32, 1024, lib.DTYPE_BF16)
+    assert "padded_width" not in lib.describe_plan(100, 32, 20, lib.DTYPE_F32, lib.MODE_AUTO)  # tiny layers stay as they are
+    # W does not fit on chip: one launch per step, a few KB of LDS (W goes from memory straight to the matrix cores)
+    text = lib.describe_plan(100, 16, 4096, lib.DTYPE_BF16, lib.MODE_AUTO)
+    assert "mode=graph" in text and "kernel=mfma_lds" in text and "lds=4096 " in text, text
+
+
 def test_op_description_contract():
     """Names, order, ndim and host-memory flags of returnn/native_op.py:1054-1068."""
     from returnn_amd import native_op
