@@ -167,8 +167,10 @@ int rtn_handover_latency_probe(void* workspace, size_t workspace_bytes, int32_t 
  * cooperative kernel runs all frames: W stays in registers, DX doubles as the self-validating exchange medium between
  * workgroups.  Otherwise one launch per visited frame (the MFMA GEMM Dy0 += DX[t'] W^T of the frame processed before,
  * fused with the frame's pointwise part), replayed through a library-owned hipGraph.  The large weight-gradient GEMM
- * (Y^T DX over all frames) is left to rocBLAS, which may allocate its own device workspace on first use; the call
- * cannot be recorded into a caller's graph.  `workspace`: rtn_native_lstm2_bwd_workspace_bytes();
+ * (Y^T DX over all frames) is left to rocBLAS, which may allocate its own device workspace on first use.  Under stream
+ * capture the per-frame launches and the rocBLAS calls are recorded into the caller's graph (the counterpart of the
+ * reference's whole-step graph capture, returnn/torch/util/graph_capture.py); the library's rocBLAS handle has to exist
+ * by then: run the entry once outside the capture first.  `workspace`: rtn_native_lstm2_bwd_workspace_bytes();
  * rtn_native_lstm2_fwd_status(workspace, stream) reports an expired bounded wait of the persistent kernel.
  */
 int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const float* i, int32_t start, int32_t step,
@@ -228,7 +230,7 @@ size_t rtn_native_lstm2_bwd_multi_workspace_bytes(int32_t count, int64_t T, int3
  *   a negative step the loop runs from frame T-start-1 down to frame `start`, not down to frame 0.  Where that visits no
  *   frame (2*start > T-1) the reference returns an unwritten d; here the call is refused with RTN_ERR_RANGE.  Frames the
  *   loop does not visit are zero in Y and C (unwritten in the reference).  The input projection X.W[:n_in] + b is one rocBLAS GEMM over all frames into the
- *   workspace (so the call cannot be recorded into a graph and, unlike the reference, needs T*B*8n elements of scratch:
+ *   workspace (under stream capture it is recorded like the launches, after one call outside the capture; unlike the reference, the call needs T*B*8n elements of scratch:
  *   the low memory footprint of the reference's variant is not reproduced, only its results).
  */
 int rtn_lstm_generic_base_fwd(const void* Z, const void* V_h, const float* c, const float* i, void* Y, void* H, float* d,

@@ -1086,8 +1086,7 @@ int rtn_lstm_low_mem_fwd(const void* X, const void* W, const void* b, const void
   hipStream_t stream = (hipStream_t)hip_stream;
   hipStreamCaptureStatus cap_status = hipStreamCaptureStatusNone;
   if (stream) RTN_HIP(hipStreamIsCapturing(stream, &cap_status));
-  if (cap_status != hipStreamCaptureStatusNone)
-    return fail(RTN_ERR_UNSUPPORTED, "LstmLowMem: cannot be recorded into a graph (the input projection calls rocBLAS)");
+  (void)cap_status;  // under capture the rocBLAS projection is recorded like the launches (the handle must exist already)
   const size_t need = rtn_lstm_low_mem_fwd_workspace_bytes(T, B, n_in, n, dtype, mode);
   if (!workspace || workspace_bytes < need)
     return fail(RTN_ERR_WORKSPACE, "LstmLowMem: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
@@ -1163,8 +1162,10 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
   const long long nn4 = (long long)n * n * 4;
   hipStreamCaptureStatus cap_status = hipStreamCaptureStatusNone;
   if (stream) RTN_HIP(hipStreamIsCapturing(stream, &cap_status));
-  if (cap_status != hipStreamCaptureStatusNone)
-    return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2 backward: cannot be recorded into a graph (it calls rocBLAS)");
+  // Under stream capture everything is recorded into the caller's graph: one launch per frame (a cooperative launch
+  // cannot be recorded) and the rocBLAS calls of the weight gradient (the library's rocBLAS handle must exist already:
+  // run the op once outside the capture first, as for any library that sets itself up on first use).
+  const bool capturing = cap_status != hipStreamCaptureStatusNone;
   const dim3 fill_grid(256), fill_block(256);
   for (int k = 0; k < count; ++k) {
     const rtn_lstm2_bwd_call& c = calls[k];
@@ -1276,7 +1277,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
     const int S = 4 * n / KM;
     const long bwd_kernel = env_long("RTN_LSTM2_BWD_KERNEL", 0);  // 0 auto, 1 per-frame launches, 2 persistent
-    if (mfma && (4 * n) % KM == 0 && bwd_kernel != 1 && device_info().cooperative && count <= kMaxBwdMulti) {
+    if (mfma && (4 * n) % KM == 0 && bwd_kernel != 1 && !capturing && device_info().cooperative && count <= kMaxBwdMulti) {
       const long env_mt = env_long("RTN_LSTM2_BWD_MT", 0);
       const long env_waves = env_long("RTN_LSTM2_BWD_WAVES", 0);
       // (rows per group, tiles per workgroup, wavefronts per workgroup)
@@ -1487,7 +1488,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       RTN_HIP(hipGetLastError());
       return RTN_OK;
     };
-    if (env_long("RTN_LSTM2_BWD_NO_GRAPH", 0)) {
+    if (capturing || env_long("RTN_LSTM2_BWD_NO_GRAPH", 0)) {
       rc = record(stream);
     } else {
       std::string key("bwd");

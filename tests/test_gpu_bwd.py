@@ -224,3 +224,54 @@ def test_bwd_bounded_wait_expires_cleanly(T, B, n, dtype):
     want = oracle.native_lstm2_bwd(f(Xd), f(Wd), f(y0d), c0, i, 0, 1, f(Y), f(C), f(H), f(DYd), Dd, dtype=numpy.float64)
     for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), (DX, DW, Dy0, Dc0), want):
         assert _rel_to_max(f(a), b) <= (2e-5 if dtype == "f32" else 2e-2), name
+
+
+@pytest.mark.parametrize("T,B,n,dtype", [(10, 8, 128, "bf16"), (8, 5, 100, "f32"), (6, 3, 20, "f32")])
+def test_forward_and_gradient_recorded_into_a_callers_graph(T, B, n, dtype):
+    """A training step under stream capture: forward op and gradient op (one launch per frame plus the rocBLAS weight
+    gradient) are recorded into the caller's graph after one eager run (which creates the library's rocBLAS handle).
+    The graph is replayed three times with new inputs and eager work in between; every replay must agree with the
+    eager gradient op (another decomposition: equal up to rounding) and with the oracle."""
+    announce("captured training step", T, B, n, dtype)
+    op = get_op()
+    torch_native_op.OpMaker.options["NativeLstm2"]["mode"] = "auto"
+    rng = numpy.random.default_rng(5)
+    problems = [random_problem(1200 + k, T, B, n) for k in range(3)]
+    grads_in = [(rng.normal(0, 1.0, (T, B, n)).astype(numpy.float32), rng.normal(0, 1.0, (B, n)).astype(numpy.float32)) for _ in range(3)]
+    X, W, y0, c0, i = problems[0]
+    Xd, Wd, y0d, DYd = (to_dev(a, dtype) for a in (X, W, y0, grads_in[0][0]))
+    c0d, id_, Ddd = (to_dev(a, "f32") for a in (c0, i, grads_in[0][1]))
+
+    def step():
+        Y, C, H, d = op(Xd, Wd, y0d, c0d, id_, 0, 1)
+        return (Y, C, H, d), torch_native_op.native_lstm2_grad(Wd, y0d, c0d, id_, 0, 1, Y, C, H, DYd, Ddd)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()  # eager warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        fwd_out, grad_out = step()
+    f = lambda t: t.float().cpu().numpy().astype(numpy.float64)  # noqa: E731
+    tol = 2e-5 if dtype == "f32" else 2e-2
+    for k in range(3):
+        Xk, Wk, y0k, c0k, ik = problems[k]
+        for dst, src, dt in ((Xd, Xk, dtype), (Wd, Wk, dtype), (y0d, y0k, dtype), (DYd, grads_in[k][0], dtype), (c0d, c0k, "f32"),
+                             (id_, ik, "f32"), (Ddd, grads_in[k][1], "f32")):  # fmt: skip
+            dst.copy_(to_dev(src, dt))
+        graph.replay()
+        torch.cuda.synchronize()
+        got_f = [t.clone() for t in fwd_out]
+        got_g = [t.clone() for t in grad_out]
+        eager_f, eager_g = step()
+        torch.cuda.synchronize()
+        for name, a, b in zip("YCHd", got_f, eager_f):
+            assert torch.equal(a, b), (k, name)
+        for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), got_g, eager_g):
+            assert _rel_to_max(f(a), f(b)) <= tol, (k, name, "against the eager op")
+        want = oracle.native_lstm2_bwd(f(Xd), f(Wd), f(y0d), c0k, ik, 0, 1, f(got_f[0]), f(got_f[1]), f(got_f[2]), f(DYd), grads_in[k][1], dtype=numpy.float64)
+        for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), got_g, want):
+            assert _rel_to_max(f(a), b) <= tol, (k, name, "against the oracle")

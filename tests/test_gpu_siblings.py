@@ -291,3 +291,61 @@ def test_generic_base_gradient_through_autograd():
     torch.cuda.synchronize()
     for name, leaf, r in zip(("Z", "V_h", "c"), leaves, ref):
         assert _rel_to_max(leaf.grad.cpu().numpy().astype(numpy.float64), r.grad.numpy()) <= 2e-5, name
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_sibling_ops_recorded_into_a_callers_graph(dtype):
+    """LstmLowMem (whose input projection is a rocBLAS GEMM) and LstmGenericBase with its gradient under stream capture,
+    after one eager run: recorded into the caller's graph, replayed twice with new inputs, equal to the eager results
+    (bit for bit in the forward pass, up to rounding in the gradient, which takes another decomposition)."""
+    announce("siblings captured", dtype)
+    get_op()
+    T, B, n_in, n = 9, 6, 24, 64
+    for m in ("LstmLowMem", "LstmGenericBase"):
+        torch_native_op.OpMaker.options.setdefault(m, {})["mode"] = "auto"
+    lm = torch_native_op.make_op(native_op.LstmLowMem)
+    gb = torch_native_op.make_op(native_op.LstmGenericBase)
+    lm_problems = [low_mem_problem(700 + k, T, B, n_in, n) for k in range(2)]
+    gb_problems = [generic_base_problem(710 + k, T, B, n) for k in range(2)]
+    rng = numpy.random.default_rng(3)
+    DYs = [rng.normal(0, 1, (T, B, n)).astype(numpy.float32) for _ in range(2)]
+    Dds = [rng.normal(0, 1, (B, n)).astype(numpy.float32) for _ in range(2)]
+    X, W, b, y0, c0, i = lm_problems[0]
+    lm_in = [to_dev(X, dtype), to_dev(W, dtype), to_dev(b, dtype), to_dev(y0, dtype), to_dev(c0, "f32"), to_dev(i, "f32")]
+    Z, V, c, ig = gb_problems[0]
+    gb_in = [to_dev(Z, dtype), to_dev(V, dtype), to_dev(c, "f32"), to_dev(ig, "f32")]
+    DYd, Ddd = to_dev(DYs[0], dtype), to_dev(Dds[0], "f32")
+
+    def step():
+        lm_out = lm(*lm_in, 0, 1)
+        Y, H, d = gb(*gb_in)
+        grads = torch_native_op.lstm_generic_base_grad(gb_in[1], gb_in[2], gb_in[3], Y, H, DYd, Ddd)
+        return list(lm_out) + [Y, H, d], list(grads)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        fwd_out, grad_out = step()
+    for k in range(2):
+        for dst, src in zip(lm_in, lm_problems[k]):
+            dst.copy_(to_dev(src, "f32" if dst.dtype == torch.float32 else dtype))
+        for dst, src in zip(gb_in, gb_problems[k]):
+            dst.copy_(to_dev(src, "f32" if dst.dtype == torch.float32 else dtype))
+        DYd.copy_(to_dev(DYs[k], dtype))
+        Ddd.copy_(to_dev(Dds[k], "f32"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got_f = [t.clone() for t in fwd_out]
+        got_g = [t.clone() for t in grad_out]
+        eager_f, eager_g = step()
+        torch.cuda.synchronize()
+        for idx, (a, e) in enumerate(zip(got_f, eager_f)):
+            assert torch.equal(a, e), (k, "forward output", idx)
+        for idx, (a, e) in enumerate(zip(got_g, eager_g)):
+            scale = max(float(e.float().abs().max()), 1e-30)
+            assert float((a.float() - e.float()).abs().max()) / scale <= (2e-5 if dtype == "f32" else 2e-2), (k, "gradient", idx)
