@@ -297,3 +297,48 @@ def test_lstm_module_trains_one_step():
         opt.step()
         losses.append(float(loss.detach()))
     assert all(numpy.isfinite(losses)) and losses[-1] < losses[0], losses
+
+
+def test_lstm_module_training_step_recorded_into_a_graph():
+    """Forward, loss and backward of the module under stream capture (the reference engine captures whole training steps,
+    returnn/torch/util/graph_capture.py): after eager warm-up steps the graph is replayed with new inputs and must give
+    the parameter and input gradients of the eager step (the recorded gradient op takes another decomposition than the
+    eager one: equal up to bfloat16 rounding)."""
+    announce("lstm module captured training step")
+    get_op()
+    torch.manual_seed(1)
+    T, B, d_in, n = 14, 8, 16, 64
+    mod = rlstm.LSTM(d_in, n, device=DEV, dtype=torch.bfloat16)
+    x = torch.randn(T, B, d_in, device=DEV).bfloat16().requires_grad_(True)
+    target = torch.randn(T, B, n, device=DEV) * 0.1
+    lens = torch.tensor([14, 14, 9, 5, 14, 2, 11, 14], device=DEV)
+    s0 = mod.default_initial_state(batch_dims=(B,))
+    params = list(mod.parameters())
+
+    def step():
+        y, _ = mod(x, state=s0, seq_lens=lens)
+        loss = ((y.float() - target) ** 2).mean()
+        return torch.autograd.grad(loss, [x] + params)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        recorded = step()
+    for k in range(3):
+        with torch.no_grad():
+            x.copy_(torch.randn(T, B, d_in, device=DEV).bfloat16())
+            target.copy_(torch.randn(T, B, n, device=DEV) * 0.1)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [g.clone() for g in recorded]
+        eager = step()
+        torch.cuda.synchronize()
+        for idx, (a, e) in enumerate(zip(got, eager)):
+            scale = max(float(e.float().abs().max()), 1e-30)
+            assert float((a.float() - e.float()).abs().max()) / scale <= 2e-2, (k, idx)
