@@ -126,6 +126,34 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
   const int ktiles = n / 16;
   const int k0 = ((int)blockIdx.x % ktiles) * 16;
   const int b0 = ((int)blockIdx.x / ktiles) * 16 * NT;
+  // The operands of the pointwise part of the thread's (b, k) pairs do not depend on the GEMM: they are fetched first,
+  // so that their latency passes behind it.
+  const int pbl = tid >> 4, pkl = tid & 15;
+  float q_dyw[NT], q_m[NT], q_dy[NT], q_dc[NT], q_pc[NT], q_h[NT][4], q_dx0[NT][4];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int b = b0 + 16 * nt + pbl, k = k0 + pkl;
+    q_dyw[nt] = q_m[nt] = q_dy[nt] = q_dc[nt] = q_pc[nt] = 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) q_h[nt][g] = q_dx0[nt][g] = 0.f;
+    if (b >= p.B) continue;
+    const long long idx = (long long)b * n + k;
+    q_dyw[nt] = p.dyw[idx];
+    if (t >= 0) {
+      const long long bn = (long long)p.B * n;
+      const long long io = (long long)b * n4 + k;
+      const long long fo = t * bn * 4 + io;
+      q_m[nt] = p.mask[t * p.B + b];
+      q_dy[nt] = E::load(p.DY, t * bn + idx);
+      q_dc[nt] = p.Dc0[idx];
+      q_pc[nt] = bwd_prev_cell<AT>(p, prev_t, idx, io);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        q_h[nt][g] = E::load(p.H, fo + g * n);
+        q_dx0[nt][g] = E::load(p.dx0, io + g * n);
+      }
+    }
+  }
   if (t_gemm >= 0) {
     const int S = n4 / KM;
     const AT* Wr = (const AT*)p.W + (size_t)(k0 + (lane & 15)) * n4 + KE * (lane >> 4);
@@ -172,30 +200,28 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
   // the (b, k) pairs of the tile, one or NT per thread
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
-    const int bl = tid >> 4, kl = tid & 15;
+    const int bl = pbl, kl = pkl;
     const int b = b0 + 16 * nt + bl, k = k0 + kl;
     if (b >= p.B) continue;
     const long long idx = (long long)b * n + k;
-    float dyw = p.dyw[idx];
+    float dyw = q_dyw[nt];
     if (t_gemm >= 0) dyw += tile[nt][bl][kl];
     if (t >= 0) {
       const long long bn = (long long)p.B * n;
       const long long io = (long long)b * n4 + k;
       const long long fo = t * bn * 4 + io;
-      const float m = p.mask[t * p.B + b];
-      const float d_y_b = (E::load(p.DY, t * bn + idx) + dyw) * m;
-      const float dc = p.Dc0[idx];
+      const float m = q_m[nt];
+      const float d_y_b = (q_dy[nt] + dyw) * m;
+      const float dc = q_dc[nt];
       const float d_c_b = dc * m;
-      const float prev_c = bwd_prev_cell<AT>(p, prev_t, idx, io);
-      const float fgtGate = E::load(p.H, fo + 2 * n);
+      const float fgtGate = q_h[nt][2];
       float dx[4];
-      const float d_c2 = bwd_cell<AT>(p.op_flags, E::load(p.H, fo), E::load(p.H, fo + n), fgtGate, E::load(p.H, fo + 3 * n), prev_c, d_y_b, d_c_b, dx);
+      const float d_c2 = bwd_cell<AT>(p.op_flags, q_h[nt][0], q_h[nt][1], fgtGate, q_h[nt][3], q_pc[nt], d_y_b, d_c_b, dx);
       p.Dc0[idx] = fgtGate * d_c2 + dc * (1.f - m);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         E::store(p.DX, fo + g * n, dx[g]);
-        const float old = E::load(p.dx0, io + g * n);
-        E::store(p.dx0, io + g * n, dx[g] + old * (1.f - m));
+        E::store(p.dx0, io + g * n, dx[g] + q_dx0[nt][g] * (1.f - m));
       }
       dyw = (p.op_flags & kOpNoCarry) ? 0.f : dyw * (1.f - m);
     }
