@@ -287,7 +287,6 @@ def _normalise_lstm2_args(X, W, y0, c0, i):
     return (X, W, y0, c0, i), (T, B, n, bf16)
 
 
-
 def _alloc_lstm2_outputs(T, B, n, bf16, device):
     act = torch.bfloat16 if bf16 else torch.float32
     Y = torch.empty((T, B, n), dtype=act, device=device)
