@@ -68,42 +68,75 @@ def achievable_fields(probe_us, rows, n, dtype, T, call_ms):
     }
 
 
+def blas_thread_count():
+    """Threads the BLAS behind numpy uses for one SGEMM, and where that figure comes from."""
+    try:
+        from threadpoolctl import threadpool_info
+
+        counts = [int(i.get("num_threads", 1)) for i in threadpool_info() if i.get("user_api") == "blas"]
+        if counts:
+            return max(counts), "threadpoolctl (threads of the BLAS that numpy links)"
+    except Exception:
+        pass
+    if os.environ.get("OMP_NUM_THREADS"):
+        return int(os.environ["OMP_NUM_THREADS"]), "OMP_NUM_THREADS"
+    return int(os.cpu_count() or 1), "os.cpu_count()"
+
+
 def cpu_baseline(name: str, target_seconds: float = 15.0):
-    """Times the CPU restatement (test infrastructure, used here only as the reported baseline)."""
-    import numpy
+    """Times the CPU restatement (test infrastructure, used here only as the reported baseline): on all BLAS threads
+    (``value``) and, on a fifth of the time budget, on one thread (``value_1thread``; the reference's tests pin one
+    thread, tests/_set_num_threads1.py)."""
+    import contextlib
 
     from oracle import lstm2_oracle
     from returnn_amd import synthetic
 
-    try:
-        from threadpoolctl import threadpool_info
-
-        blas_threads = max([int(i.get("num_threads", 1)) for i in threadpool_info() if i.get("user_api") == "blas"] or [1])
-    except Exception:
-        blas_threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    probe_T = 25
-    p = synthetic.make_config(name, T=probe_T)
-    lstm2_oracle.native_lstm2_fwd_blas(p.X[:2], p.W, p.y0, p.c0, p.i[:2])  # warm-up (BLAS thread pool, page-in)
-    t0 = time.perf_counter()
-    lstm2_oracle.native_lstm2_fwd_blas(p.X, p.W, p.y0, p.c0, p.i)
-    per_frame = (time.perf_counter() - t0) / probe_T
+    blas_threads, source = blas_thread_count()
     full_T = synthetic.make_config.__globals__["_SPECS"][name]["T"]
-    T = int(max(probe_T, min(full_T, target_seconds / max(per_frame, 1e-9))))
-    p = synthetic.make_config(name, T=T)
-    reps = int(max(1, min(50, round(target_seconds / max(per_frame * T, 1e-9)))))
-    t0 = time.perf_counter()
-    for _ in range(reps):
+
+    def timed(seconds):
+        probe_T = 25
+        p = synthetic.make_config(name, T=probe_T)
+        lstm2_oracle.native_lstm2_fwd_blas(p.X[:2], p.W, p.y0, p.c0, p.i[:2])  # warm-up (BLAS thread pool, page-in)
+        t0 = time.perf_counter()
         lstm2_oracle.native_lstm2_fwd_blas(p.X, p.W, p.y0, p.c0, p.i)
-    dt = time.perf_counter() - t0
-    return {
-        "value": reps * p.T * p.B / dt,
+        per_frame = (time.perf_counter() - t0) / probe_T
+        T = int(max(probe_T, min(full_T, seconds / max(per_frame, 1e-9))))
+        p = synthetic.make_config(name, T=T)
+        reps = int(max(1, min(50, round(seconds / max(per_frame * T, 1e-9)))))
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            lstm2_oracle.native_lstm2_fwd_blas(p.X, p.W, p.y0, p.c0, p.i)
+        dt = time.perf_counter() - t0
+        return reps * p.T * p.B / dt, p, reps, dt
+
+    value, p, reps, dt = timed(target_seconds * 0.8)
+    one_thread = None
+    try:
+        from threadpoolctl import threadpool_limits
+
+        limit = threadpool_limits(limits=1, user_api="blas")
+    except Exception:
+        limit = None
+    if limit is not None:
+        with limit if hasattr(limit, "__enter__") else contextlib.nullcontext():
+            one_thread, p1, reps1, dt1 = timed(target_seconds * 0.2)
+    result = {
+        "value": value,
         "unit": "timesteps*seqs/s",
         "cores": blas_threads,
+        "cores_source": source,
         "kind": "port",
         "sample": "%s shape in fp32, one direction, first T=%i of %i frames (B=%i, n=%i), %i passes, %.1f s; "
-        "per frame one SGEMM on %i BLAS threads, pointwise loop on 1 thread, as the reference's CPU path"
+        "per frame one SGEMM on %i BLAS threads, pointwise loop on 1 thread, as the reference's CPU path; the frame loop "
+        "itself is Python (one numpy matmul and one ctypes call per frame)"
         % (name, p.T, full_T, p.B, p.n, reps, dt, blas_threads),
     }
+    if one_thread is not None:
+        result["value_1thread"] = one_thread
+        result["sample_1thread"] = "the same with the BLAS limited to 1 thread: first T=%i frames, %i passes, %.1f s" % (p1.T, reps1, dt1)
+    return result
 
 
 def torch_stack_baseline(prob, dev, steps, warmup):

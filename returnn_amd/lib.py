@@ -30,6 +30,9 @@ MODE_AUTO = 0
 MODE_PERSISTENT = 1
 MODE_GRAPH = 2
 MODE_STEPWISE = 3
+# The ABI version the structs and argument lists below were written for (rtn_native_lstm2_abi_version()).
+EXPECTED_ABI = 5
+
 MODES = {"auto": MODE_AUTO, "persistent": MODE_PERSISTENT, "graph": MODE_GRAPH, "stepwise": MODE_STEPWISE}
 
 # every symbol include/rtn_native_lstm2.h declares
@@ -108,6 +111,10 @@ class NativeLibraryMissing(RuntimeError):
     """The HIP library has not been built."""
 
 
+class NativeLibraryMismatch(RuntimeError):
+    """The built library reports another ABI version than this binding was written for (a stale build)."""
+
+
 def load() -> ctypes.CDLL:
     """Load the built library (once per process). Never builds, never falls back."""
     global _lib
@@ -121,6 +128,15 @@ def load() -> ctypes.CDLL:
                 "cross-compiles for gfx950 without a GPU)." % path
             )
         lib = ctypes.CDLL(path)
+        lib.rtn_native_lstm2_abi_version.restype = ctypes.c_int
+        lib.rtn_native_lstm2_abi_version.argtypes = []
+        abi = int(lib.rtn_native_lstm2_abi_version())
+        if abi != EXPECTED_ABI:
+            # calling on with other struct layouts or argument lists would write through wrong device pointers
+            raise NativeLibraryMismatch(
+                "%s reports ABI version %i, this binding is written for %i: rebuild it with `python -m returnn_amd.build`"
+                % (path, abi, EXPECTED_ABI)
+            )
         vp, i32, i64, sz = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_size_t
         lib.rtn_native_lstm2_fwd.restype = ctypes.c_int
         lib.rtn_native_lstm2_fwd.argtypes = [vp, vp, vp, vp, vp, i32, i32, vp, vp, vp, vp, i64, i32, i32, i32, i32, vp, sz, vp]

@@ -32,7 +32,15 @@ def test_header_symbols_are_exported(cabi):
 
 
 def test_abi_version(cabi):
-    assert cabi.rtn_native_lstm2_abi_version() == 5
+    assert cabi.rtn_native_lstm2_abi_version() == lib.EXPECTED_ABI
+
+
+def test_loader_refuses_another_abi_version(monkeypatch):
+    """A stale build with other struct layouts must not be called."""
+    monkeypatch.setattr(lib, "_lib", None)
+    monkeypatch.setattr(lib, "EXPECTED_ABI", lib.EXPECTED_ABI + 1)
+    with pytest.raises(lib.NativeLibraryMismatch):
+        lib.load()
 
 
 def test_error_codes_match_header():

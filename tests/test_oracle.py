@@ -305,6 +305,50 @@ def test_threads_do_not_change_results():
         assert numpy.array_equal(u, v)
 
 
+@pytest.mark.parametrize("start,step", [(0, 1), (0, -1), (1, 2), (2, -3)])
+def test_blas_variant_equals_the_restatement(start, step):
+    """The BLAS-structured variant that the benchmark times as the CPU baseline computes the same op: all five
+    outputs on a ragged batch, also on frames the loop does not visit (H = X, Y = C = 0 there)."""
+    rng = numpy.random.default_rng(23)
+    T, B, n = 13, 6, 20
+    X, W, y0, c0 = _random_problem(rng, T, B, n)
+    lens = numpy.array([13, 7, 1, 10, 13, 4])
+    i = (numpy.arange(T)[:, None] < lens[None, :]).astype(numpy.float32)
+    want = oracle.native_lstm2_fwd(X, W, y0, c0, i, start, step, dtype=numpy.float32)
+    got = oracle.native_lstm2_fwd_blas(X, W, y0, c0, i, start, step)
+    for name, a, b in zip(("Y", "C", "H", "d", "y_last"), got, want):
+        assert a.dtype == numpy.float32 and a.shape == b.shape, name
+        assert_allclose(a, b, rtol=1e-6, atol=1e-6, err_msg=name)
+
+
+@pytest.mark.parametrize("step", [1, -1])
+def test_blas_variant_vs_torch_lstm_packed_ragged(step):
+    """The same variant against torch's LSTM directly (float64, packed ragged batch), without the restatement in between."""
+    rng = numpy.random.default_rng(29)
+    T, B, n = 9, 4, 3
+    X, W, y0, c0 = _random_problem(rng, T, B, n)
+    lens = numpy.array([9, 4, 1, 6])
+    i = (numpy.arange(T)[:, None] < lens[None, :]).astype(numpy.float32)
+    Y, C, H, d, yl = oracle.native_lstm2_fwd_blas(X, W, y0, c0, i, 0, step)
+    Yt, hT, cT = torch_lstm(X, W, y0, c0, lens=lens, reverse=(step < 0))
+    assert_allclose(Y, Yt, rtol=2e-5, atol=2e-6)
+    assert_allclose(d, cT, rtol=2e-5, atol=2e-6)
+    assert_allclose(yl, hT, rtol=2e-5, atol=2e-6)
+
+
+def test_blas_variant_zero_length_and_errors():
+    B, n = 2, 3
+    z = lambda *s: numpy.zeros(s, dtype=numpy.float32)  # noqa: E731
+    c0 = numpy.arange(B * n, dtype=numpy.float32).reshape(B, n)
+    Y, C, H, d, yl = oracle.native_lstm2_fwd_blas(z(0, B, 4 * n), z(n, 4 * n), z(B, n) + 2, c0, z(0, B))
+    assert Y.shape == (0, B, n) and H.shape == (0, B, 4 * n)
+    assert numpy.array_equal(d, c0) and (yl == 2).all()  # returnn/native_op.py:1236-1237
+    with pytest.raises(ValueError):
+        oracle.native_lstm2_fwd_blas(z(3, B, 4 * n), z(n, 4 * n), z(B, n), c0, z(3, B), 3, 1)
+    with pytest.raises(ValueError):
+        oracle.native_lstm2_fwd_blas(z(3, B, 4 * n), z(n, 4 * n), z(B, n), c0, z(3, B), 0, 0)
+
+
 def test_f32_close_to_f64_cfg1():
     """benchmark configuration cfg1 (returnn_amd/synthetic.py) (T=32, B=4, n=64): float32 oracle within 1e-5 relative of the float64 one."""
     from returnn_amd import synthetic
