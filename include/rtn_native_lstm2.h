@@ -95,6 +95,23 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
  * time need distinct workspaces.  Returns 0 on invalid arguments. */
 size_t rtn_native_lstm2_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode);
 
+/*
+ * rtn_native_lstm2_fwd without a workspace argument, for callers that cannot allocate device memory at the point of the
+ * call (code under stream capture that may not grow a pool, tight serving loops, harnesses that forbid allocation).
+ * It has no counterpart in the reference.  The scratch lives in a fixed array inside the library's code object
+ * (20 MiB per GPU the library runs on, held until the process ends), so the problem's workspace
+ * (rtn_native_lstm2_fwd_workspace_bytes) must fit 20 MiB -- that covers widths up to 1024 in both element types with
+ * batches up to 128 rows (widths that are not a multiple of 32 need padded copies of all tensors and fit only when
+ * small) -- else RTN_ERR_WORKSPACE.  The call allocates nothing on the device and calls
+ * no allocating runtime routine: AUTO resolves to PERSISTENT or to plain per-step launches, GRAPH is refused
+ * (RTN_ERR_UNSUPPORTED).  Arguments, results and error codes are otherwise those of rtn_native_lstm2_fwd, bit for bit.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU race (keep them on one stream,
+ * or order them with events).  The array keeps the previous call's contents; every call re-initialises what it uses.
+ */
+int rtn_native_lstm2_fwd_static(const void* X, const void* W, const void* y0, const float* c0, const float* i,
+                                int32_t start, int32_t step, void* Y, float* C, void* H, float* d, int64_t T,
+                                int32_t B, int32_t n, int32_t dtype, int32_t mode, void* hip_stream);
+
 /* Synchronous check of the last rtn_native_lstm2_fwd that used `workspace`: waits for
  * `hip_stream`, then returns RTN_OK, RTN_ERR_ABORTED (a bounded wait inside the persistent
  * kernel expired, outputs are invalid) or RTN_ERR_HIP.  Stands in for HANDLE_LAST_ERROR
@@ -281,7 +298,7 @@ const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int3
 const char* rtn_native_lstm2_describe_multi_plan(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype,
                                                  int32_t mode);
 
-/* ABI version of this header: 5. */
+/* ABI version of this header: 6. */
 int rtn_native_lstm2_abi_version(void);
 
 #ifdef __cplusplus

@@ -23,6 +23,13 @@
 #include "lstm2_bwd_kernels.h"
 #include "lstm2_kernels.h"
 
+// Scratch memory of rtn_native_lstm2_fwd_static, the entry point for callers that cannot allocate: a fixed array in the
+// code object, one copy per GPU the library runs on, held until the process ends.  Host code never uses this name as an
+// address (on the host it is only a stand-in for the symbol): static_scratch() below asks the runtime for the device
+// address once per device and everything else works with that pointer.
+#define RTN_STATIC_SCRATCH_BYTES (20u << 20)
+static __device__ __align__(256) unsigned char scratch[RTN_STATIC_SCRATCH_BYTES];
+
 namespace rtn {
 namespace {
 
@@ -611,7 +618,8 @@ size_t workspace_each(int count, int64_t T, int32_t B, int32_t n, int32_t dtype,
 // in one cooperative launch (their workgroups share the CUs and hide each other's exchange waits);
 // otherwise they are enqueued one after the other.
 int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode,
-              void* workspace, size_t workspace_bytes, void* hip_stream, int op_flags = 0, size_t ws_stride = 0) {
+              void* workspace, size_t workspace_bytes, void* hip_stream, int op_flags = 0, size_t ws_stride = 0,
+              bool no_graph = false) {
   int rc = check_dims(T, B, n, dtype);
   if (rc != RTN_OK) return rc;
   if (mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return fail(RTN_ERR_ARG, "NativeLstm2: unknown mode %d", mode);
@@ -660,7 +668,7 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
       padded[(size_t)k] = {base + L.X, base + L.W, base + L.y0, (const float*)(base + L.c0), c.i, c.start, c.step,
                            base + L.Y, (float*)(base + L.C), base + L.H, (float*)(base + L.d)};
     }
-    rc = fwd_calls(padded.data(), count, T, B, np, dtype, mode, workspace, need, hip_stream, op_flags, each);
+    rc = fwd_calls(padded.data(), count, T, B, np, dtype, mode, workspace, need, hip_stream, op_flags, each, no_graph);
     if (rc != RTN_OK) return rc;
     for (int k = 0; k < count; ++k) {
       const rtn_lstm2_call& c = calls[k];
@@ -846,7 +854,8 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
       hipLaunchKernelGGL(k_clear_status, dim3(1), dim3(64), 0, stream, p.status);
       RTN_HIP(hipGetLastError());
     }
-    rc = (pl.mode == RTN_MODE_GRAPH && !capturing) ? launch_steps_graph(p, pl, dtype, stream) : launch_steps(p, pl, dtype, stream);
+    // (a library-owned graph needs a stream, a graph and an executable graph of its own: not for callers that cannot allocate)
+    rc = (pl.mode == RTN_MODE_GRAPH && !capturing && !no_graph) ? launch_steps_graph(p, pl, dtype, stream) : launch_steps(p, pl, dtype, stream);
     if (rc != RTN_OK) return rc;
   }
   return RTN_OK;
@@ -933,6 +942,24 @@ BwdLayout bwd_layout(int B, int n, int dtype) {
   return l;
 }
 
+// Device address of this GPU's copy of `scratch`: asked of the runtime once per device, with that device current.
+int static_scratch(void** out) {
+  static std::mutex mu;
+  static void* ptrs[64] = {nullptr};
+  int dev = 0;
+  RTN_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) return fail(RTN_ERR_HIP, "NativeLstm2: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* ptr = nullptr;
+    RTN_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return fail(RTN_ERR_HIP, "NativeLstm2: the runtime gave no address for the static scratch array");
+    ptrs[dev] = ptr;
+  }
+  *out = ptrs[dev];
+  return RTN_OK;
+}
+
 }  // namespace
 }  // namespace rtn
 
@@ -940,7 +967,7 @@ using namespace rtn;
 
 extern "C" {
 
-int rtn_native_lstm2_abi_version(void) { return 5; }
+int rtn_native_lstm2_abi_version(void) { return 6; }
 
 const char* rtn_last_error(void) { return g_last_error.c_str(); }
 
@@ -985,6 +1012,27 @@ int rtn_native_lstm2_fwd(const void* X, const void* W, const void* y0, const flo
   g_last_error.clear();
   rtn_lstm2_call call = {X, W, y0, c0, i, start, step, Y, C, H, d};
   return fwd_calls(&call, 1, T, B, n, dtype, mode, workspace, workspace_bytes, hip_stream);
+}
+
+int rtn_native_lstm2_fwd_static(const void* X, const void* W, const void* y0, const float* c0, const float* i, int32_t start,
+                                int32_t step, void* Y, float* C, void* H, float* d, int64_t T, int32_t B, int32_t n,
+                                int32_t dtype, int32_t mode, void* hip_stream) {
+  g_last_error.clear();
+  int rc = check_dims(T, B, n, dtype);
+  if (rc != RTN_OK) return rc;
+  if (mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return fail(RTN_ERR_ARG, "NativeLstm2: unknown mode %d", mode);
+  if (mode == RTN_MODE_GRAPH)
+    return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: GRAPH mode replays a library-owned graph, which has to be created; "
+                "the entry that allocates nothing takes AUTO, PERSISTENT or STEPWISE");
+  const size_t need = workspace_each(1, T, B, n, dtype, mode);
+  if (need > (size_t)RTN_STATIC_SCRATCH_BYTES)
+    return fail(RTN_ERR_WORKSPACE, "NativeLstm2: T=%lld B=%d n=%d needs %zu bytes of scratch, the static array holds %zu; "
+                "use rtn_native_lstm2_fwd with a workspace", (long long)T, B, n, need, (size_t)RTN_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc != RTN_OK) return rc;
+  rtn_lstm2_call call = {X, W, y0, c0, i, start, step, Y, C, H, d};
+  return fwd_calls(&call, 1, T, B, n, dtype, mode, ws, (size_t)RTN_STATIC_SCRATCH_BYTES, hip_stream, 0, 0, /*no_graph=*/true);
 }
 
 int rtn_native_lstm2_fwd_multi(const rtn_lstm2_call* calls, int32_t count, int64_t T, int32_t B, int32_t n,

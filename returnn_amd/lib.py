@@ -31,7 +31,7 @@ MODE_PERSISTENT = 1
 MODE_GRAPH = 2
 MODE_STEPWISE = 3
 # The ABI version the structs and argument lists below were written for (rtn_native_lstm2_abi_version()).
-EXPECTED_ABI = 5
+EXPECTED_ABI = 6
 
 MODES = {"auto": MODE_AUTO, "persistent": MODE_PERSISTENT, "graph": MODE_GRAPH, "stepwise": MODE_STEPWISE}
 
@@ -39,6 +39,7 @@ MODES = {"auto": MODE_AUTO, "persistent": MODE_PERSISTENT, "graph": MODE_GRAPH, 
 SYMBOLS = (
     "rtn_native_lstm2_fwd",
     "rtn_native_lstm2_fwd_workspace_bytes",
+    "rtn_native_lstm2_fwd_static",
     "rtn_native_lstm2_fwd_status",
     "rtn_native_lstm2_fwd_multi",
     "rtn_native_lstm2_fwd_multi_workspace_bytes",
@@ -140,6 +141,8 @@ def load() -> ctypes.CDLL:
         vp, i32, i64, sz = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_size_t
         lib.rtn_native_lstm2_fwd.restype = ctypes.c_int
         lib.rtn_native_lstm2_fwd.argtypes = [vp, vp, vp, vp, vp, i32, i32, vp, vp, vp, vp, i64, i32, i32, i32, i32, vp, sz, vp]
+        lib.rtn_native_lstm2_fwd_static.restype = ctypes.c_int
+        lib.rtn_native_lstm2_fwd_static.argtypes = [vp, vp, vp, vp, vp, i32, i32, vp, vp, vp, vp, i64, i32, i32, i32, i32, vp]
         lib.rtn_native_lstm2_fwd_workspace_bytes.restype = sz
         lib.rtn_native_lstm2_fwd_workspace_bytes.argtypes = [i64, i32, i32, i32, i32]
         lib.rtn_native_lstm2_fwd_status.restype = ctypes.c_int
