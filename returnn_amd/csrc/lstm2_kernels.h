@@ -589,6 +589,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
 // Waits are bounded as in k_lstm2_mfma.
 // ---------------------------------------------------------------------------------------------
 constexpr int kExDevice = 0;  // device-scope loads and stores: always valid
+constexpr int kExLocal = 1;   // the whole group on one XCD: plain stores into that XCD's L2, loads that bypass the first-level cache
 constexpr int kExNoWait = 3;  // measurement aid: never wait for the other workgroups (results are WRONG; status is set to 2)
 
 template <typename AT>
@@ -637,19 +638,31 @@ struct IntTag {
   static constexpr int value = V;
 };
 
-// LDS layout of k_lstm2_regw (bytes), shared with the host for the launch.
+// LDS layout of k_lstm2_regw (bytes), shared with the host for the launch.  The staging copies of X[t], H[t], Y[t] and
+// C[t] keep the frame's order [row][gate][cell] with kRowPad bytes appended to every row: without them the rows of a
+// workgroup's tile start 64, 128 or 256 bytes apart, the 16 lanes that touch the same cell of 16 rows all meet in the
+// same banks, and three quarters of the kernel's LDS cycles were bank conflicts (SQ_LDS_BANK_CONFLICT).
+constexpr unsigned kRowPad = 16;
 struct RegwLds {
   unsigned red, xl, ml, hs, ys, cs, total;
+  unsigned x_row, y_row, c_row;      // bytes from one row to the next in the X / H, Y and C copies
+  unsigned x_copy, y_copy, c_copy;   // bytes of one copy (the X / H copy ends with a 16-byte slot nobody reads)
 };
 __host__ __device__ constexpr RegwLds regw_lds(int es, int MT, int NT) {
   RegwLds l{};
   const unsigned rows = 16u * NT, cells = 4u * MT;
+  l.x_row = 4u * cells * es + kRowPad;
+  l.y_row = cells * es + kRowPad;
+  l.c_row = cells * 4u + kRowPad;
+  l.x_copy = rows * l.x_row + 16u;
+  l.y_copy = rows * l.y_row;
+  l.c_copy = rows * l.c_row;
   unsigned off = 0;
   l.red = off; off += 2u * kWaves * MT * NT * kTileBytes;
-  l.xl = off; off += 2u * (rows * 4u * cells * es + 16u);  // each copy is followed by a 16-byte slot nobody reads
-  l.hs = off; off += 2u * rows * 4u * cells * es;
-  l.ys = off; off += (2u * rows * cells * es + 15u) / 16u * 16u;
-  l.cs = off; off += 2u * rows * cells * 4u;
+  l.xl = off; off += 2u * l.x_copy;
+  l.hs = off; off += 3u * l.x_copy;
+  l.ys = off; off += (3u * l.y_copy + 15u) / 16u * 16u;
+  l.cs = off; off += 3u * l.c_copy;
   l.ml = off; off += 2u * rows * 4u;
   l.total = off;
   return l;
@@ -691,9 +704,8 @@ struct LaneMax<float> {
 template <>
 struct LaneMax<__bf16> {
   static __device__ __forceinline__ unsigned fold(unsigned acc, unsigned x) {
-    unsigned r;
-    asm("v_pk_max_u16 %0, %1, %2" : "=v"(r) : "v"(acc), "v"(x));
-    return r;
+    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(unsigned, __builtin_elementwise_max(__builtin_bit_cast(u16x2, acc), __builtin_bit_cast(u16x2, x)));
   }
   static __device__ __forceinline__ bool has_sentinel(unsigned acc) {
     return (acc & 0xFFFFu) == 0xFFFFu || (acc >> 16) == 0xFFFFu;
@@ -716,13 +728,42 @@ struct LaneMax<__bf16> {
 
 constexpr unsigned kOobOffset = 0xFFFFFF00u;  // a buffer offset beyond any frame: loads give 0, stores are dropped
 
-template <typename AT, int MT, int NT, int KSMAX>
+// The XCD (accelerator die, with an L2 of its own) this wavefront runs on.
+__device__ __forceinline__ unsigned xcc_id() {
+  unsigned x;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(x));
+  return x & 0xFu;
+}
+
+// HALF: the groups have at most 8 rows (NT == 1, MT even).  A tile then holds valid results in the lanes of rows 0..7
+// only, and the pointwise part folds two tiles into one pass: lanes of rows 0..7 take tile 2u, lanes of rows 8..15 take
+// rows 0..7 of tile 2u + 1, so that a thread owns one (sequence, cell) pair where the plain mapping gives it two, one
+// of them of a row that does not exist.
+template <typename AT, int MT, int NT, int KSMAX, bool HALF = false>
 __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi multi) {
-  // Which of the launch's problems this workgroup works on (uniform over the workgroup).
-  const int which = (int)blockIdx.x / multi.wgs_each;
-  const int bid = (int)blockIdx.x - which * multi.wgs_each;
-  if (which >= multi.count || bid >= multi.grid) return;
+  static_assert(!HALF || (NT == 1 && MT % 2 == 0), "half-tile mapping: one batch tile, an even number of cell tiles");
+  // Which of the launch's problems and which (group, rank) this workgroup works on (uniform over the workgroup).
+  int which, g, r;
+  if (multi.local) {
+    // Every batch group on ONE XCD, so that the hidden state is exchanged through that XCD's L2.  The dispatcher deals
+    // workgroup ids round-robin to the XCDs: id = slot * xcds + xcd.  An XCD hosts the groups xcd, xcd + xcds, ...
+    // of the launch (all problems counted through); that all members of a group really share an XCD is checked below.
+    const int X = multi.xcds, G = multi.p[0].wgs_per_group, per = multi.p[0].groups;
+    const int xcd = (int)blockIdx.x % X, slot = (int)blockIdx.x / X;
+    const int gg = (slot / G) * X + xcd;
+    which = gg / per;
+    if (which >= multi.count) return;
+    g = gg - which * per;
+    r = slot % G;
+  } else {
+    which = (int)blockIdx.x / multi.wgs_each;
+    const int bid = (int)blockIdx.x - which * multi.wgs_each;
+    if (which >= multi.count || bid >= multi.grid) return;
+    map_block(multi.p[which], bid, g, r);
+  }
   const Lstm2Params p = multi.p[which];
+  const int trace_id = which * p.groups * p.wgs_per_group + g * p.wgs_per_group + r;
+  (void)trace_id;
   using E = Elem<AT>;
   using SN = Sentinel<AT>;
   using LM = LaneMax<AT>;
@@ -730,7 +771,8 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   constexpr int KM = E::KM;
   constexpr int ES = (int)sizeof(AT);
   constexpr int TILES = MT * NT;
-  constexpr int EPT = (TILES + kWaves - 1) / kWaves;
+  constexpr int UNITS = HALF ? TILES / 2 : TILES;  // passes of the pointwise part over all wavefronts
+  constexpr int EPT = (UNITS + kWaves - 1) / kWaves;
   constexpr int ROWS = 16 * NT;   // rows of the MFMA tiles (>= valid rows of the group)
   constexpr int CELLS = 4 * MT;   // cells owned by this workgroup
   constexpr RegwLds L = regw_lds(ES, MT, NT);
@@ -742,8 +784,6 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in a scalar register
   const int n = p.n, S = n / KM;
-  int g, r;
-  map_block(p, bid, g, r);
   g += p.group_offset;
   const int b_base = g * p.Bg;
   const int rows = min(p.Bg, p.B - b_base);
@@ -755,13 +795,8 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   // before its own (a barrier lies between that copy and its readers); the outputs are staged in LDS by the threads that compute them and written
   // out after the barrier of the following step.  Chunks of rows the group does not have carry an
   // out-of-range buffer offset: their loads return 0 and their stores are dropped, without a branch.
-  AT* Xl = (AT*)(smem + L.xl);
   float* Ml = (float*)(smem + L.ml);
-  AT* Hs = (AT*)(smem + L.hs);
-  AT* Ys = (AT*)(smem + L.ys);
-  float* Cs = (float*)(smem + L.cs);
   constexpr int SEG = CELLS * ES;               // contiguous bytes of one (row, gate) in X and H
-  constexpr int kXlCopy = ROWS * 4 * SEG + 16;  // one LDS copy of X[t] plus the spare slot
   constexpr int CH = SEG < 16 ? 8 : 16;         // bytes moved per thread and chunk
   constexpr int CPS = SEG / CH;                 // chunks per (row, gate)
   constexpr int XCH = (ROWS * 4 * CPS + kWgThreads - 1) / kWgThreads;  // chunks per thread, X and H
@@ -780,58 +815,81 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     const int c = tid + kWgThreads * i;
     const int row = c / (4 * CPS), gate = (c / CPS) % 4, part = c % CPS;
     xoff[i] = row < rows ? (unsigned)((((b_base + row) * 4 * n) + gate * n + cell0) * ES + part * CH) : kOobOffset;
-    xlds[i] = (unsigned)(min(c, ROWS * 4 * CPS) * CH);  // threads beyond the tile write to / read from the spare slot
+    // threads beyond the tile write to / read from the spare slot at the end of the copy
+    xlds[i] = row < ROWS ? (unsigned)(row * L.x_row + gate * SEG + part * CH) : (unsigned)(ROWS * L.x_row);
   }
 #pragma unroll
   for (int i = 0; i < YCH; ++i) {
     const int c = tid + kWgThreads * i;
     const int row = c / (SEG / CHY), part = c % (SEG / CHY);
     yoff[i] = row < rows ? (unsigned)(((b_base + row) * n + cell0) * ES + part * CHY) : kOobOffset;
-    ylds[i] = (unsigned)(min(c, ROWS * (SEG / CHY) - 1) * CHY);
+    ylds[i] = (unsigned)(min(row, ROWS - 1) * L.y_row + part * CHY);
   }
 #pragma unroll
   for (int i = 0; i < CCH; ++i) {
     const int c = tid + kWgThreads * i;
     const int row = c / (SEGC / 16), part = c % (SEGC / 16);
     coff[i] = row < rows ? (unsigned)(((b_base + row) * n + cell0) * 4 + part * 16) : kOobOffset;
-    clds[i] = (unsigned)(min(c, ROWS * (SEGC / 16) - 1) * 16);
+    clds[i] = (unsigned)(min(row, ROWS - 1) * L.c_row + part * 16);
   }
   const unsigned moff = tid < rows ? (unsigned)((b_base + tid) * 4) : kOobOffset;
   const unsigned frame_x = (unsigned)((size_t)p.B * 4 * n * ES), frame_y = (unsigned)(bn * ES),
                  frame_c = (unsigned)(bn * 4), frame_m = (unsigned)(p.B * 4);
   typename XC::T xv[2][XCH];
   float mv[2] = {0.f, 0.f};
-  auto fetch = [&](int s, auto par_tag) {  // issue the loads of X[t_s] and mask[t_s] into register set PAR
+  // Frame pointers advance by a constant per step (signed: the op may run backwards in time).
+  const long long step_x = (long long)p.step * frame_x, step_y = (long long)p.step * frame_y,
+                  step_c = (long long)p.step * frame_c, step_m = (long long)p.step * frame_m;
+  auto fetch_at = [&](const unsigned char* xp, const unsigned char* mp, bool enabled, auto par_tag) {  // loads of one frame of X and the mask into register set PAR
     constexpr int PAR = decltype(par_tag)::value;
-    const long long t = frame_of(p, s);
-    __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.X + (size_t)t * frame_x, 0, frame_x, kBufFlags);
-    __amdgpu_buffer_rsrc_t mr = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.mask + (size_t)t * frame_m, 0, frame_m, kBufFlags);
+    // (a frame that does not exist: a buffer of no bytes, every load gives 0 without a memory access or a branch)
+    __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void*)xp, 0, enabled ? frame_x : 0u, kBufFlags);
+    __amdgpu_buffer_rsrc_t mr = __builtin_amdgcn_make_buffer_rsrc((void*)mp, 0, enabled ? frame_m : 0u, kBufFlags);
 #pragma unroll
     for (int i = 0; i < XCH; ++i) xv[PAR][i] = XC::load(xr, xoff[i]);
     mv[PAR] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(mr, moff, 0, 0));
   };
+  auto fetch = [&](int s, auto par_tag) {  // issue the loads of X[t_s] and mask[t_s] into register set PAR
+    const long long t = frame_of(p, s);
+    fetch_at((const unsigned char*)p.X + (size_t)t * frame_x, (const unsigned char*)p.mask + (size_t)t * frame_m, true, par_tag);
+  };
   auto put = [&](auto par_tag) {  // register set PAR -> LDS copy PAR
     constexpr int PAR = decltype(par_tag)::value;
-    unsigned char* xl = (unsigned char*)Xl + (size_t)PAR * kXlCopy;
+    unsigned char* xl = smem + L.xl + PAR * L.x_copy;
 #pragma unroll
     for (int i = 0; i < XCH; ++i) *(typename XC::T*)(xl + xlds[i]) = xv[PAR][i];
     if (tid < ROWS) Ml[PAR * ROWS + tid] = mv[PAR];
   };
-  auto flush = [&](int s, auto par_tag) {  // staged outputs of step s (LDS copy PAR) -> H[t], Y[t], C[t]
-    constexpr int PAR = decltype(par_tag)::value;
+  // Staged outputs of a step (LDS copy `copy` of three) -> registers -> H[t], Y[t], C[t]: in two halves, so that the
+  // LDS reads can be issued ahead of a batch of MFMAs and the stores behind it.
+  typename XC::T fh[XCH];
+  typename YC::T fy[YCH];
+  typename CC::T fc[CCH];
+  auto flush_read = [&](int copy) {
+    const unsigned char* hs = smem + L.hs + copy * L.x_copy;
+    const unsigned char* ys = smem + L.ys + copy * L.y_copy;
+    const unsigned char* cs = smem + L.cs + copy * L.c_copy;
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) fh[i] = *(const typename XC::T*)(hs + xlds[i]);
+#pragma unroll
+    for (int i = 0; i < YCH; ++i) fy[i] = *(const typename YC::T*)(ys + ylds[i]);
+#pragma unroll
+    for (int i = 0; i < CCH; ++i) fc[i] = *(const typename CC::T*)(cs + clds[i]);
+  };
+  auto flush_write_at = [&](unsigned char* hp, unsigned char* yp, unsigned char* cp, bool enabled) {
+    __amdgpu_buffer_rsrc_t hr = __builtin_amdgcn_make_buffer_rsrc((void*)hp, 0, enabled ? frame_x : 0u, kBufFlags);
+    __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc((void*)yp, 0, enabled ? frame_y : 0u, kBufFlags);
+    __amdgpu_buffer_rsrc_t cr = __builtin_amdgcn_make_buffer_rsrc((void*)cp, 0, enabled ? frame_c : 0u, kBufFlags);
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) XC::store(fh[i], hr, xoff[i]);
+#pragma unroll
+    for (int i = 0; i < YCH; ++i) YC::store(fy[i], yr, yoff[i]);
+#pragma unroll
+    for (int i = 0; i < CCH; ++i) CC::store(fc[i], cr, coff[i]);
+  };
+  auto flush_write = [&](int s) {
     const long long t = frame_of(p, s);
-    const unsigned char* hs = smem + L.hs + (size_t)PAR * ROWS * 4 * SEG;
-    const unsigned char* ys = smem + L.ys + (size_t)PAR * ROWS * SEG;
-    const unsigned char* cs = smem + L.cs + (size_t)PAR * ROWS * SEGC;
-    __amdgpu_buffer_rsrc_t hr = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.H + (size_t)t * frame_x, 0, frame_x, kBufFlags);
-    __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.Y + (size_t)t * frame_y, 0, frame_y, kBufFlags);
-    __amdgpu_buffer_rsrc_t cr = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.C + (size_t)t * frame_c, 0, frame_c, kBufFlags);
-#pragma unroll
-    for (int i = 0; i < XCH; ++i) XC::store(*(const typename XC::T*)(hs + xlds[i]), hr, xoff[i]);
-#pragma unroll
-    for (int i = 0; i < YCH; ++i) YC::store(*(const typename YC::T*)(ys + ylds[i]), yr, yoff[i]);
-#pragma unroll
-    for (int i = 0; i < CCH; ++i) CC::store(*(const typename CC::T*)(cs + clds[i]), cr, coff[i]);
+    flush_write_at((unsigned char*)p.H + (size_t)t * frame_x, (unsigned char*)p.Y + (size_t)t * frame_y, (unsigned char*)p.C + (size_t)t * frame_c, true);
   };
 
   // ---- the recurrence
@@ -856,8 +914,9 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const int row = (16 * nt + jl < rows) ? 16 * nt + jl : 0;  // rows the group does not have: read row 0
-      foff[ks][nt] = (unsigned)(((4 * sm + kg) * p.Bp + row) * kFragBytes);
+      // Lanes of rows the group does not have load nothing: an out-of-range offset gives zeros (a complete fragment)
+      // without a memory access, so a group of few rows moves few bytes.
+      foff[ks][nt] = (mine && 16 * nt + jl < rows) ? (unsigned)(((4 * sm + kg) * p.Bp + 16 * nt + jl) * kFragBytes) : kOobOffset;
     }
   }
 
@@ -866,15 +925,27 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   bool e_valid[EPT];
   unsigned e_hoff[EPT];            // byte offset of the pair's element in an exchange buffer
   unsigned e_row[EPT], e_cl[EPT];  // row and cell inside the workgroup's tile
+  unsigned e_tile[EPT], e_src[EPT];  // tile and lane of the partial sums of the pair
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
-    const int e = min(wave + kWaves * j, TILES - 1);
-    const int mt = e / NT, nt = e % NT;
-    const int bl = 16 * nt + (lane & 15);
+    const int u = min(wave + kWaves * j, UNITS - 1);
+    int e, bl, src;
+    if (HALF) {
+      e = 2 * u + ((lane >> 3) & 1);
+      bl = lane & 7;
+      src = (lane & 0x30) | bl;
+    } else {
+      e = u;
+      bl = 16 * (e % NT) + (lane & 15);
+      src = lane;
+    }
+    const int mt = e / NT;
     const int cell = 4 * (r * MT + mt) + (lane >> 4);
+    e_tile[j] = (unsigned)e;
+    e_src[j] = (unsigned)src;
     e_row[j] = (unsigned)bl;
     e_cl[j] = (unsigned)(4 * mt + (lane >> 4));
-    e_valid[j] = (wave + kWaves * j < TILES) && (bl < rows);
+    e_valid[j] = (wave + kWaves * j < UNITS) && (bl < rows);
     e_hoff[j] = (unsigned)((((cell / KE) * p.Bp + bl) * KE + (cell % KE)) * ES);
     c_state[j] = 0.f;
     h_prev[j] = 0.f;
@@ -885,50 +956,108 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     }
   }
 
+  // An XCD-local plan rests on all workgroups of the group being on one XCD.  Check it: every workgroup adds its XCD
+  // to the group's mask and then itself to the group's count (two words the prepare kernel cleared; device-scope
+  // atomics whose result is waited for, so the mask is complete when the count is); with one XCD in the mask the hidden
+  // state travels through that XCD's L2 (plain stores, loads that bypass the first-level cache), else with device scope.
+  __shared__ int s_local;
+  if (multi.local && tid == 0) {
+    int ok = 1;
+    if (p.wgs_per_group > 1) {
+      unsigned* words = p.flags + (size_t)g * p.wgs_per_group;
+      (void)__hip_atomic_fetch_or(words + 1, 1u << xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      (void)__hip_atomic_fetch_add(words, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      unsigned long long t0 = 0;
+      unsigned spins = 0;
+      while (__hip_atomic_load(words, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)p.wgs_per_group) {
+        if ((spins++ & 15u) == 0) {
+          if (__hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+          const unsigned long long now = wall_clock64();
+          if (spins == 1) {
+            t0 = now;
+          } else if (now - t0 > p.timeout_ticks) {
+            __hip_atomic_store(p.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+      const unsigned mask = __hip_atomic_load(words + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      ok = (mask & (mask - 1)) == 0;
+      if (!ok) __hip_atomic_store(p.status + 1, mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the record: the group was spread
+    }
+    s_local = ok;
+  }
+
   auto run = [&](auto ex_tag) {
     constexpr int EX = decltype(ex_tag)::value;
-    constexpr int AUXS = kAuxDevice, AUXL = kAuxDevice;  // exchange stores and loads: device scope
+    // Exchange loads always bypass the first-level cache (device scope).  Stores: through to memory (device scope), or,
+    // when the whole group shares an XCD, plain stores that stay in that XCD's L2, where the loads find them.
+    constexpr int AUXS = (EX == kExLocal) ? 0 : kAuxDevice, AUXL = kAuxDevice;
     i32x4 bf[KSMAX][NT];
-    // Issue the loads of this wave's fragments of ring buffer s%4.
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) bf[ks][nt] = i32x4{0, 0, 0, 0};
+    // Issue the loads of this wave's fragments of ring buffer s%4.  Lanes of rows the group does not have are switched
+    // off (their registers keep the zeros from above: a complete fragment): the address unit spends its cycles on the
+    // active lanes only, and a wavefront's eight loads are what a CU's address unit is busy with for most of the read.
     auto issue = [&](int s) {
       const unsigned soff = (unsigned)(s & (kHxRing - 1)) * hx_buf_bytes;
       asm volatile("" ::: "memory");  // other workgroups write this memory: really load again
 #pragma unroll
-      for (int ks = 0; ks < KSMAX; ++ks)
+      for (int nt = 0; nt < NT; ++nt)
+        if (16 * nt + jl < rows) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          bf[ks][nt] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(ring_rs, foff[ks][nt], soff, AUXL));
+          for (int ks = 0; ks < KSMAX; ++ks)
+            bf[ks][nt] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(ring_rs, foff[ks][nt], soff, AUXL));
+        }
     };
-    // This thread's gate inputs and mask of the step to come, read from the LDS copy PAR.
-    float x_in[EPT][4], m_in[EPT];
+    // This thread's gate inputs and mask of a step, read from the LDS copy PAR into register set PAR (as stored; they
+    // are widened where they are used, so that the reads can all be in flight together).
+    AT x_in[2][EPT][4];
+    float m_in[2][EPT];
     auto load_gate_inputs = [&](auto par_tag) {
       constexpr int PAR = decltype(par_tag)::value;
 #pragma unroll
       for (int j = 0; j < EPT; ++j) {
-        const AT* xin = (const AT*)((const unsigned char*)Xl + PAR * kXlCopy) + (e_row[j] * 4) * CELLS + e_cl[j];
+        const unsigned char* xin = smem + L.xl + PAR * L.x_copy + e_row[j] * L.x_row + e_cl[j] * ES;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) x_in[j][q] = (float)xin[q * CELLS];
-        m_in[j] = Ml[PAR * ROWS + e_row[j]];
+        for (int q = 0; q < 4; ++q) x_in[PAR][j][q] = *(const AT*)(xin + q * SEG);
+        m_in[PAR][j] = Ml[PAR * ROWS + e_row[j]];
       }
     };
     RTN_TRACE_DECL
+    unsigned char *h_out = nullptr, *y_out_p = nullptr, *c_out = nullptr;
+    const unsigned char *x_next = nullptr, *m_next = nullptr;
     int delay = p.poll_delay;  // in units of s_sleep(1), about 64 clocks; adapts, see below
-    // One time step; PAR = s & 1 selects the register set and the LDS copies.
-    auto step = [&](int s, auto par_tag) {
+    // One time step; PAR = s & 1 selects the register sets and the LDS copies of X, `stage` = s % 3 the copy that
+    // takes this step's outputs.
+    //
+    // The step's critical path is: h_{s-1} arrives -> MFMAs -> partial tiles through LDS (the one barrier) -> gates ->
+    // new hidden values out.  Everything else rides in the shadow of the MFMAs, which a wavefront issues at one per 16
+    // clocks with nothing else to do in between: the outputs of step s-2 go from LDS to memory (their staging and this
+    // point are separated by the barrier of step s-1), the gate inputs of step s+1 come from LDS into the other
+    // register set, X[t_{s+2}] moves from registers to LDS and X[t_{s+4}] from memory into the registers that became
+    // free.  LDS reads are issued ahead of a batch of MFMAs and used behind it.
+    auto step = [&](int s, auto par_tag, int stage) {
       constexpr int PAR = decltype(par_tag)::value;
 
       // Complete this wave's share of h_{s-1}: if anything that came back is not written yet, read again.
+      // (Four independent running maxima: a single chain of dependent packed operations needs a wait state after
+      // every one of them.)
       unsigned long long t0 = 0;
       unsigned spins = 0;
       for (;;) {
-        unsigned m = 0;
+        unsigned m[4] = {0, 0, 0, 0};
 #pragma unroll
         for (int ks = 0; ks < KSMAX; ++ks)
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int w = 0; w < 4; ++w) m = LM::fold(m, (unsigned)bf[ks][nt][w]);
-        if (EX == kExNoWait || !__any(LM::has_sentinel(m))) break;
+            for (int w = 0; w < 4; ++w) m[w] = LM::fold(m[w], (unsigned)bf[ks][nt][w]);
+        const unsigned seen = LM::fold(LM::fold(m[0], m[1]), LM::fold(m[2], m[3]));
+        if (EX == kExNoWait || !__any(LM::has_sentinel(seen))) break;
         if ((spins++ & 15u) == 0) {
           if (__hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
           const unsigned long long now = wall_clock64();
@@ -947,12 +1076,13 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       // (The builtin rather than inline assembly, so that the compiler's own wait-count bookkeeping sees it.)
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
       asm volatile("" ::: "memory");
-      // The first read is held back by `delay` so that it usually comes back complete: a read that
-      // comes back incomplete costs a whole extra round trip.  Lengthen the delay when that happened,
-      // shorten it slowly while it does not.
+      // The first read is held back by `delay` so that it usually comes back complete: a read that comes back
+      // incomplete costs a whole extra round trip, waiting too long costs the wait itself.  Lengthen the delay when a
+      // read had to be repeated, shorten it while none has (one unit every (delay_dec_mask + 1) steps): the repeat
+      // rate settles near 1 / (2 * (delay_dec_mask + 1)).
       if (spins)
         delay = min(delay + 2, 64);
-      else if ((s & 15) == 15 && delay > 0)
+      else if ((s & p.delay_dec_mask) == p.delay_dec_mask && delay > 0)
         --delay;
       RTN_TRACE_MARK(7)  // outstanding stores acknowledged
       RTN_TRACE_ADD(6, spins)
@@ -963,37 +1093,59 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      // Everything that is not on the path h -> MFMA -> gates -> h rides in the shadow of the MFMAs: all of it without
+      // a branch (a frame that does not exist is a buffer of no bytes; LDS copies nobody reads may take anything), in
+      // one block of straight-line code that the scheduler is told to weave: a wavefront that has a SIMD to itself
+      // issues one instruction per 4 clocks, an MFMA keeps the matrix core busy for 16, so three other instructions fit
+      // behind every MFMA for free -- but a run of them between two MFMAs drains the matrix core.
+      flush_read(stage == 2 ? 0 : stage + 1);  // the copy of step s-2 is (s+1) % 3
+      load_gate_inputs(IntTag<1 - PAR>{});
+      put(par_tag);
+      flush_write_at(h_out, y_out_p, c_out, s >= 2);
+      fetch_at(x_next, m_next, s + 4 < nsteps, par_tag);
 #pragma unroll
       for (int ks = 0; ks < KSMAX; ++ks)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+          for (int nt = 0; nt < NT; ++nt) {
+            acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+            __builtin_amdgcn_sched_group_barrier(0x008, sizeof(AT) == 2 ? 1 : 4, 0);  // the MFMA(s) of one fragment ...
+            __builtin_amdgcn_sched_group_barrier(0x096, 3, 0);                        // ... then up to three of the rest (VALU, SALU, VMEM, LDS)
+          }
+      h_out += step_x; y_out_p += step_y; c_out += step_c; x_next += step_x; m_next += step_m;
+      // (with at most 8 rows only the lanes of rows 0..7 hold columns anybody reads)
+      if (!HALF || (lane & 8) == 0) {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) redbuf[wave][mt * NT + nt][lane] = acc[mt][nt];
-      RTN_TRACE_MARK(1)  // MFMA, partial tiles to LDS
-      __syncthreads();  // the one barrier of a step: partial tiles, X[t_{s+1}] and the outputs of step s-1 are in LDS
+          for (int nt = 0; nt < NT; ++nt) redbuf[wave][mt * NT + nt][lane] = acc[mt][nt];
+      }
+      RTN_TRACE_MARK(1)  // MFMA with the streams in their shadow, partial tiles to LDS
+      __syncthreads();  // the one barrier of a step: partial tiles, X[t_{s+2}] and the outputs of step s-1 are in LDS
       RTN_TRACE_MARK(2)  // barrier
 
-      // Gates and cell update first, then straight away the new hidden values (the step's critical path);
-      // staging of the op's outputs comes after those stores are on their way.
+      // Gates and cell update, then straight away the new hidden values.
       unsigned h_bits[EPT];
       float g_act[EPT][4], y_out[EPT];
 #pragma unroll
       for (int j = 0; j < EPT; ++j) {
         h_bits[j] = 0;
-        if (TILES % kWaves == 0 || wave + kWaves * j < TILES) {  // wave-uniform
-          const int e = wave + kWaves * j;
-          f32x4 gsum = redbuf[0][e][lane];
+        if (UNITS % kWaves == 0 || wave + kWaves * j < UNITS) {  // wave-uniform
+          // (all four partial tiles on their way before the first is used: the compiler, left alone, reads them one
+          // after the other through one set of registers and pays the LDS latency three times)
+          f32x4 part[kWaves];
 #pragma unroll
-          for (int w = 1; w < kWaves; ++w) gsum += redbuf[w][e][lane];
-          const float m = m_in[j];
-          const float a0 = Act<AT>::tanh(gsum[0] + x_in[j][0]);
-          const float a1 = Act<AT>::sigmoid(gsum[1] + x_in[j][1]);
-          const float a2 = Act<AT>::sigmoid(gsum[2] + x_in[j][2]);
-          const float a3 = Act<AT>::sigmoid(gsum[3] + x_in[j][3]);
+          for (int w = 0; w < kWaves; ++w) part[w] = redbuf[w][e_tile[j]][e_src[j]];
+          __builtin_amdgcn_sched_barrier(0);
+          f32x4 gsum = part[0];
+#pragma unroll
+          for (int w = 1; w < kWaves; ++w) gsum += part[w];
+          const float m = m_in[PAR][j];
+          const float a0 = Act<AT>::tanh(gsum[0] + (float)x_in[PAR][j][0]);
+          const float a1 = Act<AT>::sigmoid(gsum[1] + (float)x_in[PAR][j][1]);
+          const float a2 = Act<AT>::sigmoid(gsum[2] + (float)x_in[PAR][j][2]);
+          const float a3 = Act<AT>::sigmoid(gsum[3] + (float)x_in[PAR][j][3]);
           const float pc = c_state[j];
           const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
           const float y = E::round(Act<AT>::tanh(c) * a3 * m);
@@ -1013,40 +1165,29 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
         const unsigned arm = (unsigned)((s + 3) & (kHxRing - 1)) * hx_buf_bytes;
 #pragma unroll
         for (int j = 0; j < EPT; ++j)
-          if (TILES % kWaves == 0 || wave + kWaves * j < TILES) SN::template store<AUXS>(ring_rs, e_hoff[j] + nxt, h_bits[j]);
+          if (UNITS % kWaves == 0 || wave + kWaves * j < UNITS) SN::template store<AUXS>(ring_rs, e_hoff[j] + nxt, h_bits[j]);
 #pragma unroll
         for (int j = 0; j < EPT; ++j)
-          if (TILES % kWaves == 0 || wave + kWaves * j < TILES) SN::template store<AUXS>(ring_rs, e_hoff[j] + arm, SN::kSentinel);
+          if (UNITS % kWaves == 0 || wave + kWaves * j < UNITS) SN::template store<AUXS>(ring_rs, e_hoff[j] + arm, SN::kSentinel);
       }
       RTN_TRACE_MARK(3)  // gates, cell update, exchange stores
-      // stage the op's outputs of this step
+      // While the new hidden values travel: stage the op's outputs of this step (they leave two steps from now), and
+      // after the delay issue the first read of the next step.
 #pragma unroll
       for (int j = 0; j < EPT; ++j) {
-        if (TILES % kWaves == 0 || wave + kWaves * j < TILES) {
-          const unsigned xi = ((PAR * ROWS + e_row[j]) * 4) * CELLS + e_cl[j];  // in the staging copies
-          Hs[xi] = (AT)g_act[j][0];
-          Hs[xi + CELLS] = (AT)g_act[j][1];
-          Hs[xi + 2 * CELLS] = (AT)g_act[j][2];
-          Hs[xi + 3 * CELLS] = (AT)g_act[j][3];
-          const unsigned yi = (PAR * ROWS + e_row[j]) * CELLS + e_cl[j];
-          Ys[yi] = (AT)y_out[j];
-          Cs[yi] = c_state[j];
+        if (UNITS % kWaves == 0 || wave + kWaves * j < UNITS) {
+          unsigned char* hq = smem + L.hs + stage * L.x_copy + e_row[j] * L.x_row + e_cl[j] * ES;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) *(AT*)(hq + q * SEG) = (AT)g_act[j][q];
+          *(AT*)(smem + L.ys + stage * L.y_copy + e_row[j] * L.y_row + e_cl[j] * ES) = (AT)y_out[j];
+          *(float*)(smem + L.cs + stage * L.c_copy + e_row[j] * L.c_row + e_cl[j] * 4) = c_state[j];
         }
       }
-      // While the new hidden values travel: X[t_{s+2}] from registers to LDS, X[t_{s+4}] from memory into the
-      // registers that have just become free; after the delay the first read of the next step; and behind that
-      // read, in its shadow, this thread's gate inputs of the next step from LDS to registers (X[t_{s+1}] got
-      // there one step ago) and the outputs of the previous step from LDS to memory.
-      if (s + 2 < nsteps) put(par_tag);
-      if (s + 4 < nsteps) fetch(s + 4, par_tag);
       if (s + 1 < nsteps) {
         for (int k = 0; k < delay; ++k) __builtin_amdgcn_s_sleep(1);
         issue(s + 1);
       }
-      RTN_TRACE_MARK(4)  // staging, put, fetch, delay, first read of the next step
-      if (s + 1 < nsteps) load_gate_inputs(IntTag<1 - PAR>{});
-      if (s >= 1) flush(s - 1, IntTag<1 - PAR>{});
-      RTN_TRACE_MARK(5)  // gate inputs, output stores
+      RTN_TRACE_MARK(4)  // staging, delay, first read of the next step
     };
     fetch(0, IntTag<0>{});
     if (nsteps > 1) fetch(1, IntTag<1>{});
@@ -1056,25 +1197,42 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     load_gate_inputs(IntTag<0>{});
     if (nsteps > 2) fetch(2, IntTag<0>{});
     if (nsteps > 3) fetch(3, IntTag<1>{});
+    __syncthreads();  // everybody has the gate inputs of step 0: its LDS copy may take X[t_2]
     issue(0);
+    int stage = 0;
+    // frames of the outputs of step s-2 and of the inputs of step s+4, as the loop reaches step s
+    h_out = (unsigned char*)p.H + (frame_of(p, 0) - 2 * (long long)p.step) * (long long)frame_x;
+    y_out_p = (unsigned char*)p.Y + (frame_of(p, 0) - 2 * (long long)p.step) * (long long)frame_y;
+    c_out = (unsigned char*)p.C + (frame_of(p, 0) - 2 * (long long)p.step) * (long long)frame_c;
+    x_next = (const unsigned char*)p.X + frame_of(p, 4) * (long long)frame_x;
+    m_next = (const unsigned char*)p.mask + frame_of(p, 4) * (long long)frame_m;
     for (int s = 0; s < nsteps; s += 2) {
-      step(s, IntTag<0>{});
-      if (s + 1 < nsteps) step(s + 1, IntTag<1>{});
+      step(s, IntTag<0>{}, stage);
+      stage = stage == 2 ? 0 : stage + 1;
+      if (s + 1 < nsteps) {
+        step(s + 1, IntTag<1>{}, stage);
+        stage = stage == 2 ? 0 : stage + 1;
+      }
     }
     RTN_TRACE_ADD(6, (unsigned long long)delay << 40)
-    RTN_TRACE_FLUSH(p, bid)
+    RTN_TRACE_FLUSH(p, trace_id)
   };
+  __syncthreads();  // s_local
   if (p.exchange == kExNoWait) {
     if (tid == 0) __hip_atomic_store(p.status, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     run(IntTag<kExNoWait>{});
+  } else if (multi.local && s_local) {
+    run(IntTag<kExLocal>{});
   } else {
     run(IntTag<kExDevice>{});
   }
   __syncthreads();  // the last step's outputs are staged
-  if ((nsteps - 1) & 1)
-    flush(nsteps - 1, IntTag<1>{});
-  else
-    flush(nsteps - 1, IntTag<0>{});
+  if (nsteps >= 2) {
+    flush_read((nsteps - 2) % 3);
+    flush_write(nsteps - 2);
+  }
+  flush_read((nsteps - 1) % 3);
+  flush_write(nsteps - 1);
 
 #pragma unroll
   for (int j = 0; j < EPT; ++j)

@@ -59,6 +59,7 @@ struct Lstm2Params {
   int xcds;           // XCDs assumed for the blockIdx -> (group, rank) mapping
   int exchange;       // register kernel: 0 = normal operation; 3, 4 = measurement aids (see kExNoWait, kExProbe)
   int poll_delay;     // register kernel: s_sleep(1) repeats between the hidden-value stores and the first read of the next step
+  int delay_dec_mask; // register kernel: the delay adapts downwards by one unit every (mask + 1) steps without a repeated read
   unsigned long long* trace;  // optional [workgroups][8] cycle totals per phase (instrumented builds only)
   int op_flags;       // OpFlags: variations of the recurrence for the sibling ops (0 = NativeLstm2)
   int w_direct;       // per-step launches of the LDS kernel: 1 = W fragments go from memory straight to the matrix cores (no LDS copy)
@@ -74,6 +75,9 @@ struct Lstm2Multi {
   int count;     // problems, 1..kMaxMulti
   int wgs_each;  // workgroup ids reserved per problem, a multiple of the XCD count (keeps the id -> XCD dealing in phase)
   int grid;      // workgroups a problem really uses (<= wgs_each)
+  int local;     // 1: every batch group of every problem sits on one XCD (workgroup id = slot * xcds + xcd; the groups of
+                 // the launch, all problems counted through, are dealt round-robin to the XCDs); wgs_each / grid unused
+  int xcds;      // XCDs the workgroup ids are dealt to (local plans)
   int pad_;
   Lstm2Params p[kMaxMulti];
 };

@@ -81,6 +81,9 @@ DeviceInfo device_info() {
     (void)hipGetLastError();
     return fallback;
   }
+  // RTN_LSTM2_XCDS: pretend the workgroup ids are dealt to this many XCDs (an experiment and test knob: with a wrong
+  // count the groups of an XCD-local plan do not sit on one XCD each, the kernel notices and exchanges at device scope)
+  const long env_xcds = env_long("RTN_LSTM2_XCDS", 0);
   std::lock_guard<std::mutex> lock(mu);
   if (!cache[dev].valid) {
     hipDeviceProp_t prop;
@@ -97,7 +100,9 @@ DeviceInfo device_info() {
     di.valid = true;
     cache[dev] = di;
   }
-  return cache[dev];
+  DeviceInfo di = cache[dev];
+  if (env_xcds > 0 && di.cus % env_xcds == 0) di.xcds = (int)env_xcds;
+  return di;
 }
 
 enum PlanKind { kPlanEmpty, kPlanGeneric, kPlanMfma };
@@ -106,6 +111,8 @@ struct Plan {
   PlanKind kind = kPlanGeneric;
   int mode = RTN_MODE_STEPWISE;  // resolved: PERSISTENT, GRAPH or STEPWISE
   bool regw = false;             // persistent kernel with W in registers and self-validating exchange
+  bool local = false;            // regw: every batch group on one XCD, hidden state exchanged through that XCD's L2
+  bool half = false;             // regw: groups of at most 8 rows, two tiles folded into one pass of the pointwise part
   int grid = 0;                  // workgroups launched by the persistent kernel
   int KSMAX = 0;                 // its macro steps per wavefront (template bound)
   int MT = 1, NT = 1;
@@ -168,10 +175,55 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
     const int KSMAX = ks <= 2 ? 2 : (ks <= 4 ? 4 : (ks <= 8 ? 8 : (ks <= 16 ? 16 : 0)));
     if (want_mode == RTN_MODE_AUTO || want_mode == RTN_MODE_PERSISTENT) {
       struct Cand {
-        bool ok = false, regw = false;
-        int KSMAX = 0, MT = 1, NT = 1, groups = 1, G = 1, Bg = 1;
+        bool ok = false, regw = false, local = false, half = false;
+        int KSMAX = 0, MT = 1, NT = 1, groups = 1, G = 1, Bg = 1, grid = 0;
         size_t lds = 0;
         double est = 1e30;
+      };
+      // XCD-local decompositions: a group's workgroups (one per CU) all on one XCD, so that the hidden state is handed
+      // over through that XCD's L2 (a hand-over between XCDs goes through memory and takes about twice as long).  A group
+      // needs G = n / (4 MT) CUs of the XCD; the launch's groups -- those of all `count` problems -- are dealt to the
+      // XCDs, floor(CUs per XCD / G) to each.  Fewer rows per group mean fewer bytes for every CU to fetch per step, so
+      // the batch is split into as many groups as the device holds.
+      auto search_local = [&]() {
+        Cand best;
+        const long env_local = env_long("RTN_LSTM2_LOCAL", -1);  // 0: never, 1: whenever feasible, default: by estimate
+        if (env_local == 0 || env_kernel == 1 || KSMAX == 0 || di.xcds < 1) return best;
+        const int cu_x = di.cus / di.xcds;
+        for (int MT : {1, 2, 4, 8}) {
+          if (env_mt && MT != env_mt) continue;
+          if ((n / 4) % MT) continue;
+          const int G = n / (4 * MT);
+          if (G > cu_x) continue;
+          if (MT * KSMAX > (KSMAX == 16 ? 32 : 64) || (MT == 8 && KSMAX != 8)) continue;
+          const int capacity = di.xcds * (cu_x / G) / std::max(count, 1);  // groups per problem
+          if (capacity < 1) continue;
+          int groups = std::min(capacity, B);
+          if (env_groups) groups = (int)std::min<long>(env_groups, groups);
+          const int Bg = (B + groups - 1) / groups;
+          groups = (B + Bg - 1) / Bg;
+          if ((Bg + 15) / 16 > 4) continue;
+          const int NT = round_nt((Bg + 15) / 16);
+          if (NT * KSMAX > 32 || MT * NT > 8) continue;
+          const bool half = Bg <= 8 && NT == 1 && MT % 2 == 0 && !env_long("RTN_LSTM2_NO_HALF", 0);
+          const size_t lds = (size_t)regw_lds((int)es, MT, NT).total;
+          if (lds > di.lds_per_wg) continue;
+          const double mfma_us = (double)MT * NT * ks * (dtype == RTN_DTYPE_BF16 ? 16 : 128) / 2400.0;
+          const int units = half ? MT / 2 : MT * NT;
+          const int ept = (units + kWaves - 1) / kWaves;
+          // Step time in microseconds, fitted to MI355X measurements (n = 1024 bf16 with 1, 4 and 8 rows per group,
+          // n = 512 float32 with 8): a constant, the MFMA issue time of a wavefront and the KB of hidden state every
+          // CU fetches per step; a second pass of the pointwise part costs about a quarter of a microsecond.
+          const double est = 1.16 + 0.873 * mfma_us + 0.020 * (double)Bg * n * es / 1024.0 + 0.25 * (ept - 1);
+          if (est < best.est) {
+            best.ok = true; best.regw = true; best.local = true; best.half = half;
+            best.est = est; best.KSMAX = KSMAX; best.MT = MT; best.NT = NT; best.groups = groups; best.G = G; best.Bg = Bg;
+            best.lds = lds;
+            const int total_groups = groups * std::max(count, 1);
+            best.grid = di.xcds * G * ((total_groups + di.xcds - 1) / di.xcds);
+          }
+        }
+        return best;
       };
       // The best persistent decomposition for Bq batch rows in one launch.
       auto search = [&](int Bq, bool regw_only) {
@@ -238,10 +290,30 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
         return best;
       };
       Cand chosen = search(B, false);
+      {
+        const Cand loc = search_local();
+        // Local or spread?  Measured on MI355X (bf16 n = 256 ... 1024 with 8 ... 128 rows, one and two problems, float32
+        // n = 256 and 512): the hand-over inside an XCD is worth about 0.1 us per step, 0.25 us more once the spread
+        // plan keeps more than half of the CUs busy (its exchange then competes for the memory fabric) and 0.1 us
+        // more when its groups have more than 64 workgroups; against that stands the longer MFMA chain of a
+        // wavefront when W is packed into the 32 CUs of one XCD (0.87 us per us of MFMA issue time) and a second pass
+        // of the pointwise part (0.25 us).  Problems that would have to share CUs in a spread launch always go local.
+        bool take_local = loc.ok && !(chosen.ok && chosen.regw);
+        if (loc.ok && chosen.ok && chosen.regw) {
+          auto mfma_us = [&](const Cand& c) { return (double)c.MT * c.NT * ks * (dtype == RTN_DTYPE_BF16 ? 16 : 128) / 2400.0; };
+          auto passes = [&](const Cand& c) { return ((c.half ? c.MT / 2 : c.MT * c.NT) + kWaves - 1) / kWaves; };
+          const long long each = (long long)align_up((size_t)(chosen.groups * chosen.G), (size_t)di.xcds);
+          const bool shares = count > 1 && di.cus / each < count;
+          const double cost = 0.873 * (mfma_us(loc) - mfma_us(chosen)) + 0.25 * (passes(loc) - passes(chosen));
+          const double gain = 0.10 + (each * std::max(count, 1) > di.cus / 2 ? 0.25 : 0.0) + (chosen.G > 64 ? 0.10 : 0.0);
+          take_local = shares || cost < gain;
+        }
+        if (loc.ok && (env_long("RTN_LSTM2_LOCAL", -1) == 1 || take_local)) chosen = loc;
+      }
       // A batch too large for one launch of the register kernel runs as several launches in turn, each on a
       // share of the batch groups (the rows of a batch are independent).  That beats the LDS-resident kernel
       // for a few turns and per-step launches (which read W from HBM every step) for some more.
-      if (!(chosen.ok && chosen.regw)) {
+      if (!(chosen.ok && chosen.regw) && !chosen.local) {
         const long env_passes = env_long("RTN_LSTM2_MAX_PASSES", -1);
         const int limit = (int)(env_passes >= 0 ? env_passes : (chosen.ok ? kMaxPassesOverLds : kMaxPassesOverSteps));
         for (int passes = 2; passes <= std::min(limit, B); ++passes) {
@@ -254,6 +326,8 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
       }
       if (chosen.ok) {
         pl.regw = chosen.regw;
+        pl.local = chosen.local;
+        pl.half = chosen.half;
         pl.KSMAX = chosen.KSMAX;
         pl.MT = chosen.MT;
         pl.NT = chosen.NT;
@@ -262,7 +336,7 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
         pl.groups_total = (B + chosen.Bg - 1) / chosen.Bg;
         pl.groups = std::min(chosen.groups, pl.groups_total);
         pl.passes = (pl.groups_total + pl.groups - 1) / pl.groups;
-        pl.grid = pl.groups * chosen.G;
+        pl.grid = chosen.local ? chosen.grid : pl.groups * chosen.G;
         pl.lds_bytes = chosen.lds;
         persistent_ok = true;
       }
@@ -280,6 +354,7 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
       // Per-step launches have no co-residency limit: 4 cells per workgroup, groups of <= 64 rows.
       int MT = 1;
       pl.regw = false;
+      pl.local = pl.half = false;
       pl.KSMAX = 0;
       // A step's launch takes W from memory straight into the matrix cores (every fragment is used once per launch).
       pl.w_direct = env_long("RTN_LSTM2_W_DIRECT", 1) != 0;
@@ -365,7 +440,16 @@ MfmaKernel mfma_kernel(int dtype, int MT, int NT) {
 typedef void (*RegwKernel)(const Lstm2Multi);
 
 template <typename AT>
-RegwKernel regw_kernel_for(int MT, int NT, int KSMAX) {
+RegwKernel regw_kernel_for(int MT, int NT, int KSMAX, bool half) {
+  if (half) {
+#define RTN_CASE(mt, ks) \
+  if (MT == mt && NT == 1 && KSMAX == ks) return &k_lstm2_regw<AT, mt, 1, ks, true>;
+    RTN_CASE(2, 2) RTN_CASE(2, 4) RTN_CASE(2, 8) RTN_CASE(2, 16)
+    RTN_CASE(4, 2) RTN_CASE(4, 4) RTN_CASE(4, 8)
+    RTN_CASE(8, 8)
+#undef RTN_CASE
+    return nullptr;
+  }
 #define RTN_CASE(mt, nt, ks) \
   if (MT == mt && NT == nt && KSMAX == ks) return &k_lstm2_regw<AT, mt, nt, ks>;
   RTN_CASE(1, 1, 2) RTN_CASE(1, 2, 2) RTN_CASE(1, 4, 2)
@@ -384,8 +468,8 @@ RegwKernel regw_kernel_for(int MT, int NT, int KSMAX) {
   return nullptr;
 }
 
-RegwKernel regw_kernel(int dtype, int MT, int NT, int KSMAX) {
-  return dtype == RTN_DTYPE_BF16 ? regw_kernel_for<__bf16>(MT, NT, KSMAX) : regw_kernel_for<float>(MT, NT, KSMAX);
+RegwKernel regw_kernel(int dtype, int MT, int NT, int KSMAX, bool half) {
+  return dtype == RTN_DTYPE_BF16 ? regw_kernel_for<__bf16>(MT, NT, KSMAX, half) : regw_kernel_for<float>(MT, NT, KSMAX, half);
 }
 
 // Kernels that use more than the default LDS limit need the limit raised once per device.
@@ -710,7 +794,7 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
   const void* pk = nullptr;  // the persistent kernel, if any
   int fused = 1;             // problems per cooperative launch
   for (int attempt = 0; pl.kind == kPlanMfma && pl.mode == RTN_MODE_PERSISTENT; ++attempt) {
-    pk = pl.regw ? (const void*)regw_kernel(dtype, pl.MT, pl.NT, pl.KSMAX) : (const void*)mfma_kernel(dtype, pl.MT, pl.NT);
+    pk = pl.regw ? (const void*)regw_kernel(dtype, pl.MT, pl.NT, pl.KSMAX, pl.half) : (const void*)mfma_kernel(dtype, pl.MT, pl.NT);
     if (!pk) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d ks=%d", pl.MT, pl.NT, pl.KSMAX);
     rc = ensure_lds_limit(pk, pl.lds_bytes);
     if (rc != RTN_OK) return rc;
@@ -719,7 +803,9 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, pk, kWgThreads, pl.lds_bytes));
     const long long capacity = (long long)per_cu * device_info().cus;
     if (capacity >= wgs) {
-      if (pl.regw && count > 1 && pl.passes == 1 && !env_long("RTN_LSTM2_NO_FUSE", 0)) {
+      if (pl.local) {
+        fused = plan_count;  // the plan's grid holds the groups of that many problems
+      } else if (pl.regw && count > 1 && pl.passes == 1 && !env_long("RTN_LSTM2_NO_FUSE", 0)) {
         const long long each = (long long)align_up((size_t)wgs, (size_t)device_info().xcds);
         fused = (int)std::min<long long>(std::min(count, kMaxMulti), capacity / each);
         if (fused < 1) fused = 1;
@@ -780,7 +866,13 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     if (p.exchange != kExNoWait) p.exchange = kExDevice;  // no-wait: a timing aid, results invalid (status 2)
     // Device-scope stores take about a microsecond to become visible: a first read issued at once would
     // come back incomplete and cost a second round trip, so it is held back (tuned on MI355X).
-    p.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", 20)));
+    p.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", pl.local ? 6 : 20)));
+    {
+      long dec = env_long("RTN_LSTM2_DELAY_DEC", 8);  // steps per unit of downward adaptation: a power of two
+      int mask = 0;
+      while (2 * (mask + 1) <= dec && mask < 255) mask = 2 * mask + 1;
+      p.delay_dec_mask = mask;
+    }
     p.xcds = device_info().xcds;
     p.sync_policy = (int)env_long("RTN_LSTM2_SYNC", kStoreCoherent | kLoadCoherent);
     if (!((p.sync_policy & (kStoreCoherent | kReleaseFence)) && (p.sync_policy & (kLoadCoherent | kAcquireFence))))
@@ -835,8 +927,10 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
           multi.count = pending;
           multi.grid = pl.grid;
           multi.wgs_each = (int)align_up((size_t)pl.grid, (size_t)device_info().xcds);
+          multi.local = pl.local ? 1 : 0;
+          multi.xcds = device_info().xcds;
           void* args[] = {(void*)&multi};
-          const int wgs = pending == 1 ? pl.grid : multi.wgs_each * pending;
+          const int wgs = (pending == 1 || pl.local) ? pl.grid : multi.wgs_each * pending;
           RTN_HIP(hipLaunchCooperativeKernel(pk, dim3(wgs), dim3(kWgThreads), args, (unsigned)pl.lds_bytes, stream));
           pending = 0;
         }
@@ -991,7 +1085,7 @@ const char* rtn_native_lstm2_describe_multi_plan(int32_t count, int64_t T, int32
   } else {
     snprintf(buf, sizeof(buf), "mode=%s kernel=%s mt=%d nt=%d groups=%d wgs_per_group=%d wgs=%d rows_per_group=%d launches=%d lds=%zu workspace=%zu",
              mode_name(pl.mode),
-             pl.kind == kPlanMfma ? (pl.regw ? "mfma_regw" : "mfma_lds") : (pl.kind == kPlanGeneric ? "generic" : "empty"), pl.MT,
+             pl.kind == kPlanMfma ? (pl.regw ? (pl.local ? (pl.half ? "mfma_regw_xcd_half" : "mfma_regw_xcd") : "mfma_regw") : "mfma_lds") : (pl.kind == kPlanGeneric ? "generic" : "empty"), pl.MT,
              pl.NT, pl.groups, pl.wgs_per_group, (pl.mode == RTN_MODE_PERSISTENT && pl.regw) ? pl.grid : pl.groups * pl.wgs_per_group,
              pl.Bg, pl.passes, pl.lds_bytes,
              (count > 1 || n != n_asked) ? workspace_each(count, T, B, n_asked, dtype, mode) : pl.total);

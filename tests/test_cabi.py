@@ -110,6 +110,25 @@ def test_plan_of_large_batches_padded_widths_and_wide_layers(cabi):
     assert "mode=graph" in text and "kernel=mfma_lds" in text and "lds=4096 " in text, text
 
 
+def test_xcd_local_plans(cabi):
+    """Which shapes put every batch group on one XCD (planned for MI355X's 8 XCDs of 32 CUs when no device is visible)."""
+    pair = lib.describe_multi_plan(2, 1000, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)  # the benchmark pair
+    assert "kernel=mfma_regw_xcd_half mt=8 nt=1 groups=4 wgs_per_group=32 wgs=256 rows_per_group=8 " in pair, pair
+    one = lib.describe_plan(1000, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
+    assert "kernel=mfma_regw_xcd_half" in one and "groups=8 " in one and "rows_per_group=4 " in one, one
+    # a single sequence, and float32 at n = 512, keep W spread over more CUs (fewer MFMAs per wavefront and step)
+    assert "kernel=mfma_regw " in lib.describe_plan(4000, 1, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
+    assert "kernel=mfma_regw " in lib.describe_plan(500, 64, 512, lib.DTYPE_F32, lib.MODE_AUTO)
+    # the environment switch
+    os.environ["RTN_LSTM2_LOCAL"] = "0"
+    try:
+        assert "kernel=mfma_regw " in lib.describe_multi_plan(2, 1000, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
+    finally:
+        del os.environ["RTN_LSTM2_LOCAL"]
+    # a layer whose group does not fit the CUs of one XCD has no such plan
+    assert "_xcd" not in lib.describe_plan(100, 32, 2048, lib.DTYPE_BF16, lib.MODE_AUTO)
+
+
 def test_op_description_contract():
     """Names, order, ndim and host-memory flags of returnn/native_op.py:1054-1068."""
     from returnn_amd import native_op

@@ -223,9 +223,10 @@ def test_cfg3_bf16_full_size():
     want = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, 0, 1, threads=oracle.max_threads())
     got = run_op(p.X, p.W, p.y0, p.c0, p.i, 0, 1, dtype="bf16", mode="auto")
     check_bf16(got, want, "cfg3 full fwd")
-    # the backward call of the pair: properties that need no second oracle pass
+    # the backward call of the pair: against the oracle as well, and through properties
     announce("cfg3 full backward")
     gotb = run_op(p.X, p.W, p.y0, p.c0, p.i, 0, -1, dtype="bf16", mode="auto")
+    check_bf16(gotb, oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, 0, -1, threads=oracle.max_threads()), "cfg3 full bwd")
     m = p.i[:, :, None]
     assert numpy.all(numpy.isfinite(gotb[0])) and numpy.all(numpy.isfinite(gotb[1]))
     assert numpy.array_equal(gotb[0] * (1 - m), numpy.zeros_like(gotb[0]))
