@@ -31,13 +31,23 @@ if _root not in sys.path:
 PEAK_MFMA = {"bf16": 2.5e15, "f32": 157.3e12}  # MI355X dense matrix peaks, FLOP/s
 PEAK_HBM = 8.0e12  # B/s
 
-# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by
-# what the same counter reads for a plain 1 GiB device copy); see profiles/k_lstm2_regw_cfg3_*_hbm_traffic.txt.
-# Keyed by (workload, launches per step, plan as rtn_native_lstm2_describe_plan reports it up to the number of launches).
-MEASURED_TRAFFIC_BYTES = {
-    ("cfg3", 1, "mode=persistent kernel=mfma_regw mt=4 nt=1 groups=2 wgs_per_group=64 wgs=128 rows_per_group=16"): 2524.5e6,
-    ("cfg3", 2, "mode=persistent kernel=mfma_regw mt=2 nt=1 groups=2 wgs_per_group=128 wgs=256 rows_per_group=16"): 1265.2e6,
-}
+# HBM bytes per launch of the dominant kernel are not measured by this script: they come from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs of this same command (each counter scaled by what it reads for a plain 1 GiB device copy), whose
+# summaries sit under profiles/.  profiles/hbm_traffic_per_launch.json lists them by workload, launches per step and
+# plan text; a run whose plan is not in the list reports no traffic figure rather than somebody else's.
+def measured_traffic(workload: str, launches: int, plan: str):
+    """-> (bytes per launch or None, the profile summary the figure is transcribed from or None)"""
+    path = os.path.join(_root, "profiles", "hbm_traffic_per_launch.json")
+    try:
+        with open(path) as f:
+            entries = json.load(f)["entries"]
+    except (OSError, ValueError, KeyError):
+        return None, None
+    key = plan.split(" launches=")[0]
+    for e in entries:
+        if e.get("workload") == workload and e.get("launches_per_step") == launches and e.get("plan") == key:
+            return float(e["bytes_per_launch"]), e.get("source")
+    return None, None
 
 
 def algorithmic_bytes_per_unit(n: int, dtype: str) -> int:
@@ -47,25 +57,40 @@ def algorithmic_bytes_per_unit(n: int, dtype: str) -> int:
     return e * 4 * n + e * 4 * n + e * n + 4 * n + 4
 
 
-def achievable_fields(probe_us, rows, n, dtype, T, call_ms):
+def ceiling_fields(probe_us, seq_ms, rows, n, dtype, T, call_ms):
     """
-    The dependency-bound ceiling of the recurrent GEMM: the T steps are sequential, and a step cannot be shorter than
-    one hand-over of the hidden state between the CUs that hold W (``probe_us``: measured with the library's latency
-    probe -- device-scope store, visible on every CU, device-scope load, at a tiny volume) plus the time the whole
-    chip's matrix cores need for the step's GEMM at their peak (``8 n^2`` flops for each of the ``rows`` sequences of
-    a launch).  ``achievable`` is the GEMM rate at that ceiling, ``frac_of_achievable`` = ceiling time / measured time.
+    Two ceilings of the recurrent GEMM next to the nominal matrix peak.
+
+    ``achievable_mfma``: the rate at which the device runs the step's own MFMA sequence when nothing has to come from
+    another workgroup (``seq_ms``: one launch of the library's sequence probe -- the plan's grid, per step the B
+    fragments from LDS, the plan's MFMAs against W in registers, the partial tiles through LDS with one barrier, their
+    sum; no exchange, no streams, no gates), counted in the op's algorithmic flops.  This is the "achievable MFMA
+    roofline" of the decomposition; ``frac_of_achievable_mfma`` = probe time / measured time.
+
+    ``latency_ceiling``: the T steps are sequential, and a step cannot be shorter than one hand-over of the hidden state
+    between the CUs that hold W (``probe_us``: the library's latency probe -- device-scope store, visible on every CU,
+    device-scope load, at a tiny volume) plus the time the whole chip's matrix cores need for the step's GEMM at their
+    peak.  A latency bound, not a roofline: the rate at that bound and ``frac_of_latency_ceiling`` say how far the
+    kernel is from a perfect hand-over.
     """
-    if probe_us is None:
-        return {}
+    out = {}
     step_flops = 8.0 * n * n * rows
-    mfma_us = step_flops / PEAK_MFMA[dtype] * 1e6
-    ceiling_ms = (probe_us + mfma_us) * T * 1e-3
-    return {
-        "handover_latency_us": probe_us,
-        "mfma_peak_us_per_step": mfma_us,
-        "achievable": step_flops * T / (ceiling_ms * 1e-3) / 1e12,
-        "frac_of_achievable": ceiling_ms / call_ms,
-    }
+    if seq_ms is not None:
+        out.update({
+            "mfma_sequence_us_per_step": seq_ms * 1e3 / T,
+            "achievable_mfma": step_flops * T / (seq_ms * 1e-3) / 1e12,
+            "frac_of_achievable_mfma": seq_ms / call_ms,
+        })
+    if probe_us is not None:
+        mfma_us = step_flops / PEAK_MFMA[dtype] * 1e6
+        ceiling_ms = (probe_us + mfma_us) * T * 1e-3
+        out.update({
+            "handover_latency_us": probe_us,
+            "mfma_peak_us_per_step": mfma_us,
+            "latency_ceiling": step_flops * T / (ceiling_ms * 1e-3) / 1e12,
+            "frac_of_latency_ceiling": ceiling_ms / call_ms,
+        })
+    return out
 
 
 def blas_thread_count():
@@ -478,6 +503,9 @@ def bench_gradient(args, dev, cabi):
     units = T * B * len(steps_of)
     flops = 16.0 * n * n * units
     peak = PEAK_MFMA[dtype]
+    bwd_traffic, bwd_traffic_source = measured_traffic(
+        args.workload + " gradient", 1 if (fused or len(steps_of) == 1) else len(steps_of),
+        "persistent kernel, %i problem(s) per launch" % (len(steps_of) if fused else 1))
     result = {
         "metric": "LSTM gradient op timesteps*seqs/sec (T*B/s) at n=%i" % n,
         "value": units * args.steps / elapsed,
@@ -504,10 +532,10 @@ def bench_gradient(args, dev, cabi):
             "peak": peak / 1e12,
             "unit": "TFLOP/s",
             "frac": flops / (call_ms * 1e-3) / peak,
-            # k_lstm2_bwd_regw of the cfg3 pair in one entry, rocprofv3 FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
-            # (profiles/k_lstm2_bwd_regw_cfg3_pair_hbm_traffic.txt); algorithmic: 22 532 B per unit
-            "traffic": 6326.2e6 if (args.workload == "cfg3" and fused and len(steps_of) == 2) else None,
-            "traffic_unit": "bytes per launch of the persistent kernel; algorithmic (read H, DY, C, mask; write DX): %i"
+            "traffic": bwd_traffic,
+            "traffic_source": bwd_traffic_source,
+            "traffic_unit": "bytes per launch of the persistent kernel (transcribed from the profile summary named in traffic_source, "
+            "not measured by this run); algorithmic (read H, DY, C, mask; write DX): %i"
             % (((9 * (2 if dtype == "bf16" else 4) + 4) * n + 4) * units),
             "kernel": "whole gradient call: the persistent k_lstm2_bwd_regw (or one k_bwd_step launch per frame) with the "
             "recurrent GEMM, 8*n^2 flops per unit, then the weight-gradient GEMM in rocBLAS, 8*n^2 flops per unit",
@@ -814,6 +842,23 @@ def main():
     if pe and cabi.rtn_native_lstm2_fwd_status(probe_ws.data_ptr(), stream.cuda_stream) == lib.RTN_OK:
         probe_us = min(a.elapsed_time(b) for a, b in pe[1:]) * 1e3 / probe_rounds
 
+    # The MFMA roofline of the plan's own instruction sequence (no exchange): one launch of the sequence probe, T steps.
+    seq_ms = None
+    seq_ws = torch.empty((1 << 20,), dtype=torch.uint8, device=dev)
+    se = []
+    for _ in range(1 + 3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        rc = cabi.rtn_mfma_sequence_probe(2 if fused else 1, T, B, n, dt_code, T, seq_ws.data_ptr(), seq_ws.numel(), stream.cuda_stream)
+        e1.record(stream)
+        if rc != lib.RTN_OK:
+            se = []
+            break
+        se.append((e0, e1))
+    torch.cuda.synchronize()
+    if se:
+        seq_ms = min(a.elapsed_time(b) for a, b in se[1:])
+
     units_per_step = len(directions) * T * B
     value = units_per_step * args.steps / elapsed
     units_per_launch = units_per_step // launches
@@ -822,6 +867,7 @@ def main():
     peak = PEAK_MFMA[dtype]
     bytes_per_launch = algorithmic_bytes_per_unit(n, dtype) * units_per_launch
     plan = lib.describe_multi_plan(2 if fused else 1, T, B, n, dt_code, mode)
+    traffic, traffic_source = measured_traffic(args.workload, launches, plan)
 
     result = {
         "metric": "LSTM fwd timesteps*seqs/sec (T*B/s) at n=%i" % n,
@@ -855,13 +901,15 @@ def main():
             "peak": peak / 1e12,
             "unit": "TFLOP/s",
             "frac": achieved / peak,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, launches, plan.split(" launches=")[0])),
-            "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE); algorithmic: %i" % bytes_per_launch,
+            "traffic": traffic,
+            "traffic_source": traffic_source,
+            "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, transcribed from the profile summary named in "
+            "traffic_source, not measured by this run); algorithmic: %i" % bytes_per_launch,
             "kernel": "%s (one launch = %i op call(s) = %i units of T*B, 8*n^2 flops each)"
             % ("k_lstm2_regw" if "mfma_regw" in plan else ("k_lstm2_mfma" if "mfma_lds" in plan else "k_step_generic"),
                len(directions) // launches, units_per_launch),
             "launch_ms": call_ms,
-            **achievable_fields(probe_us, units_per_launch // T, n, dtype, T, call_ms),
+            **ceiling_fields(probe_us, seq_ms, units_per_launch // T, n, dtype, T, call_ms),
             "hbm_algorithmic_GBps": bytes_per_launch / (call_ms * 1e-3) / 1e9,
             "hbm_frac": bytes_per_launch / (call_ms * 1e-3) / PEAK_HBM,
         },
@@ -881,7 +929,8 @@ def main():
             "kernel": "k_lstm2_mfma, one launch per step replayed through a graph (one op call = %i launches)" % T,
             "mfma_TFLOPs": achieved / 1e12,
         })
-        for key in ("achievable", "achievable_unit", "frac_of_achievable", "mfma_peak_us_per_step"):
+        for key in ("latency_ceiling", "frac_of_latency_ceiling", "mfma_peak_us_per_step", "achievable_mfma", "frac_of_achievable_mfma",
+                    "mfma_sequence_us_per_step"):
             result["roofline"].pop(key, None)  # they describe the exchange-bound persistent kernel
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, args.cpu_seconds)

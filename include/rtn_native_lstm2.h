@@ -167,6 +167,19 @@ int rtn_native_lstm2_fwd_multi_status(const void* workspace, int32_t count, int6
 int rtn_handover_latency_probe(void* workspace, size_t workspace_bytes, int32_t rounds, void* hip_stream);
 
 /*
+ * Measurement aid, not part of the operator: the matrix-core roofline of the plan's own instruction sequence.  Launches,
+ * on as many workgroups as the persistent plan for `count` problems of this shape uses, `steps` steps of what that
+ * plan's kernel does between the arrival of the hidden state and the pointwise part -- B fragments from LDS, the
+ * plan's MFMAs per wavefront against W fragments in registers, the partial tiles through LDS with one barrier, their
+ * sum -- with nothing exchanged between workgroups, no streams and no gate arithmetic.  The caller times the call and
+ * divides the op's algorithmic flops (8 n^2 per time step and sequence) by it: the rate a kernel of this
+ * decomposition could reach at most.  `workspace`: 1 KiB per workgroup of the plan (256 workgroups at most on MI355X).
+ * RTN_ERR_UNSUPPORTED for decompositions the probe is not built for.  No counterpart in the reference.
+ */
+int rtn_mfma_sequence_probe(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t steps, void* workspace,
+                            size_t workspace_bytes, void* hip_stream);
+
+/*
  * NativeLstm2 gradient.  Replaces the generated body `c_bw_code` (returnn/native_op.py:1288-1464) with
  * `lstm_bwd_kernel` (:1123-1180) and its `affine_raw` GEMMs; the arguments are the ones `grad_input_map`
  * (:1071-1077) hands to the gradient op, minus X, which the computation never reads.
@@ -298,7 +311,7 @@ const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int3
 const char* rtn_native_lstm2_describe_multi_plan(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype,
                                                  int32_t mode);
 
-/* ABI version of this header: 6. */
+/* ABI version of this header: 7. */
 int rtn_native_lstm2_abi_version(void);
 
 #ifdef __cplusplus

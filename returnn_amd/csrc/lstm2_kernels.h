@@ -1240,6 +1240,99 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
 }
 
 
+// Measurement aid: what the matrix cores of the device can do on the step's own instruction sequence when nothing has
+// to come from another workgroup.  Every workgroup of the plan's grid runs `steps` steps of what k_lstm2_regw does
+// between the arrival of h and the pointwise part: the B-operand fragments of its k share from LDS (the same
+// fragments every step: there is no recurrence), MT * NT * KSMAX MFMAs per wavefront against W fragments held in
+// registers, the partial tiles through LDS with the step's one barrier, and their sum in wave order (kept as a running
+// value so that nothing can be dropped).  No exchange, no streams, no pointwise arithmetic.  The time of a launch over
+// the op's algorithmic flops is the MFMA roofline a kernel of this decomposition could reach at most.
+template <typename AT, int MT, int NT, int KSMAX, bool HALF>
+__global__ __launch_bounds__(kWgThreads) void k_mfma_sequence(float* out, int steps) {
+  using E = Elem<AT>;
+  constexpr int TILES = MT * NT;
+  constexpr int UNITS = HALF ? TILES / 2 : TILES;
+  constexpr int EPT = (UNITS + kWaves - 1) / kWaves;
+  extern __shared__ __align__(16) unsigned char smem[];
+  typedef f32x4 RedBuf[kWaves][TILES][64];
+  RedBuf* red = (RedBuf*)smem;                                                // [2]
+  i32x4* Bl = (i32x4*)(smem + 2 * sizeof(RedBuf));                            // [kWaves][KSMAX][NT][64]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // operands: small numbers that differ per lane and slot (their values do not matter, their being there does)
+  i32x4 wreg[MT][KSMAX];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks) {
+      const AT v = (AT)(0.001f * (float)(1 + ((lane + 3 * mt + 5 * ks + 7 * wave) & 15)));
+      AT frag[E::KE];
+#pragma unroll
+      for (int e = 0; e < E::KE; ++e) frag[e] = v;
+      wreg[mt][ks] = __builtin_bit_cast(i32x4, frag);
+    }
+#pragma unroll
+  for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      AT frag[E::KE];
+#pragma unroll
+      for (int e = 0; e < E::KE; ++e) frag[e] = (AT)(0.01f * (float)(1 + ((lane + ks + nt + e) & 7)));
+      Bl[((wave * KSMAX + ks) * NT + nt) * 64 + lane] = __builtin_bit_cast(i32x4, frag);
+    }
+  __syncthreads();
+  f32x4 total = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto step = [&](auto par_tag) {
+    constexpr int PAR = decltype(par_tag)::value;
+    RedBuf& redbuf = red[PAR];
+    i32x4 bf[KSMAX][NT];
+    asm volatile("" ::: "memory");  // read the fragments again every step
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) bf[ks][nt] = Bl[((wave * KSMAX + ks) * NT + nt) * 64 + lane];
+    f32x4 acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+    if (!HALF || (lane & 8) == 0) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) redbuf[wave][mt * NT + nt][lane] = acc[mt][nt];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      if (UNITS % kWaves == 0 || wave + kWaves * j < UNITS) {
+        const int u = wave + kWaves * j;
+        const int e = HALF ? 2 * u + ((lane >> 3) & 1) : u;
+        const int src = HALF ? ((lane & 0x30) | (lane & 7)) : lane;
+        f32x4 part[kWaves];
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) part[w] = redbuf[w][e][src];
+        __builtin_amdgcn_sched_barrier(0);
+        f32x4 g = part[0];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) g += part[w];
+        total += g;
+      }
+    }
+  };
+  for (int s = 0; s < steps; s += 2) {
+    step(IntTag<0>{});
+    if (s + 1 < steps) step(IntTag<1>{});
+  }
+  out[(size_t)blockIdx.x * kWgThreads + tid] = total[0] + total[1] + total[2] + total[3];
+}
+
 // Measurement aid: the latency of handing a value from every workgroup to every other one, the way the persistent
 // kernel hands over the hidden state (device-scope store, device-scope load until the value is there), with nothing
 // else going on: G workgroups on G CUs; per round each stores its 256-byte block of ring buffer round%4 (value =

@@ -1036,6 +1036,23 @@ BwdLayout bwd_layout(int B, int n, int dtype) {
   return l;
 }
 
+typedef void (*SeqKernel)(float*, int);
+template <typename AT>
+SeqKernel seq_kernel_for(int MT, int NT, int KSMAX, bool half) {
+  // the decompositions of the benchmark configurations and their neighbours
+  if (half) {
+    if (MT == 8 && NT == 1 && KSMAX == 8) return &k_mfma_sequence<AT, 8, 1, 8, true>;
+    if (MT == 4 && NT == 1 && KSMAX == 8) return &k_mfma_sequence<AT, 4, 1, 8, true>;
+    if (MT == 4 && NT == 1 && KSMAX == 4) return &k_mfma_sequence<AT, 4, 1, 4, true>;
+    return nullptr;
+  }
+  if (MT == 8 && NT == 1 && KSMAX == 8) return &k_mfma_sequence<AT, 8, 1, 8, false>;
+  if (MT == 4 && NT == 1 && KSMAX == 8) return &k_mfma_sequence<AT, 4, 1, 8, false>;
+  if (MT == 2 && NT == 1 && KSMAX == 8) return &k_mfma_sequence<AT, 2, 1, 8, false>;
+  if (MT == 1 && NT == 1 && KSMAX == 2) return &k_mfma_sequence<AT, 1, 1, 2, false>;
+  return nullptr;
+}
+
 // Device address of this GPU's copy of `scratch`: asked of the runtime once per device, with that device current.
 int static_scratch(void** out) {
   static std::mutex mu;
@@ -1061,7 +1078,7 @@ using namespace rtn;
 
 extern "C" {
 
-int rtn_native_lstm2_abi_version(void) { return 6; }
+int rtn_native_lstm2_abi_version(void) { return 7; }
 
 const char* rtn_last_error(void) { return g_last_error.c_str(); }
 
@@ -1155,6 +1172,34 @@ int rtn_handover_latency_probe(void* workspace, size_t workspace_bytes, int32_t 
   unsigned long long ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);
   void* args[] = {(void*)&ring, (void*)&status, (void*)&g, (void*)&rnd, (void*)&ticks};
   RTN_HIP(hipLaunchCooperativeKernel((const void*)k_handover_latency, dim3(G), dim3(kWgThreads), args, 0, stream));
+  return RTN_OK;
+}
+
+int rtn_mfma_sequence_probe(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t steps, void* workspace,
+                            size_t workspace_bytes, void* hip_stream) {
+  g_last_error.clear();
+  int rc = check_dims(T, B, n, dtype);
+  if (rc != RTN_OK) return rc;
+  if (count < 1 || steps < 1 || steps > (1 << 24)) return fail(RTN_ERR_ARG, "MFMA sequence probe: count and steps must be positive");
+  Plan pl;
+  std::string why;
+  const int c = std::min<int>(count, kMaxMulti);
+  if (!make_plan(T, B, n, dtype, RTN_MODE_PERSISTENT, false, &pl, &why, 2, c) || !pl.regw)
+    return fail(RTN_ERR_UNSUPPORTED, "MFMA sequence probe: the shape has no persistent register-kernel plan (%s)", why.c_str());
+  SeqKernel k = dtype == RTN_DTYPE_BF16 ? seq_kernel_for<__bf16>(pl.MT, pl.NT, pl.KSMAX, pl.half) : seq_kernel_for<float>(pl.MT, pl.NT, pl.KSMAX, pl.half);
+  if (!k) return fail(RTN_ERR_UNSUPPORTED, "MFMA sequence probe: no build for mt=%d nt=%d ks=%d", pl.MT, pl.NT, pl.KSMAX);
+  // the workgroups that do the plan's work: an XCD-local grid is dealt over all XCDs and part of it may leave at once
+  const int wgs = pl.local ? c * pl.groups * pl.wgs_per_group : (c == 1 ? pl.grid : pl.grid * c);
+  const size_t need = (size_t)wgs * kWgThreads * sizeof(float);
+  if (!workspace || workspace_bytes < need) return fail(RTN_ERR_WORKSPACE, "MFMA sequence probe: workspace of %zu bytes needed", need);
+  if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "MFMA sequence probe: workspace must be 16-byte aligned");
+  const size_t lds = (size_t)2 * kWaves * pl.MT * pl.NT * kTileBytes + (size_t)kWaves * pl.KSMAX * pl.NT * kTileBytes;
+  rc = ensure_lds_limit((const void*)k, lds);
+  if (rc != RTN_OK) return rc;
+  float* out = (float*)workspace;
+  int st = steps;
+  void* args[] = {(void*)&out, (void*)&st};
+  RTN_HIP(hipLaunchKernel((const void*)k, dim3((unsigned)wgs), dim3(kWgThreads), args, lds, (hipStream_t)hip_stream));
   return RTN_OK;
 }
 

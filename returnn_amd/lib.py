@@ -31,7 +31,7 @@ MODE_PERSISTENT = 1
 MODE_GRAPH = 2
 MODE_STEPWISE = 3
 # The ABI version the structs and argument lists below were written for (rtn_native_lstm2_abi_version()).
-EXPECTED_ABI = 6
+EXPECTED_ABI = 7
 
 MODES = {"auto": MODE_AUTO, "persistent": MODE_PERSISTENT, "graph": MODE_GRAPH, "stepwise": MODE_STEPWISE}
 
@@ -45,6 +45,7 @@ SYMBOLS = (
     "rtn_native_lstm2_fwd_multi_workspace_bytes",
     "rtn_native_lstm2_fwd_multi_status",
     "rtn_handover_latency_probe",
+    "rtn_mfma_sequence_probe",
     "rtn_native_lstm2_bwd",
     "rtn_native_lstm2_bwd_workspace_bytes",
     "rtn_native_lstm2_bwd_multi",
@@ -173,6 +174,8 @@ def load() -> ctypes.CDLL:
         lib.rtn_lstm_low_mem_fwd.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, vp]
         lib.rtn_lstm_low_mem_fwd_workspace_bytes.restype = sz
         lib.rtn_lstm_low_mem_fwd_workspace_bytes.argtypes = [i64, i32, i32, i32, i32, i32]
+        lib.rtn_mfma_sequence_probe.restype = ctypes.c_int
+        lib.rtn_mfma_sequence_probe.argtypes = [i32, i64, i32, i32, i32, i32, vp, sz, vp]
         lib.rtn_handover_latency_probe.restype = ctypes.c_int
         lib.rtn_handover_latency_probe.argtypes = [vp, sz, i32, vp]
         lib.rtn_native_lstm2_last_output.restype = ctypes.c_int

@@ -126,6 +126,40 @@ def test_decompositions(mt, groups, kernel):
             assert numpy.array_equal(a, b)
 
 
+@pytest.mark.parametrize("count,T,B,n,dtype", [(2, 1000, 32, 1024, "bf16"), (1, 1000, 32, 1024, "bf16"), (1, 4000, 1, 1024, "bf16"), (1, 500, 64, 512, "f32")])
+def test_mfma_sequence_probe(count, T, B, n, dtype):
+    """The roofline probe (the plan's MFMA sequence without any exchange) runs on the plan's grid, is faster per step
+    than the op itself, refuses bad arguments, and leaves the op's results as they were."""
+    announce("mfma sequence probe", count, T, B, n, dtype)
+    get_op()
+    cabi = lib.load()
+    dt = lib.DTYPE_BF16 if dtype == "bf16" else lib.DTYPE_F32
+    ws = torch.empty((1 << 20,), dtype=torch.uint8, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    p = random_problem(9, 24, B, n)
+    before = run_raw(*p, 0, 1, dtype=dtype, mode="persistent")
+    assert before[0] == 0 and before[1] == 0
+    steps = 400
+    times = []
+    for _ in range(3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        lib.check(cabi.rtn_mfma_sequence_probe(count, T, B, n, dt, steps, ws.data_ptr(), ws.numel(), stream))
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1) * 1e3 / steps)
+    us = min(times)
+    print("MFMA sequence: %.3f us per step for %s" % (us, lib.describe_multi_plan(count, T, B, n, dt, lib.MODE_PERSISTENT)[:100]))
+    assert 0.01 < us < 3.0
+    assert cabi.rtn_mfma_sequence_probe(count, T, B, n, dt, steps, ws.data_ptr(), 64, stream) == lib.RTN_ERR_WORKSPACE
+    assert cabi.rtn_mfma_sequence_probe(count, T, B, n, dt, 0, ws.data_ptr(), ws.numel(), stream) == lib.RTN_ERR_ARG
+    assert cabi.rtn_mfma_sequence_probe(1, 100, 8, 4096, lib.DTYPE_BF16, 10, ws.data_ptr(), ws.numel(), stream) == lib.RTN_ERR_UNSUPPORTED
+    after = run_raw(*p, 0, 1, dtype=dtype, mode="persistent")
+    assert after[0] == 0 and after[1] == 0
+    for a, b in zip(before[2], after[2]):
+        assert numpy.array_equal(a, b)
+
+
 def test_handover_latency_probe():
     """The latency probe (a measurement aid of the library) runs to completion within its bounded waits, refuses bad
     arguments, and the op is still right afterwards."""
