@@ -50,9 +50,16 @@ extern "C" {
 /* Execution mode.
  * AUTO:       PERSISTENT when the shape and device allow it and the stream is not
  *             being captured, else GRAPH.
- * PERSISTENT: one cooperative kernel runs all time steps; the recurrent weights stay
- *             on chip and the workgroups exchange the hidden state through the
- *             workspace with a per-step flag barrier.
+ * PERSISTENT: one cooperative kernel runs all time steps.  Where the device's registers hold
+ *             the recurrent weights (the usual case) every workgroup keeps its slice of W
+ *             in registers and the workgroups hand the hidden state over through a ring
+ *             of buffers in the workspace that validates itself (a word that still holds
+ *             the "not yet written" pattern is read again): no barrier and no flags.
+ *             Wider layers fall back to a kernel that keeps W in LDS and separates
+ *             the steps with a flag wait.  Every wait is bounded: when one expires the
+ *             status word of the workspace is set, the kernel still ends, and NaN is
+ *             written into d and the last visited frame of Y (Dy0 and Dc0 in the gradient),
+ *             so that a caller who never asks for the status sees non-finite results.
  * GRAPH:      one kernel launch per time step; outside stream capture the launches
  *             are replayed through a library-owned hipGraph, under capture they are
  *             recorded into the caller's graph.

@@ -557,13 +557,17 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   gemm(frame(F - 1));
   RTN_BTRACE_ADD(7, (unsigned long long)delay)
   RTN_BTRACE_FLUSH()
+  // After a wait that ran into its bound the gradients are wrong without looking it: the workgroups that see the mark
+  // hand out NaN, so that a caller who never asks for the status still finds a non-finite gradient.
+  const bool expired = wait_expired(q.status);
+  const float nan = __builtin_nanf("");
 #pragma unroll
   for (int j = 0; j < PT; ++j) {
     if (act[j]) {
-      E::store(q.Dy0, idx[j], dyw[j]);
-      p.Dc0[idx[j]] = dc[j];
+      E::store(q.Dy0, idx[j], expired ? nan : dyw[j]);
+      p.Dc0[idx[j]] = expired ? nan : dc[j];
 #pragma unroll
-      for (int gq = 0; gq < 4; ++gq) E::store(p.dx0, io[j] + (long long)gq * n, dx0[j][gq]);
+      for (int gq = 0; gq < 4; ++gq) E::store(p.dx0, io[j] + (long long)gq * n, expired ? nan : dx0[j][gq]);
     }
   }
 }

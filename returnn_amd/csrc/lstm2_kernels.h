@@ -5,8 +5,11 @@
 // (returnn/native_op.cpp:1032-1067).  The structure does not: the recurrent GEMM, the gate
 // non-linearities, the cell update and the mask are one fused step, the cell state and
 // the last valid output of every (sequence, cell) live in registers of the thread that
-// owns that pair, and in the persistent kernel the recurrent weights stay in LDS for
-// all time steps.
+// owns that pair, and in the persistent kernel of the default plan every workgroup keeps
+// its slice of the recurrent weights in registers (as MFMA A-operand fragments) for all
+// time steps.  The older kernel (k_lstm2_mfma), kept for layers too wide for that and for
+// per-step launches, holds its slice in LDS for the steps of one launch, or takes the
+// fragments straight from memory where LDS cannot hold them.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -95,6 +98,16 @@ struct Act<__bf16> {
 };
 
 // Frame visited at step s.
+// True once a bounded wait of the launch has expired (status word 1; 2 marks a measurement run, which is not an error).
+__device__ __forceinline__ bool wait_expired(const unsigned* status) {
+  return __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1u;
+}
+// A 32-bit word full of quiet NaNs of the activation type.
+template <typename AT>
+constexpr unsigned kNanWords = 0x7FC00000u;
+template <>
+constexpr unsigned kNanWords<__bf16> = 0x7FC07FC0u;
+
 __device__ __forceinline__ long long frame_of(const Lstm2Params& p, int s) {
   return (long long)p.first + (long long)s * p.step;
 }
@@ -551,9 +564,17 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
   }
 
   if (s_end == p.nsteps) {
+    // after a wait that ran into its bound: NaN as the final cell state and in the last visited frame of Y
+    const bool expired = wait_expired(p.status);
+    const long long t_last = frame_of(p, p.nsteps - 1);
 #pragma unroll
-    for (int j = 0; j < EPT; ++j)
-      if (e_valid[j]) p.d[(long long)(b_base + e_b[j]) * n + e_cell[j]] = c_state[j];
+    for (int j = 0; j < EPT; ++j) {
+      if (e_valid[j]) {
+        const long long bc = (long long)(b_base + e_b[j]) * n + e_cell[j];
+        p.d[bc] = expired ? __builtin_nanf("") : c_state[j];
+        if (expired) E::store(p.Y, t_last * bn + bc, __builtin_nanf(""));
+      }
+    }
   }
 }
 
@@ -677,6 +698,7 @@ struct Chunk<16> {
   static __device__ __forceinline__ T load(__amdgpu_buffer_rsrc_t rs, unsigned off) {
     return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, 0));
   }
+  static __device__ __forceinline__ T fill(unsigned word) { return T{(int)word, (int)word, (int)word, (int)word}; }
   static __device__ __forceinline__ void store(T v, __amdgpu_buffer_rsrc_t rs, unsigned off) {
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v), rs, off, 0, 0);
   }
@@ -687,6 +709,7 @@ struct Chunk<8> {
   static __device__ __forceinline__ T load(__amdgpu_buffer_rsrc_t rs, unsigned off) {
     return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, 0));
   }
+  static __device__ __forceinline__ T fill(unsigned word) { return ((T)word << 32) | word; }
   static __device__ __forceinline__ void store(T v, __amdgpu_buffer_rsrc_t rs, unsigned off) {
     __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(__attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned, v), rs, off, 0, 0);
   }
@@ -1232,11 +1255,19 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     flush_write(nsteps - 2);
   }
   flush_read((nsteps - 1) % 3);
+  // A wait that ran into its bound let the recurrence go on with values that are wrong without looking it.  Whoever
+  // consumes the outputs without asking for the status must still notice: the workgroups that see the mark hand out
+  // NaN as the final cell state and as the last visited frame of Y.
+  const bool expired = wait_expired(p.status);
+  if (expired) {
+#pragma unroll
+    for (int i = 0; i < YCH; ++i) fy[i] = YC::fill(kNanWords<AT>);
+  }
   flush_write(nsteps - 1);
 
 #pragma unroll
   for (int j = 0; j < EPT; ++j)
-    if (e_valid[j]) p.d[(long long)(b_base + e_row[j]) * n + 4 * MT * r + e_cl[j]] = c_state[j];
+    if (e_valid[j]) p.d[(long long)(b_base + e_row[j]) * n + 4 * MT * r + e_cl[j]] = expired ? __builtin_nanf("") : c_state[j];
 }
 
 

@@ -486,59 +486,169 @@ int ensure_lds_limit(const void* k, size_t lds_bytes) {
   return RTN_OK;
 }
 
-// Library-owned graphs of per-step launch sequences, keyed by everything the launches depend on (a byte string).
+// Where a sequence of kernel launches goes: onto a stream, or into a graph under construction (one kernel node per launch,
+// each depending on the one before).  Every kernel of such a sequence takes the call's parameter block by value as its
+// first argument: that is what lets a graph built for one set of buffers be aimed at another set later.
+struct GraphNode {
+  hipGraphNode_t node = nullptr;
+  const void* fn = nullptr;
+  dim3 grid, block;
+  unsigned lds = 0;
+  std::vector<std::vector<char>> args;  // a private copy of every argument
+};
+struct GraphBuild {
+  hipGraph_t graph = nullptr;
+  std::vector<GraphNode> nodes;
+};
+struct LaunchSink {
+  hipStream_t stream = nullptr;
+  GraphBuild* build = nullptr;  // non-null: add kernel nodes to build->graph instead of launching
+};
+
+void node_params(GraphNode& nd, void** ptrs, hipKernelNodeParams* kp) {
+  for (size_t i = 0; i < nd.args.size(); ++i) ptrs[i] = nd.args[i].data();
+  memset(kp, 0, sizeof(*kp));
+  kp->func = const_cast<void*>(nd.fn);
+  kp->gridDim = nd.grid;
+  kp->blockDim = nd.block;
+  kp->sharedMemBytes = nd.lds;
+  kp->kernelParams = ptrs;
+  kp->extra = nullptr;
+}
+
+constexpr size_t kMaxKernelArgs = 8;
+
+template <typename... P, size_t... I>
+int enqueue_impl(LaunchSink& sink, void (*k)(P...), dim3 grid, dim3 block, size_t lds, std::tuple<std::decay_t<P>...>& vals,
+                 std::index_sequence<I...>) {
+  static_assert(sizeof...(P) <= kMaxKernelArgs, "too many kernel arguments");
+  void* ptrs[kMaxKernelArgs] = {(void*)&std::get<I>(vals)...};
+  if (!sink.build) {
+    RTN_HIP(hipLaunchKernel((const void*)k, grid, block, ptrs, lds, sink.stream));
+    return RTN_OK;
+  }
+  GraphNode nd;
+  nd.fn = (const void*)k;
+  nd.grid = grid;
+  nd.block = block;
+  nd.lds = (unsigned)lds;
+  const size_t sizes[] = {sizeof(std::decay_t<P>)...};
+  for (size_t i = 0; i < sizeof...(P); ++i) nd.args.emplace_back((const char*)ptrs[i], (const char*)ptrs[i] + sizes[i]);
+  void* own[kMaxKernelArgs];
+  hipKernelNodeParams kp;
+  node_params(nd, own, &kp);
+  std::vector<GraphNode>& nodes = sink.build->nodes;
+  hipGraphNode_t before = nodes.empty() ? nullptr : nodes.back().node;
+  RTN_HIP(hipGraphAddKernelNode(&nd.node, sink.build->graph, nodes.empty() ? nullptr : &before, nodes.empty() ? 0 : 1, &kp));
+  nodes.push_back(std::move(nd));
+  return RTN_OK;
+}
+
+// Launch k(args...) on the sink's stream, or append it to the sink's graph.
+template <typename... P, typename... A>
+int enqueue(LaunchSink& sink, void (*k)(P...), dim3 grid, dim3 block, size_t lds, A&&... args) {
+  static_assert(sizeof...(P) == sizeof...(A), "argument count does not match the kernel's");
+  std::tuple<std::decay_t<P>...> vals(std::forward<A>(args)...);  // converted to the kernel's parameter types
+  return enqueue_impl<P...>(sink, k, grid, block, lds, vals, std::index_sequence_for<P...>{});
+}
+
+// Library-owned graphs of per-step launch sequences.  The key holds what fixes the structure of the sequence (shape,
+// element type, plan, device): no addresses.  A graph whose kernel nodes carry another parameter block than the call's
+// (other buffers, same shape) gets the new block written into every node of its executable form before the launch.
 struct GraphEntry {
   std::string key;
-  hipGraph_t graph;
-  hipGraphExec_t exec;
-};
-std::mutex g_graph_mu;
-std::list<GraphEntry> g_graphs;  // most recently used first
-constexpr size_t kMaxGraphs = 8;
-
-// Launches the graph recorded for `key`; records it first (on a private stream, by calling `record`) if there is none.
-template <typename Record>
-int replay_graph(const std::string& key, hipStream_t stream, Record record) {
-  std::lock_guard<std::mutex> lock(g_graph_mu);
-  for (auto it = g_graphs.begin(); it != g_graphs.end(); ++it) {
-    if (it->key == key) {
-      g_graphs.splice(g_graphs.begin(), g_graphs, it);
-      RTN_HIP(hipGraphLaunch(g_graphs.front().exec, stream));
-      return RTN_OK;
-    }
-  }
-  // Record the launches on a private stream; nothing runs until the graph is launched.
-  hipStream_t cap = nullptr;
-  RTN_HIP(hipStreamCreateWithFlags(&cap, hipStreamNonBlocking));
+  std::string block;  // the parameter block the executable graph's nodes carry now
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
-  int rc = RTN_OK;
-  hipError_t e = hipStreamBeginCapture(cap, hipStreamCaptureModeThreadLocal);
-  if (e == hipSuccess) {
-    rc = record(cap);
-    hipError_t e2 = hipStreamEndCapture(cap, &graph);
-    if (rc == RTN_OK && e2 != hipSuccess) rc = fail(RTN_ERR_HIP, "NativeLstm2: hipStreamEndCapture: %s", hipGetErrorString(e2));
-  } else {
-    rc = fail(RTN_ERR_HIP, "NativeLstm2: hipStreamBeginCapture: %s", hipGetErrorString(e));
+  std::vector<GraphNode> nodes;
+  hipEvent_t last = nullptr;  // recorded behind every launch: the executable graph may be destroyed once it has completed
+};
+std::mutex g_graph_mu;
+std::list<GraphEntry> g_graphs;   // most recently used first
+std::list<GraphEntry> g_retired;  // dropped from g_graphs, possibly still running
+constexpr size_t kMaxGraphs = 8;
+long long g_graph_records = 0, g_graph_retargets = 0, g_graph_destroyed = 0;
+
+void destroy_entry(GraphEntry& e) {
+  if (e.exec) (void)hipGraphExecDestroy(e.exec);
+  if (e.graph) (void)hipGraphDestroy(e.graph);
+  if (e.last) (void)hipEventDestroy(e.last);
+  ++g_graph_destroyed;
+}
+
+void sweep_retired() {  // g_graph_mu held
+  for (auto it = g_retired.begin(); it != g_retired.end();) {
+    if (hipEventQuery(it->last) == hipSuccess) {
+      destroy_entry(*it);
+      it = g_retired.erase(it);
+    } else {
+      (void)hipGetLastError();  // hipErrorNotReady is not an error of ours
+      ++it;
+    }
   }
-  (void)hipStreamDestroy(cap);
+}
+
+int launch_entry(GraphEntry& e, hipStream_t stream) {
+  RTN_HIP(hipGraphLaunch(e.exec, stream));
+  RTN_HIP(hipEventRecord(e.last, stream));
+  return RTN_OK;
+}
+
+// Launches the graph kept for `key` with the parameter block [block, block + bytes) in the first argument of every
+// kernel node; builds the graph first (by calling `record` with a sink that collects nodes) if there is none.
+template <typename Record>
+int replay_graph(const std::string& key, const void* block, size_t bytes, hipStream_t stream, Record record) {
+  std::lock_guard<std::mutex> lock(g_graph_mu);
+  sweep_retired();
+  for (auto it = g_graphs.begin(); it != g_graphs.end(); ++it) {
+    if (it->key != key) continue;
+    g_graphs.splice(g_graphs.begin(), g_graphs, it);
+    GraphEntry& e = g_graphs.front();
+    if (e.block.size() != bytes || memcmp(e.block.data(), block, bytes) != 0) {
+      // Other buffers than last time.  Launches of the executable graph that are already queued keep the arguments
+      // they were queued with; the update only shows in launches made after it.
+      for (GraphNode& nd : e.nodes) {
+        memcpy(nd.args[0].data(), block, bytes);
+        void* ptrs[kMaxKernelArgs];
+        hipKernelNodeParams kp;
+        node_params(nd, ptrs, &kp);
+        RTN_HIP(hipGraphExecKernelNodeSetParams(e.exec, nd.node, &kp));
+      }
+      e.block.assign((const char*)block, bytes);
+      ++g_graph_retargets;
+    }
+    return launch_entry(e, stream);
+  }
+  GraphEntry e;
+  e.key = key;
+  e.block.assign((const char*)block, bytes);
+  GraphBuild build;
+  RTN_HIP(hipGraphCreate(&build.graph, 0));
+  LaunchSink sink;
+  sink.build = &build;
+  int rc = record(sink);
+  for (GraphNode& nd : build.nodes)
+    if (rc == RTN_OK && (nd.args.empty() || nd.args[0].size() != bytes))
+      rc = fail(RTN_ERR_HIP, "NativeLstm2: a kernel recorded into a library graph does not take the parameter block first");
   if (rc != RTN_OK) {
-    if (graph) (void)hipGraphDestroy(graph);
+    (void)hipGraphDestroy(build.graph);
     return rc;
   }
-  e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-  if (e != hipSuccess) {
-    (void)hipGraphDestroy(graph);
-    return fail(RTN_ERR_HIP, "NativeLstm2: hipGraphInstantiate: %s", hipGetErrorString(e));
+  e.graph = build.graph;
+  e.nodes = std::move(build.nodes);
+  hipError_t err = hipGraphInstantiate(&e.exec, e.graph, nullptr, nullptr, 0);
+  if (err == hipSuccess) err = hipEventCreateWithFlags(&e.last, hipEventDisableTiming);
+  if (err != hipSuccess) {
+    destroy_entry(e);
+    return fail(RTN_ERR_HIP, "NativeLstm2: building a graph of %zu launches: %s", e.nodes.size(), hipGetErrorString(err));
   }
-  g_graphs.push_front(GraphEntry{key, graph, exec});
+  ++g_graph_records;
+  g_graphs.push_front(std::move(e));
   while (g_graphs.size() > kMaxGraphs) {
-    (void)hipGraphExecDestroy(g_graphs.back().exec);
-    (void)hipGraphDestroy(g_graphs.back().graph);
-    g_graphs.pop_back();
+    // may still be running on some stream: parked until the event behind its last launch has completed
+    g_retired.splice(g_retired.end(), g_graphs, std::prev(g_graphs.end()));
   }
-  RTN_HIP(hipGraphLaunch(exec, stream));
-  return RTN_OK;
+  return launch_entry(g_graphs.front(), stream);
 }
 
 template <typename T>
@@ -546,33 +656,48 @@ void key_append(std::string* key, const T& v) {
   key->append(reinterpret_cast<const char*>(&v), sizeof(T));
 }
 
-int launch_steps(const Lstm2Params& p, const Plan& pl, int dtype, hipStream_t stream) {
+int launch_steps(const Lstm2Params& p, const Plan& pl, int dtype, LaunchSink& sink) {
   if (pl.kind == kPlanMfma) {
     MfmaKernel k = mfma_kernel(dtype, pl.MT, pl.NT);
     const dim3 grid(pl.groups * pl.wgs_per_group), block(kWgThreads);
-    for (int s = 0; s < p.nsteps; ++s) hipLaunchKernelGGL(k, grid, block, pl.lds_bytes, stream, p, s, s + 1);
+    for (int s = 0; s < p.nsteps; ++s) {
+      const int rc = enqueue(sink, k, grid, block, pl.lds_bytes, p, s, s + 1);
+      if (rc != RTN_OK) return rc;
+    }
   } else {
     const long long bn = (long long)p.B * p.n;
     const dim3 grid((unsigned)((bn + 255) / 256)), block(256);
     for (int s = 0; s < p.nsteps; ++s) {
-      if (dtype == RTN_DTYPE_BF16)
-        hipLaunchKernelGGL(k_step_generic<__bf16>, grid, block, 0, stream, p, s);
-      else
-        hipLaunchKernelGGL(k_step_generic<float>, grid, block, 0, stream, p, s);
+      const int rc = dtype == RTN_DTYPE_BF16 ? enqueue(sink, k_step_generic<__bf16>, grid, block, 0, p, s)
+                                             : enqueue(sink, k_step_generic<float>, grid, block, 0, p, s);
+      if (rc != RTN_OK) return rc;
     }
   }
-  RTN_HIP(hipGetLastError());
   return RTN_OK;
+}
+
+int launch_steps(const Lstm2Params& p, const Plan& pl, int dtype, hipStream_t stream) {
+  LaunchSink sink;
+  sink.stream = stream;
+  return launch_steps(p, pl, dtype, sink);
 }
 
 int launch_steps_graph(const Lstm2Params& p, const Plan& pl, int dtype, hipStream_t stream) {
   std::string key("fwd");
   int dev = 0;
   RTN_HIP(hipGetDevice(&dev));
-  key.append(reinterpret_cast<const char*>(&p), sizeof(p));  // the caller zeroed p before filling it in: padding compares equal
+  Lstm2Params shape = p;  // the caller zeroed p before filling it in: padding compares equal
+  shape.X = shape.W = shape.y0 = nullptr;
+  shape.c0 = shape.mask = nullptr;
+  shape.Y = shape.H = nullptr;
+  shape.C = shape.d = nullptr;
+  shape.status = shape.flags = nullptr;
+  shape.hx = shape.Wp = shape.ycarry = nullptr;
+  shape.trace = nullptr;
+  key.append(reinterpret_cast<const char*>(&shape), sizeof(shape));
   key_append(&key, dtype); key_append(&key, pl.MT); key_append(&key, pl.NT); key_append(&key, (int)pl.kind);
   key_append(&key, pl.lds_bytes); key_append(&key, dev);
-  return replay_graph(key, stream, [&](hipStream_t cap) { return launch_steps(p, pl, dtype, cap); });
+  return replay_graph(key, &p, sizeof(p), stream, [&](LaunchSink& sink) { return launch_steps(p, pl, dtype, sink); });
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -1639,52 +1764,50 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     // else 16 (measured: float32 n=1024 B=64 29 us per frame with 16 rows, 35 with 32; 64 rows were never faster).
     int NT = B > 16 ? 2 : 1;
     if (NT > 1 && (long long)(n / 16) * ((B + 16 * NT - 1) / (16 * NT)) < device_info().cus) NT = 1;
-    auto record = [&](hipStream_t st) -> int {
+    auto record = [&](LaunchSink& sink) -> int {
       const dim3 pw_grid((unsigned)((bn + 255) / 256)), pw_block(256);
       const dim3 mm_grid((unsigned)((n / 16) * ((B + 16 * NT - 1) / (16 * NT)))), mm_block(kWgThreads);
+      const bool bf = dtype == RTN_DTYPE_BF16;
       long long t_done = -1;  // frame whose DX still has to go through the GEMM
       for (long long t = end;; t -= step) {
         const bool more = step > 0 ? t >= first : t <= first;
         const bool right = more && (step > 0 ? (t - step >= first) : (t - step <= first));
         const long long prev_t = right ? t - step : -1;
         const long long tt = more ? t : -1;
+        int rc2 = RTN_OK;
         if (mfma) {
-          if (dtype == RTN_DTYPE_BF16) {
-            if (NT == 2)
-              hipLaunchKernelGGL((k_bwd_step<__bf16, 2>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
-            else
-              hipLaunchKernelGGL((k_bwd_step<__bf16, 1>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
-          } else {
-            if (NT == 2)
-              hipLaunchKernelGGL((k_bwd_step<float, 2>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
-            else
-              hipLaunchKernelGGL((k_bwd_step<float, 1>), mm_grid, mm_block, 0, st, p, t_done, tt, prev_t);
-          }
+          void (*k)(Lstm2BwdParams, long long, long long, long long) =
+              bf ? (NT == 2 ? &k_bwd_step<__bf16, 2> : &k_bwd_step<__bf16, 1>) : (NT == 2 ? &k_bwd_step<float, 2> : &k_bwd_step<float, 1>);
+          rc2 = enqueue(sink, k, mm_grid, mm_block, 0, p, t_done, tt, prev_t);
         } else if (more) {
-          if (dtype == RTN_DTYPE_BF16) {
-            hipLaunchKernelGGL(k_bwd_pointwise<__bf16>, pw_grid, pw_block, 0, st, p, t, prev_t);
-            hipLaunchKernelGGL(k_bwd_gemm_dy_generic<__bf16>, pw_grid, pw_block, 0, st, p, t);
-          } else {
-            hipLaunchKernelGGL(k_bwd_pointwise<float>, pw_grid, pw_block, 0, st, p, t, prev_t);
-            hipLaunchKernelGGL(k_bwd_gemm_dy_generic<float>, pw_grid, pw_block, 0, st, p, t);
-          }
+          rc2 = enqueue(sink, bf ? &k_bwd_pointwise<__bf16> : &k_bwd_pointwise<float>, pw_grid, pw_block, 0, p, t, prev_t);
+          if (rc2 == RTN_OK)
+            rc2 = enqueue(sink, bf ? &k_bwd_gemm_dy_generic<__bf16> : &k_bwd_gemm_dy_generic<float>, pw_grid, pw_block, 0, p, t);
         }
+        if (rc2 != RTN_OK) return rc2;
         if (!more) break;
         t_done = t;
       }
-      RTN_HIP(hipGetLastError());
       return RTN_OK;
     };
     if (capturing || env_long("RTN_LSTM2_BWD_NO_GRAPH", 0)) {
-      rc = record(stream);
+      LaunchSink sink;
+      sink.stream = stream;
+      rc = record(sink);
     } else {
       std::string key("bwd");
       int dev = 0;
       RTN_HIP(hipGetDevice(&dev));
-      key.append(reinterpret_cast<const char*>(&p), sizeof(p));  // p was zeroed before it was filled in
+      Lstm2BwdParams shape = p;  // p was zeroed before it was filled in
+      shape.W = shape.H = shape.DY = shape.Wpk = nullptr;
+      shape.c0 = shape.mask = shape.C = nullptr;
+      shape.DX = shape.dx0 = nullptr;
+      shape.dyw = shape.Dc0 = nullptr;
+      key.append(reinterpret_cast<const char*>(&shape), sizeof(shape));
+      key_append(&key, (int)(p.Wpk != nullptr));
       key_append(&key, dtype); key_append(&key, (int)calls[0].start); key_append(&key, step); key_append(&key, dev);
       key_append(&key, (int)mfma); key_append(&key, NT);
-      rc = replay_graph(key, stream, record);
+      rc = replay_graph(key, &p, sizeof(p), stream, record);
     }
     if (rc != RTN_OK) return rc;
   }

@@ -21,6 +21,8 @@ every element; CPU tensors are rejected (no CPU implementation is shipped).
 
 from __future__ import annotations
 
+import collections
+import os
 import sys
 from threading import RLock
 from typing import Any, Dict, Optional
@@ -45,12 +47,16 @@ class OpMaker:
     """
     Registers one op with ``torch.library`` and hands out the ``torch.ops`` callable.
     Cached per op name under a process-wide lock, like the reference's OpMaker (:33-36, :430-447).
+
+    The execution mode belongs to the maker and is fixed in the op it makes: ``mode="auto"`` registers the op under the
+    reference's name (``torch.ops.NativeLstm2.NativeLstm2``), any other mode under ``<name>_<mode>``
+    (``torch.ops.NativeLstm2_stepwise.NativeLstm2_stepwise``), so that ops of different modes can be used side by side,
+    from any thread, and the mode shows in the op's name.
     """
 
     global_lock = RLock()
     op_cache: Dict[str, Any] = {}  # cache_key -> op
     lib_cache: Dict[str, Any] = {}  # cache_key -> torch.library.Library (kept alive)
-    options: Dict[str, Dict[str, Any]] = {}  # cache_key -> run-time options of the device implementation
     log_stream = sys.stdout
 
     def __init__(
@@ -72,15 +78,15 @@ class OpMaker:
         self.name = description.name
         if mode is not None and mode not in _lib.MODES:
             raise ValueError("mode must be one of %r" % sorted(_lib.MODES))
-        self.mode = mode
+        self.mode = mode or "auto"
 
     @property
     def op_name(self) -> str:
-        return self.name
+        return self.name if self.mode == "auto" else "%s_%s" % (self.name, self.mode)
 
     @property
     def cache_key(self) -> str:
-        return self.name
+        return self.op_name
 
     def schema(self) -> str:
         d = self.description
@@ -97,12 +103,15 @@ class OpMaker:
         }.get(self.description.c_abi_fw)
         if impl is None:
             raise NotImplementedError("no gfx950 implementation for op %r" % self.name)
-        return impl
+        mode_code = _lib.MODES[self.mode]
+
+        def _device_impl(*args):
+            return impl(*args, mode=mode_code)
+
+        return _device_impl
 
     def make_op(self):
         with self.global_lock:
-            if self.mode is not None or self.cache_key not in self.options:
-                self.options.setdefault(self.cache_key, {})["mode"] = self.mode or "auto"
             if self.cache_key in self.op_cache:
                 return self.op_cache[self.cache_key]
             impl = self._impl_for()
@@ -245,6 +254,89 @@ def make_op_with_grad(cls, **kwargs):
     return op
 
 
+class NativeOpAborted(RuntimeError):
+    """A bounded wait inside a persistent kernel expired: the results of that call are invalid."""
+
+
+class StatusWatch:
+    """
+    Looks after the status words of the library's workspaces without stalling the stream.
+
+    The persistent kernels bound every wait for another workgroup (2 s of wall clock by default).  A wait that runs
+    into its bound sets the first word of the call's workspace slice to 1 and the workgroups that see it put NaN into
+    results every caller consumes (final cell state, last visited frame of Y; Dy0 and Dc0 of the gradient).  On top of
+    that, every op call here queues a copy of its status words to pinned host memory behind its kernels and records an
+    event; the next op call (or :meth:`poll`) looks at the copies whose event has completed and raises
+    :class:`NativeOpAborted` for a word that is 1.  Nothing waits for the device.
+
+    ``RTN_LSTM2_CHECK_STATUS=1`` in the environment (or ``status_watch.synchronous = True``) makes every op call wait
+    for its own kernels and check at once: the error then names the call that failed, at the price of one stream
+    synchronisation per call.  ``RTN_LSTM2_CHECK_STATUS=0`` switches the watch off.  Under stream capture nothing is
+    queued (a captured copy would be replayed without anybody looking at it); captured calls rely on the NaN marks.
+    """
+
+    SLOTS = 64  # status words per pinned block; a block is reused once its event has completed
+
+    def __init__(self):
+        self.lock = RLock()
+        self.pending = collections.deque()  # (event, host block, number of words, what)
+        self.free_blocks = []
+        self.synchronous: Optional[bool] = None  # None: from the environment, read at each call
+        self.checked = 0  # completed calls looked at so far (for tests)
+
+    def _setting(self) -> str:
+        if self.synchronous is not None:
+            return "1" if self.synchronous else "lazy"
+        return os.environ.get("RTN_LSTM2_CHECK_STATUS", "lazy")
+
+    def after_call(self, what: str, ws: torch.Tensor, count: int, device) -> None:
+        """Queue the look at the status word of each of the ``count`` equal slices of ``ws`` (current device = ``device``)."""
+        setting = self._setting()
+        if setting == "0" or count > self.SLOTS or torch.cuda.is_current_stream_capturing():
+            return
+        each = ws.numel() // count
+        words = ws.view(torch.int32)[: (count - 1) * (each // 4) + 1 : max(each // 4, 1)]
+        with self.lock:
+            block = self.free_blocks.pop() if self.free_blocks else torch.zeros((self.SLOTS,), dtype=torch.int32, pin_memory=True)
+        block[:count].copy_(words, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record(torch.cuda.current_stream(device))
+        with self.lock:
+            self.pending.append((event, block, count, what))
+        if setting == "1":
+            event.synchronize()
+            self.poll()
+
+    def poll(self) -> None:
+        """Raise for the oldest completed call whose status word says that a wait expired; never blocks."""
+        if torch.cuda.is_current_stream_capturing():
+            return  # (no queries while a capture is under way)
+        failed = None
+        with self.lock:
+            while self.pending and self.pending[0][0].query():
+                _, block, count, what = self.pending.popleft()
+                self.checked += 1
+                if failed is None and any(int(w) == 1 for w in block[:count].tolist()):
+                    failed = what
+                self.free_blocks.append(block)
+        if failed is not None:
+            raise NativeOpAborted(
+                "%s: a bounded wait in the persistent kernel expired (device shared, preempted or paused?); the results of "
+                "that call are invalid.  RTN_LSTM2_TIMEOUT_TICKS sets the bound in 10 ns ticks." % failed
+            )
+
+    def drain(self) -> None:
+        """Wait for every queued look and check it (end of a step, end of the program, tests)."""
+        with self.lock:
+            events = [e for e, _, _, _ in self.pending]
+        for e in events:
+            e.synchronize()
+        self.poll()
+
+
+status_watch = StatusWatch()
+
+
 def _cpu_not_supported(name):
     def _impl(*args):
         raise RuntimeError(
@@ -296,14 +388,14 @@ def _alloc_lstm2_outputs(T, B, n, bf16, device):
     return Y, C, H, d
 
 
-def _native_lstm2_device_impl(X, W, y0, c0, i, start, step):
+def _native_lstm2_device_impl(X, W, y0, c0, i, start, step, *, mode=_lib.MODE_AUTO):
     """``NativeLstm2`` on HIP tensors: normalise the arguments, allocate outputs and scratch, enqueue the library call."""
     (X, W, y0, c0, i), (T, B, n, bf16) = _normalise_lstm2_args(X, W, y0, c0, i)
     device = X.device
     lib = _lib.load()
     dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
-    mode = _lib.MODES[OpMaker.options.get("NativeLstm2", {}).get("mode", "auto")]
     with torch.cuda.device(device):
+        status_watch.poll()
         Y, C, H, d = _alloc_lstm2_outputs(T, B, n, bf16, device)
         ws_bytes = int(lib.rtn_native_lstm2_fwd_workspace_bytes(T, B, n, dtype, mode))
         ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=device)
@@ -313,26 +405,27 @@ def _native_lstm2_device_impl(X, W, y0, c0, i, start, step):
             Y.data_ptr(), C.data_ptr(), H.data_ptr(), d.data_ptr(), T, B, n, dtype, mode,
             ws.data_ptr(), ws.numel(), stream,
         )  # fmt: skip
-    _lib.check(rc)
+        _lib.check(rc)
+        if T * B * n > 0:  # (an empty problem does not touch its workspace)
+            status_watch.after_call("NativeLstm2", ws, 1, device)
     # The workspace goes back to the caching allocator here; the allocator keeps it out of other
     # streams' hands until the work queued on this stream has passed it (stream-ordered reuse).
     return Y, C, H, d
 
 
-def _act_and_mode(first: torch.Tensor, op_name: str):
+def _act_and_dtype(first: torch.Tensor):
     bf16 = first.dtype == torch.bfloat16
     act = torch.bfloat16 if bf16 else torch.float32
     dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
-    mode = _lib.MODES[OpMaker.options.get(op_name, {}).get("mode", "auto")]
-    return act, dtype, mode
+    return act, dtype
 
 
-def _lstm_generic_base_device_impl(Z, V_h, c, i):
+def _lstm_generic_base_device_impl(Z, V_h, c, i, *, mode=_lib.MODE_AUTO):
     """``LstmGenericBase`` forward on HIP tensors (returnn/native_op.py:333-523)."""
     for t, info in zip((Z, V_h, c, i), native_op.LstmGenericBase.in_info):
         _check_ndim(t, info)
     device = Z.device
-    act, dtype, mode = _act_and_mode(Z, "LstmGenericBase")
+    act, dtype = _act_and_dtype(Z)
     Z, V_h = (t.to(act).contiguous() for t in (Z, V_h))
     c, i = (t.to(torch.float32).contiguous() for t in (c, i))
     T, B = i.shape
@@ -344,6 +437,7 @@ def _lstm_generic_base_device_impl(Z, V_h, c, i):
             raise RuntimeError("LstmGenericBase: %s is on %s but Z is on %s" % (name, t.device, device))
     lib = _lib.load()
     with torch.cuda.device(device):
+        status_watch.poll()
         Y = torch.empty((T, B, n), dtype=act, device=device)
         H = torch.empty((T, B, 4 * n), dtype=act, device=device)
         d = torch.empty((B, n), dtype=torch.float32, device=device)
@@ -352,16 +446,18 @@ def _lstm_generic_base_device_impl(Z, V_h, c, i):
             Z.data_ptr(), V_h.data_ptr(), c.data_ptr(), i.data_ptr(), Y.data_ptr(), H.data_ptr(), d.data_ptr(), T, B, n, dtype, mode,
             ws.data_ptr(), ws.numel(), torch.cuda.current_stream(device).cuda_stream,
         )  # fmt: skip
-    _lib.check(rc)
+        _lib.check(rc)
+        if T * B * n > 0:  # (an empty problem does not touch its workspace)
+            status_watch.after_call("LstmGenericBase", ws, 1, device)
     return Y, H, d
 
 
-def _lstm_low_mem_device_impl(X, W, b, y0, c0, i, start, step):
+def _lstm_low_mem_device_impl(X, W, b, y0, c0, i, start, step, *, mode=_lib.MODE_AUTO):
     """``LstmLowMem`` forward on HIP tensors (returnn/native_op.py:577-836)."""
     for t, info in zip((X, W, b, y0, c0, i), native_op.LstmLowMem.in_info):
         _check_ndim(t, info)
     device = X.device
-    act, dtype, mode = _act_and_mode(X, "LstmLowMem")
+    act, dtype = _act_and_dtype(X)
     X, W, b, y0 = (t.to(act).contiguous() for t in (X, W, b, y0))
     c0, i = (t.to(torch.float32).contiguous() for t in (c0, i))
     T, B = i.shape
@@ -374,6 +470,7 @@ def _lstm_low_mem_device_impl(X, W, b, y0, c0, i, start, step):
             raise RuntimeError("LstmLowMem: %s is on %s but X is on %s" % (name, t.device, device))
     lib = _lib.load()
     with torch.cuda.device(device):
+        status_watch.poll()
         Y = torch.empty((T, B, n), dtype=act, device=device)
         C = torch.empty((T, B, n), dtype=torch.float32, device=device)
         d = torch.empty((B, n), dtype=torch.float32, device=device)
@@ -383,7 +480,9 @@ def _lstm_low_mem_device_impl(X, W, b, y0, c0, i, start, step):
             Y.data_ptr(), C.data_ptr(), d.data_ptr(), T, B, n_in, n, dtype, mode, ws.data_ptr(), ws.numel(),
             torch.cuda.current_stream(device).cuda_stream,
         )  # fmt: skip
-    _lib.check(rc)
+        _lib.check(rc)
+        if T * B * n > 0:  # (an empty problem does not touch its workspace)
+            status_watch.after_call("LstmLowMem", ws, 1, device)
     return Y, C, d
 
 
@@ -394,7 +493,7 @@ def native_lstm2_multi(calls, *, mode: Optional[str] = None):
     device can hold them together they run in a single launch and overlap.
 
     :param calls: sequence of ``(X, W, y0, c0, i, start, step)``, all with the same T, B, n and element type
-    :param mode: as for :class:`OpMaker`; default: the mode the op was made with
+    :param mode: as for :class:`OpMaker`; default "auto"
     :return: list of ``(Y, C, H, d)``
     """
     calls = list(calls)
@@ -413,11 +512,12 @@ def native_lstm2_multi(calls, *, mode: Optional[str] = None):
         raise RuntimeError("NativeLstm2: this build implements the op for HIP (MI355X) tensors only; got CPU tensors.")
     T, B, n, bf16 = shape
     dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
-    mode_code = _lib.MODES[mode or OpMaker.options.get("NativeLstm2", {}).get("mode", "auto")]
+    mode_code = _lib.MODES[mode or "auto"]
     count = len(calls)
     arr = (_lib.Lstm2Call * count)()
     outs = []
     with torch.cuda.device(device):
+        status_watch.poll()
         for k, ((X, W, y0, c0, i), c) in enumerate(zip((t for t, _ in norm), calls)):
             Y, C, H, d = _alloc_lstm2_outputs(T, B, n, bf16, device)
             outs.append((Y, C, H, d))
@@ -429,7 +529,9 @@ def native_lstm2_multi(calls, *, mode: Optional[str] = None):
         ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=device)
         stream = torch.cuda.current_stream(device).cuda_stream
         rc = lib.rtn_native_lstm2_fwd_multi(arr, count, T, B, n, dtype, mode_code, ws.data_ptr(), ws.numel(), stream)
-    _lib.check(rc)
+        _lib.check(rc)
+        if T * B * n > 0:  # (an empty problem does not touch its workspace)
+            status_watch.after_call("NativeLstm2 (%i calls)" % count, ws, count, device)
     del norm  # the normalised inputs stay alive until here; the stream-ordered allocator covers the rest
     return outs
 
@@ -498,6 +600,7 @@ def native_lstm2_grad_multi(calls):
     dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
     count = len(norm)
     with torch.cuda.device(device):
+        status_watch.poll()
         outs = [_alloc_grad_outputs(T, B, n, bf16, device) for _ in range(count)]
         ws_bytes = int(lib.rtn_native_lstm2_bwd_multi_workspace_bytes(count, T, B, n, dtype))
         ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=device)
@@ -509,7 +612,9 @@ def native_lstm2_grad_multi(calls):
                 DY.data_ptr(), Dd.data_ptr(), DX.data_ptr(), DW.data_ptr(), Dy0.data_ptr(), Dc0.data_ptr(),
             )  # fmt: skip
         rc = lib.rtn_native_lstm2_bwd_multi(arr, count, T, B, n, dtype, ws.data_ptr(), ws.numel(), torch.cuda.current_stream(device).cuda_stream)
-    _lib.check(rc)
+        _lib.check(rc)
+        if T * B * n > 0:  # (an empty problem does not touch its workspace)
+            status_watch.after_call("NativeLstm2 gradient (%i calls)" % count, ws, count, device)
     return outs
 
 
@@ -567,6 +672,7 @@ def lstm_generic_base_grad(V_h, c, i, Y, H, DY, Dd):
     lib = _lib.load()
     dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
     with torch.cuda.device(device):
+        status_watch.poll()
         DZ = torch.empty((T, B, 4 * n), dtype=act, device=device)
         DV_h = torch.empty((n, 4 * n), dtype=torch.float32, device=device)
         Dc = torch.empty((B, n), dtype=torch.float32, device=device)
@@ -575,7 +681,9 @@ def lstm_generic_base_grad(V_h, c, i, Y, H, DY, Dd):
             V_h.data_ptr(), c.data_ptr(), i.data_ptr(), Y.data_ptr(), H.data_ptr(), DY.data_ptr(), Dd.data_ptr(), DZ.data_ptr(),
             DV_h.data_ptr(), Dc.data_ptr(), T, B, n, dtype, ws.data_ptr(), ws.numel(), torch.cuda.current_stream(device).cuda_stream,
         )  # fmt: skip
-    _lib.check(rc)
+        _lib.check(rc)
+        if T * B * n > 0:  # (an empty problem does not touch its workspace)
+            status_watch.after_call("LstmGenericBase gradient", ws, 1, device)
     return DZ, DV_h, Dc
 
 

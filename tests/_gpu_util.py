@@ -12,10 +12,10 @@ import torch
 from returnn_amd import build, lib, native_op, torch_native_op
 
 
-def get_op():
+def get_op(mode="auto"):
     if not os.path.exists(build.LIB_PATH):
         build.build_library()
-    return torch_native_op.make_op(native_op.NativeLstm2)
+    return torch_native_op.make_op(native_op.NativeLstm2, mode=mode)
 
 
 @contextlib.contextmanager
@@ -52,8 +52,7 @@ def run_op(X, W, y0, c0, i, start=0, step=1, *, dtype="f32", mode="auto", check_
     """
     :return: Y, C, H, d, y_last as float32 numpy arrays
     """
-    op = get_op()
-    torch_native_op.OpMaker.options["NativeLstm2"]["mode"] = mode
+    op = get_op(mode)
     Xd, Wd, y0d = (to_dev(a, dtype) for a in (X, W, y0))
     c0d, id_ = (to_dev(a, "f32") for a in (c0, i))
     Y, C, H, d = op(Xd, Wd, y0d, c0d, id_, start, step)

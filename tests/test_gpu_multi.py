@@ -16,8 +16,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _single(args, dtype, mode="auto"):
-    op = get_op()
-    torch_native_op.OpMaker.options["NativeLstm2"]["mode"] = mode
+    op = get_op(mode)
     return op(*args)
 
 

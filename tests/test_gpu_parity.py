@@ -419,11 +419,62 @@ def test_bounded_wait_expires_cleanly():
         assert status in (lib.RTN_OK, lib.RTN_ERR_ABORTED)
         if status == lib.RTN_OK:
             check_f32(got, oracle.native_lstm2_fwd(*p, 0, 1)[:4], "bounded wait")
+        else:
+            # a caller who never asks for the status still sees it: NaN in the final cell state and in the last frame of Y
+            Y, _, _, d = got
+            assert numpy.isnan(d).any(), "kernel %i: no NaN in d after an expired wait" % kernel
+            assert numpy.isnan(Y[-1]).any(), "kernel %i: no NaN in the last frame of Y after an expired wait" % kernel
         # and the next ordinary call is unaffected
         with env(RTN_LSTM2_KERNEL=kernel):
             rc, status, got = run_raw(*p, 0, 1, mode="persistent")
         assert rc == 0 and status == 0
         check_f32(got, oracle.native_lstm2_fwd(*p, 0, 1)[:4], "after bounded wait")
+
+
+def test_expired_wait_reaches_the_torch_caller():
+    """The same forced expiry through the torch op: the status watch raises at the next look (lazily, without
+    waiting for the device, or at once in its synchronous setting) exactly when the outputs carry the NaN marks."""
+    from returnn_amd import torch_native_op
+    from _gpu_util import to_dev
+
+    announce("bounded wait, torch op")
+    watch = torch_native_op.status_watch
+    watch.drain()
+    X, W, y0, c0, i = random_problem(62, 50, 8, 256)
+    args = [to_dev(a, "f32") for a in (X, W, y0, c0, i)]
+    op = get_op("persistent")
+    want = oracle.native_lstm2_fwd(X, W, y0, c0, i, 0, 1)[:4]
+    for synchronous in (None, True):
+        watch.synchronous = synchronous
+        try:
+            raised = False
+            with env(RTN_LSTM2_TIMEOUT_TICKS=0):
+                try:
+                    got = op(*args, 0, 1)
+                except torch_native_op.NativeOpAborted:
+                    assert synchronous, "the lazy watch must not raise inside the call that failed"
+                    raised, got = True, None
+            torch.cuda.synchronize()
+            if got is not None:
+                marked = bool(torch.isnan(got[3]).any())
+                if synchronous:
+                    assert not marked, "synchronous watch: NaN marks without an exception"
+                else:
+                    try:
+                        watch.drain()
+                    except torch_native_op.NativeOpAborted:
+                        raised = True
+                    assert raised == marked, "lazy watch raised=%r but NaN marks=%r" % (raised, marked)
+                if not marked:
+                    check_f32(tuple(t.cpu().numpy() for t in got), want, "bounded wait, torch op")
+        finally:
+            watch.synchronous = None
+        # the next ordinary call is unaffected and the watch is clean again
+        before = watch.checked
+        got = op(*args, 0, 1)
+        watch.drain()
+        assert watch.checked == before + 1
+        check_f32(tuple(t.cpu().numpy() for t in got), want, "after bounded wait, torch op")
 
 
 @pytest.mark.parametrize(
@@ -527,7 +578,6 @@ def test_forward_recorded_into_a_callers_graph(T, B, n, dtype):
     from returnn_amd import torch_native_op
 
     op = get_op()
-    torch_native_op.OpMaker.options["NativeLstm2"]["mode"] = "auto"
     problems = [random_problem(990 + k, T, B, n) for k in range(3)]
     X, W, y0, c0, i = problems[0]
     Xd, Wd, y0d = (to_dev(a, dtype) for a in (X, W, y0))

@@ -45,8 +45,7 @@ def _holes(rng, T, B, p_keep=0.7):
 
 def run_generic_base(Z, V_h, c, i, *, dtype="f32", mode="auto"):
     get_op()  # builds the library if needed
-    op = torch_native_op.make_op(native_op.LstmGenericBase)
-    torch_native_op.OpMaker.options.setdefault("LstmGenericBase", {})["mode"] = mode
+    op = torch_native_op.make_op(native_op.LstmGenericBase, mode=mode)
     Y, H, d = op(to_dev(Z, dtype), to_dev(V_h, dtype), to_dev(c, "f32"), to_dev(i, "f32"))
     torch.cuda.synchronize()
     return tuple(t.float().cpu().numpy() for t in (Y, H, d))
@@ -54,8 +53,7 @@ def run_generic_base(Z, V_h, c, i, *, dtype="f32", mode="auto"):
 
 def run_low_mem(X, W, b, y0, c0, i, start=0, step=1, *, dtype="f32", mode="auto"):
     get_op()
-    op = torch_native_op.make_op(native_op.LstmLowMem)
-    torch_native_op.OpMaker.options.setdefault("LstmLowMem", {})["mode"] = mode
+    op = torch_native_op.make_op(native_op.LstmLowMem, mode=mode)
     Y, C, d = op(to_dev(X, dtype), to_dev(W, dtype), to_dev(b, dtype), to_dev(y0, dtype), to_dev(c0, "f32"), to_dev(i, "f32"), start, step)
     torch.cuda.synchronize()
     return tuple(t.float().cpu().numpy() for t in (Y, C, d))
@@ -301,8 +299,6 @@ def test_sibling_ops_recorded_into_a_callers_graph(dtype):
     announce("siblings captured", dtype)
     get_op()
     T, B, n_in, n = 9, 6, 24, 64
-    for m in ("LstmLowMem", "LstmGenericBase"):
-        torch_native_op.OpMaker.options.setdefault(m, {})["mode"] = "auto"
     lm = torch_native_op.make_op(native_op.LstmLowMem)
     gb = torch_native_op.make_op(native_op.LstmGenericBase)
     lm_problems = [low_mem_problem(700 + k, T, B, n_in, n) for k in range(2)]
