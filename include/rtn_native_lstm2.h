@@ -206,8 +206,8 @@ int rtn_mfma_sequence_probe(int32_t count, int64_t T, int32_t B, int32_t n, int3
  * fused with the frame's pointwise part), replayed through a library-owned hipGraph.  The large weight-gradient GEMM
  * (Y^T DX over all frames) is left to rocBLAS, which may allocate its own device workspace on first use.  Under stream
  * capture the per-frame launches and the rocBLAS calls are recorded into the caller's graph (the counterpart of the
- * reference's whole-step graph capture, returnn/torch/util/graph_capture.py); the library's rocBLAS handle has to exist
- * by then: run the entry once outside the capture first.  `workspace`: rtn_native_lstm2_bwd_workspace_bytes();
+ * reference's whole-step graph capture, returnn/torch/util/graph_capture.py); the library's rocBLAS handle (one per host
+ * thread and device) has to exist by then: run the entry once outside the capture first, on the capturing thread.  `workspace`: rtn_native_lstm2_bwd_workspace_bytes();
  * rtn_native_lstm2_fwd_status(workspace, stream) reports an expired bounded wait of the persistent kernel.
  */
 int rtn_native_lstm2_bwd(const void* W, const void* y0, const float* c0, const float* i, int32_t start, int32_t step,
@@ -318,7 +318,15 @@ const char* rtn_native_lstm2_describe_plan(int64_t T, int32_t B, int32_t n, int3
 const char* rtn_native_lstm2_describe_multi_plan(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype,
                                                  int32_t mode);
 
-/* ABI version of this header: 7. */
+/* Library-owned graphs (GRAPH mode; the per-frame launches of the gradient entries): out[0] = graphs kept (at most 8,
+ * keyed by shape, element type, plan and device, never by addresses), out[1] = graphs dropped from the cache whose last
+ * launch has not completed yet (destroyed at a later call, once it has), out[2] = graphs built so far, out[3] = launches
+ * that first wrote another parameter block (other buffers, same shape) into a kept graph, out[4] = graphs destroyed.
+ * n_out >= 5.  Replaces nothing in the reference (its ops launch per step, returnn/native_op.py:1254-1277); for tests and
+ * for telling a cache that thrashes from one that does not. */
+int rtn_graph_cache_stats(int64_t* out, int32_t n_out);
+
+/* ABI version of this header: 8. */
 int rtn_native_lstm2_abi_version(void);
 
 #ifdef __cplusplus

@@ -15,6 +15,8 @@
 #include <list>
 #include <mutex>
 #include <string>
+#include <tuple>
+#include <utility>
 #include <vector>
 
 #include <rocblas/rocblas.h>
@@ -1113,14 +1115,14 @@ BwdRegwKernel bwd_regw_kernel_for(int KSB, int MT, int WV) {
   return nullptr;
 }
 
-// One rocBLAS handle per device, created on first use and kept for the life of the process.
+// One rocBLAS handle per host thread and device, created on first use and kept for the life of the thread (never
+// destroyed: at thread or process exit the runtime below it may already be gone).  A handle carries the stream its
+// calls go to; with a handle of its own a thread cannot have that stream changed under it by another thread's call.
 int blas_handle(rocblas_handle* out) {
-  static std::mutex mu;
-  static rocblas_handle handles[64] = {nullptr};
+  static thread_local rocblas_handle handles[64] = {nullptr};
   int dev = 0;
   RTN_HIP(hipGetDevice(&dev));
   if (dev < 0 || dev >= 64) return fail(RTN_ERR_HIP, "NativeLstm2: device index %d out of range", dev);
-  std::lock_guard<std::mutex> lock(mu);
   if (!handles[dev]) {
     if (rocblas_create_handle(&handles[dev]) != rocblas_status_success) {
       handles[dev] = nullptr;
@@ -1203,7 +1205,20 @@ using namespace rtn;
 
 extern "C" {
 
-int rtn_native_lstm2_abi_version(void) { return 7; }
+int rtn_native_lstm2_abi_version(void) { return 8; }
+
+int rtn_graph_cache_stats(int64_t* out, int32_t n_out) {
+  g_last_error.clear();
+  if (!out || n_out < 5) return fail(RTN_ERR_ARG, "NativeLstm2: the graph statistics need room for 5 numbers");
+  std::lock_guard<std::mutex> lock(g_graph_mu);
+  sweep_retired();
+  out[0] = (int64_t)g_graphs.size();
+  out[1] = (int64_t)g_retired.size();
+  out[2] = g_graph_records;
+  out[3] = g_graph_retargets;
+  out[4] = g_graph_destroyed;
+  return RTN_OK;
+}
 
 const char* rtn_last_error(void) { return g_last_error.c_str(); }
 

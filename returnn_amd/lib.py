@@ -31,7 +31,7 @@ MODE_PERSISTENT = 1
 MODE_GRAPH = 2
 MODE_STEPWISE = 3
 # The ABI version the structs and argument lists below were written for (rtn_native_lstm2_abi_version()).
-EXPECTED_ABI = 7
+EXPECTED_ABI = 8
 
 MODES = {"auto": MODE_AUTO, "persistent": MODE_PERSISTENT, "graph": MODE_GRAPH, "stepwise": MODE_STEPWISE}
 
@@ -60,6 +60,7 @@ SYMBOLS = (
     "rtn_last_error",
     "rtn_native_lstm2_describe_plan",
     "rtn_native_lstm2_describe_multi_plan",
+    "rtn_graph_cache_stats",
     "rtn_native_lstm2_abi_version",
 )
 
@@ -174,6 +175,8 @@ def load() -> ctypes.CDLL:
         lib.rtn_lstm_low_mem_fwd.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, vp]
         lib.rtn_lstm_low_mem_fwd_workspace_bytes.restype = sz
         lib.rtn_lstm_low_mem_fwd_workspace_bytes.argtypes = [i64, i32, i32, i32, i32, i32]
+        lib.rtn_graph_cache_stats.restype = ctypes.c_int
+        lib.rtn_graph_cache_stats.argtypes = [ctypes.POINTER(ctypes.c_int64), i32]
         lib.rtn_mfma_sequence_probe.restype = ctypes.c_int
         lib.rtn_mfma_sequence_probe.argtypes = [i32, i64, i32, i32, i32, i32, vp, sz, vp]
         lib.rtn_handover_latency_probe.restype = ctypes.c_int
@@ -201,6 +204,13 @@ def check(rc: int) -> None:
     (TORCH_CHECK -> RuntimeError, returnn/native_op.cpp:660)."""
     if rc != RTN_OK:
         raise RuntimeError(last_error() or ("NativeLstm2: error code %i" % rc))
+
+
+def graph_cache_stats() -> dict:
+    """Counters of the library-owned graph cache: kept, retiring, built, retargeted, destroyed."""
+    out = (ctypes.c_int64 * 5)()
+    check(load().rtn_graph_cache_stats(out, 5))
+    return dict(zip(("kept", "retiring", "built", "retargeted", "destroyed"), (int(v) for v in out)))
 
 
 def describe_plan(T: int, B: int, n: int, dtype: int, mode: int) -> str:

@@ -275,3 +275,53 @@ def test_forward_and_gradient_recorded_into_a_callers_graph(T, B, n, dtype):
         want = oracle.native_lstm2_bwd(f(Xd), f(Wd), f(y0d), c0k, ik, 0, 1, f(got_f[0]), f(got_f[1]), f(got_f[2]), f(DYd), grads_in[k][1], dtype=numpy.float64)
         for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), got_g, want):
             assert _rel_to_max(f(a), b) <= tol, (k, name, "against the oracle")
+
+
+def test_gradient_from_two_host_threads_on_their_own_streams():
+    """Two host threads, each with a stream of its own, run forward and gradient at the same time (the weight-gradient
+    GEMMs go through a rocBLAS handle per thread, so neither can have its stream changed by the other).  Every result must
+    equal what the main thread computes alone."""
+    import threading
+
+    announce("bwd from two threads")
+    op = get_op()
+    shapes = [(14, 6, 128, "bf16"), (11, 5, 160, "f32")]
+    inputs, want = [], []
+    for k, (T, B, n, dtype) in enumerate(shapes):
+        X, W, y0, c0, i = random_problem(640 + k, T, B, n)
+        rng = numpy.random.default_rng(650 + k)
+        DY = rng.normal(0, 1.0, (T, B, n)).astype(numpy.float32)
+        Dd = rng.normal(0, 1.0, (B, n)).astype(numpy.float32)
+        Xd, Wd, y0d, DYd = (to_dev(a, dtype) for a in (X, W, y0, DY))
+        c0d, id_, Ddd = (to_dev(a, "f32") for a in (c0, i, Dd))
+        inputs.append((Xd, Wd, y0d, c0d, id_, DYd, Ddd))
+        Y, C, H, _ = op(Xd, Wd, y0d, c0d, id_, 0, 1)
+        want.append(torch_native_op.native_lstm2_grad(Wd, y0d, c0d, id_, 0, 1, Y, C, H, DYd, Ddd))
+    torch.cuda.synchronize()
+    results, errors = {}, []
+
+    def work(k):
+        try:
+            Xd, Wd, y0d, c0d, id_, DYd, Ddd = inputs[k]
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for r in range(6):
+                    Y, C, H, _ = op(Xd, Wd, y0d, c0d, id_, 0, 1)
+                    results[(k, r)] = torch_native_op.native_lstm2_grad(Wd, y0d, c0d, id_, 0, 1, Y, C, H, DYd, Ddd)
+            stream.synchronize()
+        except Exception as exc:  # noqa: BLE001
+            errors.append((k, exc))
+
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(len(shapes))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for (k, r), grads in sorted(results.items()):
+        for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), grads, want[k]):
+            if name == "DW":  # rocBLAS may sum in another order from run to run
+                assert _rel_to_max(a.double().cpu().numpy(), b.double().cpu().numpy()) <= 1e-5, (k, r, name)
+            else:
+                assert torch.equal(a, b), "thread %i, round %i: %s differs from the single-threaded result" % (k, r, name)
