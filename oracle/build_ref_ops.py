@@ -1,0 +1,72 @@
+"""
+Test infrastructure, never shipped with the library: builds a few of the reference's OTHER native ops for gfx950 through
+this package's op loader, so that the GPU tests can run them against the known answers the reference's own tests hold.
+
+The op descriptions are read as text where they lie (``/root/reference/returnn/native_op.py``, parsed with :mod:`ast` by
+``tests/_reference_op_sources.py``; nothing of the reference is imported or executed), the loader generates the unit and
+hipcc compiles it in a temporary directory, and only the shared object is kept: ``oracle/_ref/ops/<OpName>.so`` plus
+``ops.json`` with each op's argument table (names, ranks, element types: what a caller needs to bind it).  No source of
+the reference, generated or not, is written into this tree.  ``oracle/_ref/`` is not under version control.
+
+What this checks is the loader (dialect header, generated entry point, Python wrapper), not the LSTM kernels: the ops run
+against this package's support header, where the reference would use its own ``native_op.cpp``.
+
+Run: ``python oracle/build_ref_ops.py`` (no GPU needed).  Without the reference tree it does nothing.
+"""
+
+from __future__ import annotations
+
+import json
+import os
+import shutil
+import sys
+import tempfile
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+OUT_DIR = os.path.join(HERE, "_ref", "ops")
+
+# ops whose expected results the reference's tests hold as numbers (tests/test_torch_native_op.py:95-160, :582-631,
+# :689-812, :922-1034)
+OPS = ("FastBaumWelchOp", "FastViterbiOp", "EditDistanceOp", "OptimalCompletionEditDistanceOp")
+
+
+def _plain(x):
+    """in_info / out_info as JSON: tuples become lists."""
+    if isinstance(x, (tuple, list)):
+        return [_plain(v) for v in x]
+    if isinstance(x, dict):
+        return {k: _plain(v) for k, v in x.items()}
+    return x
+
+
+def build(ops=OPS, out_dir: str = OUT_DIR, verbose: bool = True) -> bool:
+    """:return: whether anything was built (False: no reference tree here)"""
+    for p in (ROOT, os.path.join(ROOT, "tests")):
+        if p not in sys.path:
+            sys.path.insert(0, p)
+    import _reference_op_sources as ref_sources
+    from returnn_amd import op_loader
+
+    if not ref_sources.available():
+        if verbose:
+            print("build_ref_ops: no reference tree at %s, nothing to do" % ref_sources.REFERENCE_NATIVE_OP)
+        return False
+    classes, _ = ref_sources.read_descriptions()
+    os.makedirs(out_dir, exist_ok=True)
+    table = {}
+    with tempfile.TemporaryDirectory(prefix="rtn_ref_ops_") as tmp:
+        for name in ops:
+            fields = classes[name]
+            op = op_loader.compile_op(ref_sources.as_description(name, fields), compiler_opts={"cache_dir": tmp})
+            shutil.copyfile(op.compiler.so_filename, os.path.join(out_dir, name + ".so"))
+            table[name] = {"in_info": _plain(fields["in_info"]), "out_info": _plain(fields["out_info"])}
+            if verbose:
+                print("build_ref_ops: %s -> %s" % (name, os.path.join(out_dir, name + ".so")))
+    with open(os.path.join(out_dir, "ops.json"), "w") as f:
+        json.dump(table, f, indent=1, sort_keys=True)
+    return True
+
+
+if __name__ == "__main__":
+    build()
