@@ -48,9 +48,10 @@ extern "C" {
  * unpadded problem, since a padded cell has zero inputs, weights and state.  n up to 32 runs on element-wise kernels. */
 
 /* Execution mode.
- * AUTO:       PERSISTENT when the shape and device allow it and the stream is not
- *             being captured, else GRAPH.
- * PERSISTENT: one cooperative kernel runs all time steps.  Where the device's registers hold
+ * AUTO:       PERSISTENT when the shape and device allow it, else GRAPH.
+ * PERSISTENT: one kernel runs all time steps, all its workgroups on the device together
+ *             (a cooperative launch; under stream capture a kernel node that the library
+ *             adds to the capturing graph itself, see rtn_native_lstm2_capture_report).  Where the device's registers hold
  *             the recurrent weights (the usual case) every workgroup keeps its slice of W
  *             in registers and the workgroups hand the hidden state over through a ring
  *             of buffers in the workspace that validates itself (a word that still holds
@@ -205,7 +206,8 @@ int rtn_mfma_sequence_probe(int32_t count, int64_t T, int32_t B, int32_t n, int3
  * workgroups.  Otherwise one launch per visited frame (the MFMA GEMM Dy0 += DX[t'] W^T of the frame processed before,
  * fused with the frame's pointwise part), replayed through a library-owned hipGraph.  The large weight-gradient GEMM
  * (Y^T DX over all frames) is left to rocBLAS, which may allocate its own device workspace on first use.  Under stream
- * capture the per-frame launches and the rocBLAS calls are recorded into the caller's graph (the counterpart of the
+ * capture the kernels (the persistent one as a node of its own, see rtn_native_lstm2_capture_report) and the rocBLAS calls
+ * are recorded into the caller's graph (the counterpart of the
  * reference's whole-step graph capture, returnn/torch/util/graph_capture.py); the library's rocBLAS handle (one per host
  * thread and device) has to exist by then: run the entry once outside the capture first, on the capturing thread.  `workspace`: rtn_native_lstm2_bwd_workspace_bytes();
  * rtn_native_lstm2_fwd_status(workspace, stream) reports an expired bounded wait of the persistent kernel.
@@ -326,7 +328,15 @@ const char* rtn_native_lstm2_describe_multi_plan(int32_t count, int64_t T, int32
  * for telling a cache that thrashes from one that does not. */
 int rtn_graph_cache_stats(int64_t* out, int32_t n_out);
 
-/* ABI version of this header: 8. */
+/* What became of the persistent kernels in calls made under stream capture so far (the counterpart of the reference's
+ * whole-step graph capture, returnn/torch/util/graph_capture.py:1-80, where its ops are just launches on the capture
+ * stream): how many were added to the capturing graph as kernel nodes with the cooperative attribute, how many as
+ * ordinary kernel nodes, and, if the runtime refused the cooperative node, which call refused it and with what error.
+ * Thread-local text.  RTN_LSTM2_CAPTURE=steps in the environment records per-step launches instead;
+ * RTN_LSTM2_CAPTURE_NODE=plain does not try the cooperative attribute. */
+const char* rtn_native_lstm2_capture_report(void);
+
+/* ABI version of this header: 9. */
 int rtn_native_lstm2_abi_version(void);
 
 #ifdef __cplusplus

@@ -142,6 +142,12 @@ size_t mfma_lds_bytes(int n, int dtype, int MT, int NT) {
   return (size_t)MT * (n / KM) * kTileBytes + (size_t)kWaves * MT * NT * kTileBytes;
 }
 
+// Whether calls made under stream capture keep the persistent kernels (default) or record per-step launches.
+bool capture_keeps_persistent() {
+  const char* v = getenv("RTN_LSTM2_CAPTURE");
+  return !(v && strcmp(v, "steps") == 0);
+}
+
 // Chooses the decomposition.  `want_mode` is the caller's mode; `capturing` says the stream is
 // under capture (a cooperative launch cannot be recorded).  Returns false with a reason when
 // mode == PERSISTENT is impossible.
@@ -344,9 +350,9 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
       }
       if (!persistent_ok && why) *why = "no decomposition keeps W on chip with all workgroups co-resident";
     }
-    if (persistent_ok && capturing) {
+    if (persistent_ok && capturing && !capture_keeps_persistent()) {
       persistent_ok = false;
-      if (why) *why = "the stream is being captured; a cooperative launch cannot be recorded";
+      if (why) *why = "the stream is being captured and RTN_LSTM2_CAPTURE=steps asks for per-step launches there";
     }
     if (persistent_ok && !di.cooperative) {
       persistent_ok = false;
@@ -702,6 +708,77 @@ int launch_steps_graph(const Lstm2Params& p, const Plan& pl, int dtype, hipStrea
   return replay_graph(key, &p, sizeof(p), stream, [&](LaunchSink& sink) { return launch_steps(p, pl, dtype, sink); });
 }
 
+// ---- launches that need all their workgroups on the device together ------------------------------------------------
+// Outside stream capture: a cooperative launch (the runtime checks that the grid fits and keeps such launches apart).
+// Under stream capture a cooperative launch cannot be recorded with the stream API, so the kernel node is built by hand:
+// the capturing graph and the stream's current dependencies are asked of the runtime, a kernel node with the cooperative
+// attribute is added behind them and made the stream's new dependency.  If the runtime refuses any of that, the kernel
+// is recorded as an ordinary kernel node (it never uses a grid barrier; what it needs is co-residency, which the
+// occupancy check before the call has established for a device that runs nothing else at that moment; every wait inside
+// is bounded, so a replay that does find the device shared ends with the status word set and NaN marks, not hung).
+// RTN_LSTM2_CAPTURE_NODE=plain skips the attempt; RTN_LSTM2_CAPTURE=steps records per-step launches as before.
+std::mutex g_capture_mu;
+long long g_capture_cooperative = 0, g_capture_plain = 0;
+std::string g_capture_refusal;  // why a cooperative node was refused, if it was
+
+int launch_coresident(const void* k, dim3 grid, dim3 block, void** args, unsigned lds, hipStream_t stream, bool capturing) {
+  if (!capturing) {
+    RTN_HIP(hipLaunchCooperativeKernel(k, grid, block, args, lds, stream));
+    return RTN_OK;
+  }
+  const char* kind = getenv("RTN_LSTM2_CAPTURE_NODE");
+  bool try_cooperative = !(kind && strcmp(kind, "plain") == 0);
+  {
+    std::lock_guard<std::mutex> lock(g_capture_mu);
+    if (!g_capture_refusal.empty()) try_cooperative = false;  // refused once: do not ask again
+  }
+  if (try_cooperative) {
+    hipGraphNode_t node = nullptr;
+    const char* step = "hipStreamGetCaptureInfo_v2";
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    hipGraph_t graph = nullptr;
+    const hipGraphNode_t* deps = nullptr;
+    size_t ndeps = 0;
+    hipError_t e = hipStreamGetCaptureInfo_v2(stream, &st, nullptr, &graph, &deps, &ndeps);
+    if (e == hipSuccess && (st != hipStreamCaptureStatusActive || !graph)) e = hipErrorIllegalState;
+    if (e == hipSuccess) {
+      step = "hipGraphAddKernelNode";
+      hipKernelNodeParams kp;
+      memset(&kp, 0, sizeof(kp));
+      kp.func = const_cast<void*>(k);
+      kp.gridDim = grid;
+      kp.blockDim = block;
+      kp.sharedMemBytes = lds;
+      kp.kernelParams = args;
+      e = hipGraphAddKernelNode(&node, graph, deps, ndeps, &kp);
+    }
+    if (e == hipSuccess) {
+      step = "hipGraphKernelNodeSetAttribute(cooperative)";
+      hipKernelNodeAttrValue v;
+      memset(&v, 0, sizeof(v));
+      v.cooperative = 1;
+      e = hipGraphKernelNodeSetAttribute(node, hipKernelNodeAttributeCooperative, &v);
+    }
+    if (e == hipSuccess) {
+      step = "hipStreamUpdateCaptureDependencies";
+      e = hipStreamUpdateCaptureDependencies(stream, &node, 1, hipStreamSetCaptureDependencies);
+    }
+    if (e == hipSuccess) {
+      std::lock_guard<std::mutex> lock(g_capture_mu);
+      ++g_capture_cooperative;
+      return RTN_OK;
+    }
+    if (node) (void)hipGraphDestroyNode(node);
+    (void)hipGetLastError();
+    std::lock_guard<std::mutex> lock(g_capture_mu);
+    g_capture_refusal = std::string(step) + ": " + hipGetErrorString(e);
+  }
+  RTN_HIP(hipLaunchKernel(k, grid, block, args, lds, stream));
+  std::lock_guard<std::mutex> lock(g_capture_mu);
+  ++g_capture_plain;
+  return RTN_OK;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 int check_dims(int64_t T, int32_t B, int32_t n, int32_t dtype) {
@@ -1043,7 +1120,8 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
           one.grid = one.p[0].groups * pl.wgs_per_group;
           one.wgs_each = (int)align_up((size_t)one.grid, (size_t)device_info().xcds);
           void* args[] = {(void*)&one};
-          RTN_HIP(hipLaunchCooperativeKernel(pk, dim3(one.grid), dim3(kWgThreads), args, (unsigned)pl.lds_bytes, stream));
+          rc = launch_coresident(pk, dim3(one.grid), dim3(kWgThreads), args, (unsigned)pl.lds_bytes, stream, capturing);
+          if (rc != RTN_OK) return rc;
         }
         continue;
       }
@@ -1058,7 +1136,8 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
           multi.xcds = device_info().xcds;
           void* args[] = {(void*)&multi};
           const int wgs = (pending == 1 || pl.local) ? pl.grid : multi.wgs_each * pending;
-          RTN_HIP(hipLaunchCooperativeKernel(pk, dim3(wgs), dim3(kWgThreads), args, (unsigned)pl.lds_bytes, stream));
+          rc = launch_coresident(pk, dim3(wgs), dim3(kWgThreads), args, (unsigned)pl.lds_bytes, stream, capturing);
+          if (rc != RTN_OK) return rc;
           pending = 0;
         }
         continue;
@@ -1067,8 +1146,8 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
         p.groups = pl.groups;
         int s_begin = 0, s_end = p.nsteps;
         void* args_lds[] = {(void*)&p, (void*)&s_begin, (void*)&s_end};
-        RTN_HIP(hipLaunchCooperativeKernel(pk, dim3(pl.groups * pl.wgs_per_group), dim3(kWgThreads), args_lds,
-                                           (unsigned)pl.lds_bytes, stream));
+        rc = launch_coresident(pk, dim3(pl.groups * pl.wgs_per_group), dim3(kWgThreads), args_lds, (unsigned)pl.lds_bytes, stream, capturing);
+        if (rc != RTN_OK) return rc;
         continue;
       }
     } else {
@@ -1205,7 +1284,18 @@ using namespace rtn;
 
 extern "C" {
 
-int rtn_native_lstm2_abi_version(void) { return 8; }
+int rtn_native_lstm2_abi_version(void) { return 9; }
+
+const char* rtn_native_lstm2_capture_report(void) {
+  static thread_local std::string text;
+  std::lock_guard<std::mutex> lock(g_capture_mu);
+  char buf[256];
+  snprintf(buf, sizeof(buf), "persistent launches recorded under stream capture: %lld as cooperative kernel nodes, %lld as ordinary kernel nodes",
+           g_capture_cooperative, g_capture_plain);
+  text = buf;
+  if (!g_capture_refusal.empty()) text += "; cooperative node refused by " + g_capture_refusal;
+  return text.c_str();
+}
 
 int rtn_graph_cache_stats(int64_t* out, int32_t n_out) {
   g_last_error.clear();
@@ -1604,7 +1694,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
     const int S = 4 * n / KM;
     const long bwd_kernel = env_long("RTN_LSTM2_BWD_KERNEL", 0);  // 0 auto, 1 per-frame launches, 2 persistent
-    if (mfma && (4 * n) % KM == 0 && bwd_kernel != 1 && !capturing && device_info().cooperative && count <= kMaxBwdMulti) {
+    if (mfma && (4 * n) % KM == 0 && bwd_kernel != 1 && (!capturing || capture_keeps_persistent()) && device_info().cooperative && count <= kMaxBwdMulti) {
       const long env_mt = env_long("RTN_LSTM2_BWD_MT", 0);
       const long env_waves = env_long("RTN_LSTM2_BWD_WAVES", 0);
       // (rows per group, tiles per workgroup, wavefronts per workgroup)
@@ -1742,7 +1832,8 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
         multi.q[k].group_offset = g0;
       }
       void* args[] = {(void*)&multi};
-      RTN_HIP(hipLaunchCooperativeKernel(pk, dim3((unsigned)(count * multi.wgs_each)), dim3((unsigned)(64 * bwd_waves)), args, (unsigned)bwd_lds, stream));
+      rc = launch_coresident(pk, dim3((unsigned)(count * multi.wgs_each)), dim3((unsigned)(64 * bwd_waves)), args, (unsigned)bwd_lds, stream, capturing);
+      if (rc != RTN_OK) return rc;
     }
     for (int k = 0; k < count; ++k) {
       const BwdJob& j = jobs[(size_t)k];

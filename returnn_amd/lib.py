@@ -31,7 +31,7 @@ MODE_PERSISTENT = 1
 MODE_GRAPH = 2
 MODE_STEPWISE = 3
 # The ABI version the structs and argument lists below were written for (rtn_native_lstm2_abi_version()).
-EXPECTED_ABI = 8
+EXPECTED_ABI = 9
 
 MODES = {"auto": MODE_AUTO, "persistent": MODE_PERSISTENT, "graph": MODE_GRAPH, "stepwise": MODE_STEPWISE}
 
@@ -61,6 +61,7 @@ SYMBOLS = (
     "rtn_native_lstm2_describe_plan",
     "rtn_native_lstm2_describe_multi_plan",
     "rtn_graph_cache_stats",
+    "rtn_native_lstm2_capture_report",
     "rtn_native_lstm2_abi_version",
 )
 
@@ -175,6 +176,8 @@ def load() -> ctypes.CDLL:
         lib.rtn_lstm_low_mem_fwd.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, vp]
         lib.rtn_lstm_low_mem_fwd_workspace_bytes.restype = sz
         lib.rtn_lstm_low_mem_fwd_workspace_bytes.argtypes = [i64, i32, i32, i32, i32, i32]
+        lib.rtn_native_lstm2_capture_report.restype = ctypes.c_char_p
+        lib.rtn_native_lstm2_capture_report.argtypes = []
         lib.rtn_graph_cache_stats.restype = ctypes.c_int
         lib.rtn_graph_cache_stats.argtypes = [ctypes.POINTER(ctypes.c_int64), i32]
         lib.rtn_mfma_sequence_probe.restype = ctypes.c_int
@@ -204,6 +207,10 @@ def check(rc: int) -> None:
     (TORCH_CHECK -> RuntimeError, returnn/native_op.cpp:660)."""
     if rc != RTN_OK:
         raise RuntimeError(last_error() or ("NativeLstm2: error code %i" % rc))
+
+
+def capture_report() -> str:
+    return load().rtn_native_lstm2_capture_report().decode("utf8", "replace")
 
 
 def graph_cache_stats() -> dict:
