@@ -281,8 +281,7 @@ size_t rtn_lstm_generic_base_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n
  * Gradient op of LstmGenericBase (c_bw_code returnn/native_op.py:525-574, lstm_bwd_kernel :430-485; inputs as its
  * grad_input_map :374-378): V_h, c, i, the forward results Y and H, DY [T,B,n], Dd [B,n] (float32)  ->  DZ [T,B,4n],
  * DV_h [n,4n] (float32), Dc [B,n] (float32).  Runs on the NativeLstm2 gradient kernels; the reference overwrites H
- * with DZ and DY with a working array, here both inputs are left alone.  LstmLowMem has no gradient entry point: its
- * reference gradient (:838-1026) is marked unfinished where masks are concerned (:965).
+ * with DZ and DY with a working array, here both inputs are left alone.
  */
 int rtn_lstm_generic_base_bwd(const void* V_h, const float* c, const float* i, const void* Y, const void* H, const void* DY,
                               const float* Dd, void* DZ, float* DV_h, float* Dc, int64_t T, int32_t B, int32_t n,
@@ -294,6 +293,29 @@ int rtn_lstm_low_mem_fwd(const void* X, const void* W, const void* b, const void
                          int32_t n, int32_t dtype, int32_t mode, void* workspace, size_t workspace_bytes,
                          void* hip_stream);
 size_t rtn_lstm_low_mem_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n_in, int32_t n, int32_t dtype, int32_t mode);
+
+/*
+ * Gradient op of LstmLowMem (c_bw_code returnn/native_op.py:864-1026, lstm_bwd_kernel :659-712; inputs as its
+ * grad_input_map :619-625): X, W, b, y0, c0, i, start, step, the forward results Y and C, DY [T,B,n], Dd [B,n] (float32)
+ *   ->  DX [T,B,n_in], DW [n_in+n,4n] (float32), Db [4n] (float32), Dh [B,n] (error of y0), Dc [B,n] (error of c0, float32).
+ * Element type `dtype` for X W b y0 Y DY DX Dh.  The forward pass keeps no gates; where the reference computes them
+ * again frame by frame inside its loop (:966-979), here they come from GEMMs over all frames at once (the outputs are
+ * known, so that part is no recurrence), the recurrence of the errors runs on the NativeLstm2 gradient kernels over the
+ * recurrent rows of W, and DX, the input rows of DW and Db are products and sums over all frames afterwards (rocBLAS).
+ * The results are those of the reference's formulas, including what they do on masked frames: the error arriving from
+ * the frame processed before is not masked (d_y = DY * mask + d_h, :679), which is the gradient of the forward pass
+ * only while no masked frame has valid frames behind it in the recurrence (full-length batches; right-padded batches
+ * with step > 0); the reference's own comment (:965) calls the rest unfinished.  Its loop walks back from frame T-1
+ * (from frame `start` for step < 0) whatever the stride; where that is not the frame set of the forward pass (the stride
+ * does not divide the distance between the two ends) the reference reads outputs that were never written, and the call
+ * is refused here with RTN_ERR_RANGE.  Workspace: rtn_lstm_low_mem_bwd_workspace_bytes() (two arrays of T*B*4n elements
+ * besides the gradient workspace); rtn_native_lstm2_fwd_status(workspace, stream) reports an expired bounded wait.
+ */
+int rtn_lstm_low_mem_bwd(const void* X, const void* W, const void* b, const void* y0, const float* c0, const float* i,
+                         int32_t start, int32_t step, const void* Y, const float* C, const void* DY, const float* Dd, void* DX,
+                         float* DW, float* Db, void* Dh, float* Dc, int64_t T, int32_t B, int32_t n_in, int32_t n, int32_t dtype,
+                         void* workspace, size_t workspace_bytes, void* hip_stream);
+size_t rtn_lstm_low_mem_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n_in, int32_t n, int32_t dtype);
 
 /*
  * Final output per sequence.  Replaces the caller-side `_lstm_last_output`
@@ -336,7 +358,7 @@ int rtn_graph_cache_stats(int64_t* out, int32_t n_out);
  * RTN_LSTM2_CAPTURE_NODE=plain does not try the cooperative attribute. */
 const char* rtn_native_lstm2_capture_report(void);
 
-/* ABI version of this header: 9. */
+/* ABI version of this header: 10. */
 int rtn_native_lstm2_abi_version(void);
 
 #ifdef __cplusplus

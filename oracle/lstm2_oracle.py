@@ -4,6 +4,10 @@ ctypes binding of the C oracle in ``oracle/lstm2_oracle.c`` -- test infrastructu
 The C file restates the reference op (returnn/native_op.py:1081-1121, :1184-1285;
 returnn/native_op.cpp:1032-1067) and is the checker for the HIP path and the timed
 CPU baseline.  It is never the product: nothing under ``returnn_amd/`` imports it.
+
+Every function here is pinned by tests against golden vectors, closed forms, finite differences or autograd
+(tests/test_oracle*.py), with one exception stated where it applies: ``lstm_low_mem_bwd`` on masks with holes is a
+literal restatement of the reference's formulas -- parity unpinned there.
 """
 
 from __future__ import annotations
@@ -408,3 +412,81 @@ def lstm_low_mem_fwd(X, W, b, y0, c0, i, start: int = 0, step: int = 1, *, dtype
     if rc != 0:
         raise RuntimeError("oracle: error code %i" % rc)
     return Y, C, d
+
+
+def lstm_low_mem_bwd(X, W, b, y0, c0, i, start, step, Y, C, DY, Dd, *, dtype=numpy.float64):
+    """
+    Reference semantics of the ``LstmLowMem`` gradient op: the host loop of returnn/native_op.py:958-1020 with its
+    pointwise kernel :659-712, restated in numpy frame by frame (inputs as ``grad_input_map`` :619-625).  The gates are
+    recomputed from X, Y, W and b; the forward pass stores only Y and C.
+
+    Pinned for masks without holes before the last valid frame in processing order (full-length batches in both
+    directions, right-padded batches with step > 0) by finite differences of the pinned forward oracle and by torch
+    autograd (tests/test_oracle_siblings.py).  On a masked frame with valid frames behind it in the recurrence the
+    reference's kernel lets the error of the output through unmasked (``d_y_b = d_y * mask + d_h``, :679; its own
+    comment :965 calls the mask handling unfinished): what this function returns there is the literal restatement and
+    nothing else pins it -- parity unpinned for such masks.
+
+    The reference's loop starts at frame T-1 (step > 0) or at frame ``start`` (step < 0) whatever the stride; that is
+    the frame set of the forward pass only if the stride divides the distance between the two ends.  Other cases are
+    refused here (ValueError), as in the HIP entry.
+
+    :return: DX [T,B,n_in], DW [n_in+n,4n], Db [4n], Dh [B,n] (error of y0), Dc [B,n] (error of c0)
+    """
+    dtype = numpy.dtype(dtype).type
+    i = numpy.ascontiguousarray(i, dtype=dtype)
+    T, B = i.shape
+    y0 = numpy.ascontiguousarray(y0, dtype=dtype)
+    n = y0.shape[1]
+    X = numpy.ascontiguousarray(X, dtype=dtype)
+    n_in = X.shape[2]
+    W = _prep(W, dtype, (n_in + n, 4 * n), "W")
+    b = _prep(b, dtype, (4 * n,), "b")
+    c0 = _prep(c0, dtype, (B, n), "c0")
+    Y = _prep(Y, dtype, (T, B, n), "Y")
+    C = _prep(C, dtype, (T, B, n), "C")
+    DY = _prep(DY, dtype, (T, B, n), "DY")
+    Dd = _prep(Dd, dtype, (B, n), "Dd")
+    if not (T > 0 and 0 <= start < T and step != 0):
+        raise ValueError("oracle: need T > 0, 0 <= start < T and step != 0 (start=%r, step=%r, T=%r)" % (start, step, T))
+    DX = numpy.zeros((T, B, n_in), dtype=dtype)
+    DW = numpy.zeros((n_in + n, 4 * n), dtype=dtype)
+    Db = numpy.zeros((4 * n,), dtype=dtype)
+    Dh = numpy.zeros((B, n), dtype=dtype)
+    Dc = Dd.copy()
+    end = T - 1
+    if step < 0:
+        end = start
+        start = T - start - 1
+    if (step > 0 and (end - start) % step != 0) or (step < 0 and (start < end or (start - end) % (-step) != 0)):
+        raise ValueError("oracle: LstmLowMem gradient: the stride does not divide the distance between the first and the last frame")
+    one = dtype(1)
+
+    def sigmoid(z):
+        return one / (one + numpy.exp(-z))
+
+    t = end
+    while (t >= start) if step > 0 else (t <= start):
+        right = (t - step >= start) if step > 0 else (t - step <= start)
+        x_h = numpy.concatenate([X[t], Y[t - step] if right else y0], axis=1)
+        intern = x_h @ W + b[None, :]
+        prev_c = C[t - step] if right else c0
+        m = i[t][:, None]
+        d_y_b = DY[t] * m + Dh
+        d_c_b = Dc * m
+        cell_in, inp, fgt, out = numpy.tanh(intern[:, :n]), sigmoid(intern[:, n : 2 * n]), sigmoid(intern[:, 2 * n : 3 * n]), sigmoid(intern[:, 3 * n :])
+        gc = numpy.tanh(prev_c * fgt + cell_in * inp)
+        d_out = (one - out) * out * gc * d_y_b
+        d_c2 = d_c_b + out * d_y_b * (one - gc * gc)
+        d_cell_in = (one - cell_in * cell_in) * inp * d_c2
+        d_inp = (one - inp) * inp * cell_in * d_c2
+        d_fgt = (one - fgt) * fgt * prev_c * d_c2
+        Dc = fgt * d_c2 + Dc * (one - m)
+        d_intern = numpy.concatenate([d_cell_in, d_inp, d_fgt, d_out], axis=1)
+        Db += d_intern.sum(axis=0)
+        dx_h = d_intern @ W.T
+        DW += x_h.T @ d_intern
+        DX[t] = dx_h[:, :n_in]
+        Dh = dx_h[:, n_in:]
+        t -= step
+    return DX, DW, Db, Dh, Dc

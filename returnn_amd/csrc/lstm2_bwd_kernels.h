@@ -90,7 +90,8 @@ __global__ void k_bwd_pointwise(Lstm2BwdParams p, long long t, long long prev_t)
   const long long fo = t * bn * 4 + io;  // inside H / DX
   const float m = p.mask[t * p.B + b];
   const float dyw = p.dyw[idx];
-  const float d_y_b = (E::load(p.DY, t * bn + idx) + dyw) * m;
+  const bool raw_dh = (p.op_flags & kOpRawDh) != 0;
+  const float d_y_b = raw_dh ? E::load(p.DY, t * bn + idx) * m + dyw : (E::load(p.DY, t * bn + idx) + dyw) * m;
   const float dc = p.Dc0[idx];
   const float d_c_b = dc * m;
   const float prev_c = bwd_prev_cell<AT>(p, prev_t, idx, io);
@@ -102,7 +103,7 @@ __global__ void k_bwd_pointwise(Lstm2BwdParams p, long long t, long long prev_t)
   for (int g = 0; g < 4; ++g) {
     E::store(p.DX, fo + g * n, dx[g]);
     const float old = E::load(p.dx0, io + g * n);
-    E::store(p.dx0, io + g * n, dx[g] + old * (1.f - m));
+    E::store(p.dx0, io + g * n, raw_dh ? dx[g] : dx[g] + old * (1.f - m));
   }
   p.dyw[idx] = (p.op_flags & kOpNoCarry) ? 0.f : dyw * (1.f - m);
 }
@@ -211,7 +212,8 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
       const long long io = (long long)b * n4 + k;
       const long long fo = t * bn * 4 + io;
       const float m = q_m[nt];
-      const float d_y_b = (q_dy[nt] + dyw) * m;
+      const bool raw_dh = (p.op_flags & kOpRawDh) != 0;
+      const float d_y_b = raw_dh ? q_dy[nt] * m + dyw : (q_dy[nt] + dyw) * m;
       const float dc = q_dc[nt];
       const float d_c_b = dc * m;
       const float fgtGate = q_h[nt][2];
@@ -221,7 +223,7 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         E::store(p.DX, fo + g * n, dx[g]);
-        E::store(p.dx0, io + g * n, dx[g] + q_dx0[nt][g] * (1.f - m));
+        E::store(p.dx0, io + g * n, raw_dh ? dx[g] : dx[g] + q_dx0[nt][g] * (1.f - m));
       }
       dyw = (p.op_flags & kOpNoCarry) ? 0.f : dyw * (1.f - m);
     }
@@ -524,6 +526,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   };
 
   const int F = q.nframes;
+  const bool raw_dh = (p.op_flags & kOpRawDh) != 0;
   fetch(frame(0), F > 1 ? frame(1) : -1);
   for (int f = 0; f < F; ++f) {
     const long long t = frame(f);
@@ -533,7 +536,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
-      const float d_y_b = (in_dy[j] + dyw[j]) * m;
+      const float d_y_b = raw_dh ? in_dy[j] * m + dyw[j] : (in_dy[j] + dyw[j]) * m;
       const float d_c_b = dc[j] * m;
       const float fgtGate = in_gate[j][2];
       float dx[4];
@@ -544,7 +547,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
         for (int gq = 0; gq < 4; ++gq) SN::template store<kAuxDevice>(rs, (unsigned)((io[j] + (long long)gq * n) * ES), SN::bits(dx[gq]));
       }
 #pragma unroll
-      for (int gq = 0; gq < 4; ++gq) dx0[j][gq] = dx[gq] + dx0[j][gq] * (1.f - m);
+      for (int gq = 0; gq < 4; ++gq) dx0[j][gq] = raw_dh ? dx[gq] : dx[gq] + dx0[j][gq] * (1.f - m);
       dyw[j] = (p.op_flags & kOpNoCarry) ? 0.f : dyw[j] * (1.f - m);
     }
     RTN_BTRACE_MARK(5)  // pointwise part, stores of DX
@@ -583,6 +586,37 @@ __global__ void k_bwd_zero_unvisited(void* DX, long long T, long long frame_word
     const bool visited = t >= lo && t <= lo + (nframes - 1) * astep && ((t - lo) % astep) == 0;
     if (!visited) w[i] = 0u;
   }
+}
+
+// LstmLowMem gradient: the gates of every frame again from their pre-activations (returnn/native_op.py:683-687):
+// data[r, :] (rows of 4n) := [tanh, sigmoid, sigmoid, sigmoid](data[r, :] + bias), in place.
+template <typename AT>
+__global__ void k_low_mem_gates(void* data, const void* bias, long long rows, int n) {
+  using E = Elem<AT>;
+  const long long total = rows * 4 * n;
+  for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
+    const int col = (int)(i % (4 * n));
+    const float z = E::load(data, i) + E::load(bias, col);
+    E::store(data, i, col < n ? Act<AT>::tanh(z) : Act<AT>::sigmoid(z));
+  }
+}
+
+// Column sums of data[rows, width] in two deterministic stages: partial[r, c] = sum of rows r, r + R, ... (R = gridDim.y),
+// then out[c] = sum over r in ascending order.
+template <typename AT>
+__global__ void k_column_partial_sums(const void* data, float* partial, long long rows, int width) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  float acc = 0.f;
+  for (long long r = blockIdx.y; r < rows; r += gridDim.y) acc += Elem<AT>::load(data, r * width + c);
+  partial[(long long)blockIdx.y * width + c] = acc;
+}
+__global__ void k_column_final_sums(const float* partial, float* out, int parts, int width) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  float acc = 0.f;
+  for (int r = 0; r < parts; ++r) acc += partial[(long long)r * width + c];
+  out[c] = acc;
 }
 
 }  // namespace rtn

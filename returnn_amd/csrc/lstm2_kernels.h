@@ -97,7 +97,6 @@ struct Act<__bf16> {
   }
 };
 
-// Frame visited at step s.
 // True once a bounded wait of the launch has expired (status word 1; 2 marks a measurement run, which is not an error).
 __device__ __forceinline__ bool wait_expired(const unsigned* status) {
   return __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 1u;
@@ -108,6 +107,7 @@ constexpr unsigned kNanWords = 0x7FC00000u;
 template <>
 constexpr unsigned kNanWords<__bf16> = 0x7FC07FC0u;
 
+// Frame visited at step s.
 __device__ __forceinline__ long long frame_of(const Lstm2Params& p, int s) {
   return (long long)p.first + (long long)s * p.step;
 }

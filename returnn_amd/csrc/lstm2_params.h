@@ -19,6 +19,9 @@ enum OpFlags : int {
   kOpNoCarry = 1,    // the recurrent input of a frame is the OUTPUT of the frame before (0 where that frame was masked),
                      // not the last valid output carried over masked frames (LstmGenericBase, LstmLowMem)
   kOpH0IsCell = 2,   // the first block of H holds the cell state instead of tanh(cell-in) (LstmGenericBase)
+  kOpRawDh = 8,      // gradient kernels: the error arriving from the frame processed before is added to the output's error
+                     // unmasked (d_y = DY * mask + d_h) and the derivatives handed to the initial output are those of the
+                     // first visited frame alone: the LstmLowMem gradient as the reference has it (returnn/native_op.py:679)
   kOpEndAtStart = 4, // host side only: with a negative step the loop runs from frame T-start-1 down to frame `start`,
                      // not down to frame 0 (LstmLowMem's loop bounds, returnn/native_op.py:827-833)
 };

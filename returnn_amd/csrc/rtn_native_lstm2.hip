@@ -1226,6 +1226,21 @@ int dw_accumulate(rocblas_handle h, const void* A, const void* Bm, float* DW, lo
   return RTN_OK;
 }
 
+// Row-major C[M,N] = op(A) * op(B) + beta * C with float32 accumulation.  A is [M,K] (or [K,M] with trans_a), B is [K,N]
+// (or [N,K] with trans_b); A and B of element type `in`, C of element type `out`.
+int gemm_row_major(rocblas_handle h, bool trans_a, bool trans_b, long long M, long long N, long long K, const void* A, long long lda,
+                   const void* Bm, long long ldb, rocblas_datatype in, float beta, void* C, long long ldc, rocblas_datatype out) {
+  if (M <= 0 || N <= 0) return RTN_OK;
+  const float alpha = 1.f;
+  // in column-major terms: C^T [N,M] = op(B)^T * op(A)^T, and a row-major matrix is its transpose in column-major order
+  const rocblas_status st = rocblas_gemm_ex(h, trans_b ? rocblas_operation_transpose : rocblas_operation_none,
+                                            trans_a ? rocblas_operation_transpose : rocblas_operation_none, (rocblas_int)N, (rocblas_int)M,
+                                            (rocblas_int)K, &alpha, Bm, in, (rocblas_int)ldb, A, in, (rocblas_int)lda, &beta, C, out,
+                                            (rocblas_int)ldc, C, out, (rocblas_int)ldc, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+  if (st != rocblas_status_success) return fail(RTN_ERR_HIP, "rocblas_gemm_ex failed with status %d", (int)st);
+  return RTN_OK;
+}
+
 struct BwdLayout {
   size_t off_dyw = 0, off_dx0 = 0, off_wpk = 0, total = 0;  // [0, off_wpk) is cleared at the start of a call
 };
@@ -1284,7 +1299,7 @@ using namespace rtn;
 
 extern "C" {
 
-int rtn_native_lstm2_abi_version(void) { return 9; }
+int rtn_native_lstm2_abi_version(void) { return 10; }
 
 const char* rtn_native_lstm2_capture_report(void) {
   static thread_local std::string text;
@@ -1615,7 +1630,9 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     const char* names[] = {"W", "y0", "c0", "i", "Y", "C", "H", "DY", "Dd", "DX", "DW", "Dy0", "Dc0"};
     for (int q = 0; q < 13; ++q) {
       if (!ptrs[q]) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must not be null", names[q]);
-      if (q != 3 && !aligned16(ptrs[q])) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must be 16-byte aligned", names[q]);
+      // (W is read in 16-byte fragments only where n is a multiple of 16; the recurrent rows of a stacked matrix start at
+      // a multiple of 4n elements, which is aligned then)
+      if (q != 3 && !(q == 0 && n % 16 != 0) && !aligned16(ptrs[q])) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must be 16-byte aligned", names[q]);
     }
   }
   const int np = padded_width(n);
@@ -1792,6 +1809,11 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     j.abs_step = c.step > 0 ? c.step : -(long long)c.step;
     j.num_steps = (T - c.start + j.abs_step - 1) / j.abs_step;
     j.first = c.step > 0 ? c.start : T - c.start - 1;
+    if ((op_flags & kOpEndAtStart) && c.step < 0) {
+      // LstmLowMem: with a negative step the frames from T-start-1 down to `start` (returnn/native_op.py:957-963)
+      if (j.first < c.start) return fail(RTN_ERR_RANGE, "LstmLowMem gradient: start=%d with a negative step visits no frame of T=%lld", c.start, (long long)T);
+      j.num_steps = (j.first - c.start) / j.abs_step + 1;
+    }
     j.end = j.first + (j.num_steps - 1) * c.step;  // inclusive
     const long long words = (long long)((size_t)T * bn * 4 * es / 4);
     if (pk) {
@@ -1992,6 +2014,160 @@ int rtn_lstm_generic_base_bwd(const void* V_h, const float* c, const float* i, c
   // the cell states are the first block of H (kOpH0IsCell); the C argument is not read then
   const rtn_lstm2_bwd_call call = {V_h, y0, c, i, 0, 1, Y, (const float*)H, H, DY, Dd, DZ, DV_h, Dy0, Dc};
   return bwd_calls(&call, 1, T, B, n, dtype, workspace, bwd, hip_stream, kOpNoCarry | kOpH0IsCell);
+}
+
+namespace {
+constexpr int kColumnSumParts = 64;
+struct LowMemBwdLayout {
+  size_t bwd = 0, H = 0, DI = 0, partial = 0, total = 0;
+};
+void low_mem_bwd_layout(int64_t T, int B, int n, int dtype, LowMemBwdLayout* out) {
+  LowMemBwdLayout l;
+  l.bwd = 0;
+  size_t off = align_up(rtn_native_lstm2_bwd_workspace_bytes(T, B, n, dtype), 256);
+  const size_t frames = align_up((size_t)T * B * 4 * n * esize(dtype), 256);
+  l.H = off;
+  off += frames;
+  l.DI = off;
+  off += frames;
+  l.partial = off;
+  off += align_up((size_t)kColumnSumParts * 4 * n * 4, 256);
+  l.total = off;
+  *out = l;
+}
+}  // namespace
+
+size_t rtn_lstm_low_mem_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n_in, int32_t n, int32_t dtype) {
+  (void)n_in;
+  if (check_dims(T, B, n, dtype) != RTN_OK) return 0;
+  if (rtn_native_lstm2_bwd_workspace_bytes(T, B, n, dtype) == 0) return 0;
+  // gradient workspace of the recurrence | gates [T,B,4n] | their derivatives [T,B,4n] | partial column sums
+  LowMemBwdLayout l;
+  low_mem_bwd_layout(T, B, n, dtype, &l);
+  return l.total;
+}
+
+int rtn_lstm_low_mem_bwd(const void* X, const void* W, const void* b, const void* y0, const float* c0, const float* i, int32_t start,
+                         int32_t step, const void* Y, const float* C, const void* DY, const float* Dd, void* DX, float* DW, float* Db,
+                         void* Dh, float* Dc, int64_t T, int32_t B, int32_t n_in, int32_t n, int32_t dtype, void* workspace,
+                         size_t workspace_bytes, void* hip_stream) {
+  g_last_error.clear();
+  int rc = check_dims(T, B, n, dtype);
+  if (rc != RTN_OK) return rc;
+  if (n_in < 0) return fail(RTN_ERR_SHAPE, "LstmLowMem gradient: negative input dimension %d", n_in);
+  if (T == 0) return fail(RTN_ERR_SHAPE, "LstmLowMem gradient: needs T > 0");  // returnn/native_op.py:953
+  if (start < 0 || start >= T) return fail(RTN_ERR_RANGE, "LstmLowMem gradient: need 0 <= start < T, got start=%d, T=%lld", start, (long long)T);
+  if (step == 0) return fail(RTN_ERR_RANGE, "LstmLowMem gradient: step must not be 0");
+  // The reference's loop walks back from frame T-1 (step > 0) or up from frame `start` (step < 0) whatever the stride
+  // (:957-964); those are the frames its forward pass visited only if the stride divides the distance between the two
+  // ends.  Otherwise it would read outputs of frames that were never computed: refused.
+  const long long first = step > 0 ? start : T - start - 1, far_end = step > 0 ? T - 1 : start, astep = step > 0 ? step : -(long long)step;
+  if (step < 0 && first < far_end)
+    return fail(RTN_ERR_RANGE, "LstmLowMem gradient: start=%d with a negative step visits no frame of T=%lld", start, (long long)T);
+  if ((step > 0 ? far_end - first : first - far_end) % astep != 0)
+    return fail(RTN_ERR_RANGE, "LstmLowMem gradient: the stride %d does not divide the distance between frame %lld and frame %lld; the reference's gradient loop would visit frames its forward pass did not", step, first, far_end);
+  const long long num_steps = (step > 0 ? far_end - first : first - far_end) / astep + 1;
+  hipStream_t stream = (hipStream_t)hip_stream;
+  const size_t need = rtn_lstm_low_mem_bwd_workspace_bytes(T, B, n_in, n, dtype);
+  const long long bn = (long long)B * n, rows = (long long)T * B;
+  const size_t es = esize(dtype);
+  if (bn == 0) {
+    if (n_in > 0 && rows > 0) {
+      if (!DX) return fail(RTN_ERR_ARG, "LstmLowMem gradient: DX must not be null");
+      hipLaunchKernelGGL(k_fill_u32, dim3(256), dim3(256), 0, stream, (unsigned*)DX, 0u, (long long)(((size_t)rows * n_in * es + 3) / 4));
+      RTN_HIP(hipGetLastError());
+    }
+    return RTN_OK;
+  }
+  if (!workspace || workspace_bytes < need)
+    return fail(RTN_ERR_WORKSPACE, "LstmLowMem gradient: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
+  if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "LstmLowMem gradient: workspace must be 16-byte aligned");
+  {
+    const void* ptrs[] = {X, W, b, y0, c0, i, Y, C, DY, Dd, DX, DW, Db, Dh, Dc};
+    const char* names[] = {"X", "W", "b", "y0", "c0", "i", "Y", "C", "DY", "Dd", "DX", "DW", "Db", "Dh", "Dc"};
+    for (int q = 0; q < 15; ++q) {
+      if (!ptrs[q] && !((q == 0 || q == 10) && n_in == 0)) return fail(RTN_ERR_ARG, "LstmLowMem gradient: %s must not be null", names[q]);
+      if (q != 5 && ptrs[q] && !aligned16(ptrs[q])) return fail(RTN_ERR_ARG, "LstmLowMem gradient: %s must be 16-byte aligned", names[q]);
+    }
+  }
+  LowMemBwdLayout L;
+  low_mem_bwd_layout(T, B, n, dtype, &L);
+  unsigned char* ws = (unsigned char*)workspace;
+  void* H = ws + L.H;
+  void* DI = ws + L.DI;
+  float* partial = (float*)(ws + L.partial);
+  const unsigned char* W_rec = (const unsigned char*)W + (size_t)n_in * 4 * n * es;  // rows n_in.. of W: the recurrent part
+  float* DW_rec = DW + (size_t)n_in * 4 * n;
+  rocblas_handle blas = nullptr;
+  rc = blas_handle(&blas);
+  if (rc != RTN_OK) return rc;
+  if (rocblas_set_stream(blas, stream) != rocblas_status_success) return fail(RTN_ERR_HIP, "LstmLowMem gradient: rocblas_set_stream failed");
+  const rocblas_datatype ty = dtype == RTN_DTYPE_BF16 ? rocblas_datatype_bf16_r : rocblas_datatype_f32_r;
+  const int n4 = 4 * n;
+  const unsigned char* Yb = (const unsigned char*)Y;
+  unsigned char* Hb = (unsigned char*)H;
+  const size_t y_frame = (size_t)bn * es, h_frame = (size_t)bn * 4 * es;
+
+  // 1. The pre-activations of every frame again (:966-979): [X[t], Y[t-step] or y0] W.  The outputs are all known, so
+  //    this is no recurrence: one GEMM over all frames for the input part, one over all visited frames but the first
+  //    for the recurrent part (per frame if the stride is not 1), one for the first frame with y0.
+  if (n_in > 0) {
+    rc = gemm_row_major(blas, false, false, rows, n4, n_in, X, n_in, W, n4, ty, 0.f, H, n4, ty);
+    if (rc != RTN_OK) return rc;
+  } else {
+    hipLaunchKernelGGL(k_fill_u32, dim3(1024), dim3(256), 0, stream, (unsigned*)H, 0u, (long long)(((size_t)rows * n4 * es + 3) / 4));
+    RTN_HIP(hipGetLastError());
+  }
+  if (num_steps > 1) {
+    if (astep == 1) {
+      const long long lo = std::min(first, first + (num_steps - 1) * step);
+      // step +1: frames lo+1.. take Y[lo..]; step -1: frames lo.. take Y[lo+1..]
+      rc = gemm_row_major(blas, false, false, (num_steps - 1) * B, n4, n, Yb + (size_t)(lo + (step < 0 ? 1 : 0)) * y_frame, n, W_rec, n4, ty, 1.f,
+                          Hb + (size_t)(lo + (step > 0 ? 1 : 0)) * h_frame, n4, ty);
+      if (rc != RTN_OK) return rc;
+    } else {
+      for (long long s = 1; s < num_steps; ++s) {
+        const long long t = first + s * step;
+        rc = gemm_row_major(blas, false, false, B, n4, n, Yb + (size_t)(t - step) * y_frame, n, W_rec, n4, ty, 1.f, Hb + (size_t)t * h_frame, n4, ty);
+        if (rc != RTN_OK) return rc;
+      }
+    }
+  }
+  rc = gemm_row_major(blas, false, false, B, n4, n, y0, n, W_rec, n4, ty, 1.f, Hb + (size_t)first * h_frame, n4, ty);
+  if (rc != RTN_OK) return rc;
+  {
+    const long long total = rows * n4;
+    const dim3 grid((unsigned)std::min<long long>((total + 255) / 256, 65535)), block(256);
+    if (dtype == RTN_DTYPE_BF16)
+      hipLaunchKernelGGL(k_low_mem_gates<__bf16>, grid, block, 0, stream, H, b, rows, n);
+    else
+      hipLaunchKernelGGL(k_low_mem_gates<float>, grid, block, 0, stream, H, b, rows, n);
+    RTN_HIP(hipGetLastError());
+  }
+  // 2. The recurrence of the errors (:981-1017 without the two large products): the gradient kernels of NativeLstm2 on
+  //    the recurrent rows of W, with this op's variations.  Gives the derivatives of the pre-activations (DI), the
+  //    recurrent rows of DW, Dh and Dc.
+  const rtn_lstm2_bwd_call call = {W_rec, y0, c0, i, start, step, Y, C, H, DY, Dd, DI, DW_rec, Dh, Dc};
+  rc = bwd_calls(&call, 1, T, B, n, dtype, workspace, L.H, hip_stream, kOpNoCarry | kOpRawDh | kOpEndAtStart);
+  if (rc != RTN_OK) return rc;
+  // 3. What the reference accumulates frame by frame, as products over all frames at once (DI is 0 in frames that were not
+  //    visited): DX = DI W_x^T (:1001-1007, :1016), the input rows of DW = X^T DI (:1009-1014), Db = column sums of DI (:704-707).
+  if (n_in > 0) {
+    rc = gemm_row_major(blas, false, true, rows, n_in, n4, DI, n4, W, n4, ty, 0.f, DX, n_in, ty);
+    if (rc != RTN_OK) return rc;
+    rc = gemm_row_major(blas, true, false, n_in, n4, rows, X, n_in, DI, n4, ty, 0.f, DW, n4, rocblas_datatype_f32_r);
+    if (rc != RTN_OK) return rc;
+  }
+  {
+    const dim3 block(256), grid1((unsigned)((n4 + 255) / 256), kColumnSumParts), grid2((unsigned)((n4 + 255) / 256));
+    if (dtype == RTN_DTYPE_BF16)
+      hipLaunchKernelGGL(k_column_partial_sums<__bf16>, grid1, block, 0, stream, DI, partial, rows, n4);
+    else
+      hipLaunchKernelGGL(k_column_partial_sums<float>, grid1, block, 0, stream, DI, partial, rows, n4);
+    hipLaunchKernelGGL(k_column_final_sums, grid2, block, 0, stream, partial, Db, kColumnSumParts, n4);
+    RTN_HIP(hipGetLastError());
+  }
+  return RTN_OK;
 }
 
 size_t rtn_native_lstm2_bwd_multi_workspace_bytes(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype) {

@@ -31,7 +31,7 @@ MODE_PERSISTENT = 1
 MODE_GRAPH = 2
 MODE_STEPWISE = 3
 # The ABI version the structs and argument lists below were written for (rtn_native_lstm2_abi_version()).
-EXPECTED_ABI = 9
+EXPECTED_ABI = 10
 
 MODES = {"auto": MODE_AUTO, "persistent": MODE_PERSISTENT, "graph": MODE_GRAPH, "stepwise": MODE_STEPWISE}
 
@@ -56,6 +56,8 @@ SYMBOLS = (
     "rtn_lstm_generic_base_bwd_workspace_bytes",
     "rtn_lstm_low_mem_fwd",
     "rtn_lstm_low_mem_fwd_workspace_bytes",
+    "rtn_lstm_low_mem_bwd",
+    "rtn_lstm_low_mem_bwd_workspace_bytes",
     "rtn_native_lstm2_last_output",
     "rtn_last_error",
     "rtn_native_lstm2_describe_plan",
@@ -176,6 +178,10 @@ def load() -> ctypes.CDLL:
         lib.rtn_lstm_low_mem_fwd.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp, sz, vp]
         lib.rtn_lstm_low_mem_fwd_workspace_bytes.restype = sz
         lib.rtn_lstm_low_mem_fwd_workspace_bytes.argtypes = [i64, i32, i32, i32, i32, i32]
+        lib.rtn_lstm_low_mem_bwd.restype = ctypes.c_int
+        lib.rtn_lstm_low_mem_bwd.argtypes = [vp] * 6 + [i32, i32] + [vp] * 9 + [i64, i32, i32, i32, i32, vp, sz, vp]
+        lib.rtn_lstm_low_mem_bwd_workspace_bytes.restype = sz
+        lib.rtn_lstm_low_mem_bwd_workspace_bytes.argtypes = [i64, i32, i32, i32, i32]
         lib.rtn_native_lstm2_capture_report.restype = ctypes.c_char_p
         lib.rtn_native_lstm2_capture_report.argtypes = []
         lib.rtn_graph_cache_stats.restype = ctypes.c_int

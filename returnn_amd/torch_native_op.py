@@ -708,6 +708,74 @@ class LstmGenericBaseFunction(torch.autograd.Function):
         return (*(g.to(t) for g, t in zip(grads, ctx.in_dtypes)), None)
 
 
+def lstm_low_mem_grad(X, W, b, y0, c0, i, start, step, Y, C, DY, Dd):
+    """
+    The gradient op of ``LstmLowMem`` on HIP tensors (returnn/native_op.py:864-1026; arguments as its ``grad_input_map``
+    :619-625).  Results as the reference's formulas give them, also on masked frames; strides for which the reference's
+    loop would leave the frames of the forward pass are refused (see ``rtn_lstm_low_mem_bwd`` in the C header).
+
+    :return: DX [T,B,n_in] and Dh [B,n] in the element type of Y; DW [n_in+n,4n], Db [4n] and Dc [B,n] in float32
+    """
+    if not Y.is_cuda:
+        raise RuntimeError("LstmLowMem gradient: this build implements the op for HIP (MI355X) tensors only; got CPU tensors.")
+    bf16 = Y.dtype == torch.bfloat16
+    act = torch.bfloat16 if bf16 else torch.float32
+    device = Y.device
+    X, W, b, y0, Y, DY = (t.to(act).contiguous() for t in (X, W, b, y0, Y, DY))
+    c0, i, C, Dd = (t.to(torch.float32).contiguous() for t in (c0, i, C, Dd))
+    T, B = i.shape
+    n = y0.shape[1]
+    n_in = X.shape[2]
+    expect = {"X": (T, B, n_in), "W": (n_in + n, 4 * n), "b": (4 * n,), "y0": (B, n), "c0": (B, n), "Y": (T, B, n), "C": (T, B, n),
+              "DY": (T, B, n), "Dd": (B, n)}  # fmt: skip
+    for name, t in (("X", X), ("W", W), ("b", b), ("y0", y0), ("c0", c0), ("Y", Y), ("C", C), ("DY", DY), ("Dd", Dd)):
+        if tuple(t.shape) != expect[name]:
+            raise RuntimeError("LstmLowMem gradient: %s has shape %s, expected %s" % (name, tuple(t.shape), expect[name]))
+        if t.device != device:
+            raise RuntimeError("LstmLowMem gradient: %s is on %s but Y is on %s" % (name, t.device, device))
+    lib = _lib.load()
+    dtype = _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32
+    with torch.cuda.device(device):
+        status_watch.poll()
+        DX = torch.empty((T, B, n_in), dtype=act, device=device)
+        DW = torch.empty((n_in + n, 4 * n), dtype=torch.float32, device=device)
+        Db = torch.empty((4 * n,), dtype=torch.float32, device=device)
+        Dh = torch.empty((B, n), dtype=act, device=device)
+        Dc = torch.empty((B, n), dtype=torch.float32, device=device)
+        ws = torch.empty((max(int(lib.rtn_lstm_low_mem_bwd_workspace_bytes(T, B, n_in, n, dtype)), 256),), dtype=torch.uint8, device=device)
+        rc = lib.rtn_lstm_low_mem_bwd(
+            X.data_ptr(), W.data_ptr(), b.data_ptr(), y0.data_ptr(), c0.data_ptr(), i.data_ptr(), int(start), int(step), Y.data_ptr(),
+            C.data_ptr(), DY.data_ptr(), Dd.data_ptr(), DX.data_ptr(), DW.data_ptr(), Db.data_ptr(), Dh.data_ptr(), Dc.data_ptr(),
+            T, B, n_in, n, dtype, ws.data_ptr(), ws.numel(), torch.cuda.current_stream(device).cuda_stream,
+        )  # fmt: skip
+        _lib.check(rc)
+        if T * B * n > 0:  # (an empty problem does not touch its workspace)
+            status_watch.after_call("LstmLowMem gradient", ws, 1, device)
+    return DX, DW, Db, Dh, Dc
+
+
+class LstmLowMemFunction(torch.autograd.Function):
+    """``LstmLowMem`` with its gradient: ``Y, C, d = LstmLowMemFunction.apply(X, W, b, y0, c0, i, start, step)``; gradients
+    flow from Y and d to X, W, b, y0 and c0 (C is a non-differentiable output, as in the reference :596; the mask gets none)."""
+
+    @staticmethod
+    def forward(ctx, X, W, b, y0, c0, i, start, step):
+        Y, C, d = make_op(native_op.LstmLowMem)(X, W, b, y0, c0, i, int(start), int(step))
+        ctx.save_for_backward(X, W, b, y0, c0, i, Y, C)
+        ctx.start, ctx.step = int(start), int(step)
+        ctx.in_dtypes = (X.dtype, W.dtype, b.dtype, y0.dtype, c0.dtype)
+        ctx.mark_non_differentiable(C)
+        return Y, C, d
+
+    @staticmethod
+    def backward(ctx, DY, _DC, Dd):
+        X, W, b, y0, c0, i, Y, C = ctx.saved_tensors
+        DY = torch.zeros_like(Y) if DY is None else DY
+        Dd = torch.zeros_like(c0, dtype=torch.float32) if Dd is None else Dd
+        grads = lstm_low_mem_grad(X, W, b, y0, c0, i, ctx.start, ctx.step, Y, C, DY, Dd)
+        return (*(g.to(t) for g, t in zip(grads, ctx.in_dtypes)), None, None, None)
+
+
 class NativeLstm2PairFunction(torch.autograd.Function):
     """
     The two directions of a bidirectional layer as one differentiable call:

@@ -291,6 +291,111 @@ def test_generic_base_gradient_through_autograd():
         assert _rel_to_max(leaf.grad.cpu().numpy().astype(numpy.float64), r.grad.numpy()) <= 2e-5, name
 
 
+LOW_MEM_GRAD_SHAPES = [(6, 4, 12, 100), (5, 3, 4, 7), (7, 1, 16, 32), (6, 3, 40, 64), (9, 17, 24, 128), (12, 5, 8, 256), (1, 1, 1, 1), (8, 2, 5, 48)]
+
+
+def _low_mem_grad_case(seed, T, B, n_in, n, start, step, dtype, mask=None):
+    X, W, b, y0, c0, holes = low_mem_problem(seed, T, B, n_in, n)
+    mask = holes if mask is None else mask
+    rng = numpy.random.default_rng(seed + 1)
+    DY = rng.normal(0, 1, (T, B, n)).astype(numpy.float32)
+    Dd = rng.normal(0, 1, (B, n)).astype(numpy.float32)
+    get_op()
+    op = torch_native_op.make_op(native_op.LstmLowMem)
+    Xd, Wd, bd, y0d, DYd = (to_dev(a, dtype) for a in (X, W, b, y0, DY))
+    c0d, md, Ddd = to_dev(c0, "f32"), to_dev(mask, "f32"), to_dev(Dd, "f32")
+    Y, C, d = op(Xd, Wd, bd, y0d, c0d, md, start, step)
+    got = torch_native_op.lstm_low_mem_grad(Xd, Wd, bd, y0d, c0d, md, start, step, Y, C, DYd, Ddd)
+    torch.cuda.synchronize()
+    f = lambda t: t.float().cpu().numpy().astype(numpy.float64)  # noqa: E731
+    want = oracle.lstm_low_mem_bwd(f(Xd), f(Wd), f(bd), f(y0d), c0, mask, start, step, f(Y), f(C), f(DYd), Dd, dtype=numpy.float64)
+    return [f(a) for a in got], want
+
+
+@pytest.mark.parametrize("T,B,n_in,n", LOW_MEM_GRAD_SHAPES)
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_low_mem_gradient(T, B, n_in, n, dtype):
+    """
+    ``rtn_lstm_low_mem_bwd`` against the float64 restatement of the reference's gradient code, fed the GPU's own forward
+    results, with holes anywhere in the mask (on masked frames both sides follow the reference's formulas to the letter).
+    Judged like the other gradients: float32 within 2e-5, bfloat16 within 3e-2 of each array's largest magnitude (the
+    gates are computed again from bfloat16 products here, one rounding more than where the forward pass stored them).
+    """
+    announce("low_mem_gradient", T, B, n_in, n, dtype)
+    tol = 2e-5 if dtype == "f32" else 3e-2
+    for start, step in [(0, 1), (0, -1), (T - 1 - 2 * ((T - 1) // 2), 2), (1, -1), (0, -3)]:
+        if start < 0 or start >= T:
+            continue
+        first, far = (start, T - 1) if step > 0 else (T - start - 1, start)
+        if (step < 0 and first < far) or abs(first - far) % abs(step) != 0:
+            continue
+        got, want = _low_mem_grad_case(800 + T + B + n + n_in, T, B, n_in, n, start, step, dtype)
+        for name, a, w in zip(("DX", "DW", "Db", "Dh", "Dc"), got, want):
+            assert a.shape == w.shape and numpy.all(numpy.isfinite(a)), (name, start, step)
+            assert _rel_to_max(a, w) <= tol, (name, start, step, _rel_to_max(a, w))
+
+
+@pytest.mark.parametrize("kernel", [1, 2])
+def test_low_mem_gradient_kernels(kernel):
+    """Per-frame launches and the persistent gradient kernel give the same LstmLowMem gradients."""
+    from _gpu_util import env
+
+    announce("low_mem_gradient kernel", kernel)
+    with env(RTN_LSTM2_BWD_KERNEL=kernel):
+        for dtype, tol in (("f32", 2e-5), ("bf16", 3e-2)):
+            got, want = _low_mem_grad_case(850, 10, 6, 20, 128, 0, -1, dtype)
+            for name, a, w in zip(("DX", "DW", "Db", "Dh", "Dc"), got, want):
+                assert _rel_to_max(a, w) <= tol, (name, dtype, _rel_to_max(a, w))
+
+
+def test_low_mem_gradient_through_autograd():
+    """LstmLowMemFunction under torch.autograd against autograd through a plain torch restatement (float64, CPU) on a
+    right-padded batch, where the reference's formulas are the gradient of its forward pass."""
+    announce("low_mem_autograd")
+    T, B, n_in, n = 9, 5, 12, 32
+    X, W, b, y0, c0, _ = low_mem_problem(860, T, B, n_in, n)
+    lens = numpy.array([9, 4, 7, 1, 9])
+    mask = (numpy.arange(T)[:, None] < lens[None, :]).astype(numpy.float32)
+    rng = numpy.random.default_rng(861)
+    GY, Gd = rng.normal(0, 1, (T, B, n)), rng.normal(0, 1, (B, n))
+    ref = [torch.tensor(a.astype(numpy.float64), requires_grad=True) for a in (X, W, b, y0, c0)]
+    mt = torch.tensor(mask.astype(numpy.float64))
+    y_prev, c_prev, ys = ref[3], ref[4], []
+    for t in range(T):
+        z = torch.cat([ref[0][t], y_prev], dim=1) @ ref[1] + ref[2]
+        g, i, fg, o = torch.tanh(z[:, :n]), torch.sigmoid(z[:, n : 2 * n]), torch.sigmoid(z[:, 2 * n : 3 * n]), torch.sigmoid(z[:, 3 * n :])
+        m = mt[t][:, None]
+        c_new = (c_prev * fg + g * i) * m + c_prev * (1 - m)
+        y_prev, c_prev = torch.tanh(c_new) * o * m, c_new
+        ys.append(y_prev)
+    ((torch.stack(ys) * torch.tensor(GY)).sum() + (c_prev * torch.tensor(Gd)).sum()).backward()
+    get_op()
+    leaves = [to_dev(a, "f32").requires_grad_(True) for a in (X, W, b, y0, c0)]
+    Y, C, d = torch_native_op.LstmLowMemFunction.apply(*leaves, to_dev(mask, "f32"), 0, 1)
+    assert not C.requires_grad
+    ((Y * to_dev(GY, "f32")).sum() + (d * to_dev(Gd, "f32")).sum()).backward()
+    torch.cuda.synchronize()
+    for name, leaf, r in zip(("X", "W", "b", "y0", "c0"), leaves, ref):
+        assert _rel_to_max(leaf.grad.cpu().numpy().astype(numpy.float64), r.grad.numpy()) <= 2e-5, name
+
+
+def test_low_mem_gradient_refusals():
+    announce("low_mem_gradient refusals")
+    get_op()
+    T, B, n_in, n = 8, 2, 4, 32
+    z = lambda *s: torch.zeros(*s, device="cuda:0")  # noqa: E731
+    args = lambda start, step: (z(T, B, n_in), z(n_in + n, 4 * n), z(4 * n), z(B, n), z(B, n), z(T, B), start, step, z(T, B, n), z(T, B, n), z(T, B, n), z(B, n))  # noqa: E731
+    for start, step in ((0, 2), (2, 3), (1, -4)):
+        with pytest.raises(RuntimeError, match="stride"):
+            torch_native_op.lstm_low_mem_grad(*args(start, step))
+    with pytest.raises(RuntimeError, match="visits no frame"):
+        torch_native_op.lstm_low_mem_grad(*args(6, -1))
+    with pytest.raises(RuntimeError, match="step must not be 0"):
+        torch_native_op.lstm_low_mem_grad(*args(0, 0))
+    cabi = lib.load()
+    assert cabi.rtn_lstm_low_mem_bwd_workspace_bytes(T, B, n_in, n, lib.DTYPE_F32) > cabi.rtn_native_lstm2_bwd_workspace_bytes(T, B, n, lib.DTYPE_F32)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_sibling_ops_recorded_into_a_callers_graph(dtype):
     """LstmLowMem (whose input projection is a rocBLAS GEMM) and LstmGenericBase with its gradient under stream capture,

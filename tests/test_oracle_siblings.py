@@ -234,3 +234,108 @@ def test_generic_base_gradient_float32_close_to_float64():
         out[dt] = oracle.lstm_generic_base_bwd(r["V"], r["c0"], r["mask"], Y, H, GY, Gd, dtype=dt)
     for a, b in zip(out[numpy.float32], out[numpy.float64]):
         assert numpy.abs(a - b).max() <= 2e-5 * max(1.0, numpy.abs(b).max())
+
+
+def _low_mem_loss(r, start, step, GY, Gd):
+    Y, C, d = oracle.lstm_low_mem_fwd(r["X"], r["W"], r["b"], r["y0"], r["c0"], r["mask"], start, step, dtype=numpy.float64)
+    return float((Y * GY).sum() + (d * Gd).sum())
+
+
+LOW_MEM_GRAD_CASES = [
+    # T, start, step, mask: frames the forward pass visits = frames the reference's gradient loop visits
+    (6, 0, 1, "full"), (6, 0, -1, "full"), (7, 0, 2, "full"), (8, 1, 2, "full"), (7, 1, -1, "full"), (9, 2, -2, "full"),
+    (6, 0, 1, "right-padded"), (9, 2, 3, "right-padded"),
+]  # fmt: skip
+
+
+def _low_mem_mask(kind, T, B, rng):
+    if kind == "full":
+        return numpy.ones((T, B))
+    lens = rng.integers(1, T + 1, size=B)
+    lens[0] = T
+    return (numpy.arange(T)[:, None] < lens[None, :]).astype(numpy.float64)
+
+
+@pytest.mark.parametrize("T,start,step,kind", LOW_MEM_GRAD_CASES)
+def test_low_mem_gradient_vs_finite_differences(T, start, step, kind):
+    """Central differences of the (pinned) forward oracle for all five differentiable inputs."""
+    B, n, n_in = 3, 4, 5
+    r = _random(61 + T, T, B, n, n_in=n_in)
+    rng = numpy.random.default_rng(62)
+    r["mask"] = _low_mem_mask(kind, T, B, rng)
+    GY, Gd = rng.normal(0, 1, (T, B, n)), rng.normal(0, 1, (B, n))
+    Y, C, d = oracle.lstm_low_mem_fwd(r["X"], r["W"], r["b"], r["y0"], r["c0"], r["mask"], start, step, dtype=numpy.float64)
+    GY_dirty = GY + 3.0 * (1.0 - r["mask"])[:, :, None]  # error signals on masked frames must not matter
+    DX, DW, Db, Dh, Dc = oracle.lstm_low_mem_bwd(r["X"], r["W"], r["b"], r["y0"], r["c0"], r["mask"], start, step, Y, C, GY_dirty, Gd)
+    got = {"X": DX, "W": DW, "b": Db, "y0": Dh, "c0": Dc}
+    eps = 1e-6
+    for name in ("X", "W", "b", "y0", "c0"):
+        flat = r[name].reshape(-1)
+        for idx in rng.choice(flat.size, size=min(flat.size, 50), replace=False):
+            old = flat[idx]
+            flat[idx] = old + eps
+            lp = _low_mem_loss(r, start, step, GY, Gd)
+            flat[idx] = old - eps
+            lm = _low_mem_loss(r, start, step, GY, Gd)
+            flat[idx] = old
+            num = (lp - lm) / (2 * eps)
+            assert abs(num - got[name].reshape(-1)[idx]) <= 3e-6 * max(1.0, abs(num)), (name, idx, num, got[name].reshape(-1)[idx])
+
+
+def test_low_mem_gradient_vs_torch_autograd():
+    """Autograd through a plain torch restatement of the forward pass, right-padded batch, both inputs of the stacked
+    weight matrix."""
+    import torch
+
+    T, B, n, n_in = 8, 4, 5, 3
+    r = _random(63, T, B, n, n_in=n_in)
+    rng = numpy.random.default_rng(64)
+    r["mask"] = _low_mem_mask("right-padded", T, B, rng)
+    GY, Gd = rng.normal(0, 1, (T, B, n)), rng.normal(0, 1, (B, n))
+    X, W, b, y0, c0 = (torch.tensor(r[k], requires_grad=True) for k in ("X", "W", "b", "y0", "c0"))
+    mask = torch.tensor(r["mask"])
+    y_prev, c_prev, ys = y0, c0, []
+    for t in range(T):
+        z = torch.cat([X[t], y_prev], dim=1) @ W + b
+        g, i, f, o = torch.tanh(z[:, :n]), torch.sigmoid(z[:, n : 2 * n]), torch.sigmoid(z[:, 2 * n : 3 * n]), torch.sigmoid(z[:, 3 * n :])
+        m = mask[t][:, None]
+        c_new = (c_prev * f + g * i) * m + c_prev * (1 - m)
+        y_prev, c_prev = torch.tanh(c_new) * o * m, c_new
+        ys.append(y_prev)
+    ((torch.stack(ys) * torch.tensor(GY)).sum() + (c_prev * torch.tensor(Gd)).sum()).backward()
+    Y, C, d = oracle.lstm_low_mem_fwd(r["X"], r["W"], r["b"], r["y0"], r["c0"], r["mask"], 0, 1, dtype=numpy.float64)
+    got = oracle.lstm_low_mem_bwd(r["X"], r["W"], r["b"], r["y0"], r["c0"], r["mask"], 0, 1, Y, C, GY, Gd)
+    for name, a, t in zip(("DX", "DW", "Db", "Dh", "Dc"), got, (X, W, b, y0, c0)):
+        assert_allclose(a, t.grad.numpy(), rtol=1e-8, atol=1e-10, err_msg=name)
+
+
+def test_low_mem_gradient_agrees_with_native_lstm2_gradient_on_full_batches():
+    """With a full mask LstmLowMem is NativeLstm2 behind an input projection: DX = DXp W_x^T, DW = [X^T DXp; DW_rec],
+    Db = column sums of DXp, where DXp and DW_rec come from the (separately pinned) NativeLstm2 gradient oracle."""
+    T, B, n, n_in = 7, 3, 4, 6
+    r = _random(65, T, B, n, n_in=n_in)
+    r["mask"] = numpy.ones((T, B))
+    rng = numpy.random.default_rng(66)
+    GY, Gd = rng.normal(0, 1, (T, B, n)), rng.normal(0, 1, (B, n))
+    for start, step in ((0, 1), (0, -1)):
+        Y, C, d = oracle.lstm_low_mem_fwd(r["X"], r["W"], r["b"], r["y0"], r["c0"], r["mask"], start, step, dtype=numpy.float64)
+        DX, DW, Db, Dh, Dc = oracle.lstm_low_mem_bwd(r["X"], r["W"], r["b"], r["y0"], r["c0"], r["mask"], start, step, Y, C, GY, Gd)
+        Xp = r["X"] @ r["W"][:n_in] + r["b"]
+        Y2, C2, H2, d2 = oracle.native_lstm2_fwd(Xp, r["W"][n_in:], r["y0"], r["c0"], r["mask"], start, step, dtype=numpy.float64)[:4]
+        assert_allclose(Y2, Y, rtol=1e-12, atol=1e-12)
+        DXp, DWr, Dy0, Dc0 = oracle.native_lstm2_bwd(Xp, r["W"][n_in:], r["y0"], r["c0"], r["mask"], start, step, Y2, C2, H2, GY, Gd, dtype=numpy.float64)
+        assert_allclose(DX, DXp @ r["W"][:n_in].T, rtol=1e-9, atol=1e-11)
+        assert_allclose(DW[:n_in], numpy.einsum("tbi,tbj->ij", r["X"], DXp), rtol=1e-9, atol=1e-11)
+        assert_allclose(DW[n_in:], DWr, rtol=1e-9, atol=1e-11)
+        assert_allclose(Db, DXp.sum(axis=(0, 1)), rtol=1e-9, atol=1e-11)
+        assert_allclose(Dh, Dy0, rtol=1e-9, atol=1e-11)
+        assert_allclose(Dc, Dc0, rtol=1e-9, atol=1e-11)
+
+
+def test_low_mem_gradient_refuses_frame_sets_the_forward_pass_does_not_visit():
+    T, B, n, n_in = 8, 2, 3, 2
+    r = _random(67, T, B, n, n_in=n_in)
+    z = numpy.zeros
+    for start, step in ((0, 2), (2, 3), (1, -4)):  # T-1-start (or T-1-2*start) is not a multiple of the stride
+        with pytest.raises(ValueError, match="stride"):
+            oracle.lstm_low_mem_bwd(r["X"], r["W"], r["b"], r["y0"], r["c0"], r["mask"], start, step, z((T, B, n)), z((T, B, n)), z((T, B, n)), z((B, n)))
