@@ -35,6 +35,19 @@ PEAK_HBM = 8.0e12  # B/s
 # WRITE_SIZE runs of this same command (each counter scaled by what it reads for a plain 1 GiB device copy), whose
 # summaries sit under profiles/.  profiles/hbm_traffic_per_launch.json lists them by workload, launches per step and
 # plan text; a run whose plan is not in the list reports no traffic figure rather than somebody else's.
+def copy_calibration(args, dev):
+    """A plain device copy of known size before the timed region (``--copy-calibration-mib``): what FETCH_SIZE and
+    WRITE_SIZE read for it scales the counters of the kernels of interest in a profile of the same run."""
+    if args.copy_calibration_mib > 0:
+        import torch
+
+        src = torch.empty((args.copy_calibration_mib << 20,), dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads and writes copy_calibration_mib MiB each
+        torch.cuda.synchronize()
+        del src, dst
+
+
 def measured_traffic(workload: str, launches: int, plan: str):
     """-> (bytes per launch or None, the profile summary the figure is transcribed from or None)"""
     path = os.path.join(_root, "profiles", "hbm_traffic_per_launch.json")
@@ -488,6 +501,7 @@ def bench_gradient(args, dev, cabi):
                     a.W, a.y0, a.c0, a.i, a.start, a.step, a.Y, a.C, a.H, a.DY, a.Dd, a.DX, a.DW, a.Dy0, a.Dc0, T, B, n, dt_code,
                     ws.data_ptr() + k * each, each, stream.cuda_stream))  # fmt: skip
 
+    copy_calibration(args, dev)
     for _ in range(args.warmup):
         call()
     torch.cuda.synchronize()
@@ -525,6 +539,7 @@ def bench_gradient(args, dev, cabi):
                T, B, n, dtype, p.lens is not None),
             "calls_per_step": len(steps_of),
             "units_per_step": units,
+            "plan": lib.bwd_plan_text(),
         },
         "roofline": {
             "bound": "mfma",
@@ -790,12 +805,7 @@ def main():
         )  # fmt: skip
         lib.check(rc)
 
-    if args.copy_calibration_mib > 0:
-        src = torch.empty((args.copy_calibration_mib << 20,), dtype=torch.uint8, device=dev).fill_(1)
-        dst = torch.empty_like(src)
-        dst.copy_(src)  # reads and writes copy_calibration_mib MiB each
-        torch.cuda.synchronize()
-        del src, dst
+    copy_calibration(args, dev)
 
     launches = 1 if fused else len(directions)  # library entries per step
     for _ in range(args.warmup):

@@ -358,7 +358,12 @@ int rtn_graph_cache_stats(int64_t* out, int32_t n_out);
  * RTN_LSTM2_CAPTURE_NODE=plain does not try the cooperative attribute. */
 const char* rtn_native_lstm2_capture_report(void);
 
-/* ABI version of this header: 10. */
+/* The decomposition the last gradient call of the calling thread ran on (kernel, rows per batch group, tiles and
+ * wavefronts per workgroup, launches): the gradient entries' counterpart of rtn_native_lstm2_describe_plan, for logs,
+ * the benchmark line and tests.  "kernel=bwd_regw_xcd": every batch group on one XCD. */
+const char* rtn_native_lstm2_bwd_plan_text(void);
+
+/* ABI version of this header: 11. */
 int rtn_native_lstm2_abi_version(void);
 
 #ifdef __cplusplus

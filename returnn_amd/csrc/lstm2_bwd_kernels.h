@@ -262,11 +262,17 @@ __global__ void k_convert_from_f32(const float* src, void* dst, long long count)
 //    wavefront w holds the macro steps [w*ksb, (w+1)*ksb) of j, ksb <= KSB) and, in the pointwise part, the cells k of its rows.
 //    What a workgroup has to read per frame (rows x 4n values) is what its step time grows with -- a CU gets
 //    device-scope loads at only about 36 GB/s -- so the groups are made small (8 rows) when the device has the CUs.
-//  * exchange: DX itself.  The host fills DX with all-ones words (a NaN pattern no result can have: NaNs are
-//    canonicalised) before the launch; the workgroup that owns (b, k) writes the four gate derivatives of a frame
-//    once, with device-scope stores; every workgroup of the group reads the frame's rows as MFMA B fragments (DX is
-//    contiguous along j: a fragment is 16 bytes of a row) with device-scope loads and reads again until no element
-//    is all-ones.  A frame's memory is written once and never reused, so there is nothing to re-arm.
+//  * exchange: a ring of kExRing frames per group in the workspace, in MFMA B-operand order ([4n/KM macro steps][4 lane
+//    groups][Bp rows][16 bytes], Bp = 8 or 16): a wavefront's load of a fragment is contiguous memory, whole cache lines
+//    (reading DX itself, row-major, made every lane's 16 bytes a request of its own and bound the frame time by the
+//    requests a CU can have in flight).  The host fills the ring with all-ones words (a NaN pattern no result can have:
+//    NaNs are canonicalised); a workgroup stages the gate derivatives of its cells in LDS in that order and writes them
+//    with 16-byte stores: to the ring slot of the frame, to DX (row-major, the op's output, a plain stream), and all-ones
+//    again to the slot that was read two frames ago (every workgroup of the group is past it: they all delivered the
+//    frame processed before, which they could only do after reading that slot).  Readers load their share of the
+//    frame's slot as B fragments and read again until no element is all-ones.  With the group on one XCD (checked at
+//    the start, see group_on_one_xcd) the ring's stores are plain and the data goes from writer to readers through that
+//    XCD's L2; else stores and loads are device-scope.
 //  * per frame: wait for DX of the frame processed before, MFMA, sum of the 4 partial tiles through LDS, the
 //    pointwise part of this frame (inputs H, DY, C, mask fetched one frame ahead), DX out, first read of the
 //    next wait after an adaptive delay.  The cell error, the output error carried on and dx0 stay in registers.
@@ -284,7 +290,11 @@ struct Lstm2BwdPersistent {
   int ksb;            // macro steps of the contraction per wavefront (<= the kernel's KSB; the rest of its slots stay empty)
   int poll_delay;
   unsigned long long timeout_ticks;
+  unsigned* sync;     // [2 * groups of the whole problem] words of the XCD check (cleared before the launch)
+  void* ex;           // [groups of the whole problem][kExRing][4n * Bp] AT: the exchange ring (all-ones before the launch)
+  int Bp, bp_shift;   // rows of a ring frame: 8 or 16 (= 1 << bp_shift), >= Bg
 };
+constexpr int kExRing = 4;
 
 // Optional instrumentation (-DRTN_LSTM2_TRACE): thread 0 of every workgroup accumulates shader-clock ticks per phase
 // of the persistent gradient kernel into a device array that rtn_debug_bwd_trace() copies out.
@@ -307,7 +317,9 @@ constexpr int kMaxBwdMulti = 2;
 struct Lstm2BwdMulti {
   int count;     // problems, 1..kMaxBwdMulti
   int wgs_each;  // workgroups per problem = groups * n / (16 * MT)
-  int pad_[2];
+  int local;     // 1: every batch group sits on one XCD (workgroup id = slot * xcds + xcd; the groups of the launch, all
+                 // problems counted through, are dealt round-robin to the XCDs)
+  int xcds;      // XCDs the workgroup ids are dealt to (local plans)
   Lstm2BwdPersistent q[kMaxBwdMulti];
 };
 
@@ -318,13 +330,31 @@ struct Lstm2BwdMulti {
 //
 // KSL > 0: a wavefront's share of W is KSB fragments in registers plus KSL fragments in LDS (dynamic shared memory,
 // WV * KSL * 1024 bytes), for layers whose slice of W does not fit the registers next to a frame's DX.
-template <typename AT, int KSB, int MT, int WV, int KSL = 0>
+//
+// HALF (ring frames of 8 rows): a fragment of 8 rows fills only half of the 16 lanes per lane group, and what limits the
+// loads of a frame is the number of load instructions (each returns 1 KB to the registers, used or not).  So one load
+// takes two macro steps at once: the lanes of rows 0-7 read macro step 2a, the lanes of "rows" 8-15 read the same rows of
+// macro step 2a+1 -- 1 KB of consecutive memory.  As a B operand that register is right in columns 0-7 for the A
+// fragment of step 2a and right in columns 8-15 for the A fragment of step 2a+1: two MFMAs on the same register into two
+// accumulators, the first valid in columns 0-7, the second in columns 8-15, which are added when the partial tiles of
+// the wavefronts are.  Same number of MFMAs, half the load instructions, no data movement.
+template <typename AT, int KSB, int MT, int WV, int KSL = 0, bool HALF = false>
 __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti multi) {
+  static_assert(!HALF || KSL == 0, "the paired loads are not written for the chunked variants");
   constexpr int KST = KSB + KSL;           // fragment slots of a wavefront
   constexpr int TS = WV / 4;               // thread sets of 256
   constexpr int PT = (MT + TS - 1) / TS;   // tiles whose pairs a thread keeps
-  const int which = (int)blockIdx.x / multi.wgs_each;
-  const int bid = (int)blockIdx.x - which * multi.wgs_each;
+  int which, bid;
+  if (multi.local) {
+    const int kb = multi.q[0].p.n / (16 * MT), groups_now = multi.q[0].groups;
+    const int xcd = (int)blockIdx.x % multi.xcds, slot = (int)blockIdx.x / multi.xcds;
+    const int gg = (slot / kb) * multi.xcds + xcd;  // group of the launch, all problems counted through
+    which = gg / groups_now;
+    bid = (gg - which * groups_now) * kb + slot % kb;
+  } else {
+    which = (int)blockIdx.x / multi.wgs_each;
+    bid = (int)blockIdx.x - which * multi.wgs_each;
+  }
   if (which >= multi.count) return;
   const Lstm2BwdPersistent q = multi.q[which];
   using E = Elem<AT>;
@@ -332,7 +362,10 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   using LM = LaneMax<AT>;
   constexpr int KE = E::KE, KM = E::KM, ES = (int)sizeof(AT);
   const Lstm2BwdParams& p = q.p;
-  __shared__ f32x4 red[WV][MT][64];
+  // partial tiles of the wavefronts; a lane group's 16 entries are followed by 4 unused ones, so that the four groups of
+  // k that a wavefront's threads read together start 16 banks apart (without the gap they met in the same banks)
+  constexpr int kRedGroup = 20;
+  __shared__ f32x4 red[WV][MT][4 * kRedGroup];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // 0..WV-1
   const int n = p.n, n4 = 4 * n;
@@ -342,6 +375,18 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   const int rows = min(q.Bg, p.B - b_base);
   const long long bn = (long long)p.B * n;
   const unsigned frame_bytes = (unsigned)((size_t)p.B * n4 * ES);
+  // the exchange ring of this group: kExRing frames of [4n/KM][4][Bp][16 bytes]
+  const int Bp = q.Bp;
+  const unsigned ex_frame = (unsigned)((size_t)n4 * Bp * ES), frag_stride = (unsigned)(64 * Bp);
+  unsigned char* const ex_base = (unsigned char*)q.ex + (size_t)g * kExRing * ex_frame;
+  constexpr int KGW = 16 * MT / KE;  // 16-byte pieces per row and gate that this workgroup produces
+  __shared__ i32x4 stage[4 * KGW * 16];  // [gate][piece][row]: the workgroup's derivatives of a frame in ring order
+
+  // An XCD-local plan rests on all workgroups of a group being on one XCD: checked here.
+  __shared__ int s_local;
+  if (tid == 0) s_local = multi.local ? (int)group_on_one_xcd(q.sync + 2 * (size_t)g, (unsigned)kblocks, q.status, q.timeout_ticks) : 0;
+  __syncthreads();
+  const bool local = s_local != 0;
 
   // A fragments: this wavefront's macro steps [wave*ksb, (wave+1)*ksb) of the 16*MT rows of W, as far as the 4n/KM macro
   // steps reach.  Slots beyond them hold zeros in W and read nothing (or, in the chunked variants, a fragment that is
@@ -364,12 +409,10 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       for (int ks = KSB; ks < KST; ++ks) wl[(ks - KSB) * 64] = (ks < ks_here) ? *(const i32x4*)(Wr + (size_t)KM * ks) : i32x4{0, 0, 0, 0};
     }
   }
-  // byte offset of this lane's first B fragment inside a frame of DX; the others follow at KM*ES bytes each.  The lanes
-  // of rows the group lacks (half of them with 8-row groups) carry an out-of-range offset: their loads return 0 and
-  // take nothing through the CU's memory pipeline, which moves only 64 bytes per clock.
-  const unsigned foff0 = ((lane & 15) < rows)
-                             ? (unsigned)(((size_t)(b_base + (lane & 15)) * n4 + (size_t)KM * ksb * wave_at + KE * (lane >> 4)) * ES)
-                             : 0x80000000u;
+  // byte offset of this lane's first B fragment inside a ring frame; the others follow at frag_stride bytes each.  The
+  // lanes of rows the group lacks carry an out-of-range offset: their loads return 0.
+  const int lane_row = HALF ? (lane & 7) : (lane & 15), lane_hi = HALF ? ((lane >> 3) & 1) : 0;  // HALF: lanes 8-15 of a lane group take the next macro step
+  const unsigned foff0 = (lane_row < rows) ? (unsigned)(ksb * wave_at + lane_hi) * frag_stride + (unsigned)(((lane >> 4) * Bp + lane_row) * 16) : 0x80000000u;
 
   // The (row, k) pairs of this thread: one in each of its tiles.
   const int set = (TS == 1) ? 0 : __builtin_amdgcn_readfirstlane(tid >> 8);  // uniform over a wavefront
@@ -391,20 +434,42 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     for (int gq = 0; gq < 4; ++gq) dx0[j][gq] = 0.f;
   }
   // where a pair's element of the summed tile is: tile element D[kl][bl] sits in lane (kl/4)*16 + bl, component kl%4
-  const int red_lane = (kl >> 2) * 16 + bl, red_comp = kl & 3;
+  const int red_lane = (kl >> 2) * kRedGroup + (HALF ? (bl & 7) : bl), red_comp = kl & 3;
 
-  // inputs of a frame, fetched one frame ahead
-  float in_gate[PT][4], in_dy[PT], in_pc[PT], in_m;
+  // Inputs of a frame, fetched one frame ahead.  No branches around the loads and no arithmetic on what they bring: a
+  // register that receives its value on two paths, or feeds an instruction, makes the compiler wait for every load in
+  // flight at that point -- here that would be a memory latency in front of the ring's loads, every frame.  The cell
+  // state of the frame before is c0, C or (kOpH0IsCell) the first block of H: both sources are read, the one that does
+  // not apply through a descriptor of no bytes (no memory access, 0 comes back), and added where they are used.
+  float in_gate[PT][4], in_dy[PT], in_m;
+  unsigned in_pc[PT], in_ph[PT];
   auto fetch = [&](long long t, long long prev_t) {
+    const bool from_h = (p.op_flags & kOpH0IsCell) != 0 && prev_t >= 0;
+    const float* csrc = prev_t < 0 ? p.c0 : p.C + prev_t * bn;
+    __amdgpu_buffer_rsrc_t rs_c = __builtin_amdgcn_make_buffer_rsrc((void*)csrc, 0, from_h ? 0u : (unsigned)(bn * 4), kBufFlags);
+    __amdgpu_buffer_rsrc_t rs_ph = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.H + (size_t)(prev_t < 0 ? 0 : prev_t) * frame_bytes, 0,
+                                                                     from_h ? frame_bytes : 0u, kBufFlags);
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
       const long long fo = t * bn * 4 + io[j];
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) in_gate[j][gq] = E::load(p.H, fo + (long long)gq * n);
       in_dy[j] = E::load(p.DY, t * bn + idx[j]);
-      in_pc[j] = bwd_prev_cell<AT>(p, prev_t, idx[j], io[j]);
+      in_pc[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_c, (unsigned)(idx[j] * 4), 0, 0);
+      if constexpr (ES == 2)
+        in_ph[j] = __builtin_amdgcn_raw_buffer_load_b16(rs_ph, (unsigned)(io[j] * ES), 0, 0);
+      else
+        in_ph[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_ph, (unsigned)(io[j] * ES), 0, 0);
     }
     in_m = p.mask[t * p.B + b];
+  };
+  auto prev_cell = [&](int j) {
+    float vh;
+    if constexpr (ES == 2)
+      vh = (float)__builtin_bit_cast(AT, (unsigned short)in_ph[j]);
+    else
+      vh = __builtin_bit_cast(float, in_ph[j]);
+    return __builtin_bit_cast(float, in_pc[j]) + vh;
   };
   auto frame = [&](int f) { return q.t_end - (long long)f * q.step; };
 
@@ -414,16 +479,24 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   // this one.
   constexpr int CH = KSL == 0 ? KST : (WV >= 8 ? 8 : 16);
   constexpr int NCH = KST / CH;
-  i32x4 bf[NCH > 1 ? 2 : 1][CH];
-  auto issue_chunk = [&](long long t, int c, int slot) {
-    __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
+  constexpr int NB = HALF ? CH / 2 : CH;  // registers of B fragments per chunk
+  static_assert(!HALF || CH % 2 == 0, "paired loads need an even number of macro steps");
+  i32x4 bf[NCH > 1 ? 2 : 1][NB];
+  auto issue_chunk = [&](int f, int c, int slot) {  // f: ordinal of the frame whose derivatives are wanted
+    __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(ex_base + (size_t)(f & (kExRing - 1)) * ex_frame, 0, ex_frame, kBufFlags);
     asm volatile("" ::: "memory");  // other workgroups write this memory: really load again
     if constexpr (NCH == 1) {
       // an unused slot carries an out-of-range offset: 0 comes back and no memory is touched (the offsets stay in
       // registers over the frames, which measured faster than instruction immediates)
+      if constexpr (HALF) {
 #pragma unroll
-      for (int ks = 0; ks < CH; ++ks)
-        bf[slot][ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (ks < ks_here) ? foff0 + (unsigned)(ks * KM * ES) : 0x80000000u, 0, kAuxDevice));
+        for (int a = 0; a < NB; ++a)  // (an odd share: the upper lanes of its last pair read a macro step that meets zeros in W)
+          bf[slot][a] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (2 * a < ks_here) ? foff0 : 0x80000000u, (2 * a) * (int)frag_stride, kAuxDevice));
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < CH; ++ks)
+          bf[slot][ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (ks < ks_here) ? foff0 + (unsigned)ks * frag_stride : 0x80000000u, 0, kAuxDevice));
+      }
     } else {
       // 64 offsets would not fit the registers: an unused slot reads the wavefront's last used fragment again (complete
       // when the used ones are, and multiplied by zero); worked out again for every chunk
@@ -431,19 +504,19 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       asm volatile("" : "+s"(last));
 #pragma unroll
       for (int ks = 0; ks < CH; ++ks)
-        bf[slot][ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, foff0, min(c * CH + ks, last) * (KM * ES), kAuxDevice));
+        bf[slot][ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, foff0, min(c * CH + ks, last) * (int)frag_stride, kAuxDevice));
     }
   };
-  auto issue = [&](long long t) { issue_chunk(t, 0, 0); };
+  auto issue = [&](int f) { issue_chunk(f, 0, 0); };
   int delay = q.poll_delay;
   bool aborted = false;
   // d_h of the thread's pairs from DX of frame t (whose first read has been issued): wait, MFMA, sum over the
   // wavefronts; added to dyw.
   RTN_BTRACE_DECL
-  auto gemm = [&](long long t) {
+  auto gemm = [&](int t) {  // t: ordinal of the frame whose derivatives go through the product
     RTN_BTRACE_MARK(4)  // pointwise tail, fetch, delay, first read
     // independent partial sums keep the MFMA pipeline full (one chain would wait for every result)
-    constexpr int NACC = (MT >= 4 || KSB < 2) ? 1 : (MT == 2 || KSB < 4 ? 2 : 4);
+    constexpr int NACC = HALF ? 2 : ((MT >= 4 || KSB < 2) ? 1 : (MT == 2 || KSB < 4 ? 2 : 4));
     f32x4 part[MT][NACC];
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
@@ -453,7 +526,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       for (;;) {
         unsigned m = 0;
 #pragma unroll
-        for (int ks = 0; ks < CH; ++ks)
+        for (int ks = 0; ks < NB; ++ks)
 #pragma unroll
           for (int w = 0; w < 4; ++w) m = LM::fold(m, (unsigned)bf[slot][ks][w]);
         if (!__any(LM::has_sentinel(m))) break;
@@ -494,21 +567,39 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
 #pragma unroll
           for (int a = 0; a < NACC; ++a) part[mt][a] = f32x4{0.f, 0.f, 0.f, 0.f};
       }
+      if constexpr (HALF) {
 #pragma unroll
-      for (int ks = 0; ks < CH; ++ks)
+        for (int a = 0; a < NB; ++a)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const int s_ = c * CH + ks;
-          const i32x4 a = (s_ < KSB) ? wreg[mt][s_ < KSB ? s_ : 0] : wl[(s_ - KSB) * 64];
-          part[mt][ks % NACC] = E::mma(a, bf[slot][ks], part[mt][ks % NACC]);
-        }
+          for (int mt = 0; mt < MT; ++mt) {
+            part[mt][0] = E::mma(wreg[mt][2 * a], bf[slot][a], part[mt][0]);      // valid in columns 0-7
+            part[mt][1] = E::mma(wreg[mt][2 * a + 1], bf[slot][a], part[mt][1]);  // valid in columns 8-15
+          }
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < CH; ++ks)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const int s_ = c * CH + ks;
+            const i32x4 a = (s_ < KSB) ? wreg[mt][s_ < KSB ? s_ : 0] : wl[(s_ - KSB) * 64];
+            part[mt][ks % NACC] = E::mma(a, bf[slot][ks], part[mt][ks % NACC]);
+          }
+      }
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       f32x4 acc = part[mt][0];
+      if constexpr (HALF) {
+        // each column keeps the accumulator that is valid there (component by component: a select of whole vectors is
+        // compiled into an indexed read of a stack array)
+        const bool upper = (lane & 8) != 0;
 #pragma unroll
-      for (int a = 1; a < NACC; ++a) acc += part[mt][a];
-      red[wave][mt][lane] = acc;
+        for (int r = 0; r < 4; ++r) acc[r] = upper ? part[mt][1][r] : part[mt][0][r];
+      } else {
+#pragma unroll
+        for (int a = 1; a < NACC; ++a) acc += part[mt][a];
+      }
+      red[wave][mt][(lane >> 4) * kRedGroup + (lane & 15)] = acc;
     }
     RTN_BTRACE_MARK(1)  // MFMA, partial tiles to LDS
     __syncthreads();
@@ -518,7 +609,10 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       const int mt = (set + TS * j < MT) ? set + TS * j : 0;
       float sum = 0.f;
 #pragma unroll
-      for (int w = 0; w < WV; ++w) sum += ((const float*)&red[w][mt][red_lane])[red_comp];
+      for (int w = 0; w < WV; ++w) {
+        sum += ((const float*)&red[w][mt][red_lane])[red_comp];
+        if constexpr (HALF) sum += ((const float*)&red[w][mt][red_lane + 8])[red_comp];
+      }
       dyw[j] += sum;
     }
     __syncthreads();  // red is free for the next frame
@@ -527,37 +621,72 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
 
   const int F = q.nframes;
   const bool raw_dh = (p.op_flags & kOpRawDh) != 0;
+  const int bp_shift = q.bp_shift, pieces = (4 * KGW) << bp_shift;
+  const i32x4 ones = i32x4{-1, -1, -1, -1};
   fetch(frame(0), F > 1 ? frame(1) : -1);
   for (int f = 0; f < F; ++f) {
     const long long t = frame(f);
-    if (f > 0) gemm(frame(f - 1));
+    if (f > 0) gemm(f - 1);
     // pointwise part of frame t (returnn/native_op.py:1123-1180)
     const float m = in_m;
-    __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
       const float d_y_b = raw_dh ? in_dy[j] * m + dyw[j] : (in_dy[j] + dyw[j]) * m;
       const float d_c_b = dc[j] * m;
       const float fgtGate = in_gate[j][2];
       float dx[4];
-      const float d_c2 = bwd_cell<AT>(p.op_flags, in_gate[j][0], in_gate[j][1], fgtGate, in_gate[j][3], in_pc[j], d_y_b, d_c_b, dx);
+      const float d_c2 = bwd_cell<AT>(p.op_flags, in_gate[j][0], in_gate[j][1], fgtGate, in_gate[j][3], prev_cell(j), d_y_b, d_c_b, dx);
       dc[j] = fgtGate * d_c2 + dc[j] * (1.f - m);
-      if (act[j]) {
+      const int mt = set + TS * j;
+      if (mt < MT && bl < Bp) {
+        const int col = 16 * mt + kl;
 #pragma unroll
-        for (int gq = 0; gq < 4; ++gq) SN::template store<kAuxDevice>(rs, (unsigned)((io[j] + (long long)gq * n) * ES), SN::bits(dx[gq]));
+        for (int gq = 0; gq < 4; ++gq) {
+          const int at = (((gq * KGW + col / KE) << bp_shift) + bl) * KE + col % KE;  // element index inside `stage`
+          if constexpr (ES == 2)
+            ((unsigned short*)stage)[at] = (unsigned short)SN::bits(dx[gq]);
+          else
+            ((unsigned*)stage)[at] = SN::bits(dx[gq]);
+        }
       }
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) dx0[j][gq] = raw_dh ? dx[gq] : dx[gq] + dx0[j][gq] * (1.f - m);
       dyw[j] = (p.op_flags & kOpNoCarry) ? 0.f : dyw[j] * (1.f - m);
     }
-    RTN_BTRACE_MARK(5)  // pointwise part, stores of DX
-    // while the derivatives travel: the inputs of the next frame, then the first read of this frame's DX
-    if (f + 1 < F) fetch(frame(f + 1), f + 2 < F ? frame(f + 2) : -1);
+    __syncthreads();  // the frame's derivatives of this workgroup are staged
+    {
+      __amdgpu_buffer_rsrc_t rs_out = __builtin_amdgcn_make_buffer_rsrc(ex_base + (size_t)(f & (kExRing - 1)) * ex_frame, 0, ex_frame, kBufFlags);
+      __amdgpu_buffer_rsrc_t rs_arm = __builtin_amdgcn_make_buffer_rsrc(ex_base + (size_t)((f + 2) & (kExRing - 1)) * ex_frame, 0, ex_frame, kBufFlags);
+      __amdgpu_buffer_rsrc_t rs_dx = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
+      for (int c = tid; c < pieces; c += 64 * WV) {
+        const int row = c & (Bp - 1), cg = c >> bp_shift;  // cg = gate * KGW + piece
+        const int gate = cg / KGW, piece = cg - gate * KGW;
+        if (row < rows) {
+          const u32x4 v = __builtin_bit_cast(u32x4, stage[c]);
+          const unsigned eo = (unsigned)(((((gate * n + k0) / KE + piece) << bp_shift) + row) * 16);
+          const unsigned dxo = (unsigned)(((size_t)(b_base + row) * n4 + (size_t)gate * n + k0 + piece * KE) * ES);
+          if (local) {
+            __builtin_amdgcn_raw_buffer_store_b128(v, rs_out, eo, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, ones), rs_arm, eo, 0, 0);
+          } else {
+            __builtin_amdgcn_raw_buffer_store_b128(v, rs_out, eo, 0, kAuxDevice);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, ones), rs_arm, eo, 0, kAuxDevice);
+          }
+          __builtin_amdgcn_raw_buffer_store_b128(v, rs_dx, dxo, 0, 0);  // the op's output: a plain stream
+        }
+      }
+    }
+    RTN_BTRACE_MARK(5)  // pointwise part, staging, stores
+    // while the derivatives travel: the inputs of the next frame, then the first read of this frame's ring slot
+    {
+      const int fn = min(f + 1, F - 1);  // (past the end: the last frame's again, unused)
+      fetch(frame(fn), fn + 1 < F ? frame(fn + 1) : -1);
+    }
     if (!aborted)
       for (int d = 0; d < delay; ++d) __builtin_amdgcn_s_sleep(1);
-    issue(t);
+    issue(f);
   }
-  gemm(frame(F - 1));
+  gemm(F - 1);
   RTN_BTRACE_ADD(7, (unsigned long long)delay)
   RTN_BTRACE_FLUSH()
   // After a wait that ran into its bound the gradients are wrong without looking it: the workgroups that see the mark

@@ -20,6 +20,7 @@ namespace rtn {
 
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4;
+typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 
 constexpr int kWgThreads = 256;  // 4 wavefronts of 64
@@ -756,6 +757,37 @@ __device__ __forceinline__ unsigned xcc_id() {
   unsigned x;
   asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(x));
   return x & 0xFu;
+}
+
+// One thread per workgroup: are all `members` workgroups that share `words` on one XCD?  Every caller adds its XCD to the
+// mask words[1] and then itself to the count words[0] (both cleared before the launch; device-scope atomics whose result
+// is waited for, so the mask is complete when the count is).  The wait is bounded like every other (status[0] = 1 when it
+// expires; the answer is then "no").  A group found on several XCDs leaves its mask in status[1] for the record.
+__device__ __forceinline__ bool group_on_one_xcd(unsigned* words, unsigned members, unsigned* status, unsigned long long timeout_ticks) {
+  if (members <= 1) return true;
+  (void)__hip_atomic_fetch_or(words + 1, 1u << xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  (void)__hip_atomic_fetch_add(words, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  unsigned long long t0 = 0;
+  unsigned spins = 0;
+  bool complete = true;
+  while (__hip_atomic_load(words, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < members) {
+    if ((spins++ & 15u) == 0) {
+      if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { complete = false; break; }
+      const unsigned long long now = wall_clock64();
+      if (spins == 1) {
+        t0 = now;
+      } else if (now - t0 > timeout_ticks) {
+        __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        complete = false;
+        break;
+      }
+    }
+    __builtin_amdgcn_s_sleep(2);
+  }
+  const unsigned mask = __hip_atomic_load(words + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const bool ok = complete && (mask & (mask - 1)) == 0;
+  if (!ok) __hip_atomic_store(status + 1, mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return ok;
 }
 
 // HALF: the groups have at most 8 rows (NT == 1, MT even).  A tile then holds valid results in the lanes of rows 0..7

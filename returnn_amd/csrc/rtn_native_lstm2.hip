@@ -717,6 +717,7 @@ int launch_steps_graph(const Lstm2Params& p, const Plan& pl, int dtype, hipStrea
 // occupancy check before the call has established for a device that runs nothing else at that moment; every wait inside
 // is bounded, so a replay that does find the device shared ends with the status word set and NaN marks, not hung).
 // RTN_LSTM2_CAPTURE_NODE=plain skips the attempt; RTN_LSTM2_CAPTURE=steps records per-step launches as before.
+thread_local std::string g_bwd_plan_text;  // what the last gradient call of this thread ran on
 std::mutex g_capture_mu;
 long long g_capture_cooperative = 0, g_capture_plain = 0;
 std::string g_capture_refusal;  // why a cooperative node was refused, if it was
@@ -1176,10 +1177,10 @@ BwdRegwKernel bwd_regw_lds_kernel_for(int WV) {
 }
 
 // KSB: fragments of W per tile and wavefront; MT: tiles of 16 values of k per workgroup; WV: wavefronts per workgroup.
-template <typename AT>
+template <typename AT, bool HALF>
 BwdRegwKernel bwd_regw_kernel_for(int KSB, int MT, int WV) {
 #define RTN_CASE(ks, mt, wv) \
-  if (KSB == ks && MT == mt && WV == wv) return &k_lstm2_bwd_regw<AT, ks, mt, wv>;
+  if (KSB == ks && MT == mt && WV == wv) return &k_lstm2_bwd_regw<AT, ks, mt, wv, 0, HALF>;
   RTN_CASE(2, 1, 4) RTN_CASE(4, 1, 4) RTN_CASE(8, 1, 4) RTN_CASE(16, 1, 4) RTN_CASE(32, 1, 4)
   if constexpr (sizeof(AT) == 2) { RTN_CASE(64, 1, 4) }
   RTN_CASE(2, 2, 4) RTN_CASE(4, 2, 4) RTN_CASE(8, 2, 4) RTN_CASE(16, 2, 4) RTN_CASE(32, 2, 4)
@@ -1242,17 +1243,23 @@ int gemm_row_major(rocblas_handle h, bool trans_a, bool trans_b, long long M, lo
 }
 
 struct BwdLayout {
-  size_t off_dyw = 0, off_dx0 = 0, off_wpk = 0, total = 0;  // [0, off_wpk) is cleared at the start of a call
+  size_t off_sync = 0, off_dyw = 0, off_dx0 = 0, off_wpk = 0, off_ex = 0, total = 0;  // [0, off_wpk) is cleared at the start of a call
 };
 BwdLayout bwd_layout(int B, int n, int dtype) {
   BwdLayout l;
   size_t off = 256;  // status block, as in the forward workspace
+  l.off_sync = off;  // two words per batch group (at most B groups): the XCD check of the persistent kernel
+  off = align_up(off + (size_t)B * 8, 256);
   l.off_dyw = off;
   off = align_up(off + (size_t)B * n * 4, 256);
   l.off_dx0 = off;
   off = align_up(off + (size_t)B * 4 * n * esize(dtype), 256);
   l.off_wpk = off;  // W in fragment order, for per-frame launches
   if (n % 16 == 0) off = align_up(off + (size_t)4 * n * n * esize(dtype), 256);
+  // the exchange ring of the persistent kernel: kExRing frames of 4n x Bp elements per batch group; groups of at least 4
+  // rows in frames of 8, or of more than 8 rows in frames of 16: never more than 2B + 16 rows in all
+  l.off_ex = off;
+  if (n % 16 == 0) off = align_up(off + (size_t)kExRing * 4 * n * esize(dtype) * (2 * (size_t)B + 16), 256);
   l.total = off;
   return l;
 }
@@ -1299,7 +1306,9 @@ using namespace rtn;
 
 extern "C" {
 
-int rtn_native_lstm2_abi_version(void) { return 10; }
+int rtn_native_lstm2_abi_version(void) { return 11; }
+
+const char* rtn_native_lstm2_bwd_plan_text(void) { return g_bwd_plan_text.c_str(); }
 
 const char* rtn_native_lstm2_capture_report(void) {
   static thread_local std::string text;
@@ -1695,14 +1704,12 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
   // (2..32 fragments) and all workgroups of all problems can be on the device together.
   const void* pk = nullptr;
   int KSB = 0, bwd_mt = 1;  // KSB: macro steps of the contraction per wavefront
-  // Decomposition: batch groups of 8 or 16 rows (a workgroup's frame time grows with the rows x 4n values of DX it
-  // reads per frame at device scope), MT tiles of 16 values of k per workgroup (more tiles: fewer workgroups, more
-  // MFMA time each) and 4 or 8 wavefronts per workgroup (8: more loads in flight per CU and no register spills, but
-  // only with one tile).  Candidates in the order measured on MI355X (cfg3, ms per gradient call: one problem
-  // 8 x 1 x 8: 4.22, 8 x 1 x 4: 4.37; two problems in one launch 8 x 2 x 4: 5.5, 16 x 1 x 8: 6.1, 16 x 1 x 4: 6.5,
-  // 8 x 2 x 8: 6.6, 16 x 2 x 4: 7.1); the first whose workgroups are all on the device together.
+  // Decomposition: batch groups of 8 or 16 rows (a workgroup's frame time grows with the rows x 4n derivatives it
+  // reads per frame from the exchange ring), MT tiles of 16 values of k per workgroup (more tiles: fewer workgroups, more
+  // MFMA time each) and 4 or 8 wavefronts per workgroup.
   const long env_rows = env_long("RTN_LSTM2_BWD_ROWS", 0);
   int rows_per_group = 16, bwd_waves = kWaves, groups_per_launch = 0;
+  bool bwd_local = false;
   long long turn_rows = 0;
   const void* turn_pk = nullptr;
   int turn_cfg[5] = {0, 0, 0, 0, 0};
@@ -1715,7 +1722,15 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       const long env_mt = env_long("RTN_LSTM2_BWD_MT", 0);
       const long env_waves = env_long("RTN_LSTM2_BWD_WAVES", 0);
       // (rows per group, tiles per workgroup, wavefronts per workgroup)
-      const int candidates[][3] = {{8, 1, 8}, {8, 1, 4}, {8, 2, 4}, {16, 1, 8}, {16, 1, 4}, {16, 2, 4}, {8, 4, 4}, {16, 4, 4}};
+      // Candidates in the order measured on MI355X (cfg3 bf16 n=1024, ms per gradient call: one problem 8 x 1 x 4: 2.73,
+      // 8 x 1 x 8: 3.04, 8 x 2 x 4 on one XCD per group: 3.2, 16 x 1 x 8: 3.6; two problems in one launch 8 x 2 x 4 on one
+      // XCD per group: 3.53, spread: 3.78; cfg2 float32 n=512: 8 x 1 x 4 on one XCD per group 2.35, spread 2.56, 8 x 1 x 8:
+      // 2.55 / 2.79, 8 x 2 x 4: 3.4); the first whose workgroups are all on the device together.  A candidate whose groups
+      // fit an XCD each (n / (16 * tiles) workgroups, all groups of all problems in one launch) runs XCD-local: the ring
+      // then goes from writer to readers through that XCD's L2 instead of through memory.
+      const int candidates[][3] = {{8, 1, 4}, {8, 1, 8}, {8, 2, 4}, {16, 1, 4}, {16, 1, 8}, {16, 2, 4}, {8, 4, 4}, {16, 4, 4}};
+      const DeviceInfo di_b = device_info();
+      const long want_local = env_long("RTN_LSTM2_BWD_LOCAL", 1);
       for (const auto& cand : candidates) {
         const int rows = cand[0], mt = cand[1];
         const int wv = env_waves ? (int)env_waves : cand[2];
@@ -1736,7 +1751,9 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
         if (lds_share)
           kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_lds_kernel_for<__bf16>(wv) : bwd_regw_lds_kernel_for<float>(wv);
         else
-          kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16>(ksb_room, mt, wv) : bwd_regw_kernel_for<float>(ksb_room, mt, wv);
+          // ring frames of 8 rows: the variant whose loads take two macro steps at once
+          kfn = use_rows <= 8 ? (dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16, true>(ksb_room, mt, wv) : bwd_regw_kernel_for<float, true>(ksb_room, mt, wv))
+                              : (dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16, false>(ksb_room, mt, wv) : bwd_regw_kernel_for<float, false>(ksb_room, mt, wv));
         if (!kfn) continue;
         const size_t cand_lds = lds_share ? kBwdLdsShareBytes : 0;
         if (cand_lds) {
@@ -1746,6 +1763,19 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
         int per_cu = 0;
         RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kfn, 64 * wv, cand_lds));
         const long long groups_needed = (B + use_rows - 1) / use_rows;
+        const long long G_wgs = n / (16 * mt), cu_x = di_b.xcds > 0 ? di_b.cus / di_b.xcds : 0;
+        if (want_local && di_b.xcds > 1 && per_cu >= 1 && G_wgs <= cu_x * per_cu &&
+            (long long)di_b.xcds * ((cu_x * per_cu) / G_wgs) >= (long long)count * groups_needed) {
+          pk = (const void*)kfn;
+          bwd_mt = mt;
+          bwd_waves = wv;
+          KSB = ksb;
+          rows_per_group = use_rows;
+          groups_per_launch = (int)groups_needed;
+          bwd_lds = cand_lds;
+          bwd_local = true;
+          break;
+        }
         // batch groups of every problem that one launch can hold
         const long long fit = (long long)per_cu * device_info().cus / ((long long)count * (n / (16 * mt)));
         if (fit >= groups_needed) {
@@ -1789,6 +1819,16 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2 backward: the persistent kernel cannot run T=%lld B=%d n=%d", (long long)T, B, n);
   }
   const int bgroups = (B + rows_per_group - 1) / rows_per_group;
+  {
+    char buf[256];
+    if (pk)
+      snprintf(buf, sizeof(buf), "kernel=%s problems=%d rows_per_group=%d groups=%d tiles=%d waves=%d wgs_per_group=%d launches=%d",
+               bwd_local ? "bwd_regw_xcd" : "bwd_regw", count, rows_per_group, bgroups, bwd_mt, bwd_waves, n / (16 * bwd_mt),
+               (bgroups + groups_per_launch - 1) / std::max(groups_per_launch, 1));
+    else
+      snprintf(buf, sizeof(buf), "kernel=%s problems=%d launches_per_frame=%d", mfma ? "bwd_step" : "bwd_generic", count, mfma ? 1 : 2);
+    g_bwd_plan_text = buf;
+  }
 
   std::vector<BwdJob> jobs((size_t)count);
   for (int k = 0; k < count; ++k) {
@@ -1817,8 +1857,13 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     j.end = j.first + (j.num_steps - 1) * c.step;  // inclusive
     const long long words = (long long)((size_t)T * bn * 4 * es / 4);
     if (pk) {
-      // DX doubles as the exchange medium: armed with all-ones words, every visited frame is written by the kernel.
-      hipLaunchKernelGGL(k_fill_u32, dim3(2048), fill_block, 0, stream, (unsigned*)c.DX, 0xFFFFFFFFu, words);
+      // the exchange ring starts armed: all-ones words (the visited frames of DX are written by the kernel, the others
+      // zeroed behind it)
+      const int bp = rows_per_group > 8 ? 16 : 8;
+      const long long ring_words = (long long)((size_t)bgroups * kExRing * 4 * n * es * bp / 4);
+      if ((size_t)ring_words * 4 > lay.total - lay.off_ex)
+        return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: internal: exchange ring of %lld bytes does not fit its section", ring_words * 4);
+      hipLaunchKernelGGL(k_fill_u32, dim3(256), fill_block, 0, stream, (unsigned*)(j.ws + lay.off_ex), 0xFFFFFFFFu, ring_words);
       RTN_HIP(hipGetLastError());
     } else if (j.num_steps != T) {
       // frames the loop does not visit keep DX = 0 (:1385-1388)
@@ -1844,7 +1889,13 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       q.ksb = KSB;
       q.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", 20)));
       q.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);
+      q.sync = (unsigned*)(jobs[(size_t)k].ws + lay.off_sync);
+      q.ex = jobs[(size_t)k].ws + lay.off_ex;
+      q.Bp = rows_per_group > 8 ? 16 : 8;
+      q.bp_shift = rows_per_group > 8 ? 4 : 3;
     }
+    multi.local = bwd_local ? 1 : 0;
+    multi.xcds = device_info().xcds;
     // one cooperative launch per share of the batch groups (a single one unless the batch is too large for the device)
     for (int g0 = 0; g0 < bgroups; g0 += groups_per_launch) {
       const int groups_now = std::min(groups_per_launch, bgroups - g0);
@@ -1854,7 +1905,13 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
         multi.q[k].group_offset = g0;
       }
       void* args[] = {(void*)&multi};
-      rc = launch_coresident(pk, dim3((unsigned)(count * multi.wgs_each)), dim3((unsigned)(64 * bwd_waves)), args, (unsigned)bwd_lds, stream, capturing);
+      unsigned grid = (unsigned)(count * multi.wgs_each);
+      if (bwd_local) {
+        // workgroup id = slot * xcds + xcd: the groups of the launch are dealt round-robin to the XCDs
+        const int kb = n / (16 * bwd_mt), total_groups = count * groups_now;
+        grid = (unsigned)(multi.xcds * kb * ((total_groups + multi.xcds - 1) / multi.xcds));
+      }
+      rc = launch_coresident(pk, dim3(grid), dim3((unsigned)(64 * bwd_waves)), args, (unsigned)bwd_lds, stream, capturing);
       if (rc != RTN_OK) return rc;
     }
     for (int k = 0; k < count; ++k) {

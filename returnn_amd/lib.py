@@ -31,7 +31,7 @@ MODE_PERSISTENT = 1
 MODE_GRAPH = 2
 MODE_STEPWISE = 3
 # The ABI version the structs and argument lists below were written for (rtn_native_lstm2_abi_version()).
-EXPECTED_ABI = 10
+EXPECTED_ABI = 11
 
 MODES = {"auto": MODE_AUTO, "persistent": MODE_PERSISTENT, "graph": MODE_GRAPH, "stepwise": MODE_STEPWISE}
 
@@ -64,6 +64,7 @@ SYMBOLS = (
     "rtn_native_lstm2_describe_multi_plan",
     "rtn_graph_cache_stats",
     "rtn_native_lstm2_capture_report",
+    "rtn_native_lstm2_bwd_plan_text",
     "rtn_native_lstm2_abi_version",
 )
 
@@ -182,6 +183,8 @@ def load() -> ctypes.CDLL:
         lib.rtn_lstm_low_mem_bwd.argtypes = [vp] * 6 + [i32, i32] + [vp] * 9 + [i64, i32, i32, i32, i32, vp, sz, vp]
         lib.rtn_lstm_low_mem_bwd_workspace_bytes.restype = sz
         lib.rtn_lstm_low_mem_bwd_workspace_bytes.argtypes = [i64, i32, i32, i32, i32]
+        lib.rtn_native_lstm2_bwd_plan_text.restype = ctypes.c_char_p
+        lib.rtn_native_lstm2_bwd_plan_text.argtypes = []
         lib.rtn_native_lstm2_capture_report.restype = ctypes.c_char_p
         lib.rtn_native_lstm2_capture_report.argtypes = []
         lib.rtn_graph_cache_stats.restype = ctypes.c_int
@@ -213,6 +216,10 @@ def check(rc: int) -> None:
     (TORCH_CHECK -> RuntimeError, returnn/native_op.cpp:660)."""
     if rc != RTN_OK:
         raise RuntimeError(last_error() or ("NativeLstm2: error code %i" % rc))
+
+
+def bwd_plan_text() -> str:
+    return load().rtn_native_lstm2_bwd_plan_text().decode("utf8", "replace")
 
 
 def capture_report() -> str:
