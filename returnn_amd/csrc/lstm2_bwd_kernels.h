@@ -288,7 +288,7 @@ struct Lstm2BwdPersistent {
   int groups, Bg;     // batch groups of this launch and rows per group (<= 16)
   int group_offset;   // index of the launch's first group (a large batch runs as several launches in turn)
   int ksb;            // macro steps of the contraction per wavefront (<= the kernel's KSB; the rest of its slots stay empty)
-  int poll_delay;
+  int poll_delay, delay_inc, delay_dec_mask;
   unsigned long long timeout_ticks;
   unsigned* sync;     // [2 * groups of the whole problem] words of the XCD check (cleared before the launch)
   void* ex;           // [groups of the whole problem][kExRing][4n * Bp] AT: the exchange ring (all-ones before the launch)
@@ -546,10 +546,11 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       if (c == 0) {
         RTN_BTRACE_MARK(0)  // wait for the frame's DX
         RTN_BTRACE_ADD(6, spins)
+        // (as in the forward kernel: an adaptive delay across XCDs, one number for all within an XCD)
         if (spins)
-          delay = min(delay + 2, 64);
-        else if (delay > 0)
-          delay -= ((t & 15) == 15) ? 1 : 0;
+          delay = min(delay + q.delay_inc, 64);
+        else if (q.delay_inc && delay > 0)
+          delay -= ((t & q.delay_dec_mask) == q.delay_dec_mask) ? 1 : 0;
         // W lives in accumulation registers where it is at most half of that file: the B fragments fill up to half of
         // the ordinary registers, and a matrix instruction reads an A operand from either file (without this the compiler
         // parks part of W there anyway and copies four registers back in front of every MFMA, which halves the MFMA rate).

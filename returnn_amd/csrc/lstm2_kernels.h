@@ -1085,7 +1085,11 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     RTN_TRACE_DECL
     unsigned char *h_out = nullptr, *y_out_p = nullptr, *c_out = nullptr;
     const unsigned char *x_next = nullptr, *m_next = nullptr;
-    int delay = p.poll_delay;  // in units of s_sleep(1), about 64 clocks; adapts, see below
+    // in units of s_sleep(1), about 64 clocks; see below.  (A group that was planned for one XCD and found itself on
+    // several takes the numbers of a spread plan.)
+    const bool spread_after_all = multi.local && EX == kExDevice;
+    int delay = spread_after_all ? 20 : p.poll_delay;
+    const int delay_inc = spread_after_all ? 2 : p.delay_inc;
     // One time step; PAR = s & 1 selects the register sets and the LDS copies of X, `stage` = s % 3 the copy that
     // takes this step's outputs.
     //
@@ -1131,13 +1135,15 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       // (The builtin rather than inline assembly, so that the compiler's own wait-count bookkeeping sees it.)
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
       asm volatile("" ::: "memory");
-      // The first read is held back by `delay` so that it usually comes back complete: a read that comes back
-      // incomplete costs a whole extra round trip, waiting too long costs the wait itself.  Lengthen the delay when a
-      // read had to be repeated, shorten it while none has (one unit every (delay_dec_mask + 1) steps): the repeat
-      // rate settles near 1 / (2 * (delay_dec_mask + 1)).
+      // The first read is held back by `delay`: a read that comes back incomplete costs an extra round trip, waiting too
+      // long costs the wait itself.  Across XCDs a round trip is long, and the delay adapts: longer by `delay_inc` when a
+      // read had to be repeated, shorter by one unit every (delay_dec_mask + 1) steps while none has; the repeat rate
+      // settles where the two balance.  Within an XCD a repeat is cheap (a read from the L2 next
+      // door), and what costs is wavefronts drifting apart, each on a delay of its own, where every step ends with the
+      // slowest of them: there the delay is one number for all (delay_inc == 0).
       if (spins)
-        delay = min(delay + 2, 64);
-      else if ((s & p.delay_dec_mask) == p.delay_dec_mask && delay > 0)
+        delay = min(delay + delay_inc, 64);
+      else if (delay_inc && (s & p.delay_dec_mask) == p.delay_dec_mask && delay > 0)
         --delay;
       RTN_TRACE_MARK(7)  // outstanding stores acknowledged
       RTN_TRACE_ADD(6, spins)

@@ -62,6 +62,7 @@ struct Lstm2Params {
   int xcds;           // XCDs assumed for the blockIdx -> (group, rank) mapping
   int exchange;       // register kernel: 0 = normal operation; 3, 4 = measurement aids (see kExNoWait, kExProbe)
   int poll_delay;     // register kernel: s_sleep(1) repeats between the hidden-value stores and the first read of the next step
+  int delay_inc;      // register kernel: units added to the delay after a repeated read; 0 = the delay stays as it is
   int delay_dec_mask; // register kernel: the delay adapts downwards by one unit every (mask + 1) steps without a repeated read
   unsigned long long* trace;  // optional [workgroups][8] cycle totals per phase (instrumented builds only)
   int op_flags;       // OpFlags: variations of the recurrence for the sibling ops (0 = NativeLstm2)
