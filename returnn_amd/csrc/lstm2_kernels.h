@@ -685,7 +685,7 @@ __host__ __device__ constexpr RegwLds regw_lds(int es, int MT, int NT) {
   l.hs = off; off += 3u * l.x_copy;
   l.ys = off; off += (3u * l.y_copy + 15u) / 16u * 16u;
   l.cs = off; off += 3u * l.c_copy;
-  l.ml = off; off += 2u * rows * 4u;
+  l.ml = off; off += 2u * rows * 4u + 16u;  // two copies and a spare word
   l.total = off;
   return l;
 }
@@ -913,7 +913,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     unsigned char* xl = smem + L.xl + PAR * L.x_copy;
 #pragma unroll
     for (int i = 0; i < XCH; ++i) *(typename XC::T*)(xl + xlds[i]) = xv[PAR][i];
-    if (tid < ROWS) Ml[PAR * ROWS + tid] = mv[PAR];
+    Ml[tid < ROWS ? PAR * ROWS + tid : 2 * ROWS] = mv[PAR];  // (no branch: the other threads write to a spare word)
   };
   // Staged outputs of a step (LDS copy `copy` of three) -> registers -> H[t], Y[t], C[t]: in two halves, so that the
   // LDS reads can be issued ahead of a batch of MFMAs and the stores behind it.
