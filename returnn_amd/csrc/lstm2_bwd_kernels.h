@@ -343,7 +343,11 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   static_assert(!HALF || KSL == 0, "the paired loads are not written for the chunked variants");
   constexpr int KST = KSB + KSL;           // fragment slots of a wavefront
   constexpr int TS = WV / 4;               // thread sets of 256
-  constexpr int PT = (MT + TS - 1) / TS;   // tiles whose pairs a thread keeps
+  // tiles whose pairs a thread keeps.  A set of 256 threads covers 16 rows x 16 values of k; with at most 8 rows the
+  // threads of the upper 8 row slots take every other tile instead of idling (SPLIT), which halves the pairs, the loads
+  // and the pointwise work per thread.
+  constexpr bool SPLIT = HALF && ((MT + TS - 1) / TS) % 2 == 0;
+  constexpr int PT = SPLIT ? (MT + TS - 1) / TS / 2 : (MT + TS - 1) / TS;
   int which, bid;
   if (multi.local) {
     const int kb = multi.q[0].p.n / (16 * MT), groups_now = multi.q[0].groups;
@@ -365,7 +369,10 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   // partial tiles of the wavefronts; a lane group's 16 entries are followed by 4 unused ones, so that the four groups of
   // k that a wavefront's threads read together start 16 banks apart (without the gap they met in the same banks)
   constexpr int kRedGroup = 20;
-  __shared__ f32x4 red[WV][MT][4 * kRedGroup];
+  // (two copies where they are small, frames alternate: no barrier then between the sums of one frame and the partial
+  // tiles of the next)
+  constexpr int kRedCopies = (WV * MT * 4 * kRedGroup * 16 <= 24 * 1024) ? 2 : 1;
+  __shared__ f32x4 red2[kRedCopies][WV][MT][4 * kRedGroup];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // 0..WV-1
   const int n = p.n, n4 = 4 * n;
@@ -416,14 +423,17 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
 
   // The (row, k) pairs of this thread: one in each of its tiles.
   const int set = (TS == 1) ? 0 : __builtin_amdgcn_readfirstlane(tid >> 8);  // uniform over a wavefront
-  const int bl = (tid & 255) >> 4, kl = tid & 15;
+  const int kl = tid & 15;
+  const int bl = SPLIT ? ((tid & 127) >> 4) : ((tid & 255) >> 4);  // row slot
+  const int upper = SPLIT ? ((tid & 255) >> 7) : 0;                // SPLIT: which of a pair of tiles
+  auto tile_of = [&](int j) { return SPLIT ? set + TS * (2 * j + upper) : set + TS * j; };
   const int b = b_base + ((bl < rows) ? bl : 0);
   bool act[PT];  // the pair exists: the tile does, and the group has the row
   long long idx[PT], io[PT];
   float dyw[PT], dc[PT], dx0[PT][4];
 #pragma unroll
   for (int j = 0; j < PT; ++j) {
-    const int mt = set + TS * j;
+    const int mt = tile_of(j);
     act[j] = (mt < MT) && (bl < rows);
     const int k = k0 + 16 * ((mt < MT) ? mt : 0) + kl;
     idx[j] = (long long)b * n + k;
@@ -515,6 +525,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   RTN_BTRACE_DECL
   auto gemm = [&](int t) {  // t: ordinal of the frame whose derivatives go through the product
     RTN_BTRACE_MARK(4)  // pointwise tail, fetch, delay, first read
+    auto& red = red2[kRedCopies == 2 ? (t & 1) : 0];
     // independent partial sums keep the MFMA pipeline full (one chain would wait for every result)
     constexpr int NACC = HALF ? 2 : ((MT >= 4 || KSB < 2) ? 1 : (MT == 2 || KSB < 4 ? 2 : 4));
     f32x4 part[MT][NACC];
@@ -524,11 +535,14 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       unsigned long long t0 = 0;
       unsigned spins = 0;
       for (;;) {
-        unsigned m = 0;
+        // (four independent running maxima: one chain of dependent packed operations needs a wait state after every
+        // one of them, and there are up to 128 of them here)
+        unsigned mw[4] = {0, 0, 0, 0};
 #pragma unroll
         for (int ks = 0; ks < NB; ++ks)
 #pragma unroll
-          for (int w = 0; w < 4; ++w) m = LM::fold(m, (unsigned)bf[slot][ks][w]);
+          for (int w = 0; w < 4; ++w) mw[w] = LM::fold(mw[w], (unsigned)bf[slot][ks][w]);
+        const unsigned m = LM::fold(LM::fold(mw[0], mw[1]), LM::fold(mw[2], mw[3]));
         if (!__any(LM::has_sentinel(m))) break;
         if ((spins++ & 15u) == 0) {
           if (__hip_atomic_load(q.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { aborted = true; break; }
@@ -607,7 +621,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     RTN_BTRACE_MARK(2)  // barrier
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
-      const int mt = (set + TS * j < MT) ? set + TS * j : 0;
+      const int mt = (tile_of(j) < MT) ? tile_of(j) : 0;
       float sum = 0.f;
 #pragma unroll
       for (int w = 0; w < WV; ++w) {
@@ -616,8 +630,10 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       }
       dyw[j] += sum;
     }
-    __syncthreads();  // red is free for the next frame
-    RTN_BTRACE_MARK(3)  // sum over the wavefronts, barrier
+    // (With two copies this copy of `red` is written again two frames from now, behind that frame's staging barrier and
+    // the next frame's barrier above; `stage` is written again behind the barrier above.)
+    if constexpr (kRedCopies == 1) __syncthreads();  // red is free for the next frame
+    RTN_BTRACE_MARK(3)  // sum over the wavefronts
   };
 
   const int F = q.nframes;
@@ -638,7 +654,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       float dx[4];
       const float d_c2 = bwd_cell<AT>(p.op_flags, in_gate[j][0], in_gate[j][1], fgtGate, in_gate[j][3], prev_cell(j), d_y_b, d_c_b, dx);
       dc[j] = fgtGate * d_c2 + dc[j] * (1.f - m);
-      const int mt = set + TS * j;
+      const int mt = tile_of(j);
       if (mt < MT && bl < Bp) {
         const int col = 16 * mt + kl;
 #pragma unroll
