@@ -994,6 +994,13 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
 
   // A-operand fragments of this wave's k share: registers, for the whole sequence.  Slots past the
   // wave's share hold zeros and are paired with any complete fragment, so the step has no branches.
+  // With at most 8 rows per group (HALF) the lanes of rows 8-15 of a fragment would load nothing: they take the rows of
+  // the NEXT macro step instead (PAIRED), so that a wavefront's share of h comes in with half the load instructions (a
+  // CU's load path takes a wavefront's load instruction at about 16 clocks whatever its width, and the four wavefronts'
+  // loads are what the wait for h consists of).  The odd macro step's rows reach the lanes of rows 0-7 through a
+  // shift by 8 inside each group of 16 lanes.
+  constexpr bool PAIRED = HALF && NT == 1 && KSMAX % 2 == 0;
+  constexpr int NLD = PAIRED ? KSMAX / 2 : KSMAX;  // loads of B fragments per step
   i32x4 wreg[MT][KSMAX];
   unsigned foff[KSMAX][NT];  // where this lane's B-operand fragments are inside a ring buffer
 #pragma unroll
@@ -1010,6 +1017,15 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       // Lanes of rows the group does not have load nothing: an out-of-range offset gives zeros (a complete fragment)
       // without a memory access, so a group of few rows moves few bytes.
       foff[ks][nt] = (mine && 16 * nt + jl < rows) ? (unsigned)(((4 * sm + kg) * p.Bp + 16 * nt + jl) * kFragBytes) : kOobOffset;
+    }
+  }
+  if constexpr (PAIRED) {
+#pragma unroll
+    for (int a = 0; a < NLD; ++a) {
+      const int ks = 2 * a + ((jl >> 3) & 1);
+      const bool mine = ks < ks_count;
+      const int sm = mine ? wave + kWaves * ks : 0;
+      foff[a][0] = (mine && (jl & 7) < rows) ? (unsigned)(((4 * sm + kg) * p.Bp + (jl & 7)) * kFragBytes) : kOobOffset;
     }
   }
 
@@ -1100,9 +1116,9 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       asm volatile("" ::: "memory");  // other workgroups write this memory: really load again
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
-        if (16 * nt + jl < rows) {
+        if ((PAIRED ? (jl & 7) : 16 * nt + jl) < rows) {
 #pragma unroll
-          for (int ks = 0; ks < KSMAX; ++ks)
+          for (int ks = 0; ks < NLD; ++ks)
             bf[ks][nt] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(ring_rs, foff[ks][nt], soff, AUXL));
         }
     };
@@ -1148,7 +1164,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       for (;;) {
         unsigned m[4] = {0, 0, 0, 0};
 #pragma unroll
-        for (int ks = 0; ks < KSMAX; ++ks)
+        for (int ks = 0; ks < NLD; ++ks)
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -1197,6 +1213,15 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       // one block of straight-line code that the scheduler is told to weave: a wavefront that has a SIMD to itself
       // issues one instruction per 4 clocks, an MFMA keeps the matrix core busy for 16, so three other instructions fit
       // behind every MFMA for free -- but a run of them between two MFMAs drains the matrix core.
+      // PAIRED: the odd macro steps' rows, from lanes 8-15 of every group of 16 to lanes 0-7 (a row shift of the data
+      // parallel primitives: lane i takes lane i + 8, lanes without a source take 0)
+      i32x4 bf_odd[KSMAX / 2 + 1];
+      if constexpr (PAIRED) {
+#pragma unroll
+        for (int a = 0; a < NLD; ++a)
+#pragma unroll
+          for (int w = 0; w < 4; ++w) bf_odd[a][w] = __builtin_amdgcn_update_dpp(0, bf[a][0][w], 0x108 /* row_shl:8 */, 0xF, 0xF, true);
+      }
       flush_read(stage == 2 ? 0 : stage + 1);  // the copy of step s-2 is (s+1) % 3
       load_gate_inputs(IntTag<1 - PAR>{});
       put(par_tag);
@@ -1208,7 +1233,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) {
-            acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+            acc[mt][nt] = E::mma(wreg[mt][ks], PAIRED ? ((ks & 1) ? bf_odd[ks / 2] : bf[ks / 2][nt]) : bf[ks][nt], acc[mt][nt]);
             __builtin_amdgcn_sched_group_barrier(0x008, sizeof(AT) == 2 ? 1 : 4, 0);  // the MFMA(s) of one fragment ...
             __builtin_amdgcn_sched_group_barrier(0x096, 3, 0);                        // ... then up to three of the rest (VALU, SALU, VMEM, LDS)
           }

@@ -1072,8 +1072,8 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     // Device-scope stores take about a microsecond to become visible: a first read issued at once would
     // come back incomplete and cost a second round trip, so it is held back, and the kernel adapts the delay.  Within an
     // XCD the delay is a fixed one (tuned on MI355X over n = 64 ... 1024 and 1 ... 16 rows per group: the best fixed
-    // delay is within 2 % of these two everywhere, and 4 % to 13 % ahead of the adaptive one).
-    p.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", pl.local ? (pl.Bg > 8 ? 10 : 5) : 20)));
+    // delay is within 2 % of these four everywhere, and 4 % to 13 % ahead of the adaptive one).
+    p.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", pl.local ? (pl.Bg > 8 ? 10 : (dtype != RTN_DTYPE_BF16 ? 5 : (pl.MT >= 8 ? 6 : 3))) : 20)));
     {
       long dec = env_long("RTN_LSTM2_DELAY_DEC", 8);  // steps per unit of downward adaptation: a power of two
       int mask = 0;
