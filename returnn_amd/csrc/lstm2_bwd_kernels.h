@@ -2,6 +2,8 @@
 // (returnn/native_op.py:1288-1464, lstm_bwd_kernel :1123-1180).
 #pragma once
 
+#include <type_traits>
+
 #include "lstm2_kernels.h"
 
 namespace rtn {
@@ -453,6 +455,17 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   // not apply through a descriptor of no bytes (no memory access, 0 comes back), and added where they are used.
   float in_gate[PT][4], in_dy[PT], in_m;
   unsigned in_pc[PT], in_ph[PT];
+  // the frame after, on its way: as the loads bring it (a conversion next to the loads would be scheduled among the
+  // MFMAs and wait there for memory)
+  typedef typename std::conditional<ES == 2, unsigned short, unsigned>::type RawT;
+  unsigned nx_gate[PT][4], nx_dy[PT], nx_pc[PT], nx_ph[PT];
+  float nx_m;
+  auto widen = [](unsigned raw) {
+    if constexpr (ES == 2)
+      return __builtin_bit_cast(float, raw << 16);
+    else
+      return __builtin_bit_cast(float, raw);
+  };
   auto fetch = [&](long long t, long long prev_t) {
     const bool from_h = (p.op_flags & kOpH0IsCell) != 0 && prev_t >= 0;
     const float* csrc = prev_t < 0 ? p.c0 : p.C + prev_t * bn;
@@ -463,15 +476,26 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     for (int j = 0; j < PT; ++j) {
       const long long fo = t * bn * 4 + io[j];
 #pragma unroll
-      for (int gq = 0; gq < 4; ++gq) in_gate[j][gq] = E::load(p.H, fo + (long long)gq * n);
-      in_dy[j] = E::load(p.DY, t * bn + idx[j]);
-      in_pc[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_c, (unsigned)(idx[j] * 4), 0, 0);
+      for (int gq = 0; gq < 4; ++gq) nx_gate[j][gq] = ((const RawT*)p.H)[fo + (long long)gq * n];
+      nx_dy[j] = ((const RawT*)p.DY)[t * bn + idx[j]];
+      nx_pc[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_c, (unsigned)(idx[j] * 4), 0, 0);
       if constexpr (ES == 2)
-        in_ph[j] = __builtin_amdgcn_raw_buffer_load_b16(rs_ph, (unsigned)(io[j] * ES), 0, 0);
+        nx_ph[j] = __builtin_amdgcn_raw_buffer_load_b16(rs_ph, (unsigned)(io[j] * ES), 0, 0);
       else
-        in_ph[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_ph, (unsigned)(io[j] * ES), 0, 0);
+        nx_ph[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_ph, (unsigned)(io[j] * ES), 0, 0);
     }
-    in_m = p.mask[t * p.B + b];
+    nx_m = p.mask[t * p.B + b];
+  };
+  auto take_next = [&]() {  // what fetch() asked for becomes the current frame's inputs
+#pragma unroll
+    for (int j = 0; j < PT; ++j) {
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) in_gate[j][gq] = widen(nx_gate[j][gq]);
+      in_dy[j] = widen(nx_dy[j]);
+      in_pc[j] = nx_pc[j];
+      in_ph[j] = nx_ph[j];
+    }
+    in_m = nx_m;
   };
   auto prev_cell = [&](int j) {
     float vh;
@@ -481,6 +505,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       vh = __builtin_bit_cast(float, in_ph[j]);
     return __builtin_bit_cast(float, in_pc[j]) + vh;
   };
+  const int F = q.nframes;
   auto frame = [&](int f) { return q.t_end - (long long)f * q.step; };
 
   // The B fragments of a frame (the group's rows of DX, this wavefront's share of the contraction range) are taken in
@@ -577,6 +602,14 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       }
       if (c + 1 < NCH) issue_chunk(t, c + 1, slot ^ 1);
       if (c == 0) {
+        // The inputs of the frame after next's pointwise part (frame t + 2: frame t + 1's are in registers already), asked
+        // for here, behind the wait for the ring and in front of the MFMAs: a wavefront's loads count as returned in
+        // the order they were issued, so loads from memory issued in front of the ring's loads (as they were, at the
+        // end of a frame) made the wait for the ring a wait for memory.
+        if constexpr (SPLIT) {  // (= EARLY)
+          const int fn = min(t + 2, F - 1);  // (past the end: the last frame's again, unused)
+          fetch(frame(fn), fn + 1 < F ? frame(fn + 1) : -1);
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -636,14 +669,22 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     RTN_BTRACE_MARK(3)  // sum over the wavefronts
   };
 
-  const int F = q.nframes;
   const bool raw_dh = (p.op_flags & kOpRawDh) != 0;
   const int bp_shift = q.bp_shift, pieces = (4 * KGW) << bp_shift;
   const i32x4 ones = i32x4{-1, -1, -1, -1};
+  // EARLY: a frame's inputs are asked for two frames ahead, in front of the MFMAs (see gemm); otherwise one frame ahead,
+  // at the end of a frame.  (Measured: the kernels that keep one pair per thread gain 4 % from EARLY, the others lose.)
+  constexpr bool EARLY = SPLIT;
   fetch(frame(0), F > 1 ? frame(1) : -1);
+  if constexpr (EARLY) {
+    take_next();
+    const int f1 = min(1, F - 1);
+    fetch(frame(f1), f1 + 1 < F ? frame(f1 + 1) : -1);
+  }
   for (int f = 0; f < F; ++f) {
     const long long t = frame(f);
     if (f > 0) gemm(f - 1);
+    if constexpr (!EARLY) take_next();  // (asked for at the end of the frame before, or before the loop)
     // pointwise part of frame t (returnn/native_op.py:1123-1180)
     const float m = in_m;
 #pragma unroll
@@ -695,7 +736,9 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     }
     RTN_BTRACE_MARK(5)  // pointwise part, staging, stores
     // while the derivatives travel: the inputs of the next frame, then the first read of this frame's ring slot
-    {
+    if constexpr (EARLY) {
+      take_next();  // (asked for in front of the MFMAs of this frame's product, or before the loop)
+    } else {
       const int fn = min(f + 1, F - 1);  // (past the end: the last frame's again, unused)
       fetch(frame(fn), fn + 1 < F ? frame(fn + 1) : -1);
     }

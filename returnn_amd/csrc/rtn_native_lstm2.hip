@@ -1890,8 +1890,13 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       q.nframes = (int)jobs[(size_t)k].num_steps;
       q.Bg = (B + bgroups - 1) / bgroups;
       q.ksb = KSB;
-      q.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_BWD_POLL_DELAY", 20)));
-      q.delay_inc = (int)std::max<long>(0, std::min<long>(16, env_long("RTN_LSTM2_BWD_DELAY_INC", 2)));
+      // The kernels that keep one (row, k) pair per thread ask for a frame's inputs in front of the MFMAs, so only the
+      // delay stands between a frame's stores and the read of its ring slot: inside an XCD it is a fixed one there, as in
+      // the forward kernel (measured: 2.77 ms at 10 units against 2.82 adaptive and 2.87 / 2.86 at 4 / 16 for the layer).
+      const bool one_pair = rows_per_group <= 8 && ((bwd_mt + bwd_waves / 4 - 1) / (bwd_waves / 4)) % 2 == 0;
+      const bool fixed_delay = bwd_local && one_pair;
+      q.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_BWD_POLL_DELAY", fixed_delay ? 10 : 20)));
+      q.delay_inc = (int)std::max<long>(0, std::min<long>(16, env_long("RTN_LSTM2_BWD_DELAY_INC", fixed_delay ? 0 : 2)));
       {
         long dec = env_long("RTN_LSTM2_BWD_DELAY_DEC", 16);  // steps per unit of downward adaptation: a power of two
         int mask = 0;
