@@ -1731,12 +1731,17 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       // 2.55 / 2.79, 8 x 2 x 4: 3.4); the first whose workgroups are all on the device together.  A candidate whose groups
       // fit an XCD each (n / (16 * tiles) workgroups, all groups of all problems in one launch) runs XCD-local: the ring
       // then goes from writer to readers through that XCD's L2 instead of through memory.
-      const int candidates[][3] = {{8, 1, 4}, {8, 1, 8}, {8, 2, 4}, {16, 1, 4}, {16, 1, 8}, {16, 2, 4}, {8, 4, 4}, {16, 4, 4}};
+      // In front of them, for bf16 only and only where its groups fit an XCD each: 4 rows x 2 tiles, the kernel with one
+      // (row, k) pair per thread (one problem of cfg3: 4.82 ms against 5.03 for 8 x 1 x 4, whose groups of 64 workgroups
+      // span two XCDs; in float32 two tiles double an MFMA time that is long already: cfg2 3.1 ms against 2.3).
+      const int candidates[][4] = {{4, 2, 4, 1}, {8, 1, 4, 0}, {8, 1, 8, 0}, {8, 2, 4, 0}, {16, 1, 4, 0}, {16, 1, 8, 0}, {16, 2, 4, 0}, {8, 4, 4, 0}, {16, 4, 4, 0}};
       const DeviceInfo di_b = device_info();
       const long want_local = env_long("RTN_LSTM2_BWD_LOCAL", 1);
       for (const auto& cand : candidates) {
         const int rows = cand[0], mt = cand[1];
         const int wv = env_waves ? (int)env_waves : cand[2];
+        const bool local_only = cand[3] != 0;
+        if (local_only && (dtype != RTN_DTYPE_BF16 || env_mt || env_waves || (env_rows >= 1 && env_rows <= 16))) continue;
         if (env_mt && mt != env_mt) continue;
         const bool rows_forced = env_rows >= 1 && env_rows <= 16;  // an explicit row count replaces the candidates' own
         if (rows_forced && rows != 8) continue;                    // (one pass per MT is enough then)
@@ -1767,6 +1772,8 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
         RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kfn, 64 * wv, cand_lds));
         const long long groups_needed = (B + use_rows - 1) / use_rows;
         const long long G_wgs = n / (16 * mt), cu_x = di_b.xcds > 0 ? di_b.cus / di_b.xcds : 0;
+        if (local_only && n / 16 <= cu_x * per_cu) continue;  // (groups of one tile per workgroup fit an XCD themselves)
+        if (local_only && 2 * (long long)count * groups_needed * G_wgs < di_b.cus) continue;  // (few rows: the wider spread wins, cfg5 7.98 against 8.41 ms)
         if (want_local && di_b.xcds > 1 && per_cu >= 1 && G_wgs <= cu_x * per_cu &&
             (long long)di_b.xcds * ((cu_x * per_cu) / G_wgs) >= (long long)count * groups_needed) {
           pk = (const void*)kfn;
@@ -1779,6 +1786,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
           bwd_local = true;
           break;
         }
+        if (local_only) continue;
         // batch groups of every problem that one launch can hold
         const long long fit = (long long)per_cu * device_info().cus / ((long long)count * (n / (16 * mt)));
         if (fit >= groups_needed) {
