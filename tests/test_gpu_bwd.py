@@ -63,6 +63,28 @@ def test_bwd_bf16(T, B, n, step):
         assert _rel_to_max(a, b) <= 2e-2, (name, _rel_to_max(a, b))
 
 
+# (rows per group, tiles per workgroup, wavefronts per workgroup): decompositions of the persistent gradient kernel that the
+# plan picks for other shapes than the ones above -- one (row, k) pair per thread with 2 and 4 tiles, whole and half ring
+# frames, 8 wavefronts -- forced here on a small problem with ragged sequence lengths and a last group of fewer rows.
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("rows,tiles,waves", [(8, 2, 4), (8, 4, 4), (4, 2, 4), (3, 4, 4), (16, 2, 4), (12, 1, 4), (8, 1, 8), (8, 2, 8), (8, 4, 8)])
+def test_bwd_forced_decompositions(rows, tiles, waves, dtype):
+    from _gpu_util import env
+
+    T, B, n = 9, 21, 256
+    announce("bwd forced decomposition", rows, tiles, waves, dtype)
+    with env(RTN_LSTM2_BWD_KERNEL=2, RTN_LSTM2_BWD_ROWS=rows, RTN_LSTM2_BWD_MT=tiles, RTN_LSTM2_BWD_WAVES=waves):
+        got, want, _ = _run(T, B, n, dtype, 1, 2 if tiles == 2 else -1, seed=rows + 10 * tiles + waves)
+        plan = lib.bwd_plan_text()
+    if "bwd_regw" not in plan:
+        pytest.skip("no persistent kernel for this decomposition: " + plan)
+    assert "rows_per_group=%i" % rows in plan and "tiles=%i" % tiles in plan and "waves=%i" % waves in plan, plan
+    bar = 2e-2 if dtype == "bf16" else 2e-5
+    for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), got, want):
+        assert numpy.isfinite(a).all(), name
+        assert _rel_to_max(a, b) <= bar, (name, _rel_to_max(a, b), plan)
+
+
 def test_bwd_cfg2_reduced_f32():
     announce("bwd cfg2 reduced")
     p = synthetic.make_config("cfg2", T=60)

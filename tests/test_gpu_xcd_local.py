@@ -57,6 +57,10 @@ CASES = [
     (20, 200, 256, "bf16", 1),   # 13 rows per group (16 groups of 16 workgroups) or 25 (two batch tiles)
     (18, 32, 768, "bf16", 1),    # 24 workgroups per group: part of an XCD
     (22, 5, 64, "f32", 1),       # two groups per XCD
+    (15, 6, 96, "bf16", 1),      # 3 macro steps of the contraction over 4 wavefronts: one wavefront without a share
+    (13, 8, 160, "bf16", 2),     # 5 macro steps: the paired loads of h end on an odd step
+    (12, 7, 352, "bf16", 1),     # 11 macro steps
+    (11, 3, 224, "f32", 1),      # 14 macro steps in float32
     (16, 3, 32, "f32", 1),       # four groups per XCD
     (21, 9, 512, "bf16", 3),     # three problems
 ]
