@@ -506,6 +506,9 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     return __builtin_bit_cast(float, in_pc[j]) + vh;
   };
   const int F = q.nframes;
+  // EARLY: a frame's inputs are asked for two frames ahead, in front of the MFMAs (see gemm); otherwise one frame ahead,
+  // at the end of a frame.  (Measured: the kernels that keep one pair per thread gain 4 % from EARLY, the others lose.)
+  constexpr bool EARLY = SPLIT;
   auto frame = [&](int f) { return q.t_end - (long long)f * q.step; };
 
   // The B fragments of a frame (the group's rows of DX, this wavefront's share of the contraction range) are taken in
@@ -606,7 +609,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
         // for here, behind the wait for the ring and in front of the MFMAs: a wavefront's loads count as returned in
         // the order they were issued, so loads from memory issued in front of the ring's loads (as they were, at the
         // end of a frame) made the wait for the ring a wait for memory.
-        if constexpr (SPLIT) {  // (= EARLY)
+        if constexpr (EARLY) {
           const int fn = min(t + 2, F - 1);  // (past the end: the last frame's again, unused)
           fetch(frame(fn), fn + 1 < F ? frame(fn + 1) : -1);
         }
@@ -672,9 +675,6 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   const bool raw_dh = (p.op_flags & kOpRawDh) != 0;
   const int bp_shift = q.bp_shift, pieces = (4 * KGW) << bp_shift;
   const i32x4 ones = i32x4{-1, -1, -1, -1};
-  // EARLY: a frame's inputs are asked for two frames ahead, in front of the MFMAs (see gemm); otherwise one frame ahead,
-  // at the end of a frame.  (Measured: the kernels that keep one pair per thread gain 4 % from EARLY, the others lose.)
-  constexpr bool EARLY = SPLIT;
   fetch(frame(0), F > 1 ? frame(1) : -1);
   if constexpr (EARLY) {
     take_next();
