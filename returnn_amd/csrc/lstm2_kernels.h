@@ -158,7 +158,7 @@ __global__ void k_fill_unvisited(Lstm2Params p) {
 // cell = i/4, gate = i%4 -- i.e. the 16 rows of an M-tile are the 4 gates of 4 adjacent cells,
 // so that after the MFMA one lane holds all four gate pre-activations of one (cell, sequence).
 template <typename AT>
-__global__ void k_prepare_mfma(Lstm2Params p, int n_flags) {
+__device__ __forceinline__ void prepare_mfma(const Lstm2Params& p, int n_flags) {
   constexpr int KE = Elem<AT>::KE;
   constexpr int KM = Elem<AT>::KM;
   const long long gtid = blockIdx.x * (long long)blockDim.x + threadIdx.x;
@@ -234,6 +234,17 @@ __global__ void k_prepare_mfma(Lstm2Params p, int n_flags) {
 #pragma unroll
     for (int e = 0; e < KE; ++e) dst[e] = ((const AT*)p.W)[(long long)(k0 + e) * 4 * p.n + col];
   }
+}
+
+template <typename AT>
+__global__ void k_prepare_mfma(Lstm2Params p, int n_flags) {
+  prepare_mfma<AT>(p, n_flags);
+}
+
+// The same for all problems of a fused launch at once: blockIdx.y = problem.
+template <typename AT>
+__global__ void k_prepare_mfma_multi(Lstm2Multi multi, int n_flags) {
+  prepare_mfma<AT>(multi.p[blockIdx.y], n_flags);
 }
 
 // Widths the matrix-core kernels do not take run zero-padded: dst[rows_dst][blocks][n_pad] takes src[rows_src][blocks][n]

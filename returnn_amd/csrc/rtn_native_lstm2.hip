@@ -1107,11 +1107,15 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
       }
       const long long work = std::max<long long>((long long)n * n, bn);
       const dim3 pgrid((unsigned)std::min<long long>((work + 255) / 256, 2048)), pblock(256);
-      if (dtype == RTN_DTYPE_BF16)
-        hipLaunchKernelGGL(k_prepare_mfma<__bf16>, pgrid, pblock, 0, stream, p, pl.n_flags);
-      else
-        hipLaunchKernelGGL(k_prepare_mfma<float>, pgrid, pblock, 0, stream, p, pl.n_flags);
-      RTN_HIP(hipGetLastError());
+      // (the problems of a fused launch are prepared by one launch, in front of it)
+      const bool prepared_with_the_others = pk && pl.regw && pl.passes <= 1;
+      if (!prepared_with_the_others) {
+        if (dtype == RTN_DTYPE_BF16)
+          hipLaunchKernelGGL(k_prepare_mfma<__bf16>, pgrid, pblock, 0, stream, p, pl.n_flags);
+        else
+          hipLaunchKernelGGL(k_prepare_mfma<float>, pgrid, pblock, 0, stream, p, pl.n_flags);
+        RTN_HIP(hipGetLastError());
+      }
       if (pk && pl.regw && pl.passes > 1) {
         // the batch groups in turns: one cooperative launch per share of them
         for (int g0 = 0; g0 < pl.groups_total; g0 += pl.groups) {
@@ -1138,6 +1142,11 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
           multi.wgs_each = (int)align_up((size_t)pl.grid, (size_t)device_info().xcds);
           multi.local = pl.local ? 1 : 0;
           multi.xcds = device_info().xcds;
+          if (dtype == RTN_DTYPE_BF16)
+            hipLaunchKernelGGL(k_prepare_mfma_multi<__bf16>, dim3(pgrid.x, (unsigned)pending), pblock, 0, stream, multi, pl.n_flags);
+          else
+            hipLaunchKernelGGL(k_prepare_mfma_multi<float>, dim3(pgrid.x, (unsigned)pending), pblock, 0, stream, multi, pl.n_flags);
+          RTN_HIP(hipGetLastError());
           void* args[] = {(void*)&multi};
           const int wgs = (pending == 1 || pl.local) ? pl.grid : multi.wgs_each * pending;
           rc = launch_coresident(pk, dim3(wgs), dim3(kWgThreads), args, (unsigned)pl.lds_bytes, stream, capturing);
