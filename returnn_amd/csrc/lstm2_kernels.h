@@ -183,56 +183,40 @@ __device__ __forceinline__ void prepare_mfma(const Lstm2Params& p, int n_flags) 
   }
   // W -> Wp
   const int S = p.n / KM;
-  if (((unsigned long long)p.W & 15ull) == 0) {
-    // One macro step (KM rows of W) x 16 M-tiles (64 cells, 4 gates) per turn of a block, through LDS: the rows come in
-    // as 16-byte pieces of consecutive memory, the fragments leave as 1 KB per M-tile.  (Element by element from memory,
-    // as below, a lane's 8 loads of a bf16 fragment touch 8 rows of W and use 2 bytes of every line they fetch: for
-    // n = 1024 that took 14 us, four times what moving 16 MB takes.)
-    constexpr int ES = (int)sizeof(AT);
-    constexpr int MB = 16, SEG = 4 * MB * ES;           // bytes of one (row, gate) of a tile
-    constexpr int SEGP = SEG + (ES == 2 ? 8 : 16);     // padded so that the 16 (gate, cell) and 4 row groups of a
-    constexpr int ROWP = 4 * SEGP + (ES == 2 ? 4 : 0);  // fragment's lanes fall into different banks
-    constexpr int CPS = SEG / 16;
-    __shared__ unsigned tile[KM * ROWP / 4];
-    const int m_tiles = p.n / 4, m_blocks = (m_tiles + MB - 1) / MB;
-    for (int t = (int)blockIdx.x; t < S * m_blocks; t += (int)gridDim.x) {
-      const int sm = t % S, m0 = (t / S) * MB;
-      for (int c = (int)threadIdx.x; c < KM * 4 * CPS; c += (int)blockDim.x) {
-        const int part = c % CPS, gate = (c / CPS) % 4, k = c / (4 * CPS);
-        const int cell = 4 * m0 + part * (16 / ES);
-        if (cell < p.n) {
-          const u32x4 v = *(const u32x4*)((const AT*)p.W + (long long)(KM * sm + k) * 4 * p.n + gate * p.n + cell);
-          unsigned* dst = tile + (k * ROWP + gate * SEGP + part * 16) / 4;
-          dst[0] = v[0]; dst[1] = v[1]; dst[2] = v[2]; dst[3] = v[3];
-        }
+  // One macro step (KM rows of W) x 16 M-tiles (64 cells, 4 gates) per turn of a block, through LDS: the rows come in
+  // as 16-byte pieces of consecutive memory (the entries refuse a W that is not 16-byte aligned), the fragments leave as
+  // 1 KB per M-tile.  (Element by element from memory a lane's 8 loads of a bf16 fragment touch 8 rows of W and use 2
+  // bytes of every line they fetch: for n = 1024 that took 14 us, four times what moving 16 MB takes.)
+  constexpr int ES = (int)sizeof(AT);
+  constexpr int MB = 16, SEG = 4 * MB * ES;           // bytes of one (row, gate) of a tile
+  constexpr int SEGP = SEG + (ES == 2 ? 8 : 16);     // padded so that the 16 (gate, cell) and 4 row groups of a
+  constexpr int ROWP = 4 * SEGP + (ES == 2 ? 4 : 0);  // fragment's lanes fall into different banks
+  constexpr int CPS = SEG / 16;
+  __shared__ unsigned tile[KM * ROWP / 4];
+  const int m_tiles = p.n / 4, m_blocks = (m_tiles + MB - 1) / MB;
+  for (int t = (int)blockIdx.x; t < S * m_blocks; t += (int)gridDim.x) {
+    const int sm = t % S, m0 = (t / S) * MB;
+    for (int c = (int)threadIdx.x; c < KM * 4 * CPS; c += (int)blockDim.x) {
+      const int part = c % CPS, gate = (c / CPS) % 4, k = c / (4 * CPS);
+      const int cell = 4 * m0 + part * (16 / ES);
+      if (cell < p.n) {
+        const u32x4 v = *(const u32x4*)((const AT*)p.W + (long long)(KM * sm + k) * 4 * p.n + gate * p.n + cell);
+        unsigned* dst = tile + (k * ROWP + gate * SEGP + part * 16) / 4;
+        dst[0] = v[0]; dst[1] = v[1]; dst[2] = v[2]; dst[3] = v[3];
       }
-      __syncthreads();
-      for (int fi = (int)threadIdx.x; fi < MB * 64; fi += (int)blockDim.x) {
-        const int lane = fi & 63, ml = fi >> 6, i = lane & 15, kg = lane >> 4;
-        if (m0 + ml < m_tiles) {
-          const unsigned char* src = (const unsigned char*)tile + (KE * kg) * ROWP + (i & 3) * SEGP + (4 * ml + (i >> 2)) * ES;
-          struct { AT v[KE]; } frag;
-#pragma unroll
-          for (int e = 0; e < KE; ++e) frag.v[e] = *(const AT*)(src + e * ROWP);
-          *(u32x4*)((AT*)p.Wp + (((long long)(m0 + ml) * S + sm) * 64 + lane) * KE) = __builtin_bit_cast(u32x4, frag);
-        }
-      }
-      __syncthreads();
     }
-    return;
-  }
-  const long long n_frag = (long long)(p.n / 4) * S * 64;
-  for (long long f = gtid; f < n_frag; f += gsz) {
-    const int lane = (int)(f & 63);
-    const long long ms = f >> 6;
-    const int sm = (int)(ms % S);
-    const int m = (int)(ms / S);
-    const int i = lane & 15, kg = lane >> 4;
-    const int col = (i & 3) * p.n + 4 * m + (i >> 2);
-    const int k0 = KM * sm + KE * kg;
-    AT* dst = (AT*)p.Wp + f * KE;
+    __syncthreads();
+    for (int fi = (int)threadIdx.x; fi < MB * 64; fi += (int)blockDim.x) {
+      const int lane = fi & 63, ml = fi >> 6, i = lane & 15, kg = lane >> 4;
+      if (m0 + ml < m_tiles) {
+        const unsigned char* src = (const unsigned char*)tile + (KE * kg) * ROWP + (i & 3) * SEGP + (4 * ml + (i >> 2)) * ES;
+        struct { AT v[KE]; } frag;
 #pragma unroll
-    for (int e = 0; e < KE; ++e) dst[e] = ((const AT*)p.W)[(long long)(k0 + e) * 4 * p.n + col];
+        for (int e = 0; e < KE; ++e) frag.v[e] = *(const AT*)(src + e * ROWP);
+        *(u32x4*)((AT*)p.Wp + (((long long)(m0 + ml) * S + sm) * 64 + lane) * KE) = __builtin_bit_cast(u32x4, frag);
+      }
+    }
+    __syncthreads();
   }
 }
 

@@ -19,7 +19,7 @@ from oracle import lstm2_oracle as oracle
 import torch
 
 from returnn_amd import lib, synthetic
-from _gpu_util import announce, env, get_op, random_problem, run_op, run_raw
+from _gpu_util import announce, env, get_op, random_problem, run_op, run_raw, to_dev
 from _textbook import REFERENCE_START_STEP, reference_fixture, textbook_lstm, visited_slice
 
 pytestmark = pytest.mark.gpu
@@ -371,6 +371,29 @@ def test_batch_row_independence():
         for k in range(3):
             assert numpy.array_equal(full[k][:, b : b + 1], one[k])
         assert numpy.array_equal(full[3][b : b + 1], one[3])
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_weights_at_an_address_that_is_not_a_multiple_of_16(dtype):
+    """The kernels move W, X and the outputs in 16-byte pieces: a contiguous tensor that starts one element into its storage
+    is refused with a message that names it (the reference's wrapper has no such case: its tensors come from the
+    framework's allocator)."""
+    announce("unaligned W", dtype)
+    T, B, n = 7, 5, 96
+    X, W, y0, c0, i = random_problem(77, T, B, n)
+    op = get_op()
+    act = torch.bfloat16 if dtype == "bf16" else torch.float32
+    Xd, Wd, y0d = (to_dev(a, dtype) for a in (X, W, y0))
+    c0d, id_ = (to_dev(a, "f32") for a in (c0, i))
+    store = torch.empty((n * 4 * n + 8,), dtype=act, device="cuda:0")
+    shifted = store[1 : 1 + n * 4 * n].view(n, 4 * n)
+    shifted.copy_(Wd)
+    assert shifted.is_contiguous() and shifted.data_ptr() % 16 != 0 and Wd.data_ptr() % 16 == 0
+    with pytest.raises(RuntimeError, match="W must be 16-byte aligned"):
+        op(Xd, shifted, y0d, c0d, id_, 0, 1)
+    Y, C, H, d = op(Xd, Wd, y0d, c0d, id_, 0, 1)  # and the library is fine afterwards
+    torch.cuda.synchronize()
+    assert torch.isfinite(Y.float()).all()
 
 
 def test_argument_handling():
