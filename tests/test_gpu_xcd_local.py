@@ -118,3 +118,22 @@ def test_local_plan_start_step_and_masks_with_holes():
         assert "kernel=mfma_regw_xcd" in plan and words[0][:2] == [0, 0], (plan, words)
         for name, a, b in zip("YCHd", got[0], want[0]):
             assert numpy.array_equal(a, b), "%s start=%i step=%i" % (name, start, step)
+
+
+@pytest.mark.parametrize("delay,inc", [(0, 0), (64, 0), (0, 2), (20, 2)])
+def test_first_read_delay_only_moves_time(delay, inc):
+    """The delay between a step's exchange stores and the first read of the next step (fixed inside an XCD, adaptive
+    across XCDs) decides how often a read has to be repeated, never what is read: any setting gives the same bits."""
+    announce("first-read delay", delay, inc)
+    T, B, n, dtype = 30, 16, 512, "bf16"
+    problems = [random_problem(900 + k, T, B, n) for k in range(2)]
+    ss = [(0, 1), (0, -1)]
+    want, _, _ = _run(problems, dtype, "stepwise", ss)
+    for local in (1, 0):
+        with env(RTN_LSTM2_LOCAL=local, RTN_LSTM2_POLL_DELAY=delay, RTN_LSTM2_DELAY_INC=inc):
+            got, plan, words = _run(problems, dtype, "auto", ss)
+        assert ("kernel=mfma_regw_xcd" in plan) == bool(local), plan
+        for k in range(len(problems)):
+            assert words[k][0] == 0, (plan, words[k])
+            for name, a, b in zip("YCHd", got[k], want[k]):
+                assert numpy.array_equal(a, b), (plan, k, name)
