@@ -85,6 +85,24 @@ def test_bwd_forced_decompositions(rows, tiles, waves, dtype):
         assert _rel_to_max(a, b) <= bar, (name, _rel_to_max(a, b), plan)
 
 
+def test_bwd_read_delay_only_moves_time():
+    """The delay between a frame's stores and the read of its ring slot (and whether it adapts) decides how often a read is
+    repeated, never what is read: every setting gives the same bits, on a plan with one pair per thread and on one without."""
+    from _gpu_util import env
+
+    announce("bwd read delay")
+    for tiles in (2, 1):
+        results = []
+        for delay, inc in [(None, None), (0, 0), (64, 0), (3, 2)]:
+            with env(RTN_LSTM2_BWD_KERNEL=2, RTN_LSTM2_BWD_ROWS=8, RTN_LSTM2_BWD_MT=tiles, RTN_LSTM2_BWD_POLL_DELAY=delay, RTN_LSTM2_BWD_DELAY_INC=inc):
+                got, _, _ = _run(12, 19, 256, "bf16", 0, -1, seed=5)
+                assert "bwd_regw" in lib.bwd_plan_text() and "tiles=%i" % tiles in lib.bwd_plan_text(), lib.bwd_plan_text()
+            results.append(got)
+        for other in results[1:]:
+            for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), other, results[0]):
+                assert numpy.array_equal(a, b), (tiles, name)
+
+
 def test_bwd_cfg2_reduced_f32():
     announce("bwd cfg2 reduced")
     p = synthetic.make_config("cfg2", T=60)
