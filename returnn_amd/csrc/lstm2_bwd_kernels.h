@@ -546,7 +546,10 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     }
   };
   auto issue = [&](int f) { issue_chunk(f, 0, 0); };
-  int delay = q.poll_delay;
+  // (A group that was planned for one XCD and found itself on several takes the adaptive delay of a spread plan.)
+  const bool spread_after_all = multi.local && !local;
+  int delay = spread_after_all ? 20 : q.poll_delay;
+  const int delay_inc = spread_after_all ? 2 : q.delay_inc;
   bool aborted = false;
   // d_h of the thread's pairs from DX of frame t (whose first read has been issued): wait, MFMA, sum over the
   // wavefronts; added to dyw.
@@ -590,8 +593,8 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
         RTN_BTRACE_ADD(6, spins)
         // (as in the forward kernel: an adaptive delay across XCDs, one number for all within an XCD)
         if (spins)
-          delay = min(delay + q.delay_inc, 64);
-        else if (q.delay_inc && delay > 0)
+          delay = min(delay + delay_inc, 64);
+        else if (delay_inc && delay > 0)
           delay -= ((t & q.delay_dec_mask) == q.delay_dec_mask) ? 1 : 0;
         // W lives in accumulation registers where it is at most half of that file: the B fragments fill up to half of
         // the ordinary registers, and a matrix instruction reads an A operand from either file (without this the compiler
