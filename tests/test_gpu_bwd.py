@@ -103,6 +103,24 @@ def test_bwd_read_delay_only_moves_time():
                 assert numpy.array_equal(a, b), (tiles, name)
 
 
+def test_bwd_groups_found_on_several_xcds_fall_back_to_device_scope():
+    """With half the true XCD count the groups of an XCD-local gradient plan land on two XCDs each: the kernel's check
+    finds that out and exchanges the ring at device scope (and adapts its read delay): the same bits, no abort."""
+    from _gpu_util import env
+
+    announce("bwd xcd-local with a wrong XCD count")
+    T, B, n = 10, 32, 512
+    want, _, _ = _run(T, B, n, "bf16", 0, 1, seed=3)
+    plan = lib.bwd_plan_text()
+    assert "bwd_regw_xcd" in plan, plan
+    with env(RTN_LSTM2_XCDS=4):
+        got, _, _ = _run(T, B, n, "bf16", 0, 1, seed=3)
+        assert "bwd_regw_xcd" in lib.bwd_plan_text(), lib.bwd_plan_text()
+    for name, a, b in zip(("DX", "DW", "Dy0", "Dc0"), got, want):
+        assert numpy.isfinite(a).all(), name
+        assert numpy.array_equal(a, b), name
+
+
 def test_bwd_cfg2_reduced_f32():
     announce("bwd cfg2 reduced")
     p = synthetic.make_config("cfg2", T=60)
