@@ -300,12 +300,14 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
       Cand chosen = search(B, false);
       {
         const Cand loc = search_local();
-        // Local or spread?  Measured on MI355X (bf16 n = 256 ... 1024 with 8 ... 128 rows, one and two problems, float32
-        // n = 256 and 512): the hand-over inside an XCD is worth about 0.1 us per step, 0.25 us more once the spread
-        // plan keeps more than half of the CUs busy (its exchange then competes for the memory fabric) and 0.1 us
-        // more when its groups have more than 64 workgroups; against that stands the longer MFMA chain of a
-        // wavefront when W is packed into the 32 CUs of one XCD (0.87 us per us of MFMA issue time) and a second pass
-        // of the pointwise part (0.25 us).  Problems that would have to share CUs in a spread launch always go local.
+        // Local or spread?  Measured on MI355X (bf16 n = 192 ... 1024 with 1 ... 128 rows, one and two problems, float32
+        // n = 128 ... 512): the hand-over inside an XCD, where all wavefronts of a group wait the same fixed time before
+        // their first read, is worth about 0.2 us per step, 0.25 us more once the spread plan keeps more than half of
+        // the CUs busy (its exchange then competes for the memory fabric), and 0.005 us for every KB of hidden state
+        // that a CU of the spread plan fetches per step beyond what one of the local plan does; against that stands
+        // the longer MFMA chain of a wavefront when W is packed into the 32 CUs of one XCD (0.87 us per us of MFMA
+        // issue time) and a second pass of the pointwise part (0.25 us).  Problems that would have to share CUs in a
+        // spread launch always go local.
         bool take_local = loc.ok && !(chosen.ok && chosen.regw);
         if (loc.ok && chosen.ok && chosen.regw) {
           auto mfma_us = [&](const Cand& c) { return (double)c.MT * c.NT * ks * (dtype == RTN_DTYPE_BF16 ? 16 : 128) / 2400.0; };
@@ -313,7 +315,8 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
           const long long each = (long long)align_up((size_t)(chosen.groups * chosen.G), (size_t)di.xcds);
           const bool shares = count > 1 && di.cus / each < count;
           const double cost = 0.873 * (mfma_us(loc) - mfma_us(chosen)) + 0.25 * (passes(loc) - passes(chosen));
-          const double gain = 0.10 + (each * std::max(count, 1) > di.cus / 2 ? 0.25 : 0.0) + (chosen.G > 64 ? 0.10 : 0.0);
+          const double more_kb = std::max(0, chosen.Bg - loc.Bg) * (double)n * es / 1024.0;  // hidden state per CU and step
+          const double gain = 0.20 + (each * std::max(count, 1) > di.cus / 2 ? 0.25 : 0.0) + 0.005 * more_kb;
           take_local = shares || cost < gain;
         }
         if (loc.ok && (env_long("RTN_LSTM2_LOCAL", -1) == 1 || take_local)) chosen = loc;
