@@ -193,7 +193,7 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
       // needs G = n / (4 MT) CUs of the XCD; the launch's groups -- those of all `count` problems -- are dealt to the
       // XCDs, floor(CUs per XCD / G) to each.  Fewer rows per group mean fewer bytes for every CU to fetch per step, so
       // the batch is split into as many groups as the device holds.
-      auto search_local = [&]() {
+      auto search_local = [&](int Bq, int problems) {  // Bq rows of each of `problems` problems in one launch
         Cand best;
         const long env_local = env_long("RTN_LSTM2_LOCAL", -1);  // 0: never, 1: whenever feasible, default: by estimate
         if (env_local == 0 || env_kernel == 1 || KSMAX == 0 || di.xcds < 1) return best;
@@ -204,12 +204,12 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
           const int G = n / (4 * MT);
           if (G > cu_x) continue;
           if (MT * KSMAX > (KSMAX == 16 ? 32 : 64) || (MT == 8 && KSMAX != 8)) continue;
-          const int capacity = di.xcds * (cu_x / G) / std::max(count, 1);  // groups per problem
+          const int capacity = di.xcds * (cu_x / G) / std::max(problems, 1);  // groups per problem
           if (capacity < 1) continue;
-          int groups = std::min(capacity, B);
+          int groups = std::min(capacity, Bq);
           if (env_groups) groups = (int)std::min<long>(env_groups, groups);
-          const int Bg = (B + groups - 1) / groups;
-          groups = (B + Bg - 1) / Bg;
+          const int Bg = (Bq + groups - 1) / groups;
+          groups = (Bq + Bg - 1) / Bg;
           if ((Bg + 15) / 16 > 4) continue;
           const int NT = round_nt((Bg + 15) / 16);
           if (NT * KSMAX > 32 || MT * NT > 8) continue;
@@ -227,7 +227,7 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
             best.ok = true; best.regw = true; best.local = true; best.half = half;
             best.est = est; best.KSMAX = KSMAX; best.MT = MT; best.NT = NT; best.groups = groups; best.G = G; best.Bg = Bg;
             best.lds = lds;
-            const int total_groups = groups * std::max(count, 1);
+            const int total_groups = groups * std::max(problems, 1);
             best.grid = di.xcds * G * ((total_groups + di.xcds - 1) / di.xcds);
           }
         }
@@ -299,7 +299,7 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
       };
       Cand chosen = search(B, false);
       {
-        const Cand loc = search_local();
+        const Cand loc = search_local(B, count);
         // Local or spread?  Measured on MI355X (bf16 n = 192 ... 1024 with 1 ... 128 rows, one and two problems, float32
         // n = 128 ... 512): the hand-over inside an XCD, where all wavefronts of a group wait the same fixed time before
         // their first read, is worth about 0.2 us per step, 0.25 us more once the spread plan keeps more than half of
@@ -328,7 +328,10 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
         const long env_passes = env_long("RTN_LSTM2_MAX_PASSES", -1);
         const int limit = (int)(env_passes >= 0 ? env_passes : (chosen.ok ? kMaxPassesOverLds : kMaxPassesOverSteps));
         for (int passes = 2; passes <= std::min(limit, B); ++passes) {
-          const Cand c = search((B + passes - 1) / passes, true);
+          // (a turn is a launch of one problem; its groups on one XCD each where that is possible: measured at
+          // bf16 n = 512 and 1024 with 16 and 32 rows per group, 2.2 us per step and turn against 2.5)
+          Cand c = search_local((B + passes - 1) / passes, 1);
+          if (!c.ok) c = search((B + passes - 1) / passes, true);
           if (!c.ok) continue;
           if ((((B + c.Bg - 1) / c.Bg) + c.groups - 1) / c.groups > limit) continue;
           chosen = c;
@@ -1128,7 +1131,10 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
           one.p[0].group_offset = g0;
           one.p[0].groups = std::min(pl.groups, pl.groups_total - g0);
           one.count = 1;
-          one.grid = one.p[0].groups * pl.wgs_per_group;
+          one.local = pl.local ? 1 : 0;
+          one.xcds = device_info().xcds;
+          // (an XCD-local turn: the groups dealt to the XCDs, workgroup id = slot * xcds + xcd)
+          one.grid = pl.local ? one.xcds * pl.wgs_per_group * ((one.p[0].groups + one.xcds - 1) / one.xcds) : one.p[0].groups * pl.wgs_per_group;
           one.wgs_each = (int)align_up((size_t)one.grid, (size_t)device_info().xcds);
           void* args[] = {(void*)&one};
           rc = launch_coresident(pk, dim3(one.grid), dim3(kWgThreads), args, (unsigned)pl.lds_bytes, stream, capturing);

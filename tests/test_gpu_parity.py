@@ -533,10 +533,12 @@ def test_wide_and_large_shapes(T, B, n, dtype):
         assert rel <= (2e-5 if dtype == "f32" else 2e-2), (name, rel)
 
 
-@pytest.mark.parametrize("T,B,n,dtype,start,step", [(6, 256, 1024, "bf16", 0, 1), (5, 70, 1536, "bf16", 1, -1), (5, 300, 512, "f32", 0, 2), (4, 97, 2048, "bf16", 0, -1)])
+@pytest.mark.parametrize("T,B,n,dtype,start,step", [(6, 256, 1024, "bf16", 0, 1), (5, 70, 1536, "bf16", 1, -1), (5, 300, 512, "f32", 0, 2), (4, 97, 2048, "bf16", 0, -1), (5, 270, 1024, "bf16", 0, -1),
+                                                    (4, 1000, 256, "bf16", 1, 1)])
 def test_batch_in_several_persistent_launches(T, B, n, dtype, start, step):
     """A batch too large for one launch of the register kernel runs as several persistent launches in turn, each on a
-    share of the batch groups, the last one on fewer groups (and a partly filled group)."""
+    share of the batch groups, the last one on fewer groups (and a partly filled group).  Where a group fits an XCD
+    (n <= 1024 in bf16) the turns are XCD-local launches, a last turn of fewer groups leaves part of its grid idle."""
     from returnn_amd import lib
 
     announce("several_launches", T, B, n, dtype, start, step)
