@@ -1730,7 +1730,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
   // MFMA time each) and 4 or 8 wavefronts per workgroup.
   const long env_rows = env_long("RTN_LSTM2_BWD_ROWS", 0);
   int rows_per_group = 16, bwd_waves = kWaves, groups_per_launch = 0;
-  bool bwd_local = false;
+  bool bwd_local = false, turn_local = false;
   long long turn_rows = 0;
   const void* turn_pk = nullptr;
   int turn_cfg[5] = {0, 0, 0, 0, 0};
@@ -1818,12 +1818,20 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
           break;
         }
         // Too many rows for one launch: remember the candidate that takes most rows per launch; the batch groups
-        // then run in turns (the rows of a batch are independent of each other).
-        if (fit >= 1 && fit * use_rows > turn_rows && (groups_needed + fit - 1) / fit <= env_long("RTN_LSTM2_MAX_PASSES", kMaxPassesOverSteps)) {
-          turn_rows = fit * use_rows;
+        // then run in turns (the rows of a batch are independent of each other).  A turn whose groups fit an XCD each
+        // is an XCD-local launch, unless that costs more than an eighth of the groups a launch can hold.
+        long long fit_local = 0;
+        if (want_local && di_b.xcds > 1 && per_cu >= 1 && G_wgs <= cu_x * per_cu)
+          fit_local = (long long)di_b.xcds * ((cu_x * per_cu) / G_wgs) / count;
+        const bool local_turns = fit_local >= 1 && fit_local * 8 >= fit * 7;
+        const long long turn_fit = local_turns ? fit_local : fit;
+        if (turn_fit >= 1 && turn_fit * use_rows > turn_rows &&
+            (groups_needed + turn_fit - 1) / turn_fit <= env_long("RTN_LSTM2_MAX_PASSES", kMaxPassesOverSteps)) {
+          turn_rows = turn_fit * use_rows;
           turn_pk = (const void*)kfn;
-          turn_cfg[0] = use_rows; turn_cfg[1] = mt; turn_cfg[2] = wv; turn_cfg[3] = ksb; turn_cfg[4] = (int)fit;
+          turn_cfg[0] = use_rows; turn_cfg[1] = mt; turn_cfg[2] = wv; turn_cfg[3] = ksb; turn_cfg[4] = (int)turn_fit;
           turn_lds = cand_lds;
+          turn_local = local_turns;
         }
       }
       if (!pk && turn_pk) {
@@ -1834,6 +1842,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
         KSB = turn_cfg[3];
         groups_per_launch = turn_cfg[4];
         bwd_lds = turn_lds;
+        bwd_local = turn_local;
       }
     }
     if (!pk && count > 1) {
