@@ -129,6 +129,43 @@ def test_xcd_local_plans(cabi):
     assert "_xcd" not in lib.describe_plan(100, 32, 2048, lib.DTYPE_BF16, lib.MODE_AUTO)
 
 
+def test_plan_invariants_over_shapes(cabi):
+    """Every persistent plan covers the batch, keeps its grid on the device (256 CUs, at most two workgroups each) and,
+    where it is XCD-local, keeps a group within the 32 CUs of an XCD and deals whole rounds of groups to the 8 XCDs."""
+    def fields(text):
+        out = {}
+        for w in text.split():
+            if "=" in w:
+                k, v = w.split("=", 1)
+                out[k] = int(v) if v.lstrip("-").isdigit() else v
+        return out
+
+    seen_local_turns = False
+    for dt in (lib.DTYPE_BF16, lib.DTYPE_F32):
+        for n in (64, 192, 256, 320, 512, 768, 1024, 1536, 2048):
+            for B in (1, 3, 8, 9, 16, 31, 64, 100, 128, 200, 256, 513, 1024):
+                for count in (1, 2):
+                    text = lib.describe_plan(50, B, n, dt, lib.MODE_AUTO) if count == 1 else lib.describe_multi_plan(2, 50, B, n, dt, lib.MODE_AUTO)
+                    f = fields(text)
+                    if f.get("mode") != "persistent" or not str(f.get("kernel", "")).startswith("mfma_regw"):
+                        continue
+                    what = (dt, n, B, count, text)
+                    assert f["rows_per_group"] * f["groups"] * f["launches"] >= B, what
+                    assert f["rows_per_group"] * f["groups"] * (f["launches"] - 1) < B, what  # no idle turn
+                    assert 1 <= f["rows_per_group"] <= 64 and f["rows_per_group"] <= 16 * f["nt"], what
+                    assert f["wgs_per_group"] * 4 * f["mt"] == n, what
+                    assert f["wgs"] <= 512, what
+                    if "_xcd" in f["kernel"]:
+                        assert f["wgs_per_group"] <= 32 and f["wgs"] % 8 == 0 and f["wgs"] <= 256, what
+                        per_xcd = 32 // f["wgs_per_group"]
+                        problems = count if f["launches"] == 1 else 1  # a turn is a launch of one problem
+                        assert f["groups"] * problems <= 8 * per_xcd, what
+                        seen_local_turns = seen_local_turns or f["launches"] > 1
+                    if f["kernel"].endswith("_half"):
+                        assert f["rows_per_group"] <= 8 and f["nt"] == 1 and f["mt"] % 2 == 0, what
+    assert seen_local_turns
+
+
 def test_op_description_contract():
     """Names, order, ndim and host-memory flags of returnn/native_op.py:1054-1068."""
     from returnn_amd import native_op
