@@ -131,7 +131,7 @@ def test_xcd_local_plans(cabi):
 
 def test_plan_invariants_over_shapes(cabi):
     """Every persistent plan covers the batch, keeps its grid on the device (256 CUs, at most two workgroups each) and,
-    where it is XCD-local, keeps a group within the 32 CUs of an XCD and deals whole rounds of groups to the 8 XCDs."""
+    where it is XCD-local, keeps a group within the 32 CUs of an XCD and sizes its grid in multiples of the 8 XCDs."""
     def fields(text):
         out = {}
         for w in text.split():

@@ -34,7 +34,8 @@ def _assert_same(multi_out, single_out, what):
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize(
     "T,B,n,count",
-    [(12, 16, 64, 2), (7, 32, 256, 2), (9, 5, 128, 3), (6, 40, 512, 4), (5, 8, 96, 6), (6, 3, 20, 2), (5, 32, 1024, 2), (6, 9, 100, 2), (4, 7, 72, 3)],
+    [(12, 16, 64, 2), (7, 32, 256, 2), (9, 5, 128, 3), (6, 40, 512, 4), (5, 8, 96, 6), (6, 3, 20, 2), (5, 32, 1024, 2), (6, 9, 100, 2), (4, 7, 72, 3),
+     (4, 300, 512, 2)],  # (each call in several persistent launches in turn, the last one on fewer groups)
 )
 def test_multi_equals_single(T, B, n, count, dtype):
     announce("multi vs single", T, B, n, count, dtype)
