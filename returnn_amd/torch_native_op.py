@@ -632,6 +632,7 @@ class NativeLstm2Function(torch.autograd.Function):
         ctx.save_for_backward(W, y0, c0, i, Y, C, H)
         ctx.start, ctx.step = int(start), int(step)
         ctx.in_dtypes = (X.dtype, W.dtype, y0.dtype, c0.dtype)
+        ctx.set_materialize_grads(False)  # (no zero tensors for outputs without a gradient: backward takes None)
         ctx.mark_non_differentiable(C, H)
         return Y, C, H, d
 
@@ -696,6 +697,7 @@ class LstmGenericBaseFunction(torch.autograd.Function):
         Y, H, d = make_op(native_op.LstmGenericBase)(Z, V_h, c, i)
         ctx.save_for_backward(V_h, c, i, Y, H)
         ctx.in_dtypes = (Z.dtype, V_h.dtype, c.dtype)
+        ctx.set_materialize_grads(False)  # (no zero tensors for outputs without a gradient: backward takes None)
         ctx.mark_non_differentiable(H)
         return Y, H, d
 
@@ -764,6 +766,7 @@ class LstmLowMemFunction(torch.autograd.Function):
         ctx.save_for_backward(X, W, b, y0, c0, i, Y, C)
         ctx.start, ctx.step = int(start), int(step)
         ctx.in_dtypes = (X.dtype, W.dtype, b.dtype, y0.dtype, c0.dtype)
+        ctx.set_materialize_grads(False)  # (no zero tensors for outputs without a gradient: backward takes None)
         ctx.mark_non_differentiable(C)
         return Y, C, d
 
@@ -790,6 +793,7 @@ class NativeLstm2PairFunction(torch.autograd.Function):
         (Yf, Cf, Hf, df), (Yb, Cb, Hb, db) = native_lstm2_multi([(Xf, Wf, y0f, c0f, i, 0, 1), (Xb, Wb, y0b, c0b, i, 0, -1)])
         ctx.save_for_backward(Wf, y0f, c0f, Wb, y0b, c0b, i, Yf, Cf, Hf, Yb, Cb, Hb)
         ctx.in_dtypes = (Xf.dtype, Wf.dtype, y0f.dtype, c0f.dtype, Xb.dtype, Wb.dtype, y0b.dtype, c0b.dtype)
+        ctx.set_materialize_grads(False)  # (no zero tensors for outputs without a gradient: backward takes None)
         ctx.mark_non_differentiable(Cf, Hf, Cb, Hb)
         return Yf, Cf, Hf, df, Yb, Cb, Hb, db
 
