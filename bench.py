@@ -70,15 +70,20 @@ def algorithmic_bytes_per_unit(n: int, dtype: str) -> int:
     return e * 4 * n + e * 4 * n + e * n + 4 * n + 4
 
 
-def ceiling_fields(probe_us, seq_ms, rows, n, dtype, T, call_ms):
+def ceiling_fields(probe_us, seq_ms, issue_ms, rows, n, dtype, T, call_ms):
     """
-    Two ceilings of the recurrent GEMM next to the nominal matrix peak.
+    Three ceilings of the recurrent GEMM next to the nominal matrix peak.
 
-    ``achievable_mfma``: the rate at which the device runs the step's own MFMA sequence when nothing has to come from
-    another workgroup (``seq_ms``: one launch of the library's sequence probe -- the plan's grid, per step the B
-    fragments from LDS, the plan's MFMAs against W in registers, the partial tiles through LDS with one barrier, their
-    sum; no exchange, no streams, no gates), counted in the op's algorithmic flops.  This is the "achievable MFMA
-    roofline" of the decomposition; ``frac_of_achievable_mfma`` = probe time / measured time.
+    ``achievable_mfma``: the rate at which the device's matrix cores run the plan's per-workgroup MFMA tile sequence
+    when nothing else happens (``issue_ms``: one launch of the library's issue probe -- the plan's grid, W and the
+    hidden-state fragments in registers, per step the plan's MFMAs and nothing else: no LDS, no barrier, no loads),
+    counted in the op's algorithmic flops.  This is the "achievable MFMA roofline" of the tile sequence;
+    ``frac_of_achievable_mfma`` = issue-probe time / measured time.
+
+    ``decomposition_ceiling``: the same with what the split of the contraction over four wavefronts adds
+    (``seq_ms``: the sequence probe -- B fragments from LDS, the MFMAs, the partial tiles through LDS with the step's
+    one barrier, their sum; no exchange, no streams, no gates): the best a kernel of this decomposition could do if the
+    hidden state cost nothing to hand over.  ``frac_of_decomposition_ceiling`` = sequence-probe time / measured time.
 
     ``latency_ceiling``: the T steps are sequential, and a step cannot be shorter than one hand-over of the hidden state
     between the CUs that hold W (``probe_us``: the library's latency probe -- device-scope store, visible on every CU,
@@ -88,11 +93,17 @@ def ceiling_fields(probe_us, seq_ms, rows, n, dtype, T, call_ms):
     """
     out = {}
     step_flops = 8.0 * n * n * rows
+    if issue_ms is not None:
+        out.update({
+            "mfma_issue_us_per_step": issue_ms * 1e3 / T,
+            "achievable_mfma": step_flops * T / (issue_ms * 1e-3) / 1e12,
+            "frac_of_achievable_mfma": issue_ms / call_ms,
+        })
     if seq_ms is not None:
         out.update({
             "mfma_sequence_us_per_step": seq_ms * 1e3 / T,
-            "achievable_mfma": step_flops * T / (seq_ms * 1e-3) / 1e12,
-            "frac_of_achievable_mfma": seq_ms / call_ms,
+            "decomposition_ceiling": step_flops * T / (seq_ms * 1e-3) / 1e12,
+            "frac_of_decomposition_ceiling": seq_ms / call_ms,
         })
     if probe_us is not None:
         mfma_us = step_flops / PEAK_MFMA[dtype] * 1e6
@@ -852,22 +863,25 @@ def main():
     if pe and cabi.rtn_native_lstm2_fwd_status(probe_ws.data_ptr(), stream.cuda_stream) == lib.RTN_OK:
         probe_us = min(a.elapsed_time(b) for a, b in pe[1:]) * 1e3 / probe_rounds
 
-    # The MFMA roofline of the plan's own instruction sequence (no exchange): one launch of the sequence probe, T steps.
-    seq_ms = None
+    # The two MFMA ceilings of the plan (no exchange): one launch of each probe, T steps -- the MFMAs alone, and the MFMAs
+    # with the decomposition's partial-tile round trip through LDS.
     seq_ws = torch.empty((1 << 20,), dtype=torch.uint8, device=dev)
-    se = []
-    for _ in range(1 + 3):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        rc = cabi.rtn_mfma_sequence_probe(2 if fused else 1, T, B, n, dt_code, T, seq_ws.data_ptr(), seq_ws.numel(), stream.cuda_stream)
-        e1.record(stream)
-        if rc != lib.RTN_OK:
-            se = []
-            break
-        se.append((e0, e1))
-    torch.cuda.synchronize()
-    if se:
-        seq_ms = min(a.elapsed_time(b) for a, b in se[1:])
+
+    def time_probe(fn):
+        se = []
+        for _ in range(1 + 3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            rc = fn(2 if fused else 1, T, B, n, dt_code, T, seq_ws.data_ptr(), seq_ws.numel(), stream.cuda_stream)
+            e1.record(stream)
+            if rc != lib.RTN_OK:
+                return None
+            se.append((e0, e1))
+        torch.cuda.synchronize()
+        return min(a.elapsed_time(b) for a, b in se[1:])
+
+    seq_ms = time_probe(cabi.rtn_mfma_sequence_probe)
+    issue_ms = time_probe(cabi.rtn_mfma_issue_probe)
 
     units_per_step = len(directions) * T * B
     value = units_per_step * args.steps / elapsed
@@ -919,7 +933,7 @@ def main():
             % ("k_lstm2_regw" if "mfma_regw" in plan else ("k_lstm2_mfma" if "mfma_lds" in plan else "k_step_generic"),
                len(directions) // launches, units_per_launch),
             "launch_ms": call_ms,
-            **ceiling_fields(probe_us, seq_ms, units_per_launch // T, n, dtype, T, call_ms),
+            **ceiling_fields(probe_us, seq_ms, issue_ms, units_per_launch // T, n, dtype, T, call_ms),
             "hbm_algorithmic_GBps": bytes_per_launch / (call_ms * 1e-3) / 1e9,
             "hbm_frac": bytes_per_launch / (call_ms * 1e-3) / PEAK_HBM,
         },
@@ -940,7 +954,7 @@ def main():
             "mfma_TFLOPs": achieved / 1e12,
         })
         for key in ("latency_ceiling", "frac_of_latency_ceiling", "mfma_peak_us_per_step", "achievable_mfma", "frac_of_achievable_mfma",
-                    "mfma_sequence_us_per_step"):
+                    "mfma_sequence_us_per_step", "mfma_issue_us_per_step", "decomposition_ceiling", "frac_of_decomposition_ceiling"):
             result["roofline"].pop(key, None)  # they describe the exchange-bound persistent kernel
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, args.cpu_seconds)

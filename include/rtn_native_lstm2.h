@@ -188,6 +188,15 @@ int rtn_mfma_sequence_probe(int32_t count, int64_t T, int32_t B, int32_t n, int3
                             size_t workspace_bytes, void* hip_stream);
 
 /*
+ * Measurement aid: the matrix cores alone.  Like rtn_mfma_sequence_probe (same arguments, same grid, same per-wavefront
+ * tile sequence with W and the hidden-state fragments in registers), but a step is the MFMAs and nothing else: no LDS
+ * round trip of partial tiles, no barrier, no sum.  Launch time over the op's algorithmic flops = the MFMA roofline the
+ * plan's tile sequence can reach at most, whatever the rest of a step looks like.  No counterpart in the reference.
+ */
+int rtn_mfma_issue_probe(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t steps, void* workspace,
+                         size_t workspace_bytes, void* hip_stream);
+
+/*
  * NativeLstm2 gradient.  Replaces the generated body `c_bw_code` (returnn/native_op.py:1288-1464) with
  * `lstm_bwd_kernel` (:1123-1180) and its `affine_raw` GEMMs; the arguments are the ones `grad_input_map`
  * (:1071-1077) hands to the gradient op, minus X, which the computation never reads.
@@ -202,8 +211,9 @@ int rtn_mfma_sequence_probe(int32_t count, int64_t T, int32_t B, int32_t n, int3
  *
  * Element type `dtype` for W y0 Y H DY DX Dy0; c0 C i Dd Dc0 DW are float32.  Where the shape allows (n a multiple of
  * 16, a wavefront's share of 16 rows of W fits its registers, all workgroups fit on the device) ONE persistent
- * cooperative kernel runs all frames: W stays in registers, DX doubles as the self-validating exchange medium between
- * workgroups.  Otherwise one launch per visited frame (the MFMA GEMM Dy0 += DX[t'] W^T of the frame processed before,
+ * cooperative kernel runs all frames: W stays in registers, and the gate derivatives of a frame travel between the
+ * workgroups through a ring of 4 frames in the workspace (MFMA operand order, self-validating: a slot is all-ones until
+ * written); DX itself is a plain output stream, written once.  Otherwise one launch per visited frame (the MFMA GEMM Dy0 += DX[t'] W^T of the frame processed before,
  * fused with the frame's pointwise part), replayed through a library-owned hipGraph.  The large weight-gradient GEMM
  * (Y^T DX over all frames) is left to rocBLAS, which may allocate its own device workspace on first use.  Under stream
  * capture the kernels (the persistent one as a node of its own, see rtn_native_lstm2_capture_report) and the rocBLAS calls

@@ -49,25 +49,25 @@ __global__ void k_bwd_pack_w(const void* __restrict__ W, void* __restrict__ Wpk,
 // Gate derivatives of one (sequence, cell) pair in one frame (returnn/native_op.py:1148-1172).
 //   h0: first block of H -- tanh(cell-in), or with kOpH0IsCell the cell state, from which tanh(cell-in) is recovered as
 //   the reference's gradient kernel does: (state - forget * old_state) / max(input, 1e-16)  (:462-463)
-//   d_y_b, d_c_b: error of the output and of the cell state, already multiplied by the mask
+//   err_y, err_c: error of the output and of the cell state, already multiplied by the mask
 template <typename AT>
-__device__ __forceinline__ float bwd_cell(int op_flags, float h0, float inpGate, float fgtGate, float outGate, float prev_c, float d_y_b,
-                                          float d_c_b, float (&dx)[4]) {
+__device__ __forceinline__ float bwd_cell(int op_flags, float h0, float a_in, float a_fg, float a_out, float c_before, float err_y,
+                                          float err_c, float (&dx)[4]) {
   using E = Elem<AT>;
-  float cellIn, gc;
+  float a_cell, tanh_c;  // tanh(cell-in) and tanh of the frame's cell state
   if (op_flags & kOpH0IsCell) {
-    gc = Act<AT>::tanh(h0);
-    cellIn = (h0 - fgtGate * prev_c) / fmaxf(inpGate, 1e-16f);
+    tanh_c = Act<AT>::tanh(h0);
+    a_cell = (h0 - a_fg * c_before) / fmaxf(a_in, 1e-16f);
   } else {
-    cellIn = h0;
-    gc = Act<AT>::tanh(prev_c * fgtGate + cellIn * inpGate);
+    a_cell = h0;
+    tanh_c = Act<AT>::tanh(c_before * a_fg + a_cell * a_in);
   }
-  const float d_c2 = d_c_b + outGate * d_y_b * (1.f - gc * gc);
-  dx[0] = E::round((1.f - cellIn * cellIn) * inpGate * d_c2);
-  dx[1] = E::round((1.f - inpGate) * inpGate * cellIn * d_c2);
-  dx[2] = E::round((1.f - fgtGate) * fgtGate * prev_c * d_c2);
-  dx[3] = E::round((1.f - outGate) * outGate * gc * d_y_b);
-  return d_c2;
+  const float err_cell = err_c + a_out * err_y * (1.f - tanh_c * tanh_c);  // total error on the frame's cell state
+  dx[0] = E::round((1.f - a_cell * a_cell) * a_in * err_cell);
+  dx[1] = E::round((1.f - a_in) * a_in * a_cell * err_cell);
+  dx[2] = E::round((1.f - a_fg) * a_fg * c_before * err_cell);
+  dx[3] = E::round((1.f - a_out) * a_out * tanh_c * err_y);
+  return err_cell;
 }
 
 // Cell state of the frame before: the forward pass's C, or with kOpH0IsCell the first block of H of that frame.
@@ -93,14 +93,14 @@ __global__ void k_bwd_pointwise(Lstm2BwdParams p, long long t, long long prev_t)
   const float m = p.mask[t * p.B + b];
   const float dyw = p.dyw[idx];
   const bool raw_dh = (p.op_flags & kOpRawDh) != 0;
-  const float d_y_b = raw_dh ? E::load(p.DY, t * bn + idx) * m + dyw : (E::load(p.DY, t * bn + idx) + dyw) * m;
+  const float err_y = raw_dh ? E::load(p.DY, t * bn + idx) * m + dyw : (E::load(p.DY, t * bn + idx) + dyw) * m;
   const float dc = p.Dc0[idx];
-  const float d_c_b = dc * m;
+  const float err_c = dc * m;
   const float prev_c = bwd_prev_cell<AT>(p, prev_t, idx, io);
-  const float fgtGate = E::load(p.H, fo + 2 * n);
+  const float a_fg = E::load(p.H, fo + 2 * n);
   float dx[4];
-  const float d_c2 = bwd_cell<AT>(p.op_flags, E::load(p.H, fo), E::load(p.H, fo + n), fgtGate, E::load(p.H, fo + 3 * n), prev_c, d_y_b, d_c_b, dx);
-  p.Dc0[idx] = fgtGate * d_c2 + dc * (1.f - m);
+  const float err_cell = bwd_cell<AT>(p.op_flags, E::load(p.H, fo), E::load(p.H, fo + n), a_fg, E::load(p.H, fo + 3 * n), prev_c, err_y, err_c, dx);
+  p.Dc0[idx] = a_fg * err_cell + dc * (1.f - m);
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
     E::store(p.DX, fo + g * n, dx[g]);
@@ -215,13 +215,13 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
       const long long fo = t * bn * 4 + io;
       const float m = q_m[nt];
       const bool raw_dh = (p.op_flags & kOpRawDh) != 0;
-      const float d_y_b = raw_dh ? q_dy[nt] * m + dyw : (q_dy[nt] + dyw) * m;
+      const float err_y = raw_dh ? q_dy[nt] * m + dyw : (q_dy[nt] + dyw) * m;
       const float dc = q_dc[nt];
-      const float d_c_b = dc * m;
-      const float fgtGate = q_h[nt][2];
+      const float err_c = dc * m;
+      const float a_fg = q_h[nt][2];
       float dx[4];
-      const float d_c2 = bwd_cell<AT>(p.op_flags, q_h[nt][0], q_h[nt][1], fgtGate, q_h[nt][3], q_pc[nt], d_y_b, d_c_b, dx);
-      p.Dc0[idx] = fgtGate * d_c2 + dc * (1.f - m);
+      const float err_cell = bwd_cell<AT>(p.op_flags, q_h[nt][0], q_h[nt][1], a_fg, q_h[nt][3], q_pc[nt], err_y, err_c, dx);
+      p.Dc0[idx] = a_fg * err_cell + dc * (1.f - m);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         E::store(p.DX, fo + g * n, dx[g]);
@@ -692,12 +692,12 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     const float m = in_m;
 #pragma unroll
     for (int j = 0; j < PT; ++j) {
-      const float d_y_b = raw_dh ? in_dy[j] * m + dyw[j] : (in_dy[j] + dyw[j]) * m;
-      const float d_c_b = dc[j] * m;
-      const float fgtGate = in_gate[j][2];
+      const float err_y = raw_dh ? in_dy[j] * m + dyw[j] : (in_dy[j] + dyw[j]) * m;
+      const float err_c = dc[j] * m;
+      const float a_fg = in_gate[j][2];
       float dx[4];
-      const float d_c2 = bwd_cell<AT>(p.op_flags, in_gate[j][0], in_gate[j][1], fgtGate, in_gate[j][3], prev_cell(j), d_y_b, d_c_b, dx);
-      dc[j] = fgtGate * d_c2 + dc[j] * (1.f - m);
+      const float err_cell = bwd_cell<AT>(p.op_flags, in_gate[j][0], in_gate[j][1], a_fg, in_gate[j][3], prev_cell(j), err_y, err_c, dx);
+      dc[j] = a_fg * err_cell + dc[j] * (1.f - m);
       const int mt = tile_of(j);
       if (mt < MT && bl < Bp) {
         const int col = 16 * mt + kl;

@@ -1065,33 +1065,8 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   // atomics whose result is waited for, so the mask is complete when the count is); with one XCD in the mask the hidden
   // state travels through that XCD's L2 (plain stores, loads that bypass the first-level cache), else with device scope.
   __shared__ int s_local;
-  if (multi.local && tid == 0) {
-    int ok = 1;
-    if (p.wgs_per_group > 1) {
-      unsigned* words = p.flags + (size_t)g * p.wgs_per_group;
-      (void)__hip_atomic_fetch_or(words + 1, 1u << xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      (void)__hip_atomic_fetch_add(words, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      unsigned long long t0 = 0;
-      unsigned spins = 0;
-      while (__hip_atomic_load(words, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)p.wgs_per_group) {
-        if ((spins++ & 15u) == 0) {
-          if (__hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
-          const unsigned long long now = wall_clock64();
-          if (spins == 1) {
-            t0 = now;
-          } else if (now - t0 > p.timeout_ticks) {
-            __hip_atomic_store(p.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            break;
-          }
-        }
-        __builtin_amdgcn_s_sleep(2);
-      }
-      const unsigned mask = __hip_atomic_load(words + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      ok = (mask & (mask - 1)) == 0;
-      if (!ok) __hip_atomic_store(p.status + 1, mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the record: the group was spread
-    }
-    s_local = ok;
-  }
+  if (multi.local && tid == 0)
+    s_local = group_on_one_xcd(p.flags + (size_t)g * p.wgs_per_group, (unsigned)p.wgs_per_group, p.status, p.timeout_ticks) ? 1 : 0;
 
   auto run = [&](auto ex_tag) {
     constexpr int EX = decltype(ex_tag)::value;
@@ -1198,9 +1173,16 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       RTN_TRACE_ADD(6, spins)
 
       RedBuf& redbuf = red[PAR];
-      f32x4 acc[MT][NT];
+      // PAIRED: ONE accumulator for every two tiles.  A group of at most 8 rows fills columns 0-7 of a tile and leaves
+      // columns 8-15 to padding; with the B operand of tile 2u holding the rows in columns 0-7 and zeros in columns 8-15,
+      // and that of tile 2u+1 the same rows in columns 8-15 and zeros in 0-7, both tiles' MFMAs can add into the same
+      // accumulator: columns 0-7 collect tile 2u, columns 8-15 tile 2u+1 (the other tile contributes exact zeros, so
+      // every sum is bit for bit what a tile of its own would hold).  Half the accumulators, half the partial tiles
+      // through LDS -- written by all 64 lanes, in the very lane order the pointwise part reads them in.
+      constexpr int NACC = PAIRED ? MT / 2 : MT;
+      f32x4 acc[NACC][NT];
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+      for (int mt = 0; mt < NACC; ++mt)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
       // Everything that is not on the path h -> MFMA -> gates -> h rides in the shadow of the MFMAs: all of it without
@@ -1208,33 +1190,75 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       // one block of straight-line code that the scheduler is told to weave: a wavefront that has a SIMD to itself
       // issues one instruction per 4 clocks, an MFMA keeps the matrix core busy for 16, so three other instructions fit
       // behind every MFMA for free -- but a run of them between two MFMAs drains the matrix core.
-      // PAIRED: the odd macro steps' rows, from lanes 8-15 of every group of 16 to lanes 0-7 (a row shift of the data
-      // parallel primitives: lane i takes lane i + 8, lanes without a source take 0)
-      i32x4 bf_odd[KSMAX / 2 + 1];
+      // PAIRED: a loaded register holds macro step 2a in the lanes of rows 0-7 and step 2a+1 in the lanes of rows 8-15 of
+      // every group of 16 lanes.  Four B operands are made of it: each step's rows in columns 0-7 (for the even tiles)
+      // and in columns 8-15 (for the odd tiles), zeros in the other half -- a mask where the rows stay, a row shift by 8
+      // lanes (data parallel primitive; lanes without a source take 0) where they move.
+      if constexpr (PAIRED) {
+        // The MFMAs go in chunks of NACC -- one per accumulator: (macro step, even tiles), (macro step, odd tiles), ... --
+        // so that two MFMAs into the same accumulator are NACC apart.  The compiler's scheduler would otherwise line up
+        // the MFMAs of one accumulator, each waiting for the one before; nothing moves from one chunk to another
+        // (sched_barrier), and the step's other work is dealt to the chunks by hand: the B operand of the next chunk
+        // (four vector instructions) and one piece of the stream work each, woven between the chunk's MFMAs.
+        constexpr int NCH = 2 * KSMAX;
+        const int keep_lo = (jl & 8) ? 0 : -1, keep_hi = ~keep_lo;
+        auto operand = [&](int c) {  // chunk c: macro step c / 2, rows in columns 0-7 (even tiles) or 8-15 (odd tiles)
+          const int ks = c >> 1, odd = c & 1;
+          const i32x4 src = bf[ks >> 1][0];
+          i32x4 r;
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            if (!(ks & 1))
+              r[w] = odd ? __builtin_amdgcn_update_dpp(0, src[w], 0x118 /* row_shr:8 */, 0xF, 0xF, true) : (src[w] & keep_lo);
+            else
+              r[w] = odd ? (src[w] & keep_hi) : __builtin_amdgcn_update_dpp(0, src[w], 0x108 /* row_shl:8 */, 0xF, 0xF, true);
+          }
+          return r;
+        };
+        i32x4 opnd = operand(0);
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+          const int ks = c >> 1, odd = c & 1;
+          i32x4 opnd_next = opnd;
+          if (c + 1 < NCH) opnd_next = operand(c + 1);
+          if (c == 0) {
+            flush_read(stage == 2 ? 0 : stage + 1);  // the copy of step s-2 is (s+1) % 3
+            load_gate_inputs(IntTag<1 - PAR>{});
+          }
+          if (c == (NCH > 1 ? 1 : 0)) put(par_tag);
+          if (c == (NCH > 2 ? 2 : NCH - 1)) flush_write_at(h_out, y_out_p, c_out, s >= 2);
+          if (c == (NCH > 3 ? 3 : NCH - 1)) fetch_at(x_next, m_next, s + 4 < nsteps, par_tag);
+#pragma unroll
+          for (int u = 0; u < NACC; ++u) {
+            acc[u][0] = E::mma(wreg[2 * u + odd][ks], opnd, acc[u][0]);
+            __builtin_amdgcn_sched_group_barrier(0x008, sizeof(AT) == 2 ? 1 : 4, 0);  // the MFMA(s) of one fragment ...
+            __builtin_amdgcn_sched_group_barrier(0x096, 3, 0);                        // ... then up to three of the rest
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          opnd = opnd_next;
+        }
+      } else {
+        flush_read(stage == 2 ? 0 : stage + 1);  // the copy of step s-2 is (s+1) % 3
+        load_gate_inputs(IntTag<1 - PAR>{});
+        put(par_tag);
+        flush_write_at(h_out, y_out_p, c_out, s >= 2);
+        fetch_at(x_next, m_next, s + 4 < nsteps, par_tag);
+#pragma unroll
+        for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+              acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+              __builtin_amdgcn_sched_group_barrier(0x008, sizeof(AT) == 2 ? 1 : 4, 0);  // the MFMA(s) of one fragment ...
+              __builtin_amdgcn_sched_group_barrier(0x096, 3, 0);                        // ... then up to three of the rest (VALU, SALU, VMEM, LDS)
+            }
+      }
+      h_out += step_x; y_out_p += step_y; c_out += step_c; x_next += step_x; m_next += step_m;
       if constexpr (PAIRED) {
 #pragma unroll
-        for (int a = 0; a < NLD; ++a)
-#pragma unroll
-          for (int w = 0; w < 4; ++w) bf_odd[a][w] = __builtin_amdgcn_update_dpp(0, bf[a][0][w], 0x108 /* row_shl:8 */, 0xF, 0xF, true);
-      }
-      flush_read(stage == 2 ? 0 : stage + 1);  // the copy of step s-2 is (s+1) % 3
-      load_gate_inputs(IntTag<1 - PAR>{});
-      put(par_tag);
-      flush_write_at(h_out, y_out_p, c_out, s >= 2);
-      fetch_at(x_next, m_next, s + 4 < nsteps, par_tag);
-#pragma unroll
-      for (int ks = 0; ks < KSMAX; ++ks)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt) {
-            acc[mt][nt] = E::mma(wreg[mt][ks], PAIRED ? ((ks & 1) ? bf_odd[ks / 2] : bf[ks / 2][nt]) : bf[ks][nt], acc[mt][nt]);
-            __builtin_amdgcn_sched_group_barrier(0x008, sizeof(AT) == 2 ? 1 : 4, 0);  // the MFMA(s) of one fragment ...
-            __builtin_amdgcn_sched_group_barrier(0x096, 3, 0);                        // ... then up to three of the rest (VALU, SALU, VMEM, LDS)
-          }
-      h_out += step_x; y_out_p += step_y; c_out += step_c; x_next += step_x; m_next += step_m;
-      // (with at most 8 rows only the lanes of rows 0..7 hold columns anybody reads)
-      if (!HALF || (lane & 8) == 0) {
+        for (int u = 0; u < NACC; ++u) redbuf[wave][u][lane] = acc[u][0];
+      } else if (!HALF || (lane & 8) == 0) {  // (with at most 8 rows only the lanes of rows 0..7 hold columns anybody reads)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -1255,7 +1279,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
           // after the other through one set of registers and pays the LDS latency three times)
           f32x4 part[kWaves];
 #pragma unroll
-          for (int w = 0; w < kWaves; ++w) part[w] = redbuf[w][e_tile[j]][e_src[j]];
+          for (int w = 0; w < kWaves; ++w) part[w] = PAIRED ? redbuf[w][wave + kWaves * j][lane] : redbuf[w][e_tile[j]][e_src[j]];
           __builtin_amdgcn_sched_barrier(0);
           f32x4 gsum = part[0];
 #pragma unroll
@@ -1370,7 +1394,8 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
 // Measurement aid: what the matrix cores of the device can do on the step's own instruction sequence when nothing has
 // to come from another workgroup.  Every workgroup of the plan's grid runs `steps` steps of what k_lstm2_regw does
 // between the arrival of h and the pointwise part: the B-operand fragments of its k share from LDS (the same
-// fragments every step: there is no recurrence), MT * NT * KSMAX MFMAs per wavefront against W fragments held in
+// fragments every step: there is no recurrence; with groups of at most 8 rows: as loaded pairs that are masked and
+// shifted into the four operand forms, like the kernel does), MT * NT * KSMAX MFMAs per wavefront against W fragments held in
 // registers, the partial tiles through LDS with the step's one barrier, and their sum in wave order (kept as a running
 // value so that nothing can be dropped).  No exchange, no streams, no pointwise arithmetic.  The time of a launch over
 // the op's algorithmic flops is the MFMA roofline a kernel of this decomposition could reach at most.
@@ -1409,31 +1434,56 @@ __global__ __launch_bounds__(kWgThreads) void k_mfma_sequence(float* out, int st
     }
   __syncthreads();
   f32x4 total = f32x4{0.f, 0.f, 0.f, 0.f};
+  constexpr bool PAIRED = HALF && NT == 1 && KSMAX % 2 == 0;  // as in k_lstm2_regw: two tiles share an accumulator
+  constexpr int NLD = PAIRED ? KSMAX / 2 : KSMAX;
+  constexpr int NACC = PAIRED ? MT / 2 : MT;
   auto step = [&](auto par_tag) {
     constexpr int PAR = decltype(par_tag)::value;
     RedBuf& redbuf = red[PAR];
     i32x4 bf[KSMAX][NT];
     asm volatile("" ::: "memory");  // read the fragments again every step
 #pragma unroll
-    for (int ks = 0; ks < KSMAX; ++ks)
+    for (int ks = 0; ks < NLD; ++ks)
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) bf[ks][nt] = Bl[((wave * KSMAX + ks) * NT + nt) * 64 + lane];
-    f32x4 acc[MT][NT];
+    f32x4 acc[NACC][NT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int mt = 0; mt < NACC; ++mt)
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if constexpr (PAIRED) {
+      i32x4 b_lo[KSMAX + 1], b_hi[KSMAX + 1];
+      const int keep_lo = (lane & 8) ? 0 : -1, keep_hi = ~keep_lo;
 #pragma unroll
-    for (int ks = 0; ks < KSMAX; ++ks)
+      for (int a = 0; a < NLD; ++a)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+        for (int w = 0; w < 4; ++w) {
+          b_lo[2 * a][w] = bf[a][0][w] & keep_lo;
+          b_hi[2 * a][w] = __builtin_amdgcn_update_dpp(0, bf[a][0][w], 0x118 /* row_shr:8 */, 0xF, 0xF, true);
+          b_lo[2 * a + 1][w] = __builtin_amdgcn_update_dpp(0, bf[a][0][w], 0x108 /* row_shl:8 */, 0xF, 0xF, true);
+          b_hi[2 * a + 1][w] = bf[a][0][w] & keep_hi;
+        }
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
-    if (!HALF || (lane & 8) == 0) {
+      for (int ks = 0; ks < KSMAX; ++ks)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+        for (int odd = 0; odd < 2; ++odd)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) redbuf[wave][mt * NT + nt][lane] = acc[mt][nt];
+          for (int u = 0; u < NACC; ++u) acc[u][0] = E::mma(wreg[2 * u + odd][ks], odd ? b_hi[ks] : b_lo[ks], acc[u][0]);
+#pragma unroll
+      for (int u = 0; u < NACC; ++u) redbuf[wave][u][lane] = acc[u][0];
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+      if (!HALF || (lane & 8) == 0) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) redbuf[wave][mt * NT + nt][lane] = acc[mt][nt];
+      }
     }
     __syncthreads();
 #pragma unroll
@@ -1444,7 +1494,7 @@ __global__ __launch_bounds__(kWgThreads) void k_mfma_sequence(float* out, int st
         const int src = HALF ? ((lane & 0x30) | (lane & 7)) : lane;
         f32x4 part[kWaves];
 #pragma unroll
-        for (int w = 0; w < kWaves; ++w) part[w] = redbuf[w][e][src];
+        for (int w = 0; w < kWaves; ++w) part[w] = PAIRED ? redbuf[w][u][lane] : redbuf[w][e][src];
         __builtin_amdgcn_sched_barrier(0);
         f32x4 g = part[0];
 #pragma unroll
@@ -1457,6 +1507,62 @@ __global__ __launch_bounds__(kWgThreads) void k_mfma_sequence(float* out, int st
     step(IntTag<0>{});
     if (s + 1 < steps) step(IntTag<1>{});
   }
+  out[(size_t)blockIdx.x * kWgThreads + tid] = total[0] + total[1] + total[2] + total[3];
+}
+
+// Measurement aid: the matrix cores alone.  Every workgroup of the plan's grid issues, per step, the MT * NT * KSMAX MFMAs
+// of one wavefront's share -- the plan's tile sequence, in the op's order (macro steps outside, tiles inside), W fragments
+// and B fragments in registers -- and nothing else: no LDS, no barrier, no sum over the wavefronts, no loads.  (The
+// accumulators run on from step to step instead of starting at zero, and the B fragments pass through an empty
+// assembly statement every step so that the compiler cannot take a step's work for a repetition of the last.)  The time of
+// a launch over the op's algorithmic flops is what the matrix cores can reach on this tile sequence: the ceiling of the
+// recurrent GEMM that no arrangement of the rest of the step can exceed.
+template <typename AT, int MT, int NT, int KSMAX>
+__global__ __launch_bounds__(kWgThreads) void k_mfma_issue(float* out, int steps) {
+  using E = Elem<AT>;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  i32x4 wreg[MT][KSMAX], bf[KSMAX][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks) {
+      AT frag[E::KE];
+#pragma unroll
+      for (int e = 0; e < E::KE; ++e) frag[e] = (AT)(0.001f * (float)(1 + ((lane + 3 * mt + 5 * ks + 7 * wave + e) & 15)));
+      wreg[mt][ks] = __builtin_bit_cast(i32x4, frag);
+    }
+#pragma unroll
+  for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      AT frag[E::KE];
+#pragma unroll
+      for (int e = 0; e < E::KE; ++e) frag[e] = (AT)(0.01f * (float)(1 + ((lane + ks + nt + e) & 7)));
+      bf[ks][nt] = __builtin_bit_cast(i32x4, frag);
+    }
+  f32x4 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < steps; ++s) {
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) asm volatile("" : "+v"(bf[ks][nt]));
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+  }
+  f32x4 total = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) total += acc[mt][nt];
   out[(size_t)blockIdx.x * kWgThreads + tid] = total[0] + total[1] + total[2] + total[3];
 }
 

@@ -3,8 +3,8 @@
 // Validates the operator contract (returnn/native_op.py:1054-1068, 1203-1234, 1249-1252), picks a
 // decomposition, lays out the caller's workspace and enqueues the kernels of lstm2_kernels.h on the
 // caller's stream.  No device memory is allocated here and the stream is never synchronised, so a
-// call can sit inside a captured graph (per-step modes) like the reference's ops do
-// (returnn/torch/util/graph_capture.py:1-80).
+// call can sit inside a captured graph like the reference's ops do (returnn/torch/util/graph_capture.py:1-80):
+// the persistent kernel is recorded as a kernel node of its own (launch_coresident), per-step modes as their launches.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -149,8 +149,8 @@ bool capture_keeps_persistent() {
 }
 
 // Chooses the decomposition.  `want_mode` is the caller's mode; `capturing` says the stream is
-// under capture (a cooperative launch cannot be recorded).  Returns false with a reason when
-// mode == PERSISTENT is impossible.
+// under capture (the persistent kernel is then recorded as a graph node, unless RTN_LSTM2_CAPTURE=steps asks for
+// per-step launches).  Returns false with a reason when mode == PERSISTENT is impossible.
 bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing, Plan* out, std::string* why,
                int max_wgs_per_cu = 2, int count = 1) {
   Plan pl;
@@ -1302,6 +1302,51 @@ SeqKernel seq_kernel_for(int MT, int NT, int KSMAX, bool half) {
   return nullptr;
 }
 
+// The matrix cores alone on the plan's tile sequence (k_mfma_issue): same decompositions as the sequence probe.
+template <typename AT>
+SeqKernel issue_kernel_for(int MT, int NT, int KSMAX) {
+  if (MT == 8 && NT == 1 && KSMAX == 8) return &k_mfma_issue<AT, 8, 1, 8>;
+  if (MT == 4 && NT == 1 && KSMAX == 8) return &k_mfma_issue<AT, 4, 1, 8>;
+  if (MT == 4 && NT == 1 && KSMAX == 4) return &k_mfma_issue<AT, 4, 1, 4>;
+  if (MT == 2 && NT == 1 && KSMAX == 8) return &k_mfma_issue<AT, 2, 1, 8>;
+  if (MT == 1 && NT == 1 && KSMAX == 2) return &k_mfma_issue<AT, 1, 1, 2>;
+  return nullptr;
+}
+
+// Both measurement probes: the plan's grid runs `steps` steps of the plan's MFMA tile sequence -- with the partial tiles
+// through LDS, the step's barrier and their sum (the decomposition's own ceiling), or the MFMAs alone (issue_only).
+int mfma_probe(bool issue_only, int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t steps, void* workspace,
+               size_t workspace_bytes, void* hip_stream) {
+  g_last_error.clear();
+  int rc = check_dims(T, B, n, dtype);
+  if (rc != RTN_OK) return rc;
+  if (count < 1 || steps < 1 || steps > (1 << 24)) return fail(RTN_ERR_ARG, "MFMA sequence probe: count and steps must be positive");
+  Plan pl;
+  std::string why;
+  const int c = std::min<int>(count, kMaxMulti);
+  if (!make_plan(T, B, n, dtype, RTN_MODE_PERSISTENT, false, &pl, &why, 2, c) || !pl.regw)
+    return fail(RTN_ERR_UNSUPPORTED, "MFMA sequence probe: the shape has no persistent register-kernel plan (%s)", why.c_str());
+  SeqKernel k;
+  if (issue_only)
+    k = dtype == RTN_DTYPE_BF16 ? issue_kernel_for<__bf16>(pl.MT, pl.NT, pl.KSMAX) : issue_kernel_for<float>(pl.MT, pl.NT, pl.KSMAX);
+  else
+    k = dtype == RTN_DTYPE_BF16 ? seq_kernel_for<__bf16>(pl.MT, pl.NT, pl.KSMAX, pl.half) : seq_kernel_for<float>(pl.MT, pl.NT, pl.KSMAX, pl.half);
+  if (!k) return fail(RTN_ERR_UNSUPPORTED, "MFMA sequence probe: no build for mt=%d nt=%d ks=%d", pl.MT, pl.NT, pl.KSMAX);
+  // the workgroups that do the plan's work: an XCD-local grid is dealt over all XCDs and part of it may leave at once
+  const int wgs = pl.local ? c * pl.groups * pl.wgs_per_group : (c == 1 ? pl.grid : pl.grid * c);
+  const size_t need = (size_t)wgs * kWgThreads * sizeof(float);
+  if (!workspace || workspace_bytes < need) return fail(RTN_ERR_WORKSPACE, "MFMA sequence probe: workspace of %zu bytes needed", need);
+  if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "MFMA sequence probe: workspace must be 16-byte aligned");
+  const size_t lds = issue_only ? 0 : (size_t)2 * kWaves * pl.MT * pl.NT * kTileBytes + (size_t)kWaves * pl.KSMAX * pl.NT * kTileBytes;
+  rc = ensure_lds_limit((const void*)k, lds);
+  if (rc != RTN_OK) return rc;
+  float* out = (float*)workspace;
+  int st = steps;
+  void* args[] = {(void*)&out, (void*)&st};
+  RTN_HIP(hipLaunchKernel((const void*)k, dim3((unsigned)wgs), dim3(kWgThreads), args, lds, (hipStream_t)hip_stream));
+  return RTN_OK;
+}
+
 // Device address of this GPU's copy of `scratch`: asked of the runtime once per device, with that device current.
 int static_scratch(void** out) {
   static std::mutex mu;
@@ -1452,30 +1497,12 @@ int rtn_handover_latency_probe(void* workspace, size_t workspace_bytes, int32_t 
 
 int rtn_mfma_sequence_probe(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t steps, void* workspace,
                             size_t workspace_bytes, void* hip_stream) {
-  g_last_error.clear();
-  int rc = check_dims(T, B, n, dtype);
-  if (rc != RTN_OK) return rc;
-  if (count < 1 || steps < 1 || steps > (1 << 24)) return fail(RTN_ERR_ARG, "MFMA sequence probe: count and steps must be positive");
-  Plan pl;
-  std::string why;
-  const int c = std::min<int>(count, kMaxMulti);
-  if (!make_plan(T, B, n, dtype, RTN_MODE_PERSISTENT, false, &pl, &why, 2, c) || !pl.regw)
-    return fail(RTN_ERR_UNSUPPORTED, "MFMA sequence probe: the shape has no persistent register-kernel plan (%s)", why.c_str());
-  SeqKernel k = dtype == RTN_DTYPE_BF16 ? seq_kernel_for<__bf16>(pl.MT, pl.NT, pl.KSMAX, pl.half) : seq_kernel_for<float>(pl.MT, pl.NT, pl.KSMAX, pl.half);
-  if (!k) return fail(RTN_ERR_UNSUPPORTED, "MFMA sequence probe: no build for mt=%d nt=%d ks=%d", pl.MT, pl.NT, pl.KSMAX);
-  // the workgroups that do the plan's work: an XCD-local grid is dealt over all XCDs and part of it may leave at once
-  const int wgs = pl.local ? c * pl.groups * pl.wgs_per_group : (c == 1 ? pl.grid : pl.grid * c);
-  const size_t need = (size_t)wgs * kWgThreads * sizeof(float);
-  if (!workspace || workspace_bytes < need) return fail(RTN_ERR_WORKSPACE, "MFMA sequence probe: workspace of %zu bytes needed", need);
-  if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "MFMA sequence probe: workspace must be 16-byte aligned");
-  const size_t lds = (size_t)2 * kWaves * pl.MT * pl.NT * kTileBytes + (size_t)kWaves * pl.KSMAX * pl.NT * kTileBytes;
-  rc = ensure_lds_limit((const void*)k, lds);
-  if (rc != RTN_OK) return rc;
-  float* out = (float*)workspace;
-  int st = steps;
-  void* args[] = {(void*)&out, (void*)&st};
-  RTN_HIP(hipLaunchKernel((const void*)k, dim3((unsigned)wgs), dim3(kWgThreads), args, lds, (hipStream_t)hip_stream));
-  return RTN_OK;
+  return mfma_probe(false, count, T, B, n, dtype, steps, workspace, workspace_bytes, hip_stream);
+}
+
+int rtn_mfma_issue_probe(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t steps, void* workspace,
+                         size_t workspace_bytes, void* hip_stream) {
+  return mfma_probe(true, count, T, B, n, dtype, steps, workspace, workspace_bytes, hip_stream);
 }
 
 size_t rtn_native_lstm2_fwd_multi_workspace_bytes(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode) {

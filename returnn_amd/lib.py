@@ -46,6 +46,7 @@ SYMBOLS = (
     "rtn_native_lstm2_fwd_multi_status",
     "rtn_handover_latency_probe",
     "rtn_mfma_sequence_probe",
+    "rtn_mfma_issue_probe",
     "rtn_native_lstm2_bwd",
     "rtn_native_lstm2_bwd_workspace_bytes",
     "rtn_native_lstm2_bwd_multi",
@@ -191,6 +192,8 @@ def load() -> ctypes.CDLL:
         lib.rtn_graph_cache_stats.argtypes = [ctypes.POINTER(ctypes.c_int64), i32]
         lib.rtn_mfma_sequence_probe.restype = ctypes.c_int
         lib.rtn_mfma_sequence_probe.argtypes = [i32, i64, i32, i32, i32, i32, vp, sz, vp]
+        lib.rtn_mfma_issue_probe.restype = ctypes.c_int
+        lib.rtn_mfma_issue_probe.argtypes = [i32, i64, i32, i32, i32, i32, vp, sz, vp]
         lib.rtn_handover_latency_probe.restype = ctypes.c_int
         lib.rtn_handover_latency_probe.argtypes = [vp, sz, i32, vp]
         lib.rtn_native_lstm2_last_output.restype = ctypes.c_int

@@ -102,3 +102,48 @@ def random_problem(seed, T, B, n, *, ragged=True, full_first=True, scale_x=0.5):
     else:
         i = numpy.ones((T, B), dtype=numpy.float32)
     return X, W, y0, c0, i
+
+
+def run_multi_raw(problems, *, dtype="f32", mode="auto"):
+    """
+    Several op calls of one shape through ``rtn_native_lstm2_fwd_multi`` with explicit workspace and poisoned outputs.
+
+    :param problems: ``[(X, W, y0, c0, i, start, step), ...]`` as numpy arrays, all of one shape
+    :return: plan text, per call ``(Y, C, H, d, y_last)`` as float32 numpy arrays, per call the status words
+        ``(status[0], status[1])`` of its workspace slice (0, 0 = no wait expired, every group of an XCD-local plan on one XCD)
+    """
+    get_op()
+    cabi = lib.load()
+    count = len(problems)
+    T, B = problems[0][4].shape
+    n = problems[0][2].shape[1]
+    act = torch.bfloat16 if dtype == "bf16" else torch.float32
+    dt = lib.DTYPE_BF16 if dtype == "bf16" else lib.DTYPE_F32
+    md = lib.MODES[mode]
+    plan = lib.describe_multi_plan(count, T, B, n, dt, md)
+    arr = (lib.Lstm2Call * count)()
+    keep, outs = [], []
+    for k, (X, W, y0, c0, i, start, step) in enumerate(problems):
+        Xd, Wd, y0d = (to_dev(a, dtype) for a in (X, W, y0))
+        c0d, id_ = (to_dev(a, "f32") for a in (c0, i))
+        Y = torch.full((T, B, n), float("nan"), dtype=act, device="cuda:0")
+        C = torch.full((T, B, n), float("nan"), dtype=torch.float32, device="cuda:0")
+        H = torch.full((T, B, 4 * n), float("nan"), dtype=act, device="cuda:0")
+        d = torch.full((B, n), float("nan"), dtype=torch.float32, device="cuda:0")
+        keep.append((Xd, Wd, y0d, c0d, id_))
+        outs.append((Y, C, H, d, y0d, id_, start, step))
+        arr[k] = lib.Lstm2Call(Xd.data_ptr(), Wd.data_ptr(), y0d.data_ptr(), c0d.data_ptr(), id_.data_ptr(), start, step,
+                               Y.data_ptr(), C.data_ptr(), H.data_ptr(), d.data_ptr())  # fmt: skip
+    nbytes = int(cabi.rtn_native_lstm2_fwd_multi_workspace_bytes(count, T, B, n, dt, md))
+    ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    lib.check(cabi.rtn_native_lstm2_fwd_multi(arr, count, T, B, n, dt, md, ws.data_ptr(), ws.numel(), stream))
+    lib.check(cabi.rtn_native_lstm2_fwd_multi_status(ws.data_ptr(), count, T, B, n, dt, md, stream))
+    torch.cuda.synchronize()
+    each = nbytes // count
+    words = [tuple(int(v) for v in ws[k * each : k * each + 8].cpu().numpy().view(numpy.uint32)) for k in range(count)]
+    results = []
+    for Y, C, H, d, y0d, id_, start, step in outs:
+        y_last = torch_native_op.lstm_last_output(Y, y0d, id_, start, step)
+        results.append(tuple(t.float().cpu().numpy() for t in (Y, C, H, d, y_last)))
+    return plan, results, words

@@ -4,14 +4,15 @@ this package's op loader, so that the GPU tests can run them against the known a
 
 The op descriptions are read as text where they lie (``/root/reference/returnn/native_op.py``, parsed with :mod:`ast` by
 ``tests/_reference_op_sources.py``; nothing of the reference is imported or executed), the loader generates the unit and
-hipcc compiles it in a temporary directory, and only the shared object is kept: ``oracle/_ref/ops/<OpName>.so`` plus
+hipcc compiles it in a temporary directory, and only the shared object is kept: ``tests/_built_ref_ops/<OpName>.so`` plus
 ``ops.json`` with each op's argument table (names, ranks, element types: what a caller needs to bind it).  No source of
-the reference, generated or not, is written into this tree.  ``oracle/_ref/`` is not under version control.
+the reference, generated or not, is written into this tree.  ``tests/_built_ref_ops/`` is not under version control.
+These objects are neither a reference build nor an oracle: they are the thing under test.
 
 What this checks is the loader (dialect header, generated entry point, Python wrapper), not the LSTM kernels: the ops run
 against this package's support header, where the reference would use its own ``native_op.cpp``.
 
-Run: ``python oracle/build_ref_ops.py`` (no GPU needed).  Without the reference tree it does nothing.
+Run: ``python tests/build_ref_ops.py`` (no GPU needed).  Without the reference tree it does nothing.
 """
 
 from __future__ import annotations
@@ -24,7 +25,7 @@ import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-OUT_DIR = os.path.join(HERE, "_ref", "ops")
+OUT_DIR = os.path.join(HERE, "_built_ref_ops")
 
 # ops whose expected results the reference's tests hold as numbers (tests/test_torch_native_op.py:95-160, :582-631,
 # :689-812, :922-1034)

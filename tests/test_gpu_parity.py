@@ -19,7 +19,7 @@ from oracle import lstm2_oracle as oracle
 import torch
 
 from returnn_amd import lib, synthetic
-from _gpu_util import announce, env, get_op, random_problem, run_op, run_raw, to_dev
+from _gpu_util import announce, env, get_op, random_problem, run_multi_raw, run_op, run_raw, to_dev
 from _textbook import REFERENCE_START_STEP, reference_fixture, textbook_lstm, visited_slice
 
 pytestmark = pytest.mark.gpu
@@ -279,6 +279,20 @@ def test_cfg3_bf16_full_size():
         L = int(p.lens[b])
         assert numpy.array_equal(gotb[0][:L, b], gotr[0][:L, b][::-1])
         assert numpy.array_equal(gotb[1][:L, b], gotr[1][:L, b][::-1])
+    # the plan the benchmark times: both calls through the multi-call entry, one launch -- against the oracle at full
+    # length, and bit for bit against the two single calls above
+    announce("cfg3 full pair, one launch")
+    wantb = oracle.native_lstm2_fwd(p.X, p.W, p.y0, p.c0, p.i, 0, -1, threads=oracle.max_threads())
+    args = (p.X, p.W, p.y0, p.c0, p.i)
+    plan, pair, words = run_multi_raw([args + (0, 1), args + (0, -1)], dtype="bf16")
+    assert "kernel=mfma_regw_xcd_half mt=8 nt=1 groups=4 wgs_per_group=32 wgs=256 rows_per_group=8 launches=1" in plan, plan
+    assert words == [(0, 0), (0, 0)], words  # no wait expired; every group was found on one XCD
+    check_bf16(pair[0], want, "cfg3 full pair fwd")
+    check_bf16(pair[1], wantb, "cfg3 full pair bwd")
+    for name, a, b in zip("YCHdy", pair[0], got):
+        assert numpy.array_equal(a, b), "pair fwd vs single call: " + name
+    for name, a, b in zip("YCHdy", pair[1], gotb):
+        assert numpy.array_equal(a, b), "pair bwd vs single call: " + name
 
 
 def test_cfg5_bf16_single_stream():
@@ -297,6 +311,45 @@ def test_cfg5_bf16_single_stream():
     for u, v in zip(a, b):
         assert numpy.array_equal(u, v)
     assert numpy.array_equal(a[3][0], a[1][-1, 0])
+    # and the full length against the oracle (auto mode: the plan the cfg5 benchmark line runs on)
+    announce("cfg5 full vs oracle")
+    wantf = oracle.native_lstm2_fwd(pf.X, pf.W, pf.y0, pf.c0, pf.i, 0, 1, threads=oracle.max_threads())
+    check_bf16(run_op(pf.X, pf.W, pf.y0, pf.c0, pf.i, 0, 1, dtype="bf16", mode="auto"), wantf, "cfg5 T=4000")
+    check_bf16(a, wantf, "cfg5 T=4000 persistent")
+
+
+def test_cfg4_first_layer_full_length():
+    """The first layer of the benchmark encoder (cfg4: features [1000,32,80], n=1024 per direction, bf16) through the layer
+    code (projection GEMM, both directions in one launch, concatenation) against the oracle fed the float32 projection
+    of the same features: 2e-2 absolute on the outputs and the final cell states."""
+    from returnn_amd import lstm as rlstm
+
+    announce("cfg4 first layer T=1000")
+    get_op()
+    prob = synthetic.make_encoder_config("cfg4", num_layers=1)
+    T, B, n = prob.T, prob.B, prob.n
+    mask = (numpy.arange(T)[:, None] < prob.lens[None, :]).astype(numpy.float32)
+    zeros = numpy.zeros((B, n), dtype=numpy.float32)
+    want, weights = {}, {}
+    for key, step in (("fwd", 1), ("bwd", -1)):
+        par = prob.layers[0][key]
+        w = rlstm.prepare_weights(torch.from_numpy(par["ff_weight"]), torch.from_numpy(par["rec_weight"]), torch.from_numpy(par["bias"]))
+        X = (prob.features.reshape(T * B, -1) @ w.ff.numpy() + w.bias.numpy()).reshape(T, B, 4 * n).astype(numpy.float32)
+        want[key] = oracle.native_lstm2_fwd(X, numpy.ascontiguousarray(w.rec.numpy()), zeros, zeros, mask, 0, step, threads=oracle.max_threads())
+        weights[key] = rlstm.LstmWeights(*(None if t is None else t.to("cuda:0").to(torch.bfloat16) for t in w))
+    s0 = rlstm.LstmState(h=torch.zeros((B, n), dtype=torch.bfloat16, device="cuda:0"), c=torch.zeros((B, n), device="cuda:0"))
+    with torch.no_grad():
+        y, sf, sb = rlstm.blstm(torch.from_numpy(prob.features).to("cuda:0").to(torch.bfloat16), fwd=weights["fwd"], bwd=weights["bwd"],
+                                state_fwd=s0, state_bwd=s0, seq_lens=torch.from_numpy(prob.lens))
+    torch.cuda.synchronize()
+    y = y.float().cpu().numpy()
+    assert numpy.all(numpy.isfinite(y))
+    for key, ys, st in (("fwd", y[:, :, :n], sf), ("bwd", y[:, :, n:], sb)):
+        Yw, Cw, Hw, dw, hw = want[key]
+        assert_allclose(ys, Yw, rtol=0, atol=BF16_ATOL, err_msg="cfg4 layer 1 %s Y" % key)
+        assert_allclose(st.c.cpu().numpy(), dw, rtol=0, atol=BF16_ATOL, err_msg="cfg4 layer 1 %s d" % key)
+        assert_allclose(st.h.float().cpu().numpy(), hw, rtol=0, atol=BF16_ATOL, err_msg="cfg4 layer 1 %s final output" % key)
+        print("cfg4 layer 1 %s: max |Y - oracle| = %.3e" % (key, float(numpy.abs(ys - Yw).max())), flush=True)
 
 
 def test_zero_length_and_empty():
@@ -594,9 +647,9 @@ def test_widths_that_run_zero_padded(T, B, n, dtype, start, step):
 
 @pytest.mark.parametrize("T,B,n,dtype", [(12, 8, 128, "bf16"), (9, 5, 100, "f32"), (7, 3, 20, "f32")])
 def test_forward_recorded_into_a_callers_graph(T, B, n, dtype):
-    """Under stream capture the op records one launch per step into the caller's graph (a cooperative launch cannot be
-    recorded).  The graph is replayed three times, with new inputs and the program's own eager work in between; every
-    replay must equal the eager result bit for bit."""
+    """Under stream capture the op records its kernels into the caller's graph: the persistent kernel as a kernel node of
+    its own where the shape has a persistent plan, else one launch per step.  The graph is replayed three times, with new
+    inputs and the program's own eager work in between; every replay must equal the eager result bit for bit."""
     from _gpu_util import to_dev
 
     announce("captured", T, B, n, dtype)

@@ -4,8 +4,8 @@ OptimalCompletionEditDistanceOp), compiled for gfx950 by this package's op loade
 run on the GPU against the numbers the reference's tests hold (tests/golden/ref_op_cases.npz) and, beyond those, against
 the plain numpy recursions that the same numbers pin (tests/test_ref_op_cases.py).
 
-The shared objects are built where the reference tree is (``python oracle/build_ref_ops.py``, also part of the build
-step) into ``oracle/_ref/ops/``; here they are only loaded.  This checks the loader -- dialect header, generated entry
+The shared objects are built where the reference tree is (``python tests/build_ref_ops.py``, also part of the build
+step) into ``tests/_built_ref_ops/``; here they are only loaded.  This checks the loader -- dialect header, generated entry
 point, argument conversion, device allocation callbacks -- on code that was not written for it.
 """
 
@@ -25,12 +25,12 @@ from _gpu_util import announce
 pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-OPS_DIR = os.path.join(ROOT, "oracle", "_ref", "ops")
+OPS_DIR = os.path.join(ROOT, "tests", "_built_ref_ops")
 CASES = os.path.join(ROOT, "tests", "golden", "ref_op_cases.npz")
 
 needs_ops = pytest.mark.skipif(
     not os.path.exists(os.path.join(OPS_DIR, "ops.json")),
-    reason="oracle/_ref/ops is not built (python oracle/build_ref_ops.py, where the reference tree is)",
+    reason="tests/_built_ref_ops is not built (python tests/build_ref_ops.py, where the reference tree is)",
 )
 
 
