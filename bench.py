@@ -882,6 +882,13 @@ def main():
 
     seq_ms = time_probe(cabi.rtn_mfma_sequence_probe)
     issue_ms = time_probe(cabi.rtn_mfma_issue_probe)
+    issue_clock_mhz = None
+    if issue_ms is not None:
+        # threads 1 and 2 of every workgroup of the issue probe leave the loop's duration in shader clocks and in ticks
+        # of the constant 100 MHz clock: the clock rate the matrix cores ran at
+        marks = seq_ws[: 256 * 4 * 4].view(torch.float32).view(4, 256)[:, 1:3].double().cpu()
+        if float(marks[:, 1].min()) > 0:
+            issue_clock_mhz = float((marks[:, 0] / marks[:, 1]).mean()) * 100.0
 
     units_per_step = len(directions) * T * B
     value = units_per_step * args.steps / elapsed
@@ -934,6 +941,7 @@ def main():
                len(directions) // launches, units_per_launch),
             "launch_ms": call_ms,
             **ceiling_fields(probe_us, seq_ms, issue_ms, units_per_launch // T, n, dtype, T, call_ms),
+            "mfma_issue_clock_mhz": issue_clock_mhz,
             "hbm_algorithmic_GBps": bytes_per_launch / (call_ms * 1e-3) / 1e9,
             "hbm_frac": bytes_per_launch / (call_ms * 1e-3) / PEAK_HBM,
         },

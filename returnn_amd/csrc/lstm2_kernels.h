@@ -94,7 +94,8 @@ struct Act<__bf16> {
     return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
   }
   static __device__ __forceinline__ float tanh(float x) {
-    return 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-2.8853900817779268f * x)) - 1.f;
+    // (2 r - 1 as one fused multiply-add: 2 r is exact, so this is bit for bit r + r - 1)
+    return __builtin_fmaf(2.f, __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-2.8853900817779268f * x)), -1.f);
   }
 };
 
@@ -928,14 +929,21 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   // Frame pointers advance by a constant per step (signed: the op may run backwards in time).
   const long long step_x = (long long)p.step * frame_x, step_y = (long long)p.step * frame_y,
                   step_c = (long long)p.step * frame_c, step_m = (long long)p.step * frame_m;
-  auto fetch_at = [&](const unsigned char* xp, const unsigned char* mp, bool enabled, auto par_tag) {  // loads of one frame of X and the mask into register set PAR
+  auto fetch_x_at = [&](const unsigned char* xp, bool enabled, auto par_tag) {  // loads of one frame of X into register set PAR
     constexpr int PAR = decltype(par_tag)::value;
     // (a frame that does not exist: a buffer of no bytes, every load gives 0 without a memory access or a branch)
     __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void*)xp, 0, enabled ? frame_x : 0u, kBufFlags);
-    __amdgpu_buffer_rsrc_t mr = __builtin_amdgcn_make_buffer_rsrc((void*)mp, 0, enabled ? frame_m : 0u, kBufFlags);
 #pragma unroll
     for (int i = 0; i < XCH; ++i) xv[PAR][i] = XC::load(xr, xoff[i]);
+  };
+  auto fetch_m_at = [&](const unsigned char* mp, bool enabled, auto par_tag) {  // ... and of its mask row
+    constexpr int PAR = decltype(par_tag)::value;
+    __amdgpu_buffer_rsrc_t mr = __builtin_amdgcn_make_buffer_rsrc((void*)mp, 0, enabled ? frame_m : 0u, kBufFlags);
     mv[PAR] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(mr, moff, 0, 0));
+  };
+  auto fetch_at = [&](const unsigned char* xp, const unsigned char* mp, bool enabled, auto par_tag) {
+    fetch_x_at(xp, enabled, par_tag);
+    fetch_m_at(mp, enabled, par_tag);
   };
   auto fetch = [&](int s, auto par_tag) {  // issue the loads of X[t_s] and mask[t_s] into register set PAR
     const long long t = frame_of(p, s);
@@ -953,10 +961,10 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   typename XC::T fh[XCH];
   typename YC::T fy[YCH];
   typename CC::T fc[CCH];
-  auto flush_read = [&](int copy) {
-    const unsigned char* hs = smem + L.hs + copy * L.x_copy;
-    const unsigned char* ys = smem + L.ys + copy * L.y_copy;
-    const unsigned char* cs = smem + L.cs + copy * L.c_copy;
+  auto flush_read_at = [&](unsigned hs_off, unsigned ys_off, unsigned cs_off) {  // byte offsets of the copies in LDS
+    const unsigned char* hs = smem + hs_off;
+    const unsigned char* ys = smem + ys_off;
+    const unsigned char* cs = smem + cs_off;
 #pragma unroll
     for (int i = 0; i < XCH; ++i) fh[i] = *(const typename XC::T*)(hs + xlds[i]);
 #pragma unroll
@@ -964,16 +972,26 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
 #pragma unroll
     for (int i = 0; i < CCH; ++i) fc[i] = *(const typename CC::T*)(cs + clds[i]);
   };
-  auto flush_write_at = [&](unsigned char* hp, unsigned char* yp, unsigned char* cp, bool enabled) {
+  auto flush_read = [&](int copy) { flush_read_at(L.hs + copy * L.x_copy, L.ys + copy * L.y_copy, L.cs + copy * L.c_copy); };
+  auto flush_write_h = [&](unsigned char* hp, bool enabled) {
     __amdgpu_buffer_rsrc_t hr = __builtin_amdgcn_make_buffer_rsrc((void*)hp, 0, enabled ? frame_x : 0u, kBufFlags);
-    __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc((void*)yp, 0, enabled ? frame_y : 0u, kBufFlags);
-    __amdgpu_buffer_rsrc_t cr = __builtin_amdgcn_make_buffer_rsrc((void*)cp, 0, enabled ? frame_c : 0u, kBufFlags);
 #pragma unroll
     for (int i = 0; i < XCH; ++i) XC::store(fh[i], hr, xoff[i]);
+  };
+  auto flush_write_y = [&](unsigned char* yp, bool enabled) {
+    __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc((void*)yp, 0, enabled ? frame_y : 0u, kBufFlags);
 #pragma unroll
     for (int i = 0; i < YCH; ++i) YC::store(fy[i], yr, yoff[i]);
+  };
+  auto flush_write_c = [&](unsigned char* cp, bool enabled) {
+    __amdgpu_buffer_rsrc_t cr = __builtin_amdgcn_make_buffer_rsrc((void*)cp, 0, enabled ? frame_c : 0u, kBufFlags);
 #pragma unroll
     for (int i = 0; i < CCH; ++i) CC::store(fc[i], cr, coff[i]);
+  };
+  auto flush_write_at = [&](unsigned char* hp, unsigned char* yp, unsigned char* cp, bool enabled) {
+    flush_write_h(hp, enabled);
+    flush_write_y(yp, enabled);
+    flush_write_c(cp, enabled);
   };
   auto flush_write = [&](int s) {
     const long long t = frame_of(p, s);
@@ -1106,6 +1124,22 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
         m_in[PAR][j] = Ml[PAR * ROWS + e_row[j]];
       }
     };
+    // What the pointwise part needs of this step's gate inputs, the mask and the carried state, made ready in the shadow
+    // of the MFMAs (they were read from LDS one step ago, the state is that of the step before): the gate inputs as
+    // float32, 1 - mask and its products with the carried cell state and output.
+    float x_f[EPT][4], m_f[EPT], keep_c[EPT], keep_h[EPT];
+    auto widen_gate_inputs = [&](auto par_tag) {
+      constexpr int PAR = decltype(par_tag)::value;
+#pragma unroll
+      for (int j = 0; j < EPT; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) x_f[j][q] = (float)x_in[PAR][j][q];
+        m_f[j] = m_in[PAR][j];
+        const float om = 1.f - m_f[j];
+        keep_c[j] = c_state[j] * om;
+        keep_h[j] = h_prev[j] * om;
+      }
+    };
     RTN_TRACE_DECL
     unsigned char *h_out = nullptr, *y_out_p = nullptr, *c_out = nullptr;
     const unsigned char *x_next = nullptr, *m_next = nullptr;
@@ -1125,6 +1159,12 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     // free.  LDS reads are issued ahead of a batch of MFMAs and used behind it.
     auto step = [&](int s, auto par_tag, int stage) {
       constexpr int PAR = decltype(par_tag)::value;
+      // Where the step's staged outputs go and where those of step s-2 lie in LDS: scalar arithmetic done here, while the
+      // read of h is in flight, and not among the first MFMAs (the empty assembly statement keeps it here).
+      const int rd_copy = stage == 2 ? 0 : stage + 1;  // the copy of step s-2 is (s+1) % 3
+      unsigned rd_h = L.hs + rd_copy * L.x_copy, rd_y = L.ys + rd_copy * L.y_copy, rd_c = L.cs + rd_copy * L.c_copy;
+      unsigned st_h = L.hs + stage * L.x_copy, st_y = L.ys + stage * L.y_copy, st_c = L.cs + stage * L.c_copy;
+      asm volatile("" : "+s"(rd_h), "+s"(rd_y), "+s"(rd_c), "+s"(st_h), "+s"(st_y), "+s"(st_c));
 
       // Complete this wave's share of h_{s-1}: if anything that came back is not written yet, read again.
       // (Four independent running maxima: a single chain of dependent packed operations needs a wait state after
@@ -1221,13 +1261,17 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
           const int ks = c >> 1, odd = c & 1;
           i32x4 opnd_next = opnd;
           if (c + 1 < NCH) opnd_next = operand(c + 1);
-          if (c == 0) {
-            flush_read(stage == 2 ? 0 : stage + 1);  // the copy of step s-2 is (s+1) % 3
-            load_gate_inputs(IntTag<1 - PAR>{});
-          }
-          if (c == (NCH > 1 ? 1 : 0)) put(par_tag);
-          if (c == (NCH > 2 ? 2 : NCH - 1)) flush_write_at(h_out, y_out_p, c_out, s >= 2);
-          if (c == (NCH > 3 ? 3 : NCH - 1)) fetch_at(x_next, m_next, s + 4 < nsteps, par_tag);
+          // (at most a dozen instructions fit behind a chunk's four MFMAs; with fewer chunks the last one takes the rest)
+          auto at = [&](int want) { return c == (want < NCH ? want : NCH - 1); };
+          if (at(0)) flush_read_at(rd_h, rd_y, rd_c);
+          if (at(1)) load_gate_inputs(IntTag<1 - PAR>{});
+          if (at(2)) put(par_tag);
+          if (at(3)) flush_write_h(h_out, s >= 2);
+          if (at(4)) flush_write_y(y_out_p, s >= 2);
+          if (at(5)) flush_write_c(c_out, s >= 2);
+          if (at(6)) fetch_x_at(x_next, s + 4 < nsteps, par_tag);
+          if (at(7)) fetch_m_at(m_next, s + 4 < nsteps, par_tag);
+          if (at(8)) widen_gate_inputs(par_tag);
 #pragma unroll
           for (int u = 0; u < NACC; ++u) {
             acc[u][0] = E::mma(wreg[2 * u + odd][ks], opnd, acc[u][0]);
@@ -1238,11 +1282,12 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
           opnd = opnd_next;
         }
       } else {
-        flush_read(stage == 2 ? 0 : stage + 1);  // the copy of step s-2 is (s+1) % 3
+        flush_read_at(rd_h, rd_y, rd_c);
         load_gate_inputs(IntTag<1 - PAR>{});
         put(par_tag);
         flush_write_at(h_out, y_out_p, c_out, s >= 2);
         fetch_at(x_next, m_next, s + 4 < nsteps, par_tag);
+        widen_gate_inputs(par_tag);
 #pragma unroll
         for (int ks = 0; ks < KSMAX; ++ks)
 #pragma unroll
@@ -1284,15 +1329,15 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
           f32x4 gsum = part[0];
 #pragma unroll
           for (int w = 1; w < kWaves; ++w) gsum += part[w];
-          const float m = m_in[PAR][j];
-          const float a0 = Act<AT>::tanh(gsum[0] + (float)x_in[PAR][j][0]);
-          const float a1 = Act<AT>::sigmoid(gsum[1] + (float)x_in[PAR][j][1]);
-          const float a2 = Act<AT>::sigmoid(gsum[2] + (float)x_in[PAR][j][2]);
-          const float a3 = Act<AT>::sigmoid(gsum[3] + (float)x_in[PAR][j][3]);
+          const float m = m_f[j];
+          const float a0 = Act<AT>::tanh(gsum[0] + x_f[j][0]);
+          const float a1 = Act<AT>::sigmoid(gsum[1] + x_f[j][1]);
+          const float a2 = Act<AT>::sigmoid(gsum[2] + x_f[j][2]);
+          const float a3 = Act<AT>::sigmoid(gsum[3] + x_f[j][3]);
           const float pc = c_state[j];
-          const float c = (pc * a2 + a0 * a1) * m + pc * (1.f - m);
+          const float c = (pc * a2 + a0 * a1) * m + keep_c[j];   // keep_c = pc * (1 - m)
           const float y = E::round(Act<AT>::tanh(c) * a3 * m);
-          const float hn = (p.op_flags & kOpNoCarry) ? y : E::round(y + h_prev[j] * (1.f - m));
+          const float hn = (p.op_flags & kOpNoCarry) ? y : E::round(y + keep_h[j]);  // keep_h = h_prev * (1 - m)
           c_state[j] = c;
           h_prev[j] = hn;
           h_bits[j] = SN::bits(hn);
@@ -1319,11 +1364,11 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
 #pragma unroll
       for (int j = 0; j < EPT; ++j) {
         if (UNITS % kWaves == 0 || wave + kWaves * j < UNITS) {
-          unsigned char* hq = smem + L.hs + stage * L.x_copy + e_row[j] * L.x_row + e_cl[j] * ES;
+          unsigned char* hq = smem + st_h + e_row[j] * L.x_row + e_cl[j] * ES;
 #pragma unroll
           for (int q = 0; q < 4; ++q) *(AT*)(hq + q * SEG) = (AT)g_act[j][q];
-          *(AT*)(smem + L.ys + stage * L.y_copy + e_row[j] * L.y_row + e_cl[j] * ES) = (AT)y_out[j];
-          *(float*)(smem + L.cs + stage * L.c_copy + e_row[j] * L.c_row + e_cl[j] * 4) = c_state[j];
+          *(AT*)(smem + st_y + e_row[j] * L.y_row + e_cl[j] * ES) = (AT)y_out[j];
+          *(float*)(smem + st_c + e_row[j] * L.c_row + e_cl[j] * 4) = c_state[j];
         }
       }
       if (s + 1 < nsteps) {
@@ -1546,6 +1591,7 @@ __global__ __launch_bounds__(kWgThreads) void k_mfma_issue(float* out, int steps
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const unsigned long long clk0 = clock64(), wall0 = wall_clock64();
   for (int s = 0; s < steps; ++s) {
 #pragma unroll
     for (int ks = 0; ks < KSMAX; ++ks)
@@ -1563,7 +1609,13 @@ __global__ __launch_bounds__(kWgThreads) void k_mfma_issue(float* out, int steps
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) total += acc[mt][nt];
-  out[(size_t)blockIdx.x * kWgThreads + tid] = total[0] + total[1] + total[2] + total[3];
+  // Thread 0 leaves the sum (so that nothing can be dropped), threads 1 and 2 what the loop took in shader clocks and in
+  // ticks of the constant 100 MHz clock: their ratio is the clock rate the matrix cores ran at under this load.
+  const unsigned long long clk1 = clock64(), wall1 = wall_clock64();
+  float v = total[0] + total[1] + total[2] + total[3];
+  if (tid == 1) v = (float)(clk1 - clk0);
+  if (tid == 2) v = (float)(wall1 - wall0);
+  out[(size_t)blockIdx.x * kWgThreads + tid] = v;
 }
 
 // Measurement aid: the latency of handing a value from every workgroup to every other one, the way the persistent
