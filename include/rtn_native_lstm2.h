@@ -373,7 +373,17 @@ const char* rtn_native_lstm2_capture_report(void);
  * the benchmark line and tests.  "kernel=bwd_regw_xcd": every batch group on one XCD. */
 const char* rtn_native_lstm2_bwd_plan_text(void);
 
-/* ABI version of this header: 11. */
+/*
+ * The library reads its RTN_LSTM2_* environment variables (experiment and debugging knobs: plan overrides, capture
+ * behaviour, wait bounds) once, at its first use, into a snapshot that all later calls plan by; this re-reads them.
+ * For programs that change such a variable while running (the tests do).  Thread-safe (a call that runs while another
+ * thread re-reads may plan by either snapshot, never by a mixture within one lookup).  The reference has no counterpart: its knobs are Python keyword
+ * arguments of make_op (returnn/torch/util/native_op.py:39-57) and one environment variable read at compile time
+ * (returnn/util/native_code_compiler.py:63-65).
+ */
+void rtn_native_lstm2_reload_env(void);
+
+/* ABI version of this header: 12. */
 int rtn_native_lstm2_abi_version(void);
 
 #ifdef __cplusplus

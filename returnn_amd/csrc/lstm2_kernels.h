@@ -793,6 +793,11 @@ __device__ __forceinline__ unsigned xcc_id() {
   return x & 0xFu;
 }
 
+// Which XCDs does the device deal the workgroups of a grid to?  Every workgroup adds the XCD it runs on to a bit mask.
+__global__ void k_probe_xcds(unsigned* mask) {
+  if (threadIdx.x == 0) (void)__hip_atomic_fetch_or(mask, 1u << xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // One thread per workgroup: are all `members` workgroups that share `words` on one XCD?  Every caller adds its XCD to the
 // mask words[1] and then itself to the count words[0] (both cleared before the launch; device-scope atomics whose result
 // is waited for, so the mask is complete when the count is).  The wait is bounded like every other (status[0] = 1 when it
@@ -1562,8 +1567,8 @@ __global__ __launch_bounds__(kWgThreads) void k_mfma_sequence(float* out, int st
 // assembly statement every step so that the compiler cannot take a step's work for a repetition of the last.)  The time of
 // a launch over the op's algorithmic flops is what the matrix cores can reach on this tile sequence: the ceiling of the
 // recurrent GEMM that no arrangement of the rest of the step can exceed.
-template <typename AT, int MT, int NT, int KSMAX>
-__global__ __launch_bounds__(kWgThreads) void k_mfma_issue(float* out, int steps) {
+template <typename AT, int MT, int NT, int KSMAX, int THREADS = kWgThreads>
+__global__ __launch_bounds__(THREADS) void k_mfma_issue(float* out, int steps) {
   using E = Elem<AT>;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1615,7 +1620,7 @@ __global__ __launch_bounds__(kWgThreads) void k_mfma_issue(float* out, int steps
   float v = total[0] + total[1] + total[2] + total[3];
   if (tid == 1) v = (float)(clk1 - clk0);
   if (tid == 2) v = (float)(wall1 - wall0);
-  out[(size_t)blockIdx.x * kWgThreads + tid] = v;
+  if (tid < kWgThreads) out[(size_t)blockIdx.x * kWgThreads + tid] = v;
 }
 
 // Measurement aid: the latency of handing a value from every workgroup to every other one, the way the persistent

@@ -13,9 +13,12 @@
 #include <cstdlib>
 #include <cstring>
 #include <list>
+#include <map>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <tuple>
+#include <unordered_map>
 #include <utility>
 #include <vector>
 
@@ -56,8 +59,52 @@ int fail(int code, const char* fmt, ...) {
                   __FILE__, __LINE__);                                                                 \
   } while (0)
 
+// The RTN_LSTM2_* environment is read ONCE, into a snapshot (at the first use, and again when the caller asks with
+// rtn_native_lstm2_reload_env()): planning does not call getenv per knob and per call, and a setenv in another thread
+// cannot race with a reader (readers hold a reference to an immutable snapshot).  `generation` counts the snapshots;
+// whatever is cached per plan carries the generation it was made under.
+extern "C" char** environ;
+struct EnvSnapshot {
+  std::unordered_map<std::string, std::string> vars;  // RTN_LSTM2_* only
+  unsigned long long generation = 0;
+};
+std::mutex g_env_mu;
+std::shared_ptr<const EnvSnapshot> g_env;
+unsigned long long g_env_generation = 0;
+
+std::shared_ptr<const EnvSnapshot> take_env_snapshot() {  // g_env_mu held
+  auto snap = std::make_shared<EnvSnapshot>();
+  for (char** e = environ; e && *e; ++e) {
+    if (strncmp(*e, "RTN_LSTM2_", 10) != 0) continue;
+    const char* eq = strchr(*e, '=');
+    if (eq) snap->vars.emplace(std::string(*e, eq - *e), std::string(eq + 1));
+  }
+  snap->generation = ++g_env_generation;
+  return snap;
+}
+
+std::shared_ptr<const EnvSnapshot> env_snapshot() {
+  std::lock_guard<std::mutex> lock(g_env_mu);
+  if (!g_env) g_env = take_env_snapshot();
+  return g_env;
+}
+
+void reload_env() {
+  std::lock_guard<std::mutex> lock(g_env_mu);
+  g_env = take_env_snapshot();
+}
+
+// The value of an RTN_LSTM2_* variable in the snapshot, or nullptr.  (The pointer stays valid while the caller's thread
+// holds `keep`, which the accessors below do for the duration of a call through a thread-local reference.)
+thread_local std::shared_ptr<const EnvSnapshot> t_env;
+const char* env_get(const char* name) {
+  t_env = env_snapshot();
+  auto it = t_env->vars.find(name);
+  return it == t_env->vars.end() ? nullptr : it->second.c_str();
+}
+
 long env_long(const char* name, long dflt) {
-  const char* v = getenv(name);
+  const char* v = env_get(name);
   if (!v || !*v) return dflt;
   char* end = nullptr;
   long r = strtol(v, &end, 0);
@@ -74,9 +121,14 @@ struct DeviceInfo {
 
 // Properties of the current device; falls back to MI355X's published figures when no device is
 // visible (the workspace-size and plan queries must work on a build host without a GPU).
+// The XCD count is not among the runtime's device properties.  Until the device has been asked (probe_xcds below, at the
+// first call that enqueues work outside stream capture) it is taken to be 8 for devices of 64 CUs or more that divide by
+// 8; the kernels check the placement of every group at run time either way.
+std::mutex g_dev_mu;
+DeviceInfo g_dev_cache[64];
+bool g_dev_probed[64] = {false};
+
 DeviceInfo device_info() {
-  static std::mutex mu;
-  static DeviceInfo cache[64];
   int dev = 0;
   DeviceInfo fallback;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
@@ -86,8 +138,8 @@ DeviceInfo device_info() {
   // RTN_LSTM2_XCDS: pretend the workgroup ids are dealt to this many XCDs (an experiment and test knob: with a wrong
   // count the groups of an XCD-local plan do not sit on one XCD each, the kernel notices and exchanges at device scope)
   const long env_xcds = env_long("RTN_LSTM2_XCDS", 0);
-  std::lock_guard<std::mutex> lock(mu);
-  if (!cache[dev].valid) {
+  std::lock_guard<std::mutex> lock(g_dev_mu);
+  if (!g_dev_cache[dev].valid) {
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
       (void)hipGetLastError();
@@ -100,9 +152,9 @@ DeviceInfo device_info() {
     if (di.lds_per_wg < (size_t)prop.sharedMemPerBlock) di.lds_per_wg = prop.sharedMemPerBlock;
     di.cooperative = prop.cooperativeLaunch != 0;
     di.valid = true;
-    cache[dev] = di;
+    g_dev_cache[dev] = di;
   }
-  DeviceInfo di = cache[dev];
+  DeviceInfo di = g_dev_cache[dev];
   if (env_xcds > 0 && di.cus % env_xcds == 0) di.xcds = (int)env_xcds;
   return di;
 }
@@ -144,15 +196,15 @@ size_t mfma_lds_bytes(int n, int dtype, int MT, int NT) {
 
 // Whether calls made under stream capture keep the persistent kernels (default) or record per-step launches.
 bool capture_keeps_persistent() {
-  const char* v = getenv("RTN_LSTM2_CAPTURE");
+  const char* v = env_get("RTN_LSTM2_CAPTURE");
   return !(v && strcmp(v, "steps") == 0);
 }
 
 // Chooses the decomposition.  `want_mode` is the caller's mode; `capturing` says the stream is
 // under capture (the persistent kernel is then recorded as a graph node, unless RTN_LSTM2_CAPTURE=steps asks for
 // per-step launches).  Returns false with a reason when mode == PERSISTENT is impossible.
-bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing, Plan* out, std::string* why,
-               int max_wgs_per_cu = 2, int count = 1) {
+bool make_plan_uncached(int64_t T, int B, int n, int dtype, int want_mode, bool capturing, Plan* out, std::string* why,
+                        int max_wgs_per_cu, int count) {
   Plan pl;
   // One problem on its own is planned with a CU per workgroup (sharing CUs did not pay off in measurements).
   max_wgs_per_cu = (int)std::max<long>(1, std::min<long>(max_wgs_per_cu, env_long("RTN_LSTM2_WGS_PER_CU", 1)));
@@ -316,7 +368,9 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
           const bool shares = count > 1 && di.cus / each < count;
           const double cost = 0.873 * (mfma_us(loc) - mfma_us(chosen)) + 0.25 * (passes(loc) - passes(chosen));
           const double more_kb = std::max(0, chosen.Bg - loc.Bg) * (double)n * es / 1024.0;  // hidden state per CU and step
-          const double gain = 0.20 + (each * std::max(count, 1) > di.cus / 2 ? 0.25 : 0.0) + 0.005 * more_kb;
+          // (bf16: 0.40 since two tiles of a group of up to 8 rows share an accumulator -- measured again at n = 256 ... 1024
+          // with 1 ... 64 rows: the XCD-local plan is ahead or level everywhere, a single sequence of n = 1024 included)
+          const double gain = (dtype == RTN_DTYPE_BF16 ? 0.40 : 0.20) + (each * std::max(count, 1) > di.cus / 2 ? 0.25 : 0.0) + 0.005 * more_kb;
           take_local = shares || cost < gain;
         }
         if (loc.ok && (env_long("RTN_LSTM2_LOCAL", -1) == 1 || take_local)) chosen = loc;
@@ -425,6 +479,50 @@ bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing
   return true;
 }
 
+// Plans are kept per (shape class, element type, mode, capture state, workgroups per CU, problems per launch, device,
+// environment snapshot): the search above runs once per key, and two threads that plan the same call get the same plan.
+// (T only matters as "no frames at all".)
+struct PlanCacheEntry {
+  bool ok;
+  Plan plan;
+  std::string why;
+};
+std::mutex g_plan_mu;
+std::map<std::tuple<bool, int, int, int, int, bool, int, int, int, unsigned long long>, PlanCacheEntry> g_plans;
+constexpr size_t kMaxCachedPlans = 4096;
+
+bool make_plan(int64_t T, int B, int n, int dtype, int want_mode, bool capturing, Plan* out, std::string* why,
+               int max_wgs_per_cu = 2, int count = 1) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    dev = -1;
+  }
+  const auto key = std::make_tuple(T == 0, B, n, dtype, want_mode, capturing, max_wgs_per_cu, count, dev, env_snapshot()->generation);
+  {
+    std::lock_guard<std::mutex> lock(g_plan_mu);
+    auto it = g_plans.find(key);
+    if (it != g_plans.end()) {
+      if (it->second.ok) *out = it->second.plan;
+      if (why) *why = it->second.why;
+      return it->second.ok;
+    }
+  }
+  PlanCacheEntry e;
+  e.ok = make_plan_uncached(T, B, n, dtype, want_mode, capturing, &e.plan, &e.why, max_wgs_per_cu, count);
+  if (e.ok) *out = e.plan;
+  if (why) *why = e.why;
+  std::lock_guard<std::mutex> lock(g_plan_mu);
+  if (g_plans.size() >= kMaxCachedPlans) g_plans.clear();
+  g_plans.emplace(key, e);
+  return e.ok;
+}
+
+void clear_plan_cache() {
+  std::lock_guard<std::mutex> lock(g_plan_mu);
+  g_plans.clear();
+}
+
 const char* mode_name(int mode) {
   switch (mode) {
     case RTN_MODE_PERSISTENT: return "persistent";
@@ -500,6 +598,27 @@ int ensure_lds_limit(const void* k, size_t lds_bytes) {
   return RTN_OK;
 }
 
+// Workgroups of a kernel that fit a CU together, asked of the runtime once per (device, kernel, threads, LDS bytes).
+int occupancy_per_cu(const void* k, int threads, size_t lds_bytes, int* per_cu) {
+  static std::mutex mu;
+  static std::map<std::tuple<int, const void*, int, size_t>, int> known;
+  int dev = 0;
+  RTN_HIP(hipGetDevice(&dev));
+  const auto key = std::make_tuple(dev, k, threads, lds_bytes);
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = known.find(key);
+    if (it != known.end()) {
+      *per_cu = it->second;
+      return RTN_OK;
+    }
+  }
+  RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, k, threads, lds_bytes));
+  std::lock_guard<std::mutex> lock(mu);
+  known[key] = *per_cu;
+  return RTN_OK;
+}
+
 // Where a sequence of kernel launches goes: onto a stream, or into a graph under construction (one kernel node per launch,
 // each depending on the one before).  Every kernel of such a sequence takes the call's parameter block by value as its
 // first argument: that is what lets a graph built for one set of buffers be aimed at another set later.
@@ -567,7 +686,7 @@ int enqueue(LaunchSink& sink, void (*k)(P...), dim3 grid, dim3 block, size_t lds
 }
 
 // Library-owned graphs of per-step launch sequences.  The key holds what fixes the structure of the sequence (shape,
-// element type, plan, device): no addresses.  A graph whose kernel nodes carry another parameter block than the call's
+// element type, plan, device) and the stream the graph is launched on: no addresses.  A graph whose kernel nodes carry another parameter block than the call's
 // (other buffers, same shape) gets the new block written into every node of its executable form before the launch.
 struct GraphEntry {
   std::string key;
@@ -608,10 +727,20 @@ int launch_entry(GraphEntry& e, hipStream_t stream) {
   return RTN_OK;
 }
 
+template <typename T>
+void key_append(std::string* key, const T& v) {
+  key->append(reinterpret_cast<const char*>(&v), sizeof(T));
+}
+
 // Launches the graph kept for `key` with the parameter block [block, block + bytes) in the first argument of every
 // kernel node; builds the graph first (by calling `record` with a sink that collects nodes) if there is none.
+// An executable graph is only ever launched on the stream it was first launched on (the stream is part of the key): its
+// launches are then ordered by that stream, the one event behind the last of them covers them all when the entry is
+// retired, and rewriting its nodes' parameters never meets a launch of the same executable graph running on another stream.
 template <typename Record>
-int replay_graph(const std::string& key, const void* block, size_t bytes, hipStream_t stream, Record record) {
+int replay_graph(const std::string& shape_key, const void* block, size_t bytes, hipStream_t stream, Record record) {
+  std::string key(shape_key);
+  key_append(&key, stream);
   std::lock_guard<std::mutex> lock(g_graph_mu);
   sweep_retired();
   for (auto it = g_graphs.begin(); it != g_graphs.end(); ++it) {
@@ -663,11 +792,6 @@ int replay_graph(const std::string& key, const void* block, size_t bytes, hipStr
     g_retired.splice(g_retired.end(), g_graphs, std::prev(g_graphs.end()));
   }
   return launch_entry(g_graphs.front(), stream);
-}
-
-template <typename T>
-void key_append(std::string* key, const T& v) {
-  key->append(reinterpret_cast<const char*>(&v), sizeof(T));
 }
 
 int launch_steps(const Lstm2Params& p, const Plan& pl, int dtype, LaunchSink& sink) {
@@ -733,7 +857,7 @@ int launch_coresident(const void* k, dim3 grid, dim3 block, void** args, unsigne
     RTN_HIP(hipLaunchCooperativeKernel(k, grid, block, args, lds, stream));
     return RTN_OK;
   }
-  const char* kind = getenv("RTN_LSTM2_CAPTURE_NODE");
+  const char* kind = env_get("RTN_LSTM2_CAPTURE_NODE");
   bool try_cooperative = !(kind && strcmp(kind, "plain") == 0);
   {
     std::lock_guard<std::mutex> lock(g_capture_mu);
@@ -907,6 +1031,47 @@ size_t workspace_each(int count, int64_t T, int32_t B, int32_t n, int32_t dtype,
   return workspace_each_exact(count, T, B, np, dtype, mode) + fwd_pad_layout(T, B, np, dtype).total;
 }
 
+int static_scratch(void** out);
+void clear_plan_cache();
+
+// Asks the device once how many XCDs it deals workgroups to: a grid of 1024 small workgroups notes the XCD each runs on
+// (hardware register XCC_ID) in a word of the library's static device array, the word comes back over the caller's stream,
+// which is waited for -- the one time the library synchronises a stream, at the first call on a device that enqueues
+// work outside stream capture.  If the count differs from the assumed one, plans made so far are dropped.
+int probe_xcds(hipStream_t stream) {
+  int dev = 0;
+  RTN_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) return RTN_OK;
+  (void)device_info();  // fills the cache entry
+  {
+    std::lock_guard<std::mutex> lock(g_dev_mu);
+    if (g_dev_probed[dev] || !g_dev_cache[dev].valid) return RTN_OK;
+    g_dev_probed[dev] = true;  // one attempt
+  }
+  void* word = nullptr;
+  int rc = static_scratch(&word);
+  if (rc != RTN_OK) return rc;
+  unsigned mask = 0;
+  hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(64), 0, stream, (unsigned*)word, 0u, 64LL);
+  hipLaunchKernelGGL(k_probe_xcds, dim3(1024), dim3(64), 0, stream, (unsigned*)word);
+  RTN_HIP(hipGetLastError());
+  RTN_HIP(hipMemcpyAsync(&mask, word, sizeof(mask), hipMemcpyDeviceToHost, stream));
+  RTN_HIP(hipStreamSynchronize(stream));
+  int count = 0;
+  for (unsigned m = mask; m; m &= m - 1) ++count;
+  bool changed = false;
+  {
+    std::lock_guard<std::mutex> lock(g_dev_mu);
+    DeviceInfo& di = g_dev_cache[dev];
+    if (count >= 1 && di.cus % count == 0 && di.xcds != count) {
+      di.xcds = count;
+      changed = true;
+    }
+  }
+  if (changed) clear_plan_cache();
+  return RTN_OK;
+}
+
 // The calls of one entry: `count` independent problems of one shape.  Each gets the slice
 // [k * each, (k + 1) * each) of the workspace, each = workspace_each(count, ...).
 // When the persistent register kernel fits that many times on the device at once, all of them run
@@ -1011,7 +1176,8 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     if (rc != RTN_OK) return rc;
     const int wgs = pl.regw ? pl.grid : pl.groups * pl.wgs_per_group;
     int per_cu = 0;
-    RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, pk, kWgThreads, pl.lds_bytes));
+    rc = occupancy_per_cu(pk, kWgThreads, pl.lds_bytes, &per_cu);
+    if (rc != RTN_OK) return rc;
     const long long capacity = (long long)per_cu * device_info().cus;
     if (capacity >= wgs) {
       if (pl.local) {
@@ -1038,6 +1204,9 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     return fail(RTN_ERR_WORKSPACE, "NativeLstm2: workspace of %zu bytes needed, got %zu", each_ws * (size_t)count,
                 workspace ? workspace_bytes : (size_t)0);
   if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2: workspace must be 16-byte aligned");
+  // (all arguments are in order: from here on work is enqueued.  The first such call on a device asks it for its XCD
+  // count; the plan above was made with the assumed count, which the kernels verify for every group anyway.)
+  if (!capturing && (rc = probe_xcds(stream)) != RTN_OK) return rc;
 
   Lstm2Multi multi;
   memset(&multi, 0, sizeof(multi));
@@ -1327,7 +1496,17 @@ int mfma_probe(bool issue_only, int32_t count, int64_t T, int32_t B, int32_t n, 
   if (!make_plan(T, B, n, dtype, RTN_MODE_PERSISTENT, false, &pl, &why, 2, c) || !pl.regw)
     return fail(RTN_ERR_UNSUPPORTED, "MFMA sequence probe: the shape has no persistent register-kernel plan (%s)", why.c_str());
   SeqKernel k;
-  if (issue_only)
+  int threads = kWgThreads;
+  if (issue_only && env_long("RTN_LSTM2_PROBE_WAVES", 4) == 8 && dtype == RTN_DTYPE_BF16 && pl.MT == 8 && pl.NT == 1 && pl.KSMAX == 8) {
+    // experiment: the same MFMAs dealt to two wavefronts per SIMD (8 per workgroup, half the macro steps each)
+    k = &k_mfma_issue<__bf16, 8, 1, 4, 512>;
+    threads = 512;
+  } else if (issue_only && env_long("RTN_LSTM2_PROBE_WAVES", 4) == 44 && dtype == RTN_DTYPE_BF16) {
+    k = &k_mfma_issue<__bf16, 8, 1, 4, 256>;  // experiment: half the MFMAs, all operands in architectural registers
+  } else if (issue_only && env_long("RTN_LSTM2_PROBE_WAVES", 4) == 16 && dtype == RTN_DTYPE_BF16) {
+    k = &k_mfma_issue<__bf16, 8, 1, 2, 1024>;  // experiment: four wavefronts per SIMD
+    threads = 1024;
+  } else if (issue_only)
     k = dtype == RTN_DTYPE_BF16 ? issue_kernel_for<__bf16>(pl.MT, pl.NT, pl.KSMAX) : issue_kernel_for<float>(pl.MT, pl.NT, pl.KSMAX);
   else
     k = dtype == RTN_DTYPE_BF16 ? seq_kernel_for<__bf16>(pl.MT, pl.NT, pl.KSMAX, pl.half) : seq_kernel_for<float>(pl.MT, pl.NT, pl.KSMAX, pl.half);
@@ -1343,7 +1522,7 @@ int mfma_probe(bool issue_only, int32_t count, int64_t T, int32_t B, int32_t n, 
   float* out = (float*)workspace;
   int st = steps;
   void* args[] = {(void*)&out, (void*)&st};
-  RTN_HIP(hipLaunchKernel((const void*)k, dim3((unsigned)wgs), dim3(kWgThreads), args, lds, (hipStream_t)hip_stream));
+  RTN_HIP(hipLaunchKernel((const void*)k, dim3((unsigned)wgs), dim3((unsigned)threads), args, lds, (hipStream_t)hip_stream));
   return RTN_OK;
 }
 
@@ -1372,9 +1551,11 @@ using namespace rtn;
 
 extern "C" {
 
-int rtn_native_lstm2_abi_version(void) { return 11; }
+int rtn_native_lstm2_abi_version(void) { return 12; }
 
 const char* rtn_native_lstm2_bwd_plan_text(void) { return g_bwd_plan_text.c_str(); }
+
+void rtn_native_lstm2_reload_env(void) { reload_env(); }
 
 const char* rtn_native_lstm2_capture_report(void) {
   static thread_local std::string text;
@@ -1651,10 +1832,12 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
   const long long nn4 = (long long)n * n * 4;
   hipStreamCaptureStatus cap_status = hipStreamCaptureStatusNone;
   if (stream) RTN_HIP(hipStreamIsCapturing(stream, &cap_status));
-  // Under stream capture everything is recorded into the caller's graph: one launch per frame (a cooperative launch
-  // cannot be recorded) and the rocBLAS calls of the weight gradient (the library's rocBLAS handle must exist already:
-  // run the op once outside the capture first, as for any library that sets itself up on first use).
+  // Under stream capture everything is recorded into the caller's graph: the persistent kernel as a kernel node of its
+  // own (launch_coresident) or one launch per frame, and the rocBLAS calls of the weight gradient (the library's rocBLAS
+  // handle must exist already: run the op once outside the capture first, as for any library that sets itself up on
+  // first use).
   const bool capturing = cap_status != hipStreamCaptureStatusNone;
+  if (!capturing && T > 0 && bn > 0 && (rc = probe_xcds(stream)) != RTN_OK) return rc;
   const dim3 fill_grid(256), fill_block(256);
   for (int k = 0; k < count; ++k) {
     const rtn_lstm2_bwd_call& c = calls[k];
@@ -1814,7 +1997,7 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
           if (rc != RTN_OK) return rc;
         }
         int per_cu = 0;
-        RTN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kfn, 64 * wv, cand_lds));
+        if ((rc = occupancy_per_cu((const void*)kfn, 64 * wv, cand_lds, &per_cu)) != RTN_OK) return rc;
         const long long groups_needed = (B + use_rows - 1) / use_rows;
         const long long G_wgs = n / (16 * mt), cu_x = di_b.xcds > 0 ? di_b.cus / di_b.xcds : 0;
         if (local_only && n / 16 <= cu_x * per_cu) continue;  // (groups of one tile per workgroup fit an XCD themselves)

@@ -31,7 +31,7 @@ MODE_PERSISTENT = 1
 MODE_GRAPH = 2
 MODE_STEPWISE = 3
 # The ABI version the structs and argument lists below were written for (rtn_native_lstm2_abi_version()).
-EXPECTED_ABI = 11
+EXPECTED_ABI = 12
 
 MODES = {"auto": MODE_AUTO, "persistent": MODE_PERSISTENT, "graph": MODE_GRAPH, "stepwise": MODE_STEPWISE}
 
@@ -66,6 +66,7 @@ SYMBOLS = (
     "rtn_graph_cache_stats",
     "rtn_native_lstm2_capture_report",
     "rtn_native_lstm2_bwd_plan_text",
+    "rtn_native_lstm2_reload_env",
     "rtn_native_lstm2_abi_version",
 )
 
@@ -204,10 +205,19 @@ def load() -> ctypes.CDLL:
         lib.rtn_native_lstm2_describe_plan.argtypes = [i64, i32, i32, i32, i32]
         lib.rtn_native_lstm2_describe_multi_plan.restype = ctypes.c_char_p
         lib.rtn_native_lstm2_describe_multi_plan.argtypes = [i32, i64, i32, i32, i32, i32]
-        lib.rtn_native_lstm2_abi_version.restype = ctypes.c_int
-        lib.rtn_native_lstm2_abi_version.argtypes = []
+        lib.rtn_native_lstm2_reload_env.restype = None
+        lib.rtn_native_lstm2_reload_env.argtypes = []
         _lib = lib
         return lib
+
+
+def reload_env() -> None:
+    """Make the library read its ``RTN_LSTM2_*`` environment variables again (it reads them once, at first use).  Does
+    nothing while the library is not loaded: its first use will read the environment as it is then."""
+    with _lock:
+        lib = _lib
+    if lib is not None:
+        lib.rtn_native_lstm2_reload_env()
 
 
 def last_error() -> str:

@@ -20,7 +20,7 @@ def get_op(mode="auto"):
 
 @contextlib.contextmanager
 def env(**kwargs):
-    """Temporarily set environment variables the library reads at each call."""
+    """Temporarily set environment variables of the library (it reads them once and again when asked to)."""
     old = {k: os.environ.get(k) for k in kwargs}
     try:
         for k, v in kwargs.items():
@@ -28,6 +28,7 @@ def env(**kwargs):
                 os.environ.pop(k, None)
             else:
                 os.environ[k] = str(v)
+        lib.reload_env()
         yield
     finally:
         for k, v in old.items():
@@ -35,6 +36,7 @@ def env(**kwargs):
                 os.environ.pop(k, None)
             else:
                 os.environ[k] = v
+        lib.reload_env()
 
 
 def announce(*what):

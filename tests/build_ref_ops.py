@@ -1,5 +1,5 @@
 """
-Test infrastructure, never shipped with the library: builds a few of the reference's OTHER native ops for gfx950 through
+Test infrastructure, never shipped with the library: builds seven of the reference's OTHER native ops for gfx950 through
 this package's op loader, so that the GPU tests can run them against the known answers the reference's own tests hold.
 
 The op descriptions are read as text where they lie (``/root/reference/returnn/native_op.py``, parsed with :mod:`ast` by
@@ -28,8 +28,9 @@ ROOT = os.path.dirname(HERE)
 OUT_DIR = os.path.join(HERE, "_built_ref_ops")
 
 # ops whose expected results the reference's tests hold as numbers (tests/test_torch_native_op.py:95-160, :582-631,
-# :689-812, :922-1034)
-OPS = ("FastBaumWelchOp", "FastViterbiOp", "EditDistanceOp", "OptimalCompletionEditDistanceOp")
+# :689-812, :922-1034, :1036-1400)
+OPS = ("FastBaumWelchOp", "FastViterbiOp", "EditDistanceOp", "OptimalCompletionEditDistanceOp",
+       "OptimalCompletionEditDistancePerSuccessorOp", "NextEditDistanceRowOp", "NextEditDistanceReduceOp")
 
 
 def _plain(x):

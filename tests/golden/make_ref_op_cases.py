@@ -1,5 +1,5 @@
 """
-Writes ``ref_op_cases.npz``: inputs and expected results of four of the reference's other native ops, for the test
+Writes ``ref_op_cases.npz``: inputs and expected results of seven of the reference's other native ops, for the test
 that runs those ops on the GPU after the op loader of this package has compiled them.  Run from the repository root:
 ``python tests/golden/make_ref_op_cases.py``.  Needs nothing from the reference tree.
 
@@ -14,7 +14,15 @@ Everything expected here is DATA that the reference's own tests hold, retyped fr
   drawn from ``RandomState(42)``, and ``test_edit_distance_ref_np_b1`` (:905-912): seven pairs with distances
   1, 1, 2, 1, 1, 2, 1;
 * ``test_optimal_completion_edit_distance`` (:922-976): seven explicit pairs with results 1, 0, 1, 1, 1, 0, 0 inside
-  another batch of 15.
+  another batch of 15;
+* ``test_optimal_completion_edit_distance_per_successor`` (:1036-1135): seven explicit pairs with results 1, 0, 1, 1, 1, 0, 0
+  (the sixth other than above: labels stay below the 10 classes) for the successor that is the prefix's own last label,
+  inside a batch of 15; the op is given the prefixes without their last label and returns one result per successor label;
+* ``test_next_edit_distance_row`` (:1137-1276) and ``test_next_edit_distance_row_optimal_completion`` (:1278-1365): the
+  batches of ``test_edit_distance`` and ``test_optimal_completion_edit_distance`` again, computed one row of the
+  dynamic programme per op call;
+* ``test_next_edit_distance_reduce_optimal_completion`` (:1367-1400): a batch of 15 with prefixes of full length 7, one
+  result per successor label (no numbers held: every entry is left to the reference's naive routine).
 
 Where the reference's test leaves an entry of the batch to its own numpy routine (the random rest), the expected number
 is computed here by the textbook dynamic programme below; ``*_held`` marks the entries the reference holds as numbers,
@@ -162,10 +170,50 @@ def optimal_completion_edit_distance():
     return {"oc_a": a, "oc_a_len": a_len, "oc_b": b, "oc_b_len": b_len, "oc_expected": expected, "oc_held": held}
 
 
+def per_successor():
+    """OptimalCompletionEditDistancePerSuccessorOp: ``expected[i, j]`` = smallest distance between the prefix of sequence i
+    without its last label, followed by label j, and any prefix of b."""
+    num_classes = 10
+    explicit = [
+        ([1], [], 1, 0, 1),
+        ([1], [1, 2], 1, 2, 0),
+        ([1], [3, 1], 1, 2, 1),
+        ([1, 2, 3, 4], [1, 2, 4, 4], 4, 4, 1),
+        ([1, 2, 3, 4, 5], [1, 2, 3, 3, 4, 5], 5, 6, 1),
+        ([2, 2, 4, 4, 6, 6, 8, 8, 9, 1, 3], [2, 2, 4, 4, 6, 6, 8, 8, 9, 1, 3], 11, 11, 0),
+        ([2, 2, 4, 4, 6, 6, 8, 8, 9, 10, 0], [2, 2, 4, 4, 6, 6, 8, 8, 9, 10, 0, 0, 0], 11, 13, 0),
+    ]
+    a, a_len, b, b_len, whole, held = _batch(numpy.random.RandomState(42), 15, 11, 13, explicit, optimal_completion)
+    expected = numpy.zeros((a.shape[0], num_classes), dtype=numpy.int32)
+    for i in range(a.shape[0]):
+        for j in range(num_classes):
+            expected[i, j] = optimal_completion(list(a[i, : a_len[i] - 1]) + [j], list(b[i, : b_len[i]]))
+        last = int(a[i, a_len[i] - 1])
+        assert 0 <= last < num_classes and expected[i, last] == whole[i]  # the held numbers sit in this column
+    return {"ps_a": a, "ps_a_len": a_len, "ps_b": b, "ps_b_len": b_len, "ps_expected": expected, "ps_whole": whole, "ps_held": held,
+            "ps_num_classes": numpy.int32(num_classes)}  # fmt: skip
+
+
+def next_reduce():
+    """NextEditDistanceReduceOp after all of a has been consumed row by row: ``expected[i, j]`` = smallest distance between
+    a[i] followed by label j and any prefix of b[i]."""
+    rnd = numpy.random.RandomState(42)
+    n_batch, n_a, n_b, num_classes = 15, 7, 13, 10
+    a = rnd.randint(0, num_classes, size=(n_batch, n_a), dtype="int32")
+    b = rnd.randint(0, num_classes, size=(n_batch, n_b), dtype="int32")
+    a_len = numpy.array([n_a] * n_batch, dtype="int32")
+    b_len = rnd.randint(1, n_b + 1, size=(n_batch,), dtype="int32")
+    expected = numpy.zeros((n_batch, num_classes), dtype=numpy.int32)
+    for i in range(n_batch):
+        for j in range(num_classes):
+            expected[i, j] = optimal_completion(list(a[i]) + [j], list(b[i, : b_len[i]]))
+    return {"nr_a": a, "nr_a_len": a_len, "nr_b": b, "nr_b_len": b_len, "nr_expected": expected, "nr_num_classes": numpy.int32(num_classes)}
+
+
 def main():
     here = os.path.dirname(os.path.abspath(__file__))
     out = {}
-    for part in (fast_bw_uniform(), fast_viterbi(), edit_distance(), optimal_completion_edit_distance()):
+    for part in (fast_bw_uniform(), fast_viterbi(), edit_distance(), optimal_completion_edit_distance(), per_successor(), next_reduce()):
         out.update(part)
     numpy.savez_compressed(os.path.join(here, "ref_op_cases.npz"), **out)
     print("wrote ref_op_cases.npz:", ", ".join(sorted(out)))

@@ -116,17 +116,52 @@ def test_xcd_local_plans(cabi):
     assert "kernel=mfma_regw_xcd_half mt=8 nt=1 groups=4 wgs_per_group=32 wgs=256 rows_per_group=8 " in pair, pair
     one = lib.describe_plan(1000, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
     assert "kernel=mfma_regw_xcd_half" in one and "groups=8 " in one and "rows_per_group=4 " in one, one
-    # a single sequence, and float32 at n = 512, keep W spread over more CUs (fewer MFMAs per wavefront and step)
-    assert "kernel=mfma_regw " in lib.describe_plan(4000, 1, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
+    # a single bf16 sequence goes to one XCD too (its hidden state then never leaves that XCD's L2)
+    single = lib.describe_plan(4000, 1, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
+    assert "kernel=mfma_regw_xcd_half mt=8 nt=1 groups=1 wgs_per_group=32 " in single, single
+    # float32 at n = 512 keeps W spread over more CUs (fewer MFMAs per wavefront and step)
     assert "kernel=mfma_regw " in lib.describe_plan(500, 64, 512, lib.DTYPE_F32, lib.MODE_AUTO)
-    # the environment switch
+    # the environment switch: read once, and again when the library is told to
     os.environ["RTN_LSTM2_LOCAL"] = "0"
     try:
+        assert "kernel=mfma_regw_xcd_half" in lib.describe_multi_plan(2, 1000, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)  # old snapshot
+        lib.reload_env()
         assert "kernel=mfma_regw " in lib.describe_multi_plan(2, 1000, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
     finally:
         del os.environ["RTN_LSTM2_LOCAL"]
+        lib.reload_env()
+    assert "kernel=mfma_regw_xcd_half" in lib.describe_multi_plan(2, 1000, 32, 1024, lib.DTYPE_BF16, lib.MODE_AUTO)
     # a layer whose group does not fit the CUs of one XCD has no such plan
     assert "_xcd" not in lib.describe_plan(100, 32, 2048, lib.DTYPE_BF16, lib.MODE_AUTO)
+
+
+def test_two_threads_plan_alike(cabi):
+    """Planning is deterministic and safe from several host threads at once: the same shapes, planned concurrently and
+    while a third thread keeps re-reading the environment, give the same plan texts as planned alone."""
+    import threading
+
+    shapes = [(T, B, n, dt) for T in (1, 37, 1000) for B in (1, 5, 32, 200) for n in (32, 96, 512, 1024, 2048)
+              for dt in (lib.DTYPE_F32, lib.DTYPE_BF16)]
+    alone = [lib.describe_plan(*sh, lib.MODE_AUTO) for sh in shapes]
+    results, stop = {}, threading.Event()
+
+    def plan(tag, order):
+        results[tag] = {k: lib.describe_plan(*shapes[k], lib.MODE_AUTO) for k in order}
+
+    def reload():
+        while not stop.is_set():
+            lib.reload_env()
+
+    ts = [threading.Thread(target=plan, args=("a", range(len(shapes)))),
+          threading.Thread(target=plan, args=("b", range(len(shapes) - 1, -1, -1))),
+          threading.Thread(target=reload)]
+    for t in ts:
+        t.start()
+    ts[0].join(); ts[1].join()  # noqa: E702
+    stop.set()
+    ts[2].join()
+    for k, want in enumerate(alone):
+        assert results["a"][k] == want and results["b"][k] == want, (shapes[k], want, results["a"][k], results["b"][k])
 
 
 def test_plan_invariants_over_shapes(cabi):

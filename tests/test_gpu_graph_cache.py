@@ -112,6 +112,34 @@ def test_same_graph_back_to_back_on_other_buffers_without_waiting():
         _same(got[r], want[r], "queued launch %i" % r)
 
 
+def test_two_streams_share_shapes_without_waiting_for_each_other():
+    """Two streams run the same shapes at the same time, each on its own buffers, over more shapes than the cache holds,
+    with no synchronisation until the end.  A kept graph belongs to the stream it was first launched on, so one stream's
+    call never rewrites or retires an executable graph that the other stream may still be running."""
+    announce("graph cache: two streams")
+    get_op()
+    keep, got, want = [], {}, {}
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    problems = {(k, q): random_problem(4500 + 10 * k + q, *SHAPES[k][:3]) for k in range(len(SHAPES)) for q in range(2)}
+    torch.cuda.synchronize()
+    before = lib.graph_cache_stats()
+    for rnd in range(2):  # the second round meets graphs pushed out by the first
+        for k, (T, B, n, dtype) in enumerate(SHAPES):
+            for q, st in enumerate(streams):
+                with torch.cuda.stream(st):
+                    got[(rnd, k, q)] = _forward(problems[(k, q)], dtype, "graph", keep)
+    torch.cuda.synchronize()
+    for k, (T, B, n, dtype) in enumerate(SHAPES):
+        for q in range(2):
+            want[(k, q)] = _forward(problems[(k, q)], dtype, "stepwise", keep)
+    torch.cuda.synchronize()
+    for (rnd, k, q), outs in got.items():
+        _same(outs, want[(k, q)], "round %i shape %r stream %i" % (rnd, SHAPES[k], q))
+    after = lib.graph_cache_stats()
+    assert after["built"] - before["built"] >= 2 * len(SHAPES), (before, after)  # one graph per shape and stream
+    assert after["kept"] <= 8 and after["retiring"] == 0, after
+
+
 @pytest.mark.parametrize("T,B,n,dtype", [(9, 5, 128, "bf16"), (7, 3, 20, "f32")])
 def test_gradient_graph_on_other_buffers(T, B, n, dtype):
     """The per-frame launches of the gradient entry go through the same cache: other buffers of a known shape reuse the

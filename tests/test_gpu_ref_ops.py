@@ -1,6 +1,7 @@
 """
-Four of the reference's other native ops (FastBaumWelchOp, FastViterbiOp, EditDistanceOp,
-OptimalCompletionEditDistanceOp), compiled for gfx950 by this package's op loader from the reference's own op sources,
+Seven of the reference's other native ops (FastBaumWelchOp, FastViterbiOp, EditDistanceOp,
+OptimalCompletionEditDistanceOp, OptimalCompletionEditDistancePerSuccessorOp, NextEditDistanceRowOp,
+NextEditDistanceReduceOp), compiled for gfx950 by this package's op loader from the reference's own op sources,
 run on the GPU against the numbers the reference's tests hold (tests/golden/ref_op_cases.npz) and, beyond those, against
 the plain numpy recursions that the same numbers pin (tests/test_ref_op_cases.py).
 
@@ -112,3 +113,72 @@ def test_edit_distance_known_answers(name, prefix):
         assert swapped.cpu().numpy().tolist() == want.tolist()
         (got1,) = op(_dev(c["ed1_a"]), _dev(c["ed1_a_len"]), _dev(c["ed1_b"]), _dev(c["ed1_b_len"]))
         assert got1.cpu().numpy().tolist() == c["ed1_expected"].tolist()
+
+
+@needs_ops
+def test_optimal_completion_per_successor_known_answers():
+    """tests/test_torch_native_op.py:1036-1135: the op gets every prefix without its last label and answers for all ten
+    successor labels; the numbers the reference holds are those of the prefix's own last label."""
+    announce("reference op OptimalCompletionEditDistancePerSuccessorOp")
+    c = dict(numpy.load(CASES))
+    op = _op("OptimalCompletionEditDistancePerSuccessorOp")
+    a, a_len, b, b_len = c["ps_a"], c["ps_a_len"], c["ps_b"], c["ps_b_len"]
+    n_labels = int(c["ps_num_classes"])
+    (got,) = op(_dev(a), _dev(a_len - 1), _dev(b), _dev(b_len), _dev(numpy.arange(n_labels, dtype=numpy.int32)))
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    assert got.shape == (a.shape[0], n_labels)
+    assert got.tolist() == c["ps_expected"].tolist()
+    for i in range(a.shape[0]):
+        assert int(got[i, a[i, a_len[i] - 1]]) == int(c["ps_whole"][i])
+    assert c["ps_held"].sum() == 7 and c["ps_whole"][c["ps_held"]].tolist() == [1, 0, 1, 1, 1, 0, 0]
+
+
+def _rows(op, a, a_len, b, b_len):
+    """The dynamic programme one row per op call (the protocol of returnn/torch/util/native_op.py:1129-1160): the row
+    starts as 0..b_time for every sequence; call i hands over label i of every sequence and whether it has ended."""
+    n_batch, time1 = a.shape
+    row = _dev(numpy.tile(numpy.arange(b.shape[1] + 1, dtype=numpy.int32)[None], (n_batch, 1)))
+    bd, bl = _dev(b), _dev(b_len)
+    for i in range(time1):
+        ended = (i >= a_len).astype(numpy.int32)
+        (row,) = op(row, _dev(a[:, i]), _dev(numpy.full((n_batch,), i, dtype=numpy.int32)), _dev(ended), bd, bl)
+    return row
+
+
+@needs_ops
+def test_next_edit_distance_row_known_answers():
+    """tests/test_torch_native_op.py:1137-1365: the batches of the two edit-distance tests, row by row: the last entry of
+    the final row is the edit distance (whole batch, pair by pair cut to its lengths, and with the roles swapped), its
+    minimum the optimal-completion distance."""
+    announce("reference op NextEditDistanceRowOp")
+    c = dict(numpy.load(CASES))
+    op = _op("NextEditDistanceRowOp")
+    a, a_len, b, b_len, want = (c["ed_%s" % k] for k in ("a", "a_len", "b", "b_len", "expected"))
+    assert c["ed_held"].sum() == 8 and want[c["ed_held"]].tolist() == [1, 1, 2, 1, 1, 1, 0, 2]
+    assert _rows(op, a, a_len, b, b_len)[:, -1].cpu().numpy().tolist() == want.tolist()
+    assert _rows(op, b, b_len, a, a_len)[:, -1].cpu().numpy().tolist() == want.tolist()
+    for i in range(a.shape[0]):
+        ai, bi = a[i : i + 1, : a_len[i]], b[i : i + 1, : b_len[i]]
+        assert int(_rows(op, ai, a_len[i : i + 1], bi, b_len[i : i + 1])[0, -1].cpu()) == int(want[i]), i
+        assert int(_rows(op, bi, b_len[i : i + 1], ai, a_len[i : i + 1])[0, -1].cpu()) == int(want[i]), i
+    a, a_len, b, b_len, want = (c["oc_%s" % k] for k in ("a", "a_len", "b", "b_len", "expected"))
+    assert want[c["oc_held"]].tolist() == [1, 0, 1, 1, 1, 0, 0]
+    assert _rows(op, a, a_len, b, b_len).min(dim=1).values.cpu().numpy().tolist() == want.tolist()
+
+
+@needs_ops
+def test_next_edit_distance_reduce_answers():
+    """tests/test_torch_native_op.py:1367-1400 (and returnn/torch/util/native_op.py:1188-1217 for the protocol): all of a
+    row by row, then one call that answers for every successor label."""
+    announce("reference op NextEditDistanceReduceOp")
+    c = dict(numpy.load(CASES))
+    row_op, op = _op("NextEditDistanceRowOp"), _op("NextEditDistanceReduceOp")
+    a, a_len, b, b_len = c["nr_a"], c["nr_a_len"], c["nr_b"], c["nr_b_len"]
+    n_labels = int(c["nr_num_classes"])
+    last_row = _rows(row_op, a, a_len, b, b_len)
+    n_batch = a.shape[0]
+    (got,) = op(last_row, _dev(numpy.arange(n_labels, dtype=numpy.int32)[None]), _dev(numpy.full((n_batch,), a.shape[1], dtype=numpy.int32)),
+                _dev((a_len != a.shape[1]).astype(numpy.int32)), _dev(b), _dev(b_len), 1, -1)  # fmt: skip
+    torch.cuda.synchronize()
+    assert got.cpu().numpy().tolist() == c["nr_expected"].tolist()

@@ -28,7 +28,8 @@ def _cases():
 def test_file_is_what_the_script_writes():
     mod, stored = _script(), _cases()
     fresh = {}
-    for part in (mod.fast_bw_uniform(), mod.fast_viterbi(), mod.edit_distance(), mod.optimal_completion_edit_distance()):
+    for part in (mod.fast_bw_uniform(), mod.fast_viterbi(), mod.edit_distance(), mod.optimal_completion_edit_distance(),
+                 mod.per_successor(), mod.next_reduce()):
         fresh.update(part)
     assert sorted(fresh) == sorted(stored)
     for k in fresh:
@@ -63,3 +64,27 @@ def test_edit_distance_numbers():
         a, b = list(c["ed_a"][i, : c["ed_a_len"][i]]), list(c["ed_b"][i, : c["ed_b_len"][i]])
         assert mod.levenshtein(a, b) == mod.levenshtein(b, a) == c["ed_expected"][i]  # symmetric, as the reference checks by swapping
         assert abs(len(a) - len(b)) <= c["ed_expected"][i] <= max(len(a), len(b))
+
+
+def test_successor_tables():
+    """The per-successor tables: the column of a prefix's own last label holds the whole prefix's number (seven of them
+    held by the reference), and the row-by-row dynamic programme the GPU test drives gives the same numbers in numpy."""
+    mod, c = _script(), _cases()
+    assert c["ps_held"].sum() == 7 and c["ps_whole"][c["ps_held"]].tolist() == [1, 0, 1, 1, 1, 0, 0]
+    for i in range(c["ps_a"].shape[0]):
+        last = int(c["ps_a"][i, c["ps_a_len"][i] - 1])
+        assert c["ps_expected"][i, last] == c["ps_whole"][i]
+
+    def next_row(row, label, b):  # one row of Wagner-Fischer
+        new = [row[0] + 1]
+        for j in range(1, len(b) + 1):
+            new.append(min(row[j] + 1, new[j - 1] + 1, row[j - 1] + (0 if label == b[j - 1] else 1)))
+        return new
+
+    for i in range(c["nr_a"].shape[0]):
+        b = list(c["nr_b"][i, : c["nr_b_len"][i]])
+        row = list(range(len(b) + 1))
+        for label in c["nr_a"][i]:
+            row = next_row(row, int(label), b)
+        for j in range(int(c["nr_num_classes"])):
+            assert min(next_row(row, j, b)) == c["nr_expected"][i, j]
