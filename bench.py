@@ -117,6 +117,33 @@ def ceiling_fields(probe_us, seq_ms, issue_ms, rows, n, dtype, T, call_ms):
     return out
 
 
+def step_budget(call_ms, nowait_ms, seq_ms, issue_ms, T):
+    """
+    Where a time step of the persistent kernel goes, from four launches of T steps each timed in this run; the entries
+    add up to the measured step by construction, each is the difference of two measurements:
+
+    * ``mfma_issue``: the issue probe (the plan's MFMAs per wavefront and nothing else);
+    * ``partial_tiles_through_lds``: sequence probe - issue probe (operands from LDS, the four wavefronts' partial
+      tiles written to LDS, the step's barrier, their sum read back);
+    * ``gates_streams_stores``: the op's kernel with the reads of the hidden state switched off - sequence probe (gate
+      arithmetic, cell update, the exchange stores, what the X / H / Y / C streams cost although they ride behind the
+      MFMAs);
+    * ``exchange_wait``: the op's kernel - the same with those reads switched off (the delay in front of the first read
+      of the hidden state, the read's round trip through L2, its check, repeated reads).
+    """
+    if None in (call_ms, nowait_ms, seq_ms, issue_ms):
+        return None
+    us = lambda ms: ms * 1e3 / T  # noqa: E731
+    return {
+        "mfma_issue": us(issue_ms),
+        "partial_tiles_through_lds": us(seq_ms - issue_ms),
+        "gates_streams_stores": us(nowait_ms - seq_ms),
+        "exchange_wait": us(call_ms - nowait_ms),
+        "sum": us(call_ms),
+        "no_wait_launch_ms": nowait_ms,
+    }
+
+
 def blas_thread_count():
     """Threads the BLAS behind numpy uses for one SGEMM, and where that figure comes from."""
     try:
@@ -721,6 +748,9 @@ def main():
                     help="fwd: the forward op (default, the headline metric); bwd: the gradient op of one direction of "
                          "the workload (cfg1/cfg2/cfg3/cfg5; with cfg4: the encoder's training step, forward + backward); generic_base, low_mem: forward of the sibling ops on the workload's shape")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-step-budget", action="store_true",
+                    help="skip the extra launches with the exchange waits switched off (profile runs: a kernel trace then "
+                    "holds launches of the op's kernel as the op runs it, and nothing else under its name)")
     ap.add_argument("--no-torch-baseline", action="store_true", help="cfg4: skip timing the same stack through torch.nn.LSTM")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -890,6 +920,33 @@ def main():
         if float(marks[:, 1].min()) > 0:
             issue_clock_mhz = float((marks[:, 0] / marks[:, 1]).mean()) * 100.0
 
+    # The same launch with the reads of the hidden state switched off (a timing aid of the library: no loads from the
+    # exchange ring, no delay in front of them, no waiting -- the MFMAs run on zeros, the new values are still stored;
+    # results are invalid and the status word says so): what a step costs when the hidden state is there for free.
+    # The difference to the measured launch is what the step spends on getting it.
+    nowait_ms = None
+    if "mfma_regw" in lib.describe_multi_plan(2 if fused else 1, T, B, n, dt_code, mode) and not measuring_only and not args.no_step_budget:
+        os.environ["RTN_LSTM2_EXCHANGE"] = "3"
+        lib.reload_env()
+        try:
+            ne = []
+            for _ in range(1 + 3):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for k in range(launches):
+                    one_call(k)
+                e1.record(stream)
+                ne.append((e0, e1))
+            torch.cuda.synchronize()
+            nowait_ms = min(a.elapsed_time(b) for a, b in ne[1:]) / launches
+        finally:
+            del os.environ["RTN_LSTM2_EXCHANGE"]
+            lib.reload_env()
+        for k in range(launches):  # leave valid results behind
+            one_call(k)
+        torch.cuda.synchronize()
+        check_status()
+
     units_per_step = len(directions) * T * B
     value = units_per_step * args.steps / elapsed
     units_per_launch = units_per_step // launches
@@ -942,6 +999,7 @@ def main():
             "launch_ms": call_ms,
             **ceiling_fields(probe_us, seq_ms, issue_ms, units_per_launch // T, n, dtype, T, call_ms),
             "mfma_issue_clock_mhz": issue_clock_mhz,
+            "step_budget_us": step_budget(call_ms, nowait_ms, seq_ms, issue_ms, T),
             "hbm_algorithmic_GBps": bytes_per_launch / (call_ms * 1e-3) / 1e9,
             "hbm_frac": bytes_per_launch / (call_ms * 1e-3) / PEAK_HBM,
         },
@@ -962,7 +1020,8 @@ def main():
             "mfma_TFLOPs": achieved / 1e12,
         })
         for key in ("latency_ceiling", "frac_of_latency_ceiling", "mfma_peak_us_per_step", "achievable_mfma", "frac_of_achievable_mfma",
-                    "mfma_sequence_us_per_step", "mfma_issue_us_per_step", "decomposition_ceiling", "frac_of_decomposition_ceiling"):
+                    "mfma_sequence_us_per_step", "mfma_issue_us_per_step", "mfma_issue_clock_mhz", "step_budget_us", "decomposition_ceiling",
+                    "frac_of_decomposition_ceiling"):
             result["roofline"].pop(key, None)  # they describe the exchange-bound persistent kernel
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, args.cpu_seconds)

@@ -150,6 +150,13 @@ typedef struct rtn_lstm2_call {
   float* C;
   void* H;
   float* d;
+  /* Row pitch of X and of Y in elements: the distance between the rows of two consecutive (frame, sequence) pairs.
+   * 0 = contiguous (4n and n).  A larger pitch lets the calls of a bidirectional layer share arrays the way the reference's
+   * caller lays them out (returnn/tf/layers/rec.py:1229-1270 concatenates the two directions' outputs): both directions
+   * read their pre-projected gates from one [T*B, 8n] projection (X = base + 0 and base + 4n, ldX = 8n) and write their
+   * outputs into one [T, B, 2n] array (Y = base + 0 and base + n, ldY = 2n).  Rows must stay 16-byte aligned. */
+  int64_t ldX;
+  int64_t ldY;
 } rtn_lstm2_call;
 
 int rtn_native_lstm2_fwd_multi(const rtn_lstm2_call* calls, int32_t count, int64_t T, int32_t B, int32_t n,
@@ -255,6 +262,13 @@ typedef struct rtn_lstm2_bwd_call {
   float* DW;
   void* Dy0;
   float* Dc0;
+  /* Row pitch in elements of Y, DY (rows of n) and DX (rows of 4n), as ldX / ldY of rtn_lstm2_call; 0 = contiguous.  The
+   * two directions of a bidirectional layer read the error of one [T, B, 2n] output (DY = base + 0 and base + n,
+   * ldDY = 2n) and write their derivatives into one [T*B, 8n] array (DX = base + 0 and base + 4n, ldDX = 8n), from which
+   * the gradient of the input projection is then a single product.  H, C and the mask are contiguous. */
+  int64_t ldY;
+  int64_t ldDY;
+  int64_t ldDX;
 } rtn_lstm2_bwd_call;
 
 int rtn_native_lstm2_bwd_multi(const rtn_lstm2_bwd_call* calls, int32_t count, int64_t T, int32_t B, int32_t n,
@@ -331,10 +345,10 @@ size_t rtn_lstm_low_mem_bwd_workspace_bytes(int64_t T, int32_t B, int32_t n_in, 
  * Final output per sequence.  Replaces the caller-side `_lstm_last_output`
  * (returnn/tf/native_op.py:913-929): out[b] = Y[t*, b] for the last visited frame t*
  * (in processing order) with i[t*, b] != 0, else y0[b].  Y, y0, out have element
- * type `dtype`; needs no workspace.
+ * type `dtype`; ldY: row pitch of Y in elements as in rtn_lstm2_call, 0 = n; needs no workspace.
  */
 int rtn_native_lstm2_last_output(const void* Y, const void* y0, const float* i, int32_t start, int32_t step,
-                                 void* out, int64_t T, int32_t B, int32_t n, int32_t dtype, void* hip_stream);
+                                 void* out, int64_t T, int32_t B, int32_t n, int32_t dtype, int64_t ldY, void* hip_stream);
 
 /* Text of the calling thread's last error ("" if none).  Stands in for the message of the
  * exception TORCH_CHECK raises (returnn/native_op.cpp:660). */

@@ -15,9 +15,9 @@ struct Lstm2BwdParams {
   const float* mask;  // [T,B]
   const float* C;     // [T,B,n]
   const void* H;      // [T,B,4n] AT, activated gates of the forward pass
-  const void* DY;     // [T,B,n] AT
+  const void* DY;     // [T,B,n] AT, rows ldDY elements apart
   // outputs / working arrays (device)
-  void* DX;    // [T,B,4n] AT
+  void* DX;    // [T,B,4n] AT, rows ldDX elements apart
   float* dyw;  // [B,n]  error flowing into the output of the frame before (working copy of Dy0, float32)
   float* Dc0;  // [B,n]  cell error, worked on in place
   void* dx0;   // [B,4n] AT: DX of each sequence's first processed valid frame
@@ -25,6 +25,7 @@ struct Lstm2BwdParams {
   int B, n;
   int op_flags;  // OpFlags: kOpNoCarry, kOpH0IsCell select the gradient of LstmGenericBase (returnn/native_op.py:430-485)
   int pad_;
+  long long ldDY, ldDX;  // row pitch of DY and DX in elements (n and 4n when contiguous); H, C and the mask are contiguous
   const void* Wpk;  // per-frame launches: W in MFMA A-operand order, [n/16][4n/KM][64] fragments of 16 bytes (else null)
 };
 
@@ -89,11 +90,13 @@ __global__ void k_bwd_pointwise(Lstm2BwdParams p, long long t, long long prev_t)
   const int n = p.n;
   const long long b = idx / n, cell = idx % n;
   const long long io = b * 4 * n + cell;
-  const long long fo = t * bn * 4 + io;  // inside H / DX
+  const long long fo = t * bn * 4 + io;  // inside H
+  const long long xo = (t * p.B + b) * p.ldDX + cell;  // inside DX
   const float m = p.mask[t * p.B + b];
   const float dyw = p.dyw[idx];
   const bool raw_dh = (p.op_flags & kOpRawDh) != 0;
-  const float err_y = raw_dh ? E::load(p.DY, t * bn + idx) * m + dyw : (E::load(p.DY, t * bn + idx) + dyw) * m;
+  const float dy = E::load(p.DY, (t * p.B + b) * p.ldDY + cell);
+  const float err_y = raw_dh ? dy * m + dyw : (dy + dyw) * m;
   const float dc = p.Dc0[idx];
   const float err_c = dc * m;
   const float prev_c = bwd_prev_cell<AT>(p, prev_t, idx, io);
@@ -103,7 +106,7 @@ __global__ void k_bwd_pointwise(Lstm2BwdParams p, long long t, long long prev_t)
   p.Dc0[idx] = a_fg * err_cell + dc * (1.f - m);
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    E::store(p.DX, fo + g * n, dx[g]);
+    E::store(p.DX, xo + g * n, dx[g]);
     const float old = E::load(p.dx0, io + g * n);
     E::store(p.dx0, io + g * n, raw_dh ? dx[g] : dx[g] + old * (1.f - m));
   }
@@ -147,7 +150,7 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
       const long long io = (long long)b * n4 + k;
       const long long fo = t * bn * 4 + io;
       q_m[nt] = p.mask[t * p.B + b];
-      q_dy[nt] = E::load(p.DY, t * bn + idx);
+      q_dy[nt] = E::load(p.DY, (t * p.B + b) * p.ldDY + k);
       q_dc[nt] = p.Dc0[idx];
       q_pc[nt] = bwd_prev_cell<AT>(p, prev_t, idx, io);
 #pragma unroll
@@ -161,7 +164,7 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
     const int S = n4 / KM;
     const AT* Wr = (const AT*)p.W + (size_t)(k0 + (lane & 15)) * n4 + KE * (lane >> 4);
     const i32x4* Wk = p.Wpk ? (const i32x4*)p.Wpk + (size_t)(k0 / 16) * S * 64 + lane : nullptr;  // packed: fragment s at Wk[64 * s]
-    const AT* Dx = (const AT*)p.DX + (size_t)t_gemm * p.B * n4 + KE * (lane >> 4);
+    const AT* Dx = (const AT*)p.DX + (size_t)t_gemm * p.B * p.ldDX + KE * (lane >> 4);
     int brow[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) brow[nt] = min(b0 + 16 * nt + (lane & 15), p.B - 1);  // rows past B: any row, dropped below
@@ -178,7 +181,7 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
         const int s = min(s0 + kWaves * u, S - 1);  // past the end: a valid address, the product is dropped
         a[u] = Wk ? Wk[(size_t)64 * s] : *(const i32x4*)(Wr + (size_t)KM * s);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) bfrag[u][nt] = *(const i32x4*)(Dx + (size_t)brow[nt] * n4 + (size_t)KM * s);
+        for (int nt = 0; nt < NT; ++nt) bfrag[u][nt] = *(const i32x4*)(Dx + (size_t)brow[nt] * p.ldDX + (size_t)KM * s);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -210,9 +213,8 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
     float dyw = q_dyw[nt];
     if (t_gemm >= 0) dyw += tile[nt][bl][kl];
     if (t >= 0) {
-      const long long bn = (long long)p.B * n;
       const long long io = (long long)b * n4 + k;
-      const long long fo = t * bn * 4 + io;
+      const long long xo = (t * p.B + b) * p.ldDX + k;
       const float m = q_m[nt];
       const bool raw_dh = (p.op_flags & kOpRawDh) != 0;
       const float err_y = raw_dh ? q_dy[nt] * m + dyw : (q_dy[nt] + dyw) * m;
@@ -224,7 +226,7 @@ __global__ __launch_bounds__(kWgThreads) void k_bwd_step(Lstm2BwdParams p, long 
       p.Dc0[idx] = a_fg * err_cell + dc * (1.f - m);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        E::store(p.DX, fo + g * n, dx[g]);
+        E::store(p.DX, xo + g * n, dx[g]);
         E::store(p.dx0, io + g * n, raw_dh ? dx[g] : dx[g] + q_dx0[nt][g] * (1.f - m));
       }
       dyw = (p.op_flags & kOpNoCarry) ? 0.f : dyw * (1.f - m);
@@ -243,7 +245,7 @@ __global__ void k_bwd_gemm_dy_generic(Lstm2BwdParams p, long long t) {
   const int n = p.n, n4 = 4 * n;
   const long long b = idx / n, k = idx % n;
   float acc = p.dyw[idx];
-  const size_t xo = ((size_t)t * p.B + b) * n4, wo = (size_t)k * n4;
+  const size_t xo = ((size_t)t * p.B + b) * p.ldDX, wo = (size_t)k * n4;
   for (int j = 0; j < n4; ++j) acc += E::load(p.DX, xo + j) * E::load(p.W, wo + j);
   p.dyw[idx] = acc;
 }
@@ -384,6 +386,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   const int rows = min(q.Bg, p.B - b_base);
   const long long bn = (long long)p.B * n;
   const unsigned frame_bytes = (unsigned)((size_t)p.B * n4 * ES);
+  const unsigned dx_frame_bytes = (unsigned)((size_t)p.B * p.ldDX * ES);
   // the exchange ring of this group: kExRing frames of [4n/KM][4][Bp][16 bytes]
   const int Bp = q.Bp;
   const unsigned ex_frame = (unsigned)((size_t)n4 * Bp * ES), frag_stride = (unsigned)(64 * Bp);
@@ -431,7 +434,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   auto tile_of = [&](int j) { return SPLIT ? set + TS * (2 * j + upper) : set + TS * j; };
   const int b = b_base + ((bl < rows) ? bl : 0);
   bool act[PT];  // the pair exists: the tile does, and the group has the row
-  long long idx[PT], io[PT];
+  long long idx[PT], io[PT], dyo[PT];
   float dyw[PT], dc[PT], dx0[PT][4];
 #pragma unroll
   for (int j = 0; j < PT; ++j) {
@@ -440,6 +443,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     const int k = k0 + 16 * ((mt < MT) ? mt : 0) + kl;
     idx[j] = (long long)b * n + k;
     io[j] = (long long)b * n4 + k;
+    dyo[j] = (long long)b * p.ldDY + k;
     dyw[j] = 0.f;
     dc[j] = act[j] ? q.Dd[idx[j]] : 0.f;
 #pragma unroll
@@ -477,7 +481,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       const long long fo = t * bn * 4 + io[j];
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) nx_gate[j][gq] = ((const RawT*)p.H)[fo + (long long)gq * n];
-      nx_dy[j] = ((const RawT*)p.DY)[t * bn + idx[j]];
+      nx_dy[j] = ((const RawT*)p.DY)[t * p.B * p.ldDY + dyo[j]];
       nx_pc[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_c, (unsigned)(idx[j] * 4), 0, 0);
       if constexpr (ES == 2)
         nx_ph[j] = __builtin_amdgcn_raw_buffer_load_b16(rs_ph, (unsigned)(io[j] * ES), 0, 0);
@@ -718,14 +722,14 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     {
       __amdgpu_buffer_rsrc_t rs_out = __builtin_amdgcn_make_buffer_rsrc(ex_base + (size_t)(f & (kExRing - 1)) * ex_frame, 0, ex_frame, kBufFlags);
       __amdgpu_buffer_rsrc_t rs_arm = __builtin_amdgcn_make_buffer_rsrc(ex_base + (size_t)((f + 2) & (kExRing - 1)) * ex_frame, 0, ex_frame, kBufFlags);
-      __amdgpu_buffer_rsrc_t rs_dx = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * frame_bytes, 0, frame_bytes, kBufFlags);
+      __amdgpu_buffer_rsrc_t rs_dx = __builtin_amdgcn_make_buffer_rsrc((unsigned char*)p.DX + (size_t)t * dx_frame_bytes, 0, dx_frame_bytes, kBufFlags);
       for (int c = tid; c < pieces; c += 64 * WV) {
         const int row = c & (Bp - 1), cg = c >> bp_shift;  // cg = gate * KGW + piece
         const int gate = cg / KGW, piece = cg - gate * KGW;
         if (row < rows) {
           const u32x4 v = __builtin_bit_cast(u32x4, stage[c]);
           const unsigned eo = (unsigned)(((((gate * n + k0) / KE + piece) << bp_shift) + row) * 16);
-          const unsigned dxo = (unsigned)(((size_t)(b_base + row) * n4 + (size_t)gate * n + k0 + piece * KE) * ES);
+          const unsigned dxo = (unsigned)(((size_t)(b_base + row) * p.ldDX + (size_t)gate * n + k0 + piece * KE) * ES);
           if (local) {
             __builtin_amdgcn_raw_buffer_store_b128(v, rs_out, eo, 0, 0);
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, ones), rs_arm, eo, 0, 0);
@@ -767,16 +771,22 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   }
 }
 
-// Frames the forward pass did not visit: DX = 0 (they still hold the all-ones fill of the persistent kernel).
+// Frames the forward pass did not visit: DX = 0.  Rows of row_words 32-bit words, pitch_words apart, rows_per_frame
+// rows to a frame; nothing between the rows is touched.
 template <typename AT>
-__global__ void k_bwd_zero_unvisited(void* DX, long long T, long long frame_words, long long first, long long step, long long nframes) {
+__global__ void k_bwd_zero_unvisited(void* DX, long long T, long long rows_per_frame, long long row_words, long long pitch_words,
+                                     long long first, long long step, long long nframes) {
   const long long lo = step > 0 ? first : first + (nframes - 1) * step;
   const long long astep = step > 0 ? step : -step;
   unsigned* w = (unsigned*)DX;
+  const long long frame_words = rows_per_frame * row_words;
   for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < T * frame_words; i += (long long)gridDim.x * blockDim.x) {
     const long long t = i / frame_words;
     const bool visited = t >= lo && t <= lo + (nframes - 1) * astep && ((t - lo) % astep) == 0;
-    if (!visited) w[i] = 0u;
+    if (!visited) {
+      const long long r = i / row_words, c = i - r * row_words;
+      w[r * pitch_words + c] = 0u;
+    }
   }
 }
 

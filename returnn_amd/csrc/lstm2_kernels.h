@@ -130,6 +130,7 @@ __global__ void k_copy_f32(const float* __restrict__ src, float* __restrict__ ds
 template <typename AT>
 __global__ void k_fill_unvisited(Lstm2Params p) {
   const long long bn = (long long)p.B * p.n;
+  const int n4 = 4 * p.n;
   const long long per_frame = bn * 4;
   const long long total = p.T * per_frame;
   for (long long idx = blockIdx.x * (long long)blockDim.x + threadIdx.x; idx < total;
@@ -142,10 +143,11 @@ __global__ void k_fill_unvisited(Lstm2Params p) {
     else
       visited = delta <= 0 && ((-delta) % (-p.step)) == 0 && delta / p.step < p.nsteps;
     if (visited) continue;
-    ((AT*)p.H)[idx] = ((const AT*)p.X)[idx];
     const long long rem = idx - t * per_frame;
+    const long long row = t * p.B + rem / n4;  // (frame, sequence)
+    ((AT*)p.H)[idx] = ((const AT*)p.X)[row * p.ldX + rem % n4];
     if (rem < bn) {
-      Elem<AT>::store(p.Y, t * bn + rem, 0.f);
+      Elem<AT>::store(p.Y, (t * p.B + rem / p.n) * p.ldY + rem % p.n, 0.f);
       p.C[t * bn + rem] = 0.f;
     }
   }
@@ -236,23 +238,26 @@ __global__ void k_prepare_mfma_multi(Lstm2Multi multi, int n_flags) {
 // (rows_src <= rows_dst) and zeros elsewhere; ET is an unsigned integer of the element's size (bits are copied).
 template <typename ET>
 __global__ void k_pad_cells(const ET* __restrict__ src, ET* __restrict__ dst, long long rows_src, long long rows_dst, int blocks,
-                            int n, int n_pad) {
+                            int n, int n_pad, long long src_pitch) {
+  // src_pitch: elements from one row of src to the next (blocks * n when contiguous)
   const long long total = rows_dst * blocks * n_pad;
   for (long long idx = blockIdx.x * (long long)blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
     const int j = (int)(idx % n_pad);
     const long long rb = idx / n_pad;  // row * blocks + block
-    dst[idx] = (j < n && rb / blocks < rows_src) ? src[rb * n + j] : (ET)0;
+    const long long row = rb / blocks;
+    dst[idx] = (j < n && row < rows_src) ? src[row * src_pitch + (rb % blocks) * n + j] : (ET)0;
   }
 }
 
-// The inverse: dst[rows][blocks][n] from src[rows][blocks][n_pad].
+// The inverse: dst[rows][blocks][n] (rows dst_pitch elements apart) from src[rows][blocks][n_pad].
 template <typename ET>
-__global__ void k_unpad_cells(const ET* __restrict__ src, ET* __restrict__ dst, long long rows, int blocks, int n, int n_pad) {
+__global__ void k_unpad_cells(const ET* __restrict__ src, ET* __restrict__ dst, long long rows, int blocks, int n, int n_pad,
+                              long long dst_pitch) {
   const long long total = rows * blocks * n;
   for (long long idx = blockIdx.x * (long long)blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
     const int j = (int)(idx % n);
     const long long rb = idx / n;
-    dst[idx] = src[rb * n_pad + j];
+    dst[(rb / blocks) * dst_pitch + (rb % blocks) * n + j] = src[rb * n_pad + j];
   }
 }
 
@@ -261,6 +266,14 @@ __global__ void k_fill_u32(unsigned* dst, unsigned value, long long count) {
   for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < count;
        i += (long long)gridDim.x * blockDim.x)
     dst[i] = value;
+}
+
+// rows of row_words 32-bit words, pitch_words apart: := 0
+__global__ void k_clear_rows(unsigned* dst, long long rows, long long row_words, long long pitch_words) {
+  for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < rows * row_words; i += (long long)gridDim.x * blockDim.x) {
+    const long long r = i / row_words;
+    dst[r * pitch_words + (i - r * row_words)] = 0u;
+  }
 }
 
 // data[i] += bias[i % width]  (rows of `width` elements)
@@ -278,7 +291,7 @@ __global__ void k_clear_status(unsigned* status) {
 // last visited frame (in processing order) with a non-zero mask and copies that row of Y, else y0.
 template <typename AT>
 __global__ void k_last_output(const void* Y, const void* y0, const float* mask, void* out, long long T, int B, int n,
-                              int first, int step, int nsteps) {
+                              int first, int step, int nsteps, long long ldY) {
   __shared__ int s_last;
   const int b = blockIdx.x;
   if (threadIdx.x == 0) s_last = -1;
@@ -291,7 +304,7 @@ __global__ void k_last_output(const void* Y, const void* y0, const float* mask, 
   if (last >= 0) atomicMax(&s_last, last);
   __syncthreads();
   last = s_last;
-  const AT* src = (last >= 0) ? (const AT*)Y + (((long long)first + (long long)last * step) * B + b) * n
+  const AT* src = (last >= 0) ? (const AT*)Y + (((long long)first + (long long)last * step) * B + b) * ldY
                               : (const AT*)y0 + (long long)b * n;
   for (int j = threadIdx.x; j < n; j += blockDim.x) ((AT*)out)[(long long)b * n + j] = src[j];
 }
@@ -312,11 +325,12 @@ __global__ void k_step_generic(Lstm2Params p, int s) {
   const void* y_in = (s == 0) ? p.y0 : (const void*)((const AT*)p.ycarry + (size_t)(s & 1) * bn);
   void* y_out = (void*)((AT*)p.ycarry + (size_t)((s + 1) & 1) * bn);
   const float* c_in = (s == 0) ? p.c0 : p.C + (t - p.step) * bn;
-  const size_t xoff = ((size_t)t * p.B + b) * 4 * n + j;
-  float g0 = Elem<AT>::load(p.X, xoff);
-  float g1 = Elem<AT>::load(p.X, xoff + n);
-  float g2 = Elem<AT>::load(p.X, xoff + 2 * (size_t)n);
-  float g3 = Elem<AT>::load(p.X, xoff + 3 * (size_t)n);
+  const size_t xoff = ((size_t)t * p.B + b) * 4 * n + j;       // in H
+  const size_t xin = ((size_t)t * p.B + b) * (size_t)p.ldX + j;  // in X
+  float g0 = Elem<AT>::load(p.X, xin);
+  float g1 = Elem<AT>::load(p.X, xin + n);
+  float g2 = Elem<AT>::load(p.X, xin + 2 * (size_t)n);
+  float g3 = Elem<AT>::load(p.X, xin + 3 * (size_t)n);
   const size_t yrow = (size_t)b * n;
   for (int k = 0; k < n; ++k) {
     const float yk = Elem<AT>::load(y_in, yrow + k);
@@ -336,7 +350,7 @@ __global__ void k_step_generic(Lstm2Params p, int s) {
   Elem<AT>::store(p.H, xoff + 3 * (size_t)n, a3);
   p.C[t * bn + idx] = c;
   const float y = Elem<AT>::round(Act<AT>::tanh(c) * a3 * m);
-  Elem<AT>::store(p.Y, t * bn + idx, y);
+  Elem<AT>::store(p.Y, ((size_t)t * p.B + b) * (size_t)p.ldY + j, y);
   Elem<AT>::store(y_out, idx, (p.op_flags & kOpNoCarry) ? y : y + Elem<AT>::load(y_in, idx) * (1.f - m));
   if (s == p.nsteps - 1) p.d[idx] = c;
 }
@@ -475,7 +489,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
 #pragma unroll
       for (int q = 0; q < 4; ++q) xg[j][q] = 0.f;
       if (e_valid[j]) {
-        const size_t xo = ((size_t)t * p.B + (b_base + e_b[j])) * 4 * n + e_cell[j];
+        const size_t xo = ((size_t)t * p.B + (b_base + e_b[j])) * (size_t)p.ldX + e_cell[j];
 #pragma unroll
         for (int q = 0; q < 4; ++q) xg[j][q] = E::load(p.X, xo + (size_t)q * n);
         msk[j] = p.mask[t * p.B + b_base + e_b[j]];
@@ -593,7 +607,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
 #pragma unroll
         for (int q = 0; q < 4; ++q) E::store(p.H, xo + (size_t)q * n, a_out[j][q]);
         p.C[t * bn + bc] = c_state[j];
-        E::store(p.Y, t * bn + bc, y_out[j]);
+        E::store(p.Y, ((size_t)t * p.B + (b_base + e_b[j])) * (size_t)p.ldY + e_cell[j], y_out[j]);
       }
     }
   }
@@ -607,7 +621,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
       if (e_valid[j]) {
         const long long bc = (long long)(b_base + e_b[j]) * n + e_cell[j];
         p.d[bc] = expired ? __builtin_nanf("") : c_state[j];
-        if (expired) E::store(p.Y, t_last * bn + bc, __builtin_nanf(""));
+        if (expired) E::store(p.Y, ((size_t)t_last * p.B + (b_base + e_b[j])) * (size_t)p.ldY + e_cell[j], __builtin_nanf(""));
       }
     }
   }
@@ -646,7 +660,9 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_mfma(const Lstm2Params p, 
 // ---------------------------------------------------------------------------------------------
 constexpr int kExDevice = 0;  // device-scope loads and stores: always valid
 constexpr int kExLocal = 1;   // the whole group on one XCD: plain stores into that XCD's L2, loads that bypass the first-level cache
-constexpr int kExNoWait = 3;  // measurement aid: never wait for the other workgroups (results are WRONG; status is set to 2)
+// measurement aid: a step without the exchange's reads -- no loads of the hidden state (the MFMAs run on zeros), no delay,
+// no waiting; the new values are still stored (plain stores).  Results are WRONG; status is set to 2.
+constexpr int kExNoWait = 3;
 
 template <typename AT>
 struct Sentinel;
@@ -902,13 +918,15 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   typedef Chunk<CHY> YC;
   typedef Chunk<16> CC;
   const int cell0 = CELLS * r;
-  unsigned xoff[XCH], yoff[YCH], coff[CCH];  // byte offsets inside one frame (kOobOffset: nothing to move)
+  unsigned xoff[XCH], hoff[XCH], yoff[YCH], coff[CCH];  // byte offsets inside one frame (kOobOffset: nothing to move); the rows of
+                                                        // X and Y may lie further apart than those of H and C (ldX, ldY)
   unsigned xlds[XCH], ylds[YCH], clds[CCH];  // byte offsets inside one LDS copy
 #pragma unroll
   for (int i = 0; i < XCH; ++i) {
     const int c = tid + kWgThreads * i;
     const int row = c / (4 * CPS), gate = (c / CPS) % 4, part = c % CPS;
-    xoff[i] = row < rows ? (unsigned)((((b_base + row) * 4 * n) + gate * n + cell0) * ES + part * CH) : kOobOffset;
+    xoff[i] = row < rows ? (unsigned)(((long long)(b_base + row) * p.ldX + gate * n + cell0) * ES + part * CH) : kOobOffset;
+    hoff[i] = row < rows ? (unsigned)((((b_base + row) * 4 * n) + gate * n + cell0) * ES + part * CH) : kOobOffset;
     // threads beyond the tile write to / read from the spare slot at the end of the copy
     xlds[i] = row < ROWS ? (unsigned)(row * L.x_row + gate * SEG + part * CH) : (unsigned)(ROWS * L.x_row);
   }
@@ -916,7 +934,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   for (int i = 0; i < YCH; ++i) {
     const int c = tid + kWgThreads * i;
     const int row = c / (SEG / CHY), part = c % (SEG / CHY);
-    yoff[i] = row < rows ? (unsigned)(((b_base + row) * n + cell0) * ES + part * CHY) : kOobOffset;
+    yoff[i] = row < rows ? (unsigned)(((long long)(b_base + row) * p.ldY + cell0) * ES + part * CHY) : kOobOffset;
     ylds[i] = (unsigned)(min(row, ROWS - 1) * L.y_row + part * CHY);
   }
 #pragma unroll
@@ -927,12 +945,12 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     clds[i] = (unsigned)(min(row, ROWS - 1) * L.c_row + part * 16);
   }
   const unsigned moff = tid < rows ? (unsigned)((b_base + tid) * 4) : kOobOffset;
-  const unsigned frame_x = (unsigned)((size_t)p.B * 4 * n * ES), frame_y = (unsigned)(bn * ES),
-                 frame_c = (unsigned)(bn * 4), frame_m = (unsigned)(p.B * 4);
+  const unsigned frame_x = (unsigned)((size_t)p.B * p.ldX * ES), frame_h = (unsigned)((size_t)p.B * 4 * n * ES),
+                 frame_y = (unsigned)((size_t)p.B * p.ldY * ES), frame_c = (unsigned)(bn * 4), frame_m = (unsigned)(p.B * 4);
   typename XC::T xv[2][XCH];
   float mv[2] = {0.f, 0.f};
   // Frame pointers advance by a constant per step (signed: the op may run backwards in time).
-  const long long step_x = (long long)p.step * frame_x, step_y = (long long)p.step * frame_y,
+  const long long step_x = (long long)p.step * frame_x, step_h = (long long)p.step * frame_h, step_y = (long long)p.step * frame_y,
                   step_c = (long long)p.step * frame_c, step_m = (long long)p.step * frame_m;
   auto fetch_x_at = [&](const unsigned char* xp, bool enabled, auto par_tag) {  // loads of one frame of X into register set PAR
     constexpr int PAR = decltype(par_tag)::value;
@@ -979,9 +997,9 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   };
   auto flush_read = [&](int copy) { flush_read_at(L.hs + copy * L.x_copy, L.ys + copy * L.y_copy, L.cs + copy * L.c_copy); };
   auto flush_write_h = [&](unsigned char* hp, bool enabled) {
-    __amdgpu_buffer_rsrc_t hr = __builtin_amdgcn_make_buffer_rsrc((void*)hp, 0, enabled ? frame_x : 0u, kBufFlags);
+    __amdgpu_buffer_rsrc_t hr = __builtin_amdgcn_make_buffer_rsrc((void*)hp, 0, enabled ? frame_h : 0u, kBufFlags);
 #pragma unroll
-    for (int i = 0; i < XCH; ++i) XC::store(fh[i], hr, xoff[i]);
+    for (int i = 0; i < XCH; ++i) XC::store(fh[i], hr, hoff[i]);
   };
   auto flush_write_y = [&](unsigned char* yp, bool enabled) {
     __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc((void*)yp, 0, enabled ? frame_y : 0u, kBufFlags);
@@ -1000,7 +1018,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
   };
   auto flush_write = [&](int s) {
     const long long t = frame_of(p, s);
-    flush_write_at((unsigned char*)p.H + (size_t)t * frame_x, (unsigned char*)p.Y + (size_t)t * frame_y, (unsigned char*)p.C + (size_t)t * frame_c, true);
+    flush_write_at((unsigned char*)p.H + (size_t)t * frame_h, (unsigned char*)p.Y + (size_t)t * frame_y, (unsigned char*)p.C + (size_t)t * frame_c, true);
   };
 
   // ---- the recurrence
@@ -1095,7 +1113,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     constexpr int EX = decltype(ex_tag)::value;
     // Exchange loads always bypass the first-level cache (device scope).  Stores: through to memory (device scope), or,
     // when the whole group shares an XCD, plain stores that stay in that XCD's L2, where the loads find them.
-    constexpr int AUXS = (EX == kExLocal) ? 0 : kAuxDevice, AUXL = kAuxDevice;
+    constexpr int AUXS = (EX == kExDevice) ? kAuxDevice : 0, AUXL = kAuxDevice;
     i32x4 bf[KSMAX][NT];
 #pragma unroll
     for (int ks = 0; ks < KSMAX; ++ks)
@@ -1107,6 +1125,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     auto issue = [&](int s) {
       const unsigned soff = (unsigned)(s & (kHxRing - 1)) * hx_buf_bytes;
       asm volatile("" ::: "memory");  // other workgroups write this memory: really load again
+      if constexpr (EX == kExNoWait) return;
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
         if ((PAIRED ? (jl & 7) : 16 * nt + jl) < rows) {
@@ -1151,7 +1170,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     // in units of s_sleep(1), about 64 clocks; see below.  (A group that was planned for one XCD and found itself on
     // several takes the numbers of a spread plan.)
     const bool spread_after_all = multi.local && EX == kExDevice;
-    int delay = spread_after_all ? 20 : p.poll_delay;
+    int delay = EX == kExNoWait ? 0 : spread_after_all ? 20 : p.poll_delay;
     const int delay_inc = spread_after_all ? 2 : p.delay_inc;
     // One time step; PAR = s & 1 selects the register sets and the LDS copies of X, `stage` = s % 3 the copy that
     // takes this step's outputs.
@@ -1281,7 +1300,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
           for (int u = 0; u < NACC; ++u) {
             acc[u][0] = E::mma(wreg[2 * u + odd][ks], opnd, acc[u][0]);
             __builtin_amdgcn_sched_group_barrier(0x008, sizeof(AT) == 2 ? 1 : 4, 0);  // the MFMA(s) of one fragment ...
-            __builtin_amdgcn_sched_group_barrier(0x096, 3, 0);                        // ... then up to three of the rest
+            __builtin_amdgcn_sched_group_barrier(0x096, 3, 0);                        // ... then up to three of the rest (four or five: 2-3 % slower)
           }
           __builtin_amdgcn_sched_barrier(0);
           opnd = opnd_next;
@@ -1304,7 +1323,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
               __builtin_amdgcn_sched_group_barrier(0x096, 3, 0);                        // ... then up to three of the rest (VALU, SALU, VMEM, LDS)
             }
       }
-      h_out += step_x; y_out_p += step_y; c_out += step_c; x_next += step_x; m_next += step_m;
+      h_out += step_h; y_out_p += step_y; c_out += step_c; x_next += step_x; m_next += step_m;
       if constexpr (PAIRED) {
 #pragma unroll
         for (int u = 0; u < NACC; ++u) redbuf[wave][u][lane] = acc[u][0];
@@ -1394,7 +1413,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
     issue(0);
     int stage = 0;
     // frames of the outputs of step s-2 and of the inputs of step s+4, as the loop reaches step s
-    h_out = (unsigned char*)p.H + (frame_of(p, 0) - 2 * (long long)p.step) * (long long)frame_x;
+    h_out = (unsigned char*)p.H + (frame_of(p, 0) - 2 * (long long)p.step) * (long long)frame_h;
     y_out_p = (unsigned char*)p.Y + (frame_of(p, 0) - 2 * (long long)p.step) * (long long)frame_y;
     c_out = (unsigned char*)p.C + (frame_of(p, 0) - 2 * (long long)p.step) * (long long)frame_c;
     x_next = (const unsigned char*)p.X + frame_of(p, 4) * (long long)frame_x;

@@ -46,6 +46,9 @@ struct Lstm2Params {
   void* ycarry;      // [2][B][n] AT: hidden-state carry of the generic per-step kernels
   // sizes
   long long T;
+  long long ldX;  // elements between the rows of X of two consecutive (frame, sequence) pairs: 4n when X is contiguous; more when
+                  // the caller's rows are wider (e.g. [T*B, 8n]: the pre-projected gates of two directions side by side)
+  long long ldY;  // the same for the rows of Y: n when contiguous (2n: the two directions of a layer write into one [T,B,2n] array)
   int B, n;
   int first;   // first visited frame
   int step;    // signed stride between visited frames

@@ -982,28 +982,59 @@ BwdPadLayout bwd_pad_layout(int64_t T, int B, int np, int dtype) {
 }
 
 // dst[rows_dst][blocks][np] := src[rows_src][blocks][n], zeros elsewhere; elements of `es` bytes.
-int launch_pad(const void* src, void* dst, long long rows_src, long long rows_dst, int blocks, int n, int np, size_t es, hipStream_t stream) {
+int launch_pad(const void* src, void* dst, long long rows_src, long long rows_dst, int blocks, int n, int np, size_t es, hipStream_t stream,
+               long long src_pitch = 0) {
   const long long total = rows_dst * blocks * np;
   if (total <= 0) return RTN_OK;
+  if (src_pitch == 0) src_pitch = (long long)blocks * n;
   const dim3 grid((unsigned)std::min<long long>((total + 255) / 256, 8192)), block(256);
   if (es == 2)
-    hipLaunchKernelGGL(k_pad_cells<unsigned short>, grid, block, 0, stream, (const unsigned short*)src, (unsigned short*)dst, rows_src, rows_dst, blocks, n, np);
+    hipLaunchKernelGGL(k_pad_cells<unsigned short>, grid, block, 0, stream, (const unsigned short*)src, (unsigned short*)dst, rows_src, rows_dst, blocks, n, np, src_pitch);
   else
-    hipLaunchKernelGGL(k_pad_cells<unsigned>, grid, block, 0, stream, (const unsigned*)src, (unsigned*)dst, rows_src, rows_dst, blocks, n, np);
+    hipLaunchKernelGGL(k_pad_cells<unsigned>, grid, block, 0, stream, (const unsigned*)src, (unsigned*)dst, rows_src, rows_dst, blocks, n, np, src_pitch);
   RTN_HIP(hipGetLastError());
   return RTN_OK;
 }
 
-// dst[rows][blocks][n] := src[rows][blocks][np].
-int launch_unpad(const void* src, void* dst, long long rows, int blocks, int n, int np, size_t es, hipStream_t stream) {
+// dst[rows][blocks][n] := src[rows][blocks][np]; dst_pitch: elements from one row of dst to the next (0: blocks * n).
+int launch_unpad(const void* src, void* dst, long long rows, int blocks, int n, int np, size_t es, hipStream_t stream, long long dst_pitch = 0) {
   const long long total = rows * blocks * n;
   if (total <= 0) return RTN_OK;
+  if (dst_pitch == 0) dst_pitch = (long long)blocks * n;
   const dim3 grid((unsigned)std::min<long long>((total + 255) / 256, 8192)), block(256);
   if (es == 2)
-    hipLaunchKernelGGL(k_unpad_cells<unsigned short>, grid, block, 0, stream, (const unsigned short*)src, (unsigned short*)dst, rows, blocks, n, np);
+    hipLaunchKernelGGL(k_unpad_cells<unsigned short>, grid, block, 0, stream, (const unsigned short*)src, (unsigned short*)dst, rows, blocks, n, np, dst_pitch);
   else
-    hipLaunchKernelGGL(k_unpad_cells<unsigned>, grid, block, 0, stream, (const unsigned*)src, (unsigned*)dst, rows, blocks, n, np);
+    hipLaunchKernelGGL(k_unpad_cells<unsigned>, grid, block, 0, stream, (const unsigned*)src, (unsigned*)dst, rows, blocks, n, np, dst_pitch);
   RTN_HIP(hipGetLastError());
+  return RTN_OK;
+}
+
+// rows x row_elems elements := 0, rows pitch elements apart (row_elems * es a multiple of 4)
+int launch_clear_rows(void* dst, long long rows, long long row_elems, long long pitch, size_t es, hipStream_t stream) {
+  if (rows <= 0 || row_elems <= 0) return RTN_OK;
+  if (pitch == row_elems) {
+    hipLaunchKernelGGL(k_fill_u32, dim3(1024), dim3(256), 0, stream, (unsigned*)dst, 0u, (long long)((size_t)rows * row_elems * es / 4));
+  } else {
+    hipLaunchKernelGGL(k_clear_rows, dim3(1024), dim3(256), 0, stream, (unsigned*)dst, rows, (long long)((size_t)row_elems * es / 4),
+                       (long long)((size_t)pitch * es / 4));
+  }
+  RTN_HIP(hipGetLastError());
+  return RTN_OK;
+}
+
+// Row pitch of a call's array: what the caller gave, or the contiguous one; checked against what the kernels assume
+// (rows do not overlap, stay 16-byte aligned, and a frame stays within the 32-bit offsets of a buffer descriptor).
+int resolve_pitch(const char* name, long long given, long long contiguous, int B, size_t es, long long* out) {
+  const long long ld = given ? given : contiguous;
+  if (ld < contiguous) return fail(RTN_ERR_ARG, "NativeLstm2: row pitch %s=%lld is below the row length %lld", name, ld, contiguous);
+  if (ld != contiguous && ((size_t)ld * es) % 4 != 0) return fail(RTN_ERR_ARG, "NativeLstm2: row pitch %s=%lld must keep rows 4-byte aligned", name, ld);
+  // (widths whose contiguous rows are not 16-byte aligned run on element-wise kernels or on padded copies)
+  if (((size_t)contiguous * es) % 16 == 0 && ((size_t)ld * es) % 16 != 0)
+    return fail(RTN_ERR_ARG, "NativeLstm2: row pitch %s=%lld must keep rows 16-byte aligned", name, ld);
+  if ((unsigned long long)B * (unsigned long long)ld * es >= 0xFFFFFF00ull)
+    return fail(RTN_ERR_SHAPE, "NativeLstm2: a frame of %d rows with pitch %s=%lld exceeds 4 GiB", B, name, ld);
+  *out = ld;
   return RTN_OK;
 }
 
@@ -1121,19 +1152,22 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     for (int k = 0; k < count; ++k) {
       const rtn_lstm2_call& c = calls[k];
       unsigned char* base = (unsigned char*)workspace + (size_t)k * each + inner_each;
-      if ((rc = launch_pad(c.X, base + L.X, tb, tb, 4, n, np, es, stream)) != RTN_OK) return rc;
+      long long ldX = 0, ldY = 0;
+      if ((rc = resolve_pitch("ldX", c.ldX, 4LL * n, B, es, &ldX)) != RTN_OK) return rc;
+      if ((rc = resolve_pitch("ldY", c.ldY, n, B, es, &ldY)) != RTN_OK) return rc;
+      if ((rc = launch_pad(c.X, base + L.X, tb, tb, 4, n, np, es, stream, ldX)) != RTN_OK) return rc;
       if ((rc = launch_pad(c.W, base + L.W, n, np, 4, n, np, es, stream)) != RTN_OK) return rc;
       if ((rc = launch_pad(c.y0, base + L.y0, B, B, 1, n, np, es, stream)) != RTN_OK) return rc;
       if ((rc = launch_pad(c.c0, base + L.c0, B, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
       padded[(size_t)k] = {base + L.X, base + L.W, base + L.y0, (const float*)(base + L.c0), c.i, c.start, c.step,
-                           base + L.Y, (float*)(base + L.C), base + L.H, (float*)(base + L.d)};
+                           base + L.Y, (float*)(base + L.C), base + L.H, (float*)(base + L.d), 0, 0};
     }
     rc = fwd_calls(padded.data(), count, T, B, np, dtype, mode, workspace, need, hip_stream, op_flags, each, no_graph);
     if (rc != RTN_OK) return rc;
     for (int k = 0; k < count; ++k) {
       const rtn_lstm2_call& c = calls[k];
       const rtn_lstm2_call& q = padded[(size_t)k];
-      if ((rc = launch_unpad(q.Y, c.Y, tb, 1, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_unpad(q.Y, c.Y, tb, 1, n, np, es, stream, c.ldY)) != RTN_OK) return rc;
       if ((rc = launch_unpad(q.C, c.C, tb, 1, n, np, 4, stream)) != RTN_OK) return rc;
       if ((rc = launch_unpad(q.H, c.H, tb, 4, n, np, es, stream)) != RTN_OK) return rc;
       if ((rc = launch_unpad(q.d, c.d, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
@@ -1225,6 +1259,8 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     p.ycarry = ws + pl.off_ycarry;
     p.trace = pl.off_trace ? (unsigned long long*)(ws + pl.off_trace) : nullptr;
     p.T = T; p.B = B; p.n = n;
+    if ((rc = resolve_pitch("ldX", c.ldX, 4LL * n, B, esize(dtype), &p.ldX)) != RTN_OK) return rc;
+    if ((rc = resolve_pitch("ldY", c.ldY, n, B, esize(dtype), &p.ldY)) != RTN_OK) return rc;
     // returnn/native_op.py:1253-1259
     if (c.step > 0) {
       p.first = c.start;
@@ -1404,14 +1440,18 @@ int blas_handle(rocblas_handle* out) {
 }
 
 // DW[n,4n] (row major, float32) += A[rows,n]^T * Bm[rows,4n] with A, Bm of element type `dtype`, row major.
-int dw_accumulate(rocblas_handle h, const void* A, const void* Bm, float* DW, long long rows, int n, int dtype) {
+int dw_accumulate(rocblas_handle h, const void* A, const void* Bm, float* DW, long long rows, int n, int dtype, long long lda = 0,
+                  long long ldb = 0) {
   if (rows <= 0) return RTN_OK;
+  if (lda == 0) lda = n;
+  if (ldb == 0) ldb = 4LL * n;
   const float alpha = 1.f, beta = 1.f;
   const rocblas_datatype in = dtype == RTN_DTYPE_BF16 ? rocblas_datatype_bf16_r : rocblas_datatype_f32_r;
   // Row-major DW[n,4n] is column-major [4n,n]: DW^T = Bm^T * A, with row-major Bm[rows,4n] = column-major [4n,rows]
-  // (no transpose) and row-major A[rows,n] = column-major [n,rows] (transpose).
+  // (no transpose) and row-major A[rows,n] = column-major [n,rows] (transpose).  lda, ldb: row pitch of A and Bm in
+  // elements (0: contiguous).
   const rocblas_status st = rocblas_gemm_ex(h, rocblas_operation_none, rocblas_operation_transpose, 4 * n, n, (rocblas_int)rows,
-                                            &alpha, Bm, in, 4 * n, A, in, n, &beta, DW, rocblas_datatype_f32_r, 4 * n, DW,
+                                            &alpha, Bm, in, (rocblas_int)ldb, A, in, (rocblas_int)lda, &beta, DW, rocblas_datatype_f32_r, 4 * n, DW,
                                             rocblas_datatype_f32_r, 4 * n, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
   if (st != rocblas_status_success) return fail(RTN_ERR_HIP, "NativeLstm2: rocblas_gemm_ex failed with status %d", (int)st);
   return RTN_OK;
@@ -1498,14 +1538,10 @@ int mfma_probe(bool issue_only, int32_t count, int64_t T, int32_t B, int32_t n, 
   SeqKernel k;
   int threads = kWgThreads;
   if (issue_only && env_long("RTN_LSTM2_PROBE_WAVES", 4) == 8 && dtype == RTN_DTYPE_BF16 && pl.MT == 8 && pl.NT == 1 && pl.KSMAX == 8) {
-    // experiment: the same MFMAs dealt to two wavefronts per SIMD (8 per workgroup, half the macro steps each)
+    // measurement variant: the same MFMAs dealt to two wavefronts per SIMD (eight per workgroup, 32 MFMAs each) -- what
+    // the matrix cores do when a second wavefront fills the gaps one wavefront leaves between its MFMAs
     k = &k_mfma_issue<__bf16, 8, 1, 4, 512>;
     threads = 512;
-  } else if (issue_only && env_long("RTN_LSTM2_PROBE_WAVES", 4) == 44 && dtype == RTN_DTYPE_BF16) {
-    k = &k_mfma_issue<__bf16, 8, 1, 4, 256>;  // experiment: half the MFMAs, all operands in architectural registers
-  } else if (issue_only && env_long("RTN_LSTM2_PROBE_WAVES", 4) == 16 && dtype == RTN_DTYPE_BF16) {
-    k = &k_mfma_issue<__bf16, 8, 1, 2, 1024>;  // experiment: four wavefronts per SIMD
-    threads = 1024;
   } else if (issue_only)
     k = dtype == RTN_DTYPE_BF16 ? issue_kernel_for<__bf16>(pl.MT, pl.NT, pl.KSMAX) : issue_kernel_for<float>(pl.MT, pl.NT, pl.KSMAX);
   else
@@ -1817,6 +1853,7 @@ struct BwdJob {
   Lstm2BwdParams p;
   unsigned char* ws;
   long long abs_step, num_steps, first, end;
+  long long ldY;  // row pitch of Y in elements
 };
 
 // `count` gradient calls of one shape.  With the persistent kernel and count <= kMaxBwdMulti all of them share one
@@ -1895,22 +1932,27 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       if ((rc = launch_pad(c.W, base + L.W, n, np, 4, n, np, es, stream)) != RTN_OK) return rc;
       if ((rc = launch_pad(c.y0, base + L.y0, B, B, 1, n, np, es, stream)) != RTN_OK) return rc;
       if ((rc = launch_pad(c.c0, base + L.c0, B, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
-      if ((rc = launch_pad(c.Y, base + L.Y, tb, tb, 1, n, np, es, stream)) != RTN_OK) return rc;
+      long long ldY = 0, ldDY = 0, ldDX = 0;
+      if ((rc = resolve_pitch("ldY", c.ldY, n, B, es, &ldY)) != RTN_OK) return rc;
+      if ((rc = resolve_pitch("ldDY", c.ldDY, n, B, es, &ldDY)) != RTN_OK) return rc;
+      if ((rc = resolve_pitch("ldDX", c.ldDX, 4LL * n, B, es, &ldDX)) != RTN_OK) return rc;
+      if ((rc = launch_pad(c.Y, base + L.Y, tb, tb, 1, n, np, es, stream, ldY)) != RTN_OK) return rc;
       // the sibling op that keeps its cell states in H hands H in for C as well; it is not read then
       if (!(op_flags & kOpH0IsCell) && (rc = launch_pad(c.C, base + L.C, tb, tb, 1, n, np, 4, stream)) != RTN_OK) return rc;
       if ((rc = launch_pad(c.H, base + L.H, tb, tb, 4, n, np, es, stream)) != RTN_OK) return rc;
-      if ((rc = launch_pad(c.DY, base + L.DY, tb, tb, 1, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_pad(c.DY, base + L.DY, tb, tb, 1, n, np, es, stream, ldDY)) != RTN_OK) return rc;
       if ((rc = launch_pad(c.Dd, base + L.Dd, B, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
       padded[(size_t)k] = {base + L.W, base + L.y0, (const float*)(base + L.c0), c.i, c.start, c.step, base + L.Y,
                            (const float*)(base + ((op_flags & kOpH0IsCell) ? L.H : L.C)), base + L.H, base + L.DY,
-                           (const float*)(base + L.Dd), base + L.DX, (float*)(base + L.DW), base + L.Dy0, (float*)(base + L.Dc0)};
+                           (const float*)(base + L.Dd), base + L.DX, (float*)(base + L.DW), base + L.Dy0, (float*)(base + L.Dc0),
+                           0, 0, 0};
     }
     rc = bwd_calls(padded.data(), count, T, B, np, dtype, workspace, need, hip_stream, op_flags, each);
     if (rc != RTN_OK) return rc;
     for (int k = 0; k < count; ++k) {
       const rtn_lstm2_bwd_call& c = calls[k];
       const rtn_lstm2_bwd_call& q = padded[(size_t)k];
-      if ((rc = launch_unpad(q.DX, c.DX, tb, 4, n, np, es, stream)) != RTN_OK) return rc;
+      if ((rc = launch_unpad(q.DX, c.DX, tb, 4, n, np, es, stream, c.ldDX)) != RTN_OK) return rc;
       if ((rc = launch_unpad(q.DW, c.DW, n, 4, n, np, 4, stream)) != RTN_OK) return rc;
       if ((rc = launch_unpad(q.Dy0, c.Dy0, B, 1, n, np, es, stream)) != RTN_OK) return rc;
       if ((rc = launch_unpad(q.Dc0, c.Dc0, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
@@ -2091,6 +2133,9 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     p.dx0 = j.ws + lay.off_dx0;
     p.T = T; p.B = B; p.n = n;
     p.op_flags = op_flags;
+    if ((rc = resolve_pitch("ldY", c.ldY, n, B, es, &j.ldY)) != RTN_OK) return rc;
+    if ((rc = resolve_pitch("ldDY", c.ldDY, n, B, es, &p.ldDY)) != RTN_OK) return rc;
+    if ((rc = resolve_pitch("ldDX", c.ldDX, 4LL * n, B, es, &p.ldDX)) != RTN_OK) return rc;
     hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)j.ws, 0u, (long long)(lay.off_wpk / 4));
     RTN_HIP(hipGetLastError());
     // returnn/native_op.py:1383-1407: which frames are visited, and in which order
@@ -2103,7 +2148,6 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       j.num_steps = (j.first - c.start) / j.abs_step + 1;
     }
     j.end = j.first + (j.num_steps - 1) * c.step;  // inclusive
-    const long long words = (long long)((size_t)T * bn * 4 * es / 4);
     if (pk) {
       // the exchange ring starts armed: all-ones words (the visited frames of DX are written by the kernel, the others
       // zeroed behind it)
@@ -2114,9 +2158,8 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       hipLaunchKernelGGL(k_fill_u32, dim3(256), fill_block, 0, stream, (unsigned*)(j.ws + lay.off_ex), 0xFFFFFFFFu, ring_words);
       RTN_HIP(hipGetLastError());
     } else if (j.num_steps != T) {
-      // frames the loop does not visit keep DX = 0 (:1385-1388)
-      hipLaunchKernelGGL(k_fill_u32, dim3(1024), fill_block, 0, stream, (unsigned*)c.DX, 0u, words);
-      RTN_HIP(hipGetLastError());
+      // frames the loop does not visit keep DX = 0 (:1385-1388): all rows cleared here, row by row
+      if ((rc = launch_clear_rows(c.DX, (long long)T * B, 4LL * n, p.ldDX, es, stream)) != RTN_OK) return rc;
     }
   }
 
@@ -2177,13 +2220,13 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     for (int k = 0; k < count; ++k) {
       const BwdJob& j = jobs[(size_t)k];
       if (j.num_steps == T) continue;
-      const long long frame_words = (long long)((size_t)bn * 4 * es / 4);
+      const long long row_words = (long long)((size_t)n * 4 * es / 4), pitch_words = (long long)((size_t)j.p.ldDX * es / 4);
       if (dtype == RTN_DTYPE_BF16)
-        hipLaunchKernelGGL(k_bwd_zero_unvisited<__bf16>, dim3(1024), fill_block, 0, stream, calls[k].DX, (long long)T, frame_words, j.first,
-                           (long long)calls[k].step, j.num_steps);
+        hipLaunchKernelGGL(k_bwd_zero_unvisited<__bf16>, dim3(1024), fill_block, 0, stream, calls[k].DX, (long long)T, (long long)B, row_words,
+                           pitch_words, j.first, (long long)calls[k].step, j.num_steps);
       else
-        hipLaunchKernelGGL(k_bwd_zero_unvisited<float>, dim3(1024), fill_block, 0, stream, calls[k].DX, (long long)T, frame_words, j.first,
-                           (long long)calls[k].step, j.num_steps);
+        hipLaunchKernelGGL(k_bwd_zero_unvisited<float>, dim3(1024), fill_block, 0, stream, calls[k].DX, (long long)T, (long long)B, row_words,
+                           pitch_words, j.first, (long long)calls[k].step, j.num_steps);
       RTN_HIP(hipGetLastError());
     }
   } else {
@@ -2267,12 +2310,13 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
     if (j.num_steps > 1) {
       if (j.abs_step == 1) {
         const long long lo = std::min(j.first, j.end);
-        rc = dw_accumulate(blas, Yb + (size_t)(lo + std::max(0, -step)) * bn * es, DXb + (size_t)(lo + std::max(0, step)) * bn * 4 * es,
-                           c.DW, (j.num_steps - 1) * B, n, dtype);
+        rc = dw_accumulate(blas, Yb + (size_t)(lo + std::max(0, -step)) * B * j.ldY * es,
+                           DXb + (size_t)(lo + std::max(0, step)) * B * j.p.ldDX * es, c.DW, (j.num_steps - 1) * B, n, dtype, j.ldY, j.p.ldDX);
         if (rc != RTN_OK) return rc;
       } else {
         for (long long t = j.end - step; step > 0 ? t >= j.first : t <= j.first; t -= step) {
-          rc = dw_accumulate(blas, Yb + (size_t)t * bn * es, DXb + (size_t)(t + step) * bn * 4 * es, c.DW, B, n, dtype);
+          rc = dw_accumulate(blas, Yb + (size_t)t * B * j.ldY * es, DXb + (size_t)(t + step) * B * j.p.ldDX * es, c.DW, B, n, dtype, j.ldY,
+                             j.p.ldDX);
           if (rc != RTN_OK) return rc;
         }
       }
@@ -2522,12 +2566,14 @@ int rtn_native_lstm2_fwd_status(const void* workspace, void* hip_stream) {
 }
 
 int rtn_native_lstm2_last_output(const void* Y, const void* y0, const float* i, int32_t start, int32_t step, void* out,
-                                 int64_t T, int32_t B, int32_t n, int32_t dtype, void* hip_stream) {
+                                 int64_t T, int32_t B, int32_t n, int32_t dtype, int64_t ldY, void* hip_stream) {
   g_last_error.clear();
   int rc = check_dims(T, B, n, dtype);
   if (rc != RTN_OK) return rc;
   if ((long long)B * n == 0) return RTN_OK;
   if (!y0 || !out) return fail(RTN_ERR_ARG, "NativeLstm2: y0 and out must not be null");
+  if (ldY != 0 && ldY < n) return fail(RTN_ERR_ARG, "NativeLstm2: row pitch ldY=%lld is below the row length %d", (long long)ldY, n);
+  const long long ld = ldY ? ldY : n;
   int first = 0, nsteps = 0;
   if (T > 0) {
     if (start < 0 || start >= T) return fail(RTN_ERR_RANGE, "NativeLstm2: need 0 <= start < T, got start=%d, T=%lld", start, (long long)T);
@@ -2543,9 +2589,9 @@ int rtn_native_lstm2_last_output(const void* Y, const void* y0, const float* i, 
   }
   hipStream_t stream = (hipStream_t)hip_stream;
   if (dtype == RTN_DTYPE_BF16)
-    hipLaunchKernelGGL(k_last_output<__bf16>, dim3(B), dim3(256), 0, stream, Y, y0, i, out, (long long)T, B, n, first, step, nsteps);
+    hipLaunchKernelGGL(k_last_output<__bf16>, dim3(B), dim3(256), 0, stream, Y, y0, i, out, (long long)T, B, n, first, step, nsteps, ld);
   else
-    hipLaunchKernelGGL(k_last_output<float>, dim3(B), dim3(256), 0, stream, Y, y0, i, out, (long long)T, B, n, first, step, nsteps);
+    hipLaunchKernelGGL(k_last_output<float>, dim3(B), dim3(256), 0, stream, Y, y0, i, out, (long long)T, B, n, first, step, nsteps, ld);
   RTN_HIP(hipGetLastError());
   return RTN_OK;
 }

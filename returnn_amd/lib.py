@@ -87,6 +87,8 @@ class Lstm2Call(ctypes.Structure):
         ("C", ctypes.c_void_p),
         ("H", ctypes.c_void_p),
         ("d", ctypes.c_void_p),
+        ("ldX", ctypes.c_int64),  # row pitch of X in elements, 0 = contiguous (4n)
+        ("ldY", ctypes.c_int64),  # row pitch of Y in elements, 0 = contiguous (n)
     ]
 
 
@@ -109,6 +111,9 @@ class Lstm2BwdCall(ctypes.Structure):
         ("DW", ctypes.c_void_p),
         ("Dy0", ctypes.c_void_p),
         ("Dc0", ctypes.c_void_p),
+        ("ldY", ctypes.c_int64),  # row pitch of Y in elements, 0 = contiguous (n)
+        ("ldDY", ctypes.c_int64),  # row pitch of DY in elements, 0 = contiguous (n)
+        ("ldDX", ctypes.c_int64),  # row pitch of DX in elements, 0 = contiguous (4n)
     ]
 
 
@@ -198,7 +203,7 @@ def load() -> ctypes.CDLL:
         lib.rtn_handover_latency_probe.restype = ctypes.c_int
         lib.rtn_handover_latency_probe.argtypes = [vp, sz, i32, vp]
         lib.rtn_native_lstm2_last_output.restype = ctypes.c_int
-        lib.rtn_native_lstm2_last_output.argtypes = [vp, vp, vp, i32, i32, vp, i64, i32, i32, i32, vp]
+        lib.rtn_native_lstm2_last_output.argtypes = [vp, vp, vp, i32, i32, vp, i64, i32, i32, i32, i64, vp]
         lib.rtn_last_error.restype = ctypes.c_char_p
         lib.rtn_last_error.argtypes = []
         lib.rtn_native_lstm2_describe_plan.restype = ctypes.c_char_p

@@ -32,7 +32,7 @@ from typing import NamedTuple, Optional, Sequence, Tuple, Union
 import torch
 
 from . import native_op
-from .torch_native_op import NativeLstm2Function, NativeLstm2PairFunction, lstm_last_output, make_op, native_lstm2_multi
+from .torch_native_op import NativeLstm2BidirFunction, NativeLstm2Function, lstm_last_output, make_op, native_lstm2_multi
 
 __all__ = ["lstm", "blstm", "prepare_weights", "LstmWeights", "LSTM", "LstmState", "BlstmEncoder", "sequence_mask_time_major"]
 
@@ -50,6 +50,16 @@ class LstmWeights(NamedTuple):
     ff: torch.Tensor  # [in, 4*out] (from prepare_weights: a transposed view of a contiguous [4*out, in] matrix)
     rec: torch.Tensor  # [out, 4*out]
     bias: Optional[torch.Tensor]  # [4*out] or None
+
+
+class BlstmWeights(NamedTuple):
+    """Weights of a bidirectional layer with ONE input projection for both directions: along the ``8*out`` axis the forward
+    direction's gates (cell-in, input, forget, output), then the backward direction's."""
+
+    ff: torch.Tensor  # [in, 8*out] (a transposed view of a contiguous [8*out, in] matrix)
+    rec_fwd: torch.Tensor  # [out, 4*out]
+    rec_bwd: torch.Tensor  # [out, 4*out]
+    bias: Optional[torch.Tensor]  # [8*out] or None
 
 
 def _to_native_gate_order(w: torch.Tensor) -> torch.Tensor:
@@ -85,6 +95,51 @@ def prepare_weights(
     rec = _to_native_gate_order(rec_weight).t().to(dtype).contiguous()
     b = None if bias is None else _to_native_gate_order(bias).to(dtype).contiguous()
     return LstmWeights(ff=ff, rec=rec, bias=b)
+
+
+def _native_gate_blocks(w: torch.Tensor):
+    i, f, g, o = w.chunk(4, dim=0)
+    return g, i, f, o
+
+
+def prepare_blstm_weights(
+    fwd: Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]],
+    bwd: Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]],
+    *,
+    dtype: Optional[torch.dtype] = None,
+) -> BlstmWeights:
+    """
+    Frontend parameters of the two directions -> one projection matrix ``[in, 8*out]`` and the two recurrent matrices in
+    the op's layout.  The eight gate blocks are gathered in a single copy (reorder and join at once).
+
+    :param fwd: ``(ff_weight [4*out,in], rec_weight [4*out,out], bias [4*out] or None)`` of the forward-in-time direction
+    :param bwd: the same of the backward-in-time direction
+    :param dtype: activation type of the run (float32 or bfloat16); default: as ``ff_weight``
+    """
+    (ff_f, rec_f, b_f), (ff_b, rec_b, b_b) = fwd, bwd
+    if ff_f.shape != ff_b.shape or rec_f.shape != rec_b.shape or (b_f is None) != (b_b is None):
+        raise ValueError("blstm: the two directions need parameters of one shape")
+    if ff_f.dim() != 2 or rec_f.dim() != 2 or ff_f.shape[0] != rec_f.shape[0] or rec_f.shape[0] != 4 * rec_f.shape[1]:
+        raise ValueError("blstm: ff_weight %s / rec_weight %s, expected [4*out,in] / [4*out,out]" % (tuple(ff_f.shape), tuple(rec_f.shape)))
+    dtype = dtype or ff_f.dtype
+    rec = [_to_native_gate_order(r).t().to(dtype).contiguous() for r in (rec_f, rec_b)]
+    ff = torch.cat(_native_gate_blocks(ff_f.to(dtype)) + _native_gate_blocks(ff_b.to(dtype)), dim=0).t()
+    bias = None
+    if b_f is not None:
+        if tuple(b_f.shape) != (rec_f.shape[0],) or tuple(b_b.shape) != (rec_b.shape[0],):
+            raise ValueError("blstm: bias must be [4*out]")
+        bias = torch.cat(_native_gate_blocks(b_f.to(dtype)) + _native_gate_blocks(b_b.to(dtype)), dim=0)
+    return BlstmWeights(ff=ff, rec_fwd=rec[0], rec_bwd=rec[1], bias=bias)
+
+
+def join_weights(fwd: LstmWeights, bwd: LstmWeights) -> BlstmWeights:
+    """Two prepared directions -> one projection (a copy of the two projection matrices; prefer
+    :func:`prepare_blstm_weights`, which gets there from the parameters in the same single copy)."""
+    if fwd.ff.shape != bwd.ff.shape or fwd.rec.shape != bwd.rec.shape or (fwd.bias is None) != (bwd.bias is None):
+        raise ValueError("blstm: weights of the two directions do not match each other")
+    ff = torch.cat((fwd.ff.t(), bwd.ff.t()), dim=0).t()
+    bias = None if fwd.bias is None else torch.cat((fwd.bias, bwd.bias), dim=0)
+    return BlstmWeights(ff=ff, rec_fwd=fwd.rec, rec_bwd=bwd.rec, bias=bias)
 
 
 def sequence_mask_time_major(lengths: torch.Tensor, *, maxlen: int) -> torch.Tensor:
@@ -197,28 +252,36 @@ def _project(source: torch.Tensor, weights: LstmWeights, act: torch.dtype) -> to
 def blstm(
     source: torch.Tensor,
     *,
-    fwd: LstmWeights,
-    bwd: LstmWeights,
+    fwd: Optional[LstmWeights] = None,
+    bwd: Optional[LstmWeights] = None,
+    weights: Optional[BlstmWeights] = None,
     state_fwd: LstmState,
     state_bwd: LstmState,
     seq_lens: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, LstmState, LstmState]:
     """
-    Forward-in-time and backward-in-time layer on the same input: two projections, then both recurrences through
-    the library's multi-call entry (one launch when the device holds both), outputs concatenated.  Same results
-    as two :func:`lstm` calls with ``direction=+1`` and ``-1``.
+    Forward-in-time and backward-in-time layer on the same input: ONE projection ``[T*B, 8*out]`` for both directions,
+    then both recurrences through the library's multi-call entry (one launch when the device holds both), each reading
+    its columns of the projection and writing its columns of the one output array in place.  Same results as two
+    :func:`lstm` calls with ``direction=+1`` and ``-1`` and a concat.
 
     :param source: [T,B,in]
+    :param weights: joint weights (:func:`prepare_blstm_weights`), or ``fwd`` and ``bwd`` prepared one by one (joined here,
+        which copies the projection matrices)
     :return: [T,B,2*out] (forward | backward), new forward state, new backward state
     """
     if source.dim() != 3:
         raise ValueError("blstm: source must be [T,B,in], got %s" % (tuple(source.shape),))
     if not source.is_cuda:
         raise RuntimeError("blstm: this build implements the LSTM for HIP (MI355X) tensors only; got a CPU tensor")
+    if weights is None:
+        if fwd is None or bwd is None:
+            raise ValueError("blstm: give weights, or fwd and bwd")
+        weights = join_weights(fwd, bwd)
     act = torch.bfloat16 if source.dtype == torch.bfloat16 else torch.float32
     T, B, in_dim = source.shape
-    n = fwd.rec.shape[0]
-    if bwd.rec.shape[0] != n or fwd.ff.shape[0] != in_dim or bwd.ff.shape[0] != in_dim:
+    n = weights.rec_fwd.shape[0]
+    if weights.rec_bwd.shape[0] != n or tuple(weights.ff.shape) != (in_dim, 8 * n):
         raise ValueError("blstm: weights do not match each other or the input")
     for st in (state_fwd, state_bwd):
         if tuple(st.h.shape) != (B, n) or tuple(st.c.shape) != (B, n):
@@ -230,24 +293,28 @@ def blstm(
             raise ValueError("blstm: seq_lens must be [B]=[%i], got %s" % (B, tuple(seq_lens.shape)))
         mask = sequence_mask_time_major(seq_lens.to(source.device), maxlen=T)
     _native_lstm2()  # registers the op and fails loudly without the library
-    Xf, Xb = _project(source, fwd, act), _project(source, bwd, act)
-    if _wants_grad(Xf, Xb, fwd.rec, bwd.rec, state_fwd.h, state_fwd.c, state_bwd.h, state_bwd.c):
+    P = _project(source, LstmWeights(ff=weights.ff, rec=weights.rec_fwd, bias=weights.bias), act)  # [T,B,8n]
+    if _wants_grad(P, weights.rec_fwd, weights.rec_bwd, state_fwd.h, state_fwd.c, state_bwd.h, state_bwd.c):
         # training: both directions in one differentiable call (forward and gradient each one library entry)
-        Yf, _, _, df, Yb, _, _, db = NativeLstm2PairFunction.apply(
-            Xf, fwd.rec, state_fwd.h, state_fwd.c, Xb, bwd.rec, state_bwd.h, state_bwd.c, mask
+        Y, df, db = NativeLstm2BidirFunction.apply(
+            P, weights.rec_fwd, state_fwd.h, state_fwd.c, weights.rec_bwd, state_bwd.h, state_bwd.c, mask
         )
-        hf = _last_output_autograd(Yf, state_fwd.h, seq_lens, 1)
-        hb = _last_output_autograd(Yb, state_bwd.h, seq_lens, -1)
-        return torch.cat((Yf, Yb), dim=-1), LstmState(h=hf, c=df), LstmState(h=hb, c=db)
-    (Yf, _, _, df), (Yb, _, _, db) = native_lstm2_multi(
-        [(Xf, fwd.rec, state_fwd.h, state_fwd.c, mask, 0, 1), (Xb, bwd.rec, state_bwd.h, state_bwd.c, mask, 0, -1)]
+        hf = _last_output_autograd(Y[:, :, :n], state_fwd.h, seq_lens, 1)
+        hb = _last_output_autograd(Y[:, :, n:], state_bwd.h, seq_lens, -1)
+        return Y, LstmState(h=hf, c=df), LstmState(h=hb, c=db)
+    ((Yf, _, _, df), (Yb, _, _, db)), Y = native_lstm2_multi(
+        [
+            (P[:, :, : 4 * n], weights.rec_fwd, state_fwd.h, state_fwd.c, mask, 0, 1),
+            (P[:, :, 4 * n :], weights.rec_bwd, state_bwd.h, state_bwd.c, mask, 0, -1),
+        ],
+        joint_output=True,
     )
     if T > 0:
         hf = lstm_last_output(Yf, state_fwd.h, mask, 0, 1)
         hb = lstm_last_output(Yb, state_bwd.h, mask, 0, -1)
     else:
         hf, hb = state_fwd.h.to(act), state_bwd.h.to(act)
-    return torch.cat((Yf, Yb), dim=-1), LstmState(h=hf, c=df), LstmState(h=hb, c=db)
+    return Y, LstmState(h=hf, c=df), LstmState(h=hb, c=db)
 
 
 class LSTM(torch.nn.Module):
@@ -333,6 +400,21 @@ class BlstmEncoder(torch.nn.Module):
             d_in = self.in_dim if layer == 0 else 2 * self.out_dim
             self.fwd.append(LSTM(d_in, self.out_dim, with_bias=with_bias, device=device, dtype=dtype))
             self.bwd.append(LSTM(d_in, self.out_dim, with_bias=with_bias, device=device, dtype=dtype))
+        self._prepared = {}  # layer -> (key, BlstmWeights)
+
+    def _weights(self, layer: int, act: torch.dtype) -> BlstmWeights:
+        """Joint weights of a layer; kept while the parameters do not change and need no gradient."""
+        f, b = self.fwd[layer], self.bwd[layer]
+        ps = [p for m in (f, b) for p in (m.ff_weight, m.rec_weight, m.bias) if p is not None]
+        args = ((f.ff_weight, f.rec_weight, f.bias), (b.ff_weight, b.rec_weight, b.bias))
+        if _wants_grad(*ps):
+            return prepare_blstm_weights(*args, dtype=act)  # differentiable, not cached
+        key = (act,) + tuple((p.data_ptr(), p._version, p.device) for p in ps)
+        hit = self._prepared.get(layer)
+        if hit is None or hit[0] != key:
+            with torch.no_grad():
+                hit = self._prepared[layer] = (key, prepare_blstm_weights(*args, dtype=act))
+        return hit[1]
 
     def reset_parameters(self, generator: Optional[torch.Generator] = None):
         for m in list(self.fwd) + list(self.bwd):
@@ -367,10 +449,10 @@ class BlstmEncoder(torch.nn.Module):
         x = source
         B = source.shape[1]
         states = []
-        for f, b in zip(self.fwd, self.bwd):
+        for layer, f in enumerate(self.fwd):
             s0 = f.default_initial_state(batch_dims=(B,), device=source.device)
             s0 = LstmState(h=s0.h.to(x.dtype), c=s0.c)
             act = torch.bfloat16 if x.dtype == torch.bfloat16 else torch.float32
-            x, sf, sb = blstm(x, fwd=f._weights(act), bwd=b._weights(act), state_fwd=s0, state_bwd=s0, seq_lens=seq_lens)
+            x, sf, sb = blstm(x, weights=self._weights(layer, act), state_fwd=s0, state_bwd=s0, seq_lens=seq_lens)
             states.append((sf, sb))
         return (x, states) if collect_states else x

@@ -352,7 +352,24 @@ def _check_ndim(t: torch.Tensor, info: Dict[str, Any]):
         raise RuntimeError("%s shape ndim is not %i, got shape %s" % (info["name"], info["ndim"], tuple(t.shape)))
 
 
-def _normalise_lstm2_args(X, W, y0, c0, i):
+def _row_pitch(t: torch.Tensor, *, itemsize: int) -> int:
+    """
+    Row pitch in elements if ``t`` ([T,B,width]) can be handed to the library as it is: unit stride along the last axis,
+    rows of consecutive (frame, sequence) pairs a constant number of elements apart, 16-byte aligned rows.  0 if not
+    (the caller then makes a contiguous copy).  A contiguous tensor gives ``width``.
+    """
+    if t.dim() != 3:
+        return 0
+    T, B, width = t.shape
+    if T * B * width == 0:
+        return width if t.is_contiguous() else 0
+    ld = t.stride(1) if B > 1 else (t.stride(0) if T > 1 else width)
+    ok = (width == 1 or t.stride(2) == 1) and ld >= width and (B == 1 or t.stride(1) == ld) and (T == 1 or t.stride(0) == B * ld)
+    ok = ok and (ld * itemsize) % 16 == 0 and t.data_ptr() % 16 == 0
+    return int(ld) if ok else 0
+
+
+def _normalise_lstm2_args(X, W, y0, c0, i, *, pitched_x: bool = False):
     """Argument handling of the generated wrapper (returnn/torch/util/native_op.py:144-193) plus the op's shape
     asserts (returnn/native_op.py:1215-1223) as hard errors.  Returns the tensors to hand to the library and (T, B, n, bf16)."""
     infos = native_op.NativeLstm2.in_info
@@ -366,7 +383,9 @@ def _normalise_lstm2_args(X, W, y0, c0, i):
     act = torch.bfloat16 if bf16 else torch.float32
     X, W, y0 = (t if t.dtype == act else t.to(act) for t in (X, W, y0))
     c0, i = (t if t.dtype == torch.float32 else t.to(torch.float32) for t in (c0, i))
-    X, W, y0, c0, i = (t if t.is_contiguous() else t.contiguous() for t in (X, W, y0, c0, i))
+    if not (pitched_x and _row_pitch(X, itemsize=X.element_size())):  # (a view with a row pitch goes to the library as it is)
+        X = X if X.is_contiguous() else X.contiguous()
+    W, y0, c0, i = (t if t.is_contiguous() else t.contiguous() for t in (W, y0, c0, i))
     T, B = i.shape
     n = y0.shape[1]
     expect = {"X": (T, B, 4 * n), "W": (n, 4 * n), "y0": (B, n), "c0": (B, n)}
@@ -486,21 +505,26 @@ def _lstm_low_mem_device_impl(X, W, b, y0, c0, i, start, step, *, mode=_lib.MODE
     return Y, C, d
 
 
-def native_lstm2_multi(calls, *, mode: Optional[str] = None):
+def native_lstm2_multi(calls, *, mode: Optional[str] = None, joint_output: bool = False):
     """
     Several independent ``NativeLstm2`` calls of one shape through one entry of the library, e.g. the forward and
     the backward direction of a bidirectional layer.  Same results as calling the op once per element; when the
     device can hold them together they run in a single launch and overlap.
 
+    ``X`` may be a view with a row pitch (e.g. ``P[:, :, 4n:8n]`` of a projection ``P [T,B,8n]`` for both directions): it is
+    handed to the library as it is, not copied.
+
     :param calls: sequence of ``(X, W, y0, c0, i, start, step)``, all with the same T, B, n and element type
     :param mode: as for :class:`OpMaker`; default "auto"
-    :return: list of ``(Y, C, H, d)``
+    :param joint_output: the calls write their outputs side by side into ONE array ``[T,B,count*n]`` (what a bidirectional
+        layer hands on, returnn/tf/layers/rec.py:1229-1270): every ``Y`` returned is a view of it
+    :return: list of ``(Y, C, H, d)``; with ``joint_output`` a pair of that list and the joint array
     """
     calls = list(calls)
     if not calls:
         return []
     lib = _lib.load()
-    norm = [_normalise_lstm2_args(*c[:5]) for c in calls]
+    norm = [_normalise_lstm2_args(*c[:5], pitched_x=True) for c in calls]
     shape = norm[0][1]
     device = norm[0][0][0].device
     for tensors, sh in norm:
@@ -518,12 +542,19 @@ def native_lstm2_multi(calls, *, mode: Optional[str] = None):
     outs = []
     with torch.cuda.device(device):
         status_watch.poll()
+        act = torch.bfloat16 if bf16 else torch.float32
+        joint = torch.empty((T, B, count * n), dtype=act, device=device) if joint_output else None
+        if joint is not None and ((n * joint.element_size()) % 16 != 0):
+            joint = None  # (columns of the calls would not be 16-byte aligned: separate arrays, joined below)
         for k, ((X, W, y0, c0, i), c) in enumerate(zip((t for t, _ in norm), calls)):
             Y, C, H, d = _alloc_lstm2_outputs(T, B, n, bf16, device)
+            if joint is not None:
+                Y = joint[:, :, k * n : (k + 1) * n]
             outs.append((Y, C, H, d))
             arr[k] = _lib.Lstm2Call(
                 X.data_ptr(), W.data_ptr(), y0.data_ptr(), c0.data_ptr(), i.data_ptr(), int(c[5]), int(c[6]),
                 Y.data_ptr(), C.data_ptr(), H.data_ptr(), d.data_ptr(),
+                0 if X.is_contiguous() else _row_pitch(X, itemsize=X.element_size()), 0 if joint is None else count * n,
             )  # fmt: skip
         ws_bytes = int(lib.rtn_native_lstm2_fwd_multi_workspace_bytes(count, T, B, n, dtype, mode_code))
         ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=device)
@@ -533,6 +564,8 @@ def native_lstm2_multi(calls, *, mode: Optional[str] = None):
         if T * B * n > 0:  # (an empty problem does not touch its workspace)
             status_watch.after_call("NativeLstm2 (%i calls)" % count, ws, count, device)
     del norm  # the normalised inputs stay alive until here; the stream-ordered allocator covers the rest
+    if joint_output:
+        return outs, (joint if joint is not None else torch.cat([o[0] for o in outs], dim=-1))
     return outs
 
 
@@ -542,7 +575,9 @@ def _normalise_grad_args(W, y0, c0, i, Y, C, H, DY, Dd):
     bf16 = Y.dtype == torch.bfloat16
     act = torch.bfloat16 if bf16 else torch.float32
     device = Y.device
-    W, y0, Y, H, DY = (t.to(act).contiguous() for t in (W, y0, Y, H, DY))
+    W, y0, H = (t.to(act).contiguous() for t in (W, y0, H))
+    # (Y and DY may be views with a row pitch, e.g. one direction's half of a [T,B,2n] array: handed over as they are)
+    Y, DY = (t if _row_pitch(t, itemsize=t.element_size()) else t.contiguous() for t in (Y.to(act), DY.to(act)))
     c0, i, C, Dd = (t.to(torch.float32).contiguous() for t in (c0, i, C, Dd))
     T, B = i.shape
     n = y0.shape[1]
@@ -575,17 +610,23 @@ def native_lstm2_grad(W, y0, c0, i, start, step, Y, C, H, DY, Dd):
     return native_lstm2_grad_multi([(W, y0, c0, i, start, step, Y, C, H, DY, Dd)])[0]
 
 
-def native_lstm2_grad_multi(calls):
+def native_lstm2_grad_multi(calls, *, joint_dx: bool = False):
     """
     Several gradient calls of one shape in one library entry (``rtn_native_lstm2_bwd_multi``): the two directions of
     a bidirectional layer share one kernel launch when the device can hold both.
 
+    ``Y`` and ``DY`` may be views with a row pitch (one direction's columns of a ``[T,B,2n]`` array): they are handed to the
+    library as they are, not copied.
+
     :param calls: list of ``(W, y0, c0, i, start, step, Y, C, H, DY, Dd)``
-    :return: list of ``(DX, DW, Dy0, Dc0)``, element k as :func:`native_lstm2_grad` gives for ``calls[k]``
+    :param joint_dx: the calls write their ``DX`` side by side into ONE array ``[T,B,count*4n]`` (the error of a projection
+        made once for all of them): every ``DX`` returned is a view of it
+    :return: list of ``(DX, DW, Dy0, Dc0)``, element k as :func:`native_lstm2_grad` gives for ``calls[k]``; with
+        ``joint_dx`` a pair of that list and the joint array
     """
     calls = list(calls)
     if not calls:
-        return []
+        return ([], None) if joint_dx else []
     norm = []
     shape = None
     for W, y0, c0, i, start, step, Y, C, H, DY, Dd in calls:
@@ -602,6 +643,10 @@ def native_lstm2_grad_multi(calls):
     with torch.cuda.device(device):
         status_watch.poll()
         outs = [_alloc_grad_outputs(T, B, n, bf16, device) for _ in range(count)]
+        joint = None
+        if joint_dx and (4 * n * outs[0][0].element_size()) % 16 == 0:  # (else: separate arrays, joined below)
+            joint = torch.empty((T, B, count * 4 * n), dtype=outs[0][0].dtype, device=device)
+            outs = [(joint[:, :, k * 4 * n : (k + 1) * 4 * n],) + o[1:] for k, o in enumerate(outs)]
         ws_bytes = int(lib.rtn_native_lstm2_bwd_multi_workspace_bytes(count, T, B, n, dtype))
         ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=device)
         arr = (_lib.Lstm2BwdCall * count)()
@@ -610,11 +655,17 @@ def native_lstm2_grad_multi(calls):
             arr[k] = _lib.Lstm2BwdCall(
                 W.data_ptr(), y0.data_ptr(), c0.data_ptr(), i.data_ptr(), start, step, Y.data_ptr(), C.data_ptr(), H.data_ptr(),
                 DY.data_ptr(), Dd.data_ptr(), DX.data_ptr(), DW.data_ptr(), Dy0.data_ptr(), Dc0.data_ptr(),
+                0 if Y.is_contiguous() else _row_pitch(Y, itemsize=Y.element_size()),
+                0 if DY.is_contiguous() else _row_pitch(DY, itemsize=DY.element_size()),
+                0 if joint is None else count * 4 * n,
             )  # fmt: skip
         rc = lib.rtn_native_lstm2_bwd_multi(arr, count, T, B, n, dtype, ws.data_ptr(), ws.numel(), torch.cuda.current_stream(device).cuda_stream)
         _lib.check(rc)
         if T * B * n > 0:  # (an empty problem does not touch its workspace)
             status_watch.after_call("NativeLstm2 gradient (%i calls)" % count, ws, count, device)
+    del norm  # (the normalised inputs stay alive until here; the stream-ordered allocator covers the rest)
+    if joint_dx:
+        return outs, (joint if joint is not None else torch.cat([o[0] for o in outs], dim=-1))
     return outs
 
 
@@ -811,6 +862,48 @@ class NativeLstm2PairFunction(torch.autograd.Function):
         return (*grads, None)
 
 
+class NativeLstm2BidirFunction(torch.autograd.Function):
+    """
+    A bidirectional layer on ONE projection: ``Y, df, db = NativeLstm2BidirFunction.apply(P, Wf, y0f, c0f, Wb, y0b, c0b, i)``
+    with ``P [T,B,8n]`` holding the pre-projected gates of the forward direction in columns ``[0,4n)`` and of the backward
+    direction in ``[4n,8n)``, and ``Y [T,B,2n]`` the outputs side by side (what returnn/tf/layers/rec.py:1229-1270 builds
+    from two op calls and a concat).  The directions read and write their columns in place (row pitch 8n and 2n); the
+    gradient reads the error of ``Y`` the same way and writes the error of ``P`` as one array, so neither pass copies or
+    concatenates an activation.  Results are those of two :class:`NativeLstm2Function` calls, (0, 1) and (0, -1).
+    """
+
+    @staticmethod
+    def forward(ctx, P, Wf, y0f, c0f, Wb, y0b, c0b, i):
+        n = y0f.shape[1]
+        if P.dim() != 3 or P.shape[2] != 8 * n:
+            raise RuntimeError("NativeLstm2 (bidirectional): P has shape %s, expected [T,B,%i]" % (tuple(P.shape), 8 * n))
+        outs, Y = native_lstm2_multi(
+            [(P[:, :, : 4 * n], Wf, y0f, c0f, i, 0, 1), (P[:, :, 4 * n :], Wb, y0b, c0b, i, 0, -1)], joint_output=True
+        )
+        (_, Cf, Hf, df), (_, Cb, Hb, db) = outs
+        ctx.save_for_backward(Wf, y0f, c0f, Wb, y0b, c0b, i, Y, Cf, Hf, Cb, Hb)
+        ctx.in_dtypes = (P.dtype, Wf.dtype, y0f.dtype, c0f.dtype, Wb.dtype, y0b.dtype, c0b.dtype)
+        ctx.set_materialize_grads(False)  # (no zero tensors for outputs without a gradient: backward takes None)
+        return Y, df, db
+
+    @staticmethod
+    def backward(ctx, DY, Ddf, Ddb):
+        Wf, y0f, c0f, Wb, y0b, c0b, i, Y, Cf, Hf, Cb, Hb = ctx.saved_tensors
+        n = y0f.shape[1]
+        DY = torch.zeros_like(Y) if DY is None else DY
+        Ddf = torch.zeros_like(c0f, dtype=torch.float32) if Ddf is None else Ddf
+        Ddb = torch.zeros_like(c0b, dtype=torch.float32) if Ddb is None else Ddb
+        (gf, gb), DP = native_lstm2_grad_multi(
+            [
+                (Wf, y0f, c0f, i, 0, 1, Y[:, :, :n], Cf, Hf, DY[:, :, :n], Ddf),
+                (Wb, y0b, c0b, i, 0, -1, Y[:, :, n:], Cb, Hb, DY[:, :, n:], Ddb),
+            ],
+            joint_dx=True,
+        )
+        grads = (DP,) + tuple(gf[1:]) + tuple(gb[1:])
+        return (*(g.to(t) for g, t in zip(grads, ctx.in_dtypes)), None)
+
+
 def lstm_last_output(Y: torch.Tensor, y0: torch.Tensor, i: torch.Tensor, start: int = 0, step: int = 1) -> torch.Tensor:
     """
     Final output per sequence, the caller-side ``_lstm_last_output`` of the reference
@@ -825,7 +918,10 @@ def lstm_last_output(Y: torch.Tensor, y0: torch.Tensor, i: torch.Tensor, start: 
         raise RuntimeError("lstm_last_output: this build implements the op for HIP (MI355X) tensors only")
     bf16 = Y.dtype == torch.bfloat16
     act = torch.bfloat16 if bf16 else torch.float32
-    Y = Y.to(act).contiguous()
+    Y = Y.to(act)
+    ldY = _row_pitch(Y, itemsize=Y.element_size())
+    if not ldY:
+        Y, ldY = Y.contiguous(), Y.shape[2]
     y0 = y0.to(act).contiguous()
     i = i.to(torch.float32).contiguous()
     T, B, n = Y.shape
@@ -836,7 +932,7 @@ def lstm_last_output(Y: torch.Tensor, y0: torch.Tensor, i: torch.Tensor, start: 
         out = torch.empty((B, n), dtype=act, device=Y.device)
         rc = lib.rtn_native_lstm2_last_output(
             Y.data_ptr(), y0.data_ptr(), i.data_ptr(), int(start), int(step), out.data_ptr(), T, B, n,
-            _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32, torch.cuda.current_stream(Y.device).cuda_stream,
+            _lib.DTYPE_BF16 if bf16 else _lib.DTYPE_F32, int(ldY), torch.cuda.current_stream(Y.device).cuda_stream,
         )  # fmt: skip
     _lib.check(rc)
     return out

@@ -50,6 +50,34 @@ def test_error_codes_match_header():
         assert getattr(lib, py) == int(value), name
 
 
+def test_call_structs_match_the_header(tmp_path):
+    """The ctypes mirrors of the header's call structs: same size and the same offset of every member, as a C compiler
+    lays the header out."""
+    import subprocess
+
+    mirrors = {"rtn_lstm2_call": lib.Lstm2Call, "rtn_lstm2_bwd_call": lib.Lstm2BwdCall}
+    lines = ['#include <stddef.h>', '#include <stdio.h>', '#include "rtn_native_lstm2.h"', "int main(void) {"]
+    for cname, mirror in mirrors.items():
+        lines.append('  printf("%s %%zu\\n", sizeof(%s));' % (cname, cname))
+        for field, _ in mirror._fields_:
+            lines.append('  printf("%s.%s %%zu\\n", offsetof(%s, %s));' % (cname, field, cname, field))
+    lines += ["  return 0;", "}"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines) + "\n")
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(_root, "include"), "-o", str(exe), str(src)], check=True)
+    out = dict(line.split() for line in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    header = open(os.path.join(_root, "include", "rtn_native_lstm2.h")).read()
+    for cname, mirror in mirrors.items():
+        assert int(out[cname]) == ctypes.sizeof(mirror), cname
+        for field, _ in mirror._fields_:
+            assert int(out["%s.%s" % (cname, field)]) == getattr(mirror, field).offset, (cname, field)
+        # every member of the C struct has a mirror: count the declarations between the braces
+        body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), header, re.S).group(1)
+        body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+        assert len([d for d in body.split(";") if d.strip()]) == len(mirror._fields_), cname
+
+
 def _call(cabi, T, B, n, start=0, step=1, dtype=0, mode=0, ptr=4096, ws=None, ws_bytes=0):
     p = ctypes.c_void_p(ptr)
     return cabi.rtn_native_lstm2_fwd(p, p, p, p, p, start, step, p, p, p, p, T, B, n, dtype, mode, ws, ws_bytes, None)
