@@ -387,9 +387,8 @@ def bench_encoder(args, dev):
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
         assert bool(torch.isfinite(y.float()).all())
-        # the projections alone, same shapes and weights
-        ws = [(m._weights(bf), d_in) for m, d_in in
-              [(m, enc.in_dim if li == 0 else 2 * n) for li in range(L) for m in (enc.fwd[li], enc.bwd[li])]]
+        # the projections alone, same shapes and weights: one GEMM per layer into [T*B, 8n], both directions' gates
+        ws = [(enc._weights(li, bf), enc.in_dim if li == 0 else 2 * n) for li in range(L)]
         srcs = {d: torch.randn((T * B, d), device=dev).to(bf) for d in {enc.in_dim, 2 * n}}
         for w, d_in in ws:
             torch.addmm(w.bias, srcs[d_in], w.ff)
@@ -422,7 +421,8 @@ def bench_encoder(args, dev):
         "data": "synthetic",
         "config": {
             "workload": "cfg4: %i-layer bidirectional LSTM encoder forward, T=%i B=%i in=%i n=%i bf16, ragged=True; "
-            "per layer and direction one projection GEMM and one NativeLstm2 call" % (L, T, B, prob.in_dim, n),
+            "per layer one projection GEMM into [T*B, 8n] and the two NativeLstm2 calls of the directions in one launch, reading "
+            "their columns of it and writing their columns of one [T, B, 2n] output" % (L, T, B, prob.in_dim, n),
             "calls_per_step": 2 * L,
             "units_per_step": units,
             "projection_ms_per_step": proj_ms,

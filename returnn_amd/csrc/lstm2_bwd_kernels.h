@@ -813,7 +813,7 @@ __global__ void k_column_partial_sums(const void* data, float* partial, long lon
   for (long long r = blockIdx.y; r < rows; r += gridDim.y) acc += Elem<AT>::load(data, r * width + c);
   partial[(long long)blockIdx.y * width + c] = acc;
 }
-__global__ void k_column_final_sums(const float* partial, float* out, int parts, int width) {
+static __global__ void k_column_final_sums(const float* partial, float* out, int parts, int width) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= width) return;
   float acc = 0.f;

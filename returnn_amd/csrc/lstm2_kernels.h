@@ -105,9 +105,9 @@ __device__ __forceinline__ bool wait_expired(const unsigned* status) {
 }
 // A 32-bit word full of quiet NaNs of the activation type.
 template <typename AT>
-constexpr unsigned kNanWords = 0x7FC00000u;
+inline constexpr unsigned kNanWords = 0x7FC00000u;
 template <>
-constexpr unsigned kNanWords<__bf16> = 0x7FC07FC0u;
+inline constexpr unsigned kNanWords<__bf16> = 0x7FC07FC0u;
 
 // Frame visited at step s.
 __device__ __forceinline__ long long frame_of(const Lstm2Params& p, int s) {
@@ -119,7 +119,7 @@ __device__ __forceinline__ long long frame_of(const Lstm2Params& p, int s) {
 // ---------------------------------------------------------------------------------------------
 
 // T == 0: d := c0 (returnn/native_op.py:1236-1237)
-__global__ void k_copy_f32(const float* __restrict__ src, float* __restrict__ dst, long long count) {
+static __global__ void k_copy_f32(const float* __restrict__ src, float* __restrict__ dst, long long count) {
   for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < count;
        i += (long long)gridDim.x * blockDim.x)
     dst[i] = src[i];
@@ -262,14 +262,14 @@ __global__ void k_unpad_cells(const ET* __restrict__ src, ET* __restrict__ dst, 
 }
 
 // Clears the status word for the generic path.
-__global__ void k_fill_u32(unsigned* dst, unsigned value, long long count) {
+static __global__ void k_fill_u32(unsigned* dst, unsigned value, long long count) {
   for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < count;
        i += (long long)gridDim.x * blockDim.x)
     dst[i] = value;
 }
 
 // rows of row_words 32-bit words, pitch_words apart: := 0
-__global__ void k_clear_rows(unsigned* dst, long long rows, long long row_words, long long pitch_words) {
+static __global__ void k_clear_rows(unsigned* dst, long long rows, long long row_words, long long pitch_words) {
   for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < rows * row_words; i += (long long)gridDim.x * blockDim.x) {
     const long long r = i / row_words;
     dst[r * pitch_words + (i - r * row_words)] = 0u;
@@ -283,7 +283,7 @@ __global__ void k_add_bias(void* data, const void* bias, long long count, int wi
     Elem<AT>::store(data, i, Elem<AT>::load(data, i) + Elem<AT>::load(bias, i % width));
 }
 
-__global__ void k_clear_status(unsigned* status) {
+static __global__ void k_clear_status(unsigned* status) {
   if (threadIdx.x < 64) status[threadIdx.x] = 0;
 }
 
@@ -810,7 +810,7 @@ __device__ __forceinline__ unsigned xcc_id() {
 }
 
 // Which XCDs does the device deal the workgroups of a grid to?  Every workgroup adds the XCD it runs on to a bit mask.
-__global__ void k_probe_xcds(unsigned* mask) {
+static __global__ void k_probe_xcds(unsigned* mask) {
   if (threadIdx.x == 0) (void)__hip_atomic_fetch_or(mask, 1u << xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -1648,7 +1648,7 @@ __global__ __launch_bounds__(THREADS) void k_mfma_issue(float* out, int steps) {
 // round number) and reads all G blocks, 16 lanes per block, until every word carries the round number; one
 // workgroup barrier per round.  A value from an earlier use of the buffer differs from the round number, so a
 // stale read can only cost a retry.  G <= 16.  status[0] is set to 1 if a wait runs into `timeout_ticks`.
-__global__ __launch_bounds__(kWgThreads) void k_handover_latency(unsigned* ring, unsigned* status, int G, int rounds,
+static __global__ __launch_bounds__(kWgThreads) void k_handover_latency(unsigned* ring, unsigned* status, int G, int rounds,
                                                                  unsigned long long timeout_ticks) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = blockIdx.x;

@@ -26,6 +26,7 @@
 
 #include "../../include/rtn_native_lstm2.h"
 #include "lstm2_bwd_kernels.h"
+#include "lstm2_kernel_tables.h"
 #include "lstm2_kernels.h"
 
 // Scratch memory of rtn_native_lstm2_fwd_static, the entry point for callers that cannot allocate: a fixed array in the
@@ -254,9 +255,13 @@ bool make_plan_uncached(int64_t T, int B, int n, int dtype, int want_mode, bool 
           if (env_mt && MT != env_mt) continue;
           if ((n / 4) % MT) continue;
           const int G = n / (4 * MT);
-          if (G > cu_x) continue;
+          // Workgroups that can share a CU: the register kernel with few fragments per wavefront fits twice (two
+          // wavefronts per SIMD keep the matrix core busier than one, and one workgroup's MFMAs cover the other's wait).
+          const size_t lds_wg = (size_t)regw_lds((int)es, MT, 1).total;
+          const int per_cu = (MT * KSMAX <= 32 && KSMAX <= 8 && 2 * lds_wg <= di.lds_per_wg) ? max_wgs_per_cu : 1;
+          if (G > cu_x * per_cu) continue;
           if (MT * KSMAX > (KSMAX == 16 ? 32 : 64) || (MT == 8 && KSMAX != 8)) continue;
-          const int capacity = di.xcds * (cu_x / G) / std::max(problems, 1);  // groups per problem
+          const int capacity = di.xcds * (cu_x * per_cu / G) / std::max(problems, 1);  // groups per problem
           if (capacity < 1) continue;
           int groups = std::min(capacity, Bq);
           if (env_groups) groups = (int)std::min<long>(env_groups, groups);
@@ -547,41 +552,6 @@ MfmaKernel mfma_kernel_for(int MT, int NT) {
 
 MfmaKernel mfma_kernel(int dtype, int MT, int NT) {
   return dtype == RTN_DTYPE_BF16 ? mfma_kernel_for<__bf16>(MT, NT) : mfma_kernel_for<float>(MT, NT);
-}
-
-typedef void (*RegwKernel)(const Lstm2Multi);
-
-template <typename AT>
-RegwKernel regw_kernel_for(int MT, int NT, int KSMAX, bool half) {
-  if (half) {
-#define RTN_CASE(mt, ks) \
-  if (MT == mt && NT == 1 && KSMAX == ks) return &k_lstm2_regw<AT, mt, 1, ks, true>;
-    RTN_CASE(2, 2) RTN_CASE(2, 4) RTN_CASE(2, 8) RTN_CASE(2, 16)
-    RTN_CASE(4, 2) RTN_CASE(4, 4) RTN_CASE(4, 8)
-    RTN_CASE(8, 8)
-#undef RTN_CASE
-    return nullptr;
-  }
-#define RTN_CASE(mt, nt, ks) \
-  if (MT == mt && NT == nt && KSMAX == ks) return &k_lstm2_regw<AT, mt, nt, ks>;
-  RTN_CASE(1, 1, 2) RTN_CASE(1, 2, 2) RTN_CASE(1, 4, 2)
-  RTN_CASE(2, 1, 2) RTN_CASE(2, 2, 2) RTN_CASE(2, 4, 2)
-  RTN_CASE(4, 1, 2) RTN_CASE(4, 2, 2)
-  RTN_CASE(1, 1, 4) RTN_CASE(1, 2, 4) RTN_CASE(1, 4, 4)
-  RTN_CASE(2, 1, 4) RTN_CASE(2, 2, 4) RTN_CASE(2, 4, 4)
-  RTN_CASE(4, 1, 4) RTN_CASE(4, 2, 4)
-  RTN_CASE(1, 1, 8) RTN_CASE(1, 2, 8) RTN_CASE(1, 4, 8)
-  RTN_CASE(2, 1, 8) RTN_CASE(2, 2, 8) RTN_CASE(2, 4, 8)
-  RTN_CASE(4, 1, 8) RTN_CASE(4, 2, 8)
-  RTN_CASE(8, 1, 8)
-  RTN_CASE(1, 1, 16) RTN_CASE(1, 2, 16)
-  RTN_CASE(2, 1, 16) RTN_CASE(2, 2, 16)
-#undef RTN_CASE
-  return nullptr;
-}
-
-RegwKernel regw_kernel(int dtype, int MT, int NT, int KSMAX, bool half) {
-  return dtype == RTN_DTYPE_BF16 ? regw_kernel_for<__bf16>(MT, NT, KSMAX, half) : regw_kernel_for<float>(MT, NT, KSMAX, half);
 }
 
 // Kernels that use more than the default LDS limit need the limit raised once per device.
@@ -1389,37 +1359,9 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
 }
 
 
-typedef void (*BwdRegwKernel)(const Lstm2BwdMulti);
-
-// Bytes of dynamic shared memory of the variants that keep half of a wavefront's share of W in LDS (4 wavefronts with
-// 32 + 32 fragments, or 8 wavefronts with 16 + 16).
+// Bytes of dynamic shared memory of the gradient kernel's variants that keep half of a wavefront's share of W in LDS (4
+// wavefronts with 32 + 32 fragments, or 8 wavefronts with 16 + 16).
 constexpr size_t kBwdLdsShareBytes = (size_t)kWaves * 32 * 64 * 16;
-
-// The variants with half of W in registers and half in LDS (one tile per workgroup).
-template <typename AT>
-BwdRegwKernel bwd_regw_lds_kernel_for(int WV) {
-  if (WV == 8) return &k_lstm2_bwd_regw<AT, 16, 1, 8, 16>;
-  return &k_lstm2_bwd_regw<AT, 32, 1, 4, 32>;
-}
-
-// KSB: fragments of W per tile and wavefront; MT: tiles of 16 values of k per workgroup; WV: wavefronts per workgroup.
-template <typename AT, bool HALF>
-BwdRegwKernel bwd_regw_kernel_for(int KSB, int MT, int WV) {
-#define RTN_CASE(ks, mt, wv) \
-  if (KSB == ks && MT == mt && WV == wv) return &k_lstm2_bwd_regw<AT, ks, mt, wv, 0, HALF>;
-  RTN_CASE(2, 1, 4) RTN_CASE(4, 1, 4) RTN_CASE(8, 1, 4) RTN_CASE(16, 1, 4) RTN_CASE(32, 1, 4)
-  if constexpr (sizeof(AT) == 2) { RTN_CASE(64, 1, 4) }
-  RTN_CASE(2, 2, 4) RTN_CASE(4, 2, 4) RTN_CASE(8, 2, 4) RTN_CASE(16, 2, 4) RTN_CASE(32, 2, 4)
-  RTN_CASE(2, 4, 4) RTN_CASE(4, 4, 4) RTN_CASE(8, 4, 4) RTN_CASE(16, 4, 4)
-  RTN_CASE(2, 1, 8) RTN_CASE(4, 1, 8) RTN_CASE(8, 1, 8) RTN_CASE(16, 1, 8)
-  RTN_CASE(2, 2, 8) RTN_CASE(4, 2, 8) RTN_CASE(8, 2, 8) RTN_CASE(16, 2, 8)
-  RTN_CASE(2, 4, 8) RTN_CASE(4, 4, 8) RTN_CASE(8, 4, 8) RTN_CASE(16, 4, 8)
-  RTN_CASE(2, 1, 16) RTN_CASE(4, 1, 16) RTN_CASE(8, 1, 16)
-  RTN_CASE(2, 2, 16) RTN_CASE(4, 2, 16) RTN_CASE(8, 2, 16)
-  RTN_CASE(2, 4, 16) RTN_CASE(4, 4, 16) RTN_CASE(8, 4, 16)
-#undef RTN_CASE
-  return nullptr;
-}
 
 // One rocBLAS handle per host thread and device, created on first use and kept for the life of the thread (never
 // destroyed: at thread or process exit the runtime below it may already be gone).  A handle carries the stream its
@@ -2027,11 +1969,11 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
         if (lds_share && (mt != 1 || (wv != 4 && wv != 8))) continue;
         BwdRegwKernel kfn;
         if (lds_share)
-          kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_lds_kernel_for<__bf16>(wv) : bwd_regw_lds_kernel_for<float>(wv);
+          kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_lds_table_bf16(wv) : bwd_regw_lds_table_f32(wv);
         else
           // ring frames of 8 rows: the variant whose loads take two macro steps at once
-          kfn = use_rows <= 8 ? (dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16, true>(ksb_room, mt, wv) : bwd_regw_kernel_for<float, true>(ksb_room, mt, wv))
-                              : (dtype == RTN_DTYPE_BF16 ? bwd_regw_kernel_for<__bf16, false>(ksb_room, mt, wv) : bwd_regw_kernel_for<float, false>(ksb_room, mt, wv));
+          kfn = use_rows <= 8 ? (dtype == RTN_DTYPE_BF16 ? bwd_regw_table_bf16_half(ksb_room, mt, wv) : bwd_regw_table_f32_half(ksb_room, mt, wv))
+                              : (dtype == RTN_DTYPE_BF16 ? bwd_regw_table_bf16_full(ksb_room, mt, wv) : bwd_regw_table_f32_full(ksb_room, mt, wv));
         if (!kfn) continue;
         const size_t cand_lds = lds_share ? kBwdLdsShareBytes : 0;
         if (cand_lds) {
