@@ -388,7 +388,7 @@ def bench_encoder(args, dev):
         elapsed = time.perf_counter() - t0
         assert bool(torch.isfinite(y.float()).all())
         # the projections alone, same shapes and weights: one GEMM per layer into [T*B, 8n], both directions' gates
-        ws = [(enc._weights(li, bf), enc.in_dim if li == 0 else 2 * n) for li in range(L)]
+        ws = [(enc.layers[li].weights(bf), enc.in_dim if li == 0 else 2 * n) for li in range(L)]
         srcs = {d: torch.randn((T * B, d), device=dev).to(bf) for d in {enc.in_dim, 2 * n}}
         for w, d_in in ws:
             torch.addmm(w.bias, srcs[d_in], w.ff)

@@ -19,9 +19,12 @@ in memory (the caller protocol of returnn/tf/layers/rec.py:1229-1270).
 With gradients enabled and an input that requires them, the same functions go through
 ``NativeLstm2Function`` (the op with its gradient op) and torch's autograd, so the layer trains like ``rf.LSTM``.
 
-:class:`LSTM` and :class:`LstmState` mirror the module and its state; :class:`BlstmEncoder` stacks
-bidirectional layers (:func:`blstm`: both directions of a layer go through the library's multi-call entry, which
-runs them in one launch when the device can hold both; outputs concatenated).
+:class:`LSTM` and :class:`LstmState` mirror the module and its state (parameters in the frontend's names and layout).
+:class:`BLSTM` is one bidirectional layer (:func:`blstm`: ONE projection for both directions, which then go through the
+library's multi-call entry -- one launch when the device can hold both -- reading their columns of the projection and
+writing their columns of the one output); it keeps its parameters in the op's layout, so that a training step
+converts nothing, and speaks the frontend's layout in ``state_dict`` / ``load_state_dict`` / :meth:`BLSTM.frontend_params`.
+:class:`BlstmEncoder` stacks such layers.
 """
 
 from __future__ import annotations
@@ -34,7 +37,10 @@ import torch
 from . import native_op
 from .torch_native_op import NativeLstm2BidirFunction, NativeLstm2Function, lstm_last_output, make_op, native_lstm2_multi
 
-__all__ = ["lstm", "blstm", "prepare_weights", "LstmWeights", "LSTM", "LstmState", "BlstmEncoder", "sequence_mask_time_major"]
+__all__ = [
+    "lstm", "blstm", "prepare_weights", "prepare_blstm_weights", "join_weights", "LstmWeights", "BlstmWeights", "LSTM", "BLSTM",
+    "LstmState", "BlstmEncoder", "sequence_mask_time_major",
+]  # fmt: skip
 
 
 class LstmState(NamedTuple):
@@ -384,40 +390,154 @@ class LSTM(torch.nn.Module):
         return "in_dim=%i, out_dim=%i, with_bias=%s" % (self.in_dim, self.out_dim, self.bias is not None)
 
 
+def _from_native_gate_order(w: torch.Tensor) -> torch.Tensor:
+    """[4*out, ...] in (cell-in, input, forget, output) blocks -> (input, forget, cell-in, output)."""
+    g, i, f, o = w.chunk(4, dim=0)
+    return torch.cat((i, f, g, o), dim=0)
+
+
+class BLSTM(torch.nn.Module):
+    """
+    One bidirectional LSTM layer: a forward-in-time and a backward-in-time recurrence on the same input, outputs side by
+    side (``2*out_dim`` features).
+
+    The parameters live in the layout the op takes -- ``ff [8*out, in]`` (rows: the forward direction's gates cell-in,
+    input, forget, output, then the backward direction's; the projection uses its transposed view), ``rec_fwd`` /
+    ``rec_bwd [out, 4*out]``, ``bias [8*out]`` -- so that neither a forward nor a training step reorders or joins
+    anything.  The frontend's layout (returnn/frontend/rec.py:46-77: per direction ``ff_weight [4*out,in]``,
+    ``rec_weight [4*out,out]``, ``bias [4*out]`` in the order input, forget, cell-in, output; the mapping of
+    returnn/tf/frontend_layers/_backend.py:1199-1222) is what :meth:`frontend_params`, :meth:`load_frontend_params`,
+    ``state_dict()`` and ``load_state_dict()`` speak (keys ``fwd.ff_weight``, ``fwd.rec_weight``, ``fwd.bias``, ``bwd. ...``).
+    Initialisation as the frontend's: every direction's ``ff_weight`` and ``rec_weight`` Glorot-uniform
+    (returnn/frontend/init.py:189-197), biases zero.
+    """
+
+    _FRONTEND_KEYS = ("ff_weight", "rec_weight", "bias")
+
+    def __init__(self, in_dim: int, out_dim: int, *, with_bias: bool = True, device=None, dtype=None):
+        super().__init__()
+        self.in_dim, self.out_dim = int(in_dim), int(out_dim)
+        kw = dict(device=device, dtype=dtype)
+        n = self.out_dim
+        self.ff = torch.nn.Parameter(torch.empty((8 * n, self.in_dim), **kw))
+        self.rec_fwd = torch.nn.Parameter(torch.empty((n, 4 * n), **kw))
+        self.rec_bwd = torch.nn.Parameter(torch.empty((n, 4 * n), **kw))
+        self.bias = torch.nn.Parameter(torch.zeros((8 * n,), **kw)) if with_bias else None
+        self.reset_parameters()
+
+    def reset_parameters(self, generator: Optional[torch.Generator] = None):
+        n = self.out_dim
+        with torch.no_grad():
+            self.ff.uniform_(-math.sqrt(6.0 / (4 * n + self.in_dim)), math.sqrt(6.0 / (4 * n + self.in_dim)), generator=generator)
+            for p in (self.rec_fwd, self.rec_bwd):
+                p.uniform_(-math.sqrt(6.0 / (5 * n)), math.sqrt(6.0 / (5 * n)), generator=generator)
+            if self.bias is not None:
+                self.bias.zero_()
+
+    def weights(self, act: torch.dtype) -> BlstmWeights:
+        """The parameters as :func:`blstm` takes them (views; a cast only when the run's type is not the parameters')."""
+        return BlstmWeights(
+            ff=self.ff.to(act).t(), rec_fwd=self.rec_fwd.to(act), rec_bwd=self.rec_bwd.to(act),
+            bias=None if self.bias is None else self.bias.to(act),
+        )  # fmt: skip
+
+    def frontend_params(self) -> dict:
+        """``{"fwd": p, "bwd": p}`` with ``p = {"ff_weight" [4*out,in], "rec_weight" [4*out,out], "bias" [4*out] or None}`` in the
+        frontend's gate order (copies, detached)."""
+        n4 = 4 * self.out_dim
+        out = {}
+        with torch.no_grad():
+            for k, (name, rec) in enumerate((("fwd", self.rec_fwd), ("bwd", self.rec_bwd))):
+                out[name] = {
+                    "ff_weight": _from_native_gate_order(self.ff[k * n4 : (k + 1) * n4]).contiguous(),
+                    "rec_weight": _from_native_gate_order(rec.t()).contiguous(),
+                    "bias": None if self.bias is None else _from_native_gate_order(self.bias[k * n4 : (k + 1) * n4]).contiguous(),
+                }
+        return out
+
+    def load_frontend_params(self, fwd: dict, bwd: dict):
+        """Takes the two directions' parameters in the frontend's layout (arrays or tensors)."""
+        n4 = 4 * self.out_dim
+        with torch.no_grad():
+            for k, (p, rec) in enumerate(((fwd, self.rec_fwd), (bwd, self.rec_bwd))):
+                ff_w, rec_w = torch.as_tensor(p["ff_weight"]), torch.as_tensor(p["rec_weight"])
+                if tuple(ff_w.shape) != (n4, self.in_dim) or tuple(rec_w.shape) != (n4, self.out_dim):
+                    raise ValueError("BLSTM: ff_weight %s / rec_weight %s, expected %s / %s"
+                                     % (tuple(ff_w.shape), tuple(rec_w.shape), (n4, self.in_dim), (n4, self.out_dim)))  # fmt: skip
+                self.ff[k * n4 : (k + 1) * n4].copy_(_to_native_gate_order(ff_w))
+                rec.copy_(_to_native_gate_order(rec_w).t())
+                b = p.get("bias")
+                if (b is None) != (self.bias is None):
+                    raise ValueError("BLSTM: the layer was built %s a bias" % ("without" if self.bias is None else "with"))
+                if b is not None:
+                    self.bias[k * n4 : (k + 1) * n4].copy_(_to_native_gate_order(torch.as_tensor(b)))
+
+    # state_dict / load_state_dict in the frontend's layout, so that checkpoints do not depend on the op's layout
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        for name, p in self.frontend_params().items():
+            for key in self._FRONTEND_KEYS:
+                if p[key] is not None:
+                    destination[prefix + name + "." + key] = p[key]
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
+        keys = [n + "." + k for n in ("fwd", "bwd") for k in self._FRONTEND_KEYS if not (k == "bias" and self.bias is None)]
+        absent = [k for k in keys if prefix + k not in state_dict]
+        if absent:
+            if strict:
+                missing_keys.extend(prefix + k for k in absent)
+            return
+        try:
+            parts = {n: {k: state_dict.get(prefix + n + "." + k) for k in self._FRONTEND_KEYS} for n in ("fwd", "bwd")}
+            self.load_frontend_params(parts["fwd"], parts["bwd"])
+        except (ValueError, RuntimeError) as exc:
+            error_msgs.append(str(exc))
+        if strict:
+            unexpected_keys.extend(k for k in state_dict if k.startswith(prefix) and k[len(prefix) :] not in keys)
+
+    def default_initial_state(self, *, batch_dims: Sequence[int], device=None, dtype=None) -> LstmState:
+        """zeros for one direction (returnn/frontend/rec.py:78-83); h in the parameters' type (or ``dtype``), c in float32"""
+        shape = tuple(batch_dims) + (self.out_dim,)
+        device = device or self.ff.device
+        return LstmState(h=torch.zeros(shape, dtype=dtype or self.ff.dtype, device=device), c=torch.zeros(shape, dtype=torch.float32, device=device))
+
+    def forward(
+        self, source: torch.Tensor, *, state_fwd: Optional[LstmState] = None, state_bwd: Optional[LstmState] = None,
+        seq_lens: Optional[torch.Tensor] = None,
+    ) -> Tuple[torch.Tensor, LstmState, LstmState]:  # fmt: skip
+        """
+        :param source: [T,B,in]
+        :param state_fwd, state_bwd: initial states, default zeros
+        :return: [T,B,2*out_dim] (forward | backward), new forward state, new backward state
+        """
+        if source.dim() != 3 or source.shape[-1] != self.in_dim:
+            raise ValueError("%s: input %s is not [T,B,%i]" % (self, tuple(source.shape), self.in_dim))
+        act = torch.bfloat16 if source.dtype == torch.bfloat16 else torch.float32
+        zero = None
+        if state_fwd is None or state_bwd is None:
+            zero = self.default_initial_state(batch_dims=(source.shape[1],), device=source.device, dtype=act)
+        return blstm(source, weights=self.weights(act), state_fwd=state_fwd or zero, state_bwd=state_bwd or zero, seq_lens=seq_lens)
+
+    def extra_repr(self) -> str:
+        return "in_dim=%i, out_dim=%i, with_bias=%s" % (self.in_dim, self.out_dim, self.bias is not None)
+
+
 class BlstmEncoder(torch.nn.Module):
     """
-    Stack of bidirectional LSTM layers: per layer a forward-in-time and a backward-in-time :class:`LSTM` on the same
-    input, outputs concatenated to ``2*out_dim`` features, which feed the next layer.  All layers use the same
+    Stack of bidirectional LSTM layers (:class:`BLSTM`): per layer a forward-in-time and a backward-in-time recurrence on
+    the same input, outputs side by side (``2*out_dim`` features), which feed the next layer.  All layers use the same
     sequence lengths; states start at zero.
     """
 
     def __init__(self, in_dim: int, out_dim: int, num_layers: int, *, with_bias: bool = True, device=None, dtype=None):
         super().__init__()
         self.in_dim, self.out_dim, self.num_layers = int(in_dim), int(out_dim), int(num_layers)
-        self.fwd = torch.nn.ModuleList()
-        self.bwd = torch.nn.ModuleList()
-        for layer in range(self.num_layers):
-            d_in = self.in_dim if layer == 0 else 2 * self.out_dim
-            self.fwd.append(LSTM(d_in, self.out_dim, with_bias=with_bias, device=device, dtype=dtype))
-            self.bwd.append(LSTM(d_in, self.out_dim, with_bias=with_bias, device=device, dtype=dtype))
-        self._prepared = {}  # layer -> (key, BlstmWeights)
-
-    def _weights(self, layer: int, act: torch.dtype) -> BlstmWeights:
-        """Joint weights of a layer; kept while the parameters do not change and need no gradient."""
-        f, b = self.fwd[layer], self.bwd[layer]
-        ps = [p for m in (f, b) for p in (m.ff_weight, m.rec_weight, m.bias) if p is not None]
-        args = ((f.ff_weight, f.rec_weight, f.bias), (b.ff_weight, b.rec_weight, b.bias))
-        if _wants_grad(*ps):
-            return prepare_blstm_weights(*args, dtype=act)  # differentiable, not cached
-        key = (act,) + tuple((p.data_ptr(), p._version, p.device) for p in ps)
-        hit = self._prepared.get(layer)
-        if hit is None or hit[0] != key:
-            with torch.no_grad():
-                hit = self._prepared[layer] = (key, prepare_blstm_weights(*args, dtype=act))
-        return hit[1]
+        self.layers = torch.nn.ModuleList(
+            BLSTM(self.in_dim if layer == 0 else 2 * self.out_dim, self.out_dim, with_bias=with_bias, device=device, dtype=dtype)
+            for layer in range(self.num_layers)
+        )
 
     def reset_parameters(self, generator: Optional[torch.Generator] = None):
-        for m in list(self.fwd) + list(self.bwd):
+        for m in self.layers:
             m.reset_parameters(generator)
 
     @classmethod
@@ -430,11 +550,8 @@ class BlstmEncoder(torch.nn.Module):
         n = first["rec_weight"].shape[1]
         with_bias = first.get("bias") is not None
         enc = cls(first["ff_weight"].shape[1], n, len(layers), with_bias=with_bias, device=device, dtype=dtype)
-        with torch.no_grad():
-            for layer, mods in zip(layers, zip(enc.fwd, enc.bwd)):
-                for key, mod in zip(("fwd", "bwd"), mods):
-                    for name in ("ff_weight", "rec_weight") + (("bias",) if with_bias else ()):
-                        getattr(mod, name).copy_(torch.as_tensor(layer[key][name]))
+        for params, layer in zip(layers, enc.layers):
+            layer.load_frontend_params(params["fwd"], params["bwd"])
         return enc
 
     def forward(
@@ -447,12 +564,8 @@ class BlstmEncoder(torch.nn.Module):
         :return: [T,B,2*out_dim]
         """
         x = source
-        B = source.shape[1]
         states = []
-        for layer, f in enumerate(self.fwd):
-            s0 = f.default_initial_state(batch_dims=(B,), device=source.device)
-            s0 = LstmState(h=s0.h.to(x.dtype), c=s0.c)
-            act = torch.bfloat16 if x.dtype == torch.bfloat16 else torch.float32
-            x, sf, sb = blstm(x, weights=self._weights(layer, act), state_fwd=s0, state_bwd=s0, seq_lens=seq_lens)
+        for layer in self.layers:
+            x, sf, sb = layer(x, seq_lens=seq_lens)
             states.append((sf, sb))
         return (x, states) if collect_states else x

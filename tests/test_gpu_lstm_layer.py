@@ -189,12 +189,16 @@ def test_blstm_encoder_cfg4_reduced_bf16():
     x_ref_chain = prob.features
     B = prob.B
     worst_layer, worst_chain = 0.0, 0.0
-    for li, (f, b) in enumerate(zip(enc.fwd, enc.bwd)):
-        s0 = rlstm.LstmState(h=torch.zeros(B, prob.n, dtype=bf, device=DEV), c=torch.zeros(B, prob.n, device=DEV))
-        yf, sf = f(x, state=s0, seq_lens=lens, direction=1)
-        yb, sb = b(x, state=s0, seq_lens=lens, direction=-1)
-        y = torch.cat((yf, yb), dim=-1)
+    for li in range(prob.num_layers):
         layer = prob.layers[li]
+        s0 = rlstm.LstmState(h=torch.zeros(B, prob.n, dtype=bf, device=DEV), c=torch.zeros(B, prob.n, device=DEV))
+        outs = []
+        for d, direction in (("fwd", 1), ("bwd", -1)):  # the two directions as single layers, from the frontend's parameters
+            yd, (hd, cd) = rlstm.lstm(x, state_h=s0.h, state_c=s0.c, seq_lens=lens, direction=direction,
+                                      **{k: _dev(layer[d][k], bf) for k in ("ff_weight", "rec_weight", "bias")})  # fmt: skip
+            outs.append((yd, rlstm.LstmState(hd, cd)))
+        (yf, sf), (yb, sb) = outs
+        y = torch.cat((yf, yb), dim=-1)
         ref, h, c = blstm_layer(_np(x), prob.lens, layer["fwd"], layer["bwd"], dtype=torch.float32)
         err = float(numpy.abs(_np(y) - ref).max())
         err_c = max(float(numpy.abs(_np(sf.c) - c[0]).max()), float(numpy.abs(_np(sb.c) - c[1]).max()))

@@ -273,3 +273,44 @@ def test_blstm_on_one_projection_equals_two_layers(dtype, T, B, n_in, n):
     with torch.no_grad():
         y3, sf3, sb3 = rlstm.blstm(x, weights=w, state_fwd=rlstm.LstmState(h0[0], c0[0]), state_bwd=rlstm.LstmState(h0[1], c0[1]), seq_lens=lens)
     assert torch.equal(y3, y.detach()) and torch.equal(sf3.c, sf.c.detach()) and torch.equal(sb3.h, sb.h.detach())
+
+
+def test_blstm_module_keeps_the_ops_layout_and_trains_like_two_lstm_modules():
+    """:class:`BLSTM` (parameters in the op's layout, nothing converted per step) against two :class:`LSTM` modules
+    (parameters in the frontend's layout) holding the same weights: outputs, states and every parameter's gradient."""
+    announce("BLSTM module")
+    T, B, n_in, n = 8, 6, 48, 64
+    gen = torch.Generator().manual_seed(11)
+    singles = [rlstm.LSTM(n_in, n, device="cuda:0") for _ in range(2)]
+    with torch.no_grad():
+        for m in singles:
+            for p in m.parameters():
+                p.copy_((torch.randn(p.shape, generator=gen) * 0.2).to("cuda:0"))
+    layer = rlstm.BLSTM(n_in, n, device="cuda:0")
+    layer.load_frontend_params(*[{k: getattr(m, k).detach() for k in ("ff_weight", "rec_weight", "bias")} for m in singles])
+    x = torch.randn((T, B, n_in), generator=gen).to("cuda:0")
+    lens = torch.tensor([T, T - 1, 3, T, 1, 5])
+    G = torch.randn((T, B, 2 * n), generator=gen).to("cuda:0")
+    y, sf, sb = layer(x, seq_lens=lens)
+    ((y * G).sum() + sf.c.sum() + 2.0 * sb.h.sum()).backward()
+    s0 = singles[0].default_initial_state(batch_dims=(B,))
+    outs = [m(x, state=s0, seq_lens=lens, direction=d) for m, d in zip(singles, (1, -1))]
+    y2 = torch.cat([o[0] for o in outs], dim=-1)
+    ((y2 * G).sum() + outs[0][1].c.sum() + 2.0 * outs[1][1].h.sum()).backward()
+    torch.cuda.synchronize()
+    assert float((y.detach() - y2.detach()).abs().max()) <= 1e-5
+    assert float((sb.h.detach() - outs[1][1].h.detach()).abs().max()) <= 1e-5
+
+    def close(got, want, what):
+        scale = max(float(want.abs().max()), 1e-30)
+        assert float((got - want).abs().max()) / scale <= 1e-4, what
+
+    n4 = 4 * n
+    for k, (m, rec) in enumerate(zip(singles, (layer.rec_fwd, layer.rec_bwd))):
+        close(rlstm._from_native_gate_order(layer.ff.grad[k * n4 : (k + 1) * n4]), m.ff_weight.grad, "ff %i" % k)
+        close(rlstm._from_native_gate_order(rec.grad.t()), m.rec_weight.grad, "rec %i" % k)
+        close(rlstm._from_native_gate_order(layer.bias.grad[k * n4 : (k + 1) * n4]), m.bias.grad, "bias %i" % k)
+    # a checkpoint written by the layer is in the frontend's layout
+    sd = layer.state_dict()
+    assert torch.equal(sd["bwd.rec_weight"], singles[1].rec_weight.detach())
+    assert torch.equal(sd["fwd.ff_weight"], singles[0].ff_weight.detach())

@@ -124,4 +124,23 @@ def test_encoder_config_shapes():
     assert numpy.abs(w).max() <= math.sqrt(6.0 / (64 + 32))
     enc = rlstm.BlstmEncoder.from_params(p.layers)
     assert enc.num_layers == 3 and enc.in_dim == 80 and enc.out_dim == 16
-    assert torch.equal(enc.bwd[2].rec_weight.detach(), torch.from_numpy(p.layers[2]["bwd"]["rec_weight"]))
+    # the layers keep their parameters in the op's layout and hand the frontend's back, bit for bit
+    back = enc.layers[2].frontend_params()
+    for d in ("fwd", "bwd"):
+        for k in ("ff_weight", "rec_weight", "bias"):
+            assert torch.equal(back[d][k], torch.from_numpy(p.layers[2][d][k])), (d, k)
+    assert tuple(enc.layers[1].ff.shape) == (128, 32) and tuple(enc.layers[1].rec_bwd.shape) == (16, 64)
+    sd = enc.state_dict()
+    assert torch.equal(sd["layers.2.bwd.rec_weight"], torch.from_numpy(p.layers[2]["bwd"]["rec_weight"]))
+    other = rlstm.BlstmEncoder(80, 16, 3)
+    other.load_state_dict(sd)
+    assert all(torch.equal(a, b) for a, b in zip(enc.parameters(), other.parameters()))
+    # the op's layout is what prepare_blstm_weights makes of the frontend's parameters
+    w = enc.layers[1].weights(torch.float32)
+    w2 = rlstm.prepare_blstm_weights(
+        *[tuple(torch.from_numpy(p.layers[1][d][k]) for k in ("ff_weight", "rec_weight", "bias")) for d in ("fwd", "bwd")]
+    )
+    assert all(torch.equal(a, b) for a, b in zip(w, w2))
+    del sd["layers.0.fwd.bias"]
+    with pytest.raises(RuntimeError, match="layers.0.fwd.bias"):
+        other.load_state_dict(sd)
