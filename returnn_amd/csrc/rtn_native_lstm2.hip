@@ -809,7 +809,7 @@ int launch_steps_graph(const Lstm2Params& p, const Plan& pl, int dtype, hipStrea
 }
 
 // ---- launches that need all their workgroups on the device together ------------------------------------------------
-// Outside stream capture: a cooperative launch (the runtime checks that the grid fits and keeps such launches apart).
+// Outside stream capture: an ordinary launch behind an ordering of the library's own (below).
 // Under stream capture a cooperative launch cannot be recorded with the stream API, so the kernel node is built by hand:
 // the capturing graph and the stream's current dependencies are asked of the runtime, a kernel node with the cooperative
 // attribute is added behind them and made the stream's new dependency.  If the runtime refuses any of that, the kernel
@@ -822,9 +822,42 @@ std::mutex g_capture_mu;
 long long g_capture_cooperative = 0, g_capture_plain = 0;
 std::string g_capture_refusal;  // why a cooperative node was refused, if it was
 
+// Outside capture a persistent kernel goes out as an ORDINARY launch.  It uses no grid barrier; what it needs is all its
+// workgroups on the device together, which the caller has checked against the occupancy of the kernel, and which an
+// ordinary launch gives on a device that is not shared: its waits are bounded like everywhere else.  A cooperative launch
+// costs two switches of hardware queue (measured: the device idles 11 us in front of the kernel and 11 us behind it; an
+// ordinary launch follows the kernel before it without a gap).  What the cooperative queue did give is that two
+// persistent kernels never share the device, each with part of its grid, waiting for the rest: the library keeps that
+// property for its own launches itself -- one event per device behind the last persistent launch, which a launch on
+// another stream waits for (on the device, the host never blocks).
+// RTN_LSTM2_LAUNCH=cooperative brings the cooperative launch back; the entry that may not create anything at call time
+// (g_no_setup_objects) keeps it, since this scheme needs an event.
+thread_local bool g_no_setup_objects = false;
+struct PersistentOrder {
+  hipEvent_t last = nullptr;      // behind the last persistent launch on this device
+  hipStream_t stream = nullptr;   // the stream it went to
+  bool any = false;
+};
+std::mutex g_order_mu;
+PersistentOrder g_order[64];
+
 int launch_coresident(const void* k, dim3 grid, dim3 block, void** args, unsigned lds, hipStream_t stream, bool capturing) {
   if (!capturing) {
-    RTN_HIP(hipLaunchCooperativeKernel(k, grid, block, args, lds, stream));
+    const char* how = env_get("RTN_LSTM2_LAUNCH");
+    int dev = 0;
+    RTN_HIP(hipGetDevice(&dev));
+    if (g_no_setup_objects || (how && strcmp(how, "cooperative") == 0) || dev < 0 || dev >= 64) {
+      RTN_HIP(hipLaunchCooperativeKernel(k, grid, block, args, lds, stream));
+      return RTN_OK;
+    }
+    std::lock_guard<std::mutex> lock(g_order_mu);
+    PersistentOrder& o = g_order[dev];
+    if (!o.last) RTN_HIP(hipEventCreateWithFlags(&o.last, hipEventDisableTiming));
+    if (o.any && o.stream != stream) RTN_HIP(hipStreamWaitEvent(stream, o.last, 0));
+    RTN_HIP(hipLaunchKernel(k, grid, block, args, lds, stream));
+    RTN_HIP(hipEventRecord(o.last, stream));
+    o.stream = stream;
+    o.any = true;
     return RTN_OK;
   }
   const char* kind = env_get("RTN_LSTM2_CAPTURE_NODE");
@@ -1622,7 +1655,11 @@ int rtn_native_lstm2_fwd_static(const void* X, const void* W, const void* y0, co
   rc = static_scratch(&ws);
   if (rc != RTN_OK) return rc;
   rtn_lstm2_call call = {X, W, y0, c0, i, start, step, Y, C, H, d};
-  return fwd_calls(&call, 1, T, B, n, dtype, mode, ws, (size_t)RTN_STATIC_SCRATCH_BYTES, hip_stream, 0, 0, /*no_graph=*/true);
+  // (nothing may be created at call time here: the persistent kernel keeps the cooperative launch, which needs no event)
+  g_no_setup_objects = true;
+  rc = fwd_calls(&call, 1, T, B, n, dtype, mode, ws, (size_t)RTN_STATIC_SCRATCH_BYTES, hip_stream, 0, 0, /*no_graph=*/true);
+  g_no_setup_objects = false;
+  return rc;
 }
 
 int rtn_native_lstm2_fwd_multi(const rtn_lstm2_call* calls, int32_t count, int64_t T, int32_t B, int32_t n,
