@@ -397,7 +397,7 @@ const char* rtn_native_lstm2_bwd_plan_text(void);
  */
 void rtn_native_lstm2_reload_env(void);
 
-/* ABI version of this header: 12. */
+/* ABI version of this header: 13. */
 int rtn_native_lstm2_abi_version(void);
 
 #ifdef __cplusplus

@@ -387,6 +387,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   const long long bn = (long long)p.B * n;
   const unsigned frame_bytes = (unsigned)((size_t)p.B * n4 * ES);
   const unsigned dx_frame_bytes = (unsigned)((size_t)p.B * p.ldDX * ES);
+  const long long dy_frame = (long long)p.B * p.ldDY;  // elements from one frame of DY to the next
   // the exchange ring of this group: kExRing frames of [4n/KM][4][Bp][16 bytes]
   const int Bp = q.Bp;
   const unsigned ex_frame = (unsigned)((size_t)n4 * Bp * ES), frag_stride = (unsigned)(64 * Bp);
@@ -433,8 +434,9 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
   const int upper = SPLIT ? ((tid & 255) >> 7) : 0;                // SPLIT: which of a pair of tiles
   auto tile_of = [&](int j) { return SPLIT ? set + TS * (2 * j + upper) : set + TS * j; };
   const int b = b_base + ((bl < rows) ? bl : 0);
+  const long long dy_row = (long long)b * (p.ldDY - n);  // element idx = b*n + k of a contiguous array sits at dy_row + idx in DY
   bool act[PT];  // the pair exists: the tile does, and the group has the row
-  long long idx[PT], io[PT], dyo[PT];
+  long long idx[PT], io[PT];
   float dyw[PT], dc[PT], dx0[PT][4];
 #pragma unroll
   for (int j = 0; j < PT; ++j) {
@@ -443,7 +445,6 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
     const int k = k0 + 16 * ((mt < MT) ? mt : 0) + kl;
     idx[j] = (long long)b * n + k;
     io[j] = (long long)b * n4 + k;
-    dyo[j] = (long long)b * p.ldDY + k;
     dyw[j] = 0.f;
     dc[j] = act[j] ? q.Dd[idx[j]] : 0.f;
 #pragma unroll
@@ -481,7 +482,7 @@ __global__ __launch_bounds__(64 * WV) void k_lstm2_bwd_regw(const Lstm2BwdMulti 
       const long long fo = t * bn * 4 + io[j];
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) nx_gate[j][gq] = ((const RawT*)p.H)[fo + (long long)gq * n];
-      nx_dy[j] = ((const RawT*)p.DY)[t * p.B * p.ldDY + dyo[j]];
+      nx_dy[j] = ((const RawT*)p.DY)[dy_frame * t + dy_row + idx[j]];
       nx_pc[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_c, (unsigned)(idx[j] * 4), 0, 0);
       if constexpr (ES == 2)
         nx_ph[j] = __builtin_amdgcn_raw_buffer_load_b16(rs_ph, (unsigned)(io[j] * ES), 0, 0);

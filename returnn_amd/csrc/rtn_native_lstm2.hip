@@ -1562,7 +1562,7 @@ using namespace rtn;
 
 extern "C" {
 
-int rtn_native_lstm2_abi_version(void) { return 12; }
+int rtn_native_lstm2_abi_version(void) { return 13; }
 
 const char* rtn_native_lstm2_bwd_plan_text(void) { return g_bwd_plan_text.c_str(); }
 

@@ -31,7 +31,7 @@ MODE_PERSISTENT = 1
 MODE_GRAPH = 2
 MODE_STEPWISE = 3
 # The ABI version the structs and argument lists below were written for (rtn_native_lstm2_abi_version()).
-EXPECTED_ABI = 12
+EXPECTED_ABI = 13
 
 MODES = {"auto": MODE_AUTO, "persistent": MODE_PERSISTENT, "graph": MODE_GRAPH, "stepwise": MODE_STEPWISE}
 
