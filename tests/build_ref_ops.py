@@ -1,6 +1,8 @@
 """
-Test infrastructure, never shipped with the library: builds seven of the reference's OTHER native ops for gfx950 through
-this package's op loader, so that the GPU tests can run them against the known answers the reference's own tests hold.
+Test infrastructure, never shipped with the library: builds ten of the reference's native ops for gfx950 through this
+package's op loader -- seven of its OTHER ops, and its three LSTM ops with the gradient ops the loader derives for them --
+so that the GPU tests can run them against the known answers the reference's own tests hold and against the committed
+golden vectors.
 
 The op descriptions are read as text where they lie (``/root/reference/returnn/native_op.py``, parsed with :mod:`ast` by
 ``tests/_reference_op_sources.py``; nothing of the reference is imported or executed), the loader generates the unit and
@@ -30,7 +32,10 @@ OUT_DIR = os.path.join(HERE, "_built_ref_ops")
 # ops whose expected results the reference's tests hold as numbers (tests/test_torch_native_op.py:95-160, :582-631,
 # :689-812, :922-1034, :1036-1400)
 OPS = ("FastBaumWelchOp", "FastViterbiOp", "EditDistanceOp", "OptimalCompletionEditDistanceOp",
-       "OptimalCompletionEditDistancePerSuccessorOp", "NextEditDistanceRowOp", "NextEditDistanceReduceOp")
+       "OptimalCompletionEditDistancePerSuccessorOp", "NextEditDistanceRowOp", "NextEditDistanceReduceOp",
+       "NativeLstm2", "LstmGenericBase", "LstmLowMem")
+# of these also the gradient op that the loader derives from c_bw_code and grad_input_map ("GradOf<name>")
+WITH_GRADIENT = ("NativeLstm2", "LstmGenericBase", "LstmLowMem")
 
 
 def _plain(x):
@@ -65,6 +70,14 @@ def build(ops=OPS, out_dir: str = OUT_DIR, verbose: bool = True) -> bool:
             table[name] = {"in_info": _plain(fields["in_info"]), "out_info": _plain(fields["out_info"])}
             if verbose:
                 print("build_ref_ops: %s -> %s" % (name, os.path.join(out_dir, name + ".so")))
+            if name in WITH_GRADIENT:
+                grad = op_loader.grad_description(ref_sources.as_description(name, fields))
+                gname, g_in, g_out = op_loader.description_fields(grad)[:3]
+                gop = op_loader.compile_op(grad, compiler_opts={"cache_dir": tmp})
+                shutil.copyfile(gop.compiler.so_filename, os.path.join(out_dir, gname + ".so"))
+                table[gname] = {"in_info": _plain(g_in), "out_info": _plain(g_out)}
+                if verbose:
+                    print("build_ref_ops: %s -> %s" % (gname, os.path.join(out_dir, gname + ".so")))
     with open(os.path.join(out_dir, "ops.json"), "w") as f:
         json.dump(table, f, indent=1, sort_keys=True)
     return True
