@@ -1835,52 +1835,63 @@ struct BwdJob {
   long long ldY;  // row pitch of Y in elements
 };
 
-// `count` gradient calls of one shape.  With the persistent kernel and count <= kMaxBwdMulti all of them share one
-// cooperative launch (16-row batch groups when 8-row groups of all problems would not find a CU each); otherwise they
-// are enqueued one after the other.
+// What all phases of one gradient entry share.
+struct BwdCtx {
+  const rtn_lstm2_bwd_call* calls;
+  int count;
+  int64_t T;
+  int B, n, dtype, op_flags;
+  hipStream_t stream;
+  bool capturing;
+  size_t es;     // bytes per activation element
+  long long bn;  // B * n
+};
+
+// The persistent kernel and decomposition of a gradient entry (kernel == nullptr: launches per frame).
+struct BwdChoice {
+  const void* kernel = nullptr;
+  int ksb = 0;                 // macro steps of the contraction per wavefront
+  int tiles = 1;               // tiles of 16 values of k per workgroup
+  int waves = kWaves;          // wavefronts per workgroup
+  int rows_per_group = 16;     // batch rows per group
+  int groups_per_launch = 0;   // batch groups of every problem that one launch takes
+  bool local = false;          // every group on one XCD
+  size_t lds = 0;              // dynamic shared memory of the kernel
+};
+
 int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, int32_t n, int32_t dtype, void* workspace,
-              size_t workspace_bytes, void* hip_stream, int op_flags = 0, size_t ws_stride = 0) {
-  int rc = check_dims(T, B, n, dtype);
-  if (rc != RTN_OK) return rc;
-  if (count < 0 || (count > 0 && !calls)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: bad call list");
-  hipStream_t stream = (hipStream_t)hip_stream;
-  const long long bn = (long long)B * n;
-  const long long nn4 = (long long)n * n * 4;
-  hipStreamCaptureStatus cap_status = hipStreamCaptureStatusNone;
-  if (stream) RTN_HIP(hipStreamIsCapturing(stream, &cap_status));
-  // Under stream capture everything is recorded into the caller's graph: the persistent kernel as a kernel node of its
-  // own (launch_coresident) or one launch per frame, and the rocBLAS calls of the weight gradient (the library's rocBLAS
-  // handle must exist already: run the op once outside the capture first, as for any library that sets itself up on
-  // first use).
-  const bool capturing = cap_status != hipStreamCaptureStatusNone;
-  if (!capturing && T > 0 && bn > 0 && (rc = probe_xcds(stream)) != RTN_OK) return rc;
+              size_t workspace_bytes, void* hip_stream, int op_flags = 0, size_t ws_stride = 0);
+
+// Argument checks and the outputs that do not depend on the recurrence: DW := 0, Dc0 := Dd, and Dy0 := 0 where there is
+// no frame to run (returnn/native_op.py:1365-1370).
+int bwd_check_and_clear(const BwdCtx& x) {
+  const long long nn4 = (long long)x.n * x.n * 4;
   const dim3 fill_grid(256), fill_block(256);
-  for (int k = 0; k < count; ++k) {
-    const rtn_lstm2_bwd_call& c = calls[k];
+  for (int k = 0; k < x.count; ++k) {
+    const rtn_lstm2_bwd_call& c = x.calls[k];
     if (nn4 > 0 && !c.DW) return fail(RTN_ERR_ARG, "NativeLstm2 backward: DW must not be null");
-    if (bn > 0 && (!c.Dd || !c.Dy0 || !c.Dc0)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: Dd, Dy0 and Dc0 must not be null");
+    if (x.bn > 0 && (!c.Dd || !c.Dy0 || !c.Dc0)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: Dd, Dy0 and Dc0 must not be null");
   }
-  for (int k = 0; k < count; ++k) {
-    const rtn_lstm2_bwd_call& c = calls[k];
-    // returnn/native_op.py:1365-1370: DW := 0, Dy0 := 0, Dc0 := Dd
+  for (int k = 0; k < x.count; ++k) {
+    const rtn_lstm2_bwd_call& c = x.calls[k];
     if (nn4 > 0) {
-      hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)c.DW, 0u, nn4);
+      hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, x.stream, (unsigned*)c.DW, 0u, nn4);
       RTN_HIP(hipGetLastError());
     }
-    if (bn > 0) {
-      hipLaunchKernelGGL(k_copy_f32, fill_grid, fill_block, 0, stream, c.Dd, c.Dc0, bn);
+    if (x.bn > 0) {
+      hipLaunchKernelGGL(k_copy_f32, fill_grid, fill_block, 0, x.stream, c.Dd, c.Dc0, x.bn);
       RTN_HIP(hipGetLastError());
     }
-    if ((T == 0 || bn == 0) && bn > 0) {
-      hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)c.Dy0, 0u, (long long)(((size_t)bn * esize(dtype) + 3) / 4));
+    if ((x.T == 0 || x.bn == 0) && x.bn > 0) {
+      hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, x.stream, (unsigned*)c.Dy0, 0u, (long long)(((size_t)x.bn * x.es + 3) / 4));
       RTN_HIP(hipGetLastError());
     }
   }
-  if (T == 0 || bn == 0 || count == 0) return RTN_OK;
-  for (int k = 0; k < count; ++k) {
-    const rtn_lstm2_bwd_call& c = calls[k];
-    if (c.start < 0 || c.start >= T)
-      return fail(RTN_ERR_RANGE, "NativeLstm2 backward: need 0 <= start < T, got start=%d, T=%lld", c.start, (long long)T);
+  if (x.T == 0 || x.bn == 0 || x.count == 0) return RTN_OK;
+  for (int k = 0; k < x.count; ++k) {
+    const rtn_lstm2_bwd_call& c = x.calls[k];
+    if (c.start < 0 || c.start >= x.T)
+      return fail(RTN_ERR_RANGE, "NativeLstm2 backward: need 0 <= start < T, got start=%d, T=%lld", c.start, (long long)x.T);
     if (c.step == 0) return fail(RTN_ERR_RANGE, "NativeLstm2 backward: step must not be 0");
     const void* ptrs[] = {c.W, c.y0, c.c0, c.i, c.Y, c.C, c.H, c.DY, c.Dd, c.DX, c.DW, c.Dy0, c.Dc0};
     const char* names[] = {"W", "y0", "c0", "i", "Y", "C", "H", "DY", "Dd", "DX", "DW", "Dy0", "Dc0"};
@@ -1888,56 +1899,424 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
       if (!ptrs[q]) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must not be null", names[q]);
       // (W is read in 16-byte fragments only where n is a multiple of 16; the recurrent rows of a stacked matrix start at
       // a multiple of 4n elements, which is aligned then)
-      if (q != 3 && !(q == 0 && n % 16 != 0) && !aligned16(ptrs[q])) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must be 16-byte aligned", names[q]);
+      if (q != 3 && !(q == 0 && x.n % 16 != 0) && !aligned16(ptrs[q])) return fail(RTN_ERR_ARG, "NativeLstm2 backward: %s must be 16-byte aligned", names[q]);
     }
   }
-  const int np = padded_width(n);
-  if (np != n) {
-    // Run the problem zero-padded to a width the matrix-core kernels take (see padded_width), on copies in the
-    // workspace: slice k = the workspace of the padded call k, then its copies.
-    const BwdLayout lay_p = bwd_layout(B, np, dtype);
-    const BwdPadLayout L = bwd_pad_layout(T, B, np, dtype);
-    const size_t each = lay_p.total + L.total;
-    const size_t need = (size_t)count * each;
-    if (!workspace || workspace_bytes < need)
-      return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
-    if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: workspace must be 16-byte aligned");
-    const size_t es = esize(dtype);
-    const long long tb = (long long)T * B;
-    std::vector<rtn_lstm2_bwd_call> padded((size_t)count);
-    for (int k = 0; k < count; ++k) {
-      const rtn_lstm2_bwd_call& c = calls[k];
-      unsigned char* base = (unsigned char*)workspace + (size_t)k * each + lay_p.total;
-      if ((rc = launch_pad(c.W, base + L.W, n, np, 4, n, np, es, stream)) != RTN_OK) return rc;
-      if ((rc = launch_pad(c.y0, base + L.y0, B, B, 1, n, np, es, stream)) != RTN_OK) return rc;
-      if ((rc = launch_pad(c.c0, base + L.c0, B, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
-      long long ldY = 0, ldDY = 0, ldDX = 0;
-      if ((rc = resolve_pitch("ldY", c.ldY, n, B, es, &ldY)) != RTN_OK) return rc;
-      if ((rc = resolve_pitch("ldDY", c.ldDY, n, B, es, &ldDY)) != RTN_OK) return rc;
-      if ((rc = resolve_pitch("ldDX", c.ldDX, 4LL * n, B, es, &ldDX)) != RTN_OK) return rc;
-      if ((rc = launch_pad(c.Y, base + L.Y, tb, tb, 1, n, np, es, stream, ldY)) != RTN_OK) return rc;
-      // the sibling op that keeps its cell states in H hands H in for C as well; it is not read then
-      if (!(op_flags & kOpH0IsCell) && (rc = launch_pad(c.C, base + L.C, tb, tb, 1, n, np, 4, stream)) != RTN_OK) return rc;
-      if ((rc = launch_pad(c.H, base + L.H, tb, tb, 4, n, np, es, stream)) != RTN_OK) return rc;
-      if ((rc = launch_pad(c.DY, base + L.DY, tb, tb, 1, n, np, es, stream, ldDY)) != RTN_OK) return rc;
-      if ((rc = launch_pad(c.Dd, base + L.Dd, B, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
-      padded[(size_t)k] = {base + L.W, base + L.y0, (const float*)(base + L.c0), c.i, c.start, c.step, base + L.Y,
-                           (const float*)(base + ((op_flags & kOpH0IsCell) ? L.H : L.C)), base + L.H, base + L.DY,
-                           (const float*)(base + L.Dd), base + L.DX, (float*)(base + L.DW), base + L.Dy0, (float*)(base + L.Dc0),
-                           0, 0, 0};
+  return RTN_OK;
+}
+
+// The problem zero-padded to a width the matrix-core kernels take (see padded_width), on copies in the workspace: slice
+// k = the workspace of the padded call k, then its copies.
+int bwd_padded(const BwdCtx& x, int np, void* workspace, size_t workspace_bytes) {
+  const int n = x.n, B = x.B;
+  const BwdLayout lay_p = bwd_layout(B, np, x.dtype);
+  const BwdPadLayout L = bwd_pad_layout(x.T, B, np, x.dtype);
+  const size_t each = lay_p.total + L.total;
+  const size_t need = (size_t)x.count * each;
+  if (!workspace || workspace_bytes < need)
+    return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
+  if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: workspace must be 16-byte aligned");
+  const size_t es = x.es;
+  const long long tb = (long long)x.T * B;
+  int rc = RTN_OK;
+  std::vector<rtn_lstm2_bwd_call> padded((size_t)x.count);
+  for (int k = 0; k < x.count; ++k) {
+    const rtn_lstm2_bwd_call& c = x.calls[k];
+    unsigned char* base = (unsigned char*)workspace + (size_t)k * each + lay_p.total;
+    if ((rc = launch_pad(c.W, base + L.W, n, np, 4, n, np, es, x.stream)) != RTN_OK) return rc;
+    if ((rc = launch_pad(c.y0, base + L.y0, B, B, 1, n, np, es, x.stream)) != RTN_OK) return rc;
+    if ((rc = launch_pad(c.c0, base + L.c0, B, B, 1, n, np, 4, x.stream)) != RTN_OK) return rc;
+    long long ldY = 0, ldDY = 0, ldDX = 0;
+    if ((rc = resolve_pitch("ldY", c.ldY, n, B, es, &ldY)) != RTN_OK) return rc;
+    if ((rc = resolve_pitch("ldDY", c.ldDY, n, B, es, &ldDY)) != RTN_OK) return rc;
+    if ((rc = resolve_pitch("ldDX", c.ldDX, 4LL * n, B, es, &ldDX)) != RTN_OK) return rc;
+    if ((rc = launch_pad(c.Y, base + L.Y, tb, tb, 1, n, np, es, x.stream, ldY)) != RTN_OK) return rc;
+    // the sibling op that keeps its cell states in H hands H in for C as well; it is not read then
+    if (!(x.op_flags & kOpH0IsCell) && (rc = launch_pad(c.C, base + L.C, tb, tb, 1, n, np, 4, x.stream)) != RTN_OK) return rc;
+    if ((rc = launch_pad(c.H, base + L.H, tb, tb, 4, n, np, es, x.stream)) != RTN_OK) return rc;
+    if ((rc = launch_pad(c.DY, base + L.DY, tb, tb, 1, n, np, es, x.stream, ldDY)) != RTN_OK) return rc;
+    if ((rc = launch_pad(c.Dd, base + L.Dd, B, B, 1, n, np, 4, x.stream)) != RTN_OK) return rc;
+    padded[(size_t)k] = {base + L.W, base + L.y0, (const float*)(base + L.c0), c.i, c.start, c.step, base + L.Y,
+                         (const float*)(base + ((x.op_flags & kOpH0IsCell) ? L.H : L.C)), base + L.H, base + L.DY,
+                         (const float*)(base + L.Dd), base + L.DX, (float*)(base + L.DW), base + L.Dy0, (float*)(base + L.Dc0),
+                         0, 0, 0};
+  }
+  rc = bwd_calls(padded.data(), x.count, x.T, B, np, x.dtype, workspace, need, (void*)x.stream, x.op_flags, each);
+  if (rc != RTN_OK) return rc;
+  for (int k = 0; k < x.count; ++k) {
+    const rtn_lstm2_bwd_call& c = x.calls[k];
+    const rtn_lstm2_bwd_call& q = padded[(size_t)k];
+    if ((rc = launch_unpad(q.DX, c.DX, tb, 4, n, np, es, x.stream, c.ldDX)) != RTN_OK) return rc;
+    if ((rc = launch_unpad(q.DW, c.DW, n, 4, n, np, 4, x.stream)) != RTN_OK) return rc;
+    if ((rc = launch_unpad(q.Dy0, c.Dy0, B, 1, n, np, es, x.stream)) != RTN_OK) return rc;
+    if ((rc = launch_unpad(q.Dc0, c.Dc0, B, 1, n, np, 4, x.stream)) != RTN_OK) return rc;
+  }
+  return RTN_OK;
+}
+
+// Persistent kernel: W in registers for the whole call, if a wavefront's share of the 16 x 4n slice fits (2..32
+// fragments, 64 with half of them in LDS) and all workgroups of all problems can be on the device together.
+// Decomposition: batch groups of 4, 8 or 16 rows (a workgroup's frame time grows with the rows x 4n derivatives it reads
+// per frame from the exchange ring), 1, 2 or 4 tiles of 16 values of k per workgroup (more tiles: fewer workgroups, more
+// MFMA time each) and 4 or 8 wavefronts per workgroup.  Leaves out->kernel null where no candidate fits.
+int choose_bwd_kernel(const BwdCtx& x, BwdChoice* out) {
+  const int n = x.n, B = x.B, dtype = x.dtype, count = x.count;
+  int rc = RTN_OK;
+  BwdChoice best, turn;  // turn: the candidate that takes most rows per launch, for batches that need several launches
+  long long turn_rows = 0;
+  const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
+  const int S = 4 * n / KM;
+  const long env_rows = env_long("RTN_LSTM2_BWD_ROWS", 0);
+  const long env_mt = env_long("RTN_LSTM2_BWD_MT", 0);
+  const long env_waves = env_long("RTN_LSTM2_BWD_WAVES", 0);
+  // (rows per group, tiles per workgroup, wavefronts per workgroup, XCD-local only)
+  // Candidates in the order measured on MI355X (cfg3 bf16 n=1024, ms per gradient call: one problem 8 x 1 x 4: 2.73,
+  // 8 x 1 x 8: 3.04, 8 x 2 x 4 on one XCD per group: 3.2, 16 x 1 x 8: 3.6; two problems in one launch 8 x 2 x 4 on one
+  // XCD per group: 3.53, spread: 3.78; cfg2 float32 n=512: 8 x 1 x 4 on one XCD per group 2.35, spread 2.56, 8 x 1 x 8:
+  // 2.55 / 2.79, 8 x 2 x 4: 3.4); the first whose workgroups are all on the device together.  A candidate whose groups
+  // fit an XCD each (n / (16 * tiles) workgroups, all groups of all problems in one launch) runs XCD-local: the ring
+  // then goes from writer to readers through that XCD's L2 instead of through memory.
+  // In front of them, for bf16 only and only where its groups fit an XCD each: 4 rows x 2 tiles, the kernel with one
+  // (row, k) pair per thread (one problem of cfg3: 4.82 ms against 5.03 for 8 x 1 x 4, whose groups of 64 workgroups
+  // span two XCDs; in float32 two tiles double an MFMA time that is long already: cfg2 3.1 ms against 2.3).
+  const int candidates[][4] = {{4, 2, 4, 1}, {8, 1, 4, 0}, {8, 1, 8, 0}, {8, 2, 4, 0}, {16, 1, 4, 0}, {16, 1, 8, 0}, {16, 2, 4, 0}, {8, 4, 4, 0}, {16, 4, 4, 0}};
+  const DeviceInfo di = device_info();
+  const long want_local = env_long("RTN_LSTM2_BWD_LOCAL", 1);
+  for (const auto& cand : candidates) {
+    const int rows = cand[0], mt = cand[1];
+    const int wv = env_waves ? (int)env_waves : cand[2];
+    const bool local_only = cand[3] != 0;
+    if (local_only && (dtype != RTN_DTYPE_BF16 || env_mt || env_waves || (env_rows >= 1 && env_rows <= 16))) continue;
+    if (env_mt && mt != env_mt) continue;
+    const bool rows_forced = env_rows >= 1 && env_rows <= 16;  // an explicit row count replaces the candidates' own
+    if (rows_forced && rows != 8) continue;                    // (one pass per MT is enough then)
+    const int use_rows = rows_forced ? (int)env_rows : rows;
+    if (wv != 4 && wv != 8 && wv != 16) continue;
+    const int ksb = (S + wv - 1) / wv;  // macro steps per wavefront; the kernel has room for the next power of two
+    int ksb_room = 2;
+    while (ksb_room < ksb) ksb_room *= 2;
+    if (mt * ksb_room > 64 || (n / 16) % mt) continue;
+    // A share of 64 fragments does not fit the registers next to a frame's DX (with all of it in registers the compiler
+    // spills part of W, in float32 most of it): half of it lives in LDS.
+    const bool lds_share = ksb_room * wv == 256;
+    if (lds_share && (mt != 1 || (wv != 4 && wv != 8))) continue;
+    BwdRegwKernel kfn;
+    if (lds_share)
+      kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_lds_table_bf16(wv) : bwd_regw_lds_table_f32(wv);
+    else
+      // ring frames of 8 rows: the variant whose loads take two macro steps at once
+      kfn = use_rows <= 8 ? (dtype == RTN_DTYPE_BF16 ? bwd_regw_table_bf16_half(ksb_room, mt, wv) : bwd_regw_table_f32_half(ksb_room, mt, wv))
+                          : (dtype == RTN_DTYPE_BF16 ? bwd_regw_table_bf16_full(ksb_room, mt, wv) : bwd_regw_table_f32_full(ksb_room, mt, wv));
+    if (!kfn) continue;
+    BwdChoice c;
+    c.kernel = (const void*)kfn;
+    c.ksb = ksb;
+    c.tiles = mt;
+    c.waves = wv;
+    c.rows_per_group = use_rows;
+    c.lds = lds_share ? kBwdLdsShareBytes : 0;
+    if (c.lds && (rc = ensure_lds_limit(c.kernel, c.lds)) != RTN_OK) return rc;
+    int per_cu = 0;
+    if ((rc = occupancy_per_cu(c.kernel, 64 * wv, c.lds, &per_cu)) != RTN_OK) return rc;
+    const long long groups_needed = (B + use_rows - 1) / use_rows;
+    const long long G_wgs = n / (16 * mt), cu_x = di.xcds > 0 ? di.cus / di.xcds : 0;
+    if (local_only && n / 16 <= cu_x * per_cu) continue;  // (groups of one tile per workgroup fit an XCD themselves)
+    if (local_only && 2 * (long long)count * groups_needed * G_wgs < di.cus) continue;  // (few rows: the wider spread wins, cfg5 7.98 against 8.41 ms)
+    const bool fits_xcd = want_local && di.xcds > 1 && per_cu >= 1 && G_wgs <= cu_x * per_cu;
+    if (fits_xcd && (long long)di.xcds * ((cu_x * per_cu) / G_wgs) >= (long long)count * groups_needed) {
+      c.groups_per_launch = (int)groups_needed;
+      c.local = true;
+      best = c;
+      break;
     }
-    rc = bwd_calls(padded.data(), count, T, B, np, dtype, workspace, need, hip_stream, op_flags, each);
-    if (rc != RTN_OK) return rc;
+    if (local_only) continue;
+    // batch groups of every problem that one launch can hold
+    const long long fit = (long long)per_cu * di.cus / ((long long)count * G_wgs);
+    if (fit >= groups_needed) {
+      c.groups_per_launch = (int)groups_needed;
+      best = c;
+      break;
+    }
+    // Too many rows for one launch: remember the candidate that takes most rows per launch; the batch groups
+    // then run in turns (the rows of a batch are independent of each other).  A turn whose groups fit an XCD each
+    // is an XCD-local launch, unless that costs more than an eighth of the groups a launch can hold.
+    const long long fit_local = fits_xcd ? (long long)di.xcds * ((cu_x * per_cu) / G_wgs) / count : 0;
+    const bool local_turns = fit_local >= 1 && fit_local * 8 >= fit * 7;
+    const long long turn_fit = local_turns ? fit_local : fit;
+    if (turn_fit >= 1 && turn_fit * use_rows > turn_rows &&
+        (groups_needed + turn_fit - 1) / turn_fit <= env_long("RTN_LSTM2_MAX_PASSES", kMaxPassesOverSteps)) {
+      turn_rows = turn_fit * use_rows;
+      c.groups_per_launch = (int)turn_fit;
+      c.local = local_turns;
+      turn = c;
+    }
+  }
+  *out = best.kernel ? best : turn;
+  return RTN_OK;
+}
+
+// Fills in the kernels' parameter blocks: buffers, pitches, the frames the forward pass visited (returnn/native_op.py:
+// 1383-1407), and puts each call's workspace slice into its starting state.
+int bwd_prepare_jobs(const BwdCtx& x, const BwdChoice& ch, const BwdLayout& lay, void* workspace, size_t stride, std::vector<BwdJob>* jobs) {
+  const int n = x.n, B = x.B;
+  const int64_t T = x.T;
+  const int bgroups = (B + ch.rows_per_group - 1) / ch.rows_per_group;
+  const dim3 fill_grid(256), fill_block(256);
+  int rc = RTN_OK;
+  jobs->assign((size_t)x.count, BwdJob());
+  for (int k = 0; k < x.count; ++k) {
+    const rtn_lstm2_bwd_call& c = x.calls[k];
+    BwdJob& j = (*jobs)[(size_t)k];
+    Lstm2BwdParams& p = j.p;
+    memset(&p, 0, sizeof(p));
+    p.W = c.W; p.c0 = c.c0; p.mask = c.i; p.C = c.C; p.H = c.H; p.DY = c.DY;
+    p.DX = c.DX; p.Dc0 = c.Dc0;
+    j.ws = (unsigned char*)workspace + (size_t)k * stride;
+    p.dyw = (float*)(j.ws + lay.off_dyw);
+    p.dx0 = j.ws + lay.off_dx0;
+    p.T = T; p.B = B; p.n = n;
+    p.op_flags = x.op_flags;
+    if ((rc = resolve_pitch("ldY", c.ldY, n, B, x.es, &j.ldY)) != RTN_OK) return rc;
+    if ((rc = resolve_pitch("ldDY", c.ldDY, n, B, x.es, &p.ldDY)) != RTN_OK) return rc;
+    if ((rc = resolve_pitch("ldDX", c.ldDX, 4LL * n, B, x.es, &p.ldDX)) != RTN_OK) return rc;
+    hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, x.stream, (unsigned*)j.ws, 0u, (long long)(lay.off_wpk / 4));
+    RTN_HIP(hipGetLastError());
+    j.abs_step = c.step > 0 ? c.step : -(long long)c.step;
+    j.num_steps = (T - c.start + j.abs_step - 1) / j.abs_step;
+    j.first = c.step > 0 ? c.start : T - c.start - 1;
+    if ((x.op_flags & kOpEndAtStart) && c.step < 0) {
+      // LstmLowMem: with a negative step the frames from T-start-1 down to `start` (returnn/native_op.py:957-963)
+      if (j.first < c.start) return fail(RTN_ERR_RANGE, "LstmLowMem gradient: start=%d with a negative step visits no frame of T=%lld", c.start, (long long)T);
+      j.num_steps = (j.first - c.start) / j.abs_step + 1;
+    }
+    j.end = j.first + (j.num_steps - 1) * c.step;  // inclusive
+    if (ch.kernel) {
+      // the exchange ring starts armed: all-ones words (the visited frames of DX are written by the kernel, the others
+      // zeroed behind it)
+      const int bp = ch.rows_per_group > 8 ? 16 : 8;
+      const long long ring_words = (long long)((size_t)bgroups * kExRing * 4 * n * x.es * bp / 4);
+      if ((size_t)ring_words * 4 > lay.total - lay.off_ex)
+        return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: internal: exchange ring of %lld bytes does not fit its section", ring_words * 4);
+      hipLaunchKernelGGL(k_fill_u32, dim3(256), fill_block, 0, x.stream, (unsigned*)(j.ws + lay.off_ex), 0xFFFFFFFFu, ring_words);
+      RTN_HIP(hipGetLastError());
+    } else if (j.num_steps != T) {
+      // frames the loop does not visit keep DX = 0 (:1385-1388): all rows cleared here, row by row
+      if ((rc = launch_clear_rows(c.DX, (long long)T * B, 4LL * n, p.ldDX, x.es, x.stream)) != RTN_OK) return rc;
+    }
+  }
+  return RTN_OK;
+}
+
+// The recurrence of all problems on the persistent kernel: one launch per share of the batch groups (a single one unless
+// the batch is too large for the device), then DX := 0 on the frames the forward pass did not visit.
+int bwd_launch_persistent(const BwdCtx& x, const BwdChoice& ch, const BwdLayout& lay, const std::vector<BwdJob>& jobs) {
+  const int n = x.n, B = x.B, count = x.count;
+  const int bgroups = (B + ch.rows_per_group - 1) / ch.rows_per_group;
+  const dim3 fill_block(256);
+  Lstm2BwdMulti multi;
+  memset(&multi, 0, sizeof(multi));
+  multi.count = count;
+  for (int k = 0; k < count; ++k) {
+    Lstm2BwdPersistent& q = multi.q[k];
+    const BwdJob& j = jobs[(size_t)k];
+    q.p = j.p;
+    q.Dd = x.calls[k].Dd;
+    q.Dy0 = x.calls[k].Dy0;
+    q.status = (unsigned*)j.ws;
+    q.t_end = j.end;
+    q.step = x.calls[k].step;
+    q.nframes = (int)j.num_steps;
+    q.Bg = (B + bgroups - 1) / bgroups;
+    q.ksb = ch.ksb;
+    // The kernels that keep one (row, k) pair per thread ask for a frame's inputs in front of the MFMAs, so only the
+    // delay stands between a frame's stores and the read of its ring slot: inside an XCD it is a fixed one there, as in
+    // the forward kernel (measured: 2.77 ms at 10 units against 2.82 adaptive and 2.87 / 2.86 at 4 / 16 for the layer).
+    const bool one_pair = ch.rows_per_group <= 8 && ((ch.tiles + ch.waves / 4 - 1) / (ch.waves / 4)) % 2 == 0;
+    const bool fixed_delay = ch.local && one_pair;
+    q.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_BWD_POLL_DELAY", fixed_delay ? 10 : 20)));
+    q.delay_inc = (int)std::max<long>(0, std::min<long>(16, env_long("RTN_LSTM2_BWD_DELAY_INC", fixed_delay ? 0 : 2)));
+    {
+      long dec = env_long("RTN_LSTM2_BWD_DELAY_DEC", 16);  // steps per unit of downward adaptation: a power of two
+      int mask = 0;
+      while (2 * (mask + 1) <= dec && mask < 255) mask = 2 * mask + 1;
+      q.delay_dec_mask = mask;
+    }
+    q.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);
+    q.sync = (unsigned*)(j.ws + lay.off_sync);
+    q.ex = j.ws + lay.off_ex;
+    q.Bp = ch.rows_per_group > 8 ? 16 : 8;
+    q.bp_shift = ch.rows_per_group > 8 ? 4 : 3;
+  }
+  multi.local = ch.local ? 1 : 0;
+  multi.xcds = device_info().xcds;
+  const int wgs_per_group = n / (16 * ch.tiles);
+  for (int g0 = 0; g0 < bgroups; g0 += ch.groups_per_launch) {
+    const int groups_now = std::min(ch.groups_per_launch, bgroups - g0);
+    multi.wgs_each = groups_now * wgs_per_group;
     for (int k = 0; k < count; ++k) {
-      const rtn_lstm2_bwd_call& c = calls[k];
-      const rtn_lstm2_bwd_call& q = padded[(size_t)k];
-      if ((rc = launch_unpad(q.DX, c.DX, tb, 4, n, np, es, stream, c.ldDX)) != RTN_OK) return rc;
-      if ((rc = launch_unpad(q.DW, c.DW, n, 4, n, np, 4, stream)) != RTN_OK) return rc;
-      if ((rc = launch_unpad(q.Dy0, c.Dy0, B, 1, n, np, es, stream)) != RTN_OK) return rc;
-      if ((rc = launch_unpad(q.Dc0, c.Dc0, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
+      multi.q[k].groups = groups_now;
+      multi.q[k].group_offset = g0;
+    }
+    void* args[] = {(void*)&multi};
+    unsigned grid = (unsigned)(count * multi.wgs_each);
+    if (ch.local) {
+      // workgroup id = slot * xcds + xcd: the groups of the launch are dealt round-robin to the XCDs
+      const int total_groups = count * groups_now;
+      grid = (unsigned)(multi.xcds * wgs_per_group * ((total_groups + multi.xcds - 1) / multi.xcds));
+    }
+    const int rc = launch_coresident(ch.kernel, dim3(grid), dim3((unsigned)(64 * ch.waves)), args, (unsigned)ch.lds, x.stream, x.capturing);
+    if (rc != RTN_OK) return rc;
+  }
+  for (int k = 0; k < count; ++k) {
+    const BwdJob& j = jobs[(size_t)k];
+    if (j.num_steps == x.T) continue;
+    const long long row_words = (long long)((size_t)n * 4 * x.es / 4), pitch_words = (long long)((size_t)j.p.ldDX * x.es / 4);
+    if (x.dtype == RTN_DTYPE_BF16)
+      hipLaunchKernelGGL(k_bwd_zero_unvisited<__bf16>, dim3(1024), fill_block, 0, x.stream, x.calls[k].DX, (long long)x.T, (long long)B, row_words,
+                         pitch_words, j.first, (long long)x.calls[k].step, j.num_steps);
+    else
+      hipLaunchKernelGGL(k_bwd_zero_unvisited<float>, dim3(1024), fill_block, 0, x.stream, x.calls[k].DX, (long long)x.T, (long long)B, row_words,
+                         pitch_words, j.first, (long long)x.calls[k].step, j.num_steps);
+    RTN_HIP(hipGetLastError());
+  }
+  return RTN_OK;
+}
+
+// The recurrence of ONE problem as launches per frame, in reverse processing order.  MFMA shapes: one fused launch per
+// frame (the GEMM of the frame processed before, then this frame's pointwise part) and a last GEMM-only launch; other
+// shapes: a pointwise and a generic GEMM launch per frame.  Replayed through a library-owned graph outside capture.
+int bwd_launch_per_frame(const BwdCtx& x, bool mfma, const BwdLayout& lay, BwdJob& j) {
+  const int n = x.n, B = x.B, dtype = x.dtype;
+  hipStream_t stream = x.stream;
+  if (mfma && env_long("RTN_LSTM2_BWD_PACK_W", 1)) {
+    // every launch uses each fragment of W once: read them from a copy in fragment order (see k_bwd_pack_w)
+    j.p.Wpk = j.ws + lay.off_wpk;
+    const long long frags = (long long)(n / 16) * (4 * n / (dtype == RTN_DTYPE_BF16 ? 32 : 16)) * 64;
+    const dim3 pgrid((unsigned)std::min<long long>((frags + 255) / 256, 4096)), pblock(256);
+    if (dtype == RTN_DTYPE_BF16)
+      hipLaunchKernelGGL(k_bwd_pack_w<__bf16>, pgrid, pblock, 0, stream, x.calls[0].W, (void*)j.p.Wpk, n);
+    else
+      hipLaunchKernelGGL(k_bwd_pack_w<float>, pgrid, pblock, 0, stream, x.calls[0].W, (void*)j.p.Wpk, n);
+    RTN_HIP(hipGetLastError());
+  }
+  const Lstm2BwdParams& p = j.p;
+  const int step = x.calls[0].step;
+  const long long first = j.first, end = j.end;
+  // Batch rows per workgroup (16 * NT): 32 if that still leaves every CU a workgroup (each batch tile reads W again),
+  // else 16 (measured: float32 n=1024 B=64 29 us per frame with 16 rows, 35 with 32; 64 rows were never faster).
+  int NT = B > 16 ? 2 : 1;
+  if (NT > 1 && (long long)(n / 16) * ((B + 16 * NT - 1) / (16 * NT)) < device_info().cus) NT = 1;
+  auto record = [&](LaunchSink& sink) -> int {
+    const dim3 pw_grid((unsigned)((x.bn + 255) / 256)), pw_block(256);
+    const dim3 mm_grid((unsigned)((n / 16) * ((B + 16 * NT - 1) / (16 * NT)))), mm_block(kWgThreads);
+    const bool bf = dtype == RTN_DTYPE_BF16;
+    long long t_done = -1;  // frame whose DX still has to go through the GEMM
+    for (long long t = end;; t -= step) {
+      const bool more = step > 0 ? t >= first : t <= first;
+      const bool right = more && (step > 0 ? (t - step >= first) : (t - step <= first));
+      const long long prev_t = right ? t - step : -1;
+      const long long tt = more ? t : -1;
+      int rc2 = RTN_OK;
+      if (mfma) {
+        void (*k)(Lstm2BwdParams, long long, long long, long long) =
+            bf ? (NT == 2 ? &k_bwd_step<__bf16, 2> : &k_bwd_step<__bf16, 1>) : (NT == 2 ? &k_bwd_step<float, 2> : &k_bwd_step<float, 1>);
+        rc2 = enqueue(sink, k, mm_grid, mm_block, 0, p, t_done, tt, prev_t);
+      } else if (more) {
+        rc2 = enqueue(sink, bf ? &k_bwd_pointwise<__bf16> : &k_bwd_pointwise<float>, pw_grid, pw_block, 0, p, t, prev_t);
+        if (rc2 == RTN_OK)
+          rc2 = enqueue(sink, bf ? &k_bwd_gemm_dy_generic<__bf16> : &k_bwd_gemm_dy_generic<float>, pw_grid, pw_block, 0, p, t);
+      }
+      if (rc2 != RTN_OK) return rc2;
+      if (!more) break;
+      t_done = t;
     }
     return RTN_OK;
+  };
+  if (x.capturing || env_long("RTN_LSTM2_BWD_NO_GRAPH", 0)) {
+    LaunchSink sink;
+    sink.stream = stream;
+    return record(sink);
   }
+  std::string key("bwd");
+  int dev = 0;
+  RTN_HIP(hipGetDevice(&dev));
+  Lstm2BwdParams shape = p;  // p was zeroed before it was filled in
+  shape.W = shape.H = shape.DY = shape.Wpk = nullptr;
+  shape.c0 = shape.mask = shape.C = nullptr;
+  shape.DX = shape.dx0 = nullptr;
+  shape.dyw = shape.Dc0 = nullptr;
+  key.append(reinterpret_cast<const char*>(&shape), sizeof(shape));
+  key_append(&key, (int)(p.Wpk != nullptr));
+  key_append(&key, dtype); key_append(&key, (int)x.calls[0].start); key_append(&key, step); key_append(&key, dev);
+  key_append(&key, (int)mfma); key_append(&key, NT);
+  return replay_graph(key, &p, sizeof(p), stream, record);
+}
+
+// DW = sum over consecutive visited frames Y[t - step]^T * DX[t]  (returnn/native_op.py:1433-1452), then += y0^T * dx0
+// (:1456-1460), in rocBLAS; where the recurrence ran per frame, Dy0 from its float32 working copy.
+int bwd_weight_gradients(const BwdCtx& x, rocblas_handle blas, const std::vector<BwdJob>& jobs, bool persistent) {
+  const int n = x.n, B = x.B;
+  const dim3 fill_grid(256), fill_block(256);
+  int rc = RTN_OK;
+  for (int k = 0; k < x.count; ++k) {
+    const rtn_lstm2_bwd_call& c = x.calls[k];
+    const BwdJob& j = jobs[(size_t)k];
+    const int step = c.step;
+    const unsigned char* Yb = (const unsigned char*)c.Y;
+    const unsigned char* DXb = (const unsigned char*)c.DX;
+    if (j.num_steps > 1) {
+      if (j.abs_step == 1) {
+        const long long lo = std::min(j.first, j.end);
+        rc = dw_accumulate(blas, Yb + (size_t)(lo + std::max(0, -step)) * B * j.ldY * x.es,
+                           DXb + (size_t)(lo + std::max(0, step)) * B * j.p.ldDX * x.es, c.DW, (j.num_steps - 1) * B, n, x.dtype, j.ldY, j.p.ldDX);
+        if (rc != RTN_OK) return rc;
+      } else {
+        for (long long t = j.end - step; step > 0 ? t >= j.first : t <= j.first; t -= step) {
+          rc = dw_accumulate(blas, Yb + (size_t)t * B * j.ldY * x.es, DXb + (size_t)(t + step) * B * j.p.ldDX * x.es, c.DW, B, n, x.dtype, j.ldY,
+                             j.p.ldDX);
+          if (rc != RTN_OK) return rc;
+        }
+      }
+    }
+    rc = dw_accumulate(blas, c.y0, j.p.dx0, c.DW, B, n, x.dtype);
+    if (rc != RTN_OK) return rc;
+    if (!persistent) {
+      if (x.dtype == RTN_DTYPE_BF16)
+        hipLaunchKernelGGL(k_convert_from_f32<__bf16>, fill_grid, fill_block, 0, x.stream, j.p.dyw, c.Dy0, x.bn);
+      else
+        hipLaunchKernelGGL(k_convert_from_f32<float>, fill_grid, fill_block, 0, x.stream, j.p.dyw, c.Dy0, x.bn);
+      RTN_HIP(hipGetLastError());
+    }
+  }
+  return RTN_OK;
+}
+
+// `count` gradient calls of one shape.  With the persistent kernel and count <= kMaxBwdMulti all of them share one
+// launch (16-row batch groups when 8-row groups of all problems would not find a CU each); otherwise they are enqueued
+// one after the other.
+int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, int32_t n, int32_t dtype, void* workspace,
+              size_t workspace_bytes, void* hip_stream, int op_flags, size_t ws_stride) {
+  int rc = check_dims(T, B, n, dtype);
+  if (rc != RTN_OK) return rc;
+  if (count < 0 || (count > 0 && !calls)) return fail(RTN_ERR_ARG, "NativeLstm2 backward: bad call list");
+  BwdCtx x;
+  x.calls = calls; x.count = count; x.T = T; x.B = B; x.n = n; x.dtype = dtype; x.op_flags = op_flags;
+  x.stream = (hipStream_t)hip_stream;
+  x.es = esize(dtype);
+  x.bn = (long long)B * n;
+  hipStreamCaptureStatus cap_status = hipStreamCaptureStatusNone;
+  if (x.stream) RTN_HIP(hipStreamIsCapturing(x.stream, &cap_status));
+  // Under stream capture everything is recorded into the caller's graph: the persistent kernel as a kernel node of its
+  // own (launch_coresident) or one launch per frame, and the rocBLAS calls of the weight gradient (the library's rocBLAS
+  // handle must exist already: run the op once outside the capture first, as for any library that sets itself up on
+  // first use).
+  x.capturing = cap_status != hipStreamCaptureStatusNone;
+  if (!x.capturing && T > 0 && x.bn > 0 && (rc = probe_xcds(x.stream)) != RTN_OK) return rc;
+  if ((rc = bwd_check_and_clear(x)) != RTN_OK) return rc;
+  if (T == 0 || x.bn == 0 || count == 0) return RTN_OK;
+  const int np = padded_width(n);
+  if (np != n) return bwd_padded(x, np, workspace, workspace_bytes);
+
   const BwdLayout lay = bwd_layout(B, n, dtype);
   const size_t stride = ws_stride ? ws_stride : lay.total;  // distance between the calls' workspaces
   if (stride < lay.total) return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: internal: workspace slice %zu < layout %zu", stride, lay.total);
@@ -1948,369 +2327,41 @@ int bwd_calls(const rtn_lstm2_bwd_call* calls, int count, int64_t T, int32_t B, 
   rocblas_handle blas = nullptr;
   rc = blas_handle(&blas);
   if (rc != RTN_OK) return rc;
-  if (rocblas_set_stream(blas, stream) != rocblas_status_success) return fail(RTN_ERR_HIP, "NativeLstm2 backward: rocblas_set_stream failed");
-  const size_t es = esize(dtype);
+  if (rocblas_set_stream(blas, x.stream) != rocblas_status_success) return fail(RTN_ERR_HIP, "NativeLstm2 backward: rocblas_set_stream failed");
   const bool mfma = (n % 16) == 0 && !env_long("RTN_LSTM2_FORCE_GENERIC", 0);
 
-  // Persistent kernel: W in registers for the whole call, if a wavefront's share of the 16 x 4n slice fits
-  // (2..32 fragments) and all workgroups of all problems can be on the device together.
-  const void* pk = nullptr;
-  int KSB = 0, bwd_mt = 1;  // KSB: macro steps of the contraction per wavefront
-  // Decomposition: batch groups of 8 or 16 rows (a workgroup's frame time grows with the rows x 4n derivatives it
-  // reads per frame from the exchange ring), MT tiles of 16 values of k per workgroup (more tiles: fewer workgroups, more
-  // MFMA time each) and 4 or 8 wavefronts per workgroup.
-  const long env_rows = env_long("RTN_LSTM2_BWD_ROWS", 0);
-  int rows_per_group = 16, bwd_waves = kWaves, groups_per_launch = 0;
-  bool bwd_local = false, turn_local = false;
-  long long turn_rows = 0;
-  const void* turn_pk = nullptr;
-  int turn_cfg[5] = {0, 0, 0, 0, 0};
-  size_t bwd_lds = 0, turn_lds = 0;  // dynamic shared memory of the chosen kernel
-  {
-    const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
-    const int S = 4 * n / KM;
-    const long bwd_kernel = env_long("RTN_LSTM2_BWD_KERNEL", 0);  // 0 auto, 1 per-frame launches, 2 persistent
-    if (mfma && (4 * n) % KM == 0 && bwd_kernel != 1 && (!capturing || capture_keeps_persistent()) && device_info().cooperative && count <= kMaxBwdMulti) {
-      const long env_mt = env_long("RTN_LSTM2_BWD_MT", 0);
-      const long env_waves = env_long("RTN_LSTM2_BWD_WAVES", 0);
-      // (rows per group, tiles per workgroup, wavefronts per workgroup)
-      // Candidates in the order measured on MI355X (cfg3 bf16 n=1024, ms per gradient call: one problem 8 x 1 x 4: 2.73,
-      // 8 x 1 x 8: 3.04, 8 x 2 x 4 on one XCD per group: 3.2, 16 x 1 x 8: 3.6; two problems in one launch 8 x 2 x 4 on one
-      // XCD per group: 3.53, spread: 3.78; cfg2 float32 n=512: 8 x 1 x 4 on one XCD per group 2.35, spread 2.56, 8 x 1 x 8:
-      // 2.55 / 2.79, 8 x 2 x 4: 3.4); the first whose workgroups are all on the device together.  A candidate whose groups
-      // fit an XCD each (n / (16 * tiles) workgroups, all groups of all problems in one launch) runs XCD-local: the ring
-      // then goes from writer to readers through that XCD's L2 instead of through memory.
-      // In front of them, for bf16 only and only where its groups fit an XCD each: 4 rows x 2 tiles, the kernel with one
-      // (row, k) pair per thread (one problem of cfg3: 4.82 ms against 5.03 for 8 x 1 x 4, whose groups of 64 workgroups
-      // span two XCDs; in float32 two tiles double an MFMA time that is long already: cfg2 3.1 ms against 2.3).
-      const int candidates[][4] = {{4, 2, 4, 1}, {8, 1, 4, 0}, {8, 1, 8, 0}, {8, 2, 4, 0}, {16, 1, 4, 0}, {16, 1, 8, 0}, {16, 2, 4, 0}, {8, 4, 4, 0}, {16, 4, 4, 0}};
-      const DeviceInfo di_b = device_info();
-      const long want_local = env_long("RTN_LSTM2_BWD_LOCAL", 1);
-      for (const auto& cand : candidates) {
-        const int rows = cand[0], mt = cand[1];
-        const int wv = env_waves ? (int)env_waves : cand[2];
-        const bool local_only = cand[3] != 0;
-        if (local_only && (dtype != RTN_DTYPE_BF16 || env_mt || env_waves || (env_rows >= 1 && env_rows <= 16))) continue;
-        if (env_mt && mt != env_mt) continue;
-        const bool rows_forced = env_rows >= 1 && env_rows <= 16;  // an explicit row count replaces the candidates' own
-        if (rows_forced && rows != 8) continue;                    // (one pass per MT is enough then)
-        const int use_rows = rows_forced ? (int)env_rows : rows;
-        if (wv != 4 && wv != 8 && wv != 16) continue;
-        const int ksb = (S + wv - 1) / wv;  // macro steps per wavefront; the kernel has room for the next power of two
-        int ksb_room = 2;
-        while (ksb_room < ksb) ksb_room *= 2;
-        if (mt * ksb_room > 64 || (n / 16) % mt) continue;
-        // A share of 64 fragments does not fit the registers next to a frame's DX (with all of it in registers the compiler
-        // spills part of W, in float32 most of it): half of it lives in LDS.
-        const bool lds_share = ksb_room * wv == 256;
-        if (lds_share && (mt != 1 || (wv != 4 && wv != 8))) continue;
-        BwdRegwKernel kfn;
-        if (lds_share)
-          kfn = dtype == RTN_DTYPE_BF16 ? bwd_regw_lds_table_bf16(wv) : bwd_regw_lds_table_f32(wv);
-        else
-          // ring frames of 8 rows: the variant whose loads take two macro steps at once
-          kfn = use_rows <= 8 ? (dtype == RTN_DTYPE_BF16 ? bwd_regw_table_bf16_half(ksb_room, mt, wv) : bwd_regw_table_f32_half(ksb_room, mt, wv))
-                              : (dtype == RTN_DTYPE_BF16 ? bwd_regw_table_bf16_full(ksb_room, mt, wv) : bwd_regw_table_f32_full(ksb_room, mt, wv));
-        if (!kfn) continue;
-        const size_t cand_lds = lds_share ? kBwdLdsShareBytes : 0;
-        if (cand_lds) {
-          rc = ensure_lds_limit((const void*)kfn, cand_lds);
-          if (rc != RTN_OK) return rc;
-        }
-        int per_cu = 0;
-        if ((rc = occupancy_per_cu((const void*)kfn, 64 * wv, cand_lds, &per_cu)) != RTN_OK) return rc;
-        const long long groups_needed = (B + use_rows - 1) / use_rows;
-        const long long G_wgs = n / (16 * mt), cu_x = di_b.xcds > 0 ? di_b.cus / di_b.xcds : 0;
-        if (local_only && n / 16 <= cu_x * per_cu) continue;  // (groups of one tile per workgroup fit an XCD themselves)
-        if (local_only && 2 * (long long)count * groups_needed * G_wgs < di_b.cus) continue;  // (few rows: the wider spread wins, cfg5 7.98 against 8.41 ms)
-        if (want_local && di_b.xcds > 1 && per_cu >= 1 && G_wgs <= cu_x * per_cu &&
-            (long long)di_b.xcds * ((cu_x * per_cu) / G_wgs) >= (long long)count * groups_needed) {
-          pk = (const void*)kfn;
-          bwd_mt = mt;
-          bwd_waves = wv;
-          KSB = ksb;
-          rows_per_group = use_rows;
-          groups_per_launch = (int)groups_needed;
-          bwd_lds = cand_lds;
-          bwd_local = true;
-          break;
-        }
-        if (local_only) continue;
-        // batch groups of every problem that one launch can hold
-        const long long fit = (long long)per_cu * device_info().cus / ((long long)count * (n / (16 * mt)));
-        if (fit >= groups_needed) {
-          pk = (const void*)kfn;
-          bwd_mt = mt;
-          bwd_waves = wv;
-          KSB = ksb;
-          rows_per_group = use_rows;
-          groups_per_launch = (int)groups_needed;
-          bwd_lds = cand_lds;
-          break;
-        }
-        // Too many rows for one launch: remember the candidate that takes most rows per launch; the batch groups
-        // then run in turns (the rows of a batch are independent of each other).  A turn whose groups fit an XCD each
-        // is an XCD-local launch, unless that costs more than an eighth of the groups a launch can hold.
-        long long fit_local = 0;
-        if (want_local && di_b.xcds > 1 && per_cu >= 1 && G_wgs <= cu_x * per_cu)
-          fit_local = (long long)di_b.xcds * ((cu_x * per_cu) / G_wgs) / count;
-        const bool local_turns = fit_local >= 1 && fit_local * 8 >= fit * 7;
-        const long long turn_fit = local_turns ? fit_local : fit;
-        if (turn_fit >= 1 && turn_fit * use_rows > turn_rows &&
-            (groups_needed + turn_fit - 1) / turn_fit <= env_long("RTN_LSTM2_MAX_PASSES", kMaxPassesOverSteps)) {
-          turn_rows = turn_fit * use_rows;
-          turn_pk = (const void*)kfn;
-          turn_cfg[0] = use_rows; turn_cfg[1] = mt; turn_cfg[2] = wv; turn_cfg[3] = ksb; turn_cfg[4] = (int)turn_fit;
-          turn_lds = cand_lds;
-          turn_local = local_turns;
-        }
-      }
-      if (!pk && turn_pk) {
-        pk = turn_pk;
-        rows_per_group = turn_cfg[0];
-        bwd_mt = turn_cfg[1];
-        bwd_waves = turn_cfg[2];
-        KSB = turn_cfg[3];
-        groups_per_launch = turn_cfg[4];
-        bwd_lds = turn_lds;
-        bwd_local = turn_local;
-      }
+  BwdChoice ch;
+  const long bwd_kernel = env_long("RTN_LSTM2_BWD_KERNEL", 0);  // 0 auto, 1 per-frame launches, 2 persistent
+  const int KM = dtype == RTN_DTYPE_BF16 ? 32 : 16;
+  if (mfma && (4 * n) % KM == 0 && bwd_kernel != 1 && (!x.capturing || capture_keeps_persistent()) && device_info().cooperative && count <= kMaxBwdMulti)
+    if ((rc = choose_bwd_kernel(x, &ch)) != RTN_OK) return rc;
+  if (!ch.kernel && count > 1) {
+    // no joint launch: one call after the other, each with its own slice of the workspace
+    for (int k = 0; k < count; ++k) {
+      rc = bwd_calls(calls + k, 1, T, B, n, dtype, (unsigned char*)workspace + (size_t)k * stride, lay.total, hip_stream, op_flags);
+      if (rc != RTN_OK) return rc;
     }
-    if (!pk && count > 1) {
-      // no joint launch: one call after the other, each with its own slice of the workspace
-      for (int k = 0; k < count; ++k) {
-        rc = bwd_calls(calls + k, 1, T, B, n, dtype, (unsigned char*)workspace + (size_t)k * stride, lay.total, hip_stream, op_flags);
-        if (rc != RTN_OK) return rc;
-      }
-      return RTN_OK;
-    }
-    if (bwd_kernel == 2 && !pk)
-      return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2 backward: the persistent kernel cannot run T=%lld B=%d n=%d", (long long)T, B, n);
+    return RTN_OK;
   }
-  const int bgroups = (B + rows_per_group - 1) / rows_per_group;
+  if (bwd_kernel == 2 && !ch.kernel)
+    return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2 backward: the persistent kernel cannot run T=%lld B=%d n=%d", (long long)T, B, n);
   {
+    const int bgroups = (B + ch.rows_per_group - 1) / ch.rows_per_group;
     char buf[256];
-    if (pk)
+    if (ch.kernel)
       snprintf(buf, sizeof(buf), "kernel=%s problems=%d rows_per_group=%d groups=%d tiles=%d waves=%d wgs_per_group=%d launches=%d",
-               bwd_local ? "bwd_regw_xcd" : "bwd_regw", count, rows_per_group, bgroups, bwd_mt, bwd_waves, n / (16 * bwd_mt),
-               (bgroups + groups_per_launch - 1) / std::max(groups_per_launch, 1));
+               ch.local ? "bwd_regw_xcd" : "bwd_regw", count, ch.rows_per_group, bgroups, ch.tiles, ch.waves, n / (16 * ch.tiles),
+               (bgroups + ch.groups_per_launch - 1) / std::max(ch.groups_per_launch, 1));
     else
       snprintf(buf, sizeof(buf), "kernel=%s problems=%d launches_per_frame=%d", mfma ? "bwd_step" : "bwd_generic", count, mfma ? 1 : 2);
     g_bwd_plan_text = buf;
   }
 
-  std::vector<BwdJob> jobs((size_t)count);
-  for (int k = 0; k < count; ++k) {
-    const rtn_lstm2_bwd_call& c = calls[k];
-    BwdJob& j = jobs[(size_t)k];
-    Lstm2BwdParams& p = j.p;
-    memset(&p, 0, sizeof(p));
-    p.W = c.W; p.c0 = c.c0; p.mask = c.i; p.C = c.C; p.H = c.H; p.DY = c.DY;
-    p.DX = c.DX; p.Dc0 = c.Dc0;
-    j.ws = (unsigned char*)workspace + (size_t)k * stride;
-    p.dyw = (float*)(j.ws + lay.off_dyw);
-    p.dx0 = j.ws + lay.off_dx0;
-    p.T = T; p.B = B; p.n = n;
-    p.op_flags = op_flags;
-    if ((rc = resolve_pitch("ldY", c.ldY, n, B, es, &j.ldY)) != RTN_OK) return rc;
-    if ((rc = resolve_pitch("ldDY", c.ldDY, n, B, es, &p.ldDY)) != RTN_OK) return rc;
-    if ((rc = resolve_pitch("ldDX", c.ldDX, 4LL * n, B, es, &p.ldDX)) != RTN_OK) return rc;
-    hipLaunchKernelGGL(k_fill_u32, fill_grid, fill_block, 0, stream, (unsigned*)j.ws, 0u, (long long)(lay.off_wpk / 4));
-    RTN_HIP(hipGetLastError());
-    // returnn/native_op.py:1383-1407: which frames are visited, and in which order
-    j.abs_step = c.step > 0 ? c.step : -(long long)c.step;
-    j.num_steps = (T - c.start + j.abs_step - 1) / j.abs_step;
-    j.first = c.step > 0 ? c.start : T - c.start - 1;
-    if ((op_flags & kOpEndAtStart) && c.step < 0) {
-      // LstmLowMem: with a negative step the frames from T-start-1 down to `start` (returnn/native_op.py:957-963)
-      if (j.first < c.start) return fail(RTN_ERR_RANGE, "LstmLowMem gradient: start=%d with a negative step visits no frame of T=%lld", c.start, (long long)T);
-      j.num_steps = (j.first - c.start) / j.abs_step + 1;
-    }
-    j.end = j.first + (j.num_steps - 1) * c.step;  // inclusive
-    if (pk) {
-      // the exchange ring starts armed: all-ones words (the visited frames of DX are written by the kernel, the others
-      // zeroed behind it)
-      const int bp = rows_per_group > 8 ? 16 : 8;
-      const long long ring_words = (long long)((size_t)bgroups * kExRing * 4 * n * es * bp / 4);
-      if ((size_t)ring_words * 4 > lay.total - lay.off_ex)
-        return fail(RTN_ERR_WORKSPACE, "NativeLstm2 backward: internal: exchange ring of %lld bytes does not fit its section", ring_words * 4);
-      hipLaunchKernelGGL(k_fill_u32, dim3(256), fill_block, 0, stream, (unsigned*)(j.ws + lay.off_ex), 0xFFFFFFFFu, ring_words);
-      RTN_HIP(hipGetLastError());
-    } else if (j.num_steps != T) {
-      // frames the loop does not visit keep DX = 0 (:1385-1388): all rows cleared here, row by row
-      if ((rc = launch_clear_rows(c.DX, (long long)T * B, 4LL * n, p.ldDX, es, stream)) != RTN_OK) return rc;
-    }
-  }
-
-  if (pk) {
-    Lstm2BwdMulti multi;
-    memset(&multi, 0, sizeof(multi));
-    multi.count = count;
-    for (int k = 0; k < count; ++k) {
-      Lstm2BwdPersistent& q = multi.q[k];
-      q.p = jobs[(size_t)k].p;
-      q.Dd = calls[k].Dd;
-      q.Dy0 = calls[k].Dy0;
-      q.status = (unsigned*)jobs[(size_t)k].ws;
-      q.t_end = jobs[(size_t)k].end;
-      q.step = calls[k].step;
-      q.nframes = (int)jobs[(size_t)k].num_steps;
-      q.Bg = (B + bgroups - 1) / bgroups;
-      q.ksb = KSB;
-      // The kernels that keep one (row, k) pair per thread ask for a frame's inputs in front of the MFMAs, so only the
-      // delay stands between a frame's stores and the read of its ring slot: inside an XCD it is a fixed one there, as in
-      // the forward kernel (measured: 2.77 ms at 10 units against 2.82 adaptive and 2.87 / 2.86 at 4 / 16 for the layer).
-      const bool one_pair = rows_per_group <= 8 && ((bwd_mt + bwd_waves / 4 - 1) / (bwd_waves / 4)) % 2 == 0;
-      const bool fixed_delay = bwd_local && one_pair;
-      q.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_BWD_POLL_DELAY", fixed_delay ? 10 : 20)));
-      q.delay_inc = (int)std::max<long>(0, std::min<long>(16, env_long("RTN_LSTM2_BWD_DELAY_INC", fixed_delay ? 0 : 2)));
-      {
-        long dec = env_long("RTN_LSTM2_BWD_DELAY_DEC", 16);  // steps per unit of downward adaptation: a power of two
-        int mask = 0;
-        while (2 * (mask + 1) <= dec && mask < 255) mask = 2 * mask + 1;
-        q.delay_dec_mask = mask;
-      }
-      q.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);
-      q.sync = (unsigned*)(jobs[(size_t)k].ws + lay.off_sync);
-      q.ex = jobs[(size_t)k].ws + lay.off_ex;
-      q.Bp = rows_per_group > 8 ? 16 : 8;
-      q.bp_shift = rows_per_group > 8 ? 4 : 3;
-    }
-    multi.local = bwd_local ? 1 : 0;
-    multi.xcds = device_info().xcds;
-    // one cooperative launch per share of the batch groups (a single one unless the batch is too large for the device)
-    for (int g0 = 0; g0 < bgroups; g0 += groups_per_launch) {
-      const int groups_now = std::min(groups_per_launch, bgroups - g0);
-      multi.wgs_each = groups_now * (n / (16 * bwd_mt));
-      for (int k = 0; k < count; ++k) {
-        multi.q[k].groups = groups_now;
-        multi.q[k].group_offset = g0;
-      }
-      void* args[] = {(void*)&multi};
-      unsigned grid = (unsigned)(count * multi.wgs_each);
-      if (bwd_local) {
-        // workgroup id = slot * xcds + xcd: the groups of the launch are dealt round-robin to the XCDs
-        const int kb = n / (16 * bwd_mt), total_groups = count * groups_now;
-        grid = (unsigned)(multi.xcds * kb * ((total_groups + multi.xcds - 1) / multi.xcds));
-      }
-      rc = launch_coresident(pk, dim3(grid), dim3((unsigned)(64 * bwd_waves)), args, (unsigned)bwd_lds, stream, capturing);
-      if (rc != RTN_OK) return rc;
-    }
-    for (int k = 0; k < count; ++k) {
-      const BwdJob& j = jobs[(size_t)k];
-      if (j.num_steps == T) continue;
-      const long long row_words = (long long)((size_t)n * 4 * es / 4), pitch_words = (long long)((size_t)j.p.ldDX * es / 4);
-      if (dtype == RTN_DTYPE_BF16)
-        hipLaunchKernelGGL(k_bwd_zero_unvisited<__bf16>, dim3(1024), fill_block, 0, stream, calls[k].DX, (long long)T, (long long)B, row_words,
-                           pitch_words, j.first, (long long)calls[k].step, j.num_steps);
-      else
-        hipLaunchKernelGGL(k_bwd_zero_unvisited<float>, dim3(1024), fill_block, 0, stream, calls[k].DX, (long long)T, (long long)B, row_words,
-                           pitch_words, j.first, (long long)calls[k].step, j.num_steps);
-      RTN_HIP(hipGetLastError());
-    }
-  } else {
-    // count == 1 here.  The launches of all frames, in reverse processing order.  MFMA shapes: one fused launch per
-    // frame (the GEMM of the frame processed before, then this frame's pointwise part) and a last GEMM-only launch;
-    // other shapes: a pointwise and a generic GEMM launch per frame.
-    BwdJob& j = jobs[0];
-    if (mfma && env_long("RTN_LSTM2_BWD_PACK_W", 1)) {
-      // every launch uses each fragment of W once: read them from a copy in fragment order (see k_bwd_pack_w)
-      j.p.Wpk = j.ws + lay.off_wpk;
-      const long long frags = (long long)(n / 16) * (4 * n / (dtype == RTN_DTYPE_BF16 ? 32 : 16)) * 64;
-      const dim3 pgrid((unsigned)std::min<long long>((frags + 255) / 256, 4096)), pblock(256);
-      if (dtype == RTN_DTYPE_BF16)
-        hipLaunchKernelGGL(k_bwd_pack_w<__bf16>, pgrid, pblock, 0, stream, calls[0].W, (void*)j.p.Wpk, n);
-      else
-        hipLaunchKernelGGL(k_bwd_pack_w<float>, pgrid, pblock, 0, stream, calls[0].W, (void*)j.p.Wpk, n);
-      RTN_HIP(hipGetLastError());
-    }
-    const Lstm2BwdParams& p = j.p;
-    const int step = calls[0].step;
-    const long long first = j.first, end = j.end;
-    // Batch rows per workgroup (16 * NT): 32 if that still leaves every CU a workgroup (each batch tile reads W again),
-    // else 16 (measured: float32 n=1024 B=64 29 us per frame with 16 rows, 35 with 32; 64 rows were never faster).
-    int NT = B > 16 ? 2 : 1;
-    if (NT > 1 && (long long)(n / 16) * ((B + 16 * NT - 1) / (16 * NT)) < device_info().cus) NT = 1;
-    auto record = [&](LaunchSink& sink) -> int {
-      const dim3 pw_grid((unsigned)((bn + 255) / 256)), pw_block(256);
-      const dim3 mm_grid((unsigned)((n / 16) * ((B + 16 * NT - 1) / (16 * NT)))), mm_block(kWgThreads);
-      const bool bf = dtype == RTN_DTYPE_BF16;
-      long long t_done = -1;  // frame whose DX still has to go through the GEMM
-      for (long long t = end;; t -= step) {
-        const bool more = step > 0 ? t >= first : t <= first;
-        const bool right = more && (step > 0 ? (t - step >= first) : (t - step <= first));
-        const long long prev_t = right ? t - step : -1;
-        const long long tt = more ? t : -1;
-        int rc2 = RTN_OK;
-        if (mfma) {
-          void (*k)(Lstm2BwdParams, long long, long long, long long) =
-              bf ? (NT == 2 ? &k_bwd_step<__bf16, 2> : &k_bwd_step<__bf16, 1>) : (NT == 2 ? &k_bwd_step<float, 2> : &k_bwd_step<float, 1>);
-          rc2 = enqueue(sink, k, mm_grid, mm_block, 0, p, t_done, tt, prev_t);
-        } else if (more) {
-          rc2 = enqueue(sink, bf ? &k_bwd_pointwise<__bf16> : &k_bwd_pointwise<float>, pw_grid, pw_block, 0, p, t, prev_t);
-          if (rc2 == RTN_OK)
-            rc2 = enqueue(sink, bf ? &k_bwd_gemm_dy_generic<__bf16> : &k_bwd_gemm_dy_generic<float>, pw_grid, pw_block, 0, p, t);
-        }
-        if (rc2 != RTN_OK) return rc2;
-        if (!more) break;
-        t_done = t;
-      }
-      return RTN_OK;
-    };
-    if (capturing || env_long("RTN_LSTM2_BWD_NO_GRAPH", 0)) {
-      LaunchSink sink;
-      sink.stream = stream;
-      rc = record(sink);
-    } else {
-      std::string key("bwd");
-      int dev = 0;
-      RTN_HIP(hipGetDevice(&dev));
-      Lstm2BwdParams shape = p;  // p was zeroed before it was filled in
-      shape.W = shape.H = shape.DY = shape.Wpk = nullptr;
-      shape.c0 = shape.mask = shape.C = nullptr;
-      shape.DX = shape.dx0 = nullptr;
-      shape.dyw = shape.Dc0 = nullptr;
-      key.append(reinterpret_cast<const char*>(&shape), sizeof(shape));
-      key_append(&key, (int)(p.Wpk != nullptr));
-      key_append(&key, dtype); key_append(&key, (int)calls[0].start); key_append(&key, step); key_append(&key, dev);
-      key_append(&key, (int)mfma); key_append(&key, NT);
-      rc = replay_graph(key, &p, sizeof(p), stream, record);
-    }
-    if (rc != RTN_OK) return rc;
-  }
-
-  for (int k = 0; k < count; ++k) {
-    const rtn_lstm2_bwd_call& c = calls[k];
-    const BwdJob& j = jobs[(size_t)k];
-    const int step = c.step;
-    // DW = sum over consecutive visited frames Y[t - step]^T * DX[t]  (:1433-1452), then += y0^T * dx0 (:1456-1460)
-    const unsigned char* Yb = (const unsigned char*)c.Y;
-    const unsigned char* DXb = (const unsigned char*)c.DX;
-    if (j.num_steps > 1) {
-      if (j.abs_step == 1) {
-        const long long lo = std::min(j.first, j.end);
-        rc = dw_accumulate(blas, Yb + (size_t)(lo + std::max(0, -step)) * B * j.ldY * es,
-                           DXb + (size_t)(lo + std::max(0, step)) * B * j.p.ldDX * es, c.DW, (j.num_steps - 1) * B, n, dtype, j.ldY, j.p.ldDX);
-        if (rc != RTN_OK) return rc;
-      } else {
-        for (long long t = j.end - step; step > 0 ? t >= j.first : t <= j.first; t -= step) {
-          rc = dw_accumulate(blas, Yb + (size_t)t * B * j.ldY * es, DXb + (size_t)(t + step) * B * j.p.ldDX * es, c.DW, B, n, dtype, j.ldY,
-                             j.p.ldDX);
-          if (rc != RTN_OK) return rc;
-        }
-      }
-    }
-    rc = dw_accumulate(blas, c.y0, j.p.dx0, c.DW, B, n, dtype);
-    if (rc != RTN_OK) return rc;
-    if (!pk) {
-      if (dtype == RTN_DTYPE_BF16)
-        hipLaunchKernelGGL(k_convert_from_f32<__bf16>, fill_grid, fill_block, 0, stream, j.p.dyw, c.Dy0, bn);
-      else
-        hipLaunchKernelGGL(k_convert_from_f32<float>, fill_grid, fill_block, 0, stream, j.p.dyw, c.Dy0, bn);
-      RTN_HIP(hipGetLastError());
-    }
-  }
-  return RTN_OK;
+  std::vector<BwdJob> jobs;
+  if ((rc = bwd_prepare_jobs(x, ch, lay, workspace, stride, &jobs)) != RTN_OK) return rc;
+  rc = ch.kernel ? bwd_launch_persistent(x, ch, lay, jobs) : bwd_launch_per_frame(x, mfma, lay, jobs[0]);  // (per frame: count == 1)
+  if (rc != RTN_OK) return rc;
+  return bwd_weight_gradients(x, blas, jobs, ch.kernel != nullptr);
 }
 
 }  // namespace
