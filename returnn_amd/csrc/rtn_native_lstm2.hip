@@ -1106,14 +1106,161 @@ int probe_xcds(hipStream_t stream) {
   return RTN_OK;
 }
 
+int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode,
+              void* workspace, size_t workspace_bytes, void* hip_stream, int op_flags = 0, size_t ws_stride = 0,
+              bool no_graph = false);
+
+// The problems zero-padded to a width the matrix-core kernels take (see padded_width), on copies in the workspace: slice
+// k = the workspace of the padded call k, then its padded copies.
+int fwd_padded(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int32_t n, int np, int32_t dtype, int32_t mode,
+               void* workspace, size_t workspace_bytes, hipStream_t stream, int op_flags, bool no_graph) {
+  int rc = RTN_OK;
+  for (int k = 0; k < count; ++k) {
+    const rtn_lstm2_call& c = calls[k];
+    const void* ptrs[] = {c.X, c.W, c.y0, c.c0, c.i, c.Y, c.C, c.H, c.d};
+    const char* names[] = {"X", "W", "y0", "c0", "i", "Y", "C", "H", "d"};
+    for (int q = 0; q < 9; ++q)
+      if (!ptrs[q]) return fail(RTN_ERR_ARG, "NativeLstm2: %s must not be null", names[q]);
+  }
+  const size_t inner_each = workspace_each_exact(count, T, B, np, dtype, mode);
+  const FwdPadLayout L = fwd_pad_layout(T, B, np, dtype);
+  const size_t each = inner_each + L.total;
+  const size_t need = (size_t)count * each;
+  if (!workspace || workspace_bytes < need)
+    return fail(RTN_ERR_WORKSPACE, "NativeLstm2: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
+  if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2: workspace must be 16-byte aligned");
+  const size_t es = esize(dtype);
+  const long long tb = (long long)T * B;
+  std::vector<rtn_lstm2_call> padded((size_t)count);
+  for (int k = 0; k < count; ++k) {
+    const rtn_lstm2_call& c = calls[k];
+    unsigned char* base = (unsigned char*)workspace + (size_t)k * each + inner_each;
+    long long ldX = 0, ldY = 0;
+    if ((rc = resolve_pitch("ldX", c.ldX, 4LL * n, B, es, &ldX)) != RTN_OK) return rc;
+    if ((rc = resolve_pitch("ldY", c.ldY, n, B, es, &ldY)) != RTN_OK) return rc;
+    if ((rc = launch_pad(c.X, base + L.X, tb, tb, 4, n, np, es, stream, ldX)) != RTN_OK) return rc;
+    if ((rc = launch_pad(c.W, base + L.W, n, np, 4, n, np, es, stream)) != RTN_OK) return rc;
+    if ((rc = launch_pad(c.y0, base + L.y0, B, B, 1, n, np, es, stream)) != RTN_OK) return rc;
+    if ((rc = launch_pad(c.c0, base + L.c0, B, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
+    padded[(size_t)k] = {base + L.X, base + L.W, base + L.y0, (const float*)(base + L.c0), c.i, c.start, c.step,
+                         base + L.Y, (float*)(base + L.C), base + L.H, (float*)(base + L.d), 0, 0};
+  }
+  rc = fwd_calls(padded.data(), count, T, B, np, dtype, mode, workspace, need, (void*)stream, op_flags, each, no_graph);
+  if (rc != RTN_OK) return rc;
+  for (int k = 0; k < count; ++k) {
+    const rtn_lstm2_call& c = calls[k];
+    const rtn_lstm2_call& q = padded[(size_t)k];
+    if ((rc = launch_unpad(q.Y, c.Y, tb, 1, n, np, es, stream, c.ldY)) != RTN_OK) return rc;
+    if ((rc = launch_unpad(q.C, c.C, tb, 1, n, np, 4, stream)) != RTN_OK) return rc;
+    if ((rc = launch_unpad(q.H, c.H, tb, 4, n, np, es, stream)) != RTN_OK) return rc;
+    if ((rc = launch_unpad(q.d, c.d, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
+  }
+  return RTN_OK;
+}
+
+// The plan of an entry, settled against the device: a persistent plan needs all its workgroups on the device together,
+// so it is checked against what the kernel really gets per CU, planned again for that if it was too optimistic, and
+// given up for per-step launches if that does not help.  *pk: the persistent kernel (null: launches per step);
+// *fused: problems per persistent launch.
+int settle_fwd_plan(int count, int64_t T, int B, int n, int dtype, int mode, bool capturing, Plan* plan, const void** pk, int* fused) {
+  Plan& pl = *plan;
+  std::string why;
+  int rc = RTN_OK;
+  *pk = nullptr;
+  *fused = 1;
+  const int plan_count = env_long("RTN_LSTM2_NO_FUSE", 0) ? 1 : std::min(count, kMaxMulti);
+  if (!make_plan(T, B, n, dtype, mode, capturing, &pl, &why, 2, plan_count))
+    return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: persistent mode unavailable for T=%lld B=%d n=%d: %s", (long long)T, B, n, why.c_str());
+  for (int attempt = 0; pl.kind == kPlanMfma && pl.mode == RTN_MODE_PERSISTENT; ++attempt) {
+    *pk = pl.regw ? (const void*)regw_kernel(dtype, pl.MT, pl.NT, pl.KSMAX, pl.half) : (const void*)mfma_kernel(dtype, pl.MT, pl.NT);
+    if (!*pk) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d ks=%d", pl.MT, pl.NT, pl.KSMAX);
+    if ((rc = ensure_lds_limit(*pk, pl.lds_bytes)) != RTN_OK) return rc;
+    const int wgs = pl.regw ? pl.grid : pl.groups * pl.wgs_per_group;
+    int per_cu = 0;
+    if ((rc = occupancy_per_cu(*pk, kWgThreads, pl.lds_bytes, &per_cu)) != RTN_OK) return rc;
+    const long long capacity = (long long)per_cu * device_info().cus;
+    if (capacity >= wgs) {
+      if (pl.local) {
+        *fused = plan_count;  // the plan's grid holds the groups of that many problems
+      } else if (pl.regw && count > 1 && pl.passes == 1 && !env_long("RTN_LSTM2_NO_FUSE", 0)) {
+        const long long each = (long long)align_up((size_t)wgs, (size_t)device_info().xcds);
+        *fused = (int)std::max<long long>(1, std::min<long long>(std::min(count, kMaxMulti), capacity / each));
+      }
+      return RTN_OK;
+    }
+    *pk = nullptr;
+    if (attempt == 0 && per_cu >= 1 && make_plan(T, B, n, dtype, mode, capturing, &pl, &why, per_cu, plan_count)) continue;
+    if (mode == RTN_MODE_PERSISTENT)
+      return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: %d workgroups cannot be co-resident (%d per CU)", wgs, per_cu);
+    if (!make_plan(T, B, n, dtype, RTN_MODE_GRAPH, capturing, &pl, &why))
+      return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no per-step plan: %s", why.c_str());
+    break;
+  }
+  return RTN_OK;
+}
+
+// The parameter block of call `c` on plan `pl` with its workspace slice at `ws`.
+int fill_fwd_params(const rtn_lstm2_call& c, const Plan& pl, bool persistent, unsigned char* ws, int64_t T, int B, int n, int dtype,
+                    int op_flags, Lstm2Params* out) {
+  Lstm2Params& p = *out;
+  int rc = RTN_OK;
+  memset(&p, 0, sizeof(p));
+  p.X = c.X; p.W = c.W; p.y0 = c.y0; p.c0 = c.c0; p.mask = c.i;
+  p.Y = c.Y; p.C = c.C; p.H = c.H; p.d = c.d;
+  p.status = (unsigned*)(ws + pl.off_status);
+  p.flags = (unsigned*)(ws + pl.off_flags);
+  p.hx = ws + pl.off_hx;
+  p.Wp = ws + pl.off_wp;
+  p.ycarry = ws + pl.off_ycarry;
+  p.trace = pl.off_trace ? (unsigned long long*)(ws + pl.off_trace) : nullptr;
+  p.T = T; p.B = B; p.n = n;
+  if ((rc = resolve_pitch("ldX", c.ldX, 4LL * n, B, esize(dtype), &p.ldX)) != RTN_OK) return rc;
+  if ((rc = resolve_pitch("ldY", c.ldY, n, B, esize(dtype), &p.ldY)) != RTN_OK) return rc;
+  // returnn/native_op.py:1253-1259
+  if (c.step > 0) {
+    p.first = c.start;
+    p.nsteps = (int)((T - 1 - c.start) / c.step + 1);
+  } else {
+    p.first = (int)(T - c.start - 1);
+    const long long last = (op_flags & kOpEndAtStart) ? c.start : 0;
+    if (p.first < last) return fail(RTN_ERR_RANGE, "LstmLowMem: start=%d with a negative step visits no frame of T=%lld", c.start, (long long)T);
+    p.nsteps = (int)((p.first - last) / (-(long long)c.step) + 1);
+  }
+  p.step = c.step;
+  p.groups = p.groups_total = pl.groups_total; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
+  p.group_offset = 0;
+  p.op_flags = op_flags;
+  p.w_direct = (!persistent && pl.kind == kPlanMfma && pl.w_direct) ? 1 : 0;
+  p.hx_bufs = kHxRing;
+  p.hx_sentinel = pl.regw ? 1 : 0;
+  p.exchange = (int)env_long("RTN_LSTM2_EXCHANGE", 0);
+  if (p.exchange != kExNoWait) p.exchange = kExDevice;  // no-wait: a timing aid, results invalid (status 2)
+  // Device-scope stores take about a microsecond to become visible: a first read issued at once would
+  // come back incomplete and cost a second round trip, so it is held back, and the kernel adapts the delay.  Within an
+  // XCD the delay is a fixed one (tuned on MI355X over n = 64 ... 1024 and 1 ... 16 rows per group: the best fixed
+  // delay is within 2 % of these four everywhere, and 4 % to 13 % ahead of the adaptive one).
+  p.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", pl.local ? (pl.Bg > 8 ? 10 : (dtype != RTN_DTYPE_BF16 ? 5 : (pl.MT >= 8 ? 6 : 3))) : 20)));
+  {
+    long dec = env_long("RTN_LSTM2_DELAY_DEC", 8);  // steps per unit of downward adaptation: a power of two
+    int mask = 0;
+    while (2 * (mask + 1) <= dec && mask < 255) mask = 2 * mask + 1;
+    p.delay_dec_mask = mask;
+    p.delay_inc = (int)std::max<long>(0, std::min<long>(16, env_long("RTN_LSTM2_DELAY_INC", pl.local ? 0 : 2)));
+  }
+  p.xcds = device_info().xcds;
+  p.sync_policy = (int)env_long("RTN_LSTM2_SYNC", kStoreCoherent | kLoadCoherent);
+  if (!((p.sync_policy & (kStoreCoherent | kReleaseFence)) && (p.sync_policy & (kLoadCoherent | kAcquireFence))))
+    return fail(RTN_ERR_ARG, "NativeLstm2: RTN_LSTM2_SYNC=%d is not a valid publication policy", p.sync_policy);
+  p.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);  // 2 s at 100 MHz
+  return RTN_OK;
+}
+
 // The calls of one entry: `count` independent problems of one shape.  Each gets the slice
 // [k * each, (k + 1) * each) of the workspace, each = workspace_each(count, ...).
 // When the persistent register kernel fits that many times on the device at once, all of them run
-// in one cooperative launch (their workgroups share the CUs and hide each other's exchange waits);
-// otherwise they are enqueued one after the other.
+// in one launch (every workgroup with a CU to itself); otherwise they are enqueued one after the other.
 int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t mode,
-              void* workspace, size_t workspace_bytes, void* hip_stream, int op_flags = 0, size_t ws_stride = 0,
-              bool no_graph = false) {
+              void* workspace, size_t workspace_bytes, void* hip_stream, int op_flags, size_t ws_stride, bool no_graph) {
   int rc = check_dims(T, B, n, dtype);
   if (rc != RTN_OK) return rc;
   if (mode < RTN_MODE_AUTO || mode > RTN_MODE_STEPWISE) return fail(RTN_ERR_ARG, "NativeLstm2: unknown mode %d", mode);
@@ -1132,51 +1279,7 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
     return RTN_OK;
   }
   const int np = padded_width(n);
-  if (np != n) {
-    // Run the problem zero-padded to a width the matrix-core kernels take (see padded_width), on copies in the workspace.
-    for (int k = 0; k < count; ++k) {
-      const rtn_lstm2_call& c = calls[k];
-      const void* ptrs[] = {c.X, c.W, c.y0, c.c0, c.i, c.Y, c.C, c.H, c.d};
-      const char* names[] = {"X", "W", "y0", "c0", "i", "Y", "C", "H", "d"};
-      for (int q = 0; q < 9; ++q)
-        if (!ptrs[q]) return fail(RTN_ERR_ARG, "NativeLstm2: %s must not be null", names[q]);
-    }
-    // slice k of the workspace: the workspace of the padded call k, then its padded copies
-    const size_t inner_each = workspace_each_exact(count, T, B, np, dtype, mode);
-    const FwdPadLayout L = fwd_pad_layout(T, B, np, dtype);
-    const size_t each = inner_each + L.total;
-    const size_t need = (size_t)count * each;
-    if (!workspace || workspace_bytes < need)
-      return fail(RTN_ERR_WORKSPACE, "NativeLstm2: workspace of %zu bytes needed, got %zu", need, workspace ? workspace_bytes : (size_t)0);
-    if (!aligned16(workspace)) return fail(RTN_ERR_ARG, "NativeLstm2: workspace must be 16-byte aligned");
-    const size_t es = esize(dtype);
-    const long long tb = (long long)T * B;
-    std::vector<rtn_lstm2_call> padded((size_t)count);
-    for (int k = 0; k < count; ++k) {
-      const rtn_lstm2_call& c = calls[k];
-      unsigned char* base = (unsigned char*)workspace + (size_t)k * each + inner_each;
-      long long ldX = 0, ldY = 0;
-      if ((rc = resolve_pitch("ldX", c.ldX, 4LL * n, B, es, &ldX)) != RTN_OK) return rc;
-      if ((rc = resolve_pitch("ldY", c.ldY, n, B, es, &ldY)) != RTN_OK) return rc;
-      if ((rc = launch_pad(c.X, base + L.X, tb, tb, 4, n, np, es, stream, ldX)) != RTN_OK) return rc;
-      if ((rc = launch_pad(c.W, base + L.W, n, np, 4, n, np, es, stream)) != RTN_OK) return rc;
-      if ((rc = launch_pad(c.y0, base + L.y0, B, B, 1, n, np, es, stream)) != RTN_OK) return rc;
-      if ((rc = launch_pad(c.c0, base + L.c0, B, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
-      padded[(size_t)k] = {base + L.X, base + L.W, base + L.y0, (const float*)(base + L.c0), c.i, c.start, c.step,
-                           base + L.Y, (float*)(base + L.C), base + L.H, (float*)(base + L.d), 0, 0};
-    }
-    rc = fwd_calls(padded.data(), count, T, B, np, dtype, mode, workspace, need, hip_stream, op_flags, each, no_graph);
-    if (rc != RTN_OK) return rc;
-    for (int k = 0; k < count; ++k) {
-      const rtn_lstm2_call& c = calls[k];
-      const rtn_lstm2_call& q = padded[(size_t)k];
-      if ((rc = launch_unpad(q.Y, c.Y, tb, 1, n, np, es, stream, c.ldY)) != RTN_OK) return rc;
-      if ((rc = launch_unpad(q.C, c.C, tb, 1, n, np, 4, stream)) != RTN_OK) return rc;
-      if ((rc = launch_unpad(q.H, c.H, tb, 4, n, np, es, stream)) != RTN_OK) return rc;
-      if ((rc = launch_unpad(q.d, c.d, B, 1, n, np, 4, stream)) != RTN_OK) return rc;
-    }
-    return RTN_OK;
-  }
+  if (np != n) return fwd_padded(calls, count, T, B, n, np, dtype, mode, workspace, workspace_bytes, stream, op_flags, no_graph);
   for (int k = 0; k < count; ++k) {
     const rtn_lstm2_call& c = calls[k];
     if (c.start < 0 || c.start >= T)
@@ -1198,42 +1301,9 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
   const bool capturing = cap_status != hipStreamCaptureStatusNone;
 
   Plan pl;
-  std::string why;
-  const int plan_count = env_long("RTN_LSTM2_NO_FUSE", 0) ? 1 : std::min(count, kMaxMulti);
-  if (!make_plan(T, B, n, dtype, mode, capturing, &pl, &why, 2, plan_count))
-    return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: persistent mode unavailable for T=%lld B=%d n=%d: %s", (long long)T, B, n, why.c_str());
-  // A persistent plan needs all its workgroups on the device together: check against what the kernel
-  // really gets per CU, plan again for that if the plan was too optimistic, else fall back to per-step launches.
   const void* pk = nullptr;  // the persistent kernel, if any
-  int fused = 1;             // problems per cooperative launch
-  for (int attempt = 0; pl.kind == kPlanMfma && pl.mode == RTN_MODE_PERSISTENT; ++attempt) {
-    pk = pl.regw ? (const void*)regw_kernel(dtype, pl.MT, pl.NT, pl.KSMAX, pl.half) : (const void*)mfma_kernel(dtype, pl.MT, pl.NT);
-    if (!pk) return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no kernel for mt=%d nt=%d ks=%d", pl.MT, pl.NT, pl.KSMAX);
-    rc = ensure_lds_limit(pk, pl.lds_bytes);
-    if (rc != RTN_OK) return rc;
-    const int wgs = pl.regw ? pl.grid : pl.groups * pl.wgs_per_group;
-    int per_cu = 0;
-    rc = occupancy_per_cu(pk, kWgThreads, pl.lds_bytes, &per_cu);
-    if (rc != RTN_OK) return rc;
-    const long long capacity = (long long)per_cu * device_info().cus;
-    if (capacity >= wgs) {
-      if (pl.local) {
-        fused = plan_count;  // the plan's grid holds the groups of that many problems
-      } else if (pl.regw && count > 1 && pl.passes == 1 && !env_long("RTN_LSTM2_NO_FUSE", 0)) {
-        const long long each = (long long)align_up((size_t)wgs, (size_t)device_info().xcds);
-        fused = (int)std::min<long long>(std::min(count, kMaxMulti), capacity / each);
-        if (fused < 1) fused = 1;
-      }
-      break;
-    }
-    pk = nullptr;
-    if (attempt == 0 && per_cu >= 1 && make_plan(T, B, n, dtype, mode, capturing, &pl, &why, per_cu, plan_count)) continue;
-    if (mode == RTN_MODE_PERSISTENT)
-      return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: %d workgroups cannot be co-resident (%d per CU)", wgs, per_cu);
-    if (!make_plan(T, B, n, dtype, RTN_MODE_GRAPH, capturing, &pl, &why))
-      return fail(RTN_ERR_UNSUPPORTED, "NativeLstm2: no per-step plan: %s", why.c_str());
-    break;
-  }
+  int fused = 1;             // problems per persistent launch
+  if ((rc = settle_fwd_plan(count, T, B, n, dtype, mode, capturing, &pl, &pk, &fused)) != RTN_OK) return rc;
   // distance between the calls' workspaces: given by a caller that keeps more than the workspace in a call's slice
   const size_t each_ws = ws_stride ? ws_stride : (count > 1 ? workspace_each(count, T, B, n, dtype, mode) : pl.total);
   if (each_ws < pl.total) return fail(RTN_ERR_WORKSPACE, "NativeLstm2: internal: workspace slice %zu < layout %zu", each_ws, pl.total);
@@ -1247,59 +1317,11 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
 
   Lstm2Multi multi;
   memset(&multi, 0, sizeof(multi));
-  int pending = 0;  // problems prepared for the next cooperative launch
+  int pending = 0;  // problems prepared for the next persistent launch
   for (int k = 0; k < count; ++k) {
-    const rtn_lstm2_call& c = calls[k];
     Lstm2Params p;
-    memset(&p, 0, sizeof(p));
-    p.X = c.X; p.W = c.W; p.y0 = c.y0; p.c0 = c.c0; p.mask = c.i;
-    p.Y = c.Y; p.C = c.C; p.H = c.H; p.d = c.d;
-    unsigned char* ws = (unsigned char*)workspace + (size_t)k * each_ws;
-    p.status = (unsigned*)(ws + pl.off_status);
-    p.flags = (unsigned*)(ws + pl.off_flags);
-    p.hx = ws + pl.off_hx;
-    p.Wp = ws + pl.off_wp;
-    p.ycarry = ws + pl.off_ycarry;
-    p.trace = pl.off_trace ? (unsigned long long*)(ws + pl.off_trace) : nullptr;
-    p.T = T; p.B = B; p.n = n;
-    if ((rc = resolve_pitch("ldX", c.ldX, 4LL * n, B, esize(dtype), &p.ldX)) != RTN_OK) return rc;
-    if ((rc = resolve_pitch("ldY", c.ldY, n, B, esize(dtype), &p.ldY)) != RTN_OK) return rc;
-    // returnn/native_op.py:1253-1259
-    if (c.step > 0) {
-      p.first = c.start;
-      p.nsteps = (int)((T - 1 - c.start) / c.step + 1);
-    } else {
-      p.first = (int)(T - c.start - 1);
-      const long long last = (op_flags & kOpEndAtStart) ? c.start : 0;
-      if (p.first < last) return fail(RTN_ERR_RANGE, "LstmLowMem: start=%d with a negative step visits no frame of T=%lld", c.start, (long long)T);
-      p.nsteps = (int)((p.first - last) / (-(long long)c.step) + 1);
-    }
-    p.step = c.step;
-    p.groups = p.groups_total = pl.groups_total; p.wgs_per_group = pl.wgs_per_group; p.Bg = pl.Bg; p.Bp = pl.Bp;
-    p.group_offset = 0;
-    p.op_flags = op_flags;
-    p.w_direct = (!pk && pl.kind == kPlanMfma && pl.w_direct) ? 1 : 0;
-    p.hx_bufs = kHxRing;
-    p.hx_sentinel = pl.regw ? 1 : 0;
-    p.exchange = (int)env_long("RTN_LSTM2_EXCHANGE", 0);
-    if (p.exchange != kExNoWait) p.exchange = kExDevice;  // no-wait: a timing aid, results invalid (status 2)
-    // Device-scope stores take about a microsecond to become visible: a first read issued at once would
-    // come back incomplete and cost a second round trip, so it is held back, and the kernel adapts the delay.  Within an
-    // XCD the delay is a fixed one (tuned on MI355X over n = 64 ... 1024 and 1 ... 16 rows per group: the best fixed
-    // delay is within 2 % of these four everywhere, and 4 % to 13 % ahead of the adaptive one).
-    p.poll_delay = (int)std::max<long>(0, std::min<long>(64, env_long("RTN_LSTM2_POLL_DELAY", pl.local ? (pl.Bg > 8 ? 10 : (dtype != RTN_DTYPE_BF16 ? 5 : (pl.MT >= 8 ? 6 : 3))) : 20)));
-    {
-      long dec = env_long("RTN_LSTM2_DELAY_DEC", 8);  // steps per unit of downward adaptation: a power of two
-      int mask = 0;
-      while (2 * (mask + 1) <= dec && mask < 255) mask = 2 * mask + 1;
-      p.delay_dec_mask = mask;
-      p.delay_inc = (int)std::max<long>(0, std::min<long>(16, env_long("RTN_LSTM2_DELAY_INC", pl.local ? 0 : 2)));
-    }
-    p.xcds = device_info().xcds;
-    p.sync_policy = (int)env_long("RTN_LSTM2_SYNC", kStoreCoherent | kLoadCoherent);
-    if (!((p.sync_policy & (kStoreCoherent | kReleaseFence)) && (p.sync_policy & (kLoadCoherent | kAcquireFence))))
-      return fail(RTN_ERR_ARG, "NativeLstm2: RTN_LSTM2_SYNC=%d is not a valid publication policy", p.sync_policy);
-    p.timeout_ticks = (unsigned long long)env_long("RTN_LSTM2_TIMEOUT_TICKS", 200000000L);  // 2 s at 100 MHz
+    if ((rc = fill_fwd_params(calls[k], pl, pk != nullptr, (unsigned char*)workspace + (size_t)k * each_ws, T, B, n, dtype, op_flags, &p)) != RTN_OK)
+      return rc;
 
     // Frames the loop never visits.
     if (p.nsteps != T) {
@@ -1331,7 +1353,7 @@ int fwd_calls(const rtn_lstm2_call* calls, int count, int64_t T, int32_t B, int3
         RTN_HIP(hipGetLastError());
       }
       if (pk && pl.regw && pl.passes > 1) {
-        // the batch groups in turns: one cooperative launch per share of them
+        // the batch groups in turns: one persistent launch per share of them
         for (int g0 = 0; g0 < pl.groups_total; g0 += pl.groups) {
           Lstm2Multi one;
           memset(&one, 0, sizeof(one));
