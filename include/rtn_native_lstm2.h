@@ -115,6 +115,9 @@ size_t rtn_native_lstm2_fwd_workspace_bytes(int64_t T, int32_t B, int32_t n, int
  * (RTN_ERR_UNSUPPORTED).  Arguments, results and error codes are otherwise those of rtn_native_lstm2_fwd, bit for bit.
  * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU race (keep them on one stream,
  * or order them with events).  The array keeps the previous call's contents; every call re-initialises what it uses.
+ * A persistent kernel needs the whole device: do not let a call of this entry overlap in time with persistent calls of
+ * the other entries on other streams of the same GPU either (the other entries order their persistent launches among
+ * themselves with an event of the library's; this entry creates nothing and joins that order only once the event exists).
  */
 int rtn_native_lstm2_fwd_static(const void* X, const void* W, const void* y0, const float* c0, const float* i,
                                 int32_t start, int32_t step, void* Y, float* C, void* H, float* d, int64_t T,

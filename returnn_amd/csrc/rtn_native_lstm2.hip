@@ -831,7 +831,7 @@ std::string g_capture_refusal;  // why a cooperative node was refused, if it was
 // property for its own launches itself -- one event per device behind the last persistent launch, which a launch on
 // another stream waits for (on the device, the host never blocks).
 // RTN_LSTM2_LAUNCH=cooperative brings the cooperative launch back; the entry that may not create anything at call time
-// (g_no_setup_objects) keeps it, since this scheme needs an event.
+// (g_no_setup_objects) keeps it, since this scheme needs an event, and joins the ordering where the event exists.
 thread_local bool g_no_setup_objects = false;
 struct PersistentOrder {
   hipEvent_t last = nullptr;      // behind the last persistent launch on this device
@@ -846,12 +846,26 @@ int launch_coresident(const void* k, dim3 grid, dim3 block, void** args, unsigne
     const char* how = env_get("RTN_LSTM2_LAUNCH");
     int dev = 0;
     RTN_HIP(hipGetDevice(&dev));
-    if (g_no_setup_objects || (how && strcmp(how, "cooperative") == 0) || dev < 0 || dev >= 64) {
+    if ((how && strcmp(how, "cooperative") == 0) || dev < 0 || dev >= 64) {
       RTN_HIP(hipLaunchCooperativeKernel(k, grid, block, args, lds, stream));
       return RTN_OK;
     }
     std::lock_guard<std::mutex> lock(g_order_mu);
     PersistentOrder& o = g_order[dev];
+    if (g_no_setup_objects) {
+      // Cooperative launch, and part of the ordering as far as that takes no new object: behind the last ordinary
+      // persistent launch if there has been one on this device, and in front of the next.  (Before the first ordinary
+      // launch there is no event to record into: such a call is only ordered by its own stream -- as calls of that entry
+      // have to be anyway, since they share one scratch array.)
+      if (o.last && o.any && o.stream != stream) RTN_HIP(hipStreamWaitEvent(stream, o.last, 0));
+      RTN_HIP(hipLaunchCooperativeKernel(k, grid, block, args, lds, stream));
+      if (o.last) {
+        RTN_HIP(hipEventRecord(o.last, stream));
+        o.stream = stream;
+        o.any = true;
+      }
+      return RTN_OK;
+    }
     if (!o.last) RTN_HIP(hipEventCreateWithFlags(&o.last, hipEventDisableTiming));
     if (o.any && o.stream != stream) RTN_HIP(hipStreamWaitEvent(stream, o.last, 0));
     RTN_HIP(hipLaunchKernel(k, grid, block, args, lds, stream));
