@@ -123,8 +123,9 @@ def step_budget(call_ms, nowait_ms, seq_ms, issue_ms, T):
     add up to the measured step by construction, each is the difference of two measurements:
 
     * ``mfma_issue``: the issue probe (the plan's MFMAs per wavefront and nothing else);
-    * ``partial_tiles_through_lds``: sequence probe - issue probe (operands from LDS, the four wavefronts' partial
-      tiles written to LDS, the step's barrier, their sum read back);
+    * ``partial_tiles_through_lds``: sequence probe - issue probe (what the decomposition adds to the bare MFMAs: B
+      operands made ready in front of them, the matrix pipeline running empty before the four wavefronts' partial tiles
+      can be written to LDS, the step's barrier, their sum read back);
     * ``gates_streams_stores``: the op's kernel with the reads of the hidden state switched off - sequence probe (gate
       arithmetic, cell update, the exchange stores, what the X / H / Y / C streams cost although they ride behind the
       MFMAs);

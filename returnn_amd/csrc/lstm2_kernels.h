@@ -1251,9 +1251,11 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
         for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
       // Everything that is not on the path h -> MFMA -> gates -> h rides in the shadow of the MFMAs: all of it without
       // a branch (a frame that does not exist is a buffer of no bytes; LDS copies nobody reads may take anything), in
-      // one block of straight-line code that the scheduler is told to weave: a wavefront that has a SIMD to itself
-      // issues one instruction per 4 clocks, an MFMA keeps the matrix core busy for 16, so three other instructions fit
-      // behind every MFMA for free -- but a run of them between two MFMAs drains the matrix core.
+      // one block of straight-line code that the scheduler is told to weave.  A wavefront that has a SIMD to itself
+      // issues its instructions one after the other, and a 16-clock MFMA takes two issue turns of 4 clocks, a vector
+      // instruction one (measured on sequences of nothing else: an MFMA every 16.25 clocks with none, 16.4 with one or
+      // two vector instructions behind each, 20.4 with three): two other instructions fit behind every MFMA for free,
+      // and a run of them between two MFMAs drains the matrix core.
       // PAIRED: a loaded register holds macro step 2a in the lanes of rows 0-7 and step 2a+1 in the lanes of rows 8-15 of
       // every group of 16 lanes.  Four B operands are made of it: each step's rows in columns 0-7 (for the even tiles)
       // and in columns 8-15 (for the odd tiles), zeros in the other half -- a mask where the rows stay, a row shift by 8
@@ -1285,7 +1287,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
           const int ks = c >> 1, odd = c & 1;
           i32x4 opnd_next = opnd;
           if (c + 1 < NCH) opnd_next = operand(c + 1);
-          // (at most a dozen instructions fit behind a chunk's four MFMAs; with fewer chunks the last one takes the rest)
+          // (eight instructions fit behind a chunk's four MFMAs, four of them the next operand's; with fewer chunks the last one takes the rest)
           auto at = [&](int want) { return c == (want < NCH ? want : NCH - 1); };
           if (at(0)) flush_read_at(rd_h, rd_y, rd_c);
           if (at(1)) load_gate_inputs(IntTag<1 - PAR>{});
@@ -1300,7 +1302,7 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
           for (int u = 0; u < NACC; ++u) {
             acc[u][0] = E::mma(wreg[2 * u + odd][ks], opnd, acc[u][0]);
             __builtin_amdgcn_sched_group_barrier(0x008, sizeof(AT) == 2 ? 1 : 4, 0);  // the MFMA(s) of one fragment ...
-            __builtin_amdgcn_sched_group_barrier(0x096, 3, 0);                        // ... then up to three of the rest (four or five: 2-3 % slower)
+            __builtin_amdgcn_sched_group_barrier(0x096, 2, 0);                        // ... then up to two of the rest (three: 0-1 % slower; four or five: 2-3 %)
           }
           __builtin_amdgcn_sched_barrier(0);
           opnd = opnd_next;
@@ -1582,8 +1584,10 @@ __global__ __launch_bounds__(kWgThreads) void k_mfma_sequence(float* out, int st
 // Measurement aid: the matrix cores alone.  Every workgroup of the plan's grid issues, per step, the MT * NT * KSMAX MFMAs
 // of one wavefront's share -- the plan's tile sequence, in the op's order (macro steps outside, tiles inside), W fragments
 // and B fragments in registers -- and nothing else: no LDS, no barrier, no sum over the wavefronts, no loads.  (The
-// accumulators run on from step to step instead of starting at zero, and the B fragments pass through an empty
-// assembly statement every step so that the compiler cannot take a step's work for a repetition of the last.)  The time of
+// accumulators start at zero in every step, as the op's do, and end in an empty assembly statement that stands for their
+// use; the B fragments pass through another one every step, so that the compiler cannot take a step's work for a
+// repetition of the last.  Accumulators that run on from step to step instead cost a round of register copies at the
+// loop's back edge, a fifth of the step, that no kernel of the op has.)  The time of
 // a launch over the op's algorithmic flops is what the matrix cores can reach on this tile sequence: the ceiling of the
 // recurrent GEMM that no arrangement of the rest of the step can exceed.
 template <typename AT, int MT, int NT, int KSMAX, int THREADS = kWgThreads>
@@ -1614,7 +1618,7 @@ __global__ __launch_bounds__(THREADS) void k_mfma_issue(float* out, int steps) {
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};  // (steps == 0)
   const unsigned long long clk0 = clock64(), wall0 = wall_clock64();
   for (int s = 0; s < steps; ++s) {
 #pragma unroll
@@ -1622,11 +1626,19 @@ __global__ __launch_bounds__(THREADS) void k_mfma_issue(float* out, int steps) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) asm volatile("" : "+v"(bf[ks][nt]));
 #pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
     for (int ks = 0; ks < KSMAX; ++ks)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) asm volatile("" : "+a"(acc[mt][nt]));
   }
   f32x4 total = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
