@@ -921,6 +921,29 @@ def main():
         if float(marks[:, 1].min()) > 0:
             issue_clock_mhz = float((marks[:, 0] / marks[:, 1]).mean()) * 100.0
 
+    # What fits behind an MFMA: the issue probe again with one, two and three vector instructions behind every MFMA
+    # (a measurement variant of the library's probe for this plan's tile sequence, 64 MFMAs per wavefront and step),
+    # in shader clocks per MFMA as the probe's own wavefronts count them.
+    issue_clocks = None
+    if (issue_clock_mhz is not None and not measuring_only and not args.no_step_budget and dt_code == lib.DTYPE_BF16 and n == 1024
+            and " mt=8 nt=1 " in lib.describe_multi_plan(2 if fused else 1, T, B, n, dt_code, mode)):  # fmt: skip
+        def clocks_per_mfma():
+            marks = seq_ws[: 256 * 4 * 4].view(torch.float32).view(4, 256)[:, 1].double().cpu()
+            return float(marks.mean()) / (T * 64.0)
+
+        issue_clocks = {"0": clocks_per_mfma()}
+        try:
+            for others in (1, 2, 3):
+                os.environ["RTN_LSTM2_PROBE_OTHERS"] = str(others)
+                lib.reload_env()
+                if time_probe(cabi.rtn_mfma_issue_probe) is None:
+                    issue_clocks = None
+                    break
+                issue_clocks[str(others)] = clocks_per_mfma()
+        finally:
+            del os.environ["RTN_LSTM2_PROBE_OTHERS"]
+            lib.reload_env()
+
     # The same launch with the reads of the hidden state switched off (a timing aid of the library: no loads from the
     # exchange ring, no delay in front of them, no waiting -- the MFMAs run on zeros, the new values are still stored;
     # results are invalid and the status word says so): what a step costs when the hidden state is there for free.
@@ -1000,6 +1023,7 @@ def main():
             "launch_ms": call_ms,
             **ceiling_fields(probe_us, seq_ms, issue_ms, units_per_launch // T, n, dtype, T, call_ms),
             "mfma_issue_clock_mhz": issue_clock_mhz,
+            "mfma_issue_clocks_per_mfma_by_instructions_behind": issue_clocks,
             "step_budget_us": step_budget(call_ms, nowait_ms, seq_ms, issue_ms, T),
             "hbm_algorithmic_GBps": bytes_per_launch / (call_ms * 1e-3) / 1e9,
             "hbm_frac": bytes_per_launch / (call_ms * 1e-3) / PEAK_HBM,
@@ -1022,6 +1046,7 @@ def main():
         })
         for key in ("latency_ceiling", "frac_of_latency_ceiling", "mfma_peak_us_per_step", "achievable_mfma", "frac_of_achievable_mfma",
                     "mfma_sequence_us_per_step", "mfma_issue_us_per_step", "mfma_issue_clock_mhz", "step_budget_us", "decomposition_ceiling",
+                    "mfma_issue_clocks_per_mfma_by_instructions_behind",
                     "frac_of_decomposition_ceiling"):
             result["roofline"].pop(key, None)  # they describe the exchange-bound persistent kernel
     if not args.no_cpu_baseline:

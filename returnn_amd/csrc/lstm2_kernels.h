@@ -1253,9 +1253,9 @@ __global__ __launch_bounds__(kWgThreads) void k_lstm2_regw(const Lstm2Multi mult
       // a branch (a frame that does not exist is a buffer of no bytes; LDS copies nobody reads may take anything), in
       // one block of straight-line code that the scheduler is told to weave.  A wavefront that has a SIMD to itself
       // issues its instructions one after the other, and a 16-clock MFMA takes two issue turns of 4 clocks, a vector
-      // instruction one (measured on sequences of nothing else: an MFMA every 16.25 clocks with none, 16.4 with one or
-      // two vector instructions behind each, 20.4 with three): two other instructions fit behind every MFMA for free,
-      // and a run of them between two MFMAs drains the matrix core.
+      // instruction one (k_mfma_issue with OTHERS = 0 ... 3 vector instructions behind every MFMA: an MFMA every
+      // 16.2 / 16.6 / 16.7 / 20.7 clocks): two other instructions fit behind every MFMA for free, and a run of them
+      // between two MFMAs drains the matrix core.
       // PAIRED: a loaded register holds macro step 2a in the lanes of rows 0-7 and step 2a+1 in the lanes of rows 8-15 of
       // every group of 16 lanes.  Four B operands are made of it: each step's rows in columns 0-7 (for the even tiles)
       // and in columns 8-15 (for the odd tiles), zeros in the other half -- a mask where the rows stay, a row shift by 8
@@ -1590,7 +1590,9 @@ __global__ __launch_bounds__(kWgThreads) void k_mfma_sequence(float* out, int st
 // loop's back edge, a fifth of the step, that no kernel of the op has.)  The time of
 // a launch over the op's algorithmic flops is what the matrix cores can reach on this tile sequence: the ceiling of the
 // recurrent GEMM that no arrangement of the rest of the step can exceed.
-template <typename AT, int MT, int NT, int KSMAX, int THREADS = kWgThreads>
+// OTHERS > 0: that many vector instructions (register moves) behind every MFMA -- what a wavefront can issue in an
+// MFMA's shadow before the matrix core has to wait for it.
+template <typename AT, int MT, int NT, int KSMAX, int THREADS = kWgThreads, int OTHERS = 0>
 __global__ __launch_bounds__(THREADS) void k_mfma_issue(float* out, int steps) {
   using E = Elem<AT>;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -1619,6 +1621,7 @@ __global__ __launch_bounds__(THREADS) void k_mfma_issue(float* out, int steps) {
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};  // (steps == 0)
+  int moved = 0;
   const unsigned long long clk0 = clock64(), wall0 = wall_clock64();
   for (int s = 0; s < steps; ++s) {
 #pragma unroll
@@ -1634,7 +1637,15 @@ __global__ __launch_bounds__(THREADS) void k_mfma_issue(float* out, int steps) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+        for (int nt = 0; nt < NT; ++nt) {
+          acc[mt][nt] = E::mma(wreg[mt][ks], bf[ks][nt], acc[mt][nt]);
+          if constexpr (OTHERS > 0) {  // (fenced: the moves stay behind their MFMA)
+            if constexpr (OTHERS == 1) asm volatile("v_mov_b32 %0, %1" : "=v"(moved) : "v"(lane));
+            if constexpr (OTHERS == 2) asm volatile("v_mov_b32 %0, %1\n\tv_mov_b32 %0, %1" : "=v"(moved) : "v"(lane));
+            if constexpr (OTHERS >= 3) asm volatile("v_mov_b32 %0, %1\n\tv_mov_b32 %0, %1\n\tv_mov_b32 %0, %1" : "=v"(moved) : "v"(lane));
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -1648,7 +1659,7 @@ __global__ __launch_bounds__(THREADS) void k_mfma_issue(float* out, int steps) {
   // Thread 0 leaves the sum (so that nothing can be dropped), threads 1 and 2 what the loop took in shader clocks and in
   // ticks of the constant 100 MHz clock: their ratio is the clock rate the matrix cores ran at under this load.
   const unsigned long long clk1 = clock64(), wall1 = wall_clock64();
-  float v = total[0] + total[1] + total[2] + total[3];
+  float v = total[0] + total[1] + total[2] + total[3] + (float)moved;
   if (tid == 1) v = (float)(clk1 - clk0);
   if (tid == 2) v = (float)(wall1 - wall0);
   if (tid < kWgThreads) out[(size_t)blockIdx.x * kWgThreads + tid] = v;

@@ -1553,6 +1553,11 @@ int mfma_probe(bool issue_only, int32_t count, int64_t T, int32_t B, int32_t n, 
     // the matrix cores do when a second wavefront fills the gaps one wavefront leaves between its MFMAs
     k = &k_mfma_issue<__bf16, 8, 1, 4, 512>;
     threads = 512;
+  } else if (issue_only && env_long("RTN_LSTM2_PROBE_OTHERS", 0) > 0 && dtype == RTN_DTYPE_BF16 && pl.MT == 8 && pl.NT == 1 && pl.KSMAX == 8) {
+    // measurement variant: one, two or three vector instructions behind every MFMA -- how much of a step's other work a
+    // wavefront can issue in the MFMAs' shadow
+    const long others = env_long("RTN_LSTM2_PROBE_OTHERS", 0);
+    k = others == 1 ? &k_mfma_issue<__bf16, 8, 1, 8, kWgThreads, 1> : others == 2 ? &k_mfma_issue<__bf16, 8, 1, 8, kWgThreads, 2> : &k_mfma_issue<__bf16, 8, 1, 8, kWgThreads, 3>;
   } else if (issue_only)
     k = dtype == RTN_DTYPE_BF16 ? issue_kernel_for<__bf16>(pl.MT, pl.NT, pl.KSMAX) : issue_kernel_for<float>(pl.MT, pl.NT, pl.KSMAX);
   else
