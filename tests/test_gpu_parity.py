@@ -126,6 +126,40 @@ def test_decompositions(mt, groups, kernel):
             assert numpy.array_equal(a, b)
 
 
+def test_mfma_issue_probe_and_its_variants():
+    """The issue probe (the plan's MFMAs alone) is faster than the sequence probe on the same plan, and its measurement
+    variants behave as the issue of one wavefront per SIMD does: one or two vector instructions behind every MFMA cost
+    next to nothing, a third one costs a noticeable part of an MFMA."""
+    announce("mfma issue probe", 2, 1000, 32, 1024, "bf16")
+    get_op()
+    cabi = lib.load()
+    ws = torch.empty((1 << 20,), dtype=torch.uint8, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    steps = 1000
+
+    def us_per_step(fn):
+        times = []
+        for _ in range(4):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            lib.check(fn(2, 1000, 32, 1024, lib.DTYPE_BF16, steps, ws.data_ptr(), ws.numel(), stream))
+            e1.record()
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1) * 1e3 / steps)
+        return min(times[1:])
+
+    seq = us_per_step(cabi.rtn_mfma_sequence_probe)
+    by_others = {0: us_per_step(cabi.rtn_mfma_issue_probe)}
+    for others in (1, 2, 3):
+        with env(RTN_LSTM2_PROBE_OTHERS=others):
+            by_others[others] = us_per_step(cabi.rtn_mfma_issue_probe)
+    print("MFMA issue probe: %s us per step; sequence probe %.3f" % (", ".join("%i behind: %.3f" % kv for kv in sorted(by_others.items())), seq))
+    assert 0.3 < by_others[0] < seq
+    assert by_others[2] < 1.15 * by_others[0]
+    assert by_others[3] > 1.08 * by_others[2]
+    assert cabi.rtn_mfma_issue_probe(2, 1000, 32, 1024, lib.DTYPE_BF16, 0, ws.data_ptr(), ws.numel(), stream) == lib.RTN_ERR_ARG
+
+
 @pytest.mark.parametrize("count,T,B,n,dtype", [(2, 1000, 32, 1024, "bf16"), (1, 1000, 32, 1024, "bf16"), (1, 4000, 1, 1024, "bf16"), (1, 500, 64, 512, "f32")])
 def test_mfma_sequence_probe(count, T, B, n, dtype):
     """The roofline probe (the plan's MFMA sequence without any exchange) runs on the plan's grid, is faster per step
