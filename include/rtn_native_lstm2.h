@@ -201,7 +201,11 @@ int rtn_mfma_sequence_probe(int32_t count, int64_t T, int32_t B, int32_t n, int3
  * Measurement aid: the matrix cores alone.  Like rtn_mfma_sequence_probe (same arguments, same grid, same per-wavefront
  * tile sequence with W and the hidden-state fragments in registers), but a step is the MFMAs and nothing else: no LDS
  * round trip of partial tiles, no barrier, no sum.  Launch time over the op's algorithmic flops = the MFMA roofline the
- * plan's tile sequence can reach at most, whatever the rest of a step looks like.  No counterpart in the reference.
+ * plan's tile sequence can reach at most, whatever the rest of a step looks like.  Threads 1 and 2 of every workgroup
+ * leave the loop's duration in workspace words 1 and 2 of the workgroup's 1 KiB (float32: shader clocks, ticks of the
+ * 100 MHz clock).  Measurement variants for the bf16 plan with 8 tiles per workgroup, chosen by the environment:
+ * RTN_LSTM2_PROBE_OTHERS=1..3 puts that many vector instructions behind every MFMA, RTN_LSTM2_PROBE_WAVES=8 deals the
+ * MFMAs to two wavefronts per SIMD.  No counterpart in the reference.
  */
 int rtn_mfma_issue_probe(int32_t count, int64_t T, int32_t B, int32_t n, int32_t dtype, int32_t steps, void* workspace,
                          size_t workspace_bytes, void* hip_stream);
