@@ -1,8 +1,8 @@
 """
-Test infrastructure, never shipped with the library: builds ten of the reference's native ops for gfx950 through this
-package's op loader -- seven of its OTHER ops, and its three LSTM ops with the gradient ops the loader derives for them --
-so that the GPU tests can run them against the known answers the reference's own tests hold and against the committed
-golden vectors.
+Test infrastructure, never shipped with the library: builds nineteen of the reference's native ops for gfx950 through this
+package's op loader -- sixteen of its OTHER ops, and its three LSTM ops with the gradient ops the loader derives for them --
+so that the GPU tests can run them against the known answers the reference's own tests hold, against the committed
+golden vectors and, where the reference holds no numbers, against the library routines and numpy forms its own tests use.
 
 The op descriptions are read as text where they lie (``/root/reference/returnn/native_op.py``, parsed with :mod:`ast` by
 ``tests/_reference_op_sources.py``; nothing of the reference is imported or executed), the loader generates the unit and
@@ -33,7 +33,11 @@ OUT_DIR = os.path.join(HERE, "_built_ref_ops")
 # :689-812, :922-1034, :1036-1400)
 OPS = ("FastBaumWelchOp", "FastViterbiOp", "EditDistanceOp", "OptimalCompletionEditDistanceOp",
        "OptimalCompletionEditDistancePerSuccessorOp", "NextEditDistanceRowOp", "NextEditDistanceReduceOp",
-       "NativeLstm2", "LstmGenericBase", "LstmLowMem")
+       "NativeLstm2", "LstmGenericBase", "LstmLowMem",
+       # ops the reference's tests check against library routines and numpy instead (tests/test_TFNativeOp.py:1297-1560,
+       # :1629-1760); tests/test_gpu_ref_more_ops.py does the same
+       "Chunking", "UnChunking", "SubtensorBatchedIndex", "SparseToDense", "MaxAndArgmaxSparse",
+       "CrossEntropySoftmaxAndGradientZSparse", "GetCtcFsaFastBwOp", "GetCtcFsaFastBwPackedOp", "FastBaumWelchPackedOp")
 # of these also the gradient op that the loader derives from c_bw_code and grad_input_map ("GradOf<name>")
 WITH_GRADIENT = ("NativeLstm2", "LstmGenericBase", "LstmLowMem")
 
