@@ -24,6 +24,7 @@ import os
 import shutil
 import sys
 import tempfile
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
@@ -67,21 +68,32 @@ def build(ops=OPS, out_dir: str = OUT_DIR, verbose: bool = True) -> bool:
     os.makedirs(out_dir, exist_ok=True)
     table = {}
     with tempfile.TemporaryDirectory(prefix="rtn_ref_ops_") as tmp:
-        for name in ops:
+
+        def one(name):
+            """Compiles the op (and its gradient op): [(entry name, argument table)]."""
             fields = classes[name]
             op = op_loader.compile_op(ref_sources.as_description(name, fields), compiler_opts={"cache_dir": tmp})
             shutil.copyfile(op.compiler.so_filename, os.path.join(out_dir, name + ".so"))
-            table[name] = {"in_info": _plain(fields["in_info"]), "out_info": _plain(fields["out_info"])}
-            if verbose:
-                print("build_ref_ops: %s -> %s" % (name, os.path.join(out_dir, name + ".so")))
+            made = [(name, {"in_info": _plain(fields["in_info"]), "out_info": _plain(fields["out_info"])})]
             if name in WITH_GRADIENT:
                 grad = op_loader.grad_description(ref_sources.as_description(name, fields))
                 gname, g_in, g_out = op_loader.description_fields(grad)[:3]
                 gop = op_loader.compile_op(grad, compiler_opts={"cache_dir": tmp})
                 shutil.copyfile(gop.compiler.so_filename, os.path.join(out_dir, gname + ".so"))
-                table[gname] = {"in_info": _plain(g_in), "out_info": _plain(g_out)}
-                if verbose:
-                    print("build_ref_ops: %s -> %s" % (gname, os.path.join(out_dir, gname + ".so")))
+                made.append((gname, {"in_info": _plain(g_in), "out_info": _plain(g_out)}))
+            return made
+
+        # (one hipcc per op, several at a time: as many as the machine has cores, or MAX_JOBS)
+        try:
+            limit = int(os.environ.get("MAX_JOBS", "0"))
+        except ValueError:
+            limit = 0
+        with ThreadPoolExecutor(max_workers=max(1, min(len(ops), limit or (os.cpu_count() or 1)))) as pool:
+            for made in pool.map(one, ops):
+                for entry, info in made:
+                    table[entry] = info
+                    if verbose:
+                        print("build_ref_ops: %s -> %s" % (entry, os.path.join(out_dir, entry + ".so")))
     with open(os.path.join(out_dir, "ops.json"), "w") as f:
         json.dump(table, f, indent=1, sort_keys=True)
     return True
