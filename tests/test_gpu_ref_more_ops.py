@@ -296,6 +296,48 @@ def test_ctc_automaton_through_baum_welch_equals_ctc_loss(case):
     numpy.testing.assert_allclose(_host(scores)[inside], w_score[inside], rtol=1e-5)
 
 
+def _paths_by_enumeration(log_probs, target, blank, label_loop):
+    """-log of the summed probability of all frame labellings of length T that give `target`: blanks removed, and with
+    label_loop repeats of a label merged first (CTC); without it every non-blank frame is a label of its own (the
+    recurrent neural aligner's topology).  By enumeration of all C^T labellings: for a handful of frames only."""
+    import itertools
+
+    T, C = log_probs.shape
+    total = -numpy.inf
+    for path in itertools.product(range(C), repeat=T):
+        labels = [c for k, c in enumerate(path) if not (label_loop and k > 0 and path[k - 1] == c)]
+        if [c for c in labels if c != blank] == list(target):
+            total = numpy.logaddexp(total, sum(log_probs[t, c] for t, c in enumerate(path)))
+    return -total
+
+
+@needs("GetCtcFsaFastBwOp", "FastBaumWelchOp")
+@pytest.mark.parametrize("label_loop", [True, False])
+def test_ctc_automaton_with_and_without_label_loop_by_enumeration(label_loop):
+    """Both topologies of the automaton builder against the sum over all labellings, on sequences short enough to
+    enumerate (the reference checks the loop-free one against TensorFlow's loss with ctc_merge_repeated=False,
+    tests/test_TFNativeOp.py:1815-1826; torch's loss has no such switch)."""
+    announce("reference op GetCtcFsaFastBwOp, label_loop", label_loop)
+    make_fsa, baum_welch = _op("GetCtcFsaFastBwOp"), _op("FastBaumWelchOp")
+    targets = numpy.array([[0, 1, 1], [1, 1, 0], [2, 0, 0]], dtype=numpy.int32)
+    target_lens = numpy.array([3, 2, 1], dtype=numpy.int32)
+    n_classes, blank = 4, 3
+    lens = numpy.array([6, 5, 4])
+    n_time, n_batch = 6, 3
+    logits = numpy.random.RandomState(11).normal(size=(n_time, n_batch, n_classes)).astype(numpy.float32)
+    log_probs = torch.log_softmax(torch.tensor(logits, dtype=torch.float64), dim=2).numpy()
+    n_edges = n_batch * (5 * (targets.shape[1] - 1) + 10)
+    weights = torch.zeros((n_edges,), device="cuda:0")
+    edges, start_end = make_fsa(_dev(targets), _dev(target_lens), blank, weights, int(label_loop))
+    n_states = int(_host(start_end)[1].max()) + 1
+    index = (numpy.arange(n_time)[:, None] < lens[None, :]).astype(numpy.float32)
+    fwdbwd, scores = baum_welch(_dev((-log_probs).astype(numpy.float32)), edges, weights, start_end, _dev(index), n_states)
+    scores = _host(scores)
+    for b in range(n_batch):
+        want = _paths_by_enumeration(log_probs[: lens[b], b], targets[b, : target_lens[b]], blank, label_loop)
+        numpy.testing.assert_allclose(scores[: lens[b], b], want, rtol=2e-5)
+
+
 @needs("GetCtcFsaFastBwPackedOp", "FastBaumWelchOp", "FastBaumWelchPackedOp")
 @pytest.mark.parametrize("case", [0, 1, 4, 7])
 def test_packed_ctc_automaton_and_packed_baum_welch(case):
