@@ -79,7 +79,7 @@ def prepare_weights(
 ) -> LstmWeights:
     """
     Frontend parameters -> op layout (returnn/tf/frontend_layers/_backend.py:1199-1222): reorder the gate blocks
-    and transpose.  Worth caching while the parameters do not change; :class:`LSTM` does.
+    and transpose.  (:class:`LSTM` and :class:`BLSTM` keep their parameters in the op's layout and need none of this.)
 
     :param ff_weight: [4*out, in]
     :param rec_weight: [4*out, out]
@@ -325,38 +325,87 @@ def blstm(
 
 class LSTM(torch.nn.Module):
     """
-    The module of returnn/frontend/rec.py:16-83 with integer dims: parameters ``ff_weight [4*out,in]``,
-    ``rec_weight [4*out,out]`` (both Glorot-uniform, returnn/frontend/init.py:189-197) and ``bias [4*out]`` (zeros).
+    The module of returnn/frontend/rec.py:16-83 with integer dims.
+
+    Like :class:`BLSTM`, it keeps its parameters in the layout the op takes -- ``ff [4*out, in]`` with the gate blocks in
+    the order cell-in, input, forget, output (the projection uses its transposed view), ``rec [out, 4*out]``,
+    ``bias [4*out]`` -- so that neither a forward nor a training step reorders or transposes anything.  The frontend's
+    layout (``ff_weight [4*out,in]``, ``rec_weight [4*out,out]``, ``bias [4*out]`` in the order input, forget, cell-in,
+    output; the mapping of returnn/tf/frontend_layers/_backend.py:1199-1222) is what :meth:`frontend_params`,
+    :meth:`load_frontend_params`, ``state_dict()`` and ``load_state_dict()`` speak, under the frontend's parameter names.
+    Initialisation as the frontend's: ``ff_weight`` and ``rec_weight`` Glorot-uniform (returnn/frontend/init.py:189-197),
+    bias zero.
     """
+
+    _FRONTEND_KEYS = ("ff_weight", "rec_weight", "bias")
 
     def __init__(self, in_dim: int, out_dim: int, *, with_bias: bool = True, device=None, dtype=None):
         super().__init__()
         self.in_dim = int(in_dim)
         self.out_dim = int(out_dim)
         kw = dict(device=device, dtype=dtype)
-        self.ff_weight = torch.nn.Parameter(torch.empty((4 * self.out_dim, self.in_dim), **kw))
-        self.rec_weight = torch.nn.Parameter(torch.empty((4 * self.out_dim, self.out_dim), **kw))
+        self.ff = torch.nn.Parameter(torch.empty((4 * self.out_dim, self.in_dim), **kw))
+        self.rec = torch.nn.Parameter(torch.empty((self.out_dim, 4 * self.out_dim), **kw))
         self.bias = torch.nn.Parameter(torch.zeros((4 * self.out_dim,), **kw)) if with_bias else None
         self.reset_parameters()
-        self._prepared = None  # (key, LstmWeights)
 
     def reset_parameters(self, generator: Optional[torch.Generator] = None):
         with torch.no_grad():
-            for p in (self.ff_weight, self.rec_weight):
+            for p in (self.ff, self.rec):
                 limit = math.sqrt(6.0 / (p.shape[0] + p.shape[1]))  # scale 1 / fan_avg, uniform: sqrt(3*scale)
                 p.uniform_(-limit, limit, generator=generator)
             if self.bias is not None:
                 self.bias.zero_()
 
-    def _weights(self, act: torch.dtype) -> LstmWeights:
-        ps = [self.ff_weight, self.rec_weight] + ([self.bias] if self.bias is not None else [])
-        if _wants_grad(*ps):
-            return prepare_weights(self.ff_weight, self.rec_weight, self.bias, dtype=act)  # differentiable, not cached
-        key = (act,) + tuple((p.data_ptr(), p._version, p.device) for p in ps)
-        if self._prepared is None or self._prepared[0] != key:
-            with torch.no_grad():
-                self._prepared = (key, prepare_weights(self.ff_weight, self.rec_weight, self.bias, dtype=act))
-        return self._prepared[1]
+    def weights(self, act: torch.dtype) -> LstmWeights:
+        """The parameters as :func:`lstm` takes them (views; a cast only when the run's type is not the parameters')."""
+        return LstmWeights(ff=self.ff.to(act).t(), rec=self.rec.to(act), bias=None if self.bias is None else self.bias.to(act))
+
+    def frontend_params(self) -> dict:
+        """``{"ff_weight" [4*out,in], "rec_weight" [4*out,out], "bias" [4*out] or None}`` in the frontend's gate order
+        (copies, detached)."""
+        with torch.no_grad():
+            return {
+                "ff_weight": _from_native_gate_order(self.ff).contiguous(),
+                "rec_weight": _from_native_gate_order(self.rec.t()).contiguous(),
+                "bias": None if self.bias is None else _from_native_gate_order(self.bias).contiguous(),
+            }
+
+    def load_frontend_params(self, params: dict):
+        """Takes the parameters in the frontend's layout (arrays or tensors)."""
+        n4 = 4 * self.out_dim
+        ff_w, rec_w = torch.as_tensor(params["ff_weight"]), torch.as_tensor(params["rec_weight"])
+        if tuple(ff_w.shape) != (n4, self.in_dim) or tuple(rec_w.shape) != (n4, self.out_dim):
+            raise ValueError("LSTM: ff_weight %s / rec_weight %s, expected %s / %s"
+                             % (tuple(ff_w.shape), tuple(rec_w.shape), (n4, self.in_dim), (n4, self.out_dim)))  # fmt: skip
+        b = params.get("bias")
+        if (b is None) != (self.bias is None):
+            raise ValueError("LSTM: the layer was built %s a bias" % ("without" if self.bias is None else "with"))
+        with torch.no_grad():
+            self.ff.copy_(_to_native_gate_order(ff_w))
+            self.rec.copy_(_to_native_gate_order(rec_w).t())
+            if b is not None:
+                self.bias.copy_(_to_native_gate_order(torch.as_tensor(b)))
+
+    # state_dict / load_state_dict in the frontend's layout, so that checkpoints do not depend on the op's layout
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        for key, value in self.frontend_params().items():
+            if value is not None:
+                destination[prefix + key] = value
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
+        keys = [k for k in self._FRONTEND_KEYS if not (k == "bias" and self.bias is None)]
+        absent = [k for k in keys if prefix + k not in state_dict]
+        if absent:
+            if strict:
+                missing_keys.extend(prefix + k for k in absent)
+            return
+        try:
+            self.load_frontend_params({k: state_dict.get(prefix + k) for k in self._FRONTEND_KEYS})
+        except (ValueError, RuntimeError) as exc:
+            error_msgs.append(str(exc))
+        if strict:
+            unexpected_keys.extend(k for k in state_dict if k.startswith(prefix) and k[len(prefix) :] not in keys)
 
     def forward(
         self, source: torch.Tensor, *, state: LstmState, seq_lens: Optional[torch.Tensor] = None, direction: int = 1
@@ -373,16 +422,16 @@ class LSTM(torch.nn.Module):
             raise ValueError("%s: input %s does not have in_dim %i" % (self, tuple(source.shape), self.in_dim))
         act = torch.bfloat16 if source.dtype == torch.bfloat16 else torch.float32
         out, (h, c) = lstm(
-            source, state_h=state.h, state_c=state.c, weights=self._weights(act), seq_lens=seq_lens, direction=direction
+            source, state_h=state.h, state_c=state.c, weights=self.weights(act), seq_lens=seq_lens, direction=direction
         )
         return out, LstmState(h=h, c=c)
 
     def default_initial_state(self, *, batch_dims: Sequence[int], device=None) -> LstmState:
         """zeros (returnn/frontend/rec.py:78-83); h in the parameters' type, c in float32"""
-        device = device or self.rec_weight.device
+        device = device or self.rec.device
         shape = tuple(batch_dims) + (self.out_dim,)
         return LstmState(
-            h=torch.zeros(shape, dtype=self.rec_weight.dtype, device=device),
+            h=torch.zeros(shape, dtype=self.rec.dtype, device=device),
             c=torch.zeros(shape, dtype=torch.float32, device=device),
         )
 

@@ -80,9 +80,7 @@ def test_lstm_single_step_and_chaining():
     x = rng.standard_normal((T, B, d_in)).astype(numpy.float32)
     p = _params(rng, n, d_in)
     m = rlstm.LSTM(d_in, n, device=DEV)
-    with torch.no_grad():
-        for k in ("ff_weight", "rec_weight", "bias"):
-            getattr(m, k).copy_(_dev(p[k]))
+    m.load_frontend_params({k: _dev(p[k]) for k in ("ff_weight", "rec_weight", "bias")})
     h0 = (rng.standard_normal((B, n)) * 0.5).astype(numpy.float32)
     c0 = (rng.standard_normal((B, n)) * 0.5).astype(numpy.float32)
     s = rlstm.LstmState(h=_dev(h0), c=_dev(c0))
@@ -101,8 +99,8 @@ def test_lstm_single_step_and_chaining():
     assert_allclose(_np(s_all.c), c[0], rtol=F32_RTOL, atol=F32_ATOL)
 
 
-def test_module_weight_cache_follows_parameter_updates():
-    announce("lstm layer weight cache")
+def test_module_follows_parameter_updates():
+    announce("lstm layer parameter update")
     get_op()
     m = rlstm.LSTM(8, 16, device=DEV)
     s = m.default_initial_state(batch_dims=(3,))
@@ -111,10 +109,10 @@ def test_module_weight_cache_follows_parameter_updates():
     y1b, _ = m(x, state=s)
     assert torch.equal(y1, y1b)
     with torch.no_grad():
-        m.rec_weight.mul_(0.5)
+        m.rec.mul_(0.5)
     y2, _ = m(x, state=s)
-    ref, _ = rlstm.lstm(x, state_h=s.h, state_c=s.c, ff_weight=m.ff_weight.detach(), rec_weight=m.rec_weight.detach(),
-                        bias=m.bias.detach())  # fmt: skip
+    fp = m.frontend_params()
+    ref, _ = rlstm.lstm(x, state_h=s.h, state_c=s.c, ff_weight=fp["ff_weight"], rec_weight=fp["rec_weight"], bias=fp["bias"])
     assert torch.equal(y2, ref) and not torch.equal(y1, y2)
 
 
@@ -253,14 +251,12 @@ def test_blstm_layer_gradients_vs_torch(n):
     mods = []
     for p in (fwd, bwd):
         mod = rlstm.LSTM(d_in, n, device=DEV)
-        with torch.no_grad():
-            for k in ("ff_weight", "rec_weight", "bias"):
-                getattr(mod, k).copy_(_dev(p[k]))
+        mod.load_frontend_params({k: _dev(p[k]) for k in ("ff_weight", "rec_weight", "bias")})
         mods.append(mod)
     xg = _dev(x).requires_grad_(True)
     h0g = _dev(h0).requires_grad_(True)
     c0g = _dev(c0).requires_grad_(True)
-    y, sf, sb = rlstm.blstm(xg, fwd=mods[0]._weights(torch.float32), bwd=mods[1]._weights(torch.float32),
+    y, sf, sb = rlstm.blstm(xg, fwd=mods[0].weights(torch.float32), bwd=mods[1].weights(torch.float32),
                             state_fwd=rlstm.LstmState(h0g[0], c0g[0]), state_bwd=rlstm.LstmState(h0g[1], c0g[1]),
                             seq_lens=torch.from_numpy(lens))  # fmt: skip
     loss = (y * _dev(G)).sum() + (sf.h * _dev(Gh[0])).sum() + (sb.h * _dev(Gh[1])).sum() + (sf.c * _dev(Gc[0])).sum() + (sb.c * _dev(Gc[1])).sum()
@@ -276,9 +272,10 @@ def test_blstm_layer_gradients_vs_torch(n):
     close(h0g.grad, h0r.grad, "h0")
     close(c0g.grad, c0r.grad, "c0")
     for mod, sfx in zip(mods, ("", "_reverse")):
-        close(mod.ff_weight.grad, getattr(m, "weight_ih_l0" + sfx).grad, "ff_weight" + sfx)
-        close(mod.rec_weight.grad, getattr(m, "weight_hh_l0" + sfx).grad, "rec_weight" + sfx)
-        close(mod.bias.grad, getattr(m, "bias_ih_l0" + sfx).grad, "bias" + sfx)  # either half of torch's bias sees the gradient of the sum
+        # (the module's parameters are in the op's layout: back to torch's gate order and orientation)
+        close(rlstm._from_native_gate_order(mod.ff.grad), getattr(m, "weight_ih_l0" + sfx).grad, "ff_weight" + sfx)
+        close(rlstm._from_native_gate_order(mod.rec.grad.t()), getattr(m, "weight_hh_l0" + sfx).grad, "rec_weight" + sfx)
+        close(rlstm._from_native_gate_order(mod.bias.grad), getattr(m, "bias_ih_l0" + sfx).grad, "bias" + sfx)  # either half of torch's bias sees the gradient of the sum
 
 
 def test_lstm_module_trains_one_step():

@@ -277,7 +277,7 @@ def test_blstm_on_one_projection_equals_two_layers(dtype, T, B, n_in, n):
 
 def test_blstm_module_keeps_the_ops_layout_and_trains_like_two_lstm_modules():
     """:class:`BLSTM` (parameters in the op's layout, nothing converted per step) against two :class:`LSTM` modules
-    (parameters in the frontend's layout) holding the same weights: outputs, states and every parameter's gradient."""
+    holding the same weights: outputs, states and every parameter's gradient."""
     announce("BLSTM module")
     T, B, n_in, n = 8, 6, 48, 64
     gen = torch.Generator().manual_seed(11)
@@ -287,7 +287,7 @@ def test_blstm_module_keeps_the_ops_layout_and_trains_like_two_lstm_modules():
             for p in m.parameters():
                 p.copy_((torch.randn(p.shape, generator=gen) * 0.2).to("cuda:0"))
     layer = rlstm.BLSTM(n_in, n, device="cuda:0")
-    layer.load_frontend_params(*[{k: getattr(m, k).detach() for k in ("ff_weight", "rec_weight", "bias")} for m in singles])
+    layer.load_frontend_params(*[m.frontend_params() for m in singles])
     x = torch.randn((T, B, n_in), generator=gen).to("cuda:0")
     lens = torch.tensor([T, T - 1, 3, T, 1, 5])
     G = torch.randn((T, B, 2 * n), generator=gen).to("cuda:0")
@@ -307,10 +307,10 @@ def test_blstm_module_keeps_the_ops_layout_and_trains_like_two_lstm_modules():
 
     n4 = 4 * n
     for k, (m, rec) in enumerate(zip(singles, (layer.rec_fwd, layer.rec_bwd))):
-        close(rlstm._from_native_gate_order(layer.ff.grad[k * n4 : (k + 1) * n4]), m.ff_weight.grad, "ff %i" % k)
-        close(rlstm._from_native_gate_order(rec.grad.t()), m.rec_weight.grad, "rec %i" % k)
-        close(rlstm._from_native_gate_order(layer.bias.grad[k * n4 : (k + 1) * n4]), m.bias.grad, "bias %i" % k)
+        close(layer.ff.grad[k * n4 : (k + 1) * n4], m.ff.grad, "ff %i" % k)
+        close(rec.grad, m.rec.grad, "rec %i" % k)
+        close(layer.bias.grad[k * n4 : (k + 1) * n4], m.bias.grad, "bias %i" % k)
     # a checkpoint written by the layer is in the frontend's layout
     sd = layer.state_dict()
-    assert torch.equal(sd["bwd.rec_weight"], singles[1].rec_weight.detach())
-    assert torch.equal(sd["fwd.ff_weight"], singles[0].ff_weight.detach())
+    assert torch.equal(sd["bwd.rec_weight"], singles[1].state_dict()["rec_weight"])
+    assert torch.equal(sd["fwd.ff_weight"], singles[0].state_dict()["ff_weight"])

@@ -81,17 +81,47 @@ def test_sequence_mask_time_major():
 def test_module_parameters_and_init():
     torch.manual_seed(0)
     m = rlstm.LSTM(80, 64)
-    assert m.ff_weight.shape == (256, 80) and m.rec_weight.shape == (256, 64) and m.bias.shape == (256,)
+    # parameters in the op's layout; the frontend's layout and names in the state dict
+    assert m.ff.shape == (256, 80) and m.rec.shape == (64, 256) and m.bias.shape == (256,)
+    sd = m.state_dict()
+    assert sorted(sd) == ["bias", "ff_weight", "rec_weight"]
+    assert sd["ff_weight"].shape == (256, 80) and sd["rec_weight"].shape == (256, 64) and sd["bias"].shape == (256,)
     assert float(m.bias.detach().abs().max()) == 0.0
-    for p in (m.ff_weight, m.rec_weight):
+    for p in (sd["ff_weight"], sd["rec_weight"]):
         limit = math.sqrt(6.0 / sum(p.shape))
-        p = p.detach()
         assert float(p.abs().max()) <= limit
         assert float(p.abs().max()) > 0.9 * limit
         assert abs(float(p.var()) - limit * limit / 3.0) < 0.1 * limit * limit / 3.0  # variance 1/fan_avg
     assert rlstm.LSTM(4, 4, with_bias=False).bias is None
     s = m.default_initial_state(batch_dims=(3,))
     assert s.h.shape == (3, 64) and s.c.shape == (3, 64) and float(s.h.abs().sum() + s.c.abs().sum()) == 0.0
+
+
+def test_module_state_dict_speaks_the_frontend_layout():
+    """What the module keeps is the op's layout (gate blocks cell-in, input, forget, output; the recurrent matrix
+    transposed); what it saves and loads is the frontend's (returnn/tf/frontend_layers/_backend.py:1199-1222)."""
+    n, d_in = 3, 2
+    m = rlstm.LSTM(d_in, n)
+    ff = torch.arange(4 * n * d_in, dtype=torch.float32).reshape(4 * n, d_in)
+    rec = 100.0 + torch.arange(4 * n * n, dtype=torch.float32).reshape(4 * n, n)
+    bias = 1000.0 + torch.arange(4 * n, dtype=torch.float32)
+    m.load_state_dict({"ff_weight": ff, "rec_weight": rec, "bias": bias})
+    i, f, g, o = (slice(k * n, (k + 1) * n) for k in range(4))  # the frontend's blocks: input, forget, cell-in, output
+    assert torch.equal(m.ff.detach(), torch.cat((ff[g], ff[i], ff[f], ff[o])))
+    assert torch.equal(m.rec.detach(), torch.cat((rec[g], rec[i], rec[f], rec[o])).t())
+    assert torch.equal(m.bias.detach(), torch.cat((bias[g], bias[i], bias[f], bias[o])))
+    w = m.weights(torch.float32)
+    ref = rlstm.prepare_weights(ff, rec, bias)
+    assert torch.equal(w.ff, ref.ff) and torch.equal(w.rec, ref.rec) and torch.equal(w.bias, ref.bias)
+    sd = m.state_dict()
+    assert torch.equal(sd["ff_weight"], ff) and torch.equal(sd["rec_weight"], rec) and torch.equal(sd["bias"], bias)
+    m2 = rlstm.LSTM(d_in, n)
+    m2.load_state_dict(sd)
+    assert all(torch.equal(a, b) for a, b in zip(m.parameters(), m2.parameters()))
+    with pytest.raises(RuntimeError, match="ff_weight"):
+        m2.load_state_dict({"ff_weight": ff[:, :1], "rec_weight": rec, "bias": bias})
+    with pytest.raises(RuntimeError, match="Missing"):
+        m2.load_state_dict({"ff_weight": ff, "bias": bias})
 
 
 def test_no_cpu_implementation():
